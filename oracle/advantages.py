@@ -1,0 +1,179 @@
+"""Oracle for the advantage estimators on the path: GAE and GRPO (CPU torch).
+
+Test infrastructure only; see ``oracle/__init__.py``.
+"""
+
+from __future__ import annotations
+
+from collections import defaultdict
+
+import numpy as np
+import torch
+
+from .masked import masked_whiten
+
+
+@torch.no_grad()
+def gae_raw(token_level_rewards, values, response_mask, gamma, lam):
+    """The recurrence of verl/trainer/ppo/core_algos.py:244-260 without the final
+    whitening: returns ``(raw_advantages, returns)``."""
+    nv = 0
+    g = 0
+    cols = []
+    L = token_level_rewards.shape[-1]
+    for t in range(L - 1, -1, -1):
+        m = response_mask[:, t]
+        delta = token_level_rewards[:, t] + gamma * nv - values[:, t]
+        g_new = delta + gamma * lam * g
+        nv = values[:, t] * m + (1 - m) * nv
+        g = g_new * m + (1 - m) * g
+        cols.append(g)
+    adv = torch.stack(cols[::-1], dim=1)
+    return adv, adv + values
+
+
+@torch.no_grad()
+def gae_advantage_return(token_level_rewards, values, response_mask, gamma, lam):
+    """Reverse GAE recurrence with carried state on masked steps, then whiten.
+
+    Follows verl/trainer/ppo/core_algos.py:214-262 step for step, including the
+    arithmetic form of the two selects (``x*m + (1-m)*carry``), ``returns`` from
+    the RAW advantages (:260) and ``masked_whiten`` last (:261).
+    """
+    adv, returns = gae_raw(token_level_rewards, values, response_mask, gamma, lam)
+    adv = masked_whiten(adv, response_mask)
+    return adv, returns
+
+
+def gae_brute_force_fp64(rewards, values, mask, gamma, lam):
+    """Scalar double-precision recurrence over Python lists, written from the
+    textbook definition with select-by-branch instead of arithmetic selects; used
+    to pin ``gae_advantage_return`` before whitening."""
+    B = len(rewards)
+    L = len(rewards[0])
+    adv = [[0.0] * L for _ in range(B)]
+    for b in range(B):
+        nv, g = 0.0, 0.0
+        for t in range(L - 1, -1, -1):
+            if mask[b][t] != 0:
+                delta = rewards[b][t] + gamma * nv - values[b][t]
+                g = delta + gamma * lam * g
+                nv = values[b][t]
+            adv[b][t] = g
+    return adv
+
+
+def grpo_outcome_advantage(token_level_rewards, response_mask, index, epsilon=1e-6,
+                           norm_adv_by_std_in_grpo=True):
+    """Loop form, verl/trainer/ppo/core_algos.py:266-330.
+
+    Score = unmasked row sum (:303); groups keyed by ``index[i]`` with Python
+    equality (:312); singleton group -> mean 0, std 1 (:314-316); else
+    ``torch.mean`` / unbiased ``torch.std`` (:318-320); epsilon added to the std
+    (:325).  Returns the same tensor twice (:330).
+    """
+    scores = token_level_rewards.sum(dim=-1)
+    members = defaultdict(list)
+    mean_of, std_of = {}, {}
+    with torch.no_grad():
+        for i in range(scores.shape[0]):
+            members[index[i]].append(scores[i])
+        for key, vals in members.items():
+            if len(vals) == 1:
+                mean_of[key] = torch.tensor(0.0)
+                std_of[key] = torch.tensor(1.0)
+            elif len(vals) > 1:
+                stacked = torch.stack(vals)
+                mean_of[key] = torch.mean(stacked)
+                std_of[key] = torch.std(stacked)
+            else:
+                raise ValueError(f"no score in prompt index: {key}")
+        for i in range(scores.shape[0]):
+            if norm_adv_by_std_in_grpo:
+                scores[i] = (scores[i] - mean_of[index[i]]) / (std_of[index[i]] + epsilon)
+            else:
+                scores[i] = scores[i] - mean_of[index[i]]
+        out = scores.unsqueeze(-1) * response_mask
+    return out, out
+
+
+def as_torch_index(index):
+    """Labels -> contiguous int64 ids.  Follows verl/utils/groupwise.py:91-160 for
+    the cases the path meets: integer arrays pass through, near-integer floats are
+    rounded, numeric strings are coerced, everything else is factorised with
+    ``np.unique(return_inverse=True)``."""
+    if isinstance(index, torch.Tensor):
+        t = index.reshape(-1)
+        if not t.dtype.is_floating_point:
+            return t.to(torch.long)
+        t64 = t.to(torch.float64)
+        r = torch.round(t64)
+        if torch.allclose(t64, r, rtol=0.0, atol=1e-6):
+            return r.to(torch.long)
+        arr = np.array([str(x.item()) for x in t], dtype=object)
+    else:
+        try:
+            arr = np.asarray(index)
+        except Exception:
+            arr = np.array(list(index), dtype=object)
+        arr = arr.reshape(-1)
+        if arr.dtype != object and np.issubdtype(arr.dtype, np.integer):
+            return torch.from_numpy(arr.astype(np.int64, copy=False))
+        if arr.dtype != object and np.issubdtype(arr.dtype, np.floating):
+            a64 = arr.astype(np.float64, copy=False)
+            r = np.rint(a64)
+            if np.allclose(a64, r, rtol=0.0, atol=1e-6):
+                return torch.from_numpy(r.astype(np.int64))
+        try:
+            return torch.from_numpy(arr.astype(np.int64))
+        except Exception:
+            pass
+        if arr.dtype != object:
+            arr = arr.astype(object)
+    try:
+        _, inv = np.unique(arr, return_inverse=True)
+    except Exception:
+        _, inv = np.unique(np.array([str(x) for x in arr], dtype=object), return_inverse=True)
+    return torch.from_numpy(inv.astype(np.int64, copy=False))
+
+
+@torch.no_grad()
+def group_mean_std(scores, gidx, eps=1e-6):
+    """Per-group mean / std / count by ``index_add_`` of 1, x, x^2.
+
+    Follows verl/utils/groupwise.py:163-223: var = (S2 - S1^2/n)/max(n-1,1),
+    std = sqrt(clamp(var, min=eps)); singleton (n<=1) -> mean 0, std 1.
+    """
+    scores = scores.reshape(-1).to(torch.float32)
+    gidx = gidx.reshape(-1).to(torch.long)
+    if scores.numel() != gidx.numel():
+        raise ValueError(f"scores and gidx length mismatch: {scores.numel()} vs {gidx.numel()}")
+    G = int(gidx.max().item()) + 1 if gidx.numel() > 0 else 0
+    if G == 0:
+        e = torch.empty(0, dtype=torch.float32)
+        return e, e, e
+    cnt = torch.zeros(G).index_add_(0, gidx, torch.ones_like(scores))
+    s1 = torch.zeros(G).index_add_(0, gidx, scores)
+    s2 = torch.zeros(G).index_add_(0, gidx, scores * scores)
+    mean = s1 / cnt.clamp_min(1.0)
+    var = (s2 - s1 * s1 / cnt.clamp_min(1.0)) / (cnt - 1.0).clamp_min(1.0)
+    std = torch.sqrt(torch.clamp(var, min=eps))
+    single = cnt <= 1.0
+    mean = torch.where(single, torch.zeros_like(mean), mean)
+    std = torch.where(single, torch.ones_like(std), std)
+    return mean, std, cnt
+
+
+@torch.no_grad()
+def grpo_vectorized_outcome_advantage(token_level_rewards, response_mask, index, epsilon=1e-6,
+                                      norm_adv_by_std_in_grpo=True):
+    """Vectorised twin, verl/trainer/ppo/core_algos.py:333-357."""
+    scores = token_level_rewards.sum(dim=-1)
+    g = as_torch_index(index)
+    mean_g, std_g, _ = group_mean_std(scores, g, eps=epsilon)
+    if norm_adv_by_std_in_grpo:
+        a = (scores - mean_g[g]) / (std_g[g] + epsilon)
+    else:
+        a = scores - mean_g[g]
+    out = a.unsqueeze(-1) * response_mask
+    return out, out

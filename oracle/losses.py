@@ -1,0 +1,97 @@
+"""Oracle for loss aggregation, the clipped / dual-clip policy loss, the clipped
+value loss and the KL estimators (CPU torch, differentiable through autograd).
+
+Test infrastructure only; see ``oracle/__init__.py``.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .masked import clip_by_value, masked_mean, masked_sum
+
+
+def agg_loss(loss_mat, loss_mask, loss_agg_mode, dp_size=1, batch_num_tokens=None,
+             global_batch_size=None, loss_scale_factor=None):
+    """Four aggregation modes, verl/trainer/ppo/core_algos.py:1025-1080.
+
+    ``token-mean`` divides by ``mask.sum()`` with NO epsilon (:1055-1058); the two
+    ``seq-mean`` modes drop fully masked rows through a 0/1 row mask
+    (:1059-1071); ``seq-mean-token-sum-norm`` divides by the row length unless a
+    factor is given (:1072-1076).
+    """
+    if loss_agg_mode == "token-mean":
+        if batch_num_tokens is None:
+            batch_num_tokens = loss_mask.sum()
+        return masked_sum(loss_mat, loss_mask) / batch_num_tokens * dp_size
+    if loss_agg_mode == "seq-mean-token-sum":
+        row = torch.sum(loss_mat * loss_mask, dim=-1)
+        keep = (torch.sum(loss_mask, dim=-1) > 0).float()
+        if global_batch_size is None:
+            global_batch_size = keep.sum()
+        return masked_sum(row, keep) / global_batch_size * dp_size
+    if loss_agg_mode == "seq-mean-token-mean":
+        cnt = torch.sum(loss_mask, dim=-1)
+        row = torch.sum(loss_mat * loss_mask, dim=-1) / (cnt + 1e-8)
+        keep = (cnt > 0).float()
+        if global_batch_size is None:
+            global_batch_size = keep.sum()
+        return masked_sum(row, keep) / global_batch_size * dp_size
+    if loss_agg_mode == "seq-mean-token-sum-norm":
+        row = torch.sum(loss_mat * loss_mask, dim=-1)
+        if loss_scale_factor is None:
+            loss_scale_factor = loss_mask.shape[-1]
+        return torch.sum(row) / loss_scale_factor
+    raise ValueError(f"Invalid loss_agg_mode: {loss_agg_mode}")
+
+
+def policy_loss_vanilla(old_log_prob, log_prob, advantages, response_mask, loss_agg_mode="token-mean",
+                        clip_ratio_low=0.2, clip_ratio_high=0.2, clip_ratio_c=3.0,
+                        rollout_is_weights=None, global_batch_info=None):
+    """PPO clipped objective with the dual-clip floor for negative advantages.
+
+    Follows verl/trainer/ppo/core_algos.py:1159-1250 with the config fields
+    passed as plain numbers.  Returns ``(pg_loss, pg_clipfrac, ppo_kl,
+    pg_clipfrac_lower)`` as tensors (the reference turns the last three into
+    Python floats with ``.item()`` at :1245-1249).
+    """
+    assert clip_ratio_c > 1.0
+    k = torch.clamp(log_prob - old_log_prob, min=-20.0, max=20.0)
+    ratio = torch.exp(k)
+    ppo_kl = masked_mean(-k, response_mask)
+    l1 = -advantages * ratio
+    l2 = -advantages * torch.clamp(ratio, 1 - clip_ratio_low, 1 + clip_ratio_high)
+    c1 = torch.maximum(l1, l2)
+    pg_clipfrac = masked_mean(torch.gt(l2, l1).float(), response_mask)
+    l3 = -advantages * clip_ratio_c
+    c2 = torch.min(l3, c1)
+    pg_clipfrac_lower = masked_mean(torch.gt(c1, l3) * (advantages < 0).float(), response_mask)
+    losses = torch.where(advantages < 0, c2, c1)
+    if rollout_is_weights is not None:
+        losses = losses * rollout_is_weights
+    pg_loss = agg_loss(losses, response_mask, loss_agg_mode, **(global_batch_info or {}))
+    return pg_loss, pg_clipfrac, ppo_kl, pg_clipfrac_lower
+
+
+def value_loss(vpreds, returns, values, response_mask, cliprange_value, loss_agg_mode="token-mean"):
+    """Clipped value loss, verl/trainer/ppo/core_algos.py:1799-1838."""
+    clipped = clip_by_value(vpreds, values - cliprange_value, values + cliprange_value)
+    e1 = (vpreds - returns) ** 2
+    e2 = (clipped - returns) ** 2
+    vf_loss = 0.5 * agg_loss(torch.max(e1, e2), response_mask, loss_agg_mode)
+    vf_clipfrac = masked_mean(torch.gt(e2, e1).float(), response_mask)
+    return vf_loss, vf_clipfrac
+
+
+def kl_penalty_forward(logprob, ref_logprob, kind):
+    """KL estimators k1 / abs / k2 / k3, verl/trainer/ppo/core_algos.py:1868-1902."""
+    if kind in ("kl", "k1"):
+        return logprob - ref_logprob
+    if kind == "abs":
+        return (logprob - ref_logprob).abs()
+    if kind in ("mse", "k2"):
+        return 0.5 * (logprob - ref_logprob).square()
+    if kind in ("low_var_kl", "k3"):
+        d = torch.clamp(ref_logprob - logprob, min=-20, max=20)
+        return torch.clamp(torch.exp(d) - d - 1, min=-10, max=10)
+    raise NotImplementedError(kind)

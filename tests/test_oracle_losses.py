@@ -1,0 +1,169 @@
+"""Pins for oracle/losses.py: scalar Python loops written from the definitions,
+the special cases that collapse to closed forms, and the hand-derived gradients
+checked against autograd (including exact ties)."""
+import math
+
+import pytest
+import torch
+
+from oracle import losses as L
+from oracle import masked as M
+
+
+def _case(B=5, T=37, seed=0, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    old = torch.randn(B, T, generator=g, dtype=dtype) * 0.5 - 1
+    new = old + torch.randn(B, T, generator=g, dtype=dtype) * 0.3
+    adv = torch.randn(B, T, generator=g, dtype=dtype)
+    mask = (torch.rand(B, T, generator=g) < 0.7).to(dtype)
+    mask[1] = 0
+    return old, new, adv, mask
+
+
+def _scalar_policy_loss(old, new, adv, mask, lo, hi, c):
+    """Per-element loss and indicator sums by plain Python floats."""
+    n = tot = kl = cf = cfl = 0.0
+    per_elem = []
+    for o, x, a, m in zip(old.flatten().tolist(), new.flatten().tolist(), adv.flatten().tolist(),
+                          mask.flatten().tolist()):
+        k = min(max(x - o, -20.0), 20.0)
+        r = math.exp(k)
+        l1 = -a * r
+        l2 = -a * min(max(r, 1 - lo), 1 + hi)
+        c1 = max(l1, l2)
+        l3 = -a * c
+        loss = min(l3, c1) if a < 0 else c1
+        per_elem.append(loss)
+        if m:
+            n += m; tot += loss * m; kl += -k * m
+            cf += (l2 > l1) * m
+            cfl += ((c1 > l3) and (a < 0)) * m
+    return per_elem, tot, n, kl, cf, cfl
+
+
+@pytest.mark.parametrize("seed", [0, 1])
+def test_policy_loss_token_mean_against_scalar_loop(seed):
+    old, new, adv, mask = _case(seed=seed)
+    new[0, :5] = old[0, :5] + 25.0          # beyond the +-20 clamp
+    new[2, :5] = old[2, :5] + 2.0           # large ratio: dual clip for A<0
+    loss, cf, kl, cfl = L.policy_loss_vanilla(old, new, adv, mask, "token-mean", 0.2, 0.28, 3.0)
+    _, tot, n, kls, cfs, cfls = _scalar_policy_loss(old, new, adv, mask, 0.2, 0.28, 3.0)
+    assert abs(loss.item() - tot / n) < 1e-12
+    assert abs(kl.item() - kls / (n + 1e-8)) < 1e-12
+    assert abs(cf.item() - cfs / (n + 1e-8)) < 1e-12
+    assert abs(cfl.item() - cfls / (n + 1e-8)) < 1e-12
+
+
+def test_policy_loss_special_cases():
+    old, _, adv, mask = _case(seed=3)
+    # on-policy: ratio 1  =>  loss = -sum(A m)/M, kl = 0, nothing clipped
+    loss, cf, kl, cfl = L.policy_loss_vanilla(old, old.clone(), adv, mask, "token-mean")
+    assert abs(loss.item() + (adv * mask).sum().item() / mask.sum().item()) < 1e-12
+    assert kl.item() == 0 and cf.item() == 0 and cfl.item() == 0
+    # A >= 0 never dual-clips
+    _, _, _, cfl = L.policy_loss_vanilla(old, old + 3.0, adv.abs(), mask, "token-mean")
+    assert cfl.item() == 0
+    # A < 0 and a huge ratio: every valid token sits on the floor -A*c
+    loss, _, _, cfl = L.policy_loss_vanilla(old, old + 5.0, -adv.abs() - 0.1, mask, "token-mean", clip_ratio_c=3.0)
+    want = (3.0 * (adv.abs() + 0.1) * mask).sum() / mask.sum()
+    assert abs(loss.item() - want.item()) < 1e-12 and abs(cfl.item() - mask.sum().item() / (mask.sum().item() + 1e-8)) < 1e-12
+    # rollout importance weights scale the per-token loss
+    w = torch.full_like(old, 0.5)
+    a = L.policy_loss_vanilla(old, old + 0.1, adv, mask, "token-mean")[0]
+    b = L.policy_loss_vanilla(old, old + 0.1, adv, mask, "token-mean", rollout_is_weights=w)[0]
+    assert abs(b.item() - 0.5 * a.item()) < 1e-12
+    with pytest.raises(AssertionError):
+        L.policy_loss_vanilla(old, old, adv, mask, clip_ratio_c=1.0)
+
+
+def _hand_policy_grad(old, new, adv, mask, lo, hi, c):
+    """d loss / d new for token-mean, from the branch analysis (no autograd)."""
+    k = new - old
+    inside = (k >= -20) & (k <= 20)
+    r = torch.exp(k.clamp(-20, 20))
+    l1 = -adv * r
+    l2 = -adv * r.clamp(1 - lo, 1 + hi)
+    clipped_wins = l2 > l1                       # constant branch selected
+    unclipped = ~clipped_wins
+    c1 = torch.maximum(l1, l2)
+    floor_wins = (adv < 0) & (c1 > -adv * c)
+    live = unclipped & ~floor_wins & inside
+    return torch.where(live, -adv * r, torch.zeros_like(r)) * mask / mask.sum()
+
+
+def test_policy_loss_gradient_matches_branch_analysis():
+    old, new, adv, mask = _case(seed=4)
+    new[0, :6] = old[0, :6] + 1.5
+    new[3, :6] = old[3, :6] - 1.5
+    new = new.clone().requires_grad_()
+    loss = L.policy_loss_vanilla(old, new, adv, mask, "token-mean", 0.2, 0.2, 3.0)[0]
+    g, = torch.autograd.grad(loss, new)
+    assert torch.allclose(g, _hand_policy_grad(old, new.detach(), adv, mask, 0.2, 0.2, 3.0), atol=1e-14)
+
+
+def test_policy_loss_gradient_on_exact_ties():
+    # r == 1 (l1 == l2, both carry d/dlp = -A) and A == 0: torch splits max() ties 50/50, total unchanged
+    old = torch.zeros(1, 4, dtype=torch.float64)
+    new = torch.zeros(1, 4, dtype=torch.float64, requires_grad=True)
+    adv = torch.tensor([[1.0, -2.0, 0.0, 0.5]], dtype=torch.float64)
+    mask = torch.ones(1, 4, dtype=torch.float64)
+    g, = torch.autograd.grad(L.policy_loss_vanilla(old, new, adv, mask)[0], new)
+    assert torch.allclose(g, -adv / 4)
+
+
+@pytest.mark.parametrize("mode", ["token-mean", "seq-mean-token-sum", "seq-mean-token-mean", "seq-mean-token-sum-norm"])
+def test_agg_loss_modes_by_loops(mode):
+    _, x, _, mask = _case(seed=5)
+    got = L.agg_loss(x, mask, mode).item()
+    rows = [(sum(v * m for v, m in zip(xr, mr)), sum(mr)) for xr, mr in zip(x.tolist(), mask.tolist())]
+    if mode == "token-mean":
+        want = sum(s for s, _ in rows) / sum(c for _, c in rows)
+    elif mode == "seq-mean-token-sum":
+        want = sum(s for s, c in rows if c > 0) / sum(1 for _, c in rows if c > 0)
+    elif mode == "seq-mean-token-mean":
+        want = sum(s / (c + 1e-8) for s, c in rows if c > 0) / sum(1 for _, c in rows if c > 0)
+    else:
+        want = sum(s for s, _ in rows) / x.shape[-1]
+    assert abs(got - want) < 1e-12
+    # global-batch arguments
+    if mode == "token-mean":
+        assert abs(L.agg_loss(x, mask, mode, dp_size=4, batch_num_tokens=1000).item()
+                   - sum(s for s, _ in rows) / 1000 * 4) < 1e-12
+    if mode == "seq-mean-token-sum-norm":
+        assert abs(L.agg_loss(x, mask, mode, loss_scale_factor=7).item() - sum(s for s, _ in rows) / 7) < 1e-12
+    with pytest.raises(ValueError):
+        L.agg_loss(x, mask, "nope")
+
+
+def test_value_loss_against_scalar_loop_and_gradient():
+    g = torch.Generator().manual_seed(6)
+    B, T, c = 4, 29, 0.5
+    values = torch.randn(B, T, generator=g, dtype=torch.float64)
+    vpreds = (values + torch.randn(B, T, generator=g, dtype=torch.float64)).requires_grad_()
+    returns = values + torch.randn(B, T, generator=g, dtype=torch.float64)
+    mask = (torch.rand(B, T, generator=g) < 0.8).double()
+    loss, frac = L.value_loss(vpreds, returns, values, mask, c)
+    tot = cnt = cf = 0.0
+    hand = torch.zeros(B, T, dtype=torch.float64)
+    for i in range(B):
+        for t in range(T):
+            vp, R, v, m = vpreds[i, t].item(), returns[i, t].item(), values[i, t].item(), mask[i, t].item()
+            vc = max(min(vp, v + c), v - c)
+            e1, e2 = (vp - R) ** 2, (vc - R) ** 2
+            tot += max(e1, e2) * m; cnt += m; cf += (e2 > e1) * m
+            inside = v - c < vp < v + c
+            hand[i, t] = (vp - R) * m if (inside or e1 > e2) else 0.0
+    assert abs(loss.item() - 0.5 * tot / cnt) < 1e-12 and abs(frac.item() - cf / (cnt + 1e-8)) < 1e-12
+    gr, = torch.autograd.grad(loss, vpreds)
+    assert torch.allclose(gr, hand / cnt, atol=1e-14)
+
+
+def test_kl_estimators():
+    a = torch.tensor([-1.0, -2.0, -0.5], dtype=torch.float64)
+    b = torch.tensor([-1.5, -1.0, -0.5], dtype=torch.float64)
+    assert torch.equal(L.kl_penalty_forward(a, b, "kl"), a - b)
+    assert torch.equal(L.kl_penalty_forward(a, b, "abs"), (a - b).abs())
+    assert torch.allclose(L.kl_penalty_forward(a, b, "mse"), 0.5 * (a - b) ** 2)
+    d = b - a
+    assert torch.allclose(L.kl_penalty_forward(a, b, "low_var_kl"), torch.exp(d) - d - 1)
+    assert L.kl_penalty_forward(torch.tensor([0.0]), torch.tensor([30.0]), "k3").item() == 10.0   # clamp at 10

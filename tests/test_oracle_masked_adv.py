@@ -1,0 +1,203 @@
+"""Pins for oracle/masked.py and oracle/advantages.py: the reference-held
+vectors (masked_mean cases, group_mean_std known answer, the multi-turn GAE
+fixture, the GRPO loop==vectorised grids with the reference's generators),
+closed forms and fp64 brute force."""
+import math
+import random
+import uuid
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import advantages as A
+from oracle import masked as M
+
+
+# ---- masked_* ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("value,mask,want", [
+    ([1.0, 2.0, 3.0, 4.0], [1, 0, 0, 1], 2.5),
+    ([1.0, 2.0, float("nan"), 4.0], [1, 0, 0, 1], 2.5),
+    ([1.0, 2.0, float("nan"), 4.0], [1, 0, 1, 0], float("nan")),
+])
+def test_masked_mean_reference_vectors(value, mask, want):
+    # literals of tests/utils/test_torch_functional.py:60-71 (int64 mask, as there)
+    got = M.masked_mean(torch.tensor(value), torch.tensor(mask))
+    assert torch.allclose(got, torch.tensor(want), equal_nan=True)
+
+
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.int64, torch.bool])
+def test_masked_var_and_whiten_against_torch_var(mdtype):
+    g = torch.Generator().manual_seed(0)
+    v = torch.randn(7, 33, generator=g) * 3 + 1.5
+    m = (torch.rand(7, 33, generator=g) < 0.6)
+    sel = v[m]
+    mm = m.to(mdtype)
+    assert torch.allclose(M.masked_mean(v, mm), sel.mean(), rtol=1e-6)
+    assert torch.allclose(M.masked_var(v, mm), sel.var(unbiased=True), rtol=1e-5)
+    assert torch.allclose(M.masked_var(v, mm, unbiased=False), sel.var(unbiased=False), rtol=1e-5)
+    w = M.masked_whiten(v, mm)
+    assert abs(w[m].mean().item()) < 1e-6 and abs(w[m].var(unbiased=True).item() - 1) < 1e-5
+    w2 = M.masked_whiten(v, mm, shift_mean=False)
+    assert torch.allclose(w2 - w, sel.mean().expand_as(w), atol=1e-6)
+    # every element is transformed, masked or not
+    assert torch.allclose(w, (v - sel.mean()) * torch.rsqrt(sel.var() + 1e-8), rtol=1e-5, atol=1e-6)
+
+
+def test_masked_edge_cases():
+    v = torch.tensor([[1.0, 2.0], [3.0, 4.0]])
+    zero = torch.zeros(2, 2)
+    assert M.masked_mean(v, zero).item() == 0.0                     # 0 / 1e-8
+    with pytest.raises(ValueError):
+        M.masked_var(v, zero)
+    with pytest.raises(ValueError):
+        M.masked_var(v, torch.tensor([[1.0, 0.0], [0.0, 0.0]]))
+    # weighted float mask: where() keeps, then the weight multiplies
+    w = torch.tensor([[0.5, 0.0], [2.0, 1.0]])
+    assert M.masked_sum(v, w).item() == 0.5 * 1 + 2 * 3 + 4
+    assert torch.equal(M.masked_sum(v, torch.ones(2, 2), axis=-1), torch.tensor([3.0, 7.0]))
+    assert torch.equal(M.masked_mean(v, torch.tensor([[1, 0], [0, 0]]), axis=-1), torch.tensor([1.0, 0.0]))
+
+
+def test_entropy_and_logprob_definitions():
+    z = torch.tensor([[0.0, 0.0, 0.0, 0.0], [10.0, 0.0, 0.0, 0.0]])
+    ent = M.entropy_from_logits(z)
+    assert abs(ent[0].item() - math.log(4)) < 1e-6
+    p = torch.softmax(z[1].double(), -1)
+    assert abs(ent[1].item() - float(-(p * p.log()).sum())) < 1e-5
+    lp = M.logprobs_from_logits(z, torch.tensor([2, 0]))
+    assert abs(lp[0].item() + math.log(4)) < 1e-6 and abs(lp[1].item() - float(p[0].log())) < 1e-6
+    x = torch.tensor([1.0, 5.0, -3.0])
+    assert torch.equal(M.clip_by_value(x, torch.tensor([2.0, 2.0, -1.0]), torch.tensor([3.0, 4.0, 0.0])),
+                       torch.tensor([2.0, 4.0, -1.0]))
+
+
+# ---- GAE --------------------------------------------------------------------------------------
+def _raw_gae(r, v, m, gamma, lam):
+    adv, ret = A.gae_raw(r, v, m, gamma, lam)
+    assert torch.equal(ret, adv + v)
+    return adv
+
+
+@pytest.mark.parametrize("B,L", [(1, 1), (3, 7), (3, 64)])
+@pytest.mark.parametrize("gamma,lam", [(1.0, 1.0), (1.0, 0.95), (0.95, 0.5)])
+def test_gae_against_fp64_brute_force(B, L, gamma, lam):
+    g = torch.Generator().manual_seed(B * 100 + L)
+    r = torch.randn(B, L, generator=g, dtype=torch.float64)
+    v = torch.randn(B, L, generator=g, dtype=torch.float64)
+    m = (torch.rand(B, L, generator=g) < 0.7).double()
+    if B > 1:
+        m[1] = 0                                   # an all-masked row
+    got = _raw_gae(r, v, m, gamma, lam)
+    want = torch.tensor(A.gae_brute_force_fp64(r.tolist(), v.tolist(), m.tolist(), gamma, lam), dtype=torch.float64)
+    assert torch.allclose(got, want, rtol=1e-12, atol=1e-12)
+    got32 = _raw_gae(r.float(), v.float(), m.float(), gamma, lam)
+    assert torch.allclose(got32.double(), want, rtol=1e-5, atol=1e-5)
+
+
+def test_gae_gamma_lambda_one_is_reverse_cumsum_of_rewards():
+    g = torch.Generator().manual_seed(1)
+    r = torch.randn(4, 50, generator=g, dtype=torch.float64)
+    v = torch.randn(4, 50, generator=g, dtype=torch.float64)
+    m = torch.ones(4, 50, dtype=torch.float64)
+    _, ret = A.gae_advantage_return(r, v, m, 1.0, 1.0)
+    assert torch.allclose(ret, torch.flip(torch.cumsum(torch.flip(r, [1]), 1), [1]), atol=1e-12)
+
+
+def test_gae_multi_turn_fixture_invariance():
+    # rewards / mask literals and the torch.equal assertion of
+    # tests/trainer/ppo/test_core_algos_on_cpu.py:143-197
+    random.seed(0)
+    gamma, lam = random.uniform(0.0, 1.0), random.uniform(0.0, 1.0)
+    rewards = torch.tensor([[0.0, 0.0, 0.1, 0.1, 0.1, 0.0, 0.0, 0.1, 1.0, 0.0, 0.0]])
+    v1 = torch.tensor([[random.uniform(-100.0, 100.0), random.random(), 4.0, 5.0, 6.0,
+                        random.uniform(-100.0, 0), random.random(), 7.0, 9.0, 0.0, 0.0]])
+    v2 = torch.tensor([[random.random(), random.uniform(-100.0, 100.0), 4.0, 5.0, 6.0,
+                        random.random(), random.uniform(0.0, 100.0), 7.0, 9.0, 0.0, 0.0]])
+    mask = torch.tensor([[0, 0, 1, 1, 1, 0, 0, 1, 1, 0, 0]], dtype=torch.float)
+    a1, r1 = A.gae_advantage_return(rewards, v1, mask, gamma, lam)
+    a2, r2 = A.gae_advantage_return(rewards, v2, mask, gamma, lam)
+    assert torch.equal(a1, a2) and torch.equal(r1 * mask, r2 * mask)
+    # masked positions carry the state of the next valid token; trailing padding is 0 before whitening
+    raw, _ = A.gae_raw(rewards, v1, mask, gamma, lam)
+    assert raw[0, 0] == raw[0, 1] == raw[0, 2] and raw[0, 5] == raw[0, 6] == raw[0, 7]
+    assert raw[0, 9] == 0 and raw[0, 10] == 0
+
+
+# ---- GRPO -------------------------------------------------------------------------------------
+def _make_group_index(batch_size, num_groups):
+    counts = [2] * num_groups
+    for _ in range(batch_size - 2 * num_groups):
+        counts[random.randrange(num_groups)] += 1
+    index = []
+    for gid, c in enumerate(counts):
+        index.extend([gid] * c)
+    random.shuffle(index)
+    return np.asarray(index, dtype=np.int64)
+
+
+def _rand_mask(batch_size, seq_len):
+    mask = torch.randint(0, 2, (batch_size, seq_len), dtype=torch.int64).float()
+    rows = (mask.sum(dim=-1) == 0).nonzero(as_tuple=True)[0]
+    if len(rows) > 0:
+        mask[rows, -1] = 1.0
+    return mask
+
+
+@pytest.mark.parametrize("batch_size,seq_len,num_groups,seed", [(64, 128, 5, 0), (128, 256, 8, 1), (512, 512, 10, 2)])
+def test_grpo_loop_equals_vectorised_reference_grid(batch_size, seq_len, num_groups, seed):
+    # grid and tolerance of tests/trainer/ppo/test_core_algos_on_cpu.py:262-313
+    torch.manual_seed(seed); random.seed(seed); np.random.seed(seed)
+    index = _make_group_index(batch_size, num_groups)
+    mask = _rand_mask(batch_size, seq_len)
+    rewards = torch.randn(batch_size, seq_len) * mask
+    a1, r1 = A.grpo_outcome_advantage(rewards, mask, index)
+    a2, r2 = A.grpo_vectorized_outcome_advantage(rewards, mask, index)
+    assert a1.shape == (batch_size, seq_len) and a1 is r1 and a2 is r2
+    assert torch.allclose(a1, a2, rtol=1e-5, atol=1e-6)
+
+
+def test_group_mean_std_reference_known_answer():
+    # tests/utils/test_groupwise.py:51-65
+    mean_g, std_g, cnt_g = A.group_mean_std(torch.tensor([1.0, 2.0, 3.0]), A.as_torch_index([0, 1, 0]))
+    assert torch.allclose(mean_g, torch.tensor([2.0, 0.0])) and torch.allclose(cnt_g, torch.tensor([2.0, 1.0]))
+    assert std_g[1].item() == 1.0 and abs(std_g[0].item() - 2 ** 0.5) < 1e-6
+    e = A.group_mean_std(torch.tensor([]), torch.tensor([], dtype=torch.long))
+    assert all(t.numel() == 0 for t in e)
+
+
+def test_as_torch_index_cases():
+    g = A.as_torch_index(["a", "b", "a", "c", "0042", 42])
+    assert g.tolist()[4] != g.tolist()[5] and len(torch.unique(g)) == 5
+    assert A.as_torch_index(np.array([3, 3, 7])).tolist() == [3, 3, 7]
+    assert A.as_torch_index(torch.tensor([1.0, 2.0, 1.0])).tolist() == [1, 2, 1]
+    assert A.as_torch_index(["5", "6", "5"]).tolist() == [5, 6, 5]
+    ids = [str(uuid.UUID(int=i)) for i in (9, 4, 9, 1)]
+    g = A.as_torch_index(np.array(ids, dtype=object))
+    assert g[0] == g[2] and len(torch.unique(g)) == 3
+
+
+def test_grpo_toy_input_by_hand():
+    # input of tests/trainer/config/test_algo_config_on_cpu.py:187-197; answer worked by hand:
+    # scores (1.5, 3.0 | 0.7, 2.3); unbiased std of a pair = |a-b|/sqrt(2)
+    rewards = torch.tensor([[1.0, 0.5, 0.0], [2.0, 1.0, 0.0], [0.5, 0.2, 0.0], [1.5, 0.8, 0.0]])
+    mask = torch.ones(4, 3)
+    adv, _ = A.grpo_outcome_advantage(rewards, mask, np.array([0, 0, 1, 1]))
+    s0, s1 = 1.5 / math.sqrt(2), 1.6 / math.sqrt(2)
+    want = torch.tensor([-0.75 / (s0 + 1e-6), 0.75 / (s0 + 1e-6), -0.8 / (s1 + 1e-6), 0.8 / (s1 + 1e-6)])
+    assert torch.allclose(adv, want[:, None].expand(4, 3), rtol=1e-5)
+    adv2, _ = A.grpo_outcome_advantage(rewards, mask, np.array([0, 0, 1, 1]), norm_adv_by_std_in_grpo=False)
+    assert torch.allclose(adv2[:, 0], torch.tensor([-0.75, 0.75, -0.8, 0.8]), rtol=1e-5)
+
+
+def test_grpo_singletons_strings_equal_scores_and_unmasked_sum():
+    rewards = torch.tensor([[1.0, 2.0], [3.0, 0.0], [3.0, 0.0], [5.0, 5.0]])
+    mask = torch.tensor([[1.0, 0.0], [1.0, 1.0], [1.0, 1.0], [0.0, 1.0]])
+    index = np.array(["u-a", "u-b", "u-b", "u-c"], dtype=object)
+    adv, _ = A.grpo_outcome_advantage(rewards, mask, index)
+    # singleton: (s - 0)/(1 + eps), score counts the reward at the masked position too
+    assert torch.allclose(adv[0], torch.tensor([3.0 / (1 + 1e-6), 0.0]))
+    assert torch.equal(adv[1], torch.zeros(2)) and torch.equal(adv[2], torch.zeros(2))   # equal scores -> 0
+    assert torch.allclose(adv[3], torch.tensor([0.0, 10.0 / (1 + 1e-6)]))
+    adv_v, _ = A.grpo_vectorized_outcome_advantage(rewards, mask, index)
+    assert torch.allclose(adv, adv_v, rtol=1e-5, atol=1e-6)
