@@ -1,0 +1,186 @@
+/* verl_amd.h -- C ABI of libverl_amd.so: MI355X (gfx950) kernels for verl's per-token
+ * policy-math path.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its name ends in _host;
+ *   - every function is asynchronous on `stream` (a hipStream_t passed as void*), allocates
+ *     nothing and keeps no state between calls: scratch comes from the caller through
+ *     (workspace, workspace_bytes); the matching *_workspace_bytes() gives the size needed;
+ *   - return value: 0 on success, a negative VAMD_E* code otherwise; vamd_last_error() returns a
+ *     thread-local description of the last failure on the calling thread;
+ *   - "mask" arguments come with a VAMD_MASK_* code naming their element type; the value used is
+ *     (float)mask[i], and mask[i] != 0 decides membership, exactly as
+ *     masked_sum does in the reference (verl/utils/torch_functional.py:283-284).
+ *
+ * Each entry point cites the reference interface it stands behind (paths relative to the
+ * reference tree).
+ */
+#ifndef VERL_AMD_H_
+#define VERL_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VAMD_OK 0
+#define VAMD_EINVAL (-1)    /* bad shape / null pointer / unsupported option */
+#define VAMD_EWORKSPACE (-2) /* workspace missing or too small */
+#define VAMD_EHIP (-3)      /* a HIP runtime call failed; see vamd_last_error() */
+
+#define VAMD_MASK_F32 0
+#define VAMD_MASK_I64 1
+#define VAMD_MASK_U8 2 /* torch.bool and torch.uint8 */
+#define VAMD_MASK_I32 3
+
+/* loss_agg_mode of agg_loss (verl/trainer/ppo/core_algos.py:1025-1080) */
+#define VAMD_AGG_TOKEN_MEAN 0
+#define VAMD_AGG_SEQ_MEAN_TOKEN_SUM 1
+#define VAMD_AGG_SEQ_MEAN_TOKEN_MEAN 2
+#define VAMD_AGG_SEQ_MEAN_TOKEN_SUM_NORM 3
+
+int vamd_abi_version(void);
+const char* vamd_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Fused vocab-projection log-prob / entropy head.
+ * Replaces kernels.efficient_entropy_forward / efficient_entropy_backward behind
+ * LinearCrossEntropy (verl/utils/kernel/linear_cross_entropy.py:40-116,
+ * verl/utils/kernel/kernels.py:563-753 and :1512-1723).
+ *
+ *   hidden [n_tokens, hidden_size] bf16 row-major, weight [vocab, hidden_size] bf16 row-major,
+ *   labels [n_tokens] int64 in [0, vocab).  hidden_size % 128 == 0 (kernels.py:593),
+ *   vocab % 8 == 0.
+ *   z = hidden . weight^T * rcp_temperature ; logprobs = z[label] - lse(z) ;
+ *   entropy = lse(z) - sum softmax(z) z.
+ *   lse[n] and mean_z[n] (= sum softmax(z) z) are saved for the backward pass in place of the
+ *   reference's (maximum, accumulate, entropy_b) triple.
+ */
+size_t vamd_lce_forward_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab);
+int vamd_lce_forward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
+                     int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs, float* entropy,
+                     float* lse, float* mean_z, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Backward: d_logits = [g_lp (onehot - p) - g_ent p (z - mean_z)] * rcp_temperature is formed
+ * tile by tile from recomputed logits, never as a whole; d_hidden = d_logits . weight,
+ * d_weight = d_logits^T . hidden, both accumulated in fp32 and rounded to bf16 once.
+ *   d_logprobs [n] fp32 or NULL (treated as zeros);
+ *   d_entropy  [n] fp32 or NULL, in which case the constant d_entropy_scalar is used for every
+ *   token (an entropy-bonus coefficient folded into the backward pass);
+ *   d_hidden [n, hidden_size] bf16 out; d_weight [vocab, hidden_size] bf16 out.
+ *   accumulate_d_weight != 0 adds into d_weight instead of overwriting it (token-chunked use).
+ * vocab_chunk = 0 lets the library choose how many vocabulary columns of d_logits are staged
+ * at a time (the workspace holds one [n_pad, vocab_chunk] bf16 panel plus an fp32 d_hidden
+ * accumulator); pass the same value to the workspace query.
+ */
+size_t vamd_lce_backward_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab, int64_t vocab_chunk);
+int vamd_lce_backward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
+                      int64_t hidden_size, int64_t vocab, float rcp_temperature, const float* lse,
+                      const float* mean_z, const float* d_logprobs, const float* d_entropy, float d_entropy_scalar,
+                      void* d_hidden, void* d_weight, int accumulate_d_weight, int64_t vocab_chunk, void* workspace,
+                      size_t workspace_bytes, void* stream);
+
+/* Benchmark aid (no counterpart in the reference): with timing enabled on the calling thread,
+ * every head kernel launch is bracketed by HIP events on its stream.  vamd_lce_timing_collect
+ * waits for them and adds up milliseconds and launch counts per kernel, indexed
+ * 0 forward, 1 merge, 2 logit recompute, 3 d_hidden GEMM, 4 d_weight GEMM (arrays of 5). */
+int vamd_lce_timing_enable(int on);
+int vamd_lce_timing_collect(double* ms_by_kernel_host, int64_t* launches_by_kernel_host);
+
+/* ------------------------------------------------------------------------------------------
+ * Masked reductions: verl/utils/torch_functional.py:266-339.
+ * vamd_masked_moments writes out[0..3] (double): sum(m), sum(where(m,v,0)*m),
+ * sum(where(m,v,0)^2*m), count(m != 0)  -- the sufficient statistics of masked_sum / masked_mean /
+ * masked_var.  rows x cols elements; with per_row != 0 it writes 4 doubles per row instead
+ * (masked_sum / masked_mean with axis=-1).
+ */
+size_t vamd_masked_moments_workspace_bytes(int64_t rows, int64_t cols);
+int vamd_masked_moments(const float* values, const void* mask, int mask_dtype, int64_t rows, int64_t cols,
+                        int per_row, double* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* out[i] = (values[i] - stats[0]) * stats[1] + stats[2], stats being three DEVICE floats
+ * (mean, rsqrt(var + 1e-8), re-added mean or 0): the elementwise half of masked_whiten
+ * (torch_functional.py:335-339).  vamd_whiten_stats fills stats from vamd_masked_moments'
+ * output following masked_var's unbiased rule; flags_host receives nothing -- the M in {0,1}
+ * error of masked_var (:311-316) is raised by the host wrapper from the moments. */
+int vamd_whiten_stats(const double* moments, int shift_mean, float* stats, void* stream);
+int vamd_affine_by_stats(const float* values, const float* stats, int64_t n, float* out, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * GAE: compute_gae_advantage_return (verl/trainer/ppo/core_algos.py:214-262).
+ * rewards, values [B, L] fp32, mask [B, L]; advantages (whitened) and returns [B, L] fp32 out.
+ * The recurrence is evaluated as a chunked associative scan of affine maps; masked steps carry
+ * the state.  whiten == 0 leaves the raw advantages (the value before :261).
+ * moments_out (4 doubles, may be NULL) receives the masked moments of the raw advantages so the
+ * host can raise masked_var's M in {0,1} error.
+ */
+size_t vamd_gae_workspace_bytes(int64_t batch, int64_t length);
+int vamd_gae(const float* rewards, const float* values, const void* mask, int mask_dtype, int64_t batch,
+             int64_t length, float gamma, float lam, int whiten, float* advantages, float* returns,
+             double* moments_out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * GRPO: compute_grpo_outcome_advantage (core_algos.py:266-330) and its vectorised twin
+ * (:333-357) with group_mean_std (verl/utils/groupwise.py:163-223).
+ * group_ids [B] int64, contiguous ids in [0, n_groups) (the host factorises arbitrary labels as
+ * groupwise.as_torch_index does).  std_mode 0: unbiased torch.std (loop form); 1:
+ * sqrt(clamp(var, min=eps)) (vectorised form).  scores_out [B] (may be NULL) receives the
+ * normalised scalar per response.
+ */
+size_t vamd_grpo_workspace_bytes(int64_t batch, int64_t length, int64_t n_groups);
+int vamd_grpo_advantage(const float* rewards, const void* mask, int mask_dtype, const int64_t* group_ids,
+                        int64_t batch, int64_t length, int64_t n_groups, float epsilon, int norm_by_std,
+                        int std_mode, float* advantages, float* scores_out, void* workspace,
+                        size_t workspace_bytes, void* stream);
+
+/* group_mean_std (verl/utils/groupwise.py:163-223): mean/std/count per group, singleton -> (0,1). */
+int vamd_group_mean_std(const float* scores, const int64_t* group_ids, int64_t n, int64_t n_groups, float eps,
+                        float* mean, float* std, float* count, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * agg_loss (core_algos.py:1025-1080), forward and backward.
+ * out_loss: 1 device float.  coef_out [rows] floats: d loss / d loss_mat[i][t] = coef_out[i] *
+ * (float)mask[i][t]; the backward entry point multiplies by the upstream scalar *d_loss.
+ * batch_num_tokens / global_batch_size / loss_scale_factor < 0 mean "None" in the reference.
+ */
+size_t vamd_agg_loss_workspace_bytes(int64_t rows, int64_t cols);
+int vamd_agg_loss_forward(const float* loss_mat, const void* mask, int mask_dtype, int64_t rows, int64_t cols,
+                          int mode, double dp_size, double batch_num_tokens, double global_batch_size,
+                          double loss_scale_factor, float* out_loss, float* coef_out, void* workspace,
+                          size_t workspace_bytes, void* stream);
+int vamd_agg_loss_backward(const float* d_loss, const float* coef, const void* mask, int mask_dtype, int64_t rows,
+                           int64_t cols, float* d_loss_mat, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * compute_policy_loss_vanilla (core_algos.py:1159-1250): clipped + dual-clip PPO objective.
+ * Forward (one pass over old_log_prob, log_prob, advantages, mask [rows, cols]) writes
+ *   out[0] = pg_loss, out[1] = pg_clipfrac, out[2] = ppo_kl, out[3] = pg_clipfrac_lower
+ * and, when grad_unscaled != NULL, g[i][t] = d(per-token loss)/d log_prob * (float)mask (the
+ * row coefficient of agg_loss is applied in the backward entry point, which writes
+ * d_log_prob = g * coef[row] * *d_loss).  is_weights may be NULL.
+ */
+size_t vamd_policy_loss_workspace_bytes(int64_t rows, int64_t cols);
+int vamd_policy_loss_forward(const float* old_log_prob, const float* log_prob, const float* advantages,
+                             const void* mask, int mask_dtype, const float* is_weights, int64_t rows, int64_t cols,
+                             float clip_low, float clip_high, float clip_c, int mode, double dp_size,
+                             double batch_num_tokens, double global_batch_size, double loss_scale_factor,
+                             float* out, float* grad_unscaled, float* coef_out, void* workspace,
+                             size_t workspace_bytes, void* stream);
+int vamd_scale_rows(const float* g, const float* coef, const float* d_loss, float extra_scale, int64_t rows,
+                    int64_t cols, float* out, void* stream);
+
+/* compute_value_loss (core_algos.py:1799-1838): out[0] = vf_loss, out[1] = vf_clipfrac;
+ * grad_unscaled as above (d per-token loss / d vpreds * mask, before the 0.5 and agg_loss row
+ * coefficient, which vamd_scale_rows applies). */
+size_t vamd_value_loss_workspace_bytes(int64_t rows, int64_t cols);
+int vamd_value_loss_forward(const float* vpreds, const float* returns, const float* values, const void* mask,
+                            int mask_dtype, int64_t rows, int64_t cols, float cliprange_value, int mode,
+                            float* out, float* grad_unscaled, float* coef_out, void* workspace,
+                            size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VERL_AMD_H_ */

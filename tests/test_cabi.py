@@ -1,0 +1,99 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every symbol that
+include/verl_amd.h declares, answers its size queries, and the host wrappers refuse to run
+without a GPU instead of falling back."""
+import os
+import re
+
+import pytest
+import torch
+
+from verl_amd import _cabi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "verl_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(vamd_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_cabi.lib_path()):
+        from verl_amd.csrc.build import build
+        build(verbose=False)
+    return _cabi.load_library()
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    declared = _declared_symbols()
+    assert len(declared) >= 20
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/verl_amd.h but not exported"
+    assert sorted(_cabi.SIGNATURES) == declared, "ctypes prototypes and header disagree"
+    assert lib.vamd_abi_version() == 1
+
+
+def test_workspace_queries(lib):
+    assert lib.vamd_lce_forward_workspace_bytes(16384, 3584, 152064) > 0
+    assert lib.vamd_lce_forward_workspace_bytes(0, 3584, 152064) == 0
+    n, h, v = 16384, 3584, 152064
+    full = lib.vamd_lce_backward_workspace_bytes(n, h, v, 0)
+    assert full < 1 << 30                                         # d_logits panel + fp32 d_hidden accumulator
+    one = lib.vamd_lce_backward_workspace_bytes(256, 128, 1024, 0)
+    assert one == 256 * 1024 * 2                                  # a single panel, no accumulator
+    assert lib.vamd_masked_moments_workspace_bytes(512, 4096) == 512 * 4 * 8
+    assert lib.vamd_policy_loss_workspace_bytes(512, 4097) == 512 * 2 * 5 * 8
+    assert lib.vamd_gae_workspace_bytes(512, 4096) >= 512 * 4 * 8
+
+
+def test_argument_errors_are_reported_without_touching_the_gpu(lib):
+    rc = lib.vamd_lce_forward(None, None, None, 16, 100, 128, 1.0, None, None, None, None, None, 0, None)
+    assert rc == -1 and b"multiple of 128" in lib.vamd_last_error()
+    rc = lib.vamd_policy_loss_forward(None, None, None, None, 0, None, 4, 4, 0.2, 0.2, 3.0, 0, 1.0, -1.0, -1.0, -1.0,
+                                      None, None, None, None, 0, None)
+    assert rc == -1 and b"null pointer" in lib.vamd_last_error()
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="needs a machine without a GPU")
+def test_no_cpu_fallback():
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.utils import torch_functional as F
+    x = torch.ones(2, 4)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        F.masked_mean(x, x)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        CA.compute_gae_advantage_return(x, x, x, 1.0, 1.0)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        CA.agg_loss(x, x, "token-mean")
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(RuntimeError, match="is missing"):
+        _cabi.load_library(str(tmp_path / "libverl_amd.so"))
+
+
+def test_registries_and_host_logic_without_gpu():
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.utils.groupwise import as_torch_index, contiguous_group_ids
+    from verl_amd.utils.kernel.linear_cross_entropy import get_entropy_reduction_enum_number
+    assert CA.get_adv_estimator_fn("gae") is CA.compute_gae_advantage_return
+    assert CA.get_adv_estimator_fn(CA.AdvantageEstimator.GRPO) is CA.compute_grpo_outcome_advantage
+    assert CA.get_policy_loss_fn("vanilla") is CA.compute_policy_loss_vanilla
+    with pytest.raises(ValueError, match="Unsupported loss mode"):
+        CA.get_policy_loss_fn("gspo-not-here")
+    with pytest.raises(ValueError, match="Unknown advantage estimator"):
+        CA.get_adv_estimator_fn("nope")
+    with pytest.raises(ValueError, match="already been registered"):
+        CA.register_adv_est("grpo")(lambda: None)
+    with pytest.raises(ValueError, match="Invalid loss_agg_mode"):
+        CA.agg_loss(torch.ones(1, 1), torch.ones(1, 1), "bad-mode")
+    assert [get_entropy_reduction_enum_number(r) for r in ("none", "sum", "mean")] == [0, 1, 2]
+    with pytest.raises(ValueError, match="Invalid reduction"):
+        get_entropy_reduction_enum_number("max")
+    g = as_torch_index(["a", "b", "a", "c", "0042", 42])
+    assert g.tolist()[4] != g.tolist()[5] and len(torch.unique(g)) == 5
+    assert as_torch_index(["5", "6", "5"]).tolist() == [5, 6, 5]
+    ids, G = contiguous_group_ids([10, 10, 7, 99])
+    assert G == 3 and ids.tolist() == [1, 1, 0, 2]

@@ -1,0 +1,382 @@
+"""GPU parity of the PPO / GRPO policy math against the oracle (oracle/*.py, CPU torch).
+
+Tolerance (north star): advantages and losses within rtol 1e-5 in fp32; as in the reference's own
+equivalence tests an absolute floor of 1e-6 accompanies it (values that cancel to ~0).  Mask and
+index handling is checked bit-exactly (zeros stay exact zeros, group membership by label).
+"""
+import random
+import types
+import uuid
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-5, 1e-6
+
+
+def _close(got, want, rtol=RTOL, atol=ATOL, what=""):
+    got = got.detach().float().cpu(); want = want.detach().float().cpu()
+    ok = torch.allclose(got, want, rtol=rtol, atol=atol, equal_nan=True)
+    if not ok:
+        err = (got - want).abs()
+        i = err.argmax()
+        raise AssertionError(f"{what}: max err {err.max().item():.3e} at {i.item()} "
+                             f"(got {got.flatten()[i].item():.8g}, want {want.flatten()[i].item():.8g})")
+
+
+def _prefix_mask(B, L, g, lo=1):
+    lens = torch.randint(lo, L + 1, (B,), generator=g)
+    return (torch.arange(L)[None, :] < lens[:, None]).float(), lens
+
+
+def _cfg(**kw):
+    base = dict(clip_ratio=0.2, clip_ratio_low=None, clip_ratio_high=None, clip_ratio_c=3.0, global_batch_info={})
+    base.update(kw)
+    ns = types.SimpleNamespace(**base)
+    ns.get = lambda k, d=None: getattr(ns, k, d)
+    return ns
+
+
+# ---- masked_* -----------------------------------------------------------------------------------
+@pytest.mark.parametrize("value,mask,want", [
+    ([1.0, 2.0, 3.0, 4.0], [1, 0, 0, 1], 2.5),
+    ([1.0, 2.0, float("nan"), 4.0], [1, 0, 0, 1], 2.5),
+    ([1.0, 2.0, float("nan"), 4.0], [1, 0, 1, 0], float("nan")),
+])
+def test_masked_mean_reference_vectors(dev, value, mask, want):
+    from verl_amd.utils.torch_functional import masked_mean
+    for device in ("cpu", dev):
+        got = masked_mean(torch.tensor(value, device=device), torch.tensor(mask, device=device))
+        assert got.device.type == torch.device(device).type
+        assert torch.allclose(got.cpu(), torch.tensor(want), equal_nan=True)
+
+
+@pytest.mark.parametrize("shape", [(7, 33), (64, 4096), (3, 5000), (1, 100003)])
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.int64, torch.bool, torch.int32])
+def test_masked_reductions(dev, shape, mdtype):
+    from verl_amd.utils import torch_functional as F
+    g = torch.Generator().manual_seed(shape[1])
+    v = torch.randn(*shape, generator=g) * 3 + 1.5
+    m = (torch.rand(*shape, generator=g) < 0.6).to(mdtype)
+    vd, md = v.to(dev), m.to(dev)
+    _close(F.masked_sum(vd, md), O.masked_sum(v, m), rtol=1e-5, atol=1e-3, what="masked_sum")
+    _close(F.masked_mean(vd, md), O.masked_mean(v, m), what="masked_mean")
+    _close(F.masked_sum(vd, md, axis=-1), O.masked_sum(v, m, axis=-1), atol=1e-4, what="masked_sum axis")
+    _close(F.masked_mean(vd, md, axis=-1), O.masked_mean(v, m, axis=-1), what="masked_mean axis")
+    _close(F.masked_var(vd, md), O.masked_var(v, m), what="masked_var")
+    _close(F.masked_var(vd, md, unbiased=False), O.masked_var(v, m, unbiased=False), what="masked_var biased")
+    _close(F.masked_whiten(vd, md), O.masked_whiten(v, m), atol=1e-5, what="masked_whiten")
+    _close(F.masked_whiten(vd, md, shift_mean=False), O.masked_whiten(v, m, shift_mean=False), atol=1e-5,
+           what="masked_whiten keep mean")
+
+
+def test_masked_edge_cases(dev):
+    from verl_amd.utils import torch_functional as F
+    v = torch.tensor([[1.0, 2.0], [3.0, 4.0]], device=dev)
+    zero = torch.zeros(2, 2, device=dev)
+    assert F.masked_mean(v, zero).item() == 0.0
+    with pytest.raises(ValueError):
+        F.masked_var(v, zero)
+    with pytest.raises(ValueError):
+        F.masked_whiten(v, torch.tensor([[1.0, 0.0], [0.0, 0.0]], device=dev))
+    w = torch.tensor([[0.5, 0.0], [2.0, 1.0]], device=dev)                # weighted float mask
+    assert F.masked_sum(v, w).item() == 0.5 * 1 + 2 * 3 + 4
+    assert torch.equal(F.masked_mean(v, torch.tensor([[1, 0], [0, 0]], device=dev), axis=-1).cpu(),
+                       torch.tensor([1.0, 0.0]))
+
+
+# ---- GAE ----------------------------------------------------------------------------------------
+@pytest.mark.parametrize("B,L", [(1, 2), (3, 7), (3, 64), (5, 1023), (4, 1024), (3, 1025), (2, 4100), (16, 4096)])
+@pytest.mark.parametrize("gamma,lam", [(1.0, 0.95), (0.99, 0.9), (0.95, 0.5)])
+def test_gae_against_oracle(dev, B, L, gamma, lam):
+    from verl_amd.trainer.ppo.core_algos import compute_gae_advantage_return
+    g = torch.Generator().manual_seed(B * 10000 + L)
+    r = torch.randn(B, L, generator=g)
+    v = torch.randn(B, L, generator=g)
+    m = (torch.rand(B, L, generator=g) < 0.7).float()          # holes everywhere (multi-turn style)
+    m[0, -1] = 1; m[0, 0] = 1
+    if B > 2:
+        m[1] = 0                                                # an all-masked row
+        m[2, L // 2:] = 0                                       # trailing padding
+    adv, ret = compute_gae_advantage_return(r.to(dev), v.to(dev), m.to(dev), gamma, lam)
+    want_adv, want_ret = O.gae_advantage_return(r, v, m, gamma, lam)
+    _close(ret, want_ret, atol=1e-5, what="returns")
+    _close(adv, want_adv, atol=1e-5, what="advantages")
+    # int64 mask and CPU inputs give the same numbers, on the caller's device
+    adv2, ret2 = compute_gae_advantage_return(r, v, m.long(), gamma, lam)
+    assert adv2.device.type == "cpu" and torch.equal(adv2, adv.cpu()) and torch.equal(ret2, ret.cpu())
+
+
+def test_gae_gamma_lambda_one_long_rows_vs_fp64(dev):
+    """gamma = lam = 1 turns the recurrence into a 4096-term running sum, where the reference's
+    sequential fp32 loop itself carries ~1e-4 of rounding noise; the kernel is therefore held to
+    the fp64 evaluation of the same recurrence (and shown to be no further from it than the fp32
+    oracle is)."""
+    from verl_amd.trainer.ppo.core_algos import compute_gae_advantage_return
+    g = torch.Generator().manual_seed(0)
+    B, L = 8, 4096
+    r = torch.randn(B, L, generator=g); v = torch.randn(B, L, generator=g)
+    m, _ = _prefix_mask(B, L, g, lo=64)
+    adv, ret = compute_gae_advantage_return(r.to(dev), v.to(dev), m.to(dev), 1.0, 1.0)
+    adv64, ret64 = O.gae_advantage_return(r.double(), v.double(), m.double(), 1.0, 1.0)
+    adv32, ret32 = O.gae_advantage_return(r, v, m, 1.0, 1.0)
+    scale = ret64.abs().max().item()
+    err_kernel = (ret.cpu().double() - ret64).abs().max().item()
+    err_oracle32 = (ret32.double() - ret64).abs().max().item()
+    assert err_kernel <= max(2 * err_oracle32, 1e-5 * scale), (err_kernel, err_oracle32, scale)
+    _close(adv, adv64.float(), rtol=1e-5, atol=2e-5, what="whitened advantages vs fp64")
+
+
+def test_gae_multi_turn_fixture_and_errors(dev):
+    from verl_amd.trainer.ppo.core_algos import compute_gae_advantage_return
+    random.seed(0)
+    gamma, lam = random.uniform(0.0, 1.0), random.uniform(0.0, 1.0)
+    rewards = torch.tensor([[0.0, 0.0, 0.1, 0.1, 0.1, 0.0, 0.0, 0.1, 1.0, 0.0, 0.0]])
+    v1 = torch.tensor([[random.uniform(-100.0, 100.0), random.random(), 4.0, 5.0, 6.0,
+                        random.uniform(-100.0, 0), random.random(), 7.0, 9.0, 0.0, 0.0]])
+    v2 = torch.tensor([[random.random(), random.uniform(-100.0, 100.0), 4.0, 5.0, 6.0,
+                        random.random(), random.uniform(0.0, 100.0), 7.0, 9.0, 0.0, 0.0]])
+    mask = torch.tensor([[0, 0, 1, 1, 1, 0, 0, 1, 1, 0, 0]], dtype=torch.float)
+    a1, r1 = compute_gae_advantage_return(rewards.to(dev), v1.to(dev), mask.to(dev), gamma, lam)
+    a2, r2 = compute_gae_advantage_return(rewards.to(dev), v2.to(dev), mask.to(dev), gamma, lam)
+    md = mask.to(dev)
+    assert torch.equal(a1, a2) and torch.equal(r1 * md, r2 * md)       # observation tokens do not leak
+    want_a, want_r = O.gae_advantage_return(rewards, v1, mask, gamma, lam)
+    _close(a1, want_a, atol=1e-5); _close(r1, want_r, atol=1e-5)
+    with pytest.raises(ValueError):                                      # masked_var needs >= 2 valid tokens
+        compute_gae_advantage_return(rewards.to(dev), v1.to(dev), torch.zeros(1, 11, device=dev), gamma, lam)
+
+
+# ---- GRPO ---------------------------------------------------------------------------------------
+def _make_group_index(batch_size, num_groups):
+    counts = [2] * num_groups
+    for _ in range(batch_size - 2 * num_groups):
+        counts[random.randrange(num_groups)] += 1
+    index = []
+    for gid, c in enumerate(counts):
+        index.extend([gid] * c)
+    random.shuffle(index)
+    return np.asarray(index, dtype=np.int64)
+
+
+def _rand_mask(batch_size, seq_len):
+    mask = torch.randint(0, 2, (batch_size, seq_len), dtype=torch.int64).float()
+    rows = (mask.sum(dim=-1) == 0).nonzero(as_tuple=True)[0]
+    if len(rows) > 0:
+        mask[rows, -1] = 1.0
+    return mask
+
+
+@pytest.mark.parametrize("batch_size,seq_len,num_groups,seed", [(64, 128, 5, 0), (128, 256, 8, 1), (512, 512, 10, 2)])
+def test_grpo_reference_grid(dev, batch_size, seq_len, num_groups, seed):
+    from verl_amd.trainer.ppo import core_algos as CA
+    torch.manual_seed(seed); random.seed(seed); np.random.seed(seed)
+    index = _make_group_index(batch_size, num_groups)
+    mask = _rand_mask(batch_size, seq_len)
+    rewards = torch.randn(batch_size, seq_len) * mask
+    want, _ = O.grpo_outcome_advantage(rewards.clone(), mask, index)
+    want_v, _ = O.grpo_vectorized_outcome_advantage(rewards.clone(), mask, index)
+    a1, r1 = CA.compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    a2, r2 = CA.compute_grpo_vectorized_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    assert a1 is r1 and a2 is r2 and a1.shape == (batch_size, seq_len)
+    _close(a1, want, what="grpo"); _close(a2, want_v, what="grpo_vectorized"); _close(a1, a2.cpu())
+    assert torch.equal(a1 == 0, (want == 0).to(dev))                    # masked positions are exact zeros
+    # string labels give the same groups; norm_adv_by_std_in_grpo=False (Dr. GRPO)
+    names = {i: str(uuid.UUID(int=1000 + i)) for i in range(num_groups)}
+    a3, _ = CA.compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), np.array([names[i] for i in index], dtype=object))
+    assert torch.equal(a3, a1)
+    a4, _ = CA.compute_grpo_outcome_advantage(rewards, mask, index, norm_adv_by_std_in_grpo=False)
+    want4, _ = O.grpo_outcome_advantage(rewards.clone(), mask, index, norm_adv_by_std_in_grpo=False)
+    assert a4.device.type == "cpu"
+    _close(a4, want4, what="grpo without std")
+
+
+def test_grpo_singletons_equal_scores_and_group_mean_std(dev):
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.utils.groupwise import as_torch_index, group_mean_std
+    rewards = torch.tensor([[1.0, 2.0], [3.0, 0.0], [3.0, 0.0], [5.0, 5.0]])
+    mask = torch.tensor([[1.0, 0.0], [1.0, 1.0], [1.0, 1.0], [0.0, 1.0]])
+    index = np.array(["u-a", "u-b", "u-b", "u-c"], dtype=object)
+    want, _ = O.grpo_outcome_advantage(rewards.clone(), mask, index)
+    got, _ = CA.compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    _close(got, want)
+    assert torch.equal(got[1].cpu(), torch.zeros(2)) and torch.equal(got[2].cpu(), torch.zeros(2))
+    # reference known answer for group_mean_std
+    mean_g, std_g, cnt_g = group_mean_std(torch.tensor([1.0, 2.0, 3.0], device=dev), as_torch_index([0, 1, 0]))
+    assert torch.allclose(mean_g.cpu(), torch.tensor([2.0, 0.0])) and torch.allclose(cnt_g.cpu(), torch.tensor([2.0, 1.0]))
+    assert std_g[1].item() == 1.0 and abs(std_g[0].item() - 2 ** 0.5) < 1e-6
+    g = as_torch_index(["a", "b", "a", "c", "0042", 42])
+    assert g.tolist()[4] != g.tolist()[5] and len(torch.unique(g)) == 5
+    e = group_mean_std(torch.tensor([]), torch.tensor([], dtype=torch.long))
+    assert all(t.numel() == 0 for t in e)
+
+
+# ---- agg_loss / policy loss / value loss --------------------------------------------------------
+MODES = ["token-mean", "seq-mean-token-sum", "seq-mean-token-mean", "seq-mean-token-sum-norm"]
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("shape", [(5, 37), (16, 4096), (3, 4099)])
+def test_agg_loss_forward_backward(dev, mode, shape):
+    from verl_amd.trainer.ppo.core_algos import agg_loss
+    g = torch.Generator().manual_seed(shape[1])
+    x = torch.randn(*shape, generator=g)
+    m = (torch.rand(*shape, generator=g) < 0.7).float(); m[1] = 0
+    xd = x.to(dev).requires_grad_(); xo = x.clone().requires_grad_()
+    got = agg_loss(xd, m.to(dev), mode); want = O.agg_loss(xo, m, mode)
+    _close(got, want, what=mode)
+    (gg,) = torch.autograd.grad(got * 1.7, xd); (gw,) = torch.autograd.grad(want * 1.7, xo)
+    _close(gg, gw, atol=1e-9, what=mode + " grad")
+    kw = dict(dp_size=4, batch_num_tokens=1000, global_batch_size=9, loss_scale_factor=7)
+    _close(agg_loss(x.to(dev), m.to(dev), mode, **kw), O.agg_loss(x, m, mode, **kw), what=mode + " global")
+    with pytest.raises(ValueError):
+        agg_loss(x.to(dev), m.to(dev), "nope")
+
+
+def _policy_inputs(B, L, seed):
+    g = torch.Generator().manual_seed(seed)
+    old = torch.randn(B, L, generator=g) * 0.5 - 1
+    new = old + torch.randn(B, L, generator=g) * 0.3
+    adv = torch.randn(B, L, generator=g)
+    mask = (torch.rand(B, L, generator=g) < 0.7).float()
+    mask[1] = 0
+    new[0, :5] = old[0, :5] + 25.0          # beyond the +-20 clamp
+    new[2, :5] = old[2, :5] + 2.0           # large ratio -> dual clip where A < 0
+    new[3, :4] = old[3, :4]                 # ratio exactly 1
+    adv[3, :2] = 0.0                        # exact ties
+    return old, new, adv, mask
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("shape", [(5, 37), (8, 4096), (4, 1026)])
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.int64, torch.bool])
+def test_policy_loss_forward_backward(dev, mode, shape, mdtype):
+    from verl_amd.trainer.ppo.core_algos import get_policy_loss_fn
+    old, new, adv, mask = _policy_inputs(*shape, seed=shape[1])
+    cfg = _cfg(clip_ratio=0.2, clip_ratio_high=0.28)
+    fn = get_policy_loss_fn("vanilla")
+    nd = new.to(dev).requires_grad_(); no = new.clone().requires_grad_()
+    loss, metrics = fn(old_log_prob=old.to(dev), log_prob=nd, advantages=adv.to(dev),
+                       response_mask=mask.to(mdtype).to(dev), loss_agg_mode=mode, config=cfg, rollout_is_weights=None)
+    w_loss, w_cf, w_kl, w_cfl = O.policy_loss_vanilla(old, no, adv, mask, mode, 0.2, 0.28, 3.0)
+    _close(loss, w_loss, what="pg_loss " + mode)
+    assert isinstance(metrics["actor/pg_clipfrac"], float)
+    assert abs(metrics["actor/pg_clipfrac"] - w_cf.item()) <= 1e-6
+    assert abs(metrics["actor/ppo_kl"] - w_kl.item()) <= 1e-5 * abs(w_kl.item()) + 1e-6
+    assert abs(metrics["actor/pg_clipfrac_lower"] - w_cfl.item()) <= 1e-6
+    (gg,) = torch.autograd.grad(loss * 0.5, nd); (gw,) = torch.autograd.grad(w_loss * 0.5, no)
+    _close(gg, gw, atol=1e-9, what="d pg_loss / d log_prob " + mode)
+    assert torch.equal(gg.cpu() == 0, gw == 0)
+
+
+def test_policy_loss_weights_global_batch_and_special_cases(dev):
+    from verl_amd.trainer.ppo import core_algos as CA
+    old, new, adv, mask = _policy_inputs(6, 300, seed=9)
+    isw = torch.rand(6, 300, generator=torch.Generator().manual_seed(1)) + 0.5
+    info = dict(dp_size=2, batch_num_tokens=5000, global_batch_size=12, loss_scale_factor=None)
+    cfg = _cfg(global_batch_info=info)
+    for mode in MODES:
+        nd = new.to(dev).requires_grad_(); no = new.clone().requires_grad_()
+        loss, _ = CA.compute_policy_loss_vanilla(old.to(dev), nd, adv.to(dev), mask.to(dev), mode, cfg, isw.to(dev))
+        want = O.policy_loss_vanilla(old, no, adv, mask, mode, 0.2, 0.2, 3.0, isw, info)[0]
+        _close(loss, want, what="weighted " + mode)
+        _close(torch.autograd.grad(loss, nd)[0], torch.autograd.grad(want, no)[0], atol=1e-9)
+    # on-policy: ratio 1 -> loss = -masked mean of A, kl 0, nothing clipped (closed form)
+    loss, met = CA.compute_policy_loss_vanilla(old.to(dev), old.to(dev), adv.to(dev), mask.to(dev), "token-mean", _cfg())
+    assert abs(loss.item() + (adv * mask).sum().item() / mask.sum().item()) < 1e-6
+    assert met["actor/ppo_kl"] == 0 and met["actor/pg_clipfrac"] == 0 and met["actor/pg_clipfrac_lower"] == 0
+    # A < 0 with a huge ratio: every valid token sits on the dual-clip floor -A*c
+    neg = -adv.abs() - 0.1
+    loss, met = CA.compute_policy_loss_vanilla(old.to(dev), (old + 5).to(dev), neg.to(dev), mask.to(dev), "token-mean", _cfg())
+    assert abs(loss.item() - (3.0 * -neg * mask).sum().item() / mask.sum().item()) < 1e-5
+    assert abs(met["actor/pg_clipfrac_lower"] - 1.0) < 1e-6
+    # CPU tensors in -> CPU tensors out; deprecated positional form; registry errors
+    l_cpu, _ = CA.compute_policy_loss_vanilla(old, new, adv, mask, "token-mean", _cfg())
+    assert l_cpu.device.type == "cpu"
+    pl = CA.compute_policy_loss(old.to(dev), new.to(dev), adv.to(dev), mask.to(dev), cliprange=0.2)
+    want = O.policy_loss_vanilla(old, new, adv, mask)
+    for a, b in zip(pl, want):
+        _close(a, b)
+    with pytest.raises(AssertionError):
+        CA.compute_policy_loss_vanilla(old, new, adv, mask, "token-mean", _cfg(clip_ratio_c=1.0))
+    with pytest.raises(ValueError):
+        CA.get_policy_loss_fn("no-such-loss")
+    with pytest.raises(ValueError):
+        CA.get_adv_estimator_fn("no-such-estimator")
+    assert CA.get_adv_estimator_fn(CA.AdvantageEstimator.GAE) is CA.compute_gae_advantage_return
+    with pytest.raises(ValueError):
+        CA.register_adv_est("gae")(lambda: None)
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("shape", [(4, 29), (8, 4096)])
+def test_value_loss_forward_backward(dev, mode, shape):
+    from verl_amd.trainer.ppo.core_algos import compute_value_loss
+    g = torch.Generator().manual_seed(shape[1])
+    values = torch.randn(*shape, generator=g)
+    vpreds = values + torch.randn(*shape, generator=g)
+    returns = values + torch.randn(*shape, generator=g)
+    mask = (torch.rand(*shape, generator=g) < 0.8).float()
+    vpreds[0, :3] = values[0, :3] + 0.5      # exactly on the clip boundary
+    returns[0, 3] = vpreds[0, 3]             # zero error tie
+    vd = vpreds.to(dev).requires_grad_(); vo = vpreds.clone().requires_grad_()
+    loss, frac = compute_value_loss(vd, returns.to(dev), values.to(dev), mask.to(dev), 0.5, mode)
+    w_loss, w_frac = O.value_loss(vo, returns, values, mask, 0.5, mode)
+    _close(loss, w_loss, what="vf_loss " + mode); _close(frac, w_frac, what="vf_clipfrac")
+    _close(torch.autograd.grad(loss * 2.0, vd)[0], torch.autograd.grad(w_loss * 2.0, vo)[0], atol=1e-9,
+           what="d vf_loss / d vpreds")
+
+
+# ---- the two benchmark configurations end to end --------------------------------------------------
+def test_benchmark_config_grpo_policy_loss(dev):
+    """512 responses in 64 groups of 8, L = 4096, lengths U[64, 4096], Bernoulli(0.5) outcome reward
+    at the last valid token, old_lp ~ N(-1, 0.5), lp = old + N(0, 0.05); eps 1e-6, clip 0.2, c = 3."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    g = torch.Generator().manual_seed(3)
+    B, L = 512, 4096
+    mask, lens = _prefix_mask(B, L, g, lo=64)
+    rewards = torch.zeros(B, L)
+    rewards[torch.arange(B), lens - 1] = torch.bernoulli(torch.full((B,), 0.5), generator=g)
+    index = np.repeat(np.arange(64), 8)
+    old = torch.randn(B, L, generator=g) * 0.5 - 1
+    new = old + torch.randn(B, L, generator=g) * 0.05
+    adv, _ = CA.compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    want_adv, _ = O.grpo_outcome_advantage(rewards.clone(), mask, index)
+    _close(adv, want_adv, what="advantages")
+    assert torch.equal(adv.cpu() == 0, want_adv == 0)
+    nd = new.to(dev).requires_grad_(); no = new.clone().requires_grad_()
+    loss, met = CA.compute_policy_loss_vanilla(old.to(dev), nd, adv, mask.to(dev), "token-mean", _cfg())
+    w = O.policy_loss_vanilla(old, no, want_adv, mask, "token-mean")
+    _close(loss, w[0], what="pg_loss")
+    assert abs(met["actor/pg_clipfrac"] - w[1].item()) < 1e-6 and abs(met["actor/ppo_kl"] - w[2].item()) < 1e-6
+    _close(torch.autograd.grad(loss, nd)[0], torch.autograd.grad(w[0], no)[0], atol=1e-10, what="grad")
+
+
+def test_benchmark_config_gae_value_policy_loss(dev):
+    """B = 512, L = 4096, lengths U[64, 4096], reward N(0,1) at the last valid token, values N(0,1),
+    gamma 1.0, lam 0.95; whitened advantages, value loss (clip 0.5), policy loss (clip 0.2)."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    g = torch.Generator().manual_seed(4)
+    B, L = 512, 4096
+    mask, lens = _prefix_mask(B, L, g, lo=64)
+    rewards = torch.zeros(B, L)
+    rewards[torch.arange(B), lens - 1] = torch.randn(B, generator=g)
+    values = torch.randn(B, L, generator=g)
+    adv, ret = CA.compute_gae_advantage_return(rewards.to(dev), values.to(dev), mask.to(dev), 1.0, 0.95)
+    want_adv, want_ret = O.gae_advantage_return(rewards, values, mask, 1.0, 0.95)
+    _close(ret, want_ret, atol=1e-5, what="returns"); _close(adv, want_adv, atol=1e-5, what="advantages")
+    vpreds = values + torch.randn(B, L, generator=g) * 0.5
+    vd = vpreds.to(dev).requires_grad_(); vo = vpreds.clone().requires_grad_()
+    vloss, vfrac = CA.compute_value_loss(vd, ret, values.to(dev), mask.to(dev), 0.5)
+    w_vloss, w_vfrac = O.value_loss(vo, want_ret, values, mask, 0.5)
+    _close(vloss, w_vloss, what="vf_loss"); _close(vfrac, w_vfrac, what="vf_clipfrac")
+    _close(torch.autograd.grad(vloss, vd)[0], torch.autograd.grad(w_vloss, vo)[0], atol=1e-10)
+    old = torch.randn(B, L, generator=g) * 0.5 - 1
+    new = old + torch.randn(B, L, generator=g) * 0.05
+    loss, _ = CA.compute_policy_loss_vanilla(old.to(dev), new.to(dev), adv, mask.to(dev), "token-mean", _cfg())
+    _close(loss, O.policy_loss_vanilla(old, new, want_adv, mask, "token-mean")[0], rtol=1e-4, what="pg_loss")

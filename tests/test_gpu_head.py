@@ -1,0 +1,199 @@
+"""GPU parity of the fused log-prob / entropy head against the oracle (fp32 stock-torch ground
+truth of the reference's own test, oracle/head.py).
+
+Tolerances (north star): max abs error 2e-3 on log-prob and entropy (fp32 outputs).  Gradients
+come back in bf16 like the reference's, so on top of the 2e-3 absolute bar one bf16 ulp of the
+expected value (2**-8 relative) is allowed for the final rounding of the output.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import head as OH
+
+pytestmark = pytest.mark.gpu
+
+ATOL = 2e-3
+BF16_ULP = 2.0 ** -8
+
+
+def _make(n, h, v, seed, dist="uniform"):
+    g = torch.Generator().manual_seed(seed)
+    if dist == "uniform":          # distributions of the reference's test (uniform(-0.5, 0.5))
+        hidden = torch.rand(n, h, generator=g) - 0.5
+        weight = torch.rand(v, h, generator=g) - 0.5
+    else:                          # distributions of the benchmark configs
+        hidden = torch.randn(n, h, generator=g)
+        weight = torch.randn(v, h, generator=g) * 0.02
+    labels = torch.randint(0, v, (n,), generator=g)
+    return hidden.bfloat16(), weight.bfloat16(), labels
+
+
+def _oracle(hidden, weight, labels, T, g_lp=None, g_ent=None, device="cpu", chunk=1024):
+    """fp32 ground truth, chunked over tokens so the logits stay small; grads via autograd."""
+    hidden = hidden.to(device)
+    weight = weight.to(device)
+    labels = labels.to(device)
+    want_grad = g_lp is not None or g_ent is not None
+    w32 = weight.float().requires_grad_(want_grad)
+    lps, ents, dhs = [], [], []
+    dw = torch.zeros_like(w32) if want_grad else None
+    for lo in range(0, hidden.shape[0], chunk):
+        h32 = hidden[lo:lo + chunk].float().requires_grad_(want_grad)
+        lp, ent = OH.head_fp32_ground_truth(h32, w32, labels[lo:lo + chunk], T)
+        lps.append(lp.detach()); ents.append(ent.detach())
+        if want_grad:
+            outs, gos = [], []
+            if g_ent is not None:
+                outs.append(ent); gos.append(g_ent[lo:lo + chunk].to(device).float())
+            if g_lp is not None:
+                outs.append(lp); gos.append(g_lp[lo:lo + chunk].to(device).float())
+            dh, dwc = torch.autograd.grad(outs, (h32, w32), gos)
+            dhs.append(dh); dw += dwc
+    res = [torch.cat(lps), torch.cat(ents)]
+    if want_grad:
+        res += [torch.cat(dhs), dw]
+    return res
+
+
+def _close_bf16(got, want, what):
+    got = got.float().cpu(); want = want.float().cpu()
+    err = (got - want).abs()
+    bound = ATOL + BF16_ULP * want.abs()
+    worst = (err - bound).max().item()
+    assert worst <= 0, f"{what}: max abs err {err.max().item():.3e}, exceeds bound by {worst:.3e}"
+
+
+@pytest.mark.parametrize("n,h,v", [(1, 128, 128), (127, 128, 384), (128, 128, 1152), (129, 256, 1152),
+                                   (300, 384, 1000), (513, 128, 5000), (1388, 512, 2048)])
+@pytest.mark.parametrize("T", [1.0, 1.5, 0.7])
+def test_forward_small_shapes(dev, n, h, v, T):
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    hidden, weight, labels = _make(n, h, v, seed=n + v)
+    lp, ent = linear_cross_entropy(hidden.to(dev), weight.to(dev), labels.to(dev), T)
+    want_lp, want_ent = _oracle(hidden, weight, labels, T)
+    assert lp.shape == (n,) and ent.shape == (n,) and lp.dtype == torch.float32
+    assert (lp.cpu() - want_lp).abs().max().item() <= ATOL
+    assert (ent.cpu() - want_ent).abs().max().item() <= ATOL
+    assert (lp <= 1e-6).all() and (ent >= -1e-5).all() and (ent <= math.log(v) + 1e-4).all()
+
+
+@pytest.mark.parametrize("n,h,v", [(1, 128, 128), (127, 128, 384), (129, 256, 1152), (300, 384, 1000),
+                                   (513, 128, 5000), (700, 256, 8192)])
+@pytest.mark.parametrize("T", [1.0, 1.5])
+def test_backward_small_shapes(dev, n, h, v, T):
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    hidden, weight, labels = _make(n, h, v, seed=7 * n + v)
+    g = torch.Generator().manual_seed(n)
+    g_ent = (torch.rand(n, generator=g) - 0.5).bfloat16()          # bf16 upstream grads, as the reference test
+    g_lp = ((torch.rand(n, generator=g) - 0.5) * 2).bfloat16()
+    hd = hidden.to(dev).requires_grad_(); wd = weight.to(dev).requires_grad_()
+    lp, ent = linear_cross_entropy(hd, wd, labels.to(dev), T)
+    dh, dw = torch.autograd.grad((ent, lp), (hd, wd), (g_ent.to(dev).float(), g_lp.to(dev).float()))
+    assert dh.dtype == torch.bfloat16 and dw.dtype == torch.bfloat16 and dh.shape == hd.shape and dw.shape == wd.shape
+    _, _, want_dh, want_dw = _oracle(hidden, weight, labels, T, g_lp.float(), g_ent.float())
+    _close_bf16(dh, want_dh, "d_hidden")
+    _close_bf16(dw, want_dw, "d_weight")
+
+
+def test_backward_multi_chunk_and_accumulate(dev):
+    """Several vocabulary chunks (fp32 d_hidden accumulation across them), entropy gradient as a
+    scalar coefficient, and accumulation into an existing d_weight."""
+    from verl_amd.utils.kernel import linear_cross_entropy as K
+    n, h, v, T = 600, 256, 3000, 0.7
+    hidden, weight, labels = _make(n, h, v, seed=11, dist="normal")
+    hd, wd, ld = hidden.to(dev), weight.to(dev), labels.to(dev)
+    g_lp = torch.randn(n, generator=torch.Generator().manual_seed(1))
+    lp, ent, lse, mz = K.efficient_entropy_forward(hd, wd, ld, 0, T)
+    dh, dw = K.efficient_entropy_backward(g_lp.to(dev), None, hd, wd, ld, lse, mz, 0, T,
+                                          d_entropy_scalar=-0.001, vocab_chunk=768)
+    _, _, want_dh, want_dw = _oracle(hidden, weight, labels, T, g_lp, torch.full((n,), -0.001))
+    _close_bf16(dh, want_dh, "d_hidden")
+    _close_bf16(dw, want_dw, "d_weight")
+    # single-chunk path gives the same numbers up to the final rounding
+    dh1, dw1 = K.efficient_entropy_backward(g_lp.to(dev), None, hd, wd, ld, lse, mz, 0, T, d_entropy_scalar=-0.001)
+    _close_bf16(dh1, want_dh, "d_hidden (one chunk)")
+    _close_bf16(dw1, want_dw, "d_weight (one chunk)")
+    # accumulate: second call adds into the first call's d_weight
+    dw_acc = dw1.clone()
+    K.efficient_entropy_backward(g_lp.to(dev), None, hd, wd, ld, lse, mz, 0, T, d_entropy_scalar=-0.001,
+                                 d_weight_out=dw_acc)
+    _close_bf16(dw_acc, 2 * want_dw, "d_weight accumulated twice")
+
+
+def test_reductions_3d_input_and_argument_errors(dev):
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    b, s, h, v = 2, 70, 128, 512
+    hidden, weight, labels = _make(b * s, h, v, seed=3)
+    hd = hidden.view(b, s, h).to(dev).requires_grad_()
+    wd = weight.to(dev).requires_grad_()
+    ld = labels.view(b, s).to(dev)
+    lp, ent = linear_cross_entropy(hd, wd, ld, 1.5, "none")
+    assert lp.shape == (b * s,) and ent.shape == (b * s,)                    # flat, like the reference
+    want_lp, want_ent, want_dh, want_dw = _oracle(hidden, weight, labels, 1.5, torch.ones(b * s), torch.zeros(b * s))
+    lp_sum, _ = linear_cross_entropy(hd, wd, ld, 1.5, "sum")
+    lp_mean, _ = linear_cross_entropy(hd, wd, ld, 1.5, "MEAN")
+    assert lp_sum.dim() == 0 and abs(lp_sum.item() - want_lp.sum().item()) <= ATOL * b * s
+    assert abs(lp_mean.item() - want_lp.mean().item()) <= ATOL
+    dh, dw = torch.autograd.grad(lp_sum, (hd, wd))
+    assert dh.shape == hd.shape
+    _close_bf16(dh.view(b * s, h), want_dh, "d_hidden (sum)")
+    _close_bf16(dw, want_dw, "d_weight (sum)")
+    with pytest.raises(ValueError):
+        linear_cross_entropy(hd, wd, ld, 1.5, "max")
+    with pytest.raises(AssertionError):
+        linear_cross_entropy(hd, wd, ld, 1, "none")                          # temperature must be a float
+    with pytest.raises(AssertionError):
+        linear_cross_entropy(hd.float(), wd.float(), ld, 1.5, "none")        # bf16 only
+    with pytest.raises(AssertionError):
+        linear_cross_entropy(hd[..., :64], wd[:, :64], ld, 1.5, "none")      # non-contiguous / H % 128
+
+
+@pytest.mark.parametrize("n,h,v,T", [(2169, 896, 151936, 1.5), (1530, 2048, 32256, 1.5)])
+def test_reference_test_shapes_fwd_bwd(dev, n, h, v, T):
+    """Two of the five (N, H, V) cases of the reference's own test, its input distributions and
+    bf16 upstream grads; ground truth evaluated in fp32 on the GPU."""
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    hidden, weight, labels = _make(n, h, v, seed=5)
+    g = torch.Generator().manual_seed(6)
+    g_ent = (torch.rand(n, generator=g) - 0.5).bfloat16().float()
+    g_lp = ((torch.rand(n, generator=g) - 0.5) * 2).bfloat16().float()
+    hd = hidden.to(dev).requires_grad_(); wd = weight.to(dev).requires_grad_()
+    lp, ent = linear_cross_entropy(hd, wd, labels.to(dev), T)
+    dh, dw = torch.autograd.grad((ent, lp), (hd, wd), (g_ent.to(dev), g_lp.to(dev)))
+    want_lp, want_ent, want_dh, want_dw = _oracle(hidden, weight, labels, T, g_lp, g_ent, device=dev, chunk=512)
+    assert (lp - want_lp).abs().max().item() <= ATOL
+    assert (ent - want_ent).abs().max().item() <= ATOL
+    _close_bf16(dh, want_dh, "d_hidden")
+    _close_bf16(dw, want_dw, "d_weight")
+
+
+def test_benchmark_config_7b_head_full_size(dev):
+    """Full Qwen2.5-7B head shape (N=16384, H=3584, V=152064, T=1, dlogprob ~ N(0,1), dentropy =
+    0.001): every output compared with the fp32 ground truth evaluated on the GPU in 1024-token
+    chunks, plus size-independent properties (entropy in [0, log V], log-prob <= 0, softmax
+    gradient rows summing to zero over the vocabulary, linearity in the upstream gradient)."""
+    from verl_amd.utils.kernel import linear_cross_entropy as K
+    n, h, v, T = 16384, 3584, 152064, 1.0
+    g = torch.Generator(device=dev).manual_seed(0)
+    hidden = torch.randn(n, h, device=dev, generator=g).bfloat16()
+    weight = (torch.randn(v, h, device=dev, generator=g) * 0.02).bfloat16()
+    labels = torch.randint(0, v, (n,), device=dev, generator=g)
+    g_lp = torch.randn(n, device=dev, generator=g)
+    g_ent = torch.full((n,), 0.001, device=dev)
+    lp, ent, lse, mz = K.efficient_entropy_forward(hidden, weight, labels, 0, T)
+    dh, dw = K.efficient_entropy_backward(g_lp, None, hidden, weight, labels, lse, mz, 0, T, d_entropy_scalar=0.001)
+    assert (lp <= 0).all() and (ent >= 0).all() and (ent <= math.log(v) + 1e-4).all()
+    want_lp, want_ent, want_dh, want_dw = _oracle(hidden, weight, labels, T, g_lp, g_ent, device=dev, chunk=1024)
+    assert (lp - want_lp).abs().max().item() <= ATOL
+    assert (ent - want_ent).abs().max().item() <= ATOL
+    _close_bf16(dh, want_dh, "d_hidden")
+    _close_bf16(dw, want_dw, "d_weight")
+    del want_dw, want_dh
+    # sum_j dz_j = 0 for every token  =>  the vocabulary-axis sum of d_weight vanishes (bf16 rounding of 152064 rows)
+    col_sum = dw.float().sum(0)
+    assert col_sum.abs().max().item() < 0.5, col_sum.abs().max().item()
+    # linearity in the upstream gradient: backward(2 g) == 2 backward(g) up to output rounding
+    dh2, _ = K.efficient_entropy_backward(2 * g_lp, None, hidden, weight, labels, lse, mz, 0, T, d_entropy_scalar=0.002)
+    _close_bf16(dh2, 2 * dh.float(), "linearity of d_hidden")

@@ -1,0 +1,143 @@
+"""ctypes binding of ``libverl_amd.so`` (declared in ``include/verl_amd.h``).
+
+The library is loaded lazily, after ``import torch``, so that it binds to the HIP runtime torch
+has already mapped (same ``libamdhip64.so.7`` soname) and torch's streams are valid in it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p
+
+import torch
+
+_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libverl_amd.so")
+_lock = threading.Lock()
+_lib = None
+
+MASK_F32, MASK_I64, MASK_U8, MASK_I32 = 0, 1, 2, 3
+AGG_MODES = {
+    "token-mean": 0,
+    "seq-mean-token-sum": 1,
+    "seq-mean-token-mean": 2,
+    "seq-mean-token-sum-norm": 3,
+}
+
+# name -> (restype, argtypes); one entry per symbol of include/verl_amd.h
+SIGNATURES = {
+    "vamd_abi_version": (c_int, []),
+    "vamd_last_error": (c_char_p, []),
+    "vamd_lce_forward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
+    "vamd_lce_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p,
+                                 c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "vamd_lce_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
+    "vamd_lce_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p,
+                                  c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int, c_int64,
+                                  c_void_p, c_size_t, c_void_p]),
+    "vamd_lce_timing_enable": (c_int, [c_int]),
+    "vamd_lce_timing_collect": (c_int, [c_void_p, c_void_p]),
+    "vamd_masked_moments_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "vamd_masked_moments": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_void_p, c_void_p,
+                                    c_size_t, c_void_p]),
+    "vamd_whiten_stats": (c_int, [c_void_p, c_int, c_void_p, c_void_p]),
+    "vamd_affine_by_stats": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
+    "vamd_gae_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "vamd_gae": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_float, c_float, c_int, c_void_p,
+                         c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "vamd_grpo_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
+    "vamd_grpo_advantage": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_float, c_int,
+                                    c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "vamd_group_mean_std": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_float, c_void_p, c_void_p, c_void_p,
+                                    c_void_p]),
+    "vamd_agg_loss_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "vamd_agg_loss_forward": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_double, c_double,
+                                      c_double, c_double, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "vamd_agg_loss_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
+    "vamd_policy_loss_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "vamd_policy_loss_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64,
+                                         c_float, c_float, c_float, c_int, c_double, c_double, c_double, c_double,
+                                         c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "vamd_scale_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int64, c_void_p, c_void_p]),
+    "vamd_value_loss_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "vamd_value_loss_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_float,
+                                        c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+}
+
+
+def lib_path() -> str:
+    return _LIB_PATH
+
+
+def load_library(path: str | None = None) -> ctypes.CDLL:
+    """dlopen the library and attach prototypes.  Raises if it has not been built."""
+    path = path or _LIB_PATH
+    if not os.path.exists(path):
+        raise RuntimeError(
+            f"{path} is missing: build it with `python -m verl_amd.csrc.build` (hipcc, gfx950). "
+            "verl_amd has no CPU fallback."
+        )
+    lib = ctypes.CDLL(path)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError names the missing symbol
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                _lib = load_library()
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        msg = lib().vamd_last_error().decode("utf-8", "replace")
+        raise RuntimeError(f"libverl_amd error {rc}: {msg}")
+
+
+def compute_device(*tensors: torch.Tensor) -> torch.device:
+    """Device the kernels will run on: the tensors' GPU, or the current GPU for CPU inputs."""
+    for t in tensors:
+        if t is not None and t.is_cuda:
+            return t.device
+    if not torch.cuda.is_available():
+        raise RuntimeError("verl_amd needs a ROCm GPU: no device is visible and there is no CPU fallback")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def ptr(t: torch.Tensor | None):
+    return None if t is None else t.data_ptr()
+
+
+def workspace(nbytes: int, device: torch.device) -> torch.Tensor:
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def mask_code(mask: torch.Tensor) -> tuple[torch.Tensor, int]:
+    """Contiguous mask in one of the element types the kernels read, with its VAMD_MASK_* code."""
+    if mask.dtype == torch.float32:
+        code = MASK_F32
+    elif mask.dtype == torch.int64:
+        code = MASK_I64
+    elif mask.dtype in (torch.bool, torch.uint8):
+        code = MASK_U8
+    elif mask.dtype == torch.int32:
+        code = MASK_I32
+    else:  # fp16 / bf16 / fp64 / int8 / int16: exact in fp32 for 0/1 masks
+        mask = mask.to(torch.float32)
+        code = MASK_F32
+    return mask.contiguous(), code
+
+
+def as_f32(t: torch.Tensor, device: torch.device) -> torch.Tensor:
+    """fp32, contiguous, on `device` (a no-op for tensors that already are)."""
+    return t.detach().to(device=device, dtype=torch.float32).contiguous()

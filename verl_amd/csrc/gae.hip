@@ -1,0 +1,206 @@
+// Generalised Advantage Estimation as a chunked associative scan (one workgroup per sequence).
+//
+// Reference: compute_gae_advantage_return, verl/trainer/ppo/core_algos.py:214-262.  Walking a
+// row from its last column to its first, a valid step maps the carried state (nv, g) to
+//     nv' = v_t ,   g' = (r_t - v_t) + gamma * nv + gamma*lam * g ,
+// and a masked step leaves it unchanged.  Every step is therefore an affine map
+//     nv' = a nv + b ,  g' = P nv + Q g + R           (a in {0,1})
+// and maps compose associatively, so the recurrence is a prefix "sum" over maps.  A row is cut
+// into segments of 1024 columns walked right to left; inside a segment each of the 256 threads
+// composes its 4 columns, a wavefront scan (shuffles) plus a 4-entry LDS pass yields every
+// thread's incoming state, and the thread then replays its 4 columns to emit the advantages.
+// Loads and stores are float4 and contiguous across the wavefront.
+#include "rowchunk.h"
+
+namespace vamd {
+
+struct Affine {
+  float a, b, P, Q, R;
+};
+
+__device__ __forceinline__ Affine affine_identity() { return Affine{1.f, 0.f, 0.f, 1.f, 0.f}; }
+
+// later o earlier : apply `earlier` first
+__device__ __forceinline__ Affine compose(const Affine& later, const Affine& earlier) {
+  Affine o;
+  o.a = later.a * earlier.a;
+  o.b = fmaf(later.a, earlier.b, later.b);
+  o.P = fmaf(later.P, earlier.a, later.Q * earlier.P);
+  o.Q = later.Q * earlier.Q;
+  o.R = fmaf(later.P, earlier.b, fmaf(later.Q, earlier.R, later.R));
+  return o;
+}
+
+__device__ __forceinline__ Affine shfl_up_affine(const Affine& x, int d) {
+  Affine o;
+  o.a = __shfl_up(x.a, d, 64);
+  o.b = __shfl_up(x.b, d, 64);
+  o.P = __shfl_up(x.P, d, 64);
+  o.Q = __shfl_up(x.Q, d, 64);
+  o.R = __shfl_up(x.R, d, 64);
+  return o;
+}
+
+constexpr int kSeg = 1024;  // columns per segment = 256 threads x 4
+
+template <bool VEC, class M>
+__global__ __launch_bounds__(kRcThreads) void gae_scan_kernel(const float* __restrict__ rewards,
+                                                              const float* __restrict__ values,
+                                                              const M* __restrict__ mask, int64_t cols, float gamma,
+                                                              float gl, float* __restrict__ adv,
+                                                              float* __restrict__ ret,
+                                                              double* __restrict__ partials) {
+  const int64_t row = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int slot = kRcThreads - 1 - tid;  // thread 0 owns the right-most 4 columns of a segment
+  __shared__ Affine wave_tot[2][4];
+  __shared__ float carry[2][2];
+  if (tid == 0) {
+    carry[0][0] = 0.f;  // nv
+    carry[0][1] = 0.f;  // g
+  }
+  float m0 = 0, m1 = 0, m2 = 0, mc = 0;  // masked moments of the raw advantages
+  const int nseg = (int)((cols + kSeg - 1) / kSeg);
+  int par = 0;
+  __syncthreads();
+  for (int seg = nseg - 1; seg >= 0; --seg, par ^= 1) {
+    const int64_t c = (int64_t)seg * kSeg + slot * 4;
+    const int64_t left = cols - c;
+    const int valid = left >= 4 ? 4 : (left > 0 ? (int)left : 0);
+    float r[4] = {0, 0, 0, 0}, v[4] = {0, 0, 0, 0}, w[4] = {0, 0, 0, 0};
+    if (valid > 0) {
+      const int64_t i = row * cols + c;
+      if (VEC) {
+        ld4<true>(rewards, i, 4, r);
+        ld4<true>(values, i, 4, v);
+        ldmask4<true>(mask, i, 4, w);
+      } else {
+        ld4<false>(rewards, i, valid, r);
+        ld4<false>(values, i, valid, v);
+        ldmask4<false>(mask, i, valid, w);
+      }
+    }
+    // this thread's 4 columns as one map (right to left: e = 3 .. 0)
+    Affine f = affine_identity();
+#pragma unroll
+    for (int e = 3; e >= 0; --e) {
+      if (w[e] != 0.f) {
+        Affine n;
+        n.a = 0.f;
+        n.b = v[e];
+        n.P = fmaf(gl, f.P, gamma * f.a);
+        n.Q = gl * f.Q;
+        n.R = fmaf(gamma, f.b, fmaf(gl, f.R, r[e] - v[e]));
+        f = n;
+      }
+    }
+    // inclusive scan over the wavefront (lane order = walk order)
+    Affine inc = f;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const Affine nb = shfl_up_affine(inc, d);
+      if (lane >= d) inc = compose(inc, nb);
+    }
+    if (lane == 63) wave_tot[par][wave] = inc;
+    Affine exc = shfl_up_affine(inc, 1);
+    if (lane == 0) exc = affine_identity();
+    __syncthreads();
+    // state entering this wavefront, then this thread
+    float nv = carry[par][0], g = carry[par][1];
+    for (int k = 0; k < wave; ++k) {
+      const Affine t = wave_tot[par][k];
+      const float nv2 = fmaf(t.a, nv, t.b);
+      g = fmaf(t.P, nv, fmaf(t.Q, g, t.R));
+      nv = nv2;
+    }
+    {
+      const float nv2 = fmaf(exc.a, nv, exc.b);
+      g = fmaf(exc.P, nv, fmaf(exc.Q, g, exc.R));
+      nv = nv2;
+    }
+    // replay the 4 columns
+    float a_out[4], r_out[4];
+#pragma unroll
+    for (int e = 3; e >= 0; --e) {
+      if (w[e] != 0.f) {
+        const float delta = r[e] + gamma * nv - v[e];
+        g = fmaf(gl, g, delta);
+        nv = v[e];
+        m1 += g * w[e];
+        m2 += g * g * w[e];
+        mc += 1.f;
+      }
+      m0 += w[e];
+      a_out[e] = g;
+      r_out[e] = g + v[e];
+    }
+    if (tid == kRcThreads - 1) {
+      carry[par ^ 1][0] = nv;
+      carry[par ^ 1][1] = g;
+    }
+    if (valid > 0) {
+      const int64_t i = row * cols + c;
+      if (VEC) {
+        st4<true>(adv, i, 4, a_out);
+        st4<true>(ret, i, 4, r_out);
+      } else {
+        st4<false>(adv, i, valid, a_out);
+        st4<false>(ret, i, valid, r_out);
+      }
+    }
+    __syncthreads();
+  }
+  __shared__ double smem[16];
+  double acc[4] = {m0, m1, m2, mc};
+  block_sum<4, kRcThreads>(acc, smem);
+  if (tid == 0) {
+    double* o = partials + row * 4;
+    o[0] = acc[0]; o[1] = acc[1]; o[2] = acc[2]; o[3] = acc[3];
+  }
+}
+
+}  // namespace vamd
+
+using namespace vamd;
+
+extern "C" size_t vamd_gae_workspace_bytes(int64_t batch, int64_t length) {
+  if (batch <= 0 || length <= 0) return 0;
+  return align_up((size_t)batch * 4 * sizeof(double), 256) + 256 /* moments */ + 256 /* stats */;
+}
+
+extern "C" int vamd_gae(const float* rewards, const float* values, const void* mask, int mask_dtype, int64_t batch,
+                        int64_t length, float gamma, float lam, int whiten, float* advantages, float* returns,
+                        double* moments_out, void* workspace, size_t workspace_bytes, void* stream) {
+  VAMD_REQUIRE(batch > 0 && length > 0, "gae: empty input");
+  VAMD_REQUIRE(batch < (1ll << 31), "gae: batch too large");
+  VAMD_REQUIRE(rewards && values && mask && advantages && returns, "gae: null pointer");
+  if (!workspace || workspace_bytes < vamd_gae_workspace_bytes(batch, length)) {
+    set_error("gae: workspace too small");
+    return VAMD_EWORKSPACE;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  Carver carve(workspace);
+  double* partials = carve.take<double>((size_t)batch * 4);
+  double* moments = carve.take<double>(4);
+  float* stats = carve.take<float>(4);
+  const float gl = (float)((double)gamma * (double)lam);
+  VAMD_MASK_DISPATCH(mask_dtype, M, {
+    const bool vec = can_vectorize(length, {rewards, values, advantages, returns}, mask, sizeof(M));
+    if (vec)
+      hipLaunchKernelGGL((gae_scan_kernel<true, M>), dim3((unsigned)batch), dim3(kRcThreads), 0, s, rewards, values,
+                         static_cast<const M*>(mask), length, gamma, gl, advantages, returns, partials);
+    else
+      hipLaunchKernelGGL((gae_scan_kernel<false, M>), dim3((unsigned)batch), dim3(kRcThreads), 0, s, rewards, values,
+                         static_cast<const M*>(mask), length, gamma, gl, advantages, returns, partials);
+  });
+  VAMD_LAUNCH_CHECK();
+  double* mom = moments_out ? moments_out : moments;
+  int st = launch_moments_finalize(partials, batch, 1, 0, mom, s);
+  if (st != VAMD_OK) return st;
+  if (whiten) {
+    if ((st = vamd_whiten_stats(mom, 1, stats, stream)) != VAMD_OK) return st;
+    return vamd_affine_by_stats(advantages, stats, batch * length, advantages, stream);
+  }
+  return VAMD_OK;
+}

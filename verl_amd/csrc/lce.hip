@@ -1,0 +1,689 @@
+// Fused vocab-projection log-prob / entropy head for gfx950.
+//
+// Forward : logits tiles are produced by the MFMA tile engine and consumed in registers by an
+//           online-softmax epilogue (running max, sum exp, sum z*exp, label logit per token);
+//           the [tokens, vocab] logits never reach memory.
+// Backward: logits tiles are recomputed, turned into d_logits tiles in registers and staged as
+//           one bf16 [tokens, vocab_chunk] panel; the same tile engine then forms
+//           d_hidden (+)= panel . W[chunk]  and  d_weight[chunk] = panel^T . hidden.
+//
+// Arithmetic follows LinearCrossEntropy (verl/utils/kernel/linear_cross_entropy.py:40-116) /
+// efficient_entropy_forward+backward (verl/utils/kernel/kernels.py:563-753, :1512-1723): bf16
+// products, fp32 accumulation, logits scaled by 1/temperature in fp32, fp32 softmax state.
+#include <mutex>
+#include <vector>
+
+#include "common.h"
+#include "gemm_core.h"
+
+namespace vamd {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kNegBig = -1.0e30f;  // stands in for -inf so that (x - x) and 0 * x stay finite
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Optional per-kernel timing for benchmarks: when enabled on the calling thread, every head
+// kernel launch is bracketed by a pair of HIP events on the launch stream.
+enum : int { kTagForward = 0, kTagMerge = 1, kTagRecompute = 2, kTagDHidden = 3, kTagDWeight = 4, kNumTags = 5 };
+struct TimedLaunch {
+  int tag;
+  hipEvent_t start, stop;
+};
+static thread_local bool g_timing_on = false;
+static thread_local std::vector<TimedLaunch> g_timed;
+
+struct ScopedTiming {
+  hipStream_t s;
+  TimedLaunch t;
+  bool on;
+  ScopedTiming(int tag, hipStream_t stream) : s(stream), on(g_timing_on) {
+    if (!on) return;
+    t.tag = tag;
+    if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) {
+      on = false;
+      return;
+    }
+    (void)hipEventRecord(t.start, s);
+  }
+  ~ScopedTiming() {
+    if (!on) return;
+    (void)hipEventRecord(t.stop, s);
+    g_timed.push_back(t);
+  }
+};
+
+// =============================================================================================
+// Forward
+// =============================================================================================
+struct FwdArgs {
+  Operand hidden;  // R operand: [n_tokens][H]
+  Operand weight;  // C operand: [vocab][H]
+  const int64_t* labels;
+  int n_tokens, vocab, k_slabs;
+  int tok_tiles, voc_tiles, splits;
+  float scale2;      // log2(e) / temperature
+  float4* partials;  // [splits][tok_tiles * 256] : (max2, sum, sum_y, label logit)
+};
+
+struct SplitSched {
+  int r0_, vt_begin, vt_count;
+  __device__ __forceinline__ int count() const { return vt_count; }
+  __device__ __forceinline__ void tile(int i, int& r0, int& c0) const {
+    r0 = r0_;
+    c0 = (vt_begin + i) * kTile;
+  }
+};
+
+// Per-lane online-softmax state for the 4 token slots (nb) the lane owns.
+struct FwdEpi {
+  LanePos p;
+  float scale2;
+  int vocab;
+  float m[4], s[4], sy[4], zl[4];
+  int lab[4];
+
+  __device__ __forceinline__ void operator()(Accum& acc, int /*r0*/, int c0) {
+    const bool ragged = c0 + kTile > vocab;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+      float ymax = kNegBig;
+      // pass 1: scale into the log2 domain in place, mask the vocabulary tail, tile max
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          float y = acc.a[mb][nb][v] * scale2;
+          if (ragged) y = (c0 + acc_col(p, mb, v) < vocab) ? y : kNegBig;
+          acc.a[mb][nb][v] = y;
+          ymax = fmaxf(ymax, y);
+        }
+      // label logit: only when some lane's label falls in this wavefront's 128 columns
+      const int rel = lab[nb] - c0 - p.wc * 128;
+      if (__any(rel >= 0 && rel < 128)) {
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int col = mb * 32 + 8 * (v >> 2) + 4 * p.lh + (v & 3);
+            zl[nb] += (col == rel) ? acc.a[mb][nb][v] * kLn2 : 0.f;
+          }
+      }
+      const float m_new = fmaxf(m[nb], ymax);
+      const float resc = fast_exp2(m[nb] - m_new);
+      float s_ = s[nb] * resc, sy_ = sy[nb] * resc;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const float y = acc.a[mb][nb][v];
+          const float e = fast_exp2(y - m_new);
+          s_ += e;
+          sy_ = fmaf(e, y, sy_);
+        }
+      m[nb] = m_new;
+      s[nb] = s_;
+      sy[nb] = sy_;
+    }
+  }
+};
+
+__device__ __forceinline__ void merge_state(float& m, float& s, float& sy, float m2, float s2, float sy2) {
+  const float mm = fmaxf(m, m2);
+  const float a = fast_exp2(m - mm), b = fast_exp2(m2 - mm);
+  s = s * a + s2 * b;
+  sy = sy * a + sy2 * b;
+  m = mm;
+}
+
+__global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  // workgroup -> (token tile, vocabulary split); bands of 8 token tiles x all splits per XCD
+  const int nwg = a.tok_tiles * a.splits;
+  const int q = xcd_regroup(blockIdx.x, nwg);
+  const int band = 8 * a.splits;
+  const int bidx = q / band;
+  const int first = bidx * 8;
+  const int rows = (a.tok_tiles - first) < 8 ? (a.tok_tiles - first) : 8;
+  const int w = q - bidx * band;
+  const int tn = first + w % rows;
+  const int sp = w / rows;
+
+  SplitSched sched;
+  sched.r0_ = tn * kTile;
+  sched.vt_begin = (int)(((int64_t)sp * a.voc_tiles) / a.splits);
+  sched.vt_count = (int)(((int64_t)(sp + 1) * a.voc_tiles) / a.splits) - sched.vt_begin;
+
+  FwdEpi epi;
+  epi.p = lane_pos();
+  epi.scale2 = a.scale2;
+  epi.vocab = a.vocab;
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb) {
+    epi.m[nb] = kNegBig;
+    epi.s[nb] = 0.f;
+    epi.sy[nb] = 0.f;
+    epi.zl[nb] = 0.f;
+    const int tok = sched.r0_ + acc_row(epi.p, nb);
+    epi.lab[nb] = tok < a.n_tokens ? (int)a.labels[tok] : -1;
+  }
+
+  run_tiles<false, false>(a.hidden, a.weight, a.k_slabs, sched, epi, lds);
+
+  // merge the two lane halves (they hold disjoint vocabulary columns of the same token) ...
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb) {
+    const float m2 = __shfl_xor(epi.m[nb], 32, 64);
+    const float s2 = __shfl_xor(epi.s[nb], 32, 64);
+    const float sy2 = __shfl_xor(epi.sy[nb], 32, 64);
+    const float z2 = __shfl_xor(epi.zl[nb], 32, 64);
+    merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], m2, s2, sy2);
+    epi.zl[nb] += z2;
+  }
+  // ... then the two wavefronts that share a token half (wc = 0/1), through LDS.
+  float4* red = reinterpret_cast<float4*>(lds);  // [2][256]
+  if (epi.p.lh == 0) {
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+      red[epi.p.wc * kTile + acc_row(epi.p, nb)] = make_float4(epi.m[nb], epi.s[nb], epi.sy[nb], epi.zl[nb]);
+  }
+  __syncthreads();
+  {
+    const int t = threadIdx.x;
+    float4 x = red[t], y = red[kTile + t];
+    merge_state(x.x, x.y, x.z, y.x, y.y, y.z);
+    x.w += y.w;
+    a.partials[(int64_t)sp * a.tok_tiles * kTile + tn * kTile + t] = x;
+  }
+}
+
+struct MergeArgs {
+  const float4* partials;
+  int splits, stride, n_tokens;
+  float* logprobs;
+  float* entropy;
+  float* lse;
+  float* mean_z;
+};
+
+__global__ __launch_bounds__(256) void lce_merge_kernel(MergeArgs a) {
+  const int tok = blockIdx.x * 256 + threadIdx.x;
+  if (tok >= a.n_tokens) return;
+  float m = kNegBig, s = 0.f, sy = 0.f, zl = 0.f;
+  for (int sp = 0; sp < a.splits; ++sp) {
+    const float4 x = a.partials[(int64_t)sp * a.stride + tok];
+    merge_state(m, s, sy, x.x, x.y, x.z);
+    zl += x.w;
+  }
+  const float lse = (m + log2f(s)) * kLn2;
+  const float mz = (sy / s) * kLn2;
+  a.lse[tok] = lse;
+  a.mean_z[tok] = mz;
+  a.entropy[tok] = lse - mz;
+  a.logprobs[tok] = zl - lse;
+}
+
+// =============================================================================================
+// Backward
+// =============================================================================================
+__device__ __forceinline__ u32x2 pack_bf16x4(float a, float b, float c, float d) {
+  bf16x4 o;
+  o[0] = (__bf16)a;
+  o[1] = (__bf16)b;
+  o[2] = (__bf16)c;
+  o[3] = (__bf16)d;
+  return __builtin_bit_cast(u32x2, o);
+}
+
+__device__ __forceinline__ float bf16_bits_to_float(unsigned h) { return __uint_as_float(h << 16); }
+
+struct RecomputeArgs {
+  Operand hidden;  // R: [n_tokens][H]
+  Operand weight;  // C: rows of this vocabulary chunk, x_extent = vocab - chunk_c0
+  const int64_t* labels;
+  const float* lse;
+  const float* mean_z;
+  const float* g_lp;   // may be null
+  const float* g_ent;  // may be null -> g_ent_scalar
+  float g_ent_scalar;
+  int n_tokens, vocab_left;  // vocab_left = vocab - chunk_c0
+  int chunk_c0;
+  int k_slabs, tok_tiles, chunk_tiles;
+  float scale2, rcp_t;
+  uint16_t* dz;  // [tok_tiles*256][dz_ld] bf16
+  int dz_ld;
+};
+
+struct RecomputeEpi {
+  LanePos p;
+  const RecomputeArgs* a;
+  __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
+    const RecomputeArgs& A = *a;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+      const int tok = r0 + acc_row(p, nb);
+      const bool live = tok < A.n_tokens;
+      float lse2 = 0.f, mz = 0.f, glp = 0.f, gent = 0.f;
+      int rel = -1;
+      if (live) {
+        lse2 = A.lse[tok] * kLog2e;
+        mz = A.mean_z[tok];
+        glp = (A.g_lp ? A.g_lp[tok] : 0.f) * A.rcp_t;
+        gent = (A.g_ent ? A.g_ent[tok] : A.g_ent_scalar) * A.rcp_t;
+        rel = (int)A.labels[tok] - A.chunk_c0 - c0 - p.wc * 128;
+      }
+      const bool hit = __any(rel >= 0 && rel < 128);
+      uint16_t* out_row = A.dz + (int64_t)tok * A.dz_ld + c0;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          float d[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float x = acc.a[mb][nb][4 * g + e];
+            const float prob = fast_exp2(fmaf(x, A.scale2, -lse2));
+            const float u = fmaf(gent, fmaf(x, A.rcp_t, -mz), glp);  // g_lp/T + g_ent/T * (z - mean_z)
+            float dzv = -prob * u;
+            const int col = mb * 32 + 8 * g + 4 * p.lh + e;
+            if (hit) dzv += (col == rel) ? glp : 0.f;
+            const bool ok = live && (c0 + p.wc * 128 + col) < A.vocab_left;
+            d[e] = ok ? dzv : 0.f;
+          }
+          const int col0 = p.wc * 128 + mb * 32 + 8 * g + 4 * p.lh;
+          *reinterpret_cast<u32x2*>(out_row + col0) = pack_bf16x4(d[0], d[1], d[2], d[3]);
+        }
+    }
+  }
+};
+
+__global__ __launch_bounds__(kThreads) void lce_recompute_kernel(RecomputeArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  GroupedSched sched;
+  sched.r_tiles = a.tok_tiles;
+  sched.c_tiles = a.chunk_tiles;
+  sched.nwg = gridDim.x;
+  sched.wg = xcd_regroup(blockIdx.x, gridDim.x);
+  RecomputeEpi epi;
+  epi.p = lane_pos();
+  epi.a = &a;
+  run_tiles<false, false>(a.hidden, a.weight, a.k_slabs, sched, epi, lds);
+}
+
+// ---------------------------------------------------------------------------------------------
+// d_hidden (+)= dz_panel . W[chunk]          R = dz (direct), C = W (kmajor, k = vocab)
+// d_weight[chunk] (+)= dz_panel^T . hidden    R = dz (kmajor, k = token), C = hidden (kmajor)
+enum : int { kStoreF32 = 0, kAddF32 = 1, kFinalBf16 = 2, kFinalBf16AddPrev = 3 };
+
+struct GemmOutArgs {
+  Operand R, C;
+  int k_slabs, r_tiles, c_tiles;
+  int r_valid, c_valid;  // rows / cols of the output that exist
+  int mode;              // d_hidden: one of the enum above; d_weight: 0 = overwrite, 1 = accumulate
+  float* acc32;          // fp32 accumulator [r_valid][ld_out] (d_hidden only)
+  uint16_t* out;         // bf16 output
+  int64_t ld_out;
+};
+
+struct DHiddenEpi {
+  LanePos p;
+  const GemmOutArgs* a;
+  __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
+    const GemmOutArgs& A = *a;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+      const int row = r0 + acc_row(p, nb);
+      if (row >= A.r_valid) continue;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int col = c0 + p.wc * 128 + mb * 32 + 8 * g + 4 * p.lh;
+          if (col >= A.c_valid) continue;
+          f32x4 v = {acc.a[mb][nb][4 * g], acc.a[mb][nb][4 * g + 1], acc.a[mb][nb][4 * g + 2],
+                     acc.a[mb][nb][4 * g + 3]};
+          const int64_t off = (int64_t)row * A.ld_out + col;
+          if (A.mode == kStoreF32) {
+            *reinterpret_cast<f32x4*>(A.acc32 + off) = v;
+          } else if (A.mode == kAddF32) {
+            f32x4 o = *reinterpret_cast<const f32x4*>(A.acc32 + off);
+            *reinterpret_cast<f32x4*>(A.acc32 + off) = o + v;
+          } else {
+            if (A.mode == kFinalBf16AddPrev) v = v + *reinterpret_cast<const f32x4*>(A.acc32 + off);
+            *reinterpret_cast<u32x2*>(A.out + off) = pack_bf16x4(v[0], v[1], v[2], v[3]);
+          }
+        }
+    }
+  }
+};
+
+struct DWeightEpi {
+  LanePos p;
+  const GemmOutArgs* a;
+  __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
+    const GemmOutArgs& A = *a;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+      const int row = r0 + acc_row(p, nb);
+      if (row >= A.r_valid) continue;
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int col = c0 + p.wc * 128 + mb * 32 + 8 * g + 4 * p.lh;
+          if (col >= A.c_valid) continue;
+          float v0 = acc.a[mb][nb][4 * g], v1 = acc.a[mb][nb][4 * g + 1], v2 = acc.a[mb][nb][4 * g + 2],
+                v3 = acc.a[mb][nb][4 * g + 3];
+          u32x2* dst = reinterpret_cast<u32x2*>(A.out + (int64_t)row * A.ld_out + col);
+          if (A.mode == 1) {
+            const u32x2 o = *dst;
+            v0 += bf16_bits_to_float(o[0] & 0xffffu);
+            v1 += bf16_bits_to_float(o[0] >> 16);
+            v2 += bf16_bits_to_float(o[1] & 0xffffu);
+            v3 += bf16_bits_to_float(o[1] >> 16);
+          }
+          *dst = pack_bf16x4(v0, v1, v2, v3);
+        }
+    }
+  }
+};
+
+__global__ __launch_bounds__(kThreads) void lce_dhidden_kernel(GemmOutArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  GroupedSched sched;
+  sched.r_tiles = a.r_tiles;
+  sched.c_tiles = a.c_tiles;
+  sched.nwg = gridDim.x;
+  sched.wg = xcd_regroup(blockIdx.x, gridDim.x);
+  DHiddenEpi epi;
+  epi.p = lane_pos();
+  epi.a = &a;
+  run_tiles<false, true>(a.R, a.C, a.k_slabs, sched, epi, lds);
+}
+
+__global__ __launch_bounds__(kThreads) void lce_dweight_kernel(GemmOutArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char lds[];
+  GroupedSched sched;
+  sched.r_tiles = a.r_tiles;
+  sched.c_tiles = a.c_tiles;
+  sched.nwg = gridDim.x;
+  sched.wg = xcd_regroup(blockIdx.x, gridDim.x);
+  DWeightEpi epi;
+  epi.p = lane_pos();
+  epi.a = &a;
+  run_tiles<true, true>(a.R, a.C, a.k_slabs, sched, epi, lds);
+}
+
+// =============================================================================================
+// Host side
+// =============================================================================================
+template <class K>
+static int allow_big_lds(K kernel) {
+  VAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                               kLdsBytes));
+  return VAMD_OK;
+}
+
+static int ensure_lds_attributes() {
+  static std::once_flag once;
+  static int status = VAMD_OK;
+  std::call_once(once, [] {
+    int s;
+    if ((s = allow_big_lds(lce_forward_kernel)) != VAMD_OK) { status = s; return; }
+    if ((s = allow_big_lds(lce_recompute_kernel)) != VAMD_OK) { status = s; return; }
+    if ((s = allow_big_lds(lce_dhidden_kernel)) != VAMD_OK) { status = s; return; }
+    if ((s = allow_big_lds(lce_dweight_kernel)) != VAMD_OK) { status = s; return; }
+  });
+  return status;
+}
+
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+static int fwd_splits(int64_t tok_tiles, int64_t voc_tiles) {
+  const int cus = device_cu_count();
+  int64_t sp = cus / tok_tiles;  // as many workgroups as fit in one round over the CUs
+  if (sp < 1) sp = 1;
+  if (sp > voc_tiles) sp = voc_tiles;
+  return (int)sp;
+}
+
+static int check_head_shapes(int64_t n, int64_t h, int64_t v) {
+  VAMD_REQUIRE(n > 0 && h > 0 && v > 0, "lce: empty problem n=%lld h=%lld v=%lld", (long long)n, (long long)h,
+               (long long)v);
+  VAMD_REQUIRE(h % 128 == 0, "lce: hidden_size %lld must be a multiple of 128", (long long)h);
+  VAMD_REQUIRE(v % 8 == 0 && v >= 8, "lce: vocab %lld must be a multiple of 8", (long long)v);
+  VAMD_REQUIRE(n < (1ll << 30) && v < (1ll << 30), "lce: n_tokens / vocab too large");
+  return VAMD_OK;
+}
+
+static int64_t default_vocab_chunk(int64_t n_tokens, int64_t vocab, int64_t requested) {
+  const int64_t n_pad = ceil_div(n_tokens, kTile) * kTile;
+  const int64_t v_pad = ceil_div(vocab, kTile) * kTile;
+  int64_t cv = requested;
+  if (cv <= 0) {
+    const int64_t budget = 512ll << 20;  // bytes of bf16 d_logits staged at a time
+    cv = budget / (n_pad * 2) / kTile * kTile;
+  }
+  cv = ceil_div(cv, kTile) * kTile;
+  if (cv < kTile) cv = kTile;
+  if (cv > v_pad) cv = v_pad;
+  return cv;
+}
+
+}  // namespace vamd
+
+using namespace vamd;
+
+extern "C" int vamd_lce_timing_enable(int on) {
+  g_timing_on = on != 0;
+  return VAMD_OK;
+}
+
+extern "C" int vamd_lce_timing_collect(double* ms_by_kernel, int64_t* launches_by_kernel) {
+  VAMD_REQUIRE(ms_by_kernel && launches_by_kernel, "timing_collect: null pointer");
+  for (int i = 0; i < kNumTags; ++i) {
+    ms_by_kernel[i] = 0;
+    launches_by_kernel[i] = 0;
+  }
+  int status = VAMD_OK;
+  for (TimedLaunch& t : g_timed) {
+    float ms = 0.f;
+    if (hipEventSynchronize(t.stop) != hipSuccess || hipEventElapsedTime(&ms, t.start, t.stop) != hipSuccess) {
+      set_error("timing_collect: event query failed");
+      status = VAMD_EHIP;
+    } else {
+      ms_by_kernel[t.tag] += ms;
+      launches_by_kernel[t.tag] += 1;
+    }
+    (void)hipEventDestroy(t.start);
+    (void)hipEventDestroy(t.stop);
+  }
+  g_timed.clear();
+  return status;
+}
+
+extern "C" size_t vamd_lce_forward_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab) {
+  (void)hidden_size;
+  if (n_tokens <= 0 || vocab <= 0) return 0;
+  const int64_t tok_tiles = ceil_div(n_tokens, kTile), voc_tiles = ceil_div(vocab, kTile);
+  const int sp = fwd_splits(tok_tiles, voc_tiles);
+  return align_up((size_t)sp * tok_tiles * kTile * sizeof(float4), 256);
+}
+
+extern "C" int vamd_lce_forward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
+                                int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs,
+                                float* entropy, float* lse, float* mean_z, void* workspace, size_t workspace_bytes,
+                                void* stream) {
+  int st = check_head_shapes(n_tokens, hidden_size, vocab);
+  if (st != VAMD_OK) return st;
+  VAMD_REQUIRE(hidden && weight && labels && logprobs && entropy && lse && mean_z, "lce_forward: null pointer");
+  VAMD_REQUIRE(rcp_temperature > 0.f, "lce_forward: temperature must be positive");
+  const size_t need = vamd_lce_forward_workspace_bytes(n_tokens, hidden_size, vocab);
+  if (!workspace || workspace_bytes < need) {
+    set_error("lce_forward: workspace %zu bytes, need %zu", workspace_bytes, need);
+    return VAMD_EWORKSPACE;
+  }
+  if ((st = ensure_lds_attributes()) != VAMD_OK) return st;
+
+  FwdArgs a;
+  a.hidden = Operand{static_cast<const uint16_t*>(hidden), hidden_size, (int)n_tokens, (int)hidden_size};
+  a.weight = Operand{static_cast<const uint16_t*>(weight), hidden_size, (int)vocab, (int)hidden_size};
+  a.labels = labels;
+  a.n_tokens = (int)n_tokens;
+  a.vocab = (int)vocab;
+  a.k_slabs = (int)(hidden_size / kBK);
+  a.tok_tiles = (int)ceil_div(n_tokens, kTile);
+  a.voc_tiles = (int)ceil_div(vocab, kTile);
+  a.splits = fwd_splits(a.tok_tiles, a.voc_tiles);
+  a.scale2 = rcp_temperature * kLog2e;
+  a.partials = static_cast<float4*>(workspace);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  {
+    ScopedTiming tm(kTagForward, s);
+    hipLaunchKernelGGL(lce_forward_kernel, dim3(a.tok_tiles * a.splits), dim3(kThreads), kLdsBytes, s, a);
+  }
+  VAMD_LAUNCH_CHECK();
+
+  MergeArgs m;
+  m.partials = a.partials;
+  m.splits = a.splits;
+  m.stride = a.tok_tiles * kTile;
+  m.n_tokens = (int)n_tokens;
+  m.logprobs = logprobs;
+  m.entropy = entropy;
+  m.lse = lse;
+  m.mean_z = mean_z;
+  {
+    ScopedTiming tm(kTagMerge, s);
+    hipLaunchKernelGGL(lce_merge_kernel, dim3((unsigned)ceil_div(n_tokens, 256)), dim3(256), 0, s, m);
+  }
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
+
+extern "C" size_t vamd_lce_backward_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab,
+                                                    int64_t vocab_chunk) {
+  if (n_tokens <= 0 || vocab <= 0 || hidden_size <= 0) return 0;
+  const int64_t n_pad = ceil_div(n_tokens, kTile) * kTile;
+  const int64_t cv = default_vocab_chunk(n_tokens, vocab, vocab_chunk);
+  size_t bytes = align_up((size_t)n_pad * cv * 2, 256);
+  if (cv < ceil_div(vocab, kTile) * kTile) bytes += align_up((size_t)n_tokens * hidden_size * 4, 256);
+  return bytes;
+}
+
+extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
+                                 int64_t hidden_size, int64_t vocab, float rcp_temperature, const float* lse,
+                                 const float* mean_z, const float* d_logprobs, const float* d_entropy,
+                                 float d_entropy_scalar, void* d_hidden, void* d_weight, int accumulate_d_weight,
+                                 int64_t vocab_chunk, void* workspace, size_t workspace_bytes, void* stream) {
+  int st = check_head_shapes(n_tokens, hidden_size, vocab);
+  if (st != VAMD_OK) return st;
+  VAMD_REQUIRE(hidden && weight && labels && lse && mean_z && d_hidden && d_weight, "lce_backward: null pointer");
+  VAMD_REQUIRE(rcp_temperature > 0.f, "lce_backward: temperature must be positive");
+  const size_t need = vamd_lce_backward_workspace_bytes(n_tokens, hidden_size, vocab, vocab_chunk);
+  if (!workspace || workspace_bytes < need) {
+    set_error("lce_backward: workspace %zu bytes, need %zu", workspace_bytes, need);
+    return VAMD_EWORKSPACE;
+  }
+  if ((st = ensure_lds_attributes()) != VAMD_OK) return st;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int cus = device_cu_count();
+
+  const int tok_tiles = (int)ceil_div(n_tokens, kTile);
+  const int64_t n_pad = (int64_t)tok_tiles * kTile;
+  const int64_t cv = default_vocab_chunk(n_tokens, vocab, vocab_chunk);
+  const int n_chunks = (int)ceil_div(vocab, cv);
+  Carver carve(workspace);
+  uint16_t* dz = carve.take<uint16_t>((size_t)n_pad * cv);
+  float* acc32 = n_chunks > 1 ? carve.take<float>((size_t)n_tokens * hidden_size) : nullptr;
+  const uint16_t* hid = static_cast<const uint16_t*>(hidden);
+  const uint16_t* wgt = static_cast<const uint16_t*>(weight);
+  const int h_tiles = (int)ceil_div(hidden_size, kTile);
+
+  for (int ci = 0; ci < n_chunks; ++ci) {
+    const int64_t c0 = (int64_t)ci * cv;
+    const int64_t left = vocab - c0;                   // vocabulary rows from c0 on
+    const int64_t cols = left < cv ? left : cv;        // valid columns in this chunk
+    const int chunk_tiles = (int)ceil_div(cols, kTile);
+
+    RecomputeArgs r;
+    r.hidden = Operand{hid, hidden_size, (int)n_tokens, (int)hidden_size};
+    r.weight = Operand{wgt + c0 * hidden_size, hidden_size, (int)left, (int)hidden_size};
+    r.labels = labels;
+    r.lse = lse;
+    r.mean_z = mean_z;
+    r.g_lp = d_logprobs;
+    r.g_ent = d_entropy;
+    r.g_ent_scalar = d_entropy_scalar;
+    r.n_tokens = (int)n_tokens;
+    r.vocab_left = (int)left;
+    r.chunk_c0 = (int)c0;
+    r.k_slabs = (int)(hidden_size / kBK);
+    r.tok_tiles = tok_tiles;
+    r.chunk_tiles = chunk_tiles;
+    r.scale2 = rcp_temperature * kLog2e;
+    r.rcp_t = rcp_temperature;
+    r.dz = dz;
+    r.dz_ld = (int)cv;
+    {
+      const int tiles = tok_tiles * chunk_tiles;
+      const int grid = tiles < cus ? tiles : cus;
+      {
+        ScopedTiming tm(kTagRecompute, s);
+        hipLaunchKernelGGL(lce_recompute_kernel, dim3(grid), dim3(kThreads), kLdsBytes, s, r);
+      }
+      VAMD_LAUNCH_CHECK();
+    }
+
+    // d_hidden: k runs over the chunk's vocabulary columns (staged zeros beyond `cols`)
+    GemmOutArgs gh;
+    gh.R = Operand{dz, cv, (int)n_pad, (int)cv};
+    gh.C = Operand{wgt + c0 * hidden_size, hidden_size, (int)hidden_size, (int)left};
+    gh.k_slabs = (int)ceil_div(cols, kBK);
+    gh.r_tiles = tok_tiles;
+    gh.c_tiles = h_tiles;
+    gh.r_valid = (int)n_tokens;
+    gh.c_valid = (int)hidden_size;
+    if (n_chunks == 1) gh.mode = kFinalBf16;
+    else if (ci == 0) gh.mode = kStoreF32;
+    else if (ci == n_chunks - 1) gh.mode = kFinalBf16AddPrev;
+    else gh.mode = kAddF32;
+    gh.acc32 = acc32;
+    gh.out = static_cast<uint16_t*>(d_hidden);
+    gh.ld_out = hidden_size;
+    {
+      const int tiles = gh.r_tiles * gh.c_tiles;
+      const int grid = tiles < cus ? tiles : cus;
+      {
+        ScopedTiming tm(kTagDHidden, s);
+        hipLaunchKernelGGL(lce_dhidden_kernel, dim3(grid), dim3(kThreads), kLdsBytes, s, gh);
+      }
+      VAMD_LAUNCH_CHECK();
+    }
+
+    // d_weight rows of this chunk: k runs over tokens (staged zeros beyond n_tokens)
+    GemmOutArgs gw;
+    gw.R = Operand{dz, cv, (int)(ceil_div(cols, 8) * 8), (int)n_pad};
+    gw.C = Operand{hid, hidden_size, (int)hidden_size, (int)n_tokens};
+    gw.k_slabs = (int)ceil_div(n_tokens, kBK);
+    gw.r_tiles = chunk_tiles;
+    gw.c_tiles = h_tiles;
+    gw.r_valid = (int)cols;
+    gw.c_valid = (int)hidden_size;
+    gw.mode = accumulate_d_weight ? 1 : 0;
+    gw.acc32 = nullptr;
+    gw.out = static_cast<uint16_t*>(d_weight) + c0 * hidden_size;
+    gw.ld_out = hidden_size;
+    {
+      const int tiles = gw.r_tiles * gw.c_tiles;
+      const int grid = tiles < cus ? tiles : cus;
+      {
+        ScopedTiming tm(kTagDWeight, s);
+        hipLaunchKernelGGL(lce_dweight_kernel, dim3(grid), dim3(kThreads), kLdsBytes, s, gw);
+      }
+      VAMD_LAUNCH_CHECK();
+    }
+  }
+  return VAMD_OK;
+}

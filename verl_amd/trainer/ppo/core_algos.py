@@ -1,0 +1,410 @@
+"""PPO / GRPO policy math on MI355X.
+
+Drop-ins for the functions of ``verl.trainer.ppo.core_algos`` that sit on the per-token hot path:
+the two registries, GAE, GRPO (loop and vectorised forms), ``agg_loss``, the vanilla clipped /
+dual-clip policy loss and the clipped value loss.  Signatures, return tuples, error types and
+messages follow the reference (verl/trainer/ppo/core_algos.py); the arithmetic runs in
+``libverl_amd.so``.  Inputs may be CPU tensors (the trainer computes advantages on the driver):
+they are staged to the current GPU and results come back on the input's device.
+"""
+from __future__ import annotations
+
+from enum import Enum
+from typing import Any, Callable, Optional
+
+import numpy as np
+import torch
+
+from ... import _cabi
+from ...utils import torch_functional as verl_F
+from ...utils.groupwise import as_torch_index, contiguous_group_ids, group_mean_std  # noqa: F401
+
+PolicyLossFn = Callable[..., tuple[torch.Tensor, dict[str, Any]]]
+
+POLICY_LOSS_REGISTRY: dict[str, PolicyLossFn] = {}
+
+
+def register_policy_loss(name: str) -> Callable[[PolicyLossFn], PolicyLossFn]:
+    """Decorator: ``POLICY_LOSS_REGISTRY[name] = fn`` (reference core_algos.py:53-67)."""
+
+    def decorator(func: PolicyLossFn) -> PolicyLossFn:
+        POLICY_LOSS_REGISTRY[name] = func
+        return func
+
+    return decorator
+
+
+def get_policy_loss_fn(name):
+    """Look a policy loss up by name; unknown names raise ``ValueError`` with the reference's
+    message (core_algos.py:70-85)."""
+    loss_name = name
+    if loss_name not in POLICY_LOSS_REGISTRY:
+        raise ValueError(
+            f"Unsupported loss mode: {loss_name}. Supported modes are: {list(POLICY_LOSS_REGISTRY.keys())}"
+        )
+    return POLICY_LOSS_REGISTRY[loss_name]
+
+
+class AdvantageEstimator(str, Enum):
+    """Names of the reference's advantage estimators (core_algos.py:88-109); only GAE, GRPO and
+    GRPO_VECTORIZED are implemented here, the other names exist so configs keep parsing."""
+
+    GAE = "gae"
+    GRPO = "grpo"
+    REINFORCE_PLUS_PLUS = "reinforce_plus_plus"
+    REINFORCE_PLUS_PLUS_BASELINE = "reinforce_plus_plus_baseline"
+    REMAX = "remax"
+    RLOO = "rloo"
+    OPO = "opo"
+    GRPO_PASSK = "grpo_passk"
+    GPG = "gpg"
+    RLOO_VECTORIZED = "rloo_vectorized"
+    GRPO_VECTORIZED = "grpo_vectorized"
+    OPTIMAL_TOKEN_BASELINE = "optimal_token_baseline"
+    TIR_OPTIMAL_TOKEN_BASELINE = "tir_optimal_token_baseline"
+
+
+ADV_ESTIMATOR_REGISTRY: dict[str, Any] = {}
+
+
+def register_adv_est(name_or_enum) -> Any:
+    """Decorator registering an advantage estimator; re-registering a name with a different
+    function raises ``ValueError`` (reference core_algos.py:115-133)."""
+
+    def decorator(fn):
+        name = name_or_enum.value if isinstance(name_or_enum, Enum) else name_or_enum
+        if name in ADV_ESTIMATOR_REGISTRY and ADV_ESTIMATOR_REGISTRY[name] != fn:
+            raise ValueError(
+                f"Adv estimator {name} has already been registered: {ADV_ESTIMATOR_REGISTRY[name]} vs {fn}"
+            )
+        ADV_ESTIMATOR_REGISTRY[name] = fn
+        return fn
+
+    return decorator
+
+
+def get_adv_estimator_fn(name_or_enum):
+    """Reference core_algos.py:136-149."""
+    name = name_or_enum.value if isinstance(name_or_enum, Enum) else name_or_enum
+    if name not in ADV_ESTIMATOR_REGISTRY:
+        raise ValueError(f"Unknown advantage estimator simply: {name}")
+    return ADV_ESTIMATOR_REGISTRY[name]
+
+
+# ---------------------------------------------------------------------------------------------
+def _matrix(t: torch.Tensor, dev: torch.device) -> torch.Tensor:
+    x = _cabi.as_f32(t, dev)
+    if x.dim() == 1:
+        x = x.view(1, -1)
+    assert x.dim() == 2, f"expected a (batch, length) tensor, got shape {tuple(t.shape)}"
+    return x
+
+
+def _mask_matrix(mask: torch.Tensor, dev: torch.device, shape) -> tuple[torch.Tensor, int]:
+    m, code = _cabi.mask_code(mask.detach().to(dev))
+    if m.dim() == 1:
+        m = m.view(1, -1)
+    assert tuple(m.shape) == tuple(shape), f"mask shape {tuple(mask.shape)} does not match {tuple(shape)}"
+    return m, code
+
+
+@register_adv_est(AdvantageEstimator.GAE)
+def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torch.Tensor,
+                                 response_mask: torch.Tensor, gamma, lam):
+    """GAE with state carried over masked tokens, then ``masked_whiten`` of the advantages.
+
+    Args / returns as in the reference (core_algos.py:214-262): all ``(bs, response_length)``;
+    returns ``(advantages, returns)`` with ``returns = raw advantages + values``.  Runs under
+    ``no_grad``.  The recurrence is evaluated as a parallel scan of affine maps, so results agree
+    with the sequential fp32 loop to rounding, not bit for bit.
+    """
+    with torch.no_grad():
+        dev = _cabi.compute_device(token_level_rewards, values, response_mask)
+        r = _matrix(token_level_rewards, dev)
+        v = _matrix(values, dev)
+        assert r.shape == v.shape
+        m, code = _mask_matrix(response_mask, dev, r.shape)
+        B, Lc = r.shape
+        adv = torch.empty_like(r)
+        ret = torch.empty_like(r)
+        mom = torch.empty(4, dtype=torch.float64, device=dev)
+        Lb = _cabi.lib()
+        ws = _cabi.workspace(Lb.vamd_gae_workspace_bytes(B, Lc), dev)
+        with torch.cuda.device(dev):
+            _cabi.check(Lb.vamd_gae(r.data_ptr(), v.data_ptr(), m.data_ptr(), code, B, Lc, float(gamma), float(lam),
+                                    1, adv.data_ptr(), ret.data_ptr(), mom.data_ptr(), ws.data_ptr(), ws.numel(),
+                                    _cabi.stream_ptr(dev)))
+        verl_F._raise_on_tiny_mask(float(mom[0].item()))
+        out_dev = token_level_rewards.device
+        return adv.view(token_level_rewards.shape).to(out_dev), ret.view(token_level_rewards.shape).to(out_dev)
+
+
+def _grpo(token_level_rewards, response_mask, index, epsilon, norm_adv_by_std_in_grpo, std_mode):
+    with torch.no_grad():
+        dev = _cabi.compute_device(token_level_rewards, response_mask)
+        r = _matrix(token_level_rewards, dev)
+        m, code = _mask_matrix(response_mask, dev, r.shape)
+        B, Lc = r.shape
+        ids, G = contiguous_group_ids(index)
+        if ids.numel() != B:
+            raise ValueError(f"index has {ids.numel()} entries for a batch of {B}")
+        ids = ids.to(dev)
+        adv = torch.empty_like(r)
+        Lb = _cabi.lib()
+        ws = _cabi.workspace(Lb.vamd_grpo_workspace_bytes(B, Lc, G), dev)
+        with torch.cuda.device(dev):
+            _cabi.check(Lb.vamd_grpo_advantage(r.data_ptr(), m.data_ptr(), code, ids.data_ptr(), B, Lc, G,
+                                               float(epsilon), int(bool(norm_adv_by_std_in_grpo)), std_mode,
+                                               adv.data_ptr(), None, ws.data_ptr(), ws.numel(),
+                                               _cabi.stream_ptr(dev)))
+        out = adv.view(token_level_rewards.shape).to(token_level_rewards.device)
+        return out, out
+
+
+@register_adv_est(AdvantageEstimator.GRPO)
+def compute_grpo_outcome_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor,
+                                   index: np.ndarray, epsilon: float = 1e-6,
+                                   norm_adv_by_std_in_grpo: bool = True, config: Optional[Any] = None):
+    """Outcome-reward GRPO advantage (reference core_algos.py:266-330).
+
+    Score = unmasked row sum of ``token_level_rewards``; per group ``mean`` and unbiased ``std``
+    (a single-member group uses mean 0, std 1); ``(score - mean) / (std + epsilon)`` (or without
+    the division) broadcast over the row and multiplied by ``response_mask``.  ``index`` may hold
+    any hashable labels.  Returns the same tensor twice, like the reference.
+    """
+    return _grpo(token_level_rewards, response_mask, index, epsilon, norm_adv_by_std_in_grpo, std_mode=0)
+
+
+@register_adv_est(AdvantageEstimator.GRPO_VECTORIZED)
+def compute_grpo_vectorized_outcome_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor,
+                                              index: np.ndarray, epsilon: float = 1e-6,
+                                              norm_adv_by_std_in_grpo: bool = True, config: Optional[Any] = None):
+    """Vectorised twin (reference core_algos.py:333-357): std = sqrt(clamp(var, min=epsilon))."""
+    return _grpo(token_level_rewards, response_mask, index, epsilon, norm_adv_by_std_in_grpo, std_mode=1)
+
+
+# ---------------------------------------------------------------------------------------------
+def _agg_mode(loss_agg_mode: str) -> int:
+    if loss_agg_mode not in _cabi.AGG_MODES:
+        raise ValueError(f"Invalid loss_agg_mode: {loss_agg_mode}")
+    return _cabi.AGG_MODES[loss_agg_mode]
+
+
+def _opt(x) -> float:
+    """``None`` -> -1 (the C ABI's "not given"); tensors and numbers -> float."""
+    if x is None:
+        return -1.0
+    return float(x.item()) if isinstance(x, torch.Tensor) else float(x)
+
+
+class _AggLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, loss_mat, loss_mask, mode, dp_size, bnt, gbs, lsf):
+        dev = _cabi.compute_device(loss_mat, loss_mask)
+        x = _matrix(loss_mat, dev)
+        m, code = _mask_matrix(loss_mask, dev, x.shape)
+        rows, cols = x.shape
+        Lb = _cabi.lib()
+        out = torch.empty((), dtype=torch.float32, device=dev)
+        coef = torch.empty(rows, dtype=torch.float32, device=dev)
+        ws = _cabi.workspace(Lb.vamd_agg_loss_workspace_bytes(rows, cols), dev)
+        with torch.cuda.device(dev):
+            _cabi.check(Lb.vamd_agg_loss_forward(x.data_ptr(), m.data_ptr(), code, rows, cols, mode, dp_size, bnt,
+                                                 gbs, lsf, out.data_ptr(), coef.data_ptr(), ws.data_ptr(),
+                                                 ws.numel(), _cabi.stream_ptr(dev)))
+        ctx.save_for_backward(coef, m)
+        ctx.code = code
+        ctx.in_shape = loss_mat.shape
+        ctx.in_device = loss_mat.device
+        ctx.in_dtype = loss_mat.dtype
+        return out.to(loss_mat.device)
+
+    @staticmethod
+    def backward(ctx, d_loss):
+        coef, m = ctx.saved_tensors
+        dev = coef.device
+        rows, cols = m.shape
+        g = torch.empty((rows, cols), dtype=torch.float32, device=dev)
+        d = _cabi.as_f32(d_loss, dev).reshape(1)
+        with torch.cuda.device(dev):
+            _cabi.check(_cabi.lib().vamd_agg_loss_backward(d.data_ptr(), coef.data_ptr(), m.data_ptr(), ctx.code,
+                                                           rows, cols, g.data_ptr(), _cabi.stream_ptr(dev)))
+        g = g.view(ctx.in_shape).to(device=ctx.in_device, dtype=ctx.in_dtype)
+        return g, None, None, None, None, None, None
+
+
+def agg_loss(loss_mat: torch.Tensor, loss_mask: torch.Tensor, loss_agg_mode: str, dp_size: int = 1,
+             batch_num_tokens: Optional[int] = None, global_batch_size: Optional[int] = None,
+             loss_scale_factor: Optional[int] = None):
+    """Aggregate a ``(bs, response_length)`` loss matrix to a scalar (reference
+    core_algos.py:1025-1080): ``token-mean``, ``seq-mean-token-sum``, ``seq-mean-token-mean`` or
+    ``seq-mean-token-sum-norm``; any other mode raises ``ValueError``.  Differentiable with
+    respect to ``loss_mat``."""
+    mode = _agg_mode(loss_agg_mode)
+    return _AggLoss.apply(loss_mat, loss_mask, mode, float(dp_size), _opt(batch_num_tokens),
+                          _opt(global_batch_size), _opt(loss_scale_factor))
+
+
+# ---------------------------------------------------------------------------------------------
+class _PolicyLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, log_prob, old_log_prob, advantages, response_mask, is_weights, clip_low, clip_high, clip_c,
+                mode, dp_size, bnt, gbs, lsf):
+        dev = _cabi.compute_device(log_prob, old_log_prob, advantages, response_mask)
+        lp = _matrix(log_prob, dev)
+        old = _matrix(old_log_prob, dev)
+        adv = _matrix(advantages, dev)
+        assert lp.shape == old.shape == adv.shape
+        m, code = _mask_matrix(response_mask, dev, lp.shape)
+        isw = _matrix(is_weights, dev) if is_weights is not None else None
+        rows, cols = lp.shape
+        need_grad = ctx.needs_input_grad[0]
+        Lb = _cabi.lib()
+        out = torch.empty(4, dtype=torch.float32, device=dev)
+        coef = torch.empty(rows, dtype=torch.float32, device=dev)
+        g = torch.empty_like(lp) if need_grad else None
+        ws = _cabi.workspace(Lb.vamd_policy_loss_workspace_bytes(rows, cols), dev)
+        with torch.cuda.device(dev):
+            _cabi.check(Lb.vamd_policy_loss_forward(old.data_ptr(), lp.data_ptr(), adv.data_ptr(), m.data_ptr(), code,
+                                                    _cabi.ptr(isw), rows, cols, clip_low, clip_high, clip_c, mode,
+                                                    dp_size, bnt, gbs, lsf, out.data_ptr(), _cabi.ptr(g),
+                                                    coef.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                    _cabi.stream_ptr(dev)))
+        if need_grad:
+            ctx.save_for_backward(g, coef)
+        ctx.in_shape = log_prob.shape
+        ctx.in_device = log_prob.device
+        ctx.in_dtype = log_prob.dtype
+        out = out.to(log_prob.device)
+        ctx.mark_non_differentiable(out)
+        return out[0].clone(), out
+
+    @staticmethod
+    def backward(ctx, d_loss, _d_out):
+        g, coef = ctx.saved_tensors
+        dev = g.device
+        rows, cols = g.shape
+        d = _cabi.as_f32(d_loss, dev).reshape(1)
+        res = torch.empty_like(g)
+        with torch.cuda.device(dev):
+            _cabi.check(_cabi.lib().vamd_scale_rows(g.data_ptr(), coef.data_ptr(), d.data_ptr(), 1.0, rows, cols,
+                                                    res.data_ptr(), _cabi.stream_ptr(dev)))
+        res = res.view(ctx.in_shape).to(device=ctx.in_device, dtype=ctx.in_dtype)
+        return (res,) + (None,) * 12
+
+
+def _cfg_get(config, key, default=None):
+    getter = getattr(config, "get", None)
+    if callable(getter):
+        return getter(key, default)
+    return getattr(config, key, default)
+
+
+@register_policy_loss("vanilla")
+def compute_policy_loss_vanilla(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                                response_mask: torch.Tensor, loss_agg_mode: str = "token-mean",
+                                config: Optional[Any] = None, rollout_is_weights: torch.Tensor | None = None):
+    """Clipped PPO objective with the dual-clip floor (reference core_algos.py:1159-1250).
+
+    ``config`` needs ``clip_ratio``, optional ``clip_ratio_low`` / ``clip_ratio_high``,
+    ``get("clip_ratio_c", 3.0)`` and a ``global_batch_info`` dict that is forwarded to
+    ``agg_loss``.  Returns ``(pg_loss, metrics)`` with ``actor/pg_clipfrac``, ``actor/ppo_kl``
+    and ``actor/pg_clipfrac_lower`` as Python floats.  One fused kernel pass produces the loss,
+    the three metrics and the gradient with respect to ``log_prob``.
+    """
+    assert config is not None
+    clip_ratio = config.clip_ratio
+    low = getattr(config, "clip_ratio_low", None)
+    high = getattr(config, "clip_ratio_high", None)
+    clip_ratio_low = low if low is not None else clip_ratio
+    clip_ratio_high = high if high is not None else clip_ratio
+    clip_ratio_c = _cfg_get(config, "clip_ratio_c", 3.0)
+    assert clip_ratio_c > 1.0, (
+        "The lower bound of the clip_ratio_c for dual-clip PPO should be greater than 1.0,"
+        + f" but get the value: {clip_ratio_c}."
+    )
+    info = dict(getattr(config, "global_batch_info", None) or {})
+    mode = _agg_mode(loss_agg_mode)
+    pg_loss, out = _PolicyLoss.apply(
+        log_prob, old_log_prob, advantages, response_mask, rollout_is_weights, float(clip_ratio_low),
+        float(clip_ratio_high), float(clip_ratio_c), mode, float(info.get("dp_size", 1)),
+        _opt(info.get("batch_num_tokens")), _opt(info.get("global_batch_size")), _opt(info.get("loss_scale_factor")))
+    vals = out.detach().tolist()
+    pg_metrics = {
+        "actor/pg_clipfrac": vals[1],
+        "actor/ppo_kl": vals[2],
+        "actor/pg_clipfrac_lower": vals[3],
+    }
+    return pg_loss, pg_metrics
+
+
+def compute_policy_loss(old_log_prob, log_prob, advantages, response_mask, cliprange=None, cliprange_low=None,
+                        cliprange_high=None, clip_ratio_c=3.0, loss_agg_mode: str = "token-mean"):
+    """Deprecated positional form (reference core_algos.py:1083-1156): returns
+    ``(pg_loss, pg_clipfrac, ppo_kl, pg_clipfrac_lower)`` as tensors."""
+    assert clip_ratio_c > 1.0, (
+        "The lower bound of the clip_ratio_c for dual-clip PPO should be greater than 1.0,"
+        + f" but get the value: {clip_ratio_c}."
+    )
+    if cliprange_low is None:
+        cliprange_low = cliprange
+    if cliprange_high is None:
+        cliprange_high = cliprange
+    pg_loss, out = _PolicyLoss.apply(log_prob, old_log_prob, advantages, response_mask, None, float(cliprange_low),
+                                     float(cliprange_high), float(clip_ratio_c), _agg_mode(loss_agg_mode), 1.0,
+                                     -1.0, -1.0, -1.0)
+    return pg_loss, out[1], out[2], out[3]
+
+
+# ---------------------------------------------------------------------------------------------
+class _ValueLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, vpreds, returns, values, response_mask, cliprange_value, mode):
+        dev = _cabi.compute_device(vpreds, returns, values, response_mask)
+        vp = _matrix(vpreds, dev)
+        ret = _matrix(returns, dev)
+        val = _matrix(values, dev)
+        assert vp.shape == ret.shape == val.shape
+        m, code = _mask_matrix(response_mask, dev, vp.shape)
+        rows, cols = vp.shape
+        need_grad = ctx.needs_input_grad[0]
+        Lb = _cabi.lib()
+        out = torch.empty(2, dtype=torch.float32, device=dev)
+        coef = torch.empty(rows, dtype=torch.float32, device=dev)
+        g = torch.empty_like(vp) if need_grad else None
+        ws = _cabi.workspace(Lb.vamd_value_loss_workspace_bytes(rows, cols), dev)
+        with torch.cuda.device(dev):
+            _cabi.check(Lb.vamd_value_loss_forward(vp.data_ptr(), ret.data_ptr(), val.data_ptr(), m.data_ptr(), code,
+                                                   rows, cols, cliprange_value, mode, out.data_ptr(), _cabi.ptr(g),
+                                                   coef.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                   _cabi.stream_ptr(dev)))
+        if need_grad:
+            ctx.save_for_backward(g, coef)
+        ctx.in_shape = vpreds.shape
+        ctx.in_device = vpreds.device
+        ctx.in_dtype = vpreds.dtype
+        out = out.to(vpreds.device)
+        ctx.mark_non_differentiable(out)
+        return out[0].clone(), out
+
+    @staticmethod
+    def backward(ctx, d_loss, _d_out):
+        g, coef = ctx.saved_tensors
+        dev = g.device
+        rows, cols = g.shape
+        d = _cabi.as_f32(d_loss, dev).reshape(1)
+        res = torch.empty_like(g)
+        with torch.cuda.device(dev):
+            _cabi.check(_cabi.lib().vamd_scale_rows(g.data_ptr(), coef.data_ptr(), d.data_ptr(), 0.5, rows, cols,
+                                                    res.data_ptr(), _cabi.stream_ptr(dev)))
+        res = res.view(ctx.in_shape).to(device=ctx.in_device, dtype=ctx.in_dtype)
+        return res, None, None, None, None, None
+
+
+def compute_value_loss(vpreds: torch.Tensor, returns: torch.Tensor, values: torch.Tensor,
+                       response_mask: torch.Tensor, cliprange_value: float, loss_agg_mode: str = "token-mean"):
+    """Clipped value loss (reference core_algos.py:1799-1838): returns ``(vf_loss, vf_clipfrac)``,
+    ``vf_loss`` differentiable with respect to ``vpreds``."""
+    vf_loss, out = _ValueLoss.apply(vpreds, returns, values, response_mask, float(cliprange_value),
+                                    _agg_mode(loss_agg_mode))
+    return vf_loss, out[1]

@@ -1,0 +1,171 @@
+"""Fused vocab-projection log-prob / entropy head on MI355X.
+
+Drop-in for ``verl.utils.kernel.linear_cross_entropy`` (reference
+verl/utils/kernel/linear_cross_entropy.py:38-119): same class name, ``forward`` / ``backward``
+signatures, argument checks and return tuple.  The arithmetic runs in ``libverl_amd.so``
+(``vamd_lce_forward`` / ``vamd_lce_backward``): bf16 MFMA logits tiles with an in-register online
+softmax; the ``[tokens, vocab]`` logits are never stored.
+"""
+from __future__ import annotations
+
+import typing
+
+import torch
+import torch.distributed as dist
+
+from ... import _cabi
+
+
+def get_entropy_reduction_enum_number(reduction: str) -> int:
+    """"none" -> 0, "sum" -> 1, "mean" -> 2; anything else raises ``ValueError``
+    (reference verl/utils/kernel/kernels.py:110-126)."""
+    table = {"none": 0, "sum": 1, "mean": 2}
+    if reduction not in table:
+        raise ValueError(f"Invalid reduction: {reduction}")
+    return table[reduction]
+
+
+def _check_inputs(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor) -> None:
+    # the assertions of efficient_entropy_forward (reference kernels.py:574-593)
+    assert hidden.is_cuda and weight.is_cuda and labels.is_cuda
+    assert weight.device == hidden.device and labels.device == hidden.device
+    assert hidden.dim() == 2 and weight.dim() == 2 and labels.dim() == 1
+    assert hidden.is_contiguous() and weight.is_contiguous() and labels.is_contiguous()
+    assert hidden.shape[0] == labels.shape[0] and hidden.shape[1] == weight.shape[1]
+    assert hidden.shape[1] % 128 == 0
+    assert hidden.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, (
+        f"the MI355X head computes on bf16 inputs, got {hidden.dtype} / {weight.dtype}"
+    )
+    assert weight.shape[0] % 8 == 0, "vocab size must be a multiple of 8"
+
+
+def efficient_entropy_forward(hidden, weight, labels, reduction: int = 0, temperature: float = 1.0,
+                              dist_process_group=None):
+    """Host side of the forward kernels (reference kernels.py:563-753).
+
+    Returns ``(logprobs, entropy, lse, mean_z)``; the last two are the per-token statistics the
+    backward pass needs (log-sum-exp and softmax-weighted mean of the scaled logits).
+    """
+    if dist_process_group is not None:
+        raise NotImplementedError("vocab-parallel process groups are not supported on this single-GPU path")
+    _check_inputs(hidden, weight, labels)
+    if labels.dtype != torch.int64:
+        labels = labels.to(torch.int64)
+    n, h = hidden.shape
+    v = weight.shape[0]
+    dev = hidden.device
+    L = _cabi.lib()
+    logprobs = torch.empty((n,), device=dev, dtype=torch.float32)
+    entropy = torch.empty((n,), device=dev, dtype=torch.float32)
+    lse = torch.empty((n,), device=dev, dtype=torch.float32)
+    mean_z = torch.empty((n,), device=dev, dtype=torch.float32)
+    ws = _cabi.workspace(L.vamd_lce_forward_workspace_bytes(n, h, v), dev)
+    with torch.cuda.device(dev):
+        _cabi.check(L.vamd_lce_forward(hidden.data_ptr(), weight.data_ptr(), labels.data_ptr(), n, h, v,
+                                       1.0 / temperature, logprobs.data_ptr(), entropy.data_ptr(), lse.data_ptr(),
+                                       mean_z.data_ptr(), ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
+    if reduction == 1:
+        logprobs = _sum_f32(logprobs)
+    elif reduction == 2:
+        logprobs = _sum_f32(logprobs) / n
+    return logprobs, entropy, lse, mean_z
+
+
+def _sum_f32(x: torch.Tensor) -> torch.Tensor:
+    """Sum of a 1-D fp32 device tensor through the masked-moments kernel (mask of ones)."""
+    from ..torch_functional import _moments
+
+    ones = torch.ones_like(x, dtype=torch.uint8)
+    return _moments(x.view(1, -1), ones.view(1, -1), per_row=False)[1].to(torch.float32)
+
+
+def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse, mean_z, reduction: int = 0,
+                               temperature: float = 1.0, dist_process_group=None, d_entropy_scalar: float = 0.0,
+                               d_weight_out: torch.Tensor | None = None, vocab_chunk: int = 0):
+    """Host side of the backward kernels (reference kernels.py:1512-1723).
+
+    ``dlogprobs`` / ``dentropy`` may be ``None`` (no contribution).  ``d_entropy_scalar`` adds a
+    constant upstream entropy gradient for every token without materialising it.  When
+    ``d_weight_out`` is given the weight gradient is ACCUMULATED into it (token-chunked use).
+    Returns ``(d_hidden, d_weight)`` in ``hidden.dtype``.
+    """
+    if dist_process_group is not None:
+        raise NotImplementedError("vocab-parallel process groups are not supported on this single-GPU path")
+    _check_inputs(hidden, weight, labels)
+    n, h = hidden.shape
+    v = weight.shape[0]
+    dev = hidden.device
+    if dlogprobs is not None:
+        if reduction == 0:
+            assert dlogprobs.shape == (n,)
+        else:
+            assert dlogprobs.dim() == 0
+            scale = 1.0 if reduction == 1 else 1.0 / n
+            dlogprobs = (dlogprobs.to(torch.float32) * scale).expand(n)
+        assert dlogprobs.is_cuda and dlogprobs.device == dev
+        dlogprobs = dlogprobs.to(torch.float32).contiguous()
+    if dentropy is not None:
+        assert dentropy.shape == (n,)
+        assert dentropy.is_cuda and dentropy.device == dev
+        dentropy = dentropy.to(torch.float32).contiguous()
+        assert d_entropy_scalar == 0.0, "pass the entropy gradient either as a tensor or as a scalar"
+    assert lse.shape == (n,) and mean_z.shape == (n,)
+    if labels.dtype != torch.int64:
+        labels = labels.to(torch.int64)
+    L = _cabi.lib()
+    d_hidden = torch.empty_like(hidden)
+    accumulate = d_weight_out is not None
+    d_weight = d_weight_out if accumulate else torch.empty_like(weight)
+    assert d_weight.shape == weight.shape and d_weight.dtype == weight.dtype and d_weight.is_contiguous()
+    ws = _cabi.workspace(L.vamd_lce_backward_workspace_bytes(n, h, v, vocab_chunk), dev)
+    with torch.cuda.device(dev):
+        _cabi.check(L.vamd_lce_backward(hidden.data_ptr(), weight.data_ptr(), labels.data_ptr(), n, h, v,
+                                        1.0 / temperature, lse.data_ptr(), mean_z.data_ptr(), _cabi.ptr(dlogprobs),
+                                        _cabi.ptr(dentropy), float(d_entropy_scalar), d_hidden.data_ptr(),
+                                        d_weight.data_ptr(), int(accumulate), int(vocab_chunk), ws.data_ptr(),
+                                        ws.numel(), _cabi.stream_ptr(dev)))
+    return d_hidden, d_weight
+
+
+class LinearCrossEntropy(torch.autograd.Function):
+    """``linear_cross_entropy(hidden, weight, labels, temperature, reduction, group)``.
+
+    hidden ``(..., hidden_size)`` bf16 -> flattened to ``(num_tokens, hidden_size)``;
+    weight ``(vocab_size, hidden_size)`` bf16; labels ``(...)`` -> ``(num_tokens,)``.
+    Returns ``(logprobs, entropy)`` as FLAT fp32 ``(num_tokens,)`` tensors (``logprobs`` is a
+    scalar for ``reduction`` "sum" / "mean"), like the reference
+    (verl/utils/kernel/linear_cross_entropy.py:40-87).
+    """
+
+    @staticmethod
+    def forward(ctx, hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor,
+                temperature: typing.Optional[float] = 1.0, reduction: typing.Optional[str] = "none",
+                dist_process_group: typing.Optional[dist.ProcessGroup] = None):
+        assert isinstance(temperature, float), f"temperature must be a float, but got {type(temperature)}"
+        assert isinstance(reduction, str), f"reduction must be a str, but got {type(reduction)}"
+        REDUCTION = get_entropy_reduction_enum_number(reduction.lower())
+        original_hidden_shape = hidden.shape
+        if len(hidden.shape) != 2:
+            hidden = hidden.view(-1, hidden.shape[-1])
+        if len(labels.shape) != 1:
+            labels = labels.view(-1)
+        logprobs, entropy, lse, mean_z = efficient_entropy_forward(
+            hidden, weight, labels, REDUCTION, temperature, dist_process_group)
+        ctx.save_for_backward(hidden, weight, labels, lse, mean_z)
+        ctx.original_hidden_shape = original_hidden_shape
+        ctx.REDUCTION = REDUCTION
+        ctx.dist_process_group = dist_process_group
+        ctx.temperature = temperature
+        return logprobs, entropy
+
+    @staticmethod
+    def backward(ctx, dlogprobs: torch.Tensor, dentropy: torch.Tensor):
+        hidden, weight, labels, lse, mean_z = ctx.saved_tensors
+        d_hidden, d_weight = efficient_entropy_backward(
+            dlogprobs, dentropy, hidden, weight, labels, lse, mean_z, ctx.REDUCTION, ctx.temperature,
+            ctx.dist_process_group)
+        d_hidden = d_hidden.view(ctx.original_hidden_shape)
+        return (d_hidden, d_weight, None, None, None, None)
+
+
+linear_cross_entropy = LinearCrossEntropy.apply
