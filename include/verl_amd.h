@@ -82,8 +82,8 @@ int vamd_lce_backward(const void* hidden, const void* weight, const int64_t* lab
                       void* d_hidden, void* d_weight, int accumulate_d_weight, int64_t vocab_chunk, void* workspace,
                       size_t workspace_bytes, void* stream);
 
-/* Benchmark aid (no counterpart in the reference): with timing enabled on the calling thread,
- * every head kernel launch is bracketed by HIP events on its stream.  vamd_lce_timing_collect
+/* Benchmark aid (no counterpart in the reference): with timing enabled, every head kernel
+ * launch of the process is bracketed by HIP events on its stream.  vamd_lce_timing_collect
  * waits for them and adds up milliseconds and launch counts per kernel, indexed
  * 0 forward, 1 merge, 2 logit recompute, 3 d_hidden GEMM, 4 d_weight GEMM (arrays of 5). */
 int vamd_lce_timing_enable(int on);

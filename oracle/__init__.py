@@ -22,6 +22,7 @@ from .head import (  # noqa: F401
     fused_linear_for_ppo_bwd,
     fused_linear_for_ppo_chunked,
     head_grads_closed_form,
+    head_fwd_bwd_chunked_fp32,
 )
 from .masked import (  # noqa: F401
     clip_by_value,

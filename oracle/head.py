@@ -140,3 +140,45 @@ def head_grads_closed_form(hidden, weight, labels, temperature, dlogprobs, dentr
     g_h = dentropy.to(dtype).unsqueeze(-1)
     dz = (g_lp * (onehot - p) - g_h * p * (z - mean_z)) / temperature
     return dz @ w, dz.t() @ h
+
+
+@torch.no_grad()
+def head_fwd_bwd_chunked_fp32(hidden, weight, labels, temperature, dlogprobs, dentropy, chunk=1024):
+    """fp32 forward outputs, closed-form gradients (the same formula as
+    ``head_grads_closed_form``, which is pinned against autograd) and, for each gradient, the
+    L1 magnitude of the products that form it:
+
+        E_dh = |dz| @ |W| ,   E_dw = |dz|^T @ |hidden| .
+
+    Both reference implementations round ``d_logits`` to the input dtype before the two GEMMs
+    (verl/utils/experimental/torch_functional.py:65, verl/utils/kernel/kernels.py:1664), so a
+    bf16 implementation can differ from the fp32 ground truth by up to 2**-8 * E (half an ulp,
+    8 significant bits, per product); tests use E to state that bound.  Works on any device; tokens are processed
+    in chunks so that ``[chunk, vocab]`` is the largest temporary.
+    """
+    w32 = weight.to(torch.float32)
+    aw = w32.abs()
+    dw = torch.zeros_like(w32)
+    e_dw = torch.zeros_like(w32)
+    lps, ents, dhs, e_dhs = [], [], [], []
+    for lo in range(0, hidden.shape[0], chunk):
+        hi = min(lo + chunk, hidden.shape[0])
+        h32 = hidden[lo:hi].to(torch.float32)
+        lab = labels[lo:hi]
+        z = (h32 @ w32.t()) / temperature
+        lse = torch.logsumexp(z, dim=-1, keepdim=True)
+        p = torch.exp(z - lse)
+        mean_z = (p * z).sum(-1, keepdim=True)
+        lps.append(z.gather(-1, lab.unsqueeze(-1)).squeeze(-1) - lse.squeeze(-1))
+        ents.append((lse - mean_z).squeeze(-1))
+        g_lp = dlogprobs[lo:hi].to(torch.float32).unsqueeze(-1)
+        g_en = dentropy[lo:hi].to(torch.float32).unsqueeze(-1)
+        dz = -(g_lp * p) - g_en * p * (z - mean_z)
+        dz.scatter_add_(-1, lab.unsqueeze(-1), g_lp)
+        dz /= temperature
+        dhs.append(dz @ w32)
+        dw += dz.t() @ h32
+        dz.abs_()
+        e_dhs.append(dz @ aw)
+        e_dw += dz.t() @ h32.abs()
+    return torch.cat(lps), torch.cat(ents), torch.cat(dhs), dw, torch.cat(e_dhs), e_dw

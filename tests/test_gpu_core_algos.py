@@ -193,7 +193,8 @@ def test_grpo_reference_grid(dev, batch_size, seq_len, num_groups, seed):
     a4, _ = CA.compute_grpo_outcome_advantage(rewards, mask, index, norm_adv_by_std_in_grpo=False)
     want4, _ = O.grpo_outcome_advantage(rewards.clone(), mask, index, norm_adv_by_std_in_grpo=False)
     assert a4.device.type == "cpu"
-    _close(a4, want4, what="grpo without std")
+    # un-normalised scores are row sums of magnitude ~30 (fp32 ulp 3.8e-6): the absolute floor is one ulp of that
+    _close(a4, want4, atol=1e-5, what="grpo without std")
 
 
 def test_grpo_singletons_equal_scores_and_group_mean_std(dev):

@@ -122,3 +122,26 @@ def test_gradient_rows_sum_to_zero_over_vocab():
     hidden, weight, labels = _inputs(11, 16, 40, 7)
     _, dw = H.head_grads_closed_form(hidden, weight, labels, 1.2, torch.randn(11), torch.randn(11))
     assert dw.sum(0).abs().max() < 1e-9
+
+
+def test_chunked_fp32_closed_form_matches_autograd_and_bounds_bf16_dlogits():
+    n, h, v = 300, 64, 520
+    hidden, weight, labels = _inputs(n, h, v, 8)
+    g = torch.Generator().manual_seed(3)
+    g_lp, g_ent = torch.randn(n, generator=g), torch.randn(n, generator=g) * 0.1
+    hr, wr = hidden.clone().requires_grad_(), weight.clone().requires_grad_()
+    lp, ent = H.head_fp32_ground_truth(hr, wr, labels, 0.9)
+    dh, dw = torch.autograd.grad((lp, ent), (hr, wr), (g_lp, g_ent))
+    lp2, ent2, dh2, dw2, e_dh, e_dw = H.head_fwd_bwd_chunked_fp32(hidden, weight, labels, 0.9, g_lp, g_ent, chunk=128)
+    assert torch.allclose(lp, lp2, atol=1e-5) and torch.allclose(ent, ent2, atol=1e-5)
+    assert torch.allclose(dh, dh2, atol=1e-5) and torch.allclose(dw, dw2, atol=1e-5)
+    # the L1 scales really bound what rounding d_logits to bf16 does to the two GEMMs
+    dh3, dw3 = H.fused_linear_for_ppo_bwd(g_lp, g_ent, hidden, weight, labels, 0.9)          # fp32, no rounding
+    z = (hidden @ weight.t()) / 0.9
+    p = z.softmax(-1)
+    dz = (g_lp[:, None] * (torch.zeros_like(z).scatter_(-1, labels[:, None], 1) - p)
+          - g_ent[:, None] * p * (z - (p * z).sum(-1, keepdim=True))) / 0.9
+    dzr = dz.bfloat16().float()
+    assert ((dzr @ weight - dh).abs() <= 2.0 ** -8 * e_dh + 1e-6).all()
+    assert ((dzr.t() @ hidden - dw).abs() <= 2.0 ** -8 * e_dw + 1e-6).all()
+    assert torch.allclose(dh3, dh, atol=1e-5)

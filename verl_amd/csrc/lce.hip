@@ -10,6 +10,7 @@
 // Arithmetic follows LinearCrossEntropy (verl/utils/kernel/linear_cross_entropy.py:40-116) /
 // efficient_entropy_forward+backward (verl/utils/kernel/kernels.py:563-753, :1512-1723): bf16
 // products, fp32 accumulation, logits scaled by 1/temperature in fp32, fp32 softmax state.
+#include <atomic>
 #include <mutex>
 #include <vector>
 
@@ -24,21 +25,23 @@ constexpr float kNegBig = -1.0e30f;  // stands in for -inf so that (x - x) and 0
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Optional per-kernel timing for benchmarks: when enabled on the calling thread, every head
-// kernel launch is bracketed by a pair of HIP events on the launch stream.
+// Optional per-kernel timing for benchmarks: when enabled, every head kernel launch (from any
+// thread: autograd runs backward on its own) is bracketed by a pair of HIP events on the launch
+// stream.
 enum : int { kTagForward = 0, kTagMerge = 1, kTagRecompute = 2, kTagDHidden = 3, kTagDWeight = 4, kNumTags = 5 };
 struct TimedLaunch {
   int tag;
   hipEvent_t start, stop;
 };
-static thread_local bool g_timing_on = false;
-static thread_local std::vector<TimedLaunch> g_timed;
+static std::atomic<bool> g_timing_on{false};
+static std::mutex g_timed_mu;
+static std::vector<TimedLaunch> g_timed;
 
 struct ScopedTiming {
   hipStream_t s;
   TimedLaunch t;
   bool on;
-  ScopedTiming(int tag, hipStream_t stream) : s(stream), on(g_timing_on) {
+  ScopedTiming(int tag, hipStream_t stream) : s(stream), on(g_timing_on.load()) {
     if (!on) return;
     t.tag = tag;
     if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) {
@@ -50,6 +53,7 @@ struct ScopedTiming {
   ~ScopedTiming() {
     if (!on) return;
     (void)hipEventRecord(t.stop, s);
+    std::lock_guard<std::mutex> lock(g_timed_mu);
     g_timed.push_back(t);
   }
 };
@@ -476,7 +480,7 @@ static int64_t default_vocab_chunk(int64_t n_tokens, int64_t vocab, int64_t requ
 using namespace vamd;
 
 extern "C" int vamd_lce_timing_enable(int on) {
-  g_timing_on = on != 0;
+  g_timing_on.store(on != 0);
   return VAMD_OK;
 }
 
@@ -487,6 +491,7 @@ extern "C" int vamd_lce_timing_collect(double* ms_by_kernel, int64_t* launches_b
     launches_by_kernel[i] = 0;
   }
   int status = VAMD_OK;
+  std::lock_guard<std::mutex> lock(g_timed_mu);
   for (TimedLaunch& t : g_timed) {
     float ms = 0.f;
     if (hipEventSynchronize(t.stop) != hipSuccess || hipEventElapsedTime(&ms, t.start, t.stop) != hipSuccess) {
