@@ -208,8 +208,10 @@ def test_benchmark_config_7b_head_full_size(dev):
     assert (dh.float() - want_dh).pow(2).mean().sqrt().item() < 1.5e-3
     del want_dw, want_dh, e_dw, e_dh
     # sum_j dz_j = 0 for every token  =>  the vocabulary-axis sum of d_weight vanishes (bf16 rounding of 152064 rows)
+    # (each of the ~16384 label rows carries its own bf16 rounding error, so the sum is noise of relative size ~1e-5)
     col_sum = dw.float().sum(0)
-    assert col_sum.abs().max().item() < 0.5, col_sum.abs().max().item()
+    col_abs = dw.float().abs().sum(0)
+    assert (col_sum.abs() <= 1e-3 * col_abs).all(), (col_sum.abs() / col_abs).max().item()
     # linearity in the upstream gradient: backward(2 g) == 2 backward(g) up to output rounding
     dh2, _ = K.efficient_entropy_backward(2 * g_lp, None, hidden, weight, labels, lse, mz, 0, T, d_entropy_scalar=0.002)
     _close_bf16(dh2, 2 * dh.float(), "linearity of d_hidden")

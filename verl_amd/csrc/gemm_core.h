@@ -17,8 +17,8 @@
 // vectors.
 //
 // Each operand is staged through LDS as a [256 rows][64 k] bf16 slab (128 B per
-// row, 16-byte chunks XOR-swizzled by row % 8 so that both the staging writes
-// and the ds_read_b128 fragment reads are bank-conflict free).  Two slabs per
+// row, 16-byte chunks XOR-swizzled by the row index so that both the staging
+// writes and the ds_read_b128 fragment reads are bank-conflict free).  Two slabs per
 // operand are double-buffered: 4 x 32 KB = 128 KB of the CU's 160 KB LDS.
 //
 // An operand may live in memory either K-contiguous ("direct": element (x,k) at
@@ -92,6 +92,13 @@ __device__ __forceinline__ int acc_col(const LanePos& p, int mb, int v) {
 // Row offset inside the 256-tall tile of accumulator block nb for this lane.
 __device__ __forceinline__ int acc_row(const LanePos& p, int nb) { return p.wr * 128 + nb * 32 + p.lr; }
 
+// LDS swizzle: the 16-byte chunk c of slab row r lives at chunk position c ^ swizzle_of(r).
+// ds_read_b128 is served 16 lanes (256 B, all 64 banks) per cycle; a fragment read touches 16
+// consecutive rows at one logical chunk, i.e. 8 even and 8 odd rows (two rows span the 64
+// banks), so rows of equal parity must land on 8 different chunk positions: (r >> 1) & 7.
+// Staging writes go 8 lanes (one whole row) per cycle and are conflict free under any XOR.
+__device__ __forceinline__ int swizzle_of(int row) { return (row >> 1) & 7; }
+
 // ---------------------------------------------------------------------------------------------
 // Global -> register staging for one 256 x 64 slab of an operand.
 //
@@ -157,7 +164,7 @@ struct SlabLoader {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int row = row_in + 32 * i;
-        *reinterpret_cast<u32x4*>(slab + row * 128 + ((kc ^ (row & 7)) << 4)) = reg[i];
+        *reinterpret_cast<u32x4*>(slab + row * 128 + ((kc ^ swizzle_of(row)) << 4)) = reg[i];
       }
     } else {
       const int kg = t & 7;
@@ -173,16 +180,14 @@ struct SlabLoader {
           o[p] = (j & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
         }
         const int row = xg * 8 + j;
-        *reinterpret_cast<u32x4*>(slab + row * 128 + ((kg ^ j) << 4)) = o;
+        *reinterpret_cast<u32x4*>(slab + row * 128 + ((kg ^ swizzle_of(row)) << 4)) = o;
       }
     }
   }
 };
 
 // ---------------------------------------------------------------------------------------------
-// 4 k-steps of 16 over one pair of slabs: 8 ds_read_b128 + 16 MFMA per step.  The fragments of
-// step kk+1 are read while the MFMAs of step kk issue; scheduling barriers keep that order and
-// stop the compiler from hoisting all 32 fragment reads (128 VGPRs) to the top.
+// MFMA fragments of one 16-k step: 4 blocks of each operand, 8 ds_read_b128 per lane.
 struct Frags {
   bf16x8 c[4], r[4];
 };
@@ -202,23 +207,94 @@ __device__ __forceinline__ void mma_frags(const Frags& f, Accum& acc) {
       acc.a[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c[mb], f.r[nb], acc.a[mb][nb], 0, 0, 0);
 }
 
-__device__ __forceinline__ void slab_mma(const char* r_slab, const char* c_slab, const LanePos& p, Accum& acc) {
-  const int sw = p.lr & 7;
-  const char* r_lane = r_slab + (p.wr * 128 + p.lr) * 128;
-  const char* c_lane = c_slab + (p.wc * 128 + p.lr) * 128;
-  Frags f0, f1;
-  load_frags(f0, r_lane, c_lane, ((0 + p.lh) ^ sw) << 4);
-  __builtin_amdgcn_sched_barrier(0);
+// Workgroup barrier that only waits for this wavefront's LDS traffic: global loads issued for
+// later slabs stay in flight across it (a __syncthreads() would drain them too).
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// Scheduling hint: the next `n` instructions of class `mask` come next in program order.
+// 0x008 MFMA, 0x100 DS read, 0x200 DS write, 0x020 VMEM read, 0x002 VALU.
+#define VAMD_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
+
+// ---------------------------------------------------------------------------------------------
+// One slab (64 k) of the software pipeline.  On entry: f0 holds the step-0 fragments of this
+// slab, the staging registers of both loaders hold slab it+1 (loads issued one iteration ago),
+// `cur` is the LDS stage of this slab and `nxt` the other stage (free: its last readers passed
+// the previous barrier).  The four 16-k steps interleave, in MFMA issue shadows,
+//   step 0 : fragment reads of step 1 | R staging -> LDS(nxt) | R global loads of slab it+2
+//   step 1 : fragment reads of step 2 | C staging -> LDS(nxt) | C global loads of slab it+2
+//   step 2 : fragment reads of step 3
+//   barrier (LDS only)
+//   step 3 : step-0 fragment reads of slab it+1 from nxt
+// so neither the staging writes, nor the barrier, nor the first fragment reads of a slab sit on
+// the critical path; only MFMA issue does.
+template <bool RK, bool CK>
+__device__ __forceinline__ void slab_iter(SlabLoader<RK>& lr, SlabLoader<CK>& lc, const Operand& R, const Operand& C,
+                                          int r2, int c2, int k2, const char* cur, char* nxt, const LanePos& p,
+                                          Frags& f0, Accum& acc) {
+  const int sw = swizzle_of(p.lr);
+  const int lane_r = (p.wr * 128 + p.lr) * 128;
+  const int lane_c = kSlabBytes + (p.wc * 128 + p.lr) * 128;
+  const char* r_lane = cur + lane_r;
+  const char* c_lane = cur + lane_c;
+  Frags f1;
+  // ---- step 0
   load_frags(f1, r_lane, c_lane, ((2 + p.lh) ^ sw) << 4);
+#ifndef VAMD_DBG_NO_STORE
+  lr.store(nxt);
+#endif
+#ifndef VAMD_DBG_NO_GLOBAL
+  lr.issue(R, r2, k2);
+#endif
   mma_frags(f0, acc);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    VAMD_SGB(0x008, 1);
+    VAMD_SGB(0x100, 1);
+    if (RK) VAMD_SGB(0x002, 4);
+    VAMD_SGB(0x008, 1);
+    VAMD_SGB(0x200, 1);
+    VAMD_SGB(0x020, 1);
+  }
   __builtin_amdgcn_sched_barrier(0);
+  // ---- step 1
   load_frags(f0, r_lane, c_lane, ((4 + p.lh) ^ sw) << 4);
+#ifndef VAMD_DBG_NO_STORE
+  lc.store(nxt + kSlabBytes);
+#endif
+#ifndef VAMD_DBG_NO_GLOBAL
+  lc.issue(C, c2, k2);
+#endif
   mma_frags(f1, acc);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    VAMD_SGB(0x008, 1);
+    VAMD_SGB(0x100, 1);
+    if (CK) VAMD_SGB(0x002, 4);
+    VAMD_SGB(0x008, 1);
+    VAMD_SGB(0x200, 1);
+    VAMD_SGB(0x020, 1);
+  }
   __builtin_amdgcn_sched_barrier(0);
+  // ---- step 2
   load_frags(f1, r_lane, c_lane, ((6 + p.lh) ^ sw) << 4);
   mma_frags(f0, acc);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    VAMD_SGB(0x008, 2);
+    VAMD_SGB(0x100, 1);
+  }
   __builtin_amdgcn_sched_barrier(0);
+  lds_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  // ---- step 3
+  load_frags(f0, nxt + lane_r, nxt + lane_c, ((0 + p.lh) ^ sw) << 4);
   mma_frags(f1, acc);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    VAMD_SGB(0x008, 2);
+    VAMD_SGB(0x100, 1);
+  }
+  __builtin_amdgcn_sched_barrier(0);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -227,8 +303,9 @@ __device__ __forceinline__ void slab_mma(const char* r_slab, const char* c_slab,
 //   Sched : int count();  void tile(int i, int& r0, int& c0);
 //   Epi   : void operator()(Accum& acc, int r0, int c0);   (registers + global memory only)
 //
-// The first slab of the next tile is fetched during the last slab of the current one, so it
-// already sits in LDS while the epilogue runs and only the very first tile pays a cold start.
+// All (tile, slab) pairs of the workgroup form one stream of slabs; slab it+1 is staged into
+// LDS and slab it+2 is fetched from memory while slab it is multiplied, across tile boundaries
+// too, so only the very first slab pays a cold start and epilogues find their next slab ready.
 template <bool R_KMAJOR, bool C_KMAJOR, class Sched, class Epi>
 __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, int k_slabs, Sched& sched, Epi& epi,
                                           char* lds) {
@@ -237,51 +314,63 @@ __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, in
   const LanePos pos = lane_pos();
   SlabLoader<R_KMAJOR> lr;
   SlabLoader<C_KMAJOR> lc;
-  char* const r_buf0 = lds;
-  char* const c_buf0 = lds + kSlabBytes;
 
+  // slab 0 -> LDS stage 0
   int r0, c0;
   sched.tile(0, r0, c0);
   lr.set_tile(R, r0);
   lc.set_tile(C, c0);
   lr.issue(R, r0, 0);
   lc.issue(C, c0, 0);
-  lr.store(r_buf0);
-  lc.store(c_buf0);
-  __syncthreads();
+  lr.store(lds);
+  lc.store(lds + kSlabBytes);
+  // slab 1 -> staging registers; (t2, k2, r2, c2) then names slab 2.  Past the end of the
+  // stream the cursor stays on the last slab: the pipeline re-fetches it instead of branching.
+  int t2 = 0, k2 = 0, r2 = r0, c2 = c0;
+  bool new_tile = false;
+  auto advance = [&]() {
+    new_tile = false;
+    if (t2 == ntiles - 1 && k2 == k_slabs - 1) return;
+    if (++k2 == k_slabs) {
+      k2 = 0;
+      ++t2;
+      sched.tile(t2, r2, c2);
+      new_tile = true;
+    }
+  };
+  advance();
+  if (new_tile) {
+    lr.set_tile(R, r2);
+    lc.set_tile(C, c2);
+  }
+  lr.issue(R, r2, k2 * kBK);
+  lc.issue(C, c2, k2 * kBK);
+  advance();
+  lds_barrier();
+  Frags f0;
+  {
+    const int sw = swizzle_of(pos.lr);
+    load_frags(f0, lds + (pos.wr * 128 + pos.lr) * 128, lds + kSlabBytes + (pos.wc * 128 + pos.lr) * 128,
+               ((0 + pos.lh) ^ sw) << 4);
+  }
 
-  int stage = 0;
+  int it = 0, stage = 0;
   for (int tile = 0; tile < ntiles; ++tile) {
     Accum acc;
     accum_zero(acc);
-    int nr0 = r0, nc0 = c0;
-    const bool more_tiles = (tile + 1) < ntiles;
-    if (more_tiles) sched.tile(tile + 1, nr0, nc0);
-    for (int kt = 0; kt < k_slabs; ++kt) {
-      const bool last_slab = (kt + 1) == k_slabs;
-      const bool has_next = !last_slab || more_tiles;
-      if (has_next) {
-        if (last_slab) {
-          lr.set_tile(R, nr0);
-          lc.set_tile(C, nc0);
-          lr.issue(R, nr0, 0);
-          lc.issue(C, nc0, 0);
-        } else {
-          lr.issue(R, r0, (kt + 1) * kBK);
-          lc.issue(C, c0, (kt + 1) * kBK);
-        }
+    sched.tile(tile, r0, c0);
+    for (int kt = 0; kt < k_slabs; ++kt, ++it) {
+      const char* cur = lds + stage * 2 * kSlabBytes;
+      char* nxt = lds + (stage ^ 1) * 2 * kSlabBytes;
+      if (new_tile) {
+        lr.set_tile(R, r2);
+        lc.set_tile(C, c2);
       }
-      slab_mma(lds + stage * 2 * kSlabBytes, lds + stage * 2 * kSlabBytes + kSlabBytes, pos, acc);
-      if (has_next) {
-        lr.store(lds + (stage ^ 1) * 2 * kSlabBytes);
-        lc.store(lds + (stage ^ 1) * 2 * kSlabBytes + kSlabBytes);
-      }
-      __syncthreads();
+      slab_iter<R_KMAJOR, C_KMAJOR>(lr, lc, R, C, r2, c2, k2 * kBK, cur, nxt, pos, f0, acc);
+      advance();
       stage ^= 1;
     }
     epi(acc, r0, c0);
-    r0 = nr0;
-    c0 = nc0;
   }
 }
 
