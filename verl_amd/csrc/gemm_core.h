@@ -2,10 +2,11 @@
 // GEMM-shaped kernels of the log-prob/entropy head (forward logits, backward
 // logit recompute, dHidden, dWeight).
 //
-// One workgroup = 256 threads = 4 wavefronts laid out 2 x 2 over a 256 x 256
-// output tile; each wavefront owns a 128 x 128 sub-tile as 4 x 4 blocks of
-// v_mfma_f32_32x32x16_bf16 (256 fp32 accumulators per lane).  The tile engine
-// computes
+// One workgroup = 512 threads = 8 wavefronts (two per SIMD, so that one wavefront's
+// loads, LDS traffic and epilogue arithmetic issue in the shadow of the other's
+// MFMAs) laid out 4 x 2 over a 256 x 256 output tile; each wavefront owns a
+// 64 (rows) x 128 (columns) sub-tile as 2 x 4 blocks of v_mfma_f32_32x32x16_bf16
+// (128 fp32 accumulators per lane).  The tile engine computes
 //
 //     Out[r][c] = sum_k  R[r][k] * C[c][k]
 //
@@ -18,12 +19,12 @@
 //
 // Each operand is staged through LDS as a [256 rows][64 k] bf16 slab (128 B per
 // row, 16-byte chunks XOR-swizzled by the row index so that both the staging
-// writes and the ds_read_b128 fragment reads are bank-conflict free).  Two slabs per
-// operand are double-buffered: 4 x 32 KB = 128 KB of the CU's 160 KB LDS.
+// writes and the ds_read_b128 fragment reads are bank-conflict free).  Two slabs
+// per operand are double-buffered: 4 x 32 KB = 128 KB of the CU's 160 KB LDS.
 //
 // An operand may live in memory either K-contiguous ("direct": element (x,k) at
 // base[x*ld + k]) or K-major ("kmajor": element (x,k) at base[k*ld + x]).  The
-// kmajor loader transposes 8x8 bf16 blocks in registers on the way to LDS, so
+// kmajor loader transposes 8x4 bf16 blocks in registers on the way to LDS, so
 // no transposed copy of the weight, the hidden states or dLogits is ever
 // written to memory.
 #pragma once
@@ -39,36 +40,42 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int kTile = 256;                   // output tile edge
-constexpr int kBK = 64;                      // k extent of one slab
-constexpr int kThreads = 256;                // 4 wavefronts
-constexpr int kSlabBytes = kTile * kBK * 2;  // 32 KB
-constexpr int kLdsBytes = 4 * kSlabBytes;    // R,C x 2 stages = 128 KB
+constexpr int kTile = 256;                    // output tile edge
+constexpr int kBK = 64;                       // k extent of one slab
+constexpr int kWavesR = 4;                    // wavefronts along r
+constexpr int kWavesC = 2;                    // wavefronts along c
+constexpr int kThreads = 64 * kWavesR * kWavesC;
+constexpr int kNB = kTile / 32 / kWavesR;     // 32-row blocks per wavefront    (2)
+constexpr int kMB = kTile / 32 / kWavesC;     // 32-column blocks per wavefront (4)
+constexpr int kLoads = kTile * 8 / kThreads;  // 16-byte staging loads per lane per operand slab (4)
+constexpr int kSlabBytes = kTile * kBK * 2;   // 32 KB
+constexpr int kLdsBytes = 4 * kSlabBytes;     // R,C x 2 stages = 128 KB
+static_assert(kNB == 2 && kMB == 4 && kLoads == 4, "slab_iter's slot schedule is written for this layout");
 
 // One GEMM operand as the tile engine sees it.
 struct Operand {
   const uint16_t* base;  // bf16 bits
   int64_t ld;            // leading dimension, elements
-  int x_extent;          // valid extent along the operand's output index (rows of R / cols of C)
-  int k_extent;          // valid extent along k (only used to clamp kmajor row addresses)
+  int x_extent;          // extent along the operand's output index (rows of R / columns of C)
+  int k_extent;          // extent along k (kmajor operands: number of rows in memory)
 };
 
 struct Accum {
-  f32x16 a[4][4];  // [mb: 32-wide block along c][nb: 32-wide block along r]
+  f32x16 a[kMB][kNB];  // [mb: 32-wide block along c][nb: 32-wide block along r]
 };
 
 __device__ __forceinline__ void accum_zero(Accum& acc) {
 #pragma unroll
-  for (int mb = 0; mb < 4; ++mb)
+  for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
+    for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc.a[mb][nb][v] = 0.f;
 }
 
 // Position of the calling lane inside the workgroup tile.
 struct LanePos {
-  int wr;  // wavefront's half along r (0/1)
+  int wr;  // wavefront's quarter along r (0..3)
   int wc;  // wavefront's half along c (0/1)
   int lr;  // lane % 32 : r offset inside a 32-block
   int lh;  // lane / 32 : which 4-column group of every 8 the lane holds
@@ -78,8 +85,8 @@ __device__ __forceinline__ LanePos lane_pos() {
   LanePos p;
   const int t = threadIdx.x;
   const int w = t >> 6;
-  p.wr = w & 1;
-  p.wc = w >> 1;
+  p.wr = w % kWavesR;
+  p.wc = w / kWavesR;
   p.lr = t & 31;
   p.lh = (t >> 5) & 1;
   return p;
@@ -87,214 +94,216 @@ __device__ __forceinline__ LanePos lane_pos() {
 
 // Column offset inside the 256-wide tile of accumulator element (mb, v) for this lane.
 __device__ __forceinline__ int acc_col(const LanePos& p, int mb, int v) {
-  return p.wc * 128 + mb * 32 + 8 * (v >> 2) + 4 * p.lh + (v & 3);
+  return p.wc * (kMB * 32) + mb * 32 + 8 * (v >> 2) + 4 * p.lh + (v & 3);
 }
 // Row offset inside the 256-tall tile of accumulator block nb for this lane.
-__device__ __forceinline__ int acc_row(const LanePos& p, int nb) { return p.wr * 128 + nb * 32 + p.lr; }
+__device__ __forceinline__ int acc_row(const LanePos& p, int nb) { return p.wr * (kNB * 32) + nb * 32 + p.lr; }
 
 // LDS swizzle: the 16-byte chunk c of slab row r lives at chunk position c ^ swizzle_of(r).
 // ds_read_b128 is served 16 lanes (256 B, all 64 banks) per cycle; a fragment read touches 16
 // consecutive rows at one logical chunk, i.e. 8 even and 8 odd rows (two rows span the 64
 // banks), so rows of equal parity must land on 8 different chunk positions: (r >> 1) & 7.
-// Staging writes go 8 lanes (one whole row) per cycle and are conflict free under any XOR.
+// Staging writes cover whole 128 B rows with consecutive lanes and are conflict free under
+// any XOR of the chunk index.
 __device__ __forceinline__ int swizzle_of(int row) { return (row >> 1) & 7; }
 
 // ---------------------------------------------------------------------------------------------
-// Global -> register staging for one 256 x 64 slab of an operand.
+// Where one slab of an operand comes from: a buffer resource whose base is the operand's tile
+// origin, plus the scalar byte offset of the slab's first k.  Reads past the end of the operand
+// return zero (buffer bounds check), which is what rows / k beyond the valid extent must
+// contribute, so the loaders carry no clamping arithmetic.
+struct SlabSrc {
+  __amdgpu_buffer_rsrc_t rsrc;
+  unsigned soff;
+};
+
+template <bool KMAJOR>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const Operand& op, int x0) {
+  // direct: rows x0.. of [x_extent][ld];  kmajor: columns x0.. of [k_extent][ld]
+  const int64_t first = KMAJOR ? (int64_t)x0 : (int64_t)x0 * op.ld;
+  const int64_t total = (KMAJOR ? (int64_t)op.k_extent : (int64_t)op.x_extent) * op.ld;
+  int64_t bytes = (total - first) * 2;
+  if (bytes < 0) bytes = 0;
+  if (bytes > 0xffffffffll) bytes = 0xffffffffll;
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(op.base + first), 0, (int)(unsigned)bytes, 0x00020000);
+}
+
+template <bool KMAJOR>
+__device__ __forceinline__ unsigned slab_soff(const Operand& op, int k0) {
+  return KMAJOR ? (unsigned)k0 * ((unsigned)op.ld * 2u) : (unsigned)k0 * 2u;
+}
+
+// Global -> register -> LDS staging for one 256 x 64 slab of an operand: 4 x 16 bytes per lane.
 //
-// Addresses are formed as (wave-uniform 64-bit base) + (per-lane 32-bit byte offset) so that the
-// loads use the scalar-base addressing form and cost one VGPR of address each.  Direct operands
-// use tile-relative offsets (no size limit); kmajor operands use offsets from the operand base
-// (the host checks that a kmajor operand spans less than 4 GiB).
+// direct : load i is row (t/8 + 64 i), 16-byte chunk t%8 of the slab; 8 lanes fetch one 128 B row
+//          and store i writes load i as one 16-byte chunk.
+// kmajor : thread (kq = t%16, xg = t/16) owns the 8(x) x 4(k) block at x = 8 xg, k = 4 kq; load i
+//          is the 8 x-values of k = 4 kq + i; the block is transposed in registers and store j
+//          writes the 4 k-values of x = 8 xg + j as one 8-byte half chunk, so no transposed copy
+//          of an operand ever exists in memory.
+// Either way the per-lane address is ONE 32-bit offset; everything that changes between loads,
+// slabs and tiles is scalar (buffer resource + scalar offset).
 template <bool KMAJOR>
 struct SlabLoader {
-  u32x4 reg[8];
-  unsigned off[KMAJOR ? 1 : 8];
+  static constexpr int kStores = KMAJOR ? 8 : kLoads;
+  u32x4 reg[kLoads];
+  unsigned voff;     // per-lane byte offset of load 0 inside the tile
+  unsigned step;     // scalar byte offset between consecutive loads
+  unsigned lds_off;  // per-lane byte offset of store 0 inside a slab
+  unsigned lds_xor;  // kmajor: chunk position before the (j >> 1) XOR
 
-  __device__ __forceinline__ void set_tile(const Operand& op, int x0) {
-    const int t = threadIdx.x;
+  __device__ __forceinline__ void init(const Operand& op) {
+    const unsigned t = threadIdx.x;
+    const unsigned ld_bytes = (unsigned)op.ld * 2u;
     if constexpr (!KMAJOR) {
-      // chunk id c = t + 256*i : row = c / 8, 16-byte chunk kc = c % 8
-      const int kc = t & 7;
-      const int row_in = t >> 3;
-      const int last = op.x_extent - 1 - x0;
-      const unsigned ld_bytes = (unsigned)op.ld * 2u;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        int row = row_in + 32 * i;
-        row = row < last ? row : last;
-        off[i] = (unsigned)row * ld_bytes + (unsigned)kc * 16u;
-      }
+      const unsigned kc = t & 7, row = t >> 3;  // rows 0..63, + 64 per load
+      voff = row * ld_bytes + kc * 16u;
+      step = 64u * ld_bytes;
+      // swizzle_of(row + 64 i) == swizzle_of(row): one LDS offset serves all four stores
+      lds_off = row * 128u + ((kc ^ (unsigned)swizzle_of((int)row)) << 4);
+      lds_xor = 0;
     } else {
-      // one 8(x) x 8(k) block per thread: kg = t % 8, xg = t / 8
-      const int xg = t >> 3;
-      int xcol = x0 + xg * 8;
-      const int xlast = op.x_extent - 8;
-      xcol = xcol < xlast ? xcol : xlast;
-      off[0] = (unsigned)xcol * 2u;
+      const unsigned kq = t & 15, xg = t >> 4;
+      voff = kq * 4u * ld_bytes + xg * 16u;
+      step = ld_bytes;
+      lds_off = xg * 1024u + (kq & 1u) * 8u;
+      lds_xor = (kq >> 1) ^ ((xg & 1u) << 2);  // swizzle_of(8 xg + j) = ((xg & 1) << 2) | (j >> 1)
     }
   }
 
-  // x0: first output index of the tile, k0: first k of the slab.
-  __device__ __forceinline__ void issue(const Operand& op, int x0, int k0) {
-    if constexpr (!KMAJOR) {
-      const char* tile = reinterpret_cast<const char*>(op.base + (int64_t)x0 * op.ld + k0);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) reg[i] = *reinterpret_cast<const u32x4*>(tile + off[i]);
-    } else {
-      const char* base = reinterpret_cast<const char*>(op.base);
-      const int kg = threadIdx.x & 7;
-      const int klast = op.k_extent - 1;
-      const unsigned ld_bytes = (unsigned)op.ld * 2u;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        int k = k0 + kg * 8 + i;
-        k = k < klast ? k : klast;
-        reg[i] = *reinterpret_cast<const u32x4*>(base + ((unsigned)k * ld_bytes + off[0]));
-      }
-    }
+  __device__ __forceinline__ void issue_one(int i, const SlabSrc& src) {
+    reg[i] = __builtin_amdgcn_raw_buffer_load_b128(src.rsrc, (int)voff, (int)(src.soff + (unsigned)i * step), 0);
   }
 
-  // Write the staged slab into LDS in the [row][k] swizzled layout.
-  __device__ __forceinline__ void store(char* slab) const {
-    const int t = threadIdx.x;
+  __device__ __forceinline__ void store_one(int j, char* slab) const {
     if constexpr (!KMAJOR) {
-      const int kc = t & 7;
-      const int row_in = t >> 3;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int row = row_in + 32 * i;
-        *reinterpret_cast<u32x4*>(slab + row * 128 + ((kc ^ swizzle_of(row)) << 4)) = reg[i];
-      }
+      *reinterpret_cast<u32x4*>(slab + lds_off + j * 8192) = reg[j];
     } else {
-      const int kg = t & 7;
-      const int xg = t >> 3;
+      // x = 8 xg + j : bf16 #j of each of the 4 loads (k = 4 kq .. 4 kq + 3)
+      u32x2 o;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        // output row j of the block: the 8 k values of x = xg*8 + j
-        u32x4 o;
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-          const unsigned lo = reg[2 * p][j >> 1];
-          const unsigned hi = reg[2 * p + 1][j >> 1];
-          o[p] = (j & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
-        }
-        const int row = xg * 8 + j;
-        *reinterpret_cast<u32x4*>(slab + row * 128 + ((kg ^ swizzle_of(row)) << 4)) = o;
+      for (int p = 0; p < 2; ++p) {
+        const unsigned lo = reg[2 * p][j >> 1];
+        const unsigned hi = reg[2 * p + 1][j >> 1];
+        o[p] = (j & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
       }
+      *reinterpret_cast<u32x2*>(slab + lds_off + j * 128 + ((lds_xor ^ (unsigned)(j >> 1)) << 4)) = o;
     }
   }
 };
 
 // ---------------------------------------------------------------------------------------------
-// MFMA fragments of one 16-k step: 4 blocks of each operand, 8 ds_read_b128 per lane.
+// MFMA fragments of one 16-k step: kMB blocks of C and kNB blocks of R, 6 ds_read_b128 per lane.
 struct Frags {
-  bf16x8 c[4], r[4];
+  bf16x8 c[kMB], r[kNB];
 };
-
-__device__ __forceinline__ void load_frags(Frags& f, const char* r_lane, const char* c_lane, int chunk) {
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb) f.c[mb] = *reinterpret_cast<const bf16x8*>(c_lane + mb * 4096 + chunk);
-#pragma unroll
-  for (int nb = 0; nb < 4; ++nb) f.r[nb] = *reinterpret_cast<const bf16x8*>(r_lane + nb * 4096 + chunk);
-}
-
-__device__ __forceinline__ void mma_frags(const Frags& f, Accum& acc) {
-#pragma unroll
-  for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
-      acc.a[mb][nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.c[mb], f.r[nb], acc.a[mb][nb], 0, 0, 0);
-}
 
 // Workgroup barrier that only waits for this wavefront's LDS traffic: global loads issued for
 // later slabs stay in flight across it (a __syncthreads() would drain them too).
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// Scheduling hint: the next `n` instructions of class `mask` come next in program order.
-// 0x008 MFMA, 0x100 DS read, 0x200 DS write, 0x020 VMEM read, 0x002 VALU.
-#define VAMD_SGB(mask, n) __builtin_amdgcn_sched_group_barrier(mask, n, 0)
-
 // ---------------------------------------------------------------------------------------------
-// One slab (64 k) of the software pipeline.  On entry: f0 holds the step-0 fragments of this
-// slab, the staging registers of both loaders hold slab it+1 (loads issued one iteration ago),
-// `cur` is the LDS stage of this slab and `nxt` the other stage (free: its last readers passed
-// the previous barrier).  The four 16-k steps interleave, in MFMA issue shadows,
-//   step 0 : fragment reads of step 1 | R staging -> LDS(nxt) | R global loads of slab it+2
-//   step 1 : fragment reads of step 2 | C staging -> LDS(nxt) | C global loads of slab it+2
-//   step 2 : fragment reads of step 3
-//   barrier (LDS only)
-//   step 3 : step-0 fragment reads of slab it+1 from nxt
-// so neither the staging writes, nor the barrier, nor the first fragment reads of a slab sit on
-// the critical path; only MFMA issue does.
+// One slab (64 k = four 16-k steps of 8 MFMAs per wavefront) of the software pipeline.
+//
+// The body is written as 32 slots "one MFMA + a few short memory instructions", each closed by
+// a scheduling barrier so the compiler keeps the order; memory instructions are spread evenly so
+// the vector-memory and LDS pipes see a steady duty instead of bursts:
+//
+//   step 0 : fragment reads of step 1 | R staging -> LDS(nxt)  | loads C[2..3] of slab it+1
+//   step 1 : fragment reads of step 2 |                        | loads R[0..1] of slab it+2
+//   step 2 : fragment reads of step 3 | C staging -> LDS(nxt)  | loads R[2..3] of slab it+2
+//   -- LDS-only barrier --
+//   step 3 : step-0 fragment reads of slab it+1 from nxt       | loads C[0..1] of slab it+2
+//
+// Every staging register has at least two steps between its load and its LDS write, and
+// neither the barrier nor the first fragment reads of a slab sit at the head of the stream.
 template <bool RK, bool CK>
-__device__ __forceinline__ void slab_iter(SlabLoader<RK>& lr, SlabLoader<CK>& lc, const Operand& R, const Operand& C,
-                                          int r2, int c2, int k2, const char* cur, char* nxt, const LanePos& p,
-                                          Frags& f0, Accum& acc) {
+__device__ __forceinline__ void slab_iter(SlabLoader<RK>& lr, SlabLoader<CK>& lc, const SlabSrc& c1,
+                                          const SlabSrc& r2, const SlabSrc& c2, const char* cur, char* nxt,
+                                          const LanePos& p, Frags& f0, Accum& acc) {
   const int sw = swizzle_of(p.lr);
-  const int lane_r = (p.wr * 128 + p.lr) * 128;
-  const int lane_c = kSlabBytes + (p.wc * 128 + p.lr) * 128;
-  const char* r_lane = cur + lane_r;
-  const char* c_lane = cur + lane_c;
+  const int lane_r = (p.wr * (kNB * 32) + p.lr) * 128;
+  const int lane_c = kSlabBytes + (p.wc * (kMB * 32) + p.lr) * 128;
   Frags f1;
-  // ---- step 0
-  load_frags(f1, r_lane, c_lane, ((2 + p.lh) ^ sw) << 4);
+#define VAMD_MFMA(F, i)                                                                                            \
+  acc.a[(i) >> 1][(i) & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F.c[(i) >> 1], F.r[(i) & 1],                    \
+                                                                     acc.a[(i) >> 1][(i) & 1], 0, 0, 0)
+#define VAMD_FRAG(G, base, i, chunk)                                                                    \
+  do {                                                                                                  \
+    if ((i) < kMB) G.c[(i)] = *reinterpret_cast<const bf16x8*>((base) + lane_c + (i) * 4096 + (chunk));  \
+    else if ((i) < kMB + kNB)                                                                           \
+      G.r[(i) - kMB] = *reinterpret_cast<const bf16x8*>((base) + lane_r + ((i) - kMB) * 4096 + (chunk)); \
+  } while (0)
+#define VAMD_SLOT_END __builtin_amdgcn_sched_barrier(0)
+  constexpr int kRS = SlabLoader<RK>::kStores, kCS = SlabLoader<CK>::kStores;
+
+  // ---- step 0 : MFMA(f0); f1 <- step 1 fragments; R staging -> nxt; C[2..3] of slab it+1
+  {
+    const int chunk = ((2 + p.lh) ^ sw) << 4;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      VAMD_MFMA(f0, i);
+      VAMD_FRAG(f1, cur, i, chunk);
 #ifndef VAMD_DBG_NO_STORE
-  lr.store(nxt);
+      if (kRS == 8 || i < 4) lr.store_one(i, nxt);
 #endif
 #ifndef VAMD_DBG_NO_GLOBAL
-  lr.issue(R, r2, k2);
+      if (i == 5) lc.issue_one(2, c1);
+      if (i == 7) lc.issue_one(3, c1);
 #endif
-  mma_frags(f0, acc);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    VAMD_SGB(0x008, 1);
-    VAMD_SGB(0x100, 1);
-    if (RK) VAMD_SGB(0x002, 4);
-    VAMD_SGB(0x008, 1);
-    VAMD_SGB(0x200, 1);
-    VAMD_SGB(0x020, 1);
+      VAMD_SLOT_END;
+    }
   }
-  __builtin_amdgcn_sched_barrier(0);
-  // ---- step 1
-  load_frags(f0, r_lane, c_lane, ((4 + p.lh) ^ sw) << 4);
+  // ---- step 1 : MFMA(f1); f0 <- step 2 fragments; R[0..1] of slab it+2
+  {
+    const int chunk = ((4 + p.lh) ^ sw) << 4;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      VAMD_MFMA(f1, i);
+      VAMD_FRAG(f0, cur, i, chunk);
+#ifndef VAMD_DBG_NO_GLOBAL
+      if (i == 1) lr.issue_one(0, r2);
+      if (i == 5) lr.issue_one(1, r2);
+#endif
+      VAMD_SLOT_END;
+    }
+  }
+  // ---- step 2 : MFMA(f0); f1 <- step 3 fragments; C staging -> nxt; R[2..3] of slab it+2
+  {
+    const int chunk = ((6 + p.lh) ^ sw) << 4;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      VAMD_MFMA(f0, i);
+      VAMD_FRAG(f1, cur, i, chunk);
 #ifndef VAMD_DBG_NO_STORE
-  lc.store(nxt + kSlabBytes);
+      if (kCS == 8 || i < 4) lc.store_one(i, nxt + kSlabBytes);
 #endif
 #ifndef VAMD_DBG_NO_GLOBAL
-  lc.issue(C, c2, k2);
+      if (i == 5) lr.issue_one(2, r2);
+      if (i == 7) lr.issue_one(3, r2);
 #endif
-  mma_frags(f1, acc);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    VAMD_SGB(0x008, 1);
-    VAMD_SGB(0x100, 1);
-    if (CK) VAMD_SGB(0x002, 4);
-    VAMD_SGB(0x008, 1);
-    VAMD_SGB(0x200, 1);
-    VAMD_SGB(0x020, 1);
+      VAMD_SLOT_END;
+    }
   }
-  __builtin_amdgcn_sched_barrier(0);
-  // ---- step 2
-  load_frags(f1, r_lane, c_lane, ((6 + p.lh) ^ sw) << 4);
-  mma_frags(f0, acc);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    VAMD_SGB(0x008, 2);
-    VAMD_SGB(0x100, 1);
-  }
-  __builtin_amdgcn_sched_barrier(0);
   lds_barrier();
-  __builtin_amdgcn_sched_barrier(0);
-  // ---- step 3
-  load_frags(f0, nxt + lane_r, nxt + lane_c, ((0 + p.lh) ^ sw) << 4);
-  mma_frags(f1, acc);
+  VAMD_SLOT_END;
+  // ---- step 3 : MFMA(f1); f0 <- step 0 fragments of the next slab; C[0..1] of slab it+2
+  {
+    const int chunk = ((0 + p.lh) ^ sw) << 4;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    VAMD_SGB(0x008, 2);
-    VAMD_SGB(0x100, 1);
+    for (int i = 0; i < 8; ++i) {
+      VAMD_MFMA(f1, i);
+      VAMD_FRAG(f0, nxt, i, chunk);
+#ifndef VAMD_DBG_NO_GLOBAL
+      if (i == 1) lc.issue_one(0, c2);
+      if (i == 5) lc.issue_one(1, c2);
+#endif
+      VAMD_SLOT_END;
+    }
   }
-  __builtin_amdgcn_sched_barrier(0);
+#undef VAMD_MFMA
+#undef VAMD_FRAG
+#undef VAMD_SLOT_END
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -306,6 +315,8 @@ __device__ __forceinline__ void slab_iter(SlabLoader<RK>& lr, SlabLoader<CK>& lc
 // All (tile, slab) pairs of the workgroup form one stream of slabs; slab it+1 is staged into
 // LDS and slab it+2 is fetched from memory while slab it is multiplied, across tile boundaries
 // too, so only the very first slab pays a cold start and epilogues find their next slab ready.
+// Past the end of the stream the fetch cursor stays on the last slab (two redundant fetches)
+// instead of branching, which keeps the loop body a single basic block.
 template <bool R_KMAJOR, bool C_KMAJOR, class Sched, class Epi>
 __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, int k_slabs, Sched& sched, Epi& epi,
                                           char* lds) {
@@ -314,59 +325,75 @@ __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, in
   const LanePos pos = lane_pos();
   SlabLoader<R_KMAJOR> lr;
   SlabLoader<C_KMAJOR> lc;
+  lr.init(R);
+  lc.init(C);
 
-  // slab 0 -> LDS stage 0
-  int r0, c0;
+  // fetch cursor: (t2, k2) names the slab whose sources are (src_r, src_c)
+  int t2 = 0, k2 = 0, r0, c0;
   sched.tile(0, r0, c0);
-  lr.set_tile(R, r0);
-  lc.set_tile(C, c0);
-  lr.issue(R, r0, 0);
-  lc.issue(C, c0, 0);
-  lr.store(lds);
-  lc.store(lds + kSlabBytes);
-  // slab 1 -> staging registers; (t2, k2, r2, c2) then names slab 2.  Past the end of the
-  // stream the cursor stays on the last slab: the pipeline re-fetches it instead of branching.
-  int t2 = 0, k2 = 0, r2 = r0, c2 = c0;
-  bool new_tile = false;
+  __amdgpu_buffer_rsrc_t rs_r = tile_rsrc<R_KMAJOR>(R, r0), rs_c = tile_rsrc<C_KMAJOR>(C, c0);
+  SlabSrc src_r{rs_r, 0u}, src_c{rs_c, 0u};
   auto advance = [&]() {
-    new_tile = false;
     if (t2 == ntiles - 1 && k2 == k_slabs - 1) return;
     if (++k2 == k_slabs) {
       k2 = 0;
       ++t2;
-      sched.tile(t2, r2, c2);
-      new_tile = true;
+      int tr, tc;
+      sched.tile(t2, tr, tc);
+      rs_r = tile_rsrc<R_KMAJOR>(R, tr);
+      rs_c = tile_rsrc<C_KMAJOR>(C, tc);
     }
+#ifdef VAMD_DBG_SAME_SLAB
+    src_r = SlabSrc{rs_r, 0u};
+    src_c = SlabSrc{rs_c, (unsigned)(k2 & 1) * 128u};
+#else
+    src_r = SlabSrc{rs_r, slab_soff<R_KMAJOR>(R, k2 * kBK)};
+    src_c = SlabSrc{rs_c, slab_soff<C_KMAJOR>(C, k2 * kBK)};
+#endif
   };
-  advance();
-  if (new_tile) {
-    lr.set_tile(R, r2);
-    lc.set_tile(C, c2);
+
+  // slab 0 -> LDS stage 0
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) {
+    lr.issue_one(i, src_r);
+    lc.issue_one(i, src_c);
   }
-  lr.issue(R, r2, k2 * kBK);
-  lc.issue(C, c2, k2 * kBK);
+#pragma unroll
+  for (int j = 0; j < SlabLoader<R_KMAJOR>::kStores; ++j) lr.store_one(j, lds);
+#pragma unroll
+  for (int j = 0; j < SlabLoader<C_KMAJOR>::kStores; ++j) lc.store_one(j, lds + kSlabBytes);
+  // slab 1 -> staging registers, except C[2..3] which the first iteration fetches itself
   advance();
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) lr.issue_one(i, src_r);
+#pragma unroll
+  for (int i = 0; i < kLoads / 2; ++i) lc.issue_one(i, src_c);
+  SlabSrc c1 = src_c;
+  advance();  // cursor now on slab 2
   lds_barrier();
   Frags f0;
   {
     const int sw = swizzle_of(pos.lr);
-    load_frags(f0, lds + (pos.wr * 128 + pos.lr) * 128, lds + kSlabBytes + (pos.wc * 128 + pos.lr) * 128,
-               ((0 + pos.lh) ^ sw) << 4);
+    const int chunk = ((0 + pos.lh) ^ sw) << 4;
+#pragma unroll
+    for (int i = 0; i < kMB; ++i)
+      f0.c[i] = *reinterpret_cast<const bf16x8*>(lds + kSlabBytes + (pos.wc * (kMB * 32) + pos.lr) * 128 + i * 4096 +
+                                                 chunk);
+#pragma unroll
+    for (int i = 0; i < kNB; ++i)
+      f0.r[i] = *reinterpret_cast<const bf16x8*>(lds + (pos.wr * (kNB * 32) + pos.lr) * 128 + i * 4096 + chunk);
   }
 
-  int it = 0, stage = 0;
+  int stage = 0;
   for (int tile = 0; tile < ntiles; ++tile) {
     Accum acc;
     accum_zero(acc);
     sched.tile(tile, r0, c0);
-    for (int kt = 0; kt < k_slabs; ++kt, ++it) {
+    for (int kt = 0; kt < k_slabs; ++kt) {
       const char* cur = lds + stage * 2 * kSlabBytes;
       char* nxt = lds + (stage ^ 1) * 2 * kSlabBytes;
-      if (new_tile) {
-        lr.set_tile(R, r2);
-        lc.set_tile(C, c2);
-      }
-      slab_iter<R_KMAJOR, C_KMAJOR>(lr, lc, R, C, r2, c2, k2 * kBK, cur, nxt, pos, f0, acc);
+      slab_iter<R_KMAJOR, C_KMAJOR>(lr, lc, c1, src_r, src_c, cur, nxt, pos, f0, acc);
+      c1 = src_c;
       advance();
       stage ^= 1;
     }

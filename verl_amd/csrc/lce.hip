@@ -80,22 +80,22 @@ struct SplitSched {
   }
 };
 
-// Per-lane online-softmax state for the 4 token slots (nb) the lane owns.
+// Per-lane online-softmax state for the kNB token slots (nb) the lane owns.
 struct FwdEpi {
   LanePos p;
   float scale2;
   int vocab;
-  float m[4], s[4], sy[4], zl[4];
-  int lab[4];
+  float m[kNB], s[kNB], sy[kNB], zl[kNB];
+  int lab[kNB];
 
   __device__ __forceinline__ void operator()(Accum& acc, int /*r0*/, int c0) {
     const bool ragged = c0 + kTile > vocab;
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
+    for (int nb = 0; nb < kNB; ++nb) {
       float ymax = kNegBig;
       // pass 1: scale into the log2 domain in place, mask the vocabulary tail, tile max
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
+      for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           float y = acc.a[mb][nb][v] * scale2;
@@ -107,7 +107,7 @@ struct FwdEpi {
       const int rel = lab[nb] - c0 - p.wc * 128;
       if (__any(rel >= 0 && rel < 128)) {
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
+        for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
             const int col = mb * 32 + 8 * (v >> 2) + 4 * p.lh + (v & 3);
@@ -118,7 +118,7 @@ struct FwdEpi {
       const float resc = fast_exp2(m[nb] - m_new);
       float s_ = s[nb] * resc, sy_ = sy[nb] * resc;
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
+      for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const float y = acc.a[mb][nb][v];
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
   epi.scale2 = a.scale2;
   epi.vocab = a.vocab;
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
+  for (int nb = 0; nb < kNB; ++nb) {
     epi.m[nb] = kNegBig;
     epi.s[nb] = 0.f;
     epi.sy[nb] = 0.f;
@@ -177,7 +177,7 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
 
   // merge the two lane halves (they hold disjoint vocabulary columns of the same token) ...
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
+  for (int nb = 0; nb < kNB; ++nb) {
     const float m2 = __shfl_xor(epi.m[nb], 32, 64);
     const float s2 = __shfl_xor(epi.s[nb], 32, 64);
     const float sy2 = __shfl_xor(epi.sy[nb], 32, 64);
@@ -185,15 +185,15 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
     merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], m2, s2, sy2);
     epi.zl[nb] += z2;
   }
-  // ... then the two wavefronts that share a token half (wc = 0/1), through LDS.
+  // ... then the two wavefronts that share a token quarter (wc = 0/1), through LDS.
   float4* red = reinterpret_cast<float4*>(lds);  // [2][256]
   if (epi.p.lh == 0) {
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
+    for (int nb = 0; nb < kNB; ++nb)
       red[epi.p.wc * kTile + acc_row(epi.p, nb)] = make_float4(epi.m[nb], epi.s[nb], epi.sy[nb], epi.zl[nb]);
   }
   __syncthreads();
-  {
+  if (threadIdx.x < kTile) {
     const int t = threadIdx.x;
     float4 x = red[t], y = red[kTile + t];
     merge_state(x.x, x.y, x.z, y.x, y.y, y.z);
@@ -265,7 +265,7 @@ struct RecomputeEpi {
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const RecomputeArgs& A = *a;
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
+    for (int nb = 0; nb < kNB; ++nb) {
       const int tok = r0 + acc_row(p, nb);
       const bool live = tok < A.n_tokens;
       float lse2 = 0.f, mz = 0.f, glp = 0.f, gent = 0.f;
@@ -280,7 +280,7 @@ struct RecomputeEpi {
       const bool hit = __any(rel >= 0 && rel < 128);
       uint16_t* out_row = A.dz + (int64_t)tok * A.dz_ld + c0;
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
+      for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           float d[4];
@@ -336,11 +336,11 @@ struct DHiddenEpi {
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const GemmOutArgs& A = *a;
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
+    for (int nb = 0; nb < kNB; ++nb) {
       const int row = r0 + acc_row(p, nb);
       if (row >= A.r_valid) continue;
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
+      for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int col = c0 + p.wc * 128 + mb * 32 + 8 * g + 4 * p.lh;
@@ -368,11 +368,11 @@ struct DWeightEpi {
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const GemmOutArgs& A = *a;
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb) {
+    for (int nb = 0; nb < kNB; ++nb) {
       const int row = r0 + acc_row(p, nb);
       if (row >= A.r_valid) continue;
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
+      for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int col = c0 + p.wc * 128 + mb * 32 + 8 * g + 4 * p.lh;
