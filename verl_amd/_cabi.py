@@ -119,7 +119,25 @@ def ptr(t: torch.Tensor | None):
 
 
 def workspace(nbytes: int, device: torch.device) -> torch.Tensor:
+    """Uninitialised scratch for the head kernels."""
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+_ticket_ws: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def ticket_workspace(nbytes: int, device: torch.device) -> torch.Tensor:
+    """Scratch for the single-launch reductions.  Their contract: the first 256 bytes (a ticket
+    counter) are zero on entry and zero again on exit, so one zero-initialised buffer per
+    (device, stream) is kept and reused; kernels on one stream run in order and never share it."""
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr(device))
+    need = max(int(nbytes), 4096)
+    with _lock:
+        buf = _ticket_ws.get(key)
+        if buf is None or buf.numel() < need:
+            buf = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
+            _ticket_ws[key] = buf
+    return buf
 
 
 def mask_code(mask: torch.Tensor) -> tuple[torch.Tensor, int]:

@@ -49,10 +49,6 @@ struct Carver {
 
 int device_cu_count();
 
-// Sums [rows][chunks][4] double records (defined next to the masked-moments kernels).
-int launch_moments_finalize(const double* partials, int64_t rows, int chunks, int per_row, double* out,
-                            hipStream_t stream);
-
 // mask element -> (weight, member) following masked_sum: weight = (float)m, member = m != 0
 template <class M>
 __device__ __forceinline__ float mask_weight(M m) {

@@ -9,7 +9,10 @@
 // into segments of 1024 columns walked right to left; inside a segment each of the 256 threads
 // composes its 4 columns, a wavefront scan (shuffles) plus a 4-entry LDS pass yields every
 // thread's incoming state, and the thread then replays its 4 columns to emit the advantages.
-// Loads and stores are float4 and contiguous across the wavefront.
+// Loads and stores are float4 and contiguous across the wavefront; the loads of four segments
+// are issued together so that memory latency is paid once per 4096 columns.  The workgroup that
+// finishes last folds the per-row masked moments and writes the whitening statistics, so the
+// whole estimator is two launches (scan, then the elementwise whitening).
 #include "rowchunk.h"
 
 namespace vamd {
@@ -42,14 +45,20 @@ __device__ __forceinline__ Affine shfl_up_affine(const Affine& x, int d) {
 }
 
 constexpr int kSeg = 1024;  // columns per segment = 256 threads x 4
+constexpr int kSegBatch = 4;  // segments whose loads are issued together (48 KiB in flight per workgroup)
+
+struct GaeWork {
+  unsigned* ticket;   // workspace head: zero on entry, zero on exit
+  double* partials;   // [rows][4] masked moments of the raw advantages
+};
 
 template <bool VEC, class M>
 __global__ __launch_bounds__(kRcThreads) void gae_scan_kernel(const float* __restrict__ rewards,
                                                               const float* __restrict__ values,
-                                                              const M* __restrict__ mask, int64_t cols, float gamma,
-                                                              float gl, float* __restrict__ adv,
-                                                              float* __restrict__ ret,
-                                                              double* __restrict__ partials) {
+                                                              const M* __restrict__ mask, int64_t rows, int64_t cols,
+                                                              float gamma, float gl, float* __restrict__ adv,
+                                                              float* __restrict__ ret, GaeWork wk,
+                                                              double* __restrict__ moments, float* __restrict__ stats) {
   const int64_t row = blockIdx.x;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -64,100 +73,116 @@ __global__ __launch_bounds__(kRcThreads) void gae_scan_kernel(const float* __res
   const int nseg = (int)((cols + kSeg - 1) / kSeg);
   int par = 0;
   __syncthreads();
-  for (int seg = nseg - 1; seg >= 0; --seg, par ^= 1) {
-    const int64_t c = (int64_t)seg * kSeg + slot * 4;
-    const int64_t left = cols - c;
-    const int valid = left >= 4 ? 4 : (left > 0 ? (int)left : 0);
-    float r[4] = {0, 0, 0, 0}, v[4] = {0, 0, 0, 0}, w[4] = {0, 0, 0, 0};
-    if (valid > 0) {
-      const int64_t i = row * cols + c;
-      if (VEC) {
-        ld4<true>(rewards, i, 4, r);
-        ld4<true>(values, i, 4, v);
-        ldmask4<true>(mask, i, 4, w);
-      } else {
-        ld4<false>(rewards, i, valid, r);
-        ld4<false>(values, i, valid, v);
-        ldmask4<false>(mask, i, valid, w);
-      }
-    }
-    // this thread's 4 columns as one map (right to left: e = 3 .. 0)
-    Affine f = affine_identity();
+  for (int top = nseg - 1; top >= 0; top -= kSegBatch) {
+    // issue every load of up to kSegBatch segments before touching any of them
+    float r[kSegBatch][4], v[kSegBatch][4], w[kSegBatch][4];
+    int valid[kSegBatch];
 #pragma unroll
-    for (int e = 3; e >= 0; --e) {
-      if (w[e] != 0.f) {
-        Affine n;
-        n.a = 0.f;
-        n.b = v[e];
-        n.P = fmaf(gl, f.P, gamma * f.a);
-        n.Q = gl * f.Q;
-        n.R = fmaf(gamma, f.b, fmaf(gl, f.R, r[e] - v[e]));
-        f = n;
-      }
-    }
-    // inclusive scan over the wavefront (lane order = walk order)
-    Affine inc = f;
+    for (int b = 0; b < kSegBatch; ++b) {
+      const int seg = top - b;
+      const int64_t c = (int64_t)seg * kSeg + slot * 4;
+      const int64_t left = cols - c;
+      valid[b] = seg < 0 ? 0 : (left >= 4 ? 4 : (left > 0 ? (int)left : 0));
 #pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const Affine nb = shfl_up_affine(inc, d);
-      if (lane >= d) inc = compose(inc, nb);
+      for (int e = 0; e < 4; ++e) r[b][e] = v[b][e] = w[b][e] = 0.f;
+      if (valid[b] > 0) {
+        const int64_t i = row * cols + c;
+        ld4<VEC>(rewards, i, valid[b], r[b]);
+        ld4<VEC>(values, i, valid[b], v[b]);
+        ldmask4<VEC>(mask, i, valid[b], w[b]);
+      }
     }
-    if (lane == 63) wave_tot[par][wave] = inc;
-    Affine exc = shfl_up_affine(inc, 1);
-    if (lane == 0) exc = affine_identity();
-    __syncthreads();
-    // state entering this wavefront, then this thread
-    float nv = carry[par][0], g = carry[par][1];
-    for (int k = 0; k < wave; ++k) {
-      const Affine t = wave_tot[par][k];
-      const float nv2 = fmaf(t.a, nv, t.b);
-      g = fmaf(t.P, nv, fmaf(t.Q, g, t.R));
-      nv = nv2;
-    }
-    {
-      const float nv2 = fmaf(exc.a, nv, exc.b);
-      g = fmaf(exc.P, nv, fmaf(exc.Q, g, exc.R));
-      nv = nv2;
-    }
-    // replay the 4 columns
-    float a_out[4], r_out[4];
 #pragma unroll
-    for (int e = 3; e >= 0; --e) {
-      if (w[e] != 0.f) {
-        const float delta = r[e] + gamma * nv - v[e];
-        g = fmaf(gl, g, delta);
-        nv = v[e];
-        m1 += g * w[e];
-        m2 += g * g * w[e];
-        mc += 1.f;
+    for (int b = 0; b < kSegBatch; ++b) {
+      const int seg = top - b;
+      if (seg < 0) break;
+      // this thread's 4 columns as one map (right to left: e = 3 .. 0)
+      Affine f = affine_identity();
+#pragma unroll
+      for (int e = 3; e >= 0; --e) {
+        if (w[b][e] != 0.f) {
+          Affine n;
+          n.a = 0.f;
+          n.b = v[b][e];
+          n.P = fmaf(gl, f.P, gamma * f.a);
+          n.Q = gl * f.Q;
+          n.R = fmaf(gamma, f.b, fmaf(gl, f.R, r[b][e] - v[b][e]));
+          f = n;
+        }
       }
-      m0 += w[e];
-      a_out[e] = g;
-      r_out[e] = g + v[e];
-    }
-    if (tid == kRcThreads - 1) {
-      carry[par ^ 1][0] = nv;
-      carry[par ^ 1][1] = g;
-    }
-    if (valid > 0) {
-      const int64_t i = row * cols + c;
-      if (VEC) {
-        st4<true>(adv, i, 4, a_out);
-        st4<true>(ret, i, 4, r_out);
-      } else {
-        st4<false>(adv, i, valid, a_out);
-        st4<false>(ret, i, valid, r_out);
+      // inclusive scan over the wavefront (lane order = walk order)
+      Affine inc = f;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const Affine nb = shfl_up_affine(inc, d);
+        if (lane >= d) inc = compose(inc, nb);
       }
+      if (lane == 63) wave_tot[par][wave] = inc;
+      Affine exc = shfl_up_affine(inc, 1);
+      if (lane == 0) exc = affine_identity();
+      __syncthreads();
+      // state entering this wavefront, then this thread
+      float nv = carry[par][0], g = carry[par][1];
+      for (int k = 0; k < wave; ++k) {
+        const Affine t = wave_tot[par][k];
+        const float nv2 = fmaf(t.a, nv, t.b);
+        g = fmaf(t.P, nv, fmaf(t.Q, g, t.R));
+        nv = nv2;
+      }
+      {
+        const float nv2 = fmaf(exc.a, nv, exc.b);
+        g = fmaf(exc.P, nv, fmaf(exc.Q, g, exc.R));
+        nv = nv2;
+      }
+      // replay the 4 columns
+      float a_out[4], r_out[4];
+#pragma unroll
+      for (int e = 3; e >= 0; --e) {
+        if (w[b][e] != 0.f) {
+          const float delta = r[b][e] + gamma * nv - v[b][e];
+          g = fmaf(gl, g, delta);
+          nv = v[b][e];
+          m1 += g * w[b][e];
+          m2 += g * g * w[b][e];
+          mc += 1.f;
+        }
+        m0 += w[b][e];
+        a_out[e] = g;
+        r_out[e] = g + v[b][e];
+      }
+      if (tid == kRcThreads - 1) {
+        carry[par ^ 1][0] = nv;
+        carry[par ^ 1][1] = g;
+      }
+      if (valid[b] > 0) {
+        const int64_t i = row * cols + (int64_t)seg * kSeg + slot * 4;
+        st4<VEC>(adv, i, valid[b], a_out);
+        st4<VEC>(ret, i, valid[b], r_out);
+      }
+      __syncthreads();
+      par ^= 1;
     }
-    __syncthreads();
   }
   __shared__ double smem[16];
   double acc[4] = {m0, m1, m2, mc};
   block_sum<4, kRcThreads>(acc, smem);
   if (tid == 0) {
-    double* o = partials + row * 4;
-    o[0] = acc[0]; o[1] = acc[1]; o[2] = acc[2]; o[3] = acc[3];
+    double* o = wk.partials + row * 4;
+    peer_store(o + 0, acc[0]); peer_store(o + 1, acc[1]); peer_store(o + 2, acc[2]); peer_store(o + 3, acc[3]);
   }
+  if (!last_block_arrives(wk.ticket)) return;
+  // the last row to finish folds the per-row moments and derives the whitening statistics
+  double a[4] = {0, 0, 0, 0};
+  for (int64_t k = tid; k < rows; k += kRcThreads)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) a[i] += peer_load(wk.partials + k * 4 + i);
+  block_sum<4, kRcThreads>(a, smem);
+  if (tid == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) moments[i] = a[i];
+    whiten_stats_from_moments(a[0], a[1], a[2], 1, stats);
+  }
+  ticket_reset(wk.ticket);
 }
 
 }  // namespace vamd
@@ -166,7 +191,7 @@ using namespace vamd;
 
 extern "C" size_t vamd_gae_workspace_bytes(int64_t batch, int64_t length) {
   if (batch <= 0 || length <= 0) return 0;
-  return align_up((size_t)batch * 4 * sizeof(double), 256) + 256 /* moments */ + 256 /* stats */;
+  return kTicketBytes + align_up((size_t)batch * 4 * sizeof(double), 256) + 256 /* moments */ + 256 /* stats */;
 }
 
 extern "C" int vamd_gae(const float* rewards, const float* values, const void* mask, int mask_dtype, int64_t batch,
@@ -180,27 +205,24 @@ extern "C" int vamd_gae(const float* rewards, const float* values, const void* m
     return VAMD_EWORKSPACE;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  Carver carve(workspace);
-  double* partials = carve.take<double>((size_t)batch * 4);
+  GaeWork wk;
+  wk.ticket = static_cast<unsigned*>(workspace);
+  Carver carve(static_cast<char*>(workspace) + kTicketBytes);
+  wk.partials = carve.take<double>((size_t)batch * 4);
   double* moments = carve.take<double>(4);
   float* stats = carve.take<float>(4);
+  double* mom = moments_out ? moments_out : moments;
   const float gl = (float)((double)gamma * (double)lam);
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(length, {rewards, values, advantages, returns}, mask, sizeof(M));
     if (vec)
       hipLaunchKernelGGL((gae_scan_kernel<true, M>), dim3((unsigned)batch), dim3(kRcThreads), 0, s, rewards, values,
-                         static_cast<const M*>(mask), length, gamma, gl, advantages, returns, partials);
+                         static_cast<const M*>(mask), batch, length, gamma, gl, advantages, returns, wk, mom, stats);
     else
       hipLaunchKernelGGL((gae_scan_kernel<false, M>), dim3((unsigned)batch), dim3(kRcThreads), 0, s, rewards, values,
-                         static_cast<const M*>(mask), length, gamma, gl, advantages, returns, partials);
+                         static_cast<const M*>(mask), batch, length, gamma, gl, advantages, returns, wk, mom, stats);
   });
   VAMD_LAUNCH_CHECK();
-  double* mom = moments_out ? moments_out : moments;
-  int st = launch_moments_finalize(partials, batch, 1, 0, mom, s);
-  if (st != VAMD_OK) return st;
-  if (whiten) {
-    if ((st = vamd_whiten_stats(mom, 1, stats, stream)) != VAMD_OK) return st;
-    return vamd_affine_by_stats(advantages, stats, batch * length, advantages, stream);
-  }
+  if (whiten) return vamd_affine_by_stats(advantages, stats, batch * length, advantages, stream);
   return VAMD_OK;
 }

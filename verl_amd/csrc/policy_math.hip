@@ -2,150 +2,135 @@
 // the clipped + dual-clip policy loss, the clipped value loss, GRPO group-normalised advantages.
 // Reference semantics: verl/utils/torch_functional.py:266-339 and
 // verl/trainer/ppo/core_algos.py:266-357, :1025-1080, :1159-1250, :1799-1838.
+//
+// Every reduction is ONE launch: workgroups stream their 4096-column chunk with all loads in
+// flight at once, leave a record of double partial sums, and the workgroup that arrives last
+// folds the records (in index order) into the outputs.
 #include <initializer_list>
 
 #include "rowchunk.h"
 
 namespace vamd {
 
+struct Work {
+  unsigned* ticket;  // workspace head: zero on entry, zero on exit
+  double* partials;  // [rows * chunks][NV]
+};
+
 // =============================================================================================
 // masked moments
 // =============================================================================================
 template <bool VEC, class M>
 __global__ __launch_bounds__(kRcThreads) void moments_kernel(const float* __restrict__ values,
-                                                             const M* __restrict__ mask, int64_t cols, int chunks,
-                                                             double* __restrict__ partials) {
+                                                             const M* __restrict__ mask, int64_t rows,
+                                                             int64_t cols, int chunks, int per_row, Work wk,
+                                                             double* __restrict__ out) {
   const int64_t row = blockIdx.x / chunks;
   const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float x[kGroups][4], w[kGroups][4];
+  load_groups<VEC>(values, pos, x);
+  load_mask_groups<VEC>(mask, pos, w);
   float s0 = 0, s1 = 0, s2 = 0, cnt = 0;
-  for_each_group(row, chunk, cols, [&](int64_t i, int valid) {
-    float x[4], w[4];
-    ld4<VEC>(values, i, valid, x);
-    ldmask4<VEC>(mask, i, valid, w);
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const bool in = w[e] != 0.f;
-      const float v = in ? x[e] : 0.f;  // where(mask.bool(), values, 0)
-      s0 += w[e];
-      s1 += v * w[e];
-      s2 += v * v * w[e];
+      const bool in = w[g][e] != 0.f;
+      const float v = in ? x[g][e] : 0.f;  // where(mask.bool(), values, 0)
+      s0 += w[g][e];
+      s1 += v * w[g][e];
+      s2 += v * v * w[g][e];
       cnt += in ? 1.f : 0.f;
     }
-  });
   __shared__ double smem[16];
   double acc[4] = {s0, s1, s2, cnt};
   block_sum<4, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
-    double* o = partials + (int64_t)blockIdx.x * 4;
-    o[0] = acc[0]; o[1] = acc[1]; o[2] = acc[2]; o[3] = acc[3];
+    double* o = wk.partials + (int64_t)blockIdx.x * 4;
+    peer_store(o + 0, acc[0]); peer_store(o + 1, acc[1]); peer_store(o + 2, acc[2]); peer_store(o + 3, acc[3]);
   }
-}
-
-// out[r][0..3] = sum over chunks (per_row) or out[0..3] = sum over everything
-__global__ __launch_bounds__(kRcThreads) void moments_finalize_kernel(const double* __restrict__ partials,
-                                                                      int64_t rows, int chunks, int per_row,
-                                                                      double* __restrict__ out) {
+  if (!last_block_arrives(wk.ticket)) return;
   if (per_row) {
-    const int64_t r = (int64_t)blockIdx.x * kRcThreads + threadIdx.x;
-    if (r >= rows) return;
-    double a[4] = {0, 0, 0, 0};
-    for (int c = 0; c < chunks; ++c)
+    for (int64_t r = threadIdx.x; r < rows; r += kRcThreads) {
+      double a[4] = {0, 0, 0, 0};
+      for (int c = 0; c < chunks; ++c)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) a[i] += partials[(r * chunks + c) * 4 + i];
+        for (int i = 0; i < 4; ++i) a[i] += peer_load(wk.partials + (r * chunks + c) * 4 + i);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) out[r * 4 + i] = a[i];
+      for (int i = 0; i < 4; ++i) out[r * 4 + i] = a[i];
+    }
   } else {
     double a[4] = {0, 0, 0, 0};
     const int64_t n = rows * chunks;
     for (int64_t k = threadIdx.x; k < n; k += kRcThreads)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) a[i] += partials[k * 4 + i];
-    __shared__ double smem[16];
+      for (int i = 0; i < 4; ++i) a[i] += peer_load(wk.partials + k * 4 + i);
     block_sum<4, kRcThreads>(a, smem);
     if (threadIdx.x == 0)
 #pragma unroll
       for (int i = 0; i < 4; ++i) out[i] = a[i];
   }
+  ticket_reset(wk.ticket);
 }
 
-// stats = (mean, rsqrt(var_unbiased + 1e-8), shift) from the four moments, following
-// masked_mean / masked_var / masked_whiten (torch_functional.py:287-339).
 __global__ void whiten_stats_kernel(const double* __restrict__ mom, int shift_mean, float* __restrict__ stats) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
-  const double s0 = mom[0], s1 = mom[1], s2 = mom[2];
-  const float mean = (float)s1 / ((float)s0 + 1e-8f);
-  const double md = (double)mean;
-  // masked_mean((v - mean)^2) with the same epsilon in the denominator
-  float var = (float)((s2 - 2.0 * md * s1 + md * md * s0)) / ((float)s0 + 1e-8f);
-  var = var * ((float)s0 / ((float)s0 - 1.f));  // Bessel factor M / (M - 1)
-  stats[0] = mean;
-  stats[1] = rsqrtf(var + 1e-8f);
-  stats[2] = shift_mean ? 0.f : mean;
+  whiten_stats_from_moments(mom[0], mom[1], mom[2], shift_mean, stats);
 }
 
+template <bool VEC>
 __global__ __launch_bounds__(kRcThreads) void affine_kernel(const float* __restrict__ values,
                                                             const float* __restrict__ stats, int64_t n,
-                                                            float* __restrict__ out, int vec) {
+                                                            float* __restrict__ out) {
   const float mean = stats[0], rstd = stats[1], shift = stats[2];
-  const int64_t stride = (int64_t)gridDim.x * kRcThreads * 4;
-  for (int64_t i = ((int64_t)blockIdx.x * kRcThreads + threadIdx.x) * 4; i < n; i += stride) {
-    const int64_t left = n - i;
-    float x[4];
-    if (vec) {
-      ld4<true>(values, i, 4, x);
+  const ChunkPos pos(0, blockIdx.x, n);  // the flat array as one long row
+  float x[kGroups][4];
+  load_groups<VEC>(values, pos, x);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) x[e] = (x[e] - mean) * rstd + shift;
-      st4<true>(out, i, 4, x);
-    } else {
-      const int valid = left < 4 ? (int)left : 4;
-      ld4<false>(values, i, valid, x);
+  for (int g = 0; g < kGroups; ++g)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) x[e] = (x[e] - mean) * rstd + shift;
-      st4<false>(out, i, valid, x);
-    }
-  }
+    for (int e = 0; e < 4; ++e) x[g][e] = (x[g][e] - mean) * rstd + shift;
+  store_groups<VEC>(out, pos, x);
 }
 
 // =============================================================================================
 // agg_loss forward / backward
 // =============================================================================================
 template <bool VEC, class M>
-__global__ __launch_bounds__(kRcThreads) void agg_partial_kernel(const float* __restrict__ loss_mat,
-                                                                 const M* __restrict__ mask, int64_t cols,
-                                                                 int chunks, int token_mean,
-                                                                 double* __restrict__ partials) {
+__global__ __launch_bounds__(kRcThreads) void agg_kernel(const float* __restrict__ loss_mat,
+                                                         const M* __restrict__ mask, int64_t rows, int64_t cols,
+                                                         int chunks, AggParams ap, Work wk,
+                                                         float* __restrict__ out_loss, float* __restrict__ coef) {
   const int64_t row = blockIdx.x / chunks;
   const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float x[kGroups][4], w[kGroups][4];
+  load_groups<VEC>(loss_mat, pos, x);
+  load_mask_groups<VEC>(mask, pos, w);
+  const bool token_mean = ap.mode == VAMD_AGG_TOKEN_MEAN;
   float s = 0, m = 0;
-  for_each_group(row, chunk, cols, [&](int64_t i, int valid) {
-    float x[4], w[4];
-    ld4<VEC>(loss_mat, i, valid, x);
-    ldmask4<VEC>(mask, i, valid, w);
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       // token-mean goes through masked_sum (where() first); the seq-* modes multiply directly
-      const float v = (token_mean && w[e] == 0.f) ? 0.f : x[e];
-      if (e < valid) s += v * w[e];
-      m += w[e];
+      const float v = (token_mean && w[g][e] == 0.f) ? 0.f : x[g][e];
+      if (e < pos.valid[g]) s += v * w[g][e];
+      m += w[g][e];
     }
-  });
-  __shared__ double smem[8];
+  __shared__ double smem[(2 + 3) * 4];
   double acc[2] = {s, m};
   block_sum<2, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
-    partials[(int64_t)blockIdx.x * 2] = acc[0];
-    partials[(int64_t)blockIdx.x * 2 + 1] = acc[1];
+    peer_store(wk.partials + (int64_t)blockIdx.x * 2, acc[0]);
+    peer_store(wk.partials + (int64_t)blockIdx.x * 2 + 1, acc[1]);
   }
-}
-
-__global__ __launch_bounds__(kRcThreads) void agg_finalize_kernel(const double* __restrict__ partials, int64_t rows,
-                                                                  int chunks, int64_t cols, AggParams ap,
-                                                                  float* __restrict__ out_loss,
-                                                                  float* __restrict__ coef) {
-  __shared__ double smem[(2 + 3) * 4];
+  if (!last_block_arrives(wk.ticket)) return;
   double loss, msum, extra[1];
-  finalize_agg<2>(partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
+  finalize_agg<2>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
   if (threadIdx.x == 0) out_loss[0] = (float)loss;
+  ticket_reset(wk.ticket);
 }
 
 // out[i][t] = coef[i] * (float)mask[i][t] * *d_loss
@@ -156,14 +141,15 @@ __global__ __launch_bounds__(kRcThreads) void agg_backward_kernel(const float* _
                                                                   int chunks, float* __restrict__ out) {
   const int64_t row = blockIdx.x / chunks;
   const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float w[kGroups][4];
+  load_mask_groups<VEC>(mask, pos, w);
   const float c = coef[row] * d_loss[0];
-  for_each_group(row, chunk, cols, [&](int64_t i, int valid) {
-    float w[4], o[4];
-    ldmask4<VEC>(mask, i, valid, w);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = c * w[e];
-    st4<VEC>(out, i, valid, o);
-  });
+  for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[g][e] *= c;
+  store_groups<VEC>(out, pos, w);
 }
 
 // out[i][t] = g[i][t] * coef[i] * *d_loss * extra
@@ -174,14 +160,15 @@ __global__ __launch_bounds__(kRcThreads) void scale_rows_kernel(const float* __r
                                                                 int64_t cols, int chunks, float* __restrict__ out) {
   const int64_t row = blockIdx.x / chunks;
   const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float x[kGroups][4];
+  load_groups<VEC>(g, pos, x);
   const float c = coef[row] * d_loss[0] * extra;
-  for_each_group(row, chunk, cols, [&](int64_t i, int valid) {
-    float x[4];
-    ld4<VEC>(g, i, valid, x);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) x[e] *= c;
-    st4<VEC>(out, i, valid, x);
-  });
+  for (int k = 0; k < kGroups; ++k)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[k][e] *= c;
+  store_groups<VEC>(out, pos, x);
 }
 
 // =============================================================================================
@@ -189,41 +176,45 @@ __global__ __launch_bounds__(kRcThreads) void scale_rows_kernel(const float* __r
 // =============================================================================================
 struct PolicyParams {
   float ratio_lo, ratio_hi, clip_c;  // 1 - clip_low, 1 + clip_high, dual-clip constant
-  int token_mean;
 };
 
 template <bool VEC, class M, bool GRAD, bool ISW>
-__global__ __launch_bounds__(kRcThreads) void policy_partial_kernel(
+__global__ __launch_bounds__(kRcThreads) void policy_kernel(
     const float* __restrict__ old_lp, const float* __restrict__ lp, const float* __restrict__ adv,
-    const M* __restrict__ mask, const float* __restrict__ isw, int64_t cols, int chunks, PolicyParams pp,
-    double* __restrict__ partials, float* __restrict__ grad) {
+    const M* __restrict__ mask, const float* __restrict__ isw, int64_t rows, int64_t cols, int chunks,
+    PolicyParams pp, AggParams ap, Work wk, float* __restrict__ out, float* __restrict__ grad,
+    float* __restrict__ coef) {
   const int64_t row = blockIdx.x / chunks;
   const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float o[kGroups][4], n[kGroups][4], a[kGroups][4], w[kGroups][4], iw[kGroups][4], gr[kGroups][4];
+  load_groups<VEC>(old_lp, pos, o);
+  load_groups<VEC>(lp, pos, n);
+  load_groups<VEC>(adv, pos, a);
+  load_mask_groups<VEC>(mask, pos, w);
+  if (ISW) load_groups<VEC>(isw, pos, iw);
+  const bool token_mean = ap.mode == VAMD_AGG_TOKEN_MEAN;
   float s_loss = 0, s_m = 0, s_kl = 0, s_cf = 0, s_cfl = 0;
-  for_each_group(row, chunk, cols, [&](int64_t i, int valid) {
-    float o[4], n[4], a[4], w[4], iw[4], g[4];
-    ld4<VEC>(old_lp, i, valid, o);
-    ld4<VEC>(lp, i, valid, n);
-    ld4<VEC>(adv, i, valid, a);
-    ldmask4<VEC>(mask, i, valid, w);
-    if (ISW) ld4<VEC>(isw, i, valid, iw);
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float d = n[e] - o[e];
+      const float A = a[g][e];
+      const float d = n[g][e] - o[g][e];
       const float k = fminf(fmaxf(d, -20.f), 20.f);
       const float r = expf(k);
-      const float l1 = -a[e] * r;
+      const float l1 = -A * r;
       const float rc = fminf(fmaxf(r, pp.ratio_lo), pp.ratio_hi);
-      const float l2 = -a[e] * rc;
+      const float l2 = -A * rc;
       const float c1 = fmaxf(l1, l2);
-      const float l3 = -a[e] * pp.clip_c;
-      const bool neg = a[e] < 0.f;
+      const float l3 = -A * pp.clip_c;
+      const bool neg = A < 0.f;
       float loss = neg ? fminf(l3, c1) : c1;
-      if (ISW) loss *= iw[e];
-      const bool in = w[e] != 0.f;
-      const float we = w[e];
-      if (e < valid) {
-        s_loss += ((pp.token_mean && !in) ? 0.f : loss) * we;
+      if (ISW) loss *= iw[g][e];
+      const float we = w[g][e];
+      const bool in = we != 0.f;
+      if (e < pos.valid[g]) {
+        s_loss += ((token_mean && !in) ? 0.f : loss) * we;
         s_m += we;
         s_kl += in ? -k * we : 0.f;
         s_cf += (in && l2 > l1) ? we : 0.f;
@@ -236,31 +227,24 @@ __global__ __launch_bounds__(kRcThreads) void policy_partial_kernel(
         const float in_clip = (r >= pp.ratio_lo && r <= pp.ratio_hi) ? 1.f : 0.f;
         const float g1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
         const float g2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
-        float dc1 = (g1 + g2 * in_clip) * (-a[e] * r) * in_k;
+        float dc1 = (g1 + g2 * in_clip) * (-A * r) * in_k;
         if (neg) dc1 *= c1 < l3 ? 1.f : (c1 == l3 ? 0.5f : 0.f);
-        if (ISW) dc1 *= iw[e];
-        g[e] = dc1 * we;
+        if (ISW) dc1 *= iw[g][e];
+        gr[g][e] = dc1 * we;
       }
     }
-    if (GRAD) st4<VEC>(grad, i, valid, g);
-  });
-  __shared__ double smem[20];
+  if (GRAD) store_groups<VEC>(grad, pos, gr);
+  __shared__ double smem[(5 + 3) * 4];
   double acc[5] = {s_loss, s_m, s_kl, s_cf, s_cfl};
   block_sum<5, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
-    double* p = partials + (int64_t)blockIdx.x * 5;
+    double* p = wk.partials + (int64_t)blockIdx.x * 5;
 #pragma unroll
-    for (int i = 0; i < 5; ++i) p[i] = acc[i];
+    for (int i = 0; i < 5; ++i) peer_store(p + i, acc[i]);
   }
-}
-
-__global__ __launch_bounds__(kRcThreads) void policy_finalize_kernel(const double* __restrict__ partials,
-                                                                     int64_t rows, int chunks, int64_t cols,
-                                                                     AggParams ap, float* __restrict__ out,
-                                                                     float* __restrict__ coef) {
-  __shared__ double smem[(5 + 3) * 4];
+  if (!last_block_arrives(wk.ticket)) return;
   double loss, msum, extra[3];
-  finalize_agg<5>(partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
+  finalize_agg<5>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
   if (threadIdx.x == 0) {
     const float denom = (float)msum + 1e-8f;  // masked_mean's denominator
     out[0] = (float)loss;
@@ -268,93 +252,149 @@ __global__ __launch_bounds__(kRcThreads) void policy_finalize_kernel(const doubl
     out[2] = (float)extra[0] / denom;  // ppo_kl
     out[3] = (float)extra[2] / denom;  // pg_clipfrac_lower
   }
+  ticket_reset(wk.ticket);
 }
 
 // =============================================================================================
 // value loss (compute_value_loss, core_algos.py:1799-1838)
 // =============================================================================================
 template <bool VEC, class M, bool GRAD>
-__global__ __launch_bounds__(kRcThreads) void value_partial_kernel(
+__global__ __launch_bounds__(kRcThreads) void value_kernel(
     const float* __restrict__ vpreds, const float* __restrict__ returns, const float* __restrict__ values,
-    const M* __restrict__ mask, int64_t cols, int chunks, float clip, int token_mean,
-    double* __restrict__ partials, float* __restrict__ grad) {
+    const M* __restrict__ mask, int64_t rows, int64_t cols, int chunks, float clip, AggParams ap, Work wk,
+    float* __restrict__ out, float* __restrict__ grad, float* __restrict__ coef) {
   const int64_t row = blockIdx.x / chunks;
   const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float vp[kGroups][4], R[kGroups][4], v[kGroups][4], w[kGroups][4], gr[kGroups][4];
+  load_groups<VEC>(vpreds, pos, vp);
+  load_groups<VEC>(returns, pos, R);
+  load_groups<VEC>(values, pos, v);
+  load_mask_groups<VEC>(mask, pos, w);
+  const bool token_mean = ap.mode == VAMD_AGG_TOKEN_MEAN;
   float s_loss = 0, s_m = 0, s_cf = 0;
-  for_each_group(row, chunk, cols, [&](int64_t i, int valid) {
-    float vp[4], R[4], v[4], w[4], g[4];
-    ld4<VEC>(vpreds, i, valid, vp);
-    ld4<VEC>(returns, i, valid, R);
-    ld4<VEC>(values, i, valid, v);
-    ldmask4<VEC>(mask, i, valid, w);
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float lo = v[e] - clip, hi = v[e] + clip;
-      const float inner = fminf(vp[e], hi);
+      const float lo = v[g][e] - clip, hi = v[g][e] + clip;
+      const float inner = fminf(vp[g][e], hi);
       const float vc = fmaxf(inner, lo);
-      const float d1 = vp[e] - R[e], d2 = vc - R[e];
+      const float d1 = vp[g][e] - R[g][e], d2 = vc - R[g][e];
       const float e1 = d1 * d1, e2 = d2 * d2;
       const float loss = fmaxf(e1, e2);
-      const bool in = w[e] != 0.f;
-      if (e < valid) {
-        s_loss += ((token_mean && !in) ? 0.f : loss) * w[e];
-        s_m += w[e];
-        s_cf += (in && e2 > e1) ? w[e] : 0.f;
+      const float we = w[g][e];
+      const bool in = we != 0.f;
+      if (e < pos.valid[g]) {
+        s_loss += ((token_mean && !in) ? 0.f : loss) * we;
+        s_m += we;
+        s_cf += (in && e2 > e1) ? we : 0.f;
       }
       if (GRAD) {
-        const float a = vp[e] < hi ? 1.f : (vp[e] == hi ? 0.5f : 0.f);
-        const float b = inner > lo ? 1.f : (inner == lo ? 0.5f : 0.f);
+        const float ga = vp[g][e] < hi ? 1.f : (vp[g][e] == hi ? 0.5f : 0.f);
+        const float gb = inner > lo ? 1.f : (inner == lo ? 0.5f : 0.f);
         const float g1 = e1 > e2 ? 1.f : (e1 == e2 ? 0.5f : 0.f);
         const float g2 = e2 > e1 ? 1.f : (e1 == e2 ? 0.5f : 0.f);
-        g[e] = (g1 * 2.f * d1 + g2 * 2.f * d2 * a * b) * w[e];
+        gr[g][e] = (g1 * 2.f * d1 + g2 * 2.f * d2 * ga * gb) * we;
       }
     }
-    if (GRAD) st4<VEC>(grad, i, valid, g);
-  });
-  __shared__ double smem[12];
+  if (GRAD) store_groups<VEC>(grad, pos, gr);
+  __shared__ double smem[(3 + 3) * 4];
   double acc[3] = {s_loss, s_m, s_cf};
   block_sum<3, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
-    double* p = partials + (int64_t)blockIdx.x * 3;
-    p[0] = acc[0]; p[1] = acc[1]; p[2] = acc[2];
+    double* p = wk.partials + (int64_t)blockIdx.x * 3;
+    peer_store(p + 0, acc[0]); peer_store(p + 1, acc[1]); peer_store(p + 2, acc[2]);
   }
-}
-
-__global__ __launch_bounds__(kRcThreads) void value_finalize_kernel(const double* __restrict__ partials,
-                                                                    int64_t rows, int chunks, int64_t cols,
-                                                                    AggParams ap, float* __restrict__ out,
-                                                                    float* __restrict__ coef) {
-  __shared__ double smem[(3 + 3) * 4];
+  if (!last_block_arrives(wk.ticket)) return;
   double loss, msum, extra[1];
-  finalize_agg<3>(partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
+  finalize_agg<3>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
   if (threadIdx.x == 0) {
     out[0] = 0.5f * (float)loss;
     out[1] = (float)extra[0] / ((float)msum + 1e-8f);
   }
+  ticket_reset(wk.ticket);
 }
 
 // =============================================================================================
 // GRPO
 // =============================================================================================
-// partial[row][chunk] = sum of rewards (the mask is NOT applied, core_algos.py:303)
+constexpr int kGrpoLdsGroups = 2048;  // groups whose statistics fit the last workgroup's LDS
+
+struct GrpoArgs {
+  const int64_t* gid;
+  int64_t rows, n_groups;
+  float eps;
+  int norm_by_std, std_mode;
+  float* scores;   // [rows] scratch
+  float* scalars;  // [rows] out: normalised scalar per response
+  float* mean;     // [n_groups] (only used by the large-group-count path)
+  float* stdv;
+};
+
+// Row sums of the rewards (the mask is NOT applied, core_algos.py:303); the last workgroup turns
+// them into scores, per-group mean / std and the per-response scalar.
+// std_mode 0: unbiased torch.std; 1: sqrt(clamp(var, min=eps)) of group_mean_std.  Singleton
+// groups get mean 0, std 1 (core_algos.py:314-316, groupwise.py:215-221).
 template <bool VEC>
-__global__ __launch_bounds__(kRcThreads) void rowsum_partial_kernel(const float* __restrict__ x, int64_t cols,
-                                                                    int chunks, double* __restrict__ partials) {
+__global__ __launch_bounds__(kRcThreads) void grpo_rowsum_kernel(const float* __restrict__ x, int64_t cols,
+                                                                 int chunks, Work wk, GrpoArgs ga) {
   const int64_t row = blockIdx.x / chunks;
   const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float v[kGroups][4];
+  load_groups<VEC>(x, pos, v);
   float s = 0;
-  for_each_group(row, chunk, cols, [&](int64_t i, int valid) {
-    float v[4];
-    ld4<VEC>(x, i, valid, v);
-    s += (v[0] + v[1]) + (v[2] + v[3]);
-  });
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g) s += (v[g][0] + v[g][1]) + (v[g][2] + v[g][3]);
   __shared__ double smem[4];
   double acc[1] = {s};
   block_sum<1, kRcThreads>(acc, smem);
-  if (threadIdx.x == 0) partials[blockIdx.x] = acc[0];
+  if (threadIdx.x == 0) peer_store(wk.partials + blockIdx.x, acc[0]);
+  if (ga.n_groups > kGrpoLdsGroups) return;  // statistics come from the separate kernels below
+  if (!last_block_arrives(wk.ticket)) return;
+
+  __shared__ int g_cnt[kGrpoLdsGroups];
+  __shared__ double g_sum[kGrpoLdsGroups];
+  __shared__ double g_sq[kGrpoLdsGroups];
+  for (int64_t g = threadIdx.x; g < ga.n_groups; g += kRcThreads) {
+    g_cnt[g] = 0;
+    g_sum[g] = 0.0;
+    g_sq[g] = 0.0;
+  }
+  __syncthreads();
+  for (int64_t r = threadIdx.x; r < ga.rows; r += kRcThreads) {
+    double t = 0;
+    for (int c = 0; c < chunks; ++c) t += peer_load(wk.partials + r * chunks + c);
+    const float sc = (float)t;
+    ga.scores[r] = sc;
+    const int64_t g = ga.gid[r];
+    atomicAdd(&g_cnt[g], 1);
+    atomicAdd(&g_sum[g], (double)sc);
+  }
+  __syncthreads();
+  for (int64_t r = threadIdx.x; r < ga.rows; r += kRcThreads) {
+    const int64_t g = ga.gid[r];
+    const double d = (double)ga.scores[r] - g_sum[g] / (double)g_cnt[g];
+    atomicAdd(&g_sq[g], d * d);
+  }
+  __syncthreads();
+  for (int64_t r = threadIdx.x; r < ga.rows; r += kRcThreads) {
+    const int64_t g = ga.gid[r];
+    const int c = g_cnt[g];
+    float mu = 0.f, sd = 1.f;
+    if (c > 1) {
+      const double var = g_sq[g] / (double)(c - 1);
+      mu = (float)(g_sum[g] / (double)c);
+      sd = ga.std_mode == 0 ? (float)sqrt(var) : sqrtf(fmaxf((float)var, ga.eps));
+    }
+    const float cen = ga.scores[r] - mu;
+    ga.scalars[r] = ga.norm_by_std ? cen / (sd + ga.eps) : cen;
+  }
+  ticket_reset(wk.ticket);
 }
 
-// scores[i] = (float) sum_c partial[i][c]
+// ---- path for more groups than fit in LDS (and for group_mean_std itself) ----
 __global__ void rowsum_finalize_kernel(const double* __restrict__ partials, int64_t rows, int chunks,
                                        float* __restrict__ scores) {
   const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -365,8 +405,6 @@ __global__ void rowsum_finalize_kernel(const double* __restrict__ partials, int6
 }
 
 // One thread per group: count, mean, std over the group's members in index order.
-// std_mode 0: unbiased torch.std (two-pass); 1: sqrt(clamp(var, min=eps)) of group_mean_std.
-// Singleton groups get mean 0, std 1 (core_algos.py:314-316, groupwise.py:215-221).
 __global__ void group_stats_kernel(const float* __restrict__ scores, const int64_t* __restrict__ gid, int64_t n,
                                    int64_t n_groups, float eps, int std_mode, float* __restrict__ mean,
                                    float* __restrict__ stdv, float* __restrict__ count) {
@@ -397,7 +435,6 @@ __global__ void group_stats_kernel(const float* __restrict__ scores, const int64
   if (count) count[g] = (float)c;
 }
 
-// scalars[i] = (score - mean_g) / (std_g + eps)   or   score - mean_g
 __global__ void grpo_scalars_kernel(const float* __restrict__ scores, const int64_t* __restrict__ gid, int64_t n,
                                     const float* __restrict__ mean, const float* __restrict__ stdv, float eps,
                                     int norm_by_std, float* __restrict__ scalars) {
@@ -415,25 +452,18 @@ __global__ __launch_bounds__(kRcThreads) void broadcast_rows_kernel(const float*
                                                                     int chunks, float* __restrict__ out) {
   const int64_t row = blockIdx.x / chunks;
   const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float w[kGroups][4];
+  load_mask_groups<VEC>(mask, pos, w);
   const float a = scalars[row];
-  for_each_group(row, chunk, cols, [&](int64_t i, int valid) {
-    float w[4], o[4];
-    ldmask4<VEC>(mask, i, valid, w);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = a * w[e];
-    st4<VEC>(out, i, valid, o);
-  });
+  for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[g][e] *= a;
+  store_groups<VEC>(out, pos, w);
 }
 
-int launch_moments_finalize(const double* partials, int64_t rows, int chunks, int per_row, double* out,
-                            hipStream_t stream) {
-  const unsigned grid = per_row ? (unsigned)((rows + kRcThreads - 1) / kRcThreads) : 1u;
-  hipLaunchKernelGGL(moments_finalize_kernel, dim3(grid), dim3(kRcThreads), 0, stream, partials, rows, chunks,
-                     per_row, out);
-  VAMD_LAUNCH_CHECK();
-  return VAMD_OK;
-}
-
+// ---------------------------------------------------------------------------------------------
 static int check_matrix(const char* what, int64_t rows, int64_t cols) {
   VAMD_REQUIRE(rows > 0 && cols > 0, "%s: empty input (%lld x %lld)", what, (long long)rows, (long long)cols);
   VAMD_REQUIRE(rows * chunks_of(cols) < (1ll << 31), "%s: too many workgroups", what);
@@ -450,6 +480,18 @@ static AggParams make_agg(int mode, double dp, double bnt, double gbs, double ls
   return a;
 }
 
+static size_t reduce_workspace_bytes(int64_t rows, int64_t cols, int nv) {
+  if (rows <= 0 || cols <= 0) return 0;
+  return kTicketBytes + align_up((size_t)rows * chunks_of(cols) * nv * sizeof(double), 256);
+}
+
+static Work carve_work(void* workspace) {
+  Work w;
+  w.ticket = static_cast<unsigned*>(workspace);
+  w.partials = reinterpret_cast<double*>(static_cast<char*>(workspace) + kTicketBytes);
+  return w;
+}
+
 }  // namespace vamd
 
 using namespace vamd;
@@ -459,8 +501,7 @@ using namespace vamd;
 
 // ---------------------------------------------------------------------------------------------
 extern "C" size_t vamd_masked_moments_workspace_bytes(int64_t rows, int64_t cols) {
-  if (rows <= 0 || cols <= 0) return 0;
-  return align_up((size_t)rows * chunks_of(cols) * 4 * sizeof(double), 256);
+  return reduce_workspace_bytes(rows, cols, 4);
 }
 
 extern "C" int vamd_masked_moments(const float* values, const void* mask, int mask_dtype, int64_t rows,
@@ -475,15 +516,15 @@ extern "C" int vamd_masked_moments(const float* values, const void* mask, int ma
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int chunks = (int)chunks_of(cols);
-  double* partials = static_cast<double*>(workspace);
+  const Work wk = carve_work(workspace);
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(cols, {values}, mask, sizeof(M));
     VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((moments_kernel<V, M>), dim3((unsigned)(rows * chunks)),
-                                                 dim3(kRcThreads), 0, s, values, static_cast<const M*>(mask), cols,
-                                                 chunks, partials));
+                                                 dim3(kRcThreads), 0, s, values, static_cast<const M*>(mask), rows,
+                                                 cols, chunks, per_row, wk, out));
   });
   VAMD_LAUNCH_CHECK();
-  return launch_moments_finalize(partials, rows, chunks, per_row, out, s);
+  return VAMD_OK;
 }
 
 extern "C" int vamd_whiten_stats(const double* moments, int shift_mean, float* stats, void* stream) {
@@ -496,20 +537,19 @@ extern "C" int vamd_whiten_stats(const double* moments, int shift_mean, float* s
 
 extern "C" int vamd_affine_by_stats(const float* values, const float* stats, int64_t n, float* out, void* stream) {
   VAMD_REQUIRE(values && stats && out && n > 0, "affine_by_stats: bad argument");
-  const int vec = (n % 4 == 0) && aligned_to(values, 16) && aligned_to(out, 16);
-  int64_t blocks = (n + kRcThreads * 16 - 1) / (kRcThreads * 16);
-  if (blocks < 1) blocks = 1;
-  if (blocks > 65535 * 16) blocks = 65535 * 16;
-  hipLaunchKernelGGL(affine_kernel, dim3((unsigned)blocks), dim3(kRcThreads), 0, static_cast<hipStream_t>(stream),
-                     values, stats, n, out, vec);
+  VAMD_REQUIRE(chunks_of(n) < (1ll << 31), "affine_by_stats: too many elements");
+  const bool vec = (n % 4 == 0) && aligned_to(values, 16) && aligned_to(out, 16);
+  const dim3 grid((unsigned)chunks_of(n));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((affine_kernel<V>), grid, dim3(kRcThreads), 0, s, values, stats, n,
+                                               out));
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }
 
 // ---------------------------------------------------------------------------------------------
 extern "C" size_t vamd_agg_loss_workspace_bytes(int64_t rows, int64_t cols) {
-  if (rows <= 0 || cols <= 0) return 0;
-  return align_up((size_t)rows * chunks_of(cols) * 2 * sizeof(double), 256);
+  return reduce_workspace_bytes(rows, cols, 2);
 }
 
 extern "C" int vamd_agg_loss_forward(const float* loss_mat, const void* mask, int mask_dtype, int64_t rows,
@@ -526,18 +566,14 @@ extern "C" int vamd_agg_loss_forward(const float* loss_mat, const void* mask, in
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int chunks = (int)chunks_of(cols);
-  double* partials = static_cast<double*>(workspace);
-  const int token_mean = mode == VAMD_AGG_TOKEN_MEAN;
+  const Work wk = carve_work(workspace);
+  const AggParams ap = make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor);
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(cols, {loss_mat}, mask, sizeof(M));
-    VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((agg_partial_kernel<V, M>), dim3((unsigned)(rows * chunks)),
+    VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((agg_kernel<V, M>), dim3((unsigned)(rows * chunks)),
                                                  dim3(kRcThreads), 0, s, loss_mat, static_cast<const M*>(mask),
-                                                 cols, chunks, token_mean, partials));
+                                                 rows, cols, chunks, ap, wk, out_loss, coef_out));
   });
-  VAMD_LAUNCH_CHECK();
-  hipLaunchKernelGGL(agg_finalize_kernel, dim3(1), dim3(kRcThreads), 0, s, partials, rows, chunks, cols,
-                     make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor), out_loss,
-                     coef_out);
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }
@@ -576,8 +612,7 @@ extern "C" int vamd_scale_rows(const float* g, const float* coef, const float* d
 
 // ---------------------------------------------------------------------------------------------
 extern "C" size_t vamd_policy_loss_workspace_bytes(int64_t rows, int64_t cols) {
-  if (rows <= 0 || cols <= 0) return 0;
-  return align_up((size_t)rows * chunks_of(cols) * 5 * sizeof(double), 256);
+  return reduce_workspace_bytes(rows, cols, 5);
 }
 
 extern "C" int vamd_policy_loss_forward(const float* old_log_prob, const float* log_prob, const float* advantages,
@@ -598,16 +633,16 @@ extern "C" int vamd_policy_loss_forward(const float* old_log_prob, const float* 
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int chunks = (int)chunks_of(cols);
-  double* partials = static_cast<double*>(workspace);
+  const Work wk = carve_work(workspace);
   PolicyParams pp;
   pp.ratio_lo = (float)(1.0 - (double)clip_low);
   pp.ratio_hi = (float)(1.0 + (double)clip_high);
   pp.clip_c = clip_c;
-  pp.token_mean = mode == VAMD_AGG_TOKEN_MEAN;
+  const AggParams ap = make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor);
   const dim3 grid((unsigned)(rows * chunks)), block(kRcThreads);
 #define VAMD_PL(V, G, W)                                                                                     \
-  hipLaunchKernelGGL((policy_partial_kernel<V, M, G, W>), grid, block, 0, s, old_log_prob, log_prob, advantages, \
-                     mk, is_weights, cols, chunks, pp, partials, grad_unscaled)
+  hipLaunchKernelGGL((policy_kernel<V, M, G, W>), grid, block, 0, s, old_log_prob, log_prob, advantages, mk, \
+                     is_weights, rows, cols, chunks, pp, ap, wk, out, grad_unscaled, coef_out)
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(cols, {old_log_prob, log_prob, advantages, is_weights, grad_unscaled}, mask,
                                    sizeof(M));
@@ -622,16 +657,12 @@ extern "C" int vamd_policy_loss_forward(const float* old_log_prob, const float* 
   });
 #undef VAMD_PL
   VAMD_LAUNCH_CHECK();
-  hipLaunchKernelGGL(policy_finalize_kernel, dim3(1), dim3(kRcThreads), 0, s, partials, rows, chunks, cols,
-                     make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor), out, coef_out);
-  VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }
 
 // ---------------------------------------------------------------------------------------------
 extern "C" size_t vamd_value_loss_workspace_bytes(int64_t rows, int64_t cols) {
-  if (rows <= 0 || cols <= 0) return 0;
-  return align_up((size_t)rows * chunks_of(cols) * 3 * sizeof(double), 256);
+  return reduce_workspace_bytes(rows, cols, 3);
 }
 
 extern "C" int vamd_value_loss_forward(const float* vpreds, const float* returns, const float* values,
@@ -649,12 +680,12 @@ extern "C" int vamd_value_loss_forward(const float* vpreds, const float* returns
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int chunks = (int)chunks_of(cols);
-  double* partials = static_cast<double*>(workspace);
-  const int token_mean = mode == VAMD_AGG_TOKEN_MEAN;
+  const Work wk = carve_work(workspace);
+  const AggParams ap = make_agg(mode, 1.0, -1.0, -1.0, -1.0);
   const dim3 grid((unsigned)(rows * chunks)), block(kRcThreads);
-#define VAMD_VL(V, G)                                                                                       \
-  hipLaunchKernelGGL((value_partial_kernel<V, M, G>), grid, block, 0, s, vpreds, returns, values, mk, cols, \
-                     chunks, cliprange_value, token_mean, partials, grad_unscaled)
+#define VAMD_VL(V, G)                                                                                     \
+  hipLaunchKernelGGL((value_kernel<V, M, G>), grid, block, 0, s, vpreds, returns, values, mk, rows, cols, \
+                     chunks, cliprange_value, ap, wk, out, grad_unscaled, coef_out)
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(cols, {vpreds, returns, values, grad_unscaled}, mask, sizeof(M));
     const M* mk = static_cast<const M*>(mask);
@@ -663,18 +694,15 @@ extern "C" int vamd_value_loss_forward(const float* vpreds, const float* returns
   });
 #undef VAMD_VL
   VAMD_LAUNCH_CHECK();
-  hipLaunchKernelGGL(value_finalize_kernel, dim3(1), dim3(kRcThreads), 0, s, partials, rows, chunks, cols,
-                     make_agg(mode, 1.0, -1.0, -1.0, -1.0), out, coef_out);
-  VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }
 
 // ---------------------------------------------------------------------------------------------
 extern "C" size_t vamd_grpo_workspace_bytes(int64_t batch, int64_t length, int64_t n_groups) {
   if (batch <= 0 || length <= 0 || n_groups <= 0) return 0;
-  size_t b = align_up((size_t)batch * chunks_of(length) * sizeof(double), 256);
+  size_t b = reduce_workspace_bytes(batch, length, 1);
   b += 2 * align_up((size_t)batch * sizeof(float), 256);     // scores, scalars
-  b += 2 * align_up((size_t)n_groups * sizeof(float), 256);  // mean, std
+  b += 2 * align_up((size_t)n_groups * sizeof(float), 256);  // mean, std (large-group-count path)
   return b;
 }
 
@@ -700,33 +728,42 @@ extern "C" int vamd_grpo_advantage(const float* rewards, const void* mask, int m
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int chunks = (int)chunks_of(length);
-  Carver carve(workspace);
-  double* partials = carve.take<double>((size_t)batch * chunks);
-  float* scores = carve.take<float>((size_t)batch);
+  const Work wk = carve_work(workspace);
+  Carver carve(static_cast<char*>(workspace) + reduce_workspace_bytes(batch, length, 1));
+  GrpoArgs ga;
+  ga.gid = group_ids;
+  ga.rows = batch;
+  ga.n_groups = n_groups;
+  ga.eps = epsilon;
+  ga.norm_by_std = norm_by_std;
+  ga.std_mode = std_mode;
+  ga.scores = carve.take<float>((size_t)batch);
   float* scalars = carve.take<float>((size_t)batch);
-  float* mean = carve.take<float>((size_t)n_groups);
-  float* stdv = carve.take<float>((size_t)n_groups);
+  ga.scalars = scores_out ? scores_out : scalars;
+  ga.mean = carve.take<float>((size_t)n_groups);
+  ga.stdv = carve.take<float>((size_t)n_groups);
   {
     const bool vec = can_vectorize(length, {rewards}, nullptr, 0);
-    VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((rowsum_partial_kernel<V>), dim3((unsigned)(batch * chunks)),
-                                                 dim3(kRcThreads), 0, s, rewards, length, chunks, partials));
+    VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((grpo_rowsum_kernel<V>), dim3((unsigned)(batch * chunks)),
+                                                 dim3(kRcThreads), 0, s, rewards, length, chunks, wk, ga));
     VAMD_LAUNCH_CHECK();
   }
-  hipLaunchKernelGGL(rowsum_finalize_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, partials, batch,
-                     chunks, scores);
-  VAMD_LAUNCH_CHECK();
-  hipLaunchKernelGGL(group_stats_kernel, dim3((unsigned)((n_groups + 63) / 64)), dim3(64), 0, s, scores, group_ids,
-                     batch, n_groups, epsilon, std_mode, mean, stdv, (float*)nullptr);
-  VAMD_LAUNCH_CHECK();
-  hipLaunchKernelGGL(grpo_scalars_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, scores, group_ids,
-                     batch, mean, stdv, epsilon, norm_by_std, scores_out ? scores_out : scalars);
-  VAMD_LAUNCH_CHECK();
-  const float* sc = scores_out ? scores_out : scalars;
+  if (n_groups > kGrpoLdsGroups) {
+    hipLaunchKernelGGL(rowsum_finalize_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, wk.partials,
+                       batch, chunks, ga.scores);
+    VAMD_LAUNCH_CHECK();
+    hipLaunchKernelGGL(group_stats_kernel, dim3((unsigned)((n_groups + 63) / 64)), dim3(64), 0, s, ga.scores,
+                       group_ids, batch, n_groups, epsilon, std_mode, ga.mean, ga.stdv, (float*)nullptr);
+    VAMD_LAUNCH_CHECK();
+    hipLaunchKernelGGL(grpo_scalars_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, ga.scores,
+                       group_ids, batch, ga.mean, ga.stdv, epsilon, norm_by_std, ga.scalars);
+    VAMD_LAUNCH_CHECK();
+  }
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(length, {advantages}, mask, sizeof(M));
     VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((broadcast_rows_kernel<V, M>), dim3((unsigned)(batch * chunks)),
-                                                 dim3(kRcThreads), 0, s, sc, static_cast<const M*>(mask), length,
-                                                 chunks, advantages));
+                                                 dim3(kRcThreads), 0, s, ga.scalars, static_cast<const M*>(mask),
+                                                 length, chunks, advantages));
   });
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;

@@ -2,10 +2,15 @@
 //
 // A launch covers the matrix with workgroups of 256 threads; workgroup (row, chunk) owns
 // kChunk = 4096 consecutive columns of one row and each thread walks them in float4 steps that
-// are contiguous across the wavefront (64 lanes x 16 B = 1 KiB per load instruction).  Partial
-// sums leave the workgroup as doubles in a fixed tree order, one record per (row, chunk); a
-// second, tiny kernel combines the records in index order, so results are bit-reproducible and
-// no floating-point atomics are used.
+// are contiguous across the wavefront (64 lanes x 16 B = 1 KiB per load instruction); all of a
+// thread's loads are issued before any arithmetic so that a workgroup keeps 16 KiB per input in
+// flight.  Partial sums leave the workgroup as doubles in a fixed tree order, one record per
+// (row, chunk); the workgroup that finishes last (ticket counter at the head of the workspace)
+// combines the records in index order inside the same launch, so results are bit-reproducible,
+// no floating-point atomics are used and a reduction costs one kernel launch.
+//
+// Workspace contract of these kernels: the first 256 bytes hold the ticket counter; they must be
+// zero on entry and are zero again when the kernel has finished.
 #pragma once
 #include "common.h"
 
@@ -13,6 +18,8 @@ namespace vamd {
 
 constexpr int kRcThreads = 256;
 constexpr int kChunk = 4096;  // columns per workgroup
+constexpr int kGroups = kChunk / (kRcThreads * 4);  // float4 groups per thread per input (4)
+constexpr size_t kTicketBytes = 256;
 
 inline int64_t chunks_of(int64_t cols) { return cols <= 0 ? 1 : (cols + kChunk - 1) / kChunk; }
 
@@ -65,6 +72,96 @@ __device__ __forceinline__ void for_each_group(int64_t row, int chunk, int64_t c
   }
 }
 
+// The 4-element groups one thread owns in its workgroup's chunk.
+struct ChunkPos {
+  int64_t idx[kGroups];  // flat index of the group's first element
+  int valid[kGroups];    // 0..4 elements of the group exist
+  __device__ __forceinline__ ChunkPos(int64_t row, int chunk, int64_t cols) {
+    const int64_t c_begin = (int64_t)chunk * kChunk;
+    const int64_t c_end = (c_begin + kChunk) < cols ? (c_begin + kChunk) : cols;
+#pragma unroll
+    for (int g = 0; g < kGroups; ++g) {
+      const int64_t c = c_begin + ((int64_t)g * kRcThreads + threadIdx.x) * 4;
+      const int64_t left = c_end - c;
+      valid[g] = left >= 4 ? 4 : (left > 0 ? (int)left : 0);
+      idx[g] = row * cols + c;
+    }
+  }
+};
+
+template <bool VEC>
+__device__ __forceinline__ void load_groups(const float* __restrict__ p, const ChunkPos& pos, float (&x)[kGroups][4]) {
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g) {
+    if (pos.valid[g] > 0) {
+      ld4<VEC>(p, pos.idx[g], pos.valid[g], x[g]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[g][e] = 0.f;
+    }
+  }
+}
+
+template <bool VEC, class M>
+__device__ __forceinline__ void load_mask_groups(const M* __restrict__ p, const ChunkPos& pos, float (&w)[kGroups][4]) {
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g) {
+    if (pos.valid[g] > 0) {
+      ldmask4<VEC>(p, pos.idx[g], pos.valid[g], w[g]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) w[g][e] = 0.f;
+    }
+  }
+}
+
+template <bool VEC>
+__device__ __forceinline__ void store_groups(float* __restrict__ p, const ChunkPos& pos, const float (&x)[kGroups][4]) {
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
+    if (pos.valid[g] > 0) st4<VEC>(p, pos.idx[g], pos.valid[g], x[g]);
+}
+
+// Publishing a record to the workgroup that will fold it, without a device-wide fence (an
+// agent-scope fence writes back / invalidates a whole XCD's L2 and costs tens of microseconds
+// when every workgroup issues one): the record is written with device-coherent stores, the
+// writer waits for their acknowledgement, then takes a ticket with a device-scope atomic; the
+// folding workgroup reads the records with device-coherent loads.
+__device__ __forceinline__ void peer_store(double* p, double v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ double peer_load(const double* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Ticket: true in exactly one workgroup of the launch, the one that arrives last.  Thread 0 must
+// have issued its peer_store()s before the call.  The last workgroup calls ticket_reset() when done.
+__device__ __forceinline__ bool last_block_arrives(unsigned* counter) {
+  __shared__ unsigned ticket;
+  if (threadIdx.x == 0) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  return ticket == gridDim.x - 1;
+}
+__device__ __forceinline__ void ticket_reset(unsigned* counter) {
+  if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// (mean, rsqrt(var_unbiased + 1e-8), shift) from the masked moments sum(m), sum(v m), sum(v^2 m),
+// following masked_mean / masked_var / masked_whiten (verl/utils/torch_functional.py:287-339).
+__device__ __forceinline__ void whiten_stats_from_moments(double s0, double s1, double s2, int shift_mean,
+                                                          float* __restrict__ stats) {
+  const float mean = (float)s1 / ((float)s0 + 1e-8f);
+  const double md = (double)mean;
+  // masked_mean((v - mean)^2) with the same epsilon in the denominator
+  float var = (float)((s2 - 2.0 * md * s1 + md * md * s0)) / ((float)s0 + 1e-8f);
+  var = var * ((float)s0 / ((float)s0 - 1.f));  // Bessel factor M / (M - 1)
+  stats[0] = mean;
+  stats[1] = rsqrtf(var + 1e-8f);
+  stats[2] = shift_mean ? 0.f : mean;
+}
+
 // The vector path needs 4-element groups that never straddle a row and 16-byte aligned rows.
 inline bool can_vectorize(int64_t cols, std::initializer_list<const void*> f32_ptrs, const void* mask,
                           size_t mask_elem) {
@@ -82,7 +179,7 @@ struct AggParams {
   double dp_size, batch_num_tokens, global_batch_size, loss_scale_factor;  // < 0 : None
 };
 
-// Called by ONE workgroup of 256 threads.  partials: [rows][chunks][NV] doubles with slot 0 =
+// Called by ONE workgroup of 256 threads (the last one to arrive).  partials: [rows][chunks][NV] doubles with slot 0 =
 // sum(loss * w) and slot 1 = sum(w); slots >= 2 are summed over everything into extra[].
 // Writes loss (double, thread 0) and coef[rows].
 template <int NV>
@@ -99,9 +196,13 @@ __device__ void finalize_agg(const double* __restrict__ partials, int64_t rows, 
     double row[NV];
 #pragma unroll
     for (int i = 0; i < NV; ++i) row[i] = 0;
-    for (int c = 0; c < chunks; ++c)
+    for (int c = 0; c < chunks; ++c) {
+      double t[NV];  // issue the record's loads together, then add
 #pragma unroll
-      for (int i = 0; i < NV; ++i) row[i] += partials[(r * chunks + c) * NV + i];
+      for (int i = 0; i < NV; ++i) t[i] = peer_load(partials + (r * chunks + c) * NV + i);
+#pragma unroll
+      for (int i = 0; i < NV; ++i) row[i] += t[i];
+    }
 #pragma unroll
     for (int i = 0; i < NV; ++i) tot[i] += row[i];
     if (row[1] > 0) {
@@ -147,7 +248,7 @@ __device__ void finalize_agg(const double* __restrict__ partials, int64_t rows, 
       double c = c_all;
       if (ap.mode == VAMD_AGG_SEQ_MEAN_TOKEN_SUM || ap.mode == VAMD_AGG_SEQ_MEAN_TOKEN_MEAN) {
         double m = 0;
-        for (int k = 0; k < chunks; ++k) m += partials[(r * chunks + k) * NV + 1];
+        for (int k = 0; k < chunks; ++k) m += peer_load(partials + (r * chunks + k) * NV + 1);
         c = 0;
         if (m > 0) c = (ap.mode == VAMD_AGG_SEQ_MEAN_TOKEN_SUM ? 1.0 : 1.0 / (m + 1e-8)) * ap.dp_size / gbs;
       }

@@ -129,7 +129,7 @@ def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torc
         ret = torch.empty_like(r)
         mom = torch.empty(4, dtype=torch.float64, device=dev)
         Lb = _cabi.lib()
-        ws = _cabi.workspace(Lb.vamd_gae_workspace_bytes(B, Lc), dev)
+        ws = _cabi.ticket_workspace(Lb.vamd_gae_workspace_bytes(B, Lc), dev)
         with torch.cuda.device(dev):
             _cabi.check(Lb.vamd_gae(r.data_ptr(), v.data_ptr(), m.data_ptr(), code, B, Lc, float(gamma), float(lam),
                                     1, adv.data_ptr(), ret.data_ptr(), mom.data_ptr(), ws.data_ptr(), ws.numel(),
@@ -151,7 +151,7 @@ def _grpo(token_level_rewards, response_mask, index, epsilon, norm_adv_by_std_in
         ids = ids.to(dev)
         adv = torch.empty_like(r)
         Lb = _cabi.lib()
-        ws = _cabi.workspace(Lb.vamd_grpo_workspace_bytes(B, Lc, G), dev)
+        ws = _cabi.ticket_workspace(Lb.vamd_grpo_workspace_bytes(B, Lc, G), dev)
         with torch.cuda.device(dev):
             _cabi.check(Lb.vamd_grpo_advantage(r.data_ptr(), m.data_ptr(), code, ids.data_ptr(), B, Lc, G,
                                                float(epsilon), int(bool(norm_adv_by_std_in_grpo)), std_mode,
@@ -207,7 +207,7 @@ class _AggLoss(torch.autograd.Function):
         Lb = _cabi.lib()
         out = torch.empty((), dtype=torch.float32, device=dev)
         coef = torch.empty(rows, dtype=torch.float32, device=dev)
-        ws = _cabi.workspace(Lb.vamd_agg_loss_workspace_bytes(rows, cols), dev)
+        ws = _cabi.ticket_workspace(Lb.vamd_agg_loss_workspace_bytes(rows, cols), dev)
         with torch.cuda.device(dev):
             _cabi.check(Lb.vamd_agg_loss_forward(x.data_ptr(), m.data_ptr(), code, rows, cols, mode, dp_size, bnt,
                                                  gbs, lsf, out.data_ptr(), coef.data_ptr(), ws.data_ptr(),
@@ -263,7 +263,7 @@ class _PolicyLoss(torch.autograd.Function):
         out = torch.empty(4, dtype=torch.float32, device=dev)
         coef = torch.empty(rows, dtype=torch.float32, device=dev)
         g = torch.empty_like(lp) if need_grad else None
-        ws = _cabi.workspace(Lb.vamd_policy_loss_workspace_bytes(rows, cols), dev)
+        ws = _cabi.ticket_workspace(Lb.vamd_policy_loss_workspace_bytes(rows, cols), dev)
         with torch.cuda.device(dev):
             _cabi.check(Lb.vamd_policy_loss_forward(old.data_ptr(), lp.data_ptr(), adv.data_ptr(), m.data_ptr(), code,
                                                     _cabi.ptr(isw), rows, cols, clip_low, clip_high, clip_c, mode,
@@ -372,7 +372,7 @@ class _ValueLoss(torch.autograd.Function):
         out = torch.empty(2, dtype=torch.float32, device=dev)
         coef = torch.empty(rows, dtype=torch.float32, device=dev)
         g = torch.empty_like(vp) if need_grad else None
-        ws = _cabi.workspace(Lb.vamd_value_loss_workspace_bytes(rows, cols), dev)
+        ws = _cabi.ticket_workspace(Lb.vamd_value_loss_workspace_bytes(rows, cols), dev)
         with torch.cuda.device(dev):
             _cabi.check(Lb.vamd_value_loss_forward(vp.data_ptr(), ret.data_ptr(), val.data_ptr(), m.data_ptr(), code,
                                                    rows, cols, cliprange_value, mode, out.data_ptr(), _cabi.ptr(g),

@@ -28,7 +28,7 @@ def _moments(values: torch.Tensor, mask: torch.Tensor, per_row: bool) -> torch.T
     L = _cabi.lib()
     out = torch.empty((rows, 4) if per_row else (4,), dtype=torch.float64, device=dev)
     mk, code = _cabi.mask_code(mask)
-    ws = _cabi.workspace(L.vamd_masked_moments_workspace_bytes(rows, cols), dev)
+    ws = _cabi.ticket_workspace(L.vamd_masked_moments_workspace_bytes(rows, cols), dev)
     with torch.cuda.device(dev):
         _cabi.check(L.vamd_masked_moments(values.data_ptr(), mk.data_ptr(), code, rows, cols, int(per_row),
                                           out.data_ptr(), ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
