@@ -23,8 +23,9 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
-KERNEL_NAMES = ["lce_forward_kernel", "lce_merge_kernel", "lce_recompute_kernel", "lce_dhidden_kernel",
-                "lce_dweight_kernel"]
+KERNEL_NAMES = ["lce_forward_kernel", "lce_merge_kernel", "lce_recompute_kernel", "lce_dgrad_kernel"]
+# MFMA GEMMs of 2*N*V*H flops each that a kernel performs per step
+GEMMS_PER_STEP = {"lce_forward_kernel": 1, "lce_recompute_kernel": 1, "lce_dgrad_kernel": 2}
 
 
 def cpu_baseline(n_cpu: int, h: int, v: int, temperature: float) -> dict:
@@ -102,8 +103,8 @@ def main() -> None:
     prof_steps = max(1, min(args.steps, 5))
     for _ in range(prof_steps):
         step()
-    ms = (ctypes.c_double * 5)()
-    cnt = (ctypes.c_int64 * 5)()
+    ms = (ctypes.c_double * len(KERNEL_NAMES))()
+    cnt = (ctypes.c_int64 * len(KERNEL_NAMES))()
     _cabi.check(L.vamd_lce_timing_collect(ms, cnt))
     L.vamd_lce_timing_enable(0)
     kernels = {}
@@ -111,10 +112,10 @@ def main() -> None:
         if cnt[i]:
             kernels[name] = {"ms_per_step": ms[i] / prof_steps, "launches_per_step": cnt[i] / prof_steps,
                              "avg_ms": ms[i] / cnt[i]}
-    gemm_flops = 2.0 * n * v * h  # every one of the four MFMA kernels performs 2NVH flops per step
-    dom = max((k for k in kernels if k != "lce_merge_kernel"), key=lambda k: kernels[k]["ms_per_step"])
+    gemm_flops = 2.0 * n * v * h
+    dom = max((k for k in kernels if k in GEMMS_PER_STEP), key=lambda k: kernels[k]["ms_per_step"])
     d = kernels[dom]
-    flops_per_launch = gemm_flops / d["launches_per_step"]
+    flops_per_launch = GEMMS_PER_STEP[dom] * gemm_flops / d["launches_per_step"]
     achieved = flops_per_launch / (d["avg_ms"] * 1e-3) / 1e12
     roofline = {
         "bound": "mfma",

@@ -89,7 +89,7 @@ int vamd_lce_backward(const void* hidden, const void* weight, const int64_t* lab
 /* Benchmark aid (no counterpart in the reference): with timing enabled, every head kernel
  * launch of the process is bracketed by HIP events on its stream.  vamd_lce_timing_collect
  * waits for them and adds up milliseconds and launch counts per kernel, indexed
- * 0 forward, 1 merge, 2 logit recompute, 3 d_hidden GEMM, 4 d_weight GEMM (arrays of 5). */
+ * 0 forward, 1 merge, 2 logit recompute, 3 gradient GEMMs (d_hidden + d_weight) (arrays of 4). */
 int vamd_lce_timing_enable(int on);
 int vamd_lce_timing_collect(double* ms_by_kernel_host, int64_t* launches_by_kernel_host);
 

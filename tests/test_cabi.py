@@ -42,7 +42,7 @@ def test_workspace_queries(lib):
     full = lib.vamd_lce_backward_workspace_bytes(n, h, v, 0)
     assert full < 1 << 30                                         # d_logits panel + fp32 d_hidden accumulator
     one = lib.vamd_lce_backward_workspace_bytes(256, 128, 1024, 0)
-    assert one == 256 * 1024 * 2                                  # a single panel, no accumulator
+    assert one == 256 * (1024 + 128) * 2                          # a single padded panel, no accumulator
     # single-launch reductions: 256-byte ticket header + one record of doubles per 4096-column chunk
     assert lib.vamd_masked_moments_workspace_bytes(512, 4096) == 256 + 512 * 4 * 8
     assert lib.vamd_policy_loss_workspace_bytes(512, 4097) == 256 + 512 * 2 * 5 * 8

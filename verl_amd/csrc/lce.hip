@@ -10,6 +10,8 @@
 // Arithmetic follows LinearCrossEntropy (verl/utils/kernel/linear_cross_entropy.py:40-116) /
 // efficient_entropy_forward+backward (verl/utils/kernel/kernels.py:563-753, :1512-1723): bf16
 // products, fp32 accumulation, logits scaled by 1/temperature in fp32, fp32 softmax state.
+#include <stdlib.h>
+
 #include <atomic>
 #include <mutex>
 #include <vector>
@@ -28,7 +30,7 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // Optional per-kernel timing for benchmarks: when enabled, every head kernel launch (from any
 // thread: autograd runs backward on its own) is bracketed by a pair of HIP events on the launch
 // stream.
-enum : int { kTagForward = 0, kTagMerge = 1, kTagRecompute = 2, kTagDHidden = 3, kTagDWeight = 4, kNumTags = 5 };
+enum : int { kTagForward = 0, kTagMerge = 1, kTagRecompute = 2, kTagDGrad = 3, kNumTags = 4 };
 struct TimedLaunch {
   int tag;
   hipEvent_t start, stop;
@@ -393,30 +395,40 @@ struct DWeightEpi {
   }
 };
 
-__global__ __launch_bounds__(kThreads) void lce_dhidden_kernel(GemmOutArgs a) {
+// Both gradient GEMMs of one vocabulary chunk in a single launch: a workgroup first walks its
+// share of the d_hidden tiles, then its share of the d_weight tiles.  The second walk starts at
+// the workgroup after the last one that received an extra tile in the first, so the combined
+// tile count, not each GEMM's, decides how full the last round is (896 + 896 tiles on 256 CUs:
+// 7 full rounds instead of 2 x 3.5).
+__global__ __launch_bounds__(kThreads) void lce_dgrad_kernel(GemmOutArgs gh, GemmOutArgs gw) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
-  GroupedSched sched;
-  sched.r_tiles = a.r_tiles;
-  sched.c_tiles = a.c_tiles;
-  sched.nwg = gridDim.x;
-  sched.wg = xcd_regroup(blockIdx.x, gridDim.x);
-  DHiddenEpi epi;
-  epi.p = lane_pos();
-  epi.a = &a;
-  run_tiles<false, true>(a.R, a.C, a.k_slabs, sched, epi, lds);
-}
-
-__global__ __launch_bounds__(kThreads) void lce_dweight_kernel(GemmOutArgs a) {
-  extern __shared__ __attribute__((aligned(16))) char lds[];
-  GroupedSched sched;
-  sched.r_tiles = a.r_tiles;
-  sched.c_tiles = a.c_tiles;
-  sched.nwg = gridDim.x;
-  sched.wg = xcd_regroup(blockIdx.x, gridDim.x);
-  DWeightEpi epi;
-  epi.p = lane_pos();
-  epi.a = &a;
-  run_tiles<true, true>(a.R, a.C, a.k_slabs, sched, epi, lds);
+  const int nwg = gridDim.x;
+  const int wg = xcd_regroup(blockIdx.x, nwg);
+  const LanePos pos = lane_pos();
+  {
+    GroupedSched sched;
+    sched.r_tiles = gh.r_tiles;
+    sched.c_tiles = gh.c_tiles;
+    sched.nwg = nwg;
+    sched.wg = wg;
+    DHiddenEpi epi;
+    epi.p = pos;
+    epi.a = &gh;
+    run_tiles<false, true>(gh.R, gh.C, gh.k_slabs, sched, epi, lds);
+  }
+  __syncthreads();
+  {
+    const int rem = (gh.r_tiles * gh.c_tiles) % nwg;
+    GroupedSched sched;
+    sched.r_tiles = gw.r_tiles;
+    sched.c_tiles = gw.c_tiles;
+    sched.nwg = nwg;
+    sched.wg = (wg - rem + nwg) % nwg;
+    DWeightEpi epi;
+    epi.p = pos;
+    epi.a = &gw;
+    run_tiles<true, true>(gw.R, gw.C, gw.k_slabs, sched, epi, lds);
+  }
 }
 
 // =============================================================================================
@@ -436,13 +448,17 @@ static int ensure_lds_attributes() {
     int s;
     if ((s = allow_big_lds(lce_forward_kernel)) != VAMD_OK) { status = s; return; }
     if ((s = allow_big_lds(lce_recompute_kernel)) != VAMD_OK) { status = s; return; }
-    if ((s = allow_big_lds(lce_dhidden_kernel)) != VAMD_OK) { status = s; return; }
-    if ((s = allow_big_lds(lce_dweight_kernel)) != VAMD_OK) { status = s; return; }
+    if ((s = allow_big_lds(lce_dgrad_kernel)) != VAMD_OK) { status = s; return; }
   });
   return status;
 }
 
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Row pitch of the staged d_logits panel: the chunk width plus 256 bytes, so that the rows a
+// wavefront touches together (32 .. 64 consecutive tokens at one column) spread over the memory
+// channels instead of landing on a power-of-two stride.
+static inline int64_t dz_pitch(int64_t cv) { return cv + 128; }
 
 static int fwd_splits(int64_t tok_tiles, int64_t voc_tiles) {
   const int cus = device_cu_count();
@@ -466,7 +482,11 @@ static int64_t default_vocab_chunk(int64_t n_tokens, int64_t vocab, int64_t requ
   const int64_t v_pad = ceil_div(vocab, kTile) * kTile;
   int64_t cv = requested;
   if (cv <= 0) {
-    const int64_t budget = 512ll << 20;  // bytes of bf16 d_logits staged at a time
+    int64_t budget = 512ll << 20;  // bytes of bf16 d_logits staged at a time
+    if (const char* e = getenv("VAMD_LCE_DZ_BUDGET_MB")) {
+      const long mb = strtol(e, nullptr, 10);
+      if (mb > 0) budget = (int64_t)mb << 20;
+    }
     cv = budget / (n_pad * 2) / kTile * kTile;
   }
   cv = ceil_div(cv, kTile) * kTile;
@@ -572,7 +592,7 @@ extern "C" size_t vamd_lce_backward_workspace_bytes(int64_t n_tokens, int64_t hi
   if (n_tokens <= 0 || vocab <= 0 || hidden_size <= 0) return 0;
   const int64_t n_pad = ceil_div(n_tokens, kTile) * kTile;
   const int64_t cv = default_vocab_chunk(n_tokens, vocab, vocab_chunk);
-  size_t bytes = align_up((size_t)n_pad * cv * 2, 256);
+  size_t bytes = align_up((size_t)n_pad * dz_pitch(cv) * 2, 256);
   if (cv < ceil_div(vocab, kTile) * kTile) bytes += align_up((size_t)n_tokens * hidden_size * 4, 256);
   return bytes;
 }
@@ -600,7 +620,8 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
   const int64_t cv = default_vocab_chunk(n_tokens, vocab, vocab_chunk);
   const int n_chunks = (int)ceil_div(vocab, cv);
   Carver carve(workspace);
-  uint16_t* dz = carve.take<uint16_t>((size_t)n_pad * cv);
+  const int64_t pitch = dz_pitch(cv);
+  uint16_t* dz = carve.take<uint16_t>((size_t)n_pad * pitch);
   float* acc32 = n_chunks > 1 ? carve.take<float>((size_t)n_tokens * hidden_size) : nullptr;
   const uint16_t* hid = static_cast<const uint16_t*>(hidden);
   const uint16_t* wgt = static_cast<const uint16_t*>(weight);
@@ -630,7 +651,7 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
     r.scale2 = rcp_temperature * kLog2e;
     r.rcp_t = rcp_temperature;
     r.dz = dz;
-    r.dz_ld = (int)cv;
+    r.dz_ld = (int)pitch;
     {
       const int tiles = tok_tiles * chunk_tiles;
       const int grid = tiles < cus ? tiles : cus;
@@ -643,7 +664,7 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
 
     // d_hidden: k runs over the chunk's vocabulary columns (staged zeros beyond `cols`)
     GemmOutArgs gh;
-    gh.R = Operand{dz, cv, (int)n_pad, (int)cv};
+    gh.R = Operand{dz, pitch, (int)n_pad, (int)cv};
     gh.C = Operand{wgt + c0 * hidden_size, hidden_size, (int)hidden_size, (int)left};
     gh.k_slabs = (int)ceil_div(cols, kBK);
     gh.r_tiles = tok_tiles;
@@ -657,19 +678,9 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
     gh.acc32 = acc32;
     gh.out = static_cast<uint16_t*>(d_hidden);
     gh.ld_out = hidden_size;
-    {
-      const int tiles = gh.r_tiles * gh.c_tiles;
-      const int grid = tiles < cus ? tiles : cus;
-      {
-        ScopedTiming tm(kTagDHidden, s);
-        hipLaunchKernelGGL(lce_dhidden_kernel, dim3(grid), dim3(kThreads), kLdsBytes, s, gh);
-      }
-      VAMD_LAUNCH_CHECK();
-    }
-
     // d_weight rows of this chunk: k runs over tokens (staged zeros beyond n_tokens)
     GemmOutArgs gw;
-    gw.R = Operand{dz, cv, (int)(ceil_div(cols, 8) * 8), (int)n_pad};
+    gw.R = Operand{dz, pitch, (int)(ceil_div(cols, 8) * 8), (int)n_pad};
     gw.C = Operand{hid, hidden_size, (int)hidden_size, (int)n_tokens};
     gw.k_slabs = (int)ceil_div(n_tokens, kBK);
     gw.r_tiles = chunk_tiles;
@@ -681,14 +692,12 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
     gw.out = static_cast<uint16_t*>(d_weight) + c0 * hidden_size;
     gw.ld_out = hidden_size;
     {
-      const int tiles = gw.r_tiles * gw.c_tiles;
+      const int tiles = gh.r_tiles * gh.c_tiles + gw.r_tiles * gw.c_tiles;
       const int grid = tiles < cus ? tiles : cus;
-      {
-        ScopedTiming tm(kTagDWeight, s);
-        hipLaunchKernelGGL(lce_dweight_kernel, dim3(grid), dim3(kThreads), kLdsBytes, s, gw);
-      }
-      VAMD_LAUNCH_CHECK();
+      ScopedTiming tm(kTagDGrad, s);
+      hipLaunchKernelGGL(lce_dgrad_kernel, dim3(grid), dim3(kThreads), kLdsBytes, s, gh, gw);
     }
+    VAMD_LAUNCH_CHECK();
   }
   return VAMD_OK;
 }
