@@ -25,6 +25,7 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 KERNEL_NAMES = ["lce_forward_kernel", "lce_merge_kernel", "lce_recompute_kernel", "lce_dgrad_kernel"]
 # MFMA GEMMs of 2*N*V*H flops each that a kernel performs per step
+COPY_YARDSTICK_BYTES = 1 << 30
 GEMMS_PER_STEP = {"lce_forward_kernel": 1, "lce_recompute_kernel": 1, "lce_dgrad_kernel": 2}
 
 
@@ -86,6 +87,15 @@ def main() -> None:
         lp, ent = linear_cross_entropy(hidden, weight, labels, T)
         return torch.autograd.grad((lp, ent), (hidden, weight), (g_lp, g_ent))
 
+    # one plain 1 GiB copy, untimed: under a counter-collecting profiler its FETCH_SIZE / WRITE_SIZE
+    # readings are the yardstick that turns the other kernels' readings into bytes
+    L = _cabi.lib()
+    src = torch.empty(COPY_YARDSTICK_BYTES, dtype=torch.uint8, device=dev).random_(0, 256)
+    dst = torch.empty_like(src)
+    _cabi.check(L.vamd_copy_bytes(src.data_ptr(), dst.data_ptr(), COPY_YARDSTICK_BYTES, _cabi.stream_ptr(dev)))
+    torch.cuda.synchronize()
+    del src, dst
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -98,7 +108,6 @@ def main() -> None:
     tokens_per_s = n * args.steps / dt
 
     # per-kernel durations from HIP events on the launch stream (a separate, untimed pass)
-    L = _cabi.lib()
     L.vamd_lce_timing_enable(1)
     prof_steps = max(1, min(args.steps, 5))
     for _ in range(prof_steps):

@@ -48,6 +48,11 @@ extern "C" {
 int vamd_abi_version(void);
 const char* vamd_last_error(void);
 
+/* Measurement aid (no counterpart in the reference): a plain 16-byte-per-lane copy of `bytes`
+ * (a multiple of 16, both pointers 16-byte aligned) from src to dst.  Profilers read its memory
+ * counters next to those of the other kernels to turn counter units into bytes. */
+int vamd_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Fused vocab-projection log-prob / entropy head.
  * Replaces kernels.efficient_entropy_forward / efficient_entropy_backward behind

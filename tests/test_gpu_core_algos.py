@@ -381,3 +381,15 @@ def test_benchmark_config_gae_value_policy_loss(dev):
     new = old + torch.randn(B, L, generator=g) * 0.05
     loss, _ = CA.compute_policy_loss_vanilla(old.to(dev), new.to(dev), adv, mask.to(dev), "token-mean", _cfg())
     _close(loss, O.policy_loss_vanilla(old, new, want_adv, mask, "token-mean")[0], rtol=1e-4, what="pg_loss")
+
+
+@pytest.mark.gpu
+def test_copy_bytes_is_exact(dev):
+    """The measurement yardstick copies every byte, including a tail shorter than one grid stride."""
+    from verl_amd import _cabi
+    for nbytes in (16, 4096 + 16, (1 << 24) + 48):
+        src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 256)
+        dst = torch.zeros_like(src)
+        _cabi.check(_cabi.lib().vamd_copy_bytes(src.data_ptr(), dst.data_ptr(), nbytes, _cabi.stream_ptr(dev)))
+        assert torch.equal(src, dst)
+    assert _cabi.lib().vamd_copy_bytes(src.data_ptr(), dst.data_ptr(), 24, _cabi.stream_ptr(dev)) == -1

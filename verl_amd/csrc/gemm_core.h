@@ -103,9 +103,20 @@ __device__ __forceinline__ int acc_row(const LanePos& p, int nb) { return p.wr *
 // ds_read_b128 is served 16 lanes (256 B, all 64 banks) per cycle; a fragment read touches 16
 // consecutive rows at one logical chunk, i.e. 8 even and 8 odd rows (two rows span the 64
 // banks), so rows of equal parity must land on 8 different chunk positions: (r >> 1) & 7.
-// Staging writes cover whole 128 B rows with consecutive lanes and are conflict free under
-// any XOR of the chunk index.
-__device__ __forceinline__ int swizzle_of(int row) { return (row >> 1) & 7; }
+// Transposing (kmajor) staging writes 8-byte half chunks of rows that are 8 apart from
+// consecutive lanes; XOR-ing in (r >> 4) spreads those over all 8 chunk positions as well
+// while only adding a constant to any run of 16 consecutive rows.
+// Direct staging writes cover whole 128 B rows with consecutive lanes and are conflict free
+// under any XOR of the chunk index.
+__device__ __forceinline__ int swizzle_of(int row) { return ((row >> 1) ^ (row >> 4)) & 7; }
+
+// Byte offset inside a slab of the fragment chunk `logical_chunk` for the lane whose block-local
+// row is lr, in the 32-row block that starts at row `block_row` of the slab: the lane part; the
+// caller XORs (block index within the wavefront) << 5, which is the compile-time part of
+// swizzle_of(block_row + 32 i + lr).
+__device__ __forceinline__ int frag_chunk_off(int logical_chunk, int block_row, int lr) {
+  return (logical_chunk ^ swizzle_of(block_row + lr)) << 4;
+}
 
 // ---------------------------------------------------------------------------------------------
 // Where one slab of an operand comes from: a buffer resource whose base is the operand's tile
@@ -137,10 +148,11 @@ __device__ __forceinline__ unsigned slab_soff(const Operand& op, int k0) {
 //
 // direct : load i is row (t/8 + 64 i), 16-byte chunk t%8 of the slab; 8 lanes fetch one 128 B row
 //          and store i writes load i as one 16-byte chunk.
-// kmajor : thread (kq = t%16, xg = t/16) owns the 8(x) x 4(k) block at x = 8 xg, k = 4 kq; load i
-//          is the 8 x-values of k = 4 kq + i; the block is transposed in registers and store j
-//          writes the 4 k-values of x = 8 xg + j as one 8-byte half chunk, so no transposed copy
-//          of an operand ever exists in memory.
+// kmajor : thread (xg, kq) owns the 8(x) x 4(k) block at x = 8 xg, k = 4 kq, with xg = lane%8 +
+//          8 (wave%4) and kq = lane/8 + 8 (wave/4): load i is the 8 x-values of k = 4 kq + i, so 8
+//          consecutive lanes fetch one whole 128 B line of a memory row; the block is transposed
+//          in registers and store j writes the 4 k-values of x = 8 xg + j as one 8-byte half
+//          chunk, so no transposed copy of an operand ever exists in memory.
 // Either way the per-lane address is ONE 32-bit offset; everything that changes between loads,
 // slabs and tiles is scalar (buffer resource + scalar offset).
 template <bool KMAJOR>
@@ -159,15 +171,17 @@ struct SlabLoader {
       const unsigned kc = t & 7, row = t >> 3;  // rows 0..63, + 64 per load
       voff = row * ld_bytes + kc * 16u;
       step = 64u * ld_bytes;
-      // swizzle_of(row + 64 i) == swizzle_of(row): one LDS offset serves all four stores
+      // swizzle_of(row + 64 i) == swizzle_of(row) ^ 4 (i & 1): store i flips bit 6 of the offset
       lds_off = row * 128u + ((kc ^ (unsigned)swizzle_of((int)row)) << 4);
       lds_xor = 0;
     } else {
-      const unsigned kq = t & 15, xg = t >> 4;
+      const unsigned lane = t & 63u, w = t >> 6;
+      const unsigned xg = (lane & 7u) + 8u * (w & 3u), kq = (lane >> 3) + 8u * (w >> 2);
       voff = kq * 4u * ld_bytes + xg * 16u;
       step = ld_bytes;
       lds_off = xg * 1024u + (kq & 1u) * 8u;
-      lds_xor = (kq >> 1) ^ ((xg & 1u) << 2);  // swizzle_of(8 xg + j) = ((xg & 1) << 2) | (j >> 1)
+      // swizzle_of(8 xg + j) = (((xg & 1) << 2) | (j >> 1)) ^ ((xg >> 1) & 7)
+      lds_xor = (kq >> 1) ^ ((xg & 1u) << 2) ^ ((xg >> 1) & 7u);
     }
   }
 
@@ -177,7 +191,7 @@ struct SlabLoader {
 
   __device__ __forceinline__ void store_one(int j, char* slab) const {
     if constexpr (!KMAJOR) {
-      *reinterpret_cast<u32x4*>(slab + lds_off + j * 8192) = reg[j];
+      *reinterpret_cast<u32x4*>(slab + (lds_off ^ ((unsigned)(j & 1) << 6)) + j * 8192) = reg[j];
     } else {
       // x = 8 xg + j : bf16 #j of each of the 4 loads (k = 4 kq .. 4 kq + 3)
       u32x2 o;
@@ -221,29 +235,32 @@ template <bool RK, bool CK>
 __device__ __forceinline__ void slab_iter(SlabLoader<RK>& lr, SlabLoader<CK>& lc, const SlabSrc& c1,
                                           const SlabSrc& r2, const SlabSrc& c2, const char* cur, char* nxt,
                                           const LanePos& p, Frags& f0, Accum& acc) {
-  const int sw = swizzle_of(p.lr);
-  const int lane_r = (p.wr * (kNB * 32) + p.lr) * 128;
-  const int lane_c = kSlabBytes + (p.wc * (kMB * 32) + p.lr) * 128;
+  const int row_r = p.wr * (kNB * 32), row_c = p.wc * (kMB * 32);
+  const int lane_r = (row_r + p.lr) * 128;
+  const int lane_c = kSlabBytes + (row_c + p.lr) * 128;
   Frags f1;
 #define VAMD_MFMA(F, i)                                                                                            \
   acc.a[(i) >> 1][(i) & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F.c[(i) >> 1], F.r[(i) & 1],                    \
                                                                      acc.a[(i) >> 1][(i) & 1], 0, 0, 0)
-#define VAMD_FRAG(G, base, i, chunk)                                                                    \
-  do {                                                                                                  \
-    if ((i) < kMB) G.c[(i)] = *reinterpret_cast<const bf16x8*>((base) + lane_c + (i) * 4096 + (chunk));  \
-    else if ((i) < kMB + kNB)                                                                           \
-      G.r[(i) - kMB] = *reinterpret_cast<const bf16x8*>((base) + lane_r + ((i) - kMB) * 4096 + (chunk)); \
+#define VAMD_FRAG(G, base, i, lc)                                                                              \
+  do {                                                                                                         \
+    if ((i) < kMB)                                                                                             \
+      G.c[(i)] = *reinterpret_cast<const bf16x8*>((base) + lane_c + (i) * 4096 +                                \
+                                                  (frag_chunk_off((lc) + p.lh, row_c, p.lr) ^ ((i) << 5)));     \
+    else if ((i) < kMB + kNB)                                                                                  \
+      G.r[(i) - kMB] = *reinterpret_cast<const bf16x8*>((base) + lane_r + ((i) - kMB) * 4096 +                  \
+                                                        (frag_chunk_off((lc) + p.lh, row_r, p.lr) ^            \
+                                                         (((i) - kMB) << 5)));                                 \
   } while (0)
 #define VAMD_SLOT_END __builtin_amdgcn_sched_barrier(0)
   constexpr int kRS = SlabLoader<RK>::kStores, kCS = SlabLoader<CK>::kStores;
 
   // ---- step 0 : MFMA(f0); f1 <- step 1 fragments; R staging -> nxt; C[2..3] of slab it+1
   {
-    const int chunk = ((2 + p.lh) ^ sw) << 4;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       VAMD_MFMA(f0, i);
-      VAMD_FRAG(f1, cur, i, chunk);
+      VAMD_FRAG(f1, cur, i, 2);
 #ifndef VAMD_DBG_NO_STORE
       if (kRS == 8 || i < 4) lr.store_one(i, nxt);
 #endif
@@ -256,11 +273,10 @@ __device__ __forceinline__ void slab_iter(SlabLoader<RK>& lr, SlabLoader<CK>& lc
   }
   // ---- step 1 : MFMA(f1); f0 <- step 2 fragments; R[0..1] of slab it+2
   {
-    const int chunk = ((4 + p.lh) ^ sw) << 4;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       VAMD_MFMA(f1, i);
-      VAMD_FRAG(f0, cur, i, chunk);
+      VAMD_FRAG(f0, cur, i, 4);
 #ifndef VAMD_DBG_NO_GLOBAL
       if (i == 1) lr.issue_one(0, r2);
       if (i == 5) lr.issue_one(1, r2);
@@ -270,11 +286,10 @@ __device__ __forceinline__ void slab_iter(SlabLoader<RK>& lr, SlabLoader<CK>& lc
   }
   // ---- step 2 : MFMA(f0); f1 <- step 3 fragments; C staging -> nxt; R[2..3] of slab it+2
   {
-    const int chunk = ((6 + p.lh) ^ sw) << 4;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       VAMD_MFMA(f0, i);
-      VAMD_FRAG(f1, cur, i, chunk);
+      VAMD_FRAG(f1, cur, i, 6);
 #ifndef VAMD_DBG_NO_STORE
       if (kCS == 8 || i < 4) lc.store_one(i, nxt + kSlabBytes);
 #endif
@@ -289,11 +304,10 @@ __device__ __forceinline__ void slab_iter(SlabLoader<RK>& lr, SlabLoader<CK>& lc
   VAMD_SLOT_END;
   // ---- step 3 : MFMA(f1); f0 <- step 0 fragments of the next slab; C[0..1] of slab it+2
   {
-    const int chunk = ((0 + p.lh) ^ sw) << 4;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       VAMD_MFMA(f1, i);
-      VAMD_FRAG(f0, nxt, i, chunk);
+      VAMD_FRAG(f0, nxt, i, 0);
 #ifndef VAMD_DBG_NO_GLOBAL
       if (i == 1) lc.issue_one(0, c2);
       if (i == 5) lc.issue_one(1, c2);
@@ -373,15 +387,15 @@ __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, in
   lds_barrier();
   Frags f0;
   {
-    const int sw = swizzle_of(pos.lr);
-    const int chunk = ((0 + pos.lh) ^ sw) << 4;
+    const int row_r = pos.wr * (kNB * 32), row_c = pos.wc * (kMB * 32);
 #pragma unroll
     for (int i = 0; i < kMB; ++i)
-      f0.c[i] = *reinterpret_cast<const bf16x8*>(lds + kSlabBytes + (pos.wc * (kMB * 32) + pos.lr) * 128 + i * 4096 +
-                                                 chunk);
+      f0.c[i] = *reinterpret_cast<const bf16x8*>(lds + kSlabBytes + (row_c + pos.lr) * 128 + i * 4096 +
+                                                 (frag_chunk_off(pos.lh, row_c, pos.lr) ^ (i << 5)));
 #pragma unroll
     for (int i = 0; i < kNB; ++i)
-      f0.r[i] = *reinterpret_cast<const bf16x8*>(lds + (pos.wr * (kNB * 32) + pos.lr) * 128 + i * 4096 + chunk);
+      f0.r[i] = *reinterpret_cast<const bf16x8*>(lds + (row_r + pos.lr) * 128 + i * 4096 +
+                                                 (frag_chunk_off(pos.lh, row_r, pos.lr) ^ (i << 5)));
   }
 
   int stage = 0;

@@ -31,7 +31,29 @@ int device_cu_count() {
   return cached[dev];
 }
 
+// Plain streaming copy, 16 bytes per lane and grid-stride: the yardstick the memory counters of
+// the other kernels are scaled by.
+__global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, int64_t n16) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
 }  // namespace vamd
+
+extern "C" int vamd_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream) {
+  using namespace vamd;
+  VAMD_REQUIRE(src && dst && bytes > 0 && bytes % 16 == 0, "copy_bytes: need non-null pointers and a multiple of 16 bytes");
+  VAMD_REQUIRE((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) % 16 == 0,
+               "copy_bytes: pointers must be 16-byte aligned");
+  const int64_t n16 = bytes / 16;
+  int64_t blocks = (n16 + 255) / 256;
+  const int64_t cap = (int64_t)device_cu_count() * 16;
+  if (blocks > cap) blocks = cap;
+  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint4*)src,
+                     (uint4*)dst, n16);
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
 
 extern "C" int vamd_abi_version(void) { return 1; }
 extern "C" const char* vamd_last_error(void) { return vamd::g_error; }
