@@ -13,6 +13,9 @@ import pytest
 import torch
 
 import oracle as O
+from conftest import load_golden
+
+GOLDEN = load_golden()
 
 pytestmark = pytest.mark.gpu
 
@@ -43,11 +46,8 @@ def _cfg(**kw):
 
 
 # ---- masked_* -----------------------------------------------------------------------------------
-@pytest.mark.parametrize("value,mask,want", [
-    ([1.0, 2.0, 3.0, 4.0], [1, 0, 0, 1], 2.5),
-    ([1.0, 2.0, float("nan"), 4.0], [1, 0, 0, 1], 2.5),
-    ([1.0, 2.0, float("nan"), 4.0], [1, 0, 1, 0], float("nan")),
-])
+@pytest.mark.parametrize("value,mask,want", [(c["value"], c["mask"], c["expected"])
+                                             for c in GOLDEN["masked_mean"]["cases"]])
 def test_masked_mean_reference_vectors(dev, value, mask, want):
     from verl_amd.utils.torch_functional import masked_mean
     for device in ("cpu", dev):
@@ -136,12 +136,20 @@ def test_gae_multi_turn_fixture_and_errors(dev):
     from verl_amd.trainer.ppo.core_algos import compute_gae_advantage_return
     random.seed(0)
     gamma, lam = random.uniform(0.0, 1.0), random.uniform(0.0, 1.0)
-    rewards = torch.tensor([[0.0, 0.0, 0.1, 0.1, 0.1, 0.0, 0.0, 0.1, 1.0, 0.0, 0.0]])
-    v1 = torch.tensor([[random.uniform(-100.0, 100.0), random.random(), 4.0, 5.0, 6.0,
-                        random.uniform(-100.0, 0), random.random(), 7.0, 9.0, 0.0, 0.0]])
-    v2 = torch.tensor([[random.random(), random.uniform(-100.0, 100.0), 4.0, 5.0, 6.0,
-                        random.random(), random.uniform(0.0, 100.0), 7.0, 9.0, 0.0, 0.0]])
-    mask = torch.tensor([[0, 0, 1, 1, 1, 0, 0, 1, 1, 0, 0]], dtype=torch.float)
+    fx = GOLDEN["gae_multi_turn"]
+    rewards = torch.tensor(fx["rewards"])
+    mask = torch.tensor(fx["response_mask"], dtype=torch.float)
+
+    def values(free):                                   # fixed values on valid tokens, anything elsewhere
+        v = torch.zeros(1, rewards.shape[1])
+        for k, x in fx["values_at_valid_and_padding"].items():
+            v[0, int(k)] = x
+        for slot, x in zip(fx["free_value_slots"], free):
+            v[0, slot] = x
+        return v
+
+    v1 = values([random.uniform(-100.0, 100.0), random.random(), random.uniform(-100.0, 0), random.random()])
+    v2 = values([random.random(), random.uniform(-100.0, 100.0), random.random(), random.uniform(0.0, 100.0)])
     a1, r1 = compute_gae_advantage_return(rewards.to(dev), v1.to(dev), mask.to(dev), gamma, lam)
     a2, r2 = compute_gae_advantage_return(rewards.to(dev), v2.to(dev), mask.to(dev), gamma, lam)
     md = mask.to(dev)
@@ -172,7 +180,7 @@ def _rand_mask(batch_size, seq_len):
     return mask
 
 
-@pytest.mark.parametrize("batch_size,seq_len,num_groups,seed", [(64, 128, 5, 0), (128, 256, 8, 1), (512, 512, 10, 2)])
+@pytest.mark.parametrize("batch_size,seq_len,num_groups,seed", GOLDEN["grpo_equivalence_grid"]["cases"])
 def test_grpo_reference_grid(dev, batch_size, seq_len, num_groups, seed):
     from verl_amd.trainer.ppo import core_algos as CA
     torch.manual_seed(seed); random.seed(seed); np.random.seed(seed)
@@ -208,9 +216,17 @@ def test_grpo_singletons_equal_scores_and_group_mean_std(dev):
     _close(got, want)
     assert torch.equal(got[1].cpu(), torch.zeros(2)) and torch.equal(got[2].cpu(), torch.zeros(2))
     # reference known answer for group_mean_std
-    mean_g, std_g, cnt_g = group_mean_std(torch.tensor([1.0, 2.0, 3.0], device=dev), as_torch_index([0, 1, 0]))
-    assert torch.allclose(mean_g.cpu(), torch.tensor([2.0, 0.0])) and torch.allclose(cnt_g.cpu(), torch.tensor([2.0, 1.0]))
-    assert std_g[1].item() == 1.0 and abs(std_g[0].item() - 2 ** 0.5) < 1e-6
+    fx = GOLDEN["group_mean_std"]
+    mean_g, std_g, cnt_g = group_mean_std(torch.tensor(fx["scores"], device=dev), as_torch_index(fx["gidx"]))
+    assert torch.allclose(mean_g.cpu(), torch.tensor(fx["expected_mean"]))
+    assert torch.allclose(cnt_g.cpu(), torch.tensor(fx["expected_count"]))
+    assert std_g[1].item() == fx["expected_std"][1] and abs(std_g[0].item() - fx["expected_std"][0]) < 1e-6
+    # the reference's toy GRPO input with the hand-worked un-normalised answer
+    toy = GOLDEN["grpo_toy"]
+    adv, _ = CA.compute_grpo_outcome_advantage(torch.tensor(toy["token_level_rewards"], device=dev),
+                                               torch.tensor(toy["response_mask"], device=dev),
+                                               np.array(toy["index"]), norm_adv_by_std_in_grpo=False)
+    assert torch.allclose(adv[:, 0].cpu(), torch.tensor(toy["expected_unnormalised"]), rtol=1e-5)
     g = as_torch_index(["a", "b", "a", "c", "0042", 42])
     assert g.tolist()[4] != g.tolist()[5] and len(torch.unique(g)) == 5
     e = group_mean_std(torch.tensor([]), torch.tensor([], dtype=torch.long))

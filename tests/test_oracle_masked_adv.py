@@ -12,14 +12,14 @@ import torch
 
 from oracle import advantages as A
 from oracle import masked as M
+from conftest import load_golden
+
+GOLDEN = load_golden()
 
 
 # ---- masked_* ---------------------------------------------------------------------------------
-@pytest.mark.parametrize("value,mask,want", [
-    ([1.0, 2.0, 3.0, 4.0], [1, 0, 0, 1], 2.5),
-    ([1.0, 2.0, float("nan"), 4.0], [1, 0, 0, 1], 2.5),
-    ([1.0, 2.0, float("nan"), 4.0], [1, 0, 1, 0], float("nan")),
-])
+@pytest.mark.parametrize("value,mask,want", [(c["value"], c["mask"], c["expected"])
+                                             for c in GOLDEN["masked_mean"]["cases"]])
 def test_masked_mean_reference_vectors(value, mask, want):
     # literals of tests/utils/test_torch_functional.py:60-71 (int64 mask, as there)
     got = M.masked_mean(torch.tensor(value), torch.tensor(mask))
@@ -109,12 +109,20 @@ def test_gae_multi_turn_fixture_invariance():
     # tests/trainer/ppo/test_core_algos_on_cpu.py:143-197
     random.seed(0)
     gamma, lam = random.uniform(0.0, 1.0), random.uniform(0.0, 1.0)
-    rewards = torch.tensor([[0.0, 0.0, 0.1, 0.1, 0.1, 0.0, 0.0, 0.1, 1.0, 0.0, 0.0]])
-    v1 = torch.tensor([[random.uniform(-100.0, 100.0), random.random(), 4.0, 5.0, 6.0,
-                        random.uniform(-100.0, 0), random.random(), 7.0, 9.0, 0.0, 0.0]])
-    v2 = torch.tensor([[random.random(), random.uniform(-100.0, 100.0), 4.0, 5.0, 6.0,
-                        random.random(), random.uniform(0.0, 100.0), 7.0, 9.0, 0.0, 0.0]])
-    mask = torch.tensor([[0, 0, 1, 1, 1, 0, 0, 1, 1, 0, 0]], dtype=torch.float)
+    fx = GOLDEN["gae_multi_turn"]
+    rewards = torch.tensor(fx["rewards"])
+    mask = torch.tensor(fx["response_mask"], dtype=torch.float)
+
+    def values(free):                                   # fixed values on valid tokens, anything elsewhere
+        v = torch.zeros(1, rewards.shape[1])
+        for k, x in fx["values_at_valid_and_padding"].items():
+            v[0, int(k)] = x
+        for slot, x in zip(fx["free_value_slots"], free):
+            v[0, slot] = x
+        return v
+
+    v1 = values([random.uniform(-100.0, 100.0), random.random(), random.uniform(-100.0, 0), random.random()])
+    v2 = values([random.random(), random.uniform(-100.0, 100.0), random.random(), random.uniform(0.0, 100.0)])
     a1, r1 = A.gae_advantage_return(rewards, v1, mask, gamma, lam)
     a2, r2 = A.gae_advantage_return(rewards, v2, mask, gamma, lam)
     assert torch.equal(a1, a2) and torch.equal(r1 * mask, r2 * mask)
@@ -144,7 +152,7 @@ def _rand_mask(batch_size, seq_len):
     return mask
 
 
-@pytest.mark.parametrize("batch_size,seq_len,num_groups,seed", [(64, 128, 5, 0), (128, 256, 8, 1), (512, 512, 10, 2)])
+@pytest.mark.parametrize("batch_size,seq_len,num_groups,seed", GOLDEN["grpo_equivalence_grid"]["cases"])
 def test_grpo_loop_equals_vectorised_reference_grid(batch_size, seq_len, num_groups, seed):
     # grid and tolerance of tests/trainer/ppo/test_core_algos_on_cpu.py:262-313
     torch.manual_seed(seed); random.seed(seed); np.random.seed(seed)
@@ -159,9 +167,11 @@ def test_grpo_loop_equals_vectorised_reference_grid(batch_size, seq_len, num_gro
 
 def test_group_mean_std_reference_known_answer():
     # tests/utils/test_groupwise.py:51-65
-    mean_g, std_g, cnt_g = A.group_mean_std(torch.tensor([1.0, 2.0, 3.0]), A.as_torch_index([0, 1, 0]))
-    assert torch.allclose(mean_g, torch.tensor([2.0, 0.0])) and torch.allclose(cnt_g, torch.tensor([2.0, 1.0]))
-    assert std_g[1].item() == 1.0 and abs(std_g[0].item() - 2 ** 0.5) < 1e-6
+    fx = GOLDEN["group_mean_std"]
+    mean_g, std_g, cnt_g = A.group_mean_std(torch.tensor(fx["scores"]), A.as_torch_index(fx["gidx"]))
+    assert torch.allclose(mean_g, torch.tensor(fx["expected_mean"]))
+    assert torch.allclose(cnt_g, torch.tensor(fx["expected_count"]))
+    assert std_g[1].item() == fx["expected_std"][1] and abs(std_g[0].item() - fx["expected_std"][0]) < 1e-6
     e = A.group_mean_std(torch.tensor([]), torch.tensor([], dtype=torch.long))
     assert all(t.numel() == 0 for t in e)
 
@@ -180,14 +190,16 @@ def test_as_torch_index_cases():
 def test_grpo_toy_input_by_hand():
     # input of tests/trainer/config/test_algo_config_on_cpu.py:187-197; answer worked by hand:
     # scores (1.5, 3.0 | 0.7, 2.3); unbiased std of a pair = |a-b|/sqrt(2)
-    rewards = torch.tensor([[1.0, 0.5, 0.0], [2.0, 1.0, 0.0], [0.5, 0.2, 0.0], [1.5, 0.8, 0.0]])
-    mask = torch.ones(4, 3)
-    adv, _ = A.grpo_outcome_advantage(rewards, mask, np.array([0, 0, 1, 1]))
+    fx = GOLDEN["grpo_toy"]
+    rewards = torch.tensor(fx["token_level_rewards"])
+    mask = torch.tensor(fx["response_mask"])
+    assert torch.allclose(rewards.sum(-1), torch.tensor(fx["scores"]))
+    adv, _ = A.grpo_outcome_advantage(rewards, mask, np.array(fx["index"]))
     s0, s1 = 1.5 / math.sqrt(2), 1.6 / math.sqrt(2)
     want = torch.tensor([-0.75 / (s0 + 1e-6), 0.75 / (s0 + 1e-6), -0.8 / (s1 + 1e-6), 0.8 / (s1 + 1e-6)])
     assert torch.allclose(adv, want[:, None].expand(4, 3), rtol=1e-5)
     adv2, _ = A.grpo_outcome_advantage(rewards, mask, np.array([0, 0, 1, 1]), norm_adv_by_std_in_grpo=False)
-    assert torch.allclose(adv2[:, 0], torch.tensor([-0.75, 0.75, -0.8, 0.8]), rtol=1e-5)
+    assert torch.allclose(adv2[:, 0], torch.tensor(fx["expected_unnormalised"]), rtol=1e-5)
 
 
 def test_grpo_singletons_strings_equal_scores_and_unmasked_sum():
