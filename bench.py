@@ -60,7 +60,7 @@ def main() -> None:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--cpu-tokens", type=int, default=2048, help="token sample for the CPU baseline (0 = skip)")
+    ap.add_argument("--cpu-tokens", type=int, default=8192, help="token sample for the CPU baseline (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (every box here has one GPU; "
