@@ -66,11 +66,16 @@ int vamd_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream);
  *   entropy = lse(z) - sum softmax(z) z.
  *   lse[n] and mean_z[n] (= sum softmax(z) z) are saved for the backward pass in place of the
  *   reference's (maximum, accumulate, entropy_b) triple.
+ *   logits_cache: NULL, or [n_tokens, vocab] fp32 (16-byte aligned) that receives z.  Handing the
+ *   same buffer to vamd_lce_backward replaces its logits-recompute GEMM by a streaming pass: a
+ *   trade of 4 * n_tokens * vocab bytes of HBM (10 GB at 16384 x 152064) for a quarter of the
+ *   step's matrix work.  Results do not depend on the choice beyond fp32 rounding of z.
  */
 size_t vamd_lce_forward_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab);
 int vamd_lce_forward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
                      int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs, float* entropy,
-                     float* lse, float* mean_z, void* workspace, size_t workspace_bytes, void* stream);
+                     float* lse, float* mean_z, float* logits_cache, void* workspace, size_t workspace_bytes,
+                     void* stream);
 
 /* Backward: d_logits = [g_lp (onehot - p) - g_ent p (z - mean_z)] * rcp_temperature is formed
  * tile by tile from recomputed logits, never as a whole; d_hidden = d_logits . weight,
@@ -88,13 +93,13 @@ size_t vamd_lce_backward_workspace_bytes(int64_t n_tokens, int64_t hidden_size, 
 int vamd_lce_backward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
                       int64_t hidden_size, int64_t vocab, float rcp_temperature, const float* lse,
                       const float* mean_z, const float* d_logprobs, const float* d_entropy, float d_entropy_scalar,
-                      void* d_hidden, void* d_weight, int accumulate_d_weight, int64_t vocab_chunk, void* workspace,
-                      size_t workspace_bytes, void* stream);
+                      const float* logits_cache, void* d_hidden, void* d_weight, int accumulate_d_weight,
+                      int64_t vocab_chunk, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Benchmark aid (no counterpart in the reference): with timing enabled, every head kernel
  * launch of the process is bracketed by HIP events on its stream.  vamd_lce_timing_collect
  * waits for them and adds up milliseconds and launch counts per kernel, indexed
- * 0 forward, 1 merge, 2 logit recompute, 3 gradient GEMMs (d_hidden + d_weight) (arrays of 4). */
+ * 0 forward, 1 merge, 2 d_logits panel (recompute GEMM or cached-logits pass), 3 gradient GEMMs (d_hidden + d_weight) (arrays of 4). */
 int vamd_lce_timing_enable(int on);
 int vamd_lce_timing_collect(double* ms_by_kernel_host, int64_t* launches_by_kernel_host);
 

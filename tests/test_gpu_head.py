@@ -24,6 +24,14 @@ ATOL = 2e-3
 BF16_HALF_ULP = 2.0 ** -8
 
 
+@pytest.fixture(params=["recompute", "logits_cache"])
+def backward_mode(request, monkeypatch):
+    """Autograd tests run twice: with the fp32 logits cache (default) and with it switched off, which makes the
+    backward pass recompute the logits."""
+    monkeypatch.setenv("VAMD_LCE_LOGITS_CACHE_GB", "0" if request.param == "recompute" else "16")
+    return request.param
+
+
 def _make(n, h, v, seed, dist="uniform"):
     g = torch.Generator().manual_seed(seed)
     if dist == "uniform":          # distributions of the reference's test (uniform(-0.5, 0.5))
@@ -95,7 +103,7 @@ def test_forward_small_shapes(dev, n, h, v, T):
 @pytest.mark.parametrize("n,h,v", [(1, 128, 128), (127, 128, 384), (129, 256, 1152), (300, 384, 1000),
                                    (513, 128, 5000), (700, 256, 8192)])
 @pytest.mark.parametrize("T", [1.0, 1.5])
-def test_backward_small_shapes(dev, n, h, v, T):
+def test_backward_small_shapes(dev, backward_mode, n, h, v, T):
     from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
     hidden, weight, labels = _make(n, h, v, seed=7 * n + v)
     g = torch.Generator().manual_seed(n)
@@ -128,6 +136,17 @@ def test_backward_multi_chunk_and_accumulate(dev):
     dh1, dw1 = K.efficient_entropy_backward(g_lp.to(dev), None, hd, wd, ld, lse, mz, 0, T, d_entropy_scalar=-0.001)
     _close_bf16(dh1, want_dh, "d_hidden (one chunk)", e_dh)
     _close_bf16(dw1, want_dw, "d_weight (one chunk)", e_dw)
+    # cached logits instead of the recompute GEMM: same outputs, same gradients (z differs by one fp32 rounding)
+    cache = torch.empty(n, v, device=dev)
+    lp_c, ent_c, lse_c, mz_c = K.efficient_entropy_forward(hd, wd, ld, 0, T, logits_cache=cache)
+    assert torch.equal(lp_c, lp) and torch.equal(ent_c, ent) and torch.equal(lse_c, lse) and torch.equal(mz_c, mz)
+    want_z = (hidden.float() @ weight.float().t()) / T
+    assert (cache.cpu() - want_z).abs().max().item() <= 1e-4 * want_z.abs().max().item() + 1e-5
+    for chunk in (768, 0):
+        dh_c, dw_c = K.efficient_entropy_backward(g_lp.to(dev), None, hd, wd, ld, lse, mz, 0, T,
+                                                  d_entropy_scalar=-0.001, vocab_chunk=chunk, logits_cache=cache)
+        _close_bf16(dh_c, want_dh, "d_hidden (cached logits)", e_dh)
+        _close_bf16(dw_c, want_dw, "d_weight (cached logits)", e_dw)
     # accumulate: second call adds into the first call's d_weight
     dw_acc = dw1.clone()
     K.efficient_entropy_backward(g_lp.to(dev), None, hd, wd, ld, lse, mz, 0, T, d_entropy_scalar=-0.001,
@@ -164,7 +183,7 @@ def test_reductions_3d_input_and_argument_errors(dev):
 
 
 @pytest.mark.parametrize("case", [1, 2, 3])
-def test_reference_test_shapes_fwd_bwd(dev, case):
+def test_reference_test_shapes_fwd_bwd(dev, backward_mode, case):
     """Three of the five (N, H, V) cases of the reference's own test (the ragged-N ones that fit a quick run),
     bf16 upstream grads as there; ground truth evaluated in fp32 on the GPU."""
     from conftest import load_golden
@@ -219,3 +238,16 @@ def test_benchmark_config_7b_head_full_size(dev):
     # linearity in the upstream gradient: backward(2 g) == 2 backward(g) up to output rounding
     dh2, _ = K.efficient_entropy_backward(2 * g_lp, None, hidden, weight, labels, lse, mz, 0, T, d_entropy_scalar=0.002)
     _close_bf16(dh2, 2 * dh.float(), "linearity of d_hidden")
+    del dh2
+    # cached-logits path at full size: identical forward outputs; gradients differ from the recompute path only
+    # where one fp32 rounding of z moves a d_logits entry across a bf16 rounding boundary
+    cache = torch.empty(n, v, device=dev)
+    lp_c, ent_c, lse_c, mz_c = K.efficient_entropy_forward(hidden, weight, labels, 0, T, logits_cache=cache)
+    assert torch.equal(lp_c, lp) and torch.equal(ent_c, ent)
+    dh_c, dw_c = K.efficient_entropy_backward(g_lp, None, hidden, weight, labels, lse_c, mz_c, 0, T,
+                                              d_entropy_scalar=0.001, logits_cache=cache)
+    del cache
+    _close_bf16(dh_c, dh.float(), "d_hidden cached vs recomputed")
+    _close_bf16(dw_c, dw.float(), "d_weight cached vs recomputed")
+    assert (dh_c.float() - dh.float()).pow(2).mean().sqrt().item() < 1e-4
+    assert (dw_c.float() - dw.float()).pow(2).mean().sqrt().item() < 1e-4

@@ -70,7 +70,9 @@ struct FwdArgs {
   int n_tokens, vocab, k_slabs;
   int tok_tiles, voc_tiles, splits;
   float scale2;      // log2(e) / temperature
+  float rcp_t;       // 1 / temperature
   float4* partials;  // [splits][tok_tiles * 256] : (max2, sum, sum_y, label logit)
+  float* z_cache;    // optional [n_tokens][vocab] fp32 logits / temperature, kept for the backward
 };
 
 struct SplitSched {
@@ -82,18 +84,62 @@ struct SplitSched {
   }
 };
 
-// Per-lane online-softmax state for the kNB token slots (nb) the lane owns.
+constexpr int kCacheStageBytes = (kThreads / 64) * 4096;  // one 32 x 32 fp32 block per wavefront
+
+// Per-lane online-softmax state for the kNB token slots (nb) the lane owns.  With CACHE the
+// scaled logits of every valid (token, vocabulary column) are also written out in fp32, so the
+// backward pass can form d_logits without repeating the GEMM.
+template <bool CACHE>
 struct FwdEpi {
   LanePos p;
   float scale2;
   int vocab;
   float m[kNB], s[kNB], sy[kNB], zl[kNB];
   int lab[kNB];
+  float rcp_t;
+  float* z_cache;  // CACHE: [n_tokens][vocab]
+  char* stage;     // CACHE: this wavefront's 4 KB LDS patch
+  int tok0;        // CACHE: first token row of the wavefront
+  int n_tokens;
 
   __device__ __forceinline__ void operator()(Accum& acc, int /*r0*/, int c0) {
     const bool ragged = c0 + kTile > vocab;
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
+      if constexpr (CACHE) {
+        // Each 32 x 32 block goes through a 4 KB LDS patch private to the wavefront so that the
+        // global stores are whole 128-byte rows (8 lanes x 16 bytes) instead of 16-byte pieces of
+        // 32 different rows.  LDS operations of one wavefront execute in issue order, so the
+        // patch needs no barrier, only the waits that order its writes and reads.
+        const int lane = threadIdx.x & 63;
+        const int rd_row = lane >> 3, rd_chunk = lane & 7;
+#pragma unroll
+        for (int mb = 0; mb < kMB; ++mb) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const f32x4 z = {acc.a[mb][nb][4 * g] * rcp_t, acc.a[mb][nb][4 * g + 1] * rcp_t,
+                             acc.a[mb][nb][4 * g + 2] * rcp_t, acc.a[mb][nb][4 * g + 3] * rcp_t};
+            *reinterpret_cast<f32x4*>(stage + p.lr * 128 + (((2 * g + p.lh) ^ ((p.lr >> 1) & 7)) << 4)) = z;
+          }
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          f32x4 out[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int row = 8 * i + rd_row;
+            out[i] = *reinterpret_cast<const f32x4*>(stage + row * 128 + ((rd_chunk ^ ((row >> 1) & 7)) << 4));
+          }
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          const int col = c0 + p.wc * 128 + mb * 32 + 4 * rd_chunk;
+          if (col < vocab) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int tok = tok0 + nb * 32 + 8 * i + rd_row;
+              if (tok < n_tokens)
+                __builtin_nontemporal_store(out[i], reinterpret_cast<f32x4*>(z_cache + (int64_t)tok * vocab + col));
+            }
+          }
+        }
+      }
       float ymax = kNegBig;
       // pass 1: scale into the log2 domain in place, mask the vocabulary tail, tile max
 #pragma unroll
@@ -143,6 +189,7 @@ __device__ __forceinline__ void merge_state(float& m, float& s, float& sy, float
   m = mm;
 }
 
+template <bool CACHE>
 __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   // workgroup -> (token tile, vocabulary split); bands of 8 token tiles x all splits per XCD
@@ -161,10 +208,11 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
   sched.vt_begin = (int)(((int64_t)sp * a.voc_tiles) / a.splits);
   sched.vt_count = (int)(((int64_t)(sp + 1) * a.voc_tiles) / a.splits) - sched.vt_begin;
 
-  FwdEpi epi;
+  FwdEpi<CACHE> epi;
   epi.p = lane_pos();
   epi.scale2 = a.scale2;
   epi.vocab = a.vocab;
+  epi.rcp_t = a.rcp_t;
 #pragma unroll
   for (int nb = 0; nb < kNB; ++nb) {
     epi.m[nb] = kNegBig;
@@ -174,6 +222,10 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
     const int tok = sched.r0_ + acc_row(epi.p, nb);
     epi.lab[nb] = tok < a.n_tokens ? (int)a.labels[tok] : -1;
   }
+  epi.z_cache = a.z_cache;
+  epi.stage = lds + kLdsBytes + (threadIdx.x >> 6) * 4096;
+  epi.tok0 = sched.r0_ + epi.p.wr * (kNB * 32);
+  epi.n_tokens = a.n_tokens;
 
   run_tiles<false, false>(a.hidden, a.weight, a.k_slabs, sched, epi, lds);
 
@@ -317,6 +369,49 @@ __global__ __launch_bounds__(kThreads) void lce_recompute_kernel(RecomputeArgs a
   run_tiles<false, false>(a.hidden, a.weight, a.k_slabs, sched, epi, lds);
 }
 
+// d_logits panel of one vocabulary chunk from cached logits: the same arithmetic as RecomputeEpi,
+// one thread per 8 consecutive columns of a token, 2048 columns per workgroup.
+struct DLogitsArgs {
+  const float* z_cache;  // [n_tokens][vocab]
+  const int64_t* labels;
+  const float* lse;
+  const float* mean_z;
+  const float* g_lp;
+  const float* g_ent;
+  float g_ent_scalar, rcp_t;
+  int n_tokens, vocab, chunk_c0, chunk_cols;  // chunk_cols: panel columns to fill (multiple of 256)
+  uint16_t* dz;
+  int dz_ld;
+};
+
+__global__ __launch_bounds__(256) void lce_dlogits_kernel(DLogitsArgs a) {
+  const int tok = blockIdx.x;
+  const int j = (blockIdx.y * 256 + threadIdx.x) * 8;  // column inside the chunk
+  if (j >= a.chunk_cols) return;
+  u32x4 out = {0u, 0u, 0u, 0u};
+  const int col = a.chunk_c0 + j;
+  if (tok < a.n_tokens && col < a.vocab) {  // vocab % 8 == 0: the 8 columns are all in or all out
+    const float lse2 = a.lse[tok] * kLog2e;
+    const float mz = a.mean_z[tok];
+    const float glp = (a.g_lp ? a.g_lp[tok] : 0.f) * a.rcp_t;
+    const float gent = (a.g_ent ? a.g_ent[tok] : a.g_ent_scalar) * a.rcp_t;
+    const int rel = (int)a.labels[tok] - col;
+    const f32x4* src = reinterpret_cast<const f32x4*>(a.z_cache + (int64_t)tok * a.vocab + col);
+    const f32x4 z0 = __builtin_nontemporal_load(src), z1 = __builtin_nontemporal_load(src + 1);
+    float d[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float z = e < 4 ? z0[e] : z1[e - 4];
+      const float prob = fast_exp2(fmaf(z, kLog2e, -lse2));
+      const float u = fmaf(gent, z - mz, glp);
+      d[e] = -prob * u + ((e == rel) ? glp : 0.f);
+    }
+    const u32x2 lo = pack_bf16x4(d[0], d[1], d[2], d[3]), hi = pack_bf16x4(d[4], d[5], d[6], d[7]);
+    out = u32x4{lo[0], lo[1], hi[0], hi[1]};
+  }
+  *reinterpret_cast<u32x4*>(a.dz + (int64_t)tok * a.dz_ld + j) = out;
+}
+
 // ---------------------------------------------------------------------------------------------
 // d_hidden (+)= dz_panel . W[chunk]          R = dz (direct), C = W (kmajor, k = vocab)
 // d_weight[chunk] (+)= dz_panel^T . hidden    R = dz (kmajor, k = token), C = hidden (kmajor)
@@ -435,9 +530,9 @@ __global__ __launch_bounds__(kThreads) void lce_dgrad_kernel(GemmOutArgs gh, Gem
 // Host side
 // =============================================================================================
 template <class K>
-static int allow_big_lds(K kernel) {
+static int allow_big_lds(K kernel, int bytes = kLdsBytes) {
   VAMD_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                               kLdsBytes));
+                               bytes));
   return VAMD_OK;
 }
 
@@ -446,7 +541,8 @@ static int ensure_lds_attributes() {
   static int status = VAMD_OK;
   std::call_once(once, [] {
     int s;
-    if ((s = allow_big_lds(lce_forward_kernel)) != VAMD_OK) { status = s; return; }
+    if ((s = allow_big_lds(lce_forward_kernel<false>)) != VAMD_OK) { status = s; return; }
+    if ((s = allow_big_lds(lce_forward_kernel<true>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) { status = s; return; }
     if ((s = allow_big_lds(lce_recompute_kernel)) != VAMD_OK) { status = s; return; }
     if ((s = allow_big_lds(lce_dgrad_kernel)) != VAMD_OK) { status = s; return; }
   });
@@ -538,8 +634,8 @@ extern "C" size_t vamd_lce_forward_workspace_bytes(int64_t n_tokens, int64_t hid
 
 extern "C" int vamd_lce_forward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
                                 int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs,
-                                float* entropy, float* lse, float* mean_z, void* workspace, size_t workspace_bytes,
-                                void* stream) {
+                                float* entropy, float* lse, float* mean_z, float* logits_cache, void* workspace,
+                                size_t workspace_bytes, void* stream) {
   int st = check_head_shapes(n_tokens, hidden_size, vocab);
   if (st != VAMD_OK) return st;
   VAMD_REQUIRE(hidden && weight && labels && logprobs && entropy && lse && mean_z, "lce_forward: null pointer");
@@ -562,11 +658,18 @@ extern "C" int vamd_lce_forward(const void* hidden, const void* weight, const in
   a.voc_tiles = (int)ceil_div(vocab, kTile);
   a.splits = fwd_splits(a.tok_tiles, a.voc_tiles);
   a.scale2 = rcp_temperature * kLog2e;
+  a.rcp_t = rcp_temperature;
   a.partials = static_cast<float4*>(workspace);
+  a.z_cache = logits_cache;
+  VAMD_REQUIRE(reinterpret_cast<uintptr_t>(logits_cache) % 16 == 0, "lce_forward: logits_cache must be 16-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
   {
     ScopedTiming tm(kTagForward, s);
-    hipLaunchKernelGGL(lce_forward_kernel, dim3(a.tok_tiles * a.splits), dim3(kThreads), kLdsBytes, s, a);
+    if (logits_cache)
+      hipLaunchKernelGGL(lce_forward_kernel<true>, dim3(a.tok_tiles * a.splits), dim3(kThreads),
+                         kLdsBytes + kCacheStageBytes, s, a);
+    else
+      hipLaunchKernelGGL(lce_forward_kernel<false>, dim3(a.tok_tiles * a.splits), dim3(kThreads), kLdsBytes, s, a);
   }
   VAMD_LAUNCH_CHECK();
 
@@ -600,12 +703,14 @@ extern "C" size_t vamd_lce_backward_workspace_bytes(int64_t n_tokens, int64_t hi
 extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
                                  int64_t hidden_size, int64_t vocab, float rcp_temperature, const float* lse,
                                  const float* mean_z, const float* d_logprobs, const float* d_entropy,
-                                 float d_entropy_scalar, void* d_hidden, void* d_weight, int accumulate_d_weight,
-                                 int64_t vocab_chunk, void* workspace, size_t workspace_bytes, void* stream) {
+                                 float d_entropy_scalar, const float* logits_cache, void* d_hidden, void* d_weight,
+                                 int accumulate_d_weight, int64_t vocab_chunk, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
   int st = check_head_shapes(n_tokens, hidden_size, vocab);
   if (st != VAMD_OK) return st;
   VAMD_REQUIRE(hidden && weight && labels && lse && mean_z && d_hidden && d_weight, "lce_backward: null pointer");
   VAMD_REQUIRE(rcp_temperature > 0.f, "lce_backward: temperature must be positive");
+  VAMD_REQUIRE(reinterpret_cast<uintptr_t>(logits_cache) % 16 == 0, "lce_backward: logits_cache must be 16-byte aligned");
   const size_t need = vamd_lce_backward_workspace_bytes(n_tokens, hidden_size, vocab, vocab_chunk);
   if (!workspace || workspace_bytes < need) {
     set_error("lce_backward: workspace %zu bytes, need %zu", workspace_bytes, need);
@@ -633,33 +738,57 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
     const int64_t cols = left < cv ? left : cv;        // valid columns in this chunk
     const int chunk_tiles = (int)ceil_div(cols, kTile);
 
-    RecomputeArgs r;
-    r.hidden = Operand{hid, hidden_size, (int)n_tokens, (int)hidden_size};
-    r.weight = Operand{wgt + c0 * hidden_size, hidden_size, (int)left, (int)hidden_size};
-    r.labels = labels;
-    r.lse = lse;
-    r.mean_z = mean_z;
-    r.g_lp = d_logprobs;
-    r.g_ent = d_entropy;
-    r.g_ent_scalar = d_entropy_scalar;
-    r.n_tokens = (int)n_tokens;
-    r.vocab_left = (int)left;
-    r.chunk_c0 = (int)c0;
-    r.k_slabs = (int)(hidden_size / kBK);
-    r.tok_tiles = tok_tiles;
-    r.chunk_tiles = chunk_tiles;
-    r.scale2 = rcp_temperature * kLog2e;
-    r.rcp_t = rcp_temperature;
-    r.dz = dz;
-    r.dz_ld = (int)pitch;
-    {
-      const int tiles = tok_tiles * chunk_tiles;
-      const int grid = tiles < cus ? tiles : cus;
+    if (logits_cache) {
+      DLogitsArgs d;
+      d.z_cache = logits_cache;
+      d.labels = labels;
+      d.lse = lse;
+      d.mean_z = mean_z;
+      d.g_lp = d_logprobs;
+      d.g_ent = d_entropy;
+      d.g_ent_scalar = d_entropy_scalar;
+      d.rcp_t = rcp_temperature;
+      d.n_tokens = (int)n_tokens;
+      d.vocab = (int)vocab;
+      d.chunk_c0 = (int)c0;
+      d.chunk_cols = chunk_tiles * kTile;
+      d.dz = dz;
+      d.dz_ld = (int)pitch;
       {
         ScopedTiming tm(kTagRecompute, s);
-        hipLaunchKernelGGL(lce_recompute_kernel, dim3(grid), dim3(kThreads), kLdsBytes, s, r);
+        hipLaunchKernelGGL(lce_dlogits_kernel, dim3((unsigned)n_pad, (unsigned)ceil_div(d.chunk_cols, 2048)), dim3(256),
+                           0, s, d);
       }
       VAMD_LAUNCH_CHECK();
+    } else {
+      RecomputeArgs r;
+      r.hidden = Operand{hid, hidden_size, (int)n_tokens, (int)hidden_size};
+      r.weight = Operand{wgt + c0 * hidden_size, hidden_size, (int)left, (int)hidden_size};
+      r.labels = labels;
+      r.lse = lse;
+      r.mean_z = mean_z;
+      r.g_lp = d_logprobs;
+      r.g_ent = d_entropy;
+      r.g_ent_scalar = d_entropy_scalar;
+      r.n_tokens = (int)n_tokens;
+      r.vocab_left = (int)left;
+      r.chunk_c0 = (int)c0;
+      r.k_slabs = (int)(hidden_size / kBK);
+      r.tok_tiles = tok_tiles;
+      r.chunk_tiles = chunk_tiles;
+      r.scale2 = rcp_temperature * kLog2e;
+      r.rcp_t = rcp_temperature;
+      r.dz = dz;
+      r.dz_ld = (int)pitch;
+      {
+        const int tiles = tok_tiles * chunk_tiles;
+        const int grid = tiles < cus ? tiles : cus;
+        {
+          ScopedTiming tm(kTagRecompute, s);
+          hipLaunchKernelGGL(lce_recompute_kernel, dim3(grid), dim3(kThreads), kLdsBytes, s, r);
+        }
+        VAMD_LAUNCH_CHECK();
+      }
     }
 
     // d_hidden: k runs over the chunk's vocabulary columns (staged zeros beyond `cols`)

@@ -4,10 +4,15 @@ Drop-in for ``verl.utils.kernel.linear_cross_entropy`` (reference
 verl/utils/kernel/linear_cross_entropy.py:38-119): same class name, ``forward`` / ``backward``
 signatures, argument checks and return tuple.  The arithmetic runs in ``libverl_amd.so``
 (``vamd_lce_forward`` / ``vamd_lce_backward``): bf16 MFMA logits tiles with an in-register online
-softmax; the ``[tokens, vocab]`` logits are never stored.
+softmax.  The ``[tokens, vocab]`` logits are never needed; when a backward pass will follow and
+``4 * tokens * vocab`` bytes fit the budget below, the forward pass keeps them in fp32 so that the
+backward pass skips its logits-recompute GEMM (a quarter of the step's matrix work) -- HBM is the
+cheap resource on a 288 GB part.  ``VAMD_LCE_LOGITS_CACHE_GB`` sets the budget (default 16,
+0 turns the cache off); results are the same either way.
 """
 from __future__ import annotations
 
+import os
 import typing
 
 import torch
@@ -39,12 +44,18 @@ def _check_inputs(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tens
     assert weight.shape[0] % 8 == 0, "vocab size must be a multiple of 8"
 
 
+def logits_cache_budget_bytes() -> int:
+    """Largest fp32 logits cache the autograd path may allocate (``VAMD_LCE_LOGITS_CACHE_GB``, default 16)."""
+    return int(float(os.environ.get("VAMD_LCE_LOGITS_CACHE_GB", "16")) * (1 << 30))
+
+
 def efficient_entropy_forward(hidden, weight, labels, reduction: int = 0, temperature: float = 1.0,
-                              dist_process_group=None):
+                              dist_process_group=None, logits_cache: torch.Tensor | None = None):
     """Host side of the forward kernels (reference kernels.py:563-753).
 
     Returns ``(logprobs, entropy, lse, mean_z)``; the last two are the per-token statistics the
     backward pass needs (log-sum-exp and softmax-weighted mean of the scaled logits).
+    ``logits_cache``: optional fp32 ``[tokens, vocab]`` tensor that receives the scaled logits.
     """
     if dist_process_group is not None:
         raise NotImplementedError("vocab-parallel process groups are not supported on this single-GPU path")
@@ -59,11 +70,15 @@ def efficient_entropy_forward(hidden, weight, labels, reduction: int = 0, temper
     entropy = torch.empty((n,), device=dev, dtype=torch.float32)
     lse = torch.empty((n,), device=dev, dtype=torch.float32)
     mean_z = torch.empty((n,), device=dev, dtype=torch.float32)
+    if logits_cache is not None:
+        assert logits_cache.shape == (n, v) and logits_cache.dtype == torch.float32
+        assert logits_cache.is_contiguous() and logits_cache.device == dev
     ws = _cabi.workspace(L.vamd_lce_forward_workspace_bytes(n, h, v), dev)
     with torch.cuda.device(dev):
         _cabi.check(L.vamd_lce_forward(hidden.data_ptr(), weight.data_ptr(), labels.data_ptr(), n, h, v,
                                        1.0 / temperature, logprobs.data_ptr(), entropy.data_ptr(), lse.data_ptr(),
-                                       mean_z.data_ptr(), ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
+                                       mean_z.data_ptr(), _cabi.ptr(logits_cache), ws.data_ptr(), ws.numel(),
+                                       _cabi.stream_ptr(dev)))
     if reduction == 1:
         logprobs = _sum_f32(logprobs)
     elif reduction == 2:
@@ -81,12 +96,14 @@ def _sum_f32(x: torch.Tensor) -> torch.Tensor:
 
 def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse, mean_z, reduction: int = 0,
                                temperature: float = 1.0, dist_process_group=None, d_entropy_scalar: float = 0.0,
-                               d_weight_out: torch.Tensor | None = None, vocab_chunk: int = 0):
+                               d_weight_out: torch.Tensor | None = None, vocab_chunk: int = 0,
+                               logits_cache: torch.Tensor | None = None):
     """Host side of the backward kernels (reference kernels.py:1512-1723).
 
     ``dlogprobs`` / ``dentropy`` may be ``None`` (no contribution).  ``d_entropy_scalar`` adds a
     constant upstream entropy gradient for every token without materialising it.  When
     ``d_weight_out`` is given the weight gradient is ACCUMULATED into it (token-chunked use).
+    ``logits_cache``: the tensor the forward call filled, if any (skips the recompute GEMM).
     Returns ``(d_hidden, d_weight)`` in ``hidden.dtype``.
     """
     if dist_process_group is not None:
@@ -110,6 +127,9 @@ def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse,
         dentropy = dentropy.to(torch.float32).contiguous()
         assert d_entropy_scalar == 0.0, "pass the entropy gradient either as a tensor or as a scalar"
     assert lse.shape == (n,) and mean_z.shape == (n,)
+    if logits_cache is not None:
+        assert logits_cache.shape == (n, v) and logits_cache.dtype == torch.float32
+        assert logits_cache.is_contiguous() and logits_cache.device == dev
     if labels.dtype != torch.int64:
         labels = labels.to(torch.int64)
     L = _cabi.lib()
@@ -121,8 +141,8 @@ def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse,
     with torch.cuda.device(dev):
         _cabi.check(L.vamd_lce_backward(hidden.data_ptr(), weight.data_ptr(), labels.data_ptr(), n, h, v,
                                         1.0 / temperature, lse.data_ptr(), mean_z.data_ptr(), _cabi.ptr(dlogprobs),
-                                        _cabi.ptr(dentropy), float(d_entropy_scalar), d_hidden.data_ptr(),
-                                        d_weight.data_ptr(), int(accumulate), int(vocab_chunk), ws.data_ptr(),
+                                        _cabi.ptr(dentropy), float(d_entropy_scalar), _cabi.ptr(logits_cache),
+                                        d_hidden.data_ptr(), d_weight.data_ptr(), int(accumulate), int(vocab_chunk), ws.data_ptr(),
                                         ws.numel(), _cabi.stream_ptr(dev)))
     return d_hidden, d_weight
 
@@ -149,9 +169,13 @@ class LinearCrossEntropy(torch.autograd.Function):
             hidden = hidden.view(-1, hidden.shape[-1])
         if len(labels.shape) != 1:
             labels = labels.view(-1)
+        cache = None
+        n_tokens, vocab = hidden.shape[0], weight.shape[0]
+        if (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]) and 4 * n_tokens * vocab <= logits_cache_budget_bytes():
+            cache = torch.empty((n_tokens, vocab), device=hidden.device, dtype=torch.float32)
         logprobs, entropy, lse, mean_z = efficient_entropy_forward(
-            hidden, weight, labels, REDUCTION, temperature, dist_process_group)
-        ctx.save_for_backward(hidden, weight, labels, lse, mean_z)
+            hidden, weight, labels, REDUCTION, temperature, dist_process_group, logits_cache=cache)
+        ctx.save_for_backward(hidden, weight, labels, lse, mean_z, cache)
         ctx.original_hidden_shape = original_hidden_shape
         ctx.REDUCTION = REDUCTION
         ctx.dist_process_group = dist_process_group
@@ -160,10 +184,10 @@ class LinearCrossEntropy(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dlogprobs: torch.Tensor, dentropy: torch.Tensor):
-        hidden, weight, labels, lse, mean_z = ctx.saved_tensors
+        hidden, weight, labels, lse, mean_z, cache = ctx.saved_tensors
         d_hidden, d_weight = efficient_entropy_backward(
             dlogprobs, dentropy, hidden, weight, labels, lse, mean_z, ctx.REDUCTION, ctx.temperature,
-            ctx.dist_process_group)
+            ctx.dist_process_group, logits_cache=cache)
         d_hidden = d_hidden.view(ctx.original_hidden_shape)
         return (d_hidden, d_weight, None, None, None, None)
 
