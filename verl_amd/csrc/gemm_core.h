@@ -1,32 +1,32 @@
-// bf16 x bf16 -> fp32 MFMA tile engine for gfx950 (MI355X), shared by the four
-// GEMM-shaped kernels of the log-prob/entropy head (forward logits, backward
-// logit recompute, dHidden, dWeight).
+// bf16 x bf16 -> fp32 MFMA tile engine for gfx950 (MI355X), shared by the GEMM-shaped kernels
+// of the log-prob/entropy head (forward logits, backward logit recompute, d_hidden, d_weight).
 //
-// One workgroup = 512 threads = 8 wavefronts (two per SIMD, so that one wavefront's
-// loads, LDS traffic and epilogue arithmetic issue in the shadow of the other's
-// MFMAs) laid out 4 x 2 over a 256 x 256 output tile; each wavefront owns a
-// 64 (rows) x 128 (columns) sub-tile as 2 x 4 blocks of v_mfma_f32_32x32x16_bf16
-// (128 fp32 accumulators per lane).  The tile engine computes
+// One workgroup = 512 threads = 8 wavefronts (two per SIMD, so that one wavefront's LDS traffic
+// and epilogue arithmetic issue in the shadow of the other's MFMAs) laid out 4 x 2 over a
+// 256 x 256 output tile; each wavefront owns a 64 (rows) x 128 (columns) sub-tile as 2 x 4
+// blocks of v_mfma_f32_32x32x16_bf16 (128 fp32 accumulators per lane).  The engine computes
 //
 //     Out[r][c] = sum_k  R[r][k] * C[c][k]
 //
-// where the R operand ("rows of the output") feeds the MFMA B input and the C
-// operand ("columns of the output") feeds the MFMA A input.  With that choice a
-// lane of the accumulator block holds ONE output row (r = lane % 32) and runs
-// of 4 consecutive output columns, so row-wise reductions over c (the softmax
-// over the vocabulary) stay inside a lane and row-major stores are 8/16-byte
-// vectors.
+// where the R operand ("rows of the output") feeds the MFMA B input and the C operand
+// ("columns of the output") feeds the MFMA A input.  With that choice a lane of the accumulator
+// block holds ONE output row (r = lane % 32) and runs of 4 consecutive output columns, so
+// row-wise reductions over c (the softmax over the vocabulary) stay inside a lane and row-major
+// stores are 8/16-byte vectors.
 //
-// Each operand is staged through LDS as a [256 rows][64 k] bf16 slab (128 B per
-// row, 16-byte chunks XOR-swizzled by the row index so that both the staging
-// writes and the ds_read_b128 fragment reads are bank-conflict free).  Two slabs
-// per operand are double-buffered: 4 x 32 KB = 128 KB of the CU's 160 KB LDS.
+// Operand slabs (256 x 64 k, 32 KB) travel from memory straight into LDS with
+// buffer_load_dwordx4 ... lds: no staging registers, no LDS store instructions, and a wavefront
+// waits for its loads once per slab (just before the barrier that publishes the slab) instead of
+// before every staging store.  Two slabs per operand are double-buffered: 4 x 32 KB = 128 KB of
+// the CU's 160 KB LDS.  A load writes the 64 lanes' 16-byte pieces to 1 KB of consecutive LDS, so
+// the bank swizzle is applied on the memory side: each lane fetches the chunk that belongs at
+// its LDS position.
 //
-// An operand may live in memory either K-contiguous ("direct": element (x,k) at
-// base[x*ld + k]) or K-major ("kmajor": element (x,k) at base[k*ld + x]).  The
-// kmajor loader transposes 8x4 bf16 blocks in registers on the way to LDS, so
-// no transposed copy of the weight, the hidden states or dLogits is ever
-// written to memory.
+// An operand may live in memory K-contiguous ("direct": element (x,k) at base[x*ld + k]) or
+// K-major ("kmajor": element (x,k) at base[k*ld + x]).  A direct slab is kept as [256 x][64 k]
+// and read with ds_read_b128; a kmajor slab is kept exactly as it lies in memory, [64 k][256 x],
+// and read with ds_read_b64_tr_b16, which hands every lane the 4 consecutive k of its own x.  No
+// transposed copy of the weight, the hidden states or d_logits is ever written anywhere.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -99,44 +99,37 @@ __device__ __forceinline__ int acc_col(const LanePos& p, int mb, int v) {
 // Row offset inside the 256-tall tile of accumulator block nb for this lane.
 __device__ __forceinline__ int acc_row(const LanePos& p, int nb) { return p.wr * (kNB * 32) + nb * 32 + p.lr; }
 
-// LDS swizzle: the 16-byte chunk c of slab row r lives at chunk position c ^ swizzle_of(r).
-// ds_read_b128 is served 16 lanes (256 B, all 64 banks) per cycle; a fragment read touches 16
-// consecutive rows at one logical chunk, i.e. 8 even and 8 odd rows (two rows span the 64
-// banks), so rows of equal parity must land on 8 different chunk positions: (r >> 1) & 7.
-// Transposing (kmajor) staging writes 8-byte half chunks of rows that are 8 apart from
-// consecutive lanes; XOR-ing in (r >> 4) spreads those over all 8 chunk positions as well
-// while only adding a constant to any run of 16 consecutive rows.
-// Direct staging writes cover whole 128 B rows with consecutive lanes and are conflict free
-// under any XOR of the chunk index.
-__device__ __forceinline__ int swizzle_of(int row) { return ((row >> 1) ^ (row >> 4)) & 7; }
-
-// Byte offset inside a slab of the fragment chunk `logical_chunk` for the lane whose block-local
-// row is lr, in the 32-row block that starts at row `block_row` of the slab: the lane part; the
-// caller XORs (block index within the wavefront) << 5, which is the compile-time part of
-// swizzle_of(block_row + 32 i + lr).
-__device__ __forceinline__ int frag_chunk_off(int logical_chunk, int block_row, int lr) {
-  return (logical_chunk ^ swizzle_of(block_row + lr)) << 4;
-}
-
 // ---------------------------------------------------------------------------------------------
+// LDS layouts and their swizzles.
+//
+// direct slab : row x (128 B = 8 chunks of 16 B); chunk c lives at position c ^ ((x >> 1) & 7).
+//   ds_read_b128 is served 16 lanes (256 B, all 64 banks) per cycle; a fragment read touches 16
+//   consecutive rows at one logical chunk, i.e. 8 even and 8 odd rows (two rows span the banks),
+//   so rows of equal parity must land on 8 different chunk positions.
+// kmajor slab : row k (512 B = 32 chunks of 16 B); chunk c lives at position c ^ (4 (k & 3)).
+//   A transposing read touches, per 32 lanes, 4 consecutive k rows x 64 B at one x block; rows
+//   are 512 B apart (the same banks), so the XOR moves the 4 rows to 4 different 64 B groups.
+__device__ __forceinline__ int swizzle_direct(int row) { return (row >> 1) & 7; }
+
 // Where one slab of an operand comes from: a buffer resource whose base is the operand's tile
 // origin, plus the scalar byte offset of the slab's first k.  Reads past the end of the operand
 // return zero (buffer bounds check), which is what rows / k beyond the valid extent must
 // contribute, so the loaders carry no clamping arithmetic.
 struct SlabSrc {
-  __amdgpu_buffer_rsrc_t rsrc;
+  u32x4 rsrc;  // buffer resource words: base, base high | stride 0, byte count, raw 32-bit format
   unsigned soff;
 };
 
 template <bool KMAJOR>
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t tile_rsrc(const Operand& op, int x0) {
+__device__ __forceinline__ u32x4 tile_rsrc(const Operand& op, int x0) {
   // direct: rows x0.. of [x_extent][ld];  kmajor: columns x0.. of [k_extent][ld]
   const int64_t first = KMAJOR ? (int64_t)x0 : (int64_t)x0 * op.ld;
   const int64_t total = (KMAJOR ? (int64_t)op.k_extent : (int64_t)op.x_extent) * op.ld;
   int64_t bytes = (total - first) * 2;
   if (bytes < 0) bytes = 0;
   if (bytes > 0xffffffffll) bytes = 0xffffffffll;
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(op.base + first), 0, (int)(unsigned)bytes, 0x00020000);
+  const uint64_t base = reinterpret_cast<uint64_t>(op.base + first);
+  return u32x4{(unsigned)base, (unsigned)(base >> 32) & 0xffffu, (unsigned)bytes, 0x00020000u};
 }
 
 template <bool KMAJOR>
@@ -144,176 +137,165 @@ __device__ __forceinline__ unsigned slab_soff(const Operand& op, int k0) {
   return KMAJOR ? (unsigned)k0 * ((unsigned)op.ld * 2u) : (unsigned)k0 * 2u;
 }
 
-// Global -> register -> LDS staging for one 256 x 64 slab of an operand: 4 x 16 bytes per lane.
-//
-// direct : load i is row (t/8 + 64 i), 16-byte chunk t%8 of the slab; 8 lanes fetch one 128 B row
-//          and store i writes load i as one 16-byte chunk.
-// kmajor : thread (xg, kq) owns the 8(x) x 4(k) block at x = 8 xg, k = 4 kq, with xg = lane%8 +
-//          8 (wave%4) and kq = lane/8 + 8 (wave/4): load i is the 8 x-values of k = 4 kq + i, so 8
-//          consecutive lanes fetch one whole 128 B line of a memory row; the block is transposed
-//          in registers and store j writes the 4 k-values of x = 8 xg + j as one 8-byte half
-//          chunk, so no transposed copy of an operand ever exists in memory.
-// Either way the per-lane address is ONE 32-bit offset; everything that changes between loads,
-// slabs and tiles is scalar (buffer resource + scalar offset).
+// LDS byte address of a pointer into the workgroup's LDS allocation.
+__device__ __forceinline__ unsigned lds_address(const char* p) {
+  return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
+// buffer_load_dwordx4 ... lds: lane L's 16 bytes from (resource, voff + soff) land at LDS address
+// lds_base + 16 L (lds_base is wave-uniform and travels in M0).  Written as inline assembly so
+// that the compiler's wait-count bookkeeping does not see an outstanding LDS write and fence
+// every later LDS read against it; the engine waits for its transfers itself, once per slab.
+__device__ __forceinline__ void load_to_lds_16(const u32x4& rsrc, unsigned voff, unsigned soff, unsigned lds_base) {
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+               :
+               : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_base)
+               : "memory", "m0");
+}
+
+// Memory -> LDS transfer of one operand slab: 4 loads of 16 bytes per lane.  Load i of wavefront
+// w fills the 1 KB LDS block (w + 8 i) of the slab:
+//   direct : block b = rows 8 b .. 8 b + 7; lane L sits at row 8 b + L / 8, chunk position L % 8,
+//            and fetches logical chunk (L % 8) ^ swizzle of that row -- 8 lanes cover one whole
+//            128 B line of the memory row;
+//   kmajor : block b = k rows 2 b, 2 b + 1; lane L sits at k row 2 b + L / 32, chunk position
+//            L % 32, and fetches logical chunk (L % 32) ^ 4 (k & 3) -- 32 lanes cover 512
+//            contiguous bytes of the memory row.
+// Both swizzles are unchanged by the + 64 rows (direct) / + 16 k rows (kmajor) between loads, so
+// the per-lane address is ONE 32-bit offset; everything that changes between loads, slabs and
+// tiles is scalar (buffer resource, scalar offset, LDS base in M0).
 template <bool KMAJOR>
-struct SlabLoader {
-  static constexpr int kStores = KMAJOR ? 8 : kLoads;
-  u32x4 reg[kLoads];
-  unsigned voff;     // per-lane byte offset of load 0 inside the tile
-  unsigned step;     // scalar byte offset between consecutive loads
-  unsigned lds_off;  // per-lane byte offset of store 0 inside a slab
-  unsigned lds_xor;  // kmajor: chunk position before the (j >> 1) XOR
+struct SlabDma {
+  unsigned voff;      // per-lane byte offset of load 0 inside the tile
+  unsigned step;      // scalar byte offset between consecutive loads
+  unsigned lds_wave;  // byte offset of this wavefront's first block inside the slab
 
   __device__ __forceinline__ void init(const Operand& op) {
-    const unsigned t = threadIdx.x;
+    const unsigned lane = threadIdx.x & 63u, w = threadIdx.x >> 6;
     const unsigned ld_bytes = (unsigned)op.ld * 2u;
     if constexpr (!KMAJOR) {
-      const unsigned kc = t & 7, row = t >> 3;  // rows 0..63, + 64 per load
-      voff = row * ld_bytes + kc * 16u;
+      const unsigned row = 8u * w + (lane >> 3);
+      voff = row * ld_bytes + (((lane & 7u) ^ (unsigned)swizzle_direct((int)row)) << 4);
       step = 64u * ld_bytes;
-      // swizzle_of(row + 64 i) == swizzle_of(row) ^ 4 (i & 1): store i flips bit 6 of the offset
-      lds_off = row * 128u + ((kc ^ (unsigned)swizzle_of((int)row)) << 4);
-      lds_xor = 0;
     } else {
-      const unsigned lane = t & 63u, w = t >> 6;
-      const unsigned xg = (lane & 7u) + 8u * (w & 3u), kq = (lane >> 3) + 8u * (w >> 2);
-      voff = kq * 4u * ld_bytes + xg * 16u;
-      step = ld_bytes;
-      lds_off = xg * 1024u + (kq & 1u) * 8u;
-      // swizzle_of(8 xg + j) = (((xg & 1) << 2) | (j >> 1)) ^ ((xg >> 1) & 7)
-      lds_xor = (kq >> 1) ^ ((xg & 1u) << 2) ^ ((xg >> 1) & 7u);
+      const unsigned k = 2u * w + (lane >> 5);
+      voff = k * ld_bytes + (((lane & 31u) ^ (4u * (k & 3u))) << 4);
+      step = 16u * ld_bytes;
     }
+    lds_wave = __builtin_amdgcn_readfirstlane(w * 1024u);
   }
 
-  __device__ __forceinline__ void issue_one(int i, const SlabSrc& src) {
-    reg[i] = __builtin_amdgcn_raw_buffer_load_b128(src.rsrc, (int)voff, (int)(src.soff + (unsigned)i * step), 0);
-  }
-
-  __device__ __forceinline__ void store_one(int j, char* slab) const {
-    if constexpr (!KMAJOR) {
-      *reinterpret_cast<u32x4*>(slab + (lds_off ^ ((unsigned)(j & 1) << 6)) + j * 8192) = reg[j];
-    } else {
-      // x = 8 xg + j : bf16 #j of each of the 4 loads (k = 4 kq .. 4 kq + 3)
-      u32x2 o;
-#pragma unroll
-      for (int p = 0; p < 2; ++p) {
-        const unsigned lo = reg[2 * p][j >> 1];
-        const unsigned hi = reg[2 * p + 1][j >> 1];
-        o[p] = (j & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
-      }
-      *reinterpret_cast<u32x2*>(slab + lds_off + j * 128 + ((lds_xor ^ (unsigned)(j >> 1)) << 4)) = o;
-    }
+  // slab_lds: LDS byte address of the operand's slab in the stage being filled
+  __device__ __forceinline__ void issue_one(int i, const SlabSrc& src, unsigned slab_lds) const {
+    load_to_lds_16(src.rsrc, voff, src.soff + (unsigned)i * step, slab_lds + lds_wave + (unsigned)i * 8192u);
   }
 };
 
 // ---------------------------------------------------------------------------------------------
-// MFMA fragments of one 16-k step: kMB blocks of C and kNB blocks of R, 6 ds_read_b128 per lane.
+// Per-lane LDS addressing of MFMA fragments.  A fragment is the 8 consecutive k (k = 16 s + 8 lh
+// + 0..7 of k-step s) of slab row x = 32 * block + lr.
+//   direct : one ds_read_b128 at  x * 128 + (((2 s + lh) ^ swizzle(x)) << 4);
+//   kmajor : two transposing 8-byte reads.  Within 16 lanes, lane i addresses the 8 bytes at
+//            (k row k0 + i / 4, x0 + 4 (i % 4)) and receives the 4 k of x0 + i; lanes 0-15 /
+//            16-31 take x0 = 0 / 16 of the block, lanes 32-63 the k-half lh = 1.
+template <bool KMAJOR>
+struct FragAddr {
+  // direct: off[s] = lane part for k-step s, block adds 4096 b.  kmajor: off[b] = lane part for
+  // block b of the wavefront, k-step adds 8192 s (+ 2048 for the second read).
+  int off[4];
+
+  // first_block: index of the wavefront's first 32-row block inside the slab
+  __device__ __forceinline__ void init(int first_block, int nblocks) {
+    const int l = threadIdx.x & 63;
+    if constexpr (!KMAJOR) {
+      const int lr = l & 31, lh = l >> 5;
+#pragma unroll
+      for (int s = 0; s < 4; ++s) off[s] = (first_block * 32 + lr) * 128 + (((2 * s + lh) ^ swizzle_direct(lr)) << 4);
+    } else {
+      const int g = l >> 4, i = l & 15;
+      const int q = i >> 2;                       // (k & 3) of the addressed row: every k offset is a multiple of 4
+      const int k0 = 8 * (g >> 1) + q;
+      const int x_in_blk = 16 * (g & 1) + 4 * (i & 3);
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+        off[b] = b < nblocks ? k0 * 512 + 64 * ((first_block + b) ^ q) + 2 * x_in_blk : 0;
+    }
+  }
+
+  __device__ __forceinline__ bf16x8 read(const char* slab, int s, int b) const {
+    if constexpr (!KMAJOR) {
+      return *reinterpret_cast<const bf16x8*>(slab + off[s] + b * 4096);
+    } else {
+      typedef bf16x4 __attribute__((address_space(3))) * tr_ptr_t;
+      const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((tr_ptr_t)(slab + off[b] + s * 8192));
+      const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((tr_ptr_t)(slab + off[b] + s * 8192 + 2048));
+      return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  }
+};
+
+// MFMA fragments of one 16-k step: kMB blocks of C and kNB blocks of R.
 struct Frags {
   bf16x8 c[kMB], r[kNB];
 };
 
-// Workgroup barrier that only waits for this wavefront's LDS traffic: global loads issued for
-// later slabs stay in flight across it (a __syncthreads() would drain them too).
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
-
 // ---------------------------------------------------------------------------------------------
 // One slab (64 k = four 16-k steps of 8 MFMAs per wavefront) of the software pipeline.
 //
-// The body is written as 32 slots "one MFMA + a few short memory instructions", each closed by
-// a scheduling barrier so the compiler keeps the order; memory instructions are spread evenly so
-// the vector-memory and LDS pipes see a steady duty instead of bursts:
+// The body is written as 32 slots "one MFMA + at most one memory instruction group", each closed
+// by a scheduling barrier so the compiler keeps the order:
 //
-//   step 0 : fragment reads of step 1 | R staging -> LDS(nxt)  | loads C[2..3] of slab it+1
-//   step 1 : fragment reads of step 2 |                        | loads R[0..1] of slab it+2
-//   step 2 : fragment reads of step 3 | C staging -> LDS(nxt)  | loads R[2..3] of slab it+2
-//   -- LDS-only barrier --
-//   step 3 : step-0 fragment reads of slab it+1 from nxt       | loads C[0..1] of slab it+2
+//   step 0..2 : MFMAs of step s | fragment reads of step s + 1 from `cur`
+//   -- wait for this wavefront's transfers of slab it+1, workgroup barrier --
+//   step 3    : MFMAs of step 3 | step-0 fragment reads of slab it+1 from `nxt`
+//                               | transfers of slab it+2 into `cur` (every wavefront has its last
+//                                 fragments of `cur` in registers once the barrier is passed)
 //
-// Every staging register has at least two steps between its load and its LDS write, and
-// neither the barrier nor the first fragment reads of a slab sit at the head of the stream.
+// so a transfer has three steps of MFMA work to land before anyone waits for it, and nothing
+// inside the steps depends on memory.
 template <bool RK, bool CK>
-__device__ __forceinline__ void slab_iter(SlabLoader<RK>& lr, SlabLoader<CK>& lc, const SlabSrc& c1,
-                                          const SlabSrc& r2, const SlabSrc& c2, const char* cur, char* nxt,
-                                          const LanePos& p, Frags& f0, Accum& acc) {
-  const int row_r = p.wr * (kNB * 32), row_c = p.wc * (kMB * 32);
-  const int lane_r = (row_r + p.lr) * 128;
-  const int lane_c = kSlabBytes + (row_c + p.lr) * 128;
+__device__ __forceinline__ void slab_iter(const SlabDma<RK>& dr, const SlabDma<CK>& dc, const SlabSrc& r2,
+                                          const SlabSrc& c2, char* cur, const char* nxt, const FragAddr<RK>& fr,
+                                          const FragAddr<CK>& fc, Frags& f0, Accum& acc) {
   Frags f1;
 #define VAMD_MFMA(F, i)                                                                                            \
   acc.a[(i) >> 1][(i) & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F.c[(i) >> 1], F.r[(i) & 1],                    \
                                                                      acc.a[(i) >> 1][(i) & 1], 0, 0, 0)
-#define VAMD_FRAG(G, base, i, lc)                                                                              \
-  do {                                                                                                         \
-    if ((i) < kMB)                                                                                             \
-      G.c[(i)] = *reinterpret_cast<const bf16x8*>((base) + lane_c + (i) * 4096 +                                \
-                                                  (frag_chunk_off((lc) + p.lh, row_c, p.lr) ^ ((i) << 5)));     \
-    else if ((i) < kMB + kNB)                                                                                  \
-      G.r[(i) - kMB] = *reinterpret_cast<const bf16x8*>((base) + lane_r + ((i) - kMB) * 4096 +                  \
-                                                        (frag_chunk_off((lc) + p.lh, row_r, p.lr) ^            \
-                                                         (((i) - kMB) << 5)));                                 \
+#define VAMD_FRAG(G, base, i, s)                                            \
+  do {                                                                      \
+    if ((i) < kMB) G.c[(i)] = fc.read((base) + kSlabBytes, (s), (i));        \
+    else if ((i) < kMB + kNB) G.r[(i) - kMB] = fr.read((base), (s), (i) - kMB); \
   } while (0)
 #define VAMD_SLOT_END __builtin_amdgcn_sched_barrier(0)
-  constexpr int kRS = SlabLoader<RK>::kStores, kCS = SlabLoader<CK>::kStores;
-
-  // ---- step 0 : MFMA(f0); f1 <- step 1 fragments; R staging -> nxt; C[2..3] of slab it+1
-  {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      VAMD_MFMA(f0, i);
-      VAMD_FRAG(f1, cur, i, 2);
-#ifndef VAMD_DBG_NO_STORE
-      if (kRS == 8 || i < 4) lr.store_one(i, nxt);
-#endif
-#ifndef VAMD_DBG_NO_GLOBAL
-      if (i == 5) lc.issue_one(2, c1);
-      if (i == 7) lc.issue_one(3, c1);
-#endif
-      VAMD_SLOT_END;
-    }
+  for (int i = 0; i < 8; ++i) {
+    VAMD_MFMA(f0, i);
+    VAMD_FRAG(f1, cur, i, 1);
+    VAMD_SLOT_END;
   }
-  // ---- step 1 : MFMA(f1); f0 <- step 2 fragments; R[0..1] of slab it+2
-  {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      VAMD_MFMA(f1, i);
-      VAMD_FRAG(f0, cur, i, 4);
-#ifndef VAMD_DBG_NO_GLOBAL
-      if (i == 1) lr.issue_one(0, r2);
-      if (i == 5) lr.issue_one(1, r2);
-#endif
-      VAMD_SLOT_END;
-    }
+  for (int i = 0; i < 8; ++i) {
+    VAMD_MFMA(f1, i);
+    VAMD_FRAG(f0, cur, i, 2);
+    VAMD_SLOT_END;
   }
-  // ---- step 2 : MFMA(f0); f1 <- step 3 fragments; C staging -> nxt; R[2..3] of slab it+2
-  {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      VAMD_MFMA(f0, i);
-      VAMD_FRAG(f1, cur, i, 6);
-#ifndef VAMD_DBG_NO_STORE
-      if (kCS == 8 || i < 4) lc.store_one(i, nxt + kSlabBytes);
-#endif
-#ifndef VAMD_DBG_NO_GLOBAL
-      if (i == 5) lr.issue_one(2, r2);
-      if (i == 7) lr.issue_one(3, r2);
-#endif
-      VAMD_SLOT_END;
-    }
+  for (int i = 0; i < 8; ++i) {
+    VAMD_MFMA(f0, i);
+    VAMD_FRAG(f1, cur, i, 3);
+    VAMD_SLOT_END;
   }
-  lds_barrier();
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   VAMD_SLOT_END;
-  // ---- step 3 : MFMA(f1); f0 <- step 0 fragments of the next slab; C[0..1] of slab it+2
-  {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      VAMD_MFMA(f1, i);
-      VAMD_FRAG(f0, nxt, i, 0);
+  for (int i = 0; i < 8; ++i) {
+    VAMD_MFMA(f1, i);
+    VAMD_FRAG(f0, nxt, i, 0);
 #ifndef VAMD_DBG_NO_GLOBAL
-      if (i == 1) lc.issue_one(0, c2);
-      if (i == 5) lc.issue_one(1, c2);
+    if (i < 4) dr.issue_one(i, r2, lds_address(cur));
+    else dc.issue_one(i - 4, c2, lds_address(cur) + kSlabBytes);
 #endif
-      VAMD_SLOT_END;
-    }
+    VAMD_SLOT_END;
   }
 #undef VAMD_MFMA
 #undef VAMD_FRAG
@@ -324,28 +306,35 @@ __device__ __forceinline__ void slab_iter(SlabLoader<RK>& lr, SlabLoader<CK>& lc
 // Persistent, software-pipelined walk over a list of output tiles.
 //
 //   Sched : int count();  void tile(int i, int& r0, int& c0);
-//   Epi   : void operator()(Accum& acc, int r0, int c0);   (registers + global memory only)
+//   Epi   : void operator()(Accum& acc, int r0, int c0);   (registers + global memory only, or LDS
+//           beyond the first kLdsBytes)
 //
-// All (tile, slab) pairs of the workgroup form one stream of slabs; slab it+1 is staged into
-// LDS and slab it+2 is fetched from memory while slab it is multiplied, across tile boundaries
-// too, so only the very first slab pays a cold start and epilogues find their next slab ready.
-// Past the end of the stream the fetch cursor stays on the last slab (two redundant fetches)
-// instead of branching, which keeps the loop body a single basic block.
+// All (tile, slab) pairs of the workgroup form one stream of slabs; slab it+1 is landing in LDS
+// and slab it+2 is requested while slab it is multiplied, across tile boundaries too, so only the
+// very first slab pays a cold start and epilogues find their next slab ready.  Past the end of
+// the stream the fetch cursor stays on the last slab (two redundant transfers) instead of
+// branching, which keeps the loop body a single basic block.  On return every transfer of the
+// calling wavefront has landed; the caller must pass a workgroup barrier before it reuses the
+// first kLdsBytes of LDS.
 template <bool R_KMAJOR, bool C_KMAJOR, class Sched, class Epi>
 __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, int k_slabs, Sched& sched, Epi& epi,
                                           char* lds) {
   const int ntiles = sched.count();
   if (ntiles <= 0) return;
   const LanePos pos = lane_pos();
-  SlabLoader<R_KMAJOR> lr;
-  SlabLoader<C_KMAJOR> lc;
-  lr.init(R);
-  lc.init(C);
+  SlabDma<R_KMAJOR> dr;
+  SlabDma<C_KMAJOR> dc;
+  dr.init(R);
+  dc.init(C);
+  FragAddr<R_KMAJOR> fr;
+  FragAddr<C_KMAJOR> fc;
+  fr.init(pos.wr * kNB, kNB);
+  fc.init(pos.wc * kMB, kMB);
 
   // fetch cursor: (t2, k2) names the slab whose sources are (src_r, src_c)
   int t2 = 0, k2 = 0, r0, c0;
   sched.tile(0, r0, c0);
-  __amdgpu_buffer_rsrc_t rs_r = tile_rsrc<R_KMAJOR>(R, r0), rs_c = tile_rsrc<C_KMAJOR>(C, c0);
+  u32x4 rs_r = tile_rsrc<R_KMAJOR>(R, r0), rs_c = tile_rsrc<C_KMAJOR>(C, c0);
   SlabSrc src_r{rs_r, 0u}, src_c{rs_c, 0u};
   auto advance = [&]() {
     if (t2 == ntiles - 1 && k2 == k_slabs - 1) return;
@@ -359,44 +348,32 @@ __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, in
     }
 #ifdef VAMD_DBG_SAME_SLAB
     src_r = SlabSrc{rs_r, 0u};
-    src_c = SlabSrc{rs_c, (unsigned)(k2 & 1) * 128u};
+    src_c = SlabSrc{rs_c, 0u};
 #else
     src_r = SlabSrc{rs_r, slab_soff<R_KMAJOR>(R, k2 * kBK)};
     src_c = SlabSrc{rs_c, slab_soff<C_KMAJOR>(C, k2 * kBK)};
 #endif
   };
 
-  // slab 0 -> LDS stage 0
+  // slab 0 -> stage 0, slab 1 -> stage 1
 #pragma unroll
   for (int i = 0; i < kLoads; ++i) {
-    lr.issue_one(i, src_r);
-    lc.issue_one(i, src_c);
+    dr.issue_one(i, src_r, lds_address(lds));
+    dc.issue_one(i, src_c, lds_address(lds) + kSlabBytes);
   }
-#pragma unroll
-  for (int j = 0; j < SlabLoader<R_KMAJOR>::kStores; ++j) lr.store_one(j, lds);
-#pragma unroll
-  for (int j = 0; j < SlabLoader<C_KMAJOR>::kStores; ++j) lc.store_one(j, lds + kSlabBytes);
-  // slab 1 -> staging registers, except C[2..3] which the first iteration fetches itself
   advance();
 #pragma unroll
-  for (int i = 0; i < kLoads; ++i) lr.issue_one(i, src_r);
-#pragma unroll
-  for (int i = 0; i < kLoads / 2; ++i) lc.issue_one(i, src_c);
-  SlabSrc c1 = src_c;
-  advance();  // cursor now on slab 2
-  lds_barrier();
-  Frags f0;
-  {
-    const int row_r = pos.wr * (kNB * 32), row_c = pos.wc * (kMB * 32);
-#pragma unroll
-    for (int i = 0; i < kMB; ++i)
-      f0.c[i] = *reinterpret_cast<const bf16x8*>(lds + kSlabBytes + (row_c + pos.lr) * 128 + i * 4096 +
-                                                 (frag_chunk_off(pos.lh, row_c, pos.lr) ^ (i << 5)));
-#pragma unroll
-    for (int i = 0; i < kNB; ++i)
-      f0.r[i] = *reinterpret_cast<const bf16x8*>(lds + (row_r + pos.lr) * 128 + i * 4096 +
-                                                 (frag_chunk_off(pos.lh, row_r, pos.lr) ^ (i << 5)));
+  for (int i = 0; i < kLoads; ++i) {
+    dr.issue_one(i, src_r, lds_address(lds) + 2 * kSlabBytes);
+    dc.issue_one(i, src_c, lds_address(lds) + 3 * kSlabBytes);
   }
+  advance();  // cursor now on slab 2
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  Frags f0;
+#pragma unroll
+  for (int i = 0; i < kMB; ++i) f0.c[i] = fc.read(lds + kSlabBytes, 0, i);
+#pragma unroll
+  for (int i = 0; i < kNB; ++i) f0.r[i] = fr.read(lds, 0, i);
 
   int stage = 0;
   for (int tile = 0; tile < ntiles; ++tile) {
@@ -404,15 +381,15 @@ __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, in
     accum_zero(acc);
     sched.tile(tile, r0, c0);
     for (int kt = 0; kt < k_slabs; ++kt) {
-      const char* cur = lds + stage * 2 * kSlabBytes;
-      char* nxt = lds + (stage ^ 1) * 2 * kSlabBytes;
-      slab_iter<R_KMAJOR, C_KMAJOR>(lr, lc, c1, src_r, src_c, cur, nxt, pos, f0, acc);
-      c1 = src_c;
+      char* cur = lds + stage * 2 * kSlabBytes;
+      const char* nxt = lds + (stage ^ 1) * 2 * kSlabBytes;
+      slab_iter<R_KMAJOR, C_KMAJOR>(dr, dc, src_r, src_c, cur, nxt, fr, fc, f0, acc);
       advance();
       stage ^= 1;
     }
     epi(acc, r0, c0);
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
 // ---------------------------------------------------------------------------------------------

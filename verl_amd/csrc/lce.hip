@@ -239,7 +239,9 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
     merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], m2, s2, sy2);
     epi.zl[nb] += z2;
   }
-  // ... then the two wavefronts that share a token quarter (wc = 0/1), through LDS.
+  // ... then the two wavefronts that share a token quarter (wc = 0/1), through LDS (once every
+  // wavefront's last slab transfers have landed).
+  __syncthreads();
   float4* red = reinterpret_cast<float4*>(lds);  // [2][256]
   if (epi.p.lh == 0) {
 #pragma unroll
