@@ -26,6 +26,11 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 KERNEL_NAMES = ["lce_forward_kernel", "lce_merge_kernel", "lce_recompute_kernel", "lce_dgrad_kernel"]
 # MFMA GEMMs of 2*N*V*H flops each that a kernel performs per step
 COPY_YARDSTICK_BYTES = 1 << 30
+# L2 <-> fabric bytes of one full-chunk launch (16384 vocabulary columns) of each kernel at this workload:
+# rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by the readings of the 1 GiB copy in the same run
+# (2048 and 1024 bytes per unit); see profiles/head_fwd_bwd_qwen7b_hbm_traffic.md.  Counters cannot be read
+# from inside this process, so the figure is recorded here and only reported for the shape it was measured on.
+MEASURED_TRAFFIC_BYTES = {"lce_dgrad_kernel": 6.42e9 + 0.357e9, "lce_forward_kernel": 31.48e9 + 9.972e9}
 GEMMS_PER_STEP = {"lce_forward_kernel": 1, "lce_recompute_kernel": 1, "lce_dgrad_kernel": 2}
 
 
@@ -70,7 +75,7 @@ def main() -> None:
     import torch
 
     from verl_amd import _cabi
-    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy, logits_cache_budget_bytes
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
@@ -122,6 +127,7 @@ def main() -> None:
             kernels[name] = {"ms_per_step": ms[i] / prof_steps, "launches_per_step": cnt[i] / prof_steps,
                              "avg_ms": ms[i] / cnt[i]}
     gemm_flops = 2.0 * n * v * h
+    cached = 4 * n * v <= logits_cache_budget_bytes()   # backward forms d_logits from cached logits: no recompute GEMM
     dom = max((k for k in kernels if k in GEMMS_PER_STEP), key=lambda k: kernels[k]["ms_per_step"])
     d = kernels[dom]
     flops_per_launch = GEMMS_PER_STEP[dom] * gemm_flops / d["launches_per_step"]
@@ -133,11 +139,11 @@ def main() -> None:
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_BF16_TFLOPS,
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(dom) if cached else None,
         "flops_per_launch": flops_per_launch,
         "avg_launch_ms": d["avg_ms"],
         "step_algorithmic_frac": 6.0 * n * v * h / (ms_per_step * 1e-3) / (PEAK_BF16_TFLOPS * 1e12),
-        "step_hardware_frac": 8.0 * n * v * h / (ms_per_step * 1e-3) / (PEAK_BF16_TFLOPS * 1e12),
+        "step_hardware_frac": (6.0 if cached else 8.0) * n * v * h / (ms_per_step * 1e-3) / (PEAK_BF16_TFLOPS * 1e12),
         "kernels": kernels,
     }
 
@@ -159,7 +165,8 @@ def main() -> None:
         "config": {"workload": "fused log-prob+entropy head forward+backward, Qwen2.5-7B head shape "
                                "(BASELINE configs[1])",
                    "n_tokens": n, "hidden_size": h, "vocab": v, "temperature": T,
-                   "upstream": "dlogprob ~ N(0,1) fp32, dentropy = 0.001"},
+                   "upstream": "dlogprob ~ N(0,1) fp32, dentropy = 0.001",
+                   "fp32_logits_cache_bytes": 4 * n * v if 4 * n * v <= logits_cache_budget_bytes() else 0},
         "mfma_util_pct": 100.0 * roofline["step_hardware_frac"],
         "roofline": roofline,
         "cpu_baseline": base,
