@@ -45,6 +45,12 @@ extern "C" {
 #define VAMD_AGG_SEQ_MEAN_TOKEN_MEAN 2
 #define VAMD_AGG_SEQ_MEAN_TOKEN_SUM_NORM 3
 
+/* estimator of kl_penalty_forward (verl/trainer/ppo/core_algos.py:1868-1902) */
+#define VAMD_KL_K1 0  /* "kl", "k1": logprob - ref */
+#define VAMD_KL_ABS 1 /* "abs" */
+#define VAMD_KL_K2 2  /* "mse", "k2": 0.5 (logprob - ref)^2 */
+#define VAMD_KL_K3 3  /* "low_var_kl", "k3": exp(k) - k - 1, k = clamp(ref - logprob, -20, 20), clamped to [-10, 10] */
+
 int vamd_abi_version(void);
 const char* vamd_last_error(void);
 
@@ -193,6 +199,24 @@ int vamd_value_loss_forward(const float* vpreds, const float* returns, const flo
                             int mask_dtype, int64_t rows, int64_t cols, float cliprange_value, int mode,
                             float* out, float* grad_unscaled, float* coef_out, void* workspace,
                             size_t workspace_bytes, void* stream);
+
+/* kl_penalty / kl_penalty_forward (core_algos.py:1841-1902), elementwise over n values:
+ * kld[i] (optional) and grad[i] = d kld / d logprob (optional; d kld / d ref_logprob is its
+ * negative).  straight_through != 0 keeps the estimator's value and replaces its gradient by
+ * that of k2, (logprob - ref): the reference's "+" variants (core_algos.py:1854-1864). */
+int vamd_kl_penalty(const float* logprob, const float* ref_logprob, int64_t n, int kind, int straight_through,
+                    float* kld, float* grad, void* stream);
+
+/* agg_loss(kl_penalty(logprob, ref_logprob), mask, mode) in one pass: the kl_loss of the actor
+ * update (verl/workers/actor/dp_actor.py:640-646).  out[0] = kl_loss; grad_unscaled (optional) =
+ * d kld / d logprob * mask, to be scaled by coef_out[row] and the upstream gradient with
+ * vamd_scale_rows.  The last four scalars are agg_loss's (negative = None). */
+size_t vamd_kl_loss_workspace_bytes(int64_t rows, int64_t cols);
+int vamd_kl_loss_forward(const float* logprob, const float* ref_logprob, const void* mask, int mask_dtype,
+                         int64_t rows, int64_t cols, int kind, int straight_through, int mode, double dp_size,
+                         double batch_num_tokens, double global_batch_size, double loss_scale_factor, float* out,
+                         float* grad_unscaled, float* coef_out, void* workspace, size_t workspace_bytes,
+                         void* stream);
 
 #ifdef __cplusplus
 }

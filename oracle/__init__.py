@@ -46,4 +46,6 @@ from .losses import (  # noqa: F401
     policy_loss_vanilla,
     value_loss,
     kl_penalty_forward,
+    kl_penalty,
+    kl_straight_through,
 )

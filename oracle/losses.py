@@ -95,3 +95,19 @@ def kl_penalty_forward(logprob, ref_logprob, kind):
         d = torch.clamp(ref_logprob - logprob, min=-20, max=20)
         return torch.clamp(torch.exp(d) - d - 1, min=-10, max=10)
     raise NotImplementedError(kind)
+
+
+def kl_penalty(logprob, ref_logprob, kind):
+    """verl/trainer/ppo/core_algos.py:1841-1866, as written: the forward score is evaluated with
+    the name as given, so a "+"-suffixed name already fails in ``kl_penalty_forward``; the
+    straight-through combination below is what the remaining lines do for a forward score."""
+    forward_score = kl_penalty_forward(logprob, ref_logprob, kind)
+    if not kind.endswith("+") or kind in ("mse", "k2"):
+        return forward_score
+    return kl_straight_through(logprob, ref_logprob, forward_score)
+
+
+def kl_straight_through(logprob, ref_logprob, forward_score):
+    """core_algos.py:1861-1866: value of ``forward_score``, gradient of k2."""
+    backward_score = 0.5 * (logprob - ref_logprob).square()
+    return backward_score - backward_score.detach() + forward_score.detach()

@@ -349,6 +349,71 @@ def test_value_loss_forward_backward(dev, mode, shape):
            what="d vf_loss / d vpreds")
 
 
+# ---- KL penalty -------------------------------------------------------------------------------------
+@pytest.mark.parametrize("kind", ["kl", "k1", "abs", "mse", "k2", "low_var_kl", "k3"])
+def test_kl_penalty_elementwise(dev, kind):
+    from verl_amd.trainer.ppo.core_algos import kl_penalty, kl_penalty_forward
+    g = torch.Generator().manual_seed(17)
+    lp = torch.randn(37, 301, generator=g) - 1
+    ref = lp + torch.randn(37, 301, generator=g) * 0.7
+    ref[0, 0] = lp[0, 0]                     # d = 0: |d| has gradient 0 there
+    ref[0, 1] = lp[0, 1] + 25.0              # ref - lp beyond the clamp at 20: value 10 (second clamp), no gradient
+    ref[0, 2] = lp[0, 2] - 25.0              # below -20
+    ref[0, 3] = lp[0, 3] + 3.0               # exp(3) - 3 - 1 = 16.1 > 10: clamped value, no gradient
+    ld = lp.to(dev).requires_grad_(); lo = lp.clone().requires_grad_()
+    got = kl_penalty(ld, ref.to(dev), kind)
+    want = O.kl_penalty(lo, ref, kind)
+    assert got.shape == lp.shape and got.device.type == "cuda"
+    _close(got, want, what="kld " + kind)
+    up = torch.randn(37, 301, generator=g)
+    _close(torch.autograd.grad(got, ld, up.to(dev))[0], torch.autograd.grad(want, lo, up)[0], atol=1e-6,
+           what="d kld / d logprob " + kind)
+    # gradient with respect to the reference log-prob is the negative
+    rd = ref.to(dev).requires_grad_(); ro = ref.clone().requires_grad_()
+    _close(torch.autograd.grad(kl_penalty_forward(lp.to(dev), rd, kind).sum(), rd)[0],
+           torch.autograd.grad(O.kl_penalty_forward(lp, ro, kind).sum(), ro)[0], atol=1e-6, what="d kld / d ref")
+
+
+def test_kl_penalty_names_that_raise(dev):
+    from verl_amd.trainer.ppo.core_algos import compute_kl_loss, kl_penalty
+    x = torch.zeros(2, 3, device=dev)
+    for name in ("k1+", "k3+", "low_var_kl+", "abs+", "mse+", "full", "nonsense"):
+        with pytest.raises(NotImplementedError):
+            kl_penalty(x, x, name)
+        with pytest.raises(NotImplementedError):
+            O.kl_penalty(x.cpu(), x.cpu(), name)
+    with pytest.raises(ValueError):
+        compute_kl_loss(x, x, torch.ones(2, 3, device=dev), "k3", "no-such-mode")
+    assert kl_penalty(x.cpu(), x.cpu() + 1, "k1").device.type == "cpu"    # CPU inputs are staged to the GPU and back
+
+
+@pytest.mark.parametrize("mode", ["token-mean", "seq-mean-token-sum", "seq-mean-token-mean", "seq-mean-token-sum-norm"])
+@pytest.mark.parametrize("kind", ["k1", "abs", "k2", "low_var_kl"])
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.bool])
+def test_kl_loss_fused(dev, mode, kind, mdtype):
+    """compute_kl_loss == agg_loss(kl_penalty(...)) of the oracle, value and gradient, every mode and estimator;
+    straight-through keeps the value and takes the k2 gradient."""
+    from verl_amd.trainer.ppo.core_algos import compute_kl_loss
+    g = torch.Generator().manual_seed(len(mode) + len(kind))
+    B, Lc = 24, 5000                                             # two column chunks, ragged tail
+    mask, _ = _prefix_mask(B, Lc, g)
+    mask[3] = 0                                                  # an empty row
+    lp = torch.randn(B, Lc, generator=g) * 0.5 - 1
+    ref = lp + torch.randn(B, Lc, generator=g) * 0.3
+    ref[1, 0] = lp[1, 0] + 30.0
+    ld = lp.to(dev).requires_grad_(); lo = lp.clone().requires_grad_()
+    got = compute_kl_loss(ld, ref.to(dev), mask.to(dev).to(mdtype), kind, mode)
+    want = O.agg_loss(O.kl_penalty(lo, ref, kind), mask, mode)
+    _close(got, want, what=f"kl_loss {kind} {mode}")
+    # 1 - exp(k) near k = 0 carries one fp32 rounding of exp (6e-8) on either side, times a row coefficient <= 3/8
+    _close(torch.autograd.grad(got * 3.0, ld)[0], torch.autograd.grad(want * 3.0, lo)[0], atol=1e-7, what="d kl_loss")
+    ld2 = lp.to(dev).requires_grad_(); lo2 = lp.clone().requires_grad_()
+    got_st = compute_kl_loss(ld2, ref.to(dev), mask.to(dev), kind, mode, straight_through=True)
+    want_st = O.agg_loss(O.kl_straight_through(lo2, ref, O.kl_penalty_forward(lo2, ref, kind)), mask, mode)
+    _close(got_st, want_st, what="straight-through value")
+    _close(torch.autograd.grad(got_st, ld2)[0], torch.autograd.grad(want_st, lo2)[0], atol=1e-7, what="straight-through grad")
+
+
 # ---- the two benchmark configurations end to end --------------------------------------------------
 def test_benchmark_config_grpo_policy_loss(dev):
     """512 responses in 64 groups of 8, L = 4096, lengths U[64, 4096], Bernoulli(0.5) outcome reward

@@ -167,3 +167,29 @@ def test_kl_estimators():
     d = b - a
     assert torch.allclose(L.kl_penalty_forward(a, b, "low_var_kl"), torch.exp(d) - d - 1)
     assert L.kl_penalty_forward(torch.tensor([0.0]), torch.tensor([30.0]), "k3").item() == 10.0   # clamp at 10
+
+
+def test_kl_penalty_as_written_and_straight_through():
+    """kl_penalty hands the name to kl_penalty_forward unchanged (core_algos.py:1853), so "+" names fail there;
+    the straight-through combination keeps the forward value and takes the k2 gradient."""
+    a = torch.tensor([-1.0, -2.0, -0.5, -3.0], dtype=torch.float64, requires_grad=True)
+    b = torch.tensor([-1.5, -1.0, -0.5, 25.0], dtype=torch.float64)
+    for name in ("kl", "abs", "mse", "low_var_kl", "k1", "k2", "k3"):
+        assert torch.equal(L.kl_penalty(a, b, name), L.kl_penalty_forward(a, b, name))
+    for name in ("k1+", "k3+", "abs+", "mse+", "full", "nonsense"):
+        with pytest.raises(NotImplementedError):
+            L.kl_penalty(a, b, name)
+    fwd = L.kl_penalty_forward(a, b, "k3")
+    st = L.kl_straight_through(a, b, fwd)
+    assert torch.equal(st.detach(), fwd.detach())
+    g, = torch.autograd.grad(st.sum(), a)
+    assert torch.allclose(g, (a - b).detach())
+    # closed-form gradients of the estimators: k1 -> 1, abs -> sign, k2 -> d, k3 -> 1 - exp(ref - lp) inside the clamps
+    for name, want in (("k1", torch.ones(4, dtype=torch.float64)), ("abs", torch.tensor([1.0, -1.0, 0.0, -1.0], dtype=torch.float64)),
+                       ("k2", (a - b).detach())):
+        g, = torch.autograd.grad(L.kl_penalty_forward(a, b, name).sum(), a)
+        assert torch.allclose(g, want)
+    g, = torch.autograd.grad(L.kl_penalty_forward(a, b, "k3").sum(), a)
+    want = 1 - torch.exp((b - a).detach())
+    want[3] = 0.0                                   # ref - lp = 28 is clamped to 20: no gradient
+    assert torch.allclose(g, want)

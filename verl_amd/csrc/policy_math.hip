@@ -317,6 +317,94 @@ __global__ __launch_bounds__(kRcThreads) void value_kernel(
 }
 
 // =============================================================================================
+// KL penalty (kl_penalty / kl_penalty_forward, core_algos.py:1841-1902)
+// =============================================================================================
+// kld and d kld / d logprob of one element.  straight: value of the chosen estimator, gradient of
+// k2 (0.5 (lp - ref)^2), the reference's "+" variants.
+__device__ __forceinline__ void kl_point(int kind, bool straight, float lp, float ref, float& kld, float& g) {
+  const float d = lp - ref;
+  switch (kind) {
+    case VAMD_KL_K1:
+      kld = d;
+      g = 1.f;
+      break;
+    case VAMD_KL_ABS:
+      kld = fabsf(d);
+      g = d > 0.f ? 1.f : (d < 0.f ? -1.f : 0.f);
+      break;
+    case VAMD_KL_K2:
+      kld = 0.5f * d * d;
+      g = d;
+      break;
+    default: {  // k3: exp(k) - k - 1 with k = clamp(ref - lp, -20, 20), result clamped to [-10, 10]
+      const float k = ref - lp;
+      const float kc = fminf(fmaxf(k, -20.f), 20.f);
+      const float ratio = expf(kc);
+      const float raw = ratio - kc - 1.f;
+      kld = fminf(fmaxf(raw, -10.f), 10.f);
+      const bool pass = k >= -20.f && k <= 20.f && raw >= -10.f && raw <= 10.f;  // clamp passes gradients on its bounds
+      g = pass ? 1.f - ratio : 0.f;
+    } break;
+  }
+  if (straight) g = d;
+}
+
+__global__ __launch_bounds__(256) void kl_elementwise_kernel(const float* __restrict__ lp, const float* __restrict__ ref,
+                                                             int64_t n, int kind, int straight,
+                                                             float* __restrict__ kld, float* __restrict__ grad) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  float k, g;
+  kl_point(kind, straight != 0, lp[i], ref[i], k, g);
+  if (kld) kld[i] = k;
+  if (grad) grad[i] = g;
+}
+
+// agg_loss(kl_penalty(logprob, ref), mask, mode) in one pass, with the per-element gradient
+// (times the mask weight, before the per-row agg_loss coefficient) on request.
+template <bool VEC, class M, bool GRAD>
+__global__ __launch_bounds__(kRcThreads) void kl_loss_kernel(
+    const float* __restrict__ logprob, const float* __restrict__ ref, const M* __restrict__ mask, int64_t rows,
+    int64_t cols, int chunks, int kind, int straight, AggParams ap, Work wk, float* __restrict__ out,
+    float* __restrict__ grad, float* __restrict__ coef) {
+  const int64_t row = blockIdx.x / chunks;
+  const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float lp[kGroups][4], rf[kGroups][4], w[kGroups][4], gr[kGroups][4];
+  load_groups<VEC>(logprob, pos, lp);
+  load_groups<VEC>(ref, pos, rf);
+  load_mask_groups<VEC>(mask, pos, w);
+  const bool token_mean = ap.mode == VAMD_AGG_TOKEN_MEAN;
+  float s_loss = 0, s_m = 0;
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float kld, dk;
+      kl_point(kind, straight != 0, lp[g][e], rf[g][e], kld, dk);
+      const float we = w[g][e];
+      if (e < pos.valid[g]) {
+        s_loss += ((token_mean && we == 0.f) ? 0.f : kld) * we;
+        s_m += we;
+      }
+      if (GRAD) gr[g][e] = dk * we;
+    }
+  if (GRAD) store_groups<VEC>(grad, pos, gr);
+  __shared__ double smem[(2 + 3) * 4];
+  double acc[2] = {s_loss, s_m};
+  block_sum<2, kRcThreads>(acc, smem);
+  if (threadIdx.x == 0) {
+    double* p = wk.partials + (int64_t)blockIdx.x * 2;
+    peer_store(p + 0, acc[0]); peer_store(p + 1, acc[1]);
+  }
+  if (!last_block_arrives(wk.ticket)) return;
+  double loss, msum, extra[1];
+  finalize_agg<2>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
+  if (threadIdx.x == 0) out[0] = (float)loss;
+  ticket_reset(wk.ticket);
+}
+
+// =============================================================================================
 // GRPO
 // =============================================================================================
 constexpr int kGrpoLdsGroups = 2048;  // groups whose statistics fit the last workgroup's LDS
@@ -693,6 +781,57 @@ extern "C" int vamd_value_loss_forward(const float* vpreds, const float* returns
     else { if (grad_unscaled) VAMD_VL(false, true); else VAMD_VL(false, false); }
   });
 #undef VAMD_VL
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
+
+// ---------------------------------------------------------------------------------------------
+extern "C" int vamd_kl_penalty(const float* logprob, const float* ref_logprob, int64_t n, int kind,
+                               int straight_through, float* kld, float* grad, void* stream) {
+  VAMD_REQUIRE(n >= 0 && n < (1ll << 40), "kl_penalty: bad element count");
+  VAMD_REQUIRE(kind >= VAMD_KL_K1 && kind <= VAMD_KL_K3, "kl_penalty: invalid estimator %d", kind);
+  if (n == 0) return VAMD_OK;
+  VAMD_REQUIRE(logprob && ref_logprob && (kld || grad), "kl_penalty: null pointer");
+  hipLaunchKernelGGL(kl_elementwise_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), logprob, ref_logprob, n, kind, straight_through, kld, grad);
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
+
+extern "C" size_t vamd_kl_loss_workspace_bytes(int64_t rows, int64_t cols) {
+  return reduce_workspace_bytes(rows, cols, 2);
+}
+
+extern "C" int vamd_kl_loss_forward(const float* logprob, const float* ref_logprob, const void* mask, int mask_dtype,
+                                    int64_t rows, int64_t cols, int kind, int straight_through, int mode,
+                                    double dp_size, double batch_num_tokens, double global_batch_size,
+                                    double loss_scale_factor, float* out, float* grad_unscaled, float* coef_out,
+                                    void* workspace, size_t workspace_bytes, void* stream) {
+  int st = check_matrix("kl_loss", rows, cols);
+  if (st != VAMD_OK) return st;
+  VAMD_REQUIRE(logprob && ref_logprob && mask && out, "kl_loss: null pointer");
+  VAMD_REQUIRE(kind >= VAMD_KL_K1 && kind <= VAMD_KL_K3, "kl_loss: invalid estimator %d", kind);
+  VAMD_REQUIRE(mode >= 0 && mode <= 3, "kl_loss: invalid mode %d", mode);
+  VAMD_REQUIRE(!grad_unscaled || coef_out, "kl_loss: grad output needs coef_out");
+  if (!workspace || workspace_bytes < vamd_kl_loss_workspace_bytes(rows, cols)) {
+    set_error("kl_loss: workspace too small");
+    return VAMD_EWORKSPACE;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int chunks = (int)chunks_of(cols);
+  const Work wk = carve_work(workspace);
+  const AggParams ap = make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor);
+  const dim3 grid((unsigned)(rows * chunks)), block(kRcThreads);
+#define VAMD_KL(V, G)                                                                                       \
+  hipLaunchKernelGGL((kl_loss_kernel<V, M, G>), grid, block, 0, s, logprob, ref_logprob, mk, rows, cols, chunks, \
+                     kind, straight_through, ap, wk, out, grad_unscaled, coef_out)
+  VAMD_MASK_DISPATCH(mask_dtype, M, {
+    const bool vec = can_vectorize(cols, {logprob, ref_logprob, grad_unscaled}, mask, sizeof(M));
+    const M* mk = static_cast<const M*>(mask);
+    if (vec) { if (grad_unscaled) VAMD_KL(true, true); else VAMD_KL(true, false); }
+    else { if (grad_unscaled) VAMD_KL(false, true); else VAMD_KL(false, false); }
+  });
+#undef VAMD_KL
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }

@@ -408,3 +408,117 @@ def compute_value_loss(vpreds: torch.Tensor, returns: torch.Tensor, values: torc
     vf_loss, out = _ValueLoss.apply(vpreds, returns, values, response_mask, float(cliprange_value),
                                     _agg_mode(loss_agg_mode))
     return vf_loss, out[1]
+
+
+# ---- KL penalty -----------------------------------------------------------------------------------
+_KL_KINDS = {"kl": 0, "k1": 0, "abs": 1, "mse": 2, "k2": 2, "low_var_kl": 3, "k3": 3}
+
+
+def _kl_kind(kl_penalty: str) -> int:
+    """Estimator code of ``kl_penalty_forward``; every other name (``"full"``, and in this reference
+    snapshot every ``"+"``-suffixed name, which reaches ``kl_penalty_forward`` unstripped,
+    core_algos.py:1853,1868-1902) raises ``NotImplementedError`` as there."""
+    if kl_penalty not in _KL_KINDS:
+        raise NotImplementedError
+    return _KL_KINDS[kl_penalty]
+
+
+class _KlPenalty(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logprob, ref_logprob, kind, straight_through):
+        dev = _cabi.compute_device(logprob, ref_logprob)
+        assert logprob.shape == ref_logprob.shape
+        lp = _cabi.as_f32(logprob, dev).contiguous()
+        ref = _cabi.as_f32(ref_logprob, dev).contiguous()
+        need_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        kld = torch.empty_like(lp)
+        g = torch.empty_like(lp) if need_grad else None
+        with torch.cuda.device(dev):
+            _cabi.check(_cabi.lib().vamd_kl_penalty(lp.data_ptr(), ref.data_ptr(), lp.numel(), kind,
+                                                    int(straight_through), kld.data_ptr(), _cabi.ptr(g),
+                                                    _cabi.stream_ptr(dev)))
+        if need_grad:
+            ctx.save_for_backward(g)
+        ctx.meta = [(t.device, t.dtype) for t in (logprob, ref_logprob)]
+        return kld.to(logprob.device)
+
+    @staticmethod
+    def backward(ctx, d_kld):
+        (g,) = ctx.saved_tensors
+        d = g * d_kld.to(device=g.device, dtype=torch.float32)
+        outs = []
+        for need, (device, dtype), sign in zip(ctx.needs_input_grad[:2], ctx.meta, (1.0, -1.0)):
+            outs.append((sign * d).to(device=device, dtype=dtype) if need else None)
+        return outs[0], outs[1], None, None
+
+
+def kl_penalty_forward(logprob: torch.Tensor, ref_logprob: torch.Tensor, kl_penalty) -> torch.Tensor:
+    """Per-token KL estimate between the policy and the reference policy
+    (reference core_algos.py:1868-1902): ``"kl"/"k1"``, ``"abs"``, ``"mse"/"k2"``,
+    ``"low_var_kl"/"k3"``; differentiable with respect to both inputs."""
+    return _KlPenalty.apply(logprob, ref_logprob, _kl_kind(kl_penalty), False)
+
+
+def kl_penalty(logprob: torch.Tensor, ref_logprob: torch.Tensor, kl_penalty) -> torch.Tensor:
+    """``kl_penalty`` of the reference (core_algos.py:1841-1866).  It evaluates
+    ``kl_penalty_forward`` with the name as given before looking at a trailing ``"+"``, so in this
+    snapshot the straight-through names raise ``NotImplementedError`` there; the kernel's
+    straight-through path (value of the estimator, gradient of k2) is reachable through
+    ``compute_kl_loss(..., straight_through=True)``."""
+    return kl_penalty_forward(logprob, ref_logprob, kl_penalty)
+
+
+class _KlLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logprob, ref_logprob, response_mask, kind, straight_through, mode, dp, bnt, gbs, lsf):
+        dev = _cabi.compute_device(logprob, ref_logprob, response_mask)
+        lp = _matrix(logprob, dev)
+        ref = _matrix(ref_logprob, dev)
+        assert lp.shape == ref.shape
+        m, code = _mask_matrix(response_mask, dev, lp.shape)
+        rows, cols = lp.shape
+        need_grad = ctx.needs_input_grad[0]
+        Lb = _cabi.lib()
+        out = torch.empty(1, dtype=torch.float32, device=dev)
+        coef = torch.empty(rows, dtype=torch.float32, device=dev)
+        g = torch.empty_like(lp) if need_grad else None
+        ws = _cabi.ticket_workspace(Lb.vamd_kl_loss_workspace_bytes(rows, cols), dev)
+        with torch.cuda.device(dev):
+            _cabi.check(Lb.vamd_kl_loss_forward(lp.data_ptr(), ref.data_ptr(), m.data_ptr(), code, rows, cols, kind,
+                                                int(straight_through), mode, dp, bnt, gbs, lsf, out.data_ptr(),
+                                                _cabi.ptr(g), coef.data_ptr(), ws.data_ptr(), ws.numel(),
+                                                _cabi.stream_ptr(dev)))
+        if need_grad:
+            ctx.save_for_backward(g, coef)
+        ctx.in_shape = logprob.shape
+        ctx.in_device = logprob.device
+        ctx.in_dtype = logprob.dtype
+        return out[0].to(logprob.device)
+
+    @staticmethod
+    def backward(ctx, d_loss):
+        g, coef = ctx.saved_tensors
+        dev = g.device
+        rows, cols = g.shape
+        d = _cabi.as_f32(d_loss, dev).reshape(1)
+        res = torch.empty_like(g)
+        with torch.cuda.device(dev):
+            _cabi.check(_cabi.lib().vamd_scale_rows(g.data_ptr(), coef.data_ptr(), d.data_ptr(), 1.0, rows, cols,
+                                                    res.data_ptr(), _cabi.stream_ptr(dev)))
+        res = res.view(ctx.in_shape).to(device=ctx.in_device, dtype=ctx.in_dtype)
+        return (res,) + (None,) * 9
+
+
+def compute_kl_loss(logprob: torch.Tensor, ref_logprob: torch.Tensor, response_mask: torch.Tensor,
+                    kl_penalty: str = "low_var_kl", loss_agg_mode: str = "token-mean", dp_size: int = 1,
+                    batch_num_tokens=None, global_batch_size=None, loss_scale_factor=None,
+                    straight_through: bool = False) -> torch.Tensor:
+    """``agg_loss(kl_penalty(logprob, ref_logprob, kl_penalty), response_mask, loss_agg_mode)`` in one
+    pass over the tensors: the ``kl_loss`` term of the actor update (reference
+    verl/workers/actor/dp_actor.py:640-646), differentiable with respect to ``logprob``.  No
+    single function of the reference does both steps; this one exists so that the pair costs one
+    read of the inputs.  ``straight_through=True`` keeps the estimator's value and uses the k2
+    gradient, the behaviour the reference documents for the ``"+"`` names."""
+    return _KlLoss.apply(logprob, ref_logprob, response_mask, _kl_kind(kl_penalty), bool(straight_through),
+                         _agg_mode(loss_agg_mode), float(dp_size), _opt(batch_num_tokens), _opt(global_batch_size),
+                         _opt(loss_scale_factor))
