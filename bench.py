@@ -60,6 +60,75 @@ def cpu_baseline(n_cpu: int, h: int, v: int, temperature: float) -> dict:
     }
 
 
+def policy_math_rates(dev, with_cpu: bool) -> dict:
+    """The [B, L] kernels at B = 512, L = 4096 (BASELINE configs 3 and 4): microseconds per call from HIP events over
+    40 calls that rotate through 8 buffer sets (more than the 256 MB Infinity Cache), the algorithmic bytes of the
+    op, and the fraction of 8 TB/s that gives.  ``cpu_ms`` is the CPU oracle on one buffer set."""
+    import torch
+
+    import oracle as O
+    from verl_amd import _cabi
+
+    L = _cabi.lib()
+    B, Lc, nset = 512, 4096, 8
+    BL = B * Lc
+    g = torch.Generator(device=dev).manual_seed(0)
+
+    def mk():
+        lens = torch.randint(64, Lc + 1, (B,), device=dev, generator=g)
+        mask = (torch.arange(Lc, device=dev)[None, :] < lens[:, None]).float()
+        t = lambda: torch.randn(B, Lc, device=dev, generator=g)
+        return dict(mask=mask, a=t(), b=t(), c=t(), o1=torch.empty(B, Lc, device=dev), o2=torch.empty(B, Lc, device=dev))
+
+    sets = [mk() for _ in range(nset)]
+    ws = torch.zeros(1 << 22, dtype=torch.uint8, device=dev)
+    out = torch.empty(8, device=dev)
+    coef = torch.empty(B, device=dev)
+    mom = torch.empty(4, dtype=torch.float64, device=dev)
+    gid = torch.arange(64, device=dev).repeat_interleave(8)
+    st = _cabi.stream_ptr(dev)
+    P = lambda t: t.data_ptr()
+    chk = _cabi.check
+    ops = {
+        "grpo_advantage": (12 * BL, lambda s: chk(L.vamd_grpo_advantage(P(s["a"]), P(s["mask"]), 0, P(gid), B, Lc, 64, 1e-6, 1, 0, P(s["o1"]), None, P(ws), ws.numel(), st))),
+        "policy_loss_fwd": (16 * BL, lambda s: chk(L.vamd_policy_loss_forward(P(s["a"]), P(s["b"]), P(s["c"]), P(s["mask"]), 0, None, B, Lc, 0.2, 0.2, 3.0, 0, 1.0, -1.0, -1.0, -1.0, P(out), None, None, P(ws), ws.numel(), st))),
+        "policy_loss_fwd_grad": (20 * BL, lambda s: chk(L.vamd_policy_loss_forward(P(s["a"]), P(s["b"]), P(s["c"]), P(s["mask"]), 0, None, B, Lc, 0.2, 0.2, 3.0, 0, 1.0, -1.0, -1.0, -1.0, P(out), P(s["o1"]), P(coef), P(ws), ws.numel(), st))),
+        "gae_scan_whiten": (28 * BL, lambda s: chk(L.vamd_gae(P(s["a"]), P(s["b"]), P(s["mask"]), 0, B, Lc, 1.0, 0.95, 1, P(s["o1"]), P(s["o2"]), P(mom), P(ws), ws.numel(), st))),
+        "value_loss_fwd_grad": (20 * BL, lambda s: chk(L.vamd_value_loss_forward(P(s["a"]), P(s["b"]), P(s["c"]), P(s["mask"]), 0, B, Lc, 0.5, 0, P(out), P(s["o1"]), P(coef), P(ws), ws.numel(), st))),
+        "kl_loss_fwd_grad": (16 * BL, lambda s: chk(L.vamd_kl_loss_forward(P(s["a"]), P(s["b"]), P(s["mask"]), 0, B, Lc, 3, 0, 0, 1.0, -1.0, -1.0, -1.0, P(out), P(s["o1"]), P(coef), P(ws), ws.numel(), st))),
+        "masked_moments": (8 * BL, lambda s: chk(L.vamd_masked_moments(P(s["a"]), P(s["mask"]), 0, B, Lc, 0, P(mom), P(ws), ws.numel(), st))),
+        "copy_yardstick": (8 * BL, lambda s: chk(L.vamd_copy_bytes(P(s["a"]), P(s["o1"]), 4 * BL, st))),
+    }
+    res = {}
+    for name, (nbytes, fn) in ops.items():
+        for s in sets:
+            fn(s)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 40
+        e0.record()
+        for i in range(reps):
+            fn(sets[i % nset])
+        e1.record()
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / reps * 1e3
+        res[name] = {"us": us, "algorithmic_bytes": nbytes, "GBps": nbytes / us / 1e3, "frac_of_8TBps": nbytes / us / 1e3 / 8000.0}
+    if with_cpu:
+        s = {k: v.cpu() for k, v in sets[0].items()}
+        idx = gid.cpu().numpy()
+
+        def cpu_ms(fn):
+            t0 = time.perf_counter()
+            fn()
+            return (time.perf_counter() - t0) * 1e3
+
+        res["grpo_advantage"]["cpu_ms"] = cpu_ms(lambda: O.grpo_outcome_advantage(s["a"].clone(), s["mask"], idx))
+        res["gae_scan_whiten"]["cpu_ms"] = cpu_ms(lambda: O.gae_advantage_return(s["a"], s["b"], s["mask"], 1.0, 0.95))
+        res["policy_loss_fwd"]["cpu_ms"] = cpu_ms(lambda: O.policy_loss_vanilla(s["a"], s["b"], s["c"], s["mask"], "token-mean"))
+        res["value_loss_fwd_grad"]["cpu_ms"] = cpu_ms(lambda: O.value_loss(s["a"], s["b"], s["c"], s["mask"], 0.5, "token-mean"))
+    return res
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -148,6 +217,9 @@ def main() -> None:
     }
 
     base = cpu_baseline(args.cpu_tokens, h, v, T) if args.cpu_tokens > 0 else None
+    del hidden, weight
+    torch.cuda.empty_cache()
+    pm = policy_math_rates(dev, with_cpu=args.cpu_tokens > 0)
 
     print(json.dumps({
         "metric": "tokens/s fwd+bwd logprob+entropy head @Qwen2.5-7B shape; MFMA util %",
@@ -170,6 +242,7 @@ def main() -> None:
         "mfma_util_pct": 100.0 * roofline["step_hardware_frac"],
         "roofline": roofline,
         "cpu_baseline": base,
+        "policy_math_b512_l4096": pm,
     }))
 
 
