@@ -251,3 +251,47 @@ def test_benchmark_config_7b_head_full_size(dev):
     _close_bf16(dw_c, dw.float(), "d_weight cached vs recomputed")
     assert (dh_c.float() - dh.float()).pow(2).mean().sqrt().item() < 1e-4
     assert (dw_c.float() - dw.float()).pow(2).mean().sqrt().item() < 1e-4
+
+
+def test_benchmark_config_small_head_forward_only(dev):
+    """Qwen2.5-0.5B head shape, forward only (N=2048, H=896, V=151936, T=1): the configuration the reference's CPU
+    path runs in full."""
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    n, h, v, T = 2048, 896, 151936, 1.0
+    hidden, weight, labels = _make(n, h, v, seed=21, dist="normal")
+    with torch.no_grad():
+        lp, ent = linear_cross_entropy(hidden.to(dev), weight.to(dev), labels.to(dev), T)
+    want_lp, want_ent = _oracle(hidden, weight, labels, T, device=dev)
+    assert lp.dtype == torch.float32 and lp.shape == (n,)
+    assert (lp - want_lp).abs().max().item() <= ATOL and (ent - want_ent).abs().max().item() <= ATOL
+
+
+def test_benchmark_config_llama_head_token_chunked(dev):
+    """Llama-3.1-8B head shape (H=4096, V=128256, T=0.7) processed in 8192-token chunks with the weight gradient
+    accumulated across chunks and the entropy coefficient 0.001 passed as a scalar folded into the backward; two
+    chunks of the configuration's eight keep the test short.  One chunk goes through the logits cache, the other
+    through the recompute path."""
+    from verl_amd.utils.kernel import linear_cross_entropy as K
+    n, h, v, T, chunk = 16384, 4096, 128256, 0.7, 8192
+    g = torch.Generator(device=dev).manual_seed(5)
+    hidden = torch.randn(n, h, device=dev, generator=g).bfloat16()
+    weight = (torch.randn(v, h, device=dev, generator=g) * 0.02).bfloat16()
+    labels = torch.randint(0, v, (n,), device=dev, generator=g)
+    g_lp = torch.randn(n, device=dev, generator=g)
+    d_weight = torch.zeros_like(weight)
+    lps, ents, dhs = [], [], []
+    for ci, lo in enumerate(range(0, n, chunk)):
+        sl = slice(lo, lo + chunk)
+        cache = torch.empty(chunk, v, device=dev) if ci == 0 else None
+        lp, ent, lse, mz = K.efficient_entropy_forward(hidden[sl], weight, labels[sl], 0, T, logits_cache=cache)
+        dh, _ = K.efficient_entropy_backward(g_lp[sl], None, hidden[sl], weight, labels[sl], lse, mz, 0, T,
+                                             d_entropy_scalar=0.001, d_weight_out=d_weight, logits_cache=cache)
+        lps.append(lp); ents.append(ent); dhs.append(dh)
+        del cache
+    want_lp, want_ent, want_dh, want_dw, e_dh, e_dw = _oracle_with_scale(
+        hidden, weight, labels, T, g_lp, torch.full((n,), 0.001, device=dev), dev)
+    assert (torch.cat(lps) - want_lp).abs().max().item() <= ATOL
+    assert (torch.cat(ents) - want_ent).abs().max().item() <= ATOL
+    _close_bf16(torch.cat(dhs), want_dh, "d_hidden", e_dh)
+    # d_weight passes through bf16 once per token chunk: one more half-ulp of the running value per accumulation
+    _close_bf16(d_weight, want_dw, "d_weight accumulated over token chunks", e_dw + want_dw.abs())

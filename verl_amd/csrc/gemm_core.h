@@ -291,10 +291,8 @@ __device__ __forceinline__ void slab_iter(const SlabDma<RK>& dr, const SlabDma<C
   for (int i = 0; i < 8; ++i) {
     VAMD_MFMA(f1, i);
     VAMD_FRAG(f0, nxt, i, 0);
-#ifndef VAMD_DBG_NO_GLOBAL
     if (i < 4) dr.issue_one(i, r2, lds_address(cur));
     else dc.issue_one(i - 4, c2, lds_address(cur) + kSlabBytes);
-#endif
     VAMD_SLOT_END;
   }
 #undef VAMD_MFMA
@@ -346,13 +344,8 @@ __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, in
       rs_r = tile_rsrc<R_KMAJOR>(R, tr);
       rs_c = tile_rsrc<C_KMAJOR>(C, tc);
     }
-#ifdef VAMD_DBG_SAME_SLAB
-    src_r = SlabSrc{rs_r, 0u};
-    src_c = SlabSrc{rs_c, 0u};
-#else
     src_r = SlabSrc{rs_r, slab_soff<R_KMAJOR>(R, k2 * kBK)};
     src_c = SlabSrc{rs_c, slab_soff<C_KMAJOR>(C, k2 * kBK)};
-#endif
   };
 
   // slab 0 -> stage 0, slab 1 -> stage 1
