@@ -51,6 +51,19 @@ extern "C" {
 #define VAMD_KL_K2 2  /* "mse", "k2": 0.5 (logprob - ref)^2 */
 #define VAMD_KL_K3 3  /* "low_var_kl", "k3": exp(k) - k - 1, k = clamp(ref - logprob, -20, 20), clamped to [-10, 10] */
 
+/* outcome-reward advantage estimators that reduce a response to one score and normalise it inside its
+ * prompt group (verl/trainer/ppo/core_algos.py:266-330, :421-579, :657-753) */
+#define VAMD_ADV_GRPO 0            /* (s - mean) / (std + eps), or s - mean */
+#define VAMD_ADV_RLOO 1            /* s n/(n-1) - mean n/(n-1); a single-member group keeps s */
+#define VAMD_ADV_RLOO_VECTORIZED 2 /* the same; a single-member group gets 0 */
+#define VAMD_ADV_MEAN_BASELINE 3   /* s - mean: REINFORCE++ baseline before its whitening */
+#define VAMD_ADV_OPO 4             /* s - sum(len s) / sum(len), len = response length */
+#define VAMD_ADV_GPG 5             /* alpha (s - mean) / f_norm, alpha = batch / max(#{s != 0}, 1) */
+
+/* token-level return recurrences (core_algos.py:582-654) */
+#define VAMD_RETURNS_REMAX 0        /* returns = reverse cumsum of r m; adv = returns - baseline_i m */
+#define VAMD_RETURNS_REINFORCE_PP 1 /* R_t = r_t + gamma c, c <- R_t m_t; adv = masked_whiten(R, m) m */
+
 int vamd_abi_version(void);
 const char* vamd_last_error(void);
 
@@ -126,6 +139,10 @@ int vamd_masked_moments(const float* values, const void* mask, int mask_dtype, i
  * output following masked_var's unbiased rule; flags_host receives nothing -- the M in {0,1}
  * error of masked_var (:311-316) is raised by the host wrapper from the moments. */
 int vamd_whiten_stats(const double* moments, int shift_mean, float* stats, void* stream);
+/* out[i] = ((values[i] - mean) * rstd + shift) * mask[i]: whitening followed by the mask product of the
+ * REINFORCE++ estimators (core_algos.py:472, :615-616). */
+int vamd_affine_by_stats_masked(const float* values, const float* stats, const void* mask, int mask_dtype, int64_t n,
+                                float* out, void* stream);
 int vamd_affine_by_stats(const float* values, const float* stats, int64_t n, float* out, void* stream);
 
 /* ------------------------------------------------------------------------------------------
@@ -156,6 +173,26 @@ int vamd_grpo_advantage(const float* rewards, const void* mask, int mask_dtype, 
                         size_t workspace_bytes, void* stream);
 
 /* group_mean_std (verl/utils/groupwise.py:163-223): mean/std/count per group, singleton -> (0,1). */
+/* The group-normalised outcome estimators above behind one entry point; vamd_grpo_advantage is the
+ * VAMD_ADV_GRPO case.  std_mode and norm_by_std only matter for GRPO, f_norm only for GPG.  Estimators
+ * other than GRPO support at most 2048 groups.  The REINFORCE++-baseline estimator is
+ * VAMD_ADV_MEAN_BASELINE followed by masked whitening (vamd_masked_moments, vamd_whiten_stats,
+ * vamd_affine_by_stats_masked). */
+size_t vamd_group_outcome_advantage_workspace_bytes(int64_t batch, int64_t length, int64_t n_groups);
+int vamd_group_outcome_advantage(const float* rewards, const void* mask, int mask_dtype, const int64_t* group_ids,
+                                 int64_t batch, int64_t length, int64_t n_groups, int estimator, float epsilon,
+                                 int norm_by_std, int std_mode, float f_norm, float* advantages, float* scores_out,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+
+/* ReMax and REINFORCE++ (core_algos.py:621-654, :582-618): returns[batch, length] by a reverse scan over
+ * each response, then the advantages (ReMax: returns - row_baseline[i] * mask; REINFORCE++: whitened
+ * returns * mask, row_baseline unused and may be NULL).  moments_out (optional, 3 doubles): sum(m),
+ * sum(R m), sum(R^2 m) of the returns, from which a caller checks that at least two tokens are valid. */
+size_t vamd_returns_advantage_workspace_bytes(int64_t batch, int64_t length);
+int vamd_returns_advantage(const float* rewards, const void* mask, int mask_dtype, const float* row_baseline,
+                           int64_t batch, int64_t length, float gamma, int mode, float* advantages, float* returns,
+                           double* moments_out, void* workspace, size_t workspace_bytes, void* stream);
+
 int vamd_group_mean_std(const float* scores, const int64_t* group_ids, int64_t n, int64_t n_groups, float eps,
                         float* mean, float* std, float* count, void* stream);
 

@@ -40,6 +40,13 @@ from .advantages import (  # noqa: F401
     grpo_vectorized_outcome_advantage,
     as_torch_index,
     group_mean_std,
+    rloo_outcome_advantage,
+    rloo_vectorized_outcome_advantage,
+    reinforce_plus_plus_baseline_outcome_advantage,
+    opo_outcome_advantage,
+    gpg_outcome_advantage,
+    reinforce_plus_plus_outcome_advantage,
+    remax_outcome_advantage,
 )
 from .losses import (  # noqa: F401
     agg_loss,

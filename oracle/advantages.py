@@ -177,3 +177,126 @@ def grpo_vectorized_outcome_advantage(token_level_rewards, response_mask, index,
         a = scores - mean_g[g]
     out = a.unsqueeze(-1) * response_mask
     return out, out
+
+
+# ---- other outcome estimators of the registry -------------------------------------------------
+def _group_members(scores, index):
+    members = defaultdict(list)
+    for i in range(scores.shape[0]):
+        members[index[i]].append(i)
+    return members
+
+
+def _group_means(scores, members):
+    """Mean per group, 0 for a single-member group (core_algos.py:446-452, :505-511)."""
+    mean_of = {}
+    for key, rows in members.items():
+        if len(rows) == 1:
+            mean_of[key] = torch.tensor(0.0)
+        elif len(rows) > 1:
+            mean_of[key] = torch.mean(torch.stack([scores[i] for i in rows]))
+        else:
+            raise ValueError(f"no score in prompt index: {key}")
+    return mean_of
+
+
+@torch.no_grad()
+def rloo_outcome_advantage(token_level_rewards, response_mask, index):
+    """Leave-one-out baseline, loop form (core_algos.py:479-528): with n members in the group
+    ``s n/(n-1) - mean n/(n-1)``; a single-member group keeps its score."""
+    scores = token_level_rewards.sum(dim=-1)
+    members = _group_members(scores, index)
+    mean_of = _group_means(scores, members)
+    out = scores.clone()
+    for i in range(scores.shape[0]):
+        n = len(members[index[i]])
+        if n > 1:
+            out[i] = scores[i] * n / (n - 1) - mean_of[index[i]] * n / (n - 1)
+    out = out.unsqueeze(-1) * response_mask
+    return out, out
+
+
+@torch.no_grad()
+def rloo_vectorized_outcome_advantage(token_level_rewards, response_mask, index):
+    """Vectorised twin (core_algos.py:720-753): ``(c s - group_sum) / max(c - 1, 1) * (c > 1)``."""
+    scores = token_level_rewards.sum(dim=-1)
+    inv = torch.from_numpy(np.unique(index, return_inverse=True)[1])
+    c = torch.bincount(inv)[inv].to(scores.dtype)
+    adv = ((c * scores - torch.bincount(inv, weights=scores)[inv]) / (c - 1).clamp_min(1)) * (c > 1)
+    adv = adv.unsqueeze(-1) * response_mask
+    return adv, adv
+
+
+@torch.no_grad()
+def reinforce_plus_plus_baseline_outcome_advantage(token_level_rewards, response_mask, index):
+    """core_algos.py:421-474: score minus the group mean, tiled over the response and masked, then
+    ``masked_whiten(.) * mask``."""
+    length = token_level_rewards.shape[-1]
+    scores = token_level_rewards.sum(dim=-1)
+    members = _group_members(scores, index)
+    mean_of = _group_means(scores, members)
+    out = scores.clone()
+    for i in range(scores.shape[0]):
+        out[i] = scores[i] - mean_of[index[i]]
+    out = out.unsqueeze(-1).tile([1, length]) * response_mask
+    out = masked_whiten(out, response_mask) * response_mask
+    return out, out
+
+
+@torch.no_grad()
+def opo_outcome_advantage(token_level_rewards, response_mask, index):
+    """core_algos.py:531-579: baseline = length-weighted mean score of the group, 0 for a single member."""
+    lengths = response_mask.sum(dim=-1)
+    scores = token_level_rewards.sum(dim=-1)
+    members = _group_members(scores, index)
+    out = scores.clone()
+    for key, rows in members.items():
+        if len(rows) == 1:
+            baseline = torch.tensor(0.0)
+        else:
+            s = torch.stack([scores[i] for i in rows])
+            n = torch.stack([lengths[i] for i in rows])
+            baseline = (n * s).sum() / n.sum()
+        for i in rows:
+            out[i] = scores[i] - baseline
+    out = out.unsqueeze(-1) * response_mask
+    return out, out
+
+
+@torch.no_grad()
+def gpg_outcome_advantage(token_level_rewards, response_mask, index, f_norm=1.0):
+    """core_algos.py:657-717: ``alpha (s - mean) / f_norm`` with ``alpha = batch / max(#{s != 0}, 1)``
+    (the ``alpha`` argument of the reference is overwritten, :697-698)."""
+    scores = token_level_rewards.sum(dim=-1)
+    bsz = scores.shape[0]
+    alpha = bsz / torch.count_nonzero(scores).clamp(min=1)
+    members = _group_members(scores, index)
+    mean_of = _group_means(scores, members)
+    out = scores.clone()
+    for i in range(bsz):
+        out[i] = alpha * (scores[i] - mean_of[index[i]]) / f_norm
+    out = out.unsqueeze(-1) * response_mask
+    return out, out
+
+
+@torch.no_grad()
+def reinforce_plus_plus_outcome_advantage(token_level_rewards, response_mask, gamma):
+    """core_algos.py:582-618: discounted return that restarts after a masked step, then
+    ``masked_whiten(returns) * mask``; returns ``(advantages, returns)``."""
+    returns = torch.zeros_like(token_level_rewards)
+    running = 0
+    for t in reversed(range(token_level_rewards.shape[1])):
+        running = token_level_rewards[:, t] + gamma * running
+        returns[:, t] = running
+        running = running * response_mask[:, t]
+    advantages = masked_whiten(returns, response_mask) * response_mask
+    return advantages, returns
+
+
+@torch.no_grad()
+def remax_outcome_advantage(token_level_rewards, reward_baselines, response_mask):
+    """core_algos.py:621-654: reverse cumulative sum of the masked rewards minus the per-response
+    baseline on the mask."""
+    returns = (token_level_rewards * response_mask).flip(dims=[-1]).cumsum(dim=-1).flip(dims=[-1])
+    advantages = returns - reward_baselines.unsqueeze(-1) * response_mask
+    return advantages, returns

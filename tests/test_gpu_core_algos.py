@@ -349,6 +349,99 @@ def test_value_loss_forward_backward(dev, mode, shape):
            what="d vf_loss / d vpreds")
 
 
+# ---- the other outcome estimators ---------------------------------------------------------------------
+_GROUP_ESTIMATORS = [
+    ("compute_rloo_outcome_advantage", "rloo_outcome_advantage", {}),
+    ("compute_rloo_vectorized_outcome_advantage", "rloo_vectorized_outcome_advantage", {}),
+    ("compute_opo_outcome_advantage", "opo_outcome_advantage", {}),
+    ("compute_gpg_outcome_advantage", "gpg_outcome_advantage", {"f_norm": 2.0}),
+    ("compute_reinforce_plus_plus_baseline_outcome_advantage", "reinforce_plus_plus_baseline_outcome_advantage", {}),
+]
+
+
+@pytest.mark.parametrize("batch_size,seq_len,num_groups,seed", GOLDEN["grpo_equivalence_grid"]["cases"] + [[37, 4099, 9, 4]])
+@pytest.mark.parametrize("fn,oracle_fn,kw", _GROUP_ESTIMATORS)
+def test_group_outcome_estimators(dev, fn, oracle_fn, kw, batch_size, seq_len, num_groups, seed):
+    """RLOO (loop and vectorised rules), OPO, GPG and REINFORCE++-baseline on the reference's test grid, with
+    single-member groups and all-zero scores mixed in."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    torch.manual_seed(seed); random.seed(seed); np.random.seed(seed)
+    index = _make_group_index(batch_size, num_groups)
+    index[:2] = [num_groups, num_groups + 1]                    # two single-member groups
+    mask = _rand_mask(batch_size, seq_len)
+    rewards = torch.randn(batch_size, seq_len) * mask
+    rewards[5] = 0                                               # a zero score (counts in GPG's alpha)
+    got, got2 = getattr(CA, fn)(rewards.to(dev), mask.to(dev), index, **kw)
+    want, _ = getattr(O, oracle_fn)(rewards.clone(), mask, index, **kw)
+    assert got is got2 and got.shape == (batch_size, seq_len)
+    # scores are sums of up to 4099 N(0,1) values: allow one fp32 ulp of a score of magnitude ~100 on top of rtol
+    _close(got, want, atol=2e-5, what=fn)
+    assert torch.equal(got.cpu() == 0, want == 0) or "plus_plus" in fn
+    names = np.array([f"prompt-{i}" for i in index], dtype=object)                 # string labels, CPU inputs
+    got3, _ = getattr(CA, fn)(rewards, mask, names, **kw)
+    assert got3.device.type == "cpu"
+    _close(got3, got.cpu(), atol=1e-7, what=fn + " with string labels")
+    assert CA.get_adv_estimator_fn(fn[len("compute_"):-len("_outcome_advantage")]) is getattr(CA, fn)
+
+
+def test_group_outcome_estimators_by_hand(dev):
+    from verl_amd.trainer.ppo import core_algos as CA
+    rewards = torch.tensor([[1.0, 2.0, 0.0], [0.5, 0.0, 0.0], [4.0, 1.0, 1.0], [0.0, 0.0, 0.0], [2.0, 2.0, 2.0]])
+    mask = torch.tensor([[1.0, 1.0, 0.0], [1.0, 0.0, 0.0], [1.0, 1.0, 1.0], [1.0, 1.0, 0.0], [1.0, 1.0, 1.0]])
+    index = np.array(["a", "a", "a", "b", "c"], dtype=object)
+    adv, _ = CA.compute_rloo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    s = [3.0, 0.5, 6.0]
+    for i in range(3):
+        others = [s[j] for j in range(3) if j != i]
+        assert torch.allclose(adv[i].cpu(), (s[i] - sum(others) / 2) * mask[i], atol=1e-6)
+    assert torch.equal(adv[4].cpu(), 6.0 * mask[4])
+    adv_v, _ = CA.compute_rloo_vectorized_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    assert torch.equal(adv_v[4].cpu(), torch.zeros(3))
+    bsl = (2 * 3.0 + 1 * 0.5 + 3 * 6.0) / 6.0
+    adv, _ = CA.compute_opo_outcome_advantage(rewards.to(dev), mask.to(dev).bool(), index)
+    for i in range(3):
+        assert torch.allclose(adv[i].cpu(), (s[i] - bsl) * mask[i], atol=1e-6)
+    adv, _ = CA.compute_gpg_outcome_advantage(rewards.to(dev), mask.to(dev), index, f_norm=2.0, alpha=123.0)
+    assert torch.allclose(adv[4].cpu(), 1.25 * 6.0 / 2.0 * mask[4])
+    with pytest.raises(ValueError):                              # whitening needs two valid tokens
+        CA.compute_reinforce_plus_plus_baseline_outcome_advantage(rewards.to(dev), torch.zeros(5, 3, device=dev), index)
+    with pytest.raises(ValueError):
+        CA.compute_rloo_outcome_advantage(rewards.to(dev), mask.to(dev), index[:3])
+
+
+@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192)])
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.int64])
+def test_reinforce_plus_plus_and_remax(dev, shape, mdtype):
+    from verl_amd.trainer.ppo import core_algos as CA
+    g = torch.Generator().manual_seed(shape[1])
+    B, Lc = shape
+    rewards = torch.randn(B, Lc, generator=g)
+    mask, lens = _prefix_mask(B, Lc, g, lo=2)
+    mask[0, Lc // 2] = 0                                         # a hole inside a response
+    cfg = types.SimpleNamespace(gamma=0.97)
+    adv, ret = CA.compute_reinforce_plus_plus_outcome_advantage(rewards.to(dev), mask.to(dev).to(mdtype), config=cfg)
+    want_adv, want_ret = O.reinforce_plus_plus_outcome_advantage(rewards, mask, 0.97)
+    ret64 = O.reinforce_plus_plus_outcome_advantage(rewards.double(), mask.double(), 0.97)[1]
+    # the scan re-associates the fp32 recurrence: hold it to the fp64 result as tightly as the sequential fp32 loop
+    scale = ret64.abs().max().item()
+    err_kernel = (ret.cpu().double() - ret64).abs().max().item()
+    err_oracle = (want_ret.double() - ret64).abs().max().item()
+    assert err_kernel <= max(2 * err_oracle, 1e-5 * scale), (err_kernel, err_oracle, scale)
+    _close(adv, want_adv, atol=2e-5, what="reinforce++ advantages")
+    assert torch.equal(adv.cpu() == 0, want_adv == 0)
+    base = torch.randn(B, generator=g)
+    adv2, ret2 = CA.compute_remax_outcome_advantage(rewards.to(dev), base.to(dev), mask.to(dev).to(mdtype))
+    want_adv2, want_ret2 = O.remax_outcome_advantage(rewards, base, mask)
+    ret2_64 = O.remax_outcome_advantage(rewards.double(), base.double(), mask.double())[1]
+    err_kernel = (ret2.cpu().double() - ret2_64).abs().max().item()
+    err_oracle = (want_ret2.double() - ret2_64).abs().max().item()
+    assert err_kernel <= max(2 * err_oracle, 1e-5 * ret2_64.abs().max().item()), (err_kernel, err_oracle)
+    _close(adv2, want_adv2, atol=1e-5 * max(1.0, ret2_64.abs().max().item()), what="remax advantages")
+    with pytest.raises(AssertionError):
+        CA.compute_reinforce_plus_plus_outcome_advantage(rewards.to(dev), mask.to(dev))       # config is required
+    assert CA.get_adv_estimator_fn("remax") is CA.compute_remax_outcome_advantage
+
+
 # ---- KL penalty -------------------------------------------------------------------------------------
 @pytest.mark.parametrize("kind", ["kl", "k1", "abs", "mse", "k2", "low_var_kl", "k3"])
 def test_kl_penalty_elementwise(dev, kind):

@@ -213,3 +213,89 @@ def test_grpo_singletons_strings_equal_scores_and_unmasked_sum():
     assert torch.allclose(adv[3], torch.tensor([0.0, 10.0 / (1 + 1e-6)]))
     adv_v, _ = A.grpo_vectorized_outcome_advantage(rewards, mask, index)
     assert torch.allclose(adv, adv_v, rtol=1e-5, atol=1e-6)
+
+
+# ---- other outcome estimators ---------------------------------------------------------------------
+@pytest.mark.parametrize("batch_size,seq_len,num_groups,seed", GOLDEN["grpo_equivalence_grid"]["cases"])
+def test_rloo_loop_equals_vectorised_reference_grid(batch_size, seq_len, num_groups, seed):
+    # the same grid, generators and tolerance: tests/trainer/ppo/test_core_algos_on_cpu.py:222-259
+    torch.manual_seed(seed); random.seed(seed); np.random.seed(seed)
+    index = _make_group_index(batch_size, num_groups)
+    mask = _rand_mask(batch_size, seq_len)
+    rewards = torch.randn(batch_size, seq_len) * mask
+    a1, r1 = A.rloo_outcome_advantage(rewards, mask, index)
+    a2, r2 = A.rloo_vectorized_outcome_advantage(rewards, mask, index)
+    assert a1.shape == a2.shape == (batch_size, seq_len) and a1 is r1 and a2 is r2
+    assert torch.allclose(a1, a2, rtol=1e-5, atol=1e-6)
+
+
+def _scores_groups():
+    rewards = torch.tensor([[1.0, 2.0, 0.0], [0.5, 0.0, 0.0], [4.0, 1.0, 1.0], [0.0, 0.0, 0.0], [2.0, 2.0, 2.0]])
+    mask = torch.tensor([[1.0, 1.0, 0.0], [1.0, 0.0, 0.0], [1.0, 1.0, 1.0], [1.0, 1.0, 0.0], [1.0, 1.0, 1.0]])
+    index = np.array(["a", "a", "a", "b", "c"], dtype=object)      # sizes 3, 1, 1; scores 3, 0.5, 6 | 0 | 6
+    return rewards, mask, index
+
+
+def test_rloo_is_leave_one_out_mean_and_singleton_rules():
+    rewards, mask, index = _scores_groups()
+    adv, _ = A.rloo_outcome_advantage(rewards, mask, index)
+    s = [3.0, 0.5, 6.0]
+    for i in range(3):                                  # s_i minus the mean of the OTHER members
+        others = [s[j] for j in range(3) if j != i]
+        assert torch.allclose(adv[i], (s[i] - sum(others) / 2) * mask[i], atol=1e-6)
+    assert torch.equal(adv[3], torch.zeros(3)) and torch.equal(adv[4], 6.0 * mask[4])   # single member keeps its score
+    adv_v, _ = A.rloo_vectorized_outcome_advantage(rewards, mask, index)
+    assert torch.allclose(adv_v[:3], adv[:3], atol=1e-6) and torch.equal(adv_v[4], torch.zeros(3))   # ... or gets 0
+
+
+def test_opo_gpg_and_mean_baseline_by_hand():
+    rewards, mask, index = _scores_groups()
+    lens = [2.0, 1.0, 3.0]
+    bsl = (2 * 3.0 + 1 * 0.5 + 3 * 6.0) / 6.0
+    adv, _ = A.opo_outcome_advantage(rewards, mask, index)
+    for i, s in enumerate([3.0, 0.5, 6.0]):
+        assert torch.allclose(adv[i], (s - bsl) * mask[i], atol=1e-6)
+    assert torch.equal(adv[4], 6.0 * mask[4])           # single member: baseline 0
+    # GPG: alpha = 5 / #{scores != 0} = 5/4, mean of group a = 19/6, f_norm = 2
+    adv, _ = A.gpg_outcome_advantage(rewards, mask, index, f_norm=2.0)
+    for i, s in enumerate([3.0, 0.5, 6.0]):
+        assert torch.allclose(adv[i], 1.25 * (s - 19.0 / 6.0) / 2.0 * mask[i], atol=1e-6)
+    assert torch.allclose(adv[4], 1.25 * 6.0 / 2.0 * mask[4])
+    # REINFORCE++ baseline: centred scores on the mask, then masked whitening, then the mask again
+    adv, _ = A.reinforce_plus_plus_baseline_outcome_advantage(rewards, mask, index)
+    cen = torch.tensor([3.0 - 19 / 6, 0.5 - 19 / 6, 6.0 - 19 / 6, 0.0, 6.0])[:, None] * mask
+    sel = cen[mask.bool()]
+    want = (cen - sel.mean()) * torch.rsqrt(sel.var(unbiased=True) + 1e-8) * mask
+    assert torch.allclose(adv, want, atol=1e-5)
+    w = adv[mask.bool()]
+    assert abs(w.mean().item()) < 1e-6 and abs(w.var(unbiased=True).item() - 1) < 1e-5
+
+
+def test_reinforce_plus_plus_and_remax_closed_forms():
+    g = torch.Generator().manual_seed(3)
+    r = torch.randn(3, 17, generator=g, dtype=torch.float64)
+    ones = torch.ones(3, 17, dtype=torch.float64)
+    # all-ones mask: plain discounted return  R_t = sum_s gamma^(s-t) r_s
+    _, ret = A.reinforce_plus_plus_outcome_advantage(r, ones, 0.9)
+    want = torch.zeros_like(r)
+    for t in range(17):
+        want[:, t] = sum(0.9 ** (s - t) * r[:, s] for s in range(t, 17))
+    assert torch.allclose(ret, want, atol=1e-12)
+    # a masked step cuts the return: position 9 is the last one that sees anything from the right of it ... no:
+    # the running value is zeroed AFTER position 10 was written, so R_9 = r_9 and nothing to the right leaks in
+    m = ones.clone(); m[:, 10] = 0
+    adv, ret = A.reinforce_plus_plus_outcome_advantage(r, m, 0.9)
+    assert torch.allclose(ret[:, 9], r[:, 9]) and torch.allclose(ret[:, 10], want[:, 10])
+    assert torch.equal(adv[:, 10], torch.zeros(3, dtype=torch.float64))
+    sel = ret[m.bool()]
+    assert torch.allclose(adv, (ret - sel.mean()) * torch.rsqrt(sel.var(unbiased=True) + 1e-8) * m, atol=1e-10)
+    # gamma = 1, all-ones mask: REINFORCE++ returns == ReMax returns == reverse cumulative sum
+    _, r1 = A.reinforce_plus_plus_outcome_advantage(r, ones, 1.0)
+    base = torch.tensor([0.5, -1.0, 2.0], dtype=torch.float64)
+    adv2, r2 = A.remax_outcome_advantage(r, base, ones)
+    cum = torch.flip(torch.cumsum(torch.flip(r, [1]), 1), [1])
+    assert torch.allclose(r1, cum, atol=1e-12) and torch.allclose(r2, cum, atol=1e-12)
+    assert torch.allclose(adv2, cum - base[:, None], atol=1e-12)
+    # ReMax with a mask: masked rewards do not count, masked positions still show the carried sum
+    adv3, r3 = A.remax_outcome_advantage(r, base, m)
+    assert torch.allclose(r3[:, 10], r3[:, 11]) and torch.allclose(adv3[:, 10], r3[:, 10])

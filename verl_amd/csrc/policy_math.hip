@@ -94,6 +94,24 @@ __global__ __launch_bounds__(kRcThreads) void affine_kernel(const float* __restr
   store_groups<VEC>(out, pos, x);
 }
 
+// out = ((v - mean) * rstd + shift) * mask
+template <bool VEC, class M>
+__global__ __launch_bounds__(kRcThreads) void affine_masked_kernel(const float* __restrict__ values,
+                                                                   const float* __restrict__ stats,
+                                                                   const M* __restrict__ mask, int64_t n,
+                                                                   float* __restrict__ out) {
+  const float mean = stats[0], rstd = stats[1], shift = stats[2];
+  const ChunkPos pos(0, blockIdx.x, n);
+  float x[kGroups][4], w[kGroups][4];
+  load_groups<VEC>(values, pos, x);
+  load_mask_groups<VEC>(mask, pos, w);
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[g][e] = ((x[g][e] - mean) * rstd + shift) * w[g][e];
+  store_groups<VEC>(out, pos, x);
+}
+
 // =============================================================================================
 // agg_loss forward / backward
 // =============================================================================================
@@ -414,6 +432,9 @@ struct GrpoArgs {
   int64_t rows, n_groups;
   float eps;
   int norm_by_std, std_mode;
+  int estimator;            // VAMD_ADV_*
+  float f_norm;             // GPG
+  const double* row_moments;  // OPO: [rows][4] per-row masked moments, slot 0 = response length
   float* scores;   // [rows] scratch
   float* scalars;  // [rows] out: normalised scalar per response
   float* mean;     // [n_groups] (only used by the large-group-count path)
@@ -421,7 +442,14 @@ struct GrpoArgs {
 };
 
 // Row sums of the rewards (the mask is NOT applied, core_algos.py:303); the last workgroup turns
-// them into scores, per-group mean / std and the per-response scalar.
+// them into scores, per-group statistics and the per-response scalar of the chosen estimator:
+//   GRPO             (s - mean) / (std + eps)  or  s - mean             core_algos.py:266-330
+//   RLOO             s n/(n-1) - mean n/(n-1); a single-member group keeps s      :479-528
+//   RLOO_VECTORIZED  the same, a single-member group gets 0                       :720-753
+//   MEAN_BASELINE    s - mean (REINFORCE++ baseline before its whitening)         :421-474
+//   OPO              s - sum(len s) / sum(len), len = response length             :531-579
+//   GPG              alpha (s - mean) / f_norm, alpha = rows / max(#{s != 0}, 1)  :657-717
+// A single-member group has mean 0 (and std 1) in every estimator.
 // std_mode 0: unbiased torch.std; 1: sqrt(clamp(var, min=eps)) of group_mean_std.  Singleton
 // groups get mean 0, std 1 (core_algos.py:314-316, groupwise.py:215-221).
 template <bool VEC>
@@ -451,33 +479,80 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rowsum_kernel(const float* __
     g_sq[g] = 0.0;
   }
   __syncthreads();
+  const bool opo = ga.estimator == VAMD_ADV_OPO;
+  double nnz_local = 0;
   for (int64_t r = threadIdx.x; r < ga.rows; r += kRcThreads) {
     double t = 0;
     for (int c = 0; c < chunks; ++c) t += peer_load(wk.partials + r * chunks + c);
     const float sc = (float)t;
     ga.scores[r] = sc;
+    nnz_local += sc != 0.f ? 1.0 : 0.0;
     const int64_t g = ga.gid[r];
     atomicAdd(&g_cnt[g], 1);
-    atomicAdd(&g_sum[g], (double)sc);
+    if (opo) {  // g_sum: sum(len * s), g_sq: sum(len)
+      const double len = ga.row_moments[r * 4];
+      atomicAdd(&g_sum[g], len * (double)sc);
+      atomicAdd(&g_sq[g], len);
+    } else {
+      atomicAdd(&g_sum[g], (double)sc);
+    }
   }
   __syncthreads();
-  for (int64_t r = threadIdx.x; r < ga.rows; r += kRcThreads) {
-    const int64_t g = ga.gid[r];
-    const double d = (double)ga.scores[r] - g_sum[g] / (double)g_cnt[g];
-    atomicAdd(&g_sq[g], d * d);
+  if (ga.estimator == VAMD_ADV_GRPO) {
+    for (int64_t r = threadIdx.x; r < ga.rows; r += kRcThreads) {
+      const int64_t g = ga.gid[r];
+      const double d = (double)ga.scores[r] - g_sum[g] / (double)g_cnt[g];
+      atomicAdd(&g_sq[g], d * d);
+    }
+    __syncthreads();
   }
-  __syncthreads();
+  float alpha = 1.f;
+  if (ga.estimator == VAMD_ADV_GPG) {
+    __shared__ double nz_smem[4];
+    __shared__ float alpha_bc;
+    double acc1[1] = {nnz_local};
+    block_sum<1, kRcThreads>(acc1, nz_smem);
+    if (threadIdx.x == 0) alpha_bc = (float)ga.rows / fmaxf((float)acc1[0], 1.f);
+    __syncthreads();
+    alpha = alpha_bc;
+  }
   for (int64_t r = threadIdx.x; r < ga.rows; r += kRcThreads) {
     const int64_t g = ga.gid[r];
     const int c = g_cnt[g];
-    float mu = 0.f, sd = 1.f;
-    if (c > 1) {
-      const double var = g_sq[g] / (double)(c - 1);
-      mu = (float)(g_sum[g] / (double)c);
-      sd = ga.std_mode == 0 ? (float)sqrt(var) : sqrtf(fmaxf((float)var, ga.eps));
+    const float sc = ga.scores[r];
+    float out;
+    switch (ga.estimator) {
+      case VAMD_ADV_GRPO: {
+        float mu = 0.f, sd = 1.f;
+        if (c > 1) {
+          const double var = g_sq[g] / (double)(c - 1);
+          mu = (float)(g_sum[g] / (double)c);
+          sd = ga.std_mode == 0 ? (float)sqrt(var) : sqrtf(fmaxf((float)var, ga.eps));
+        }
+        const float cen = sc - mu;
+        out = ga.norm_by_std ? cen / (sd + ga.eps) : cen;
+      } break;
+      case VAMD_ADV_RLOO:
+      case VAMD_ADV_RLOO_VECTORIZED: {
+        if (c > 1) {
+          const float mu = (float)(g_sum[g] / (double)c);
+          const float n = (float)c, n1 = (float)(c - 1);
+          out = sc * n / n1 - mu * n / n1;
+        } else {
+          out = ga.estimator == VAMD_ADV_RLOO ? sc : 0.f;
+        }
+      } break;
+      case VAMD_ADV_OPO:
+        out = c > 1 ? sc - (float)(g_sum[g] / g_sq[g]) : sc;
+        break;
+      case VAMD_ADV_GPG:
+        out = alpha * (sc - (c > 1 ? (float)(g_sum[g] / (double)c) : 0.f)) / ga.f_norm;
+        break;
+      default:  // VAMD_ADV_MEAN_BASELINE
+        out = sc - (c > 1 ? (float)(g_sum[g] / (double)c) : 0.f);
+        break;
     }
-    const float cen = ga.scores[r] - mu;
-    ga.scalars[r] = ga.norm_by_std ? cen / (sd + ga.eps) : cen;
+    ga.scalars[r] = out;
   }
   ticket_reset(wk.ticket);
 }
@@ -631,6 +706,21 @@ extern "C" int vamd_affine_by_stats(const float* values, const float* stats, int
   hipStream_t s = static_cast<hipStream_t>(stream);
   VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((affine_kernel<V>), grid, dim3(kRcThreads), 0, s, values, stats, n,
                                                out));
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
+
+extern "C" int vamd_affine_by_stats_masked(const float* values, const float* stats, const void* mask, int mask_dtype,
+                                           int64_t n, float* out, void* stream) {
+  VAMD_REQUIRE(values && stats && mask && out && n > 0, "affine_by_stats_masked: bad argument");
+  VAMD_REQUIRE(chunks_of(n) < (1ll << 31), "affine_by_stats_masked: too many elements");
+  const dim3 grid((unsigned)chunks_of(n));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  VAMD_MASK_DISPATCH(mask_dtype, M, {
+    const bool vec = can_vectorize(n, {values, out}, mask, sizeof(M));
+    VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((affine_masked_kernel<V, M>), grid, dim3(kRcThreads), 0, s, values,
+                                                 stats, static_cast<const M*>(mask), n, out));
+  });
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }
@@ -854,21 +944,49 @@ extern "C" int vamd_group_mean_std(const float* scores, const int64_t* group_ids
   return VAMD_OK;
 }
 
+extern "C" size_t vamd_group_outcome_advantage_workspace_bytes(int64_t batch, int64_t length, int64_t n_groups) {
+  if (batch <= 0 || length <= 0 || n_groups <= 0) return 0;
+  // sized for the estimator that needs most: OPO runs a per-row moments pass (4 doubles per workgroup) first
+  return vamd_grpo_workspace_bytes(batch, length, n_groups) - reduce_workspace_bytes(batch, length, 1) +
+         reduce_workspace_bytes(batch, length, 4) + align_up((size_t)batch * 4 * sizeof(double), 256);
+}
+
 extern "C" int vamd_grpo_advantage(const float* rewards, const void* mask, int mask_dtype, const int64_t* group_ids,
                                    int64_t batch, int64_t length, int64_t n_groups, float epsilon, int norm_by_std,
                                    int std_mode, float* advantages, float* scores_out, void* workspace,
                                    size_t workspace_bytes, void* stream) {
-  int st = check_matrix("grpo", batch, length);
-  if (st != VAMD_OK) return st;
-  VAMD_REQUIRE(rewards && mask && group_ids && advantages && n_groups > 0, "grpo: bad argument");
   if (!workspace || workspace_bytes < vamd_grpo_workspace_bytes(batch, length, n_groups)) {
     set_error("grpo: workspace too small");
+    return VAMD_EWORKSPACE;
+  }
+  // GRPO uses neither the wider partial records nor the per-row moments the general query reserves room for
+  return vamd_group_outcome_advantage(rewards, mask, mask_dtype, group_ids, batch, length, n_groups, VAMD_ADV_GRPO,
+                                      epsilon, norm_by_std, std_mode, 1.f, advantages, scores_out, workspace,
+                                      vamd_group_outcome_advantage_workspace_bytes(batch, length, n_groups), stream);
+}
+
+extern "C" int vamd_group_outcome_advantage(const float* rewards, const void* mask, int mask_dtype,
+                                            const int64_t* group_ids, int64_t batch, int64_t length,
+                                            int64_t n_groups, int estimator, float epsilon, int norm_by_std,
+                                            int std_mode, float f_norm, float* advantages, float* scores_out,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+  int st = check_matrix("group_outcome_advantage", batch, length);
+  if (st != VAMD_OK) return st;
+  VAMD_REQUIRE(rewards && mask && group_ids && advantages && n_groups > 0, "group_outcome_advantage: bad argument");
+  VAMD_REQUIRE(estimator >= VAMD_ADV_GRPO && estimator <= VAMD_ADV_GPG, "group_outcome_advantage: invalid estimator %d",
+               estimator);
+  VAMD_REQUIRE(estimator == VAMD_ADV_GRPO || n_groups <= kGrpoLdsGroups,
+               "group_outcome_advantage: estimators other than GRPO support at most %d groups", kGrpoLdsGroups);
+  VAMD_REQUIRE(estimator != VAMD_ADV_GPG || f_norm != 0.f, "group_outcome_advantage: f_norm must not be 0");
+  if (!workspace || workspace_bytes < vamd_group_outcome_advantage_workspace_bytes(batch, length, n_groups)) {
+    set_error("group_outcome_advantage: workspace too small");
     return VAMD_EWORKSPACE;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int chunks = (int)chunks_of(length);
   const Work wk = carve_work(workspace);
-  Carver carve(static_cast<char*>(workspace) + reduce_workspace_bytes(batch, length, 1));
+  const bool opo = estimator == VAMD_ADV_OPO;
+  Carver carve(static_cast<char*>(workspace) + reduce_workspace_bytes(batch, length, opo ? 4 : 1));
   GrpoArgs ga;
   ga.gid = group_ids;
   ga.rows = batch;
@@ -876,11 +994,21 @@ extern "C" int vamd_grpo_advantage(const float* rewards, const void* mask, int m
   ga.eps = epsilon;
   ga.norm_by_std = norm_by_std;
   ga.std_mode = std_mode;
+  ga.estimator = estimator;
+  ga.f_norm = f_norm;
   ga.scores = carve.take<float>((size_t)batch);
   float* scalars = carve.take<float>((size_t)batch);
   ga.scalars = scores_out ? scores_out : scalars;
   ga.mean = carve.take<float>((size_t)n_groups);
   ga.stdv = carve.take<float>((size_t)n_groups);
+  ga.row_moments = nullptr;
+  if (opo) {  // response lengths: per-row masked moments of the rewards, slot 0 = sum(mask)
+    double* row_moments = carve.take<double>((size_t)batch * 4);
+    ga.row_moments = row_moments;
+    st = vamd_masked_moments(rewards, mask, mask_dtype, batch, length, 1, row_moments, workspace,
+                             reduce_workspace_bytes(batch, length, 4), stream);
+    if (st != VAMD_OK) return st;
+  }
   {
     const bool vec = can_vectorize(length, {rewards}, nullptr, 0);
     VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((grpo_rowsum_kernel<V>), dim3((unsigned)(batch * chunks)),

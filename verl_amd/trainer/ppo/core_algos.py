@@ -46,8 +46,9 @@ def get_policy_loss_fn(name):
 
 
 class AdvantageEstimator(str, Enum):
-    """Names of the reference's advantage estimators (core_algos.py:88-109); only GAE, GRPO and
-    GRPO_VECTORIZED are implemented here, the other names exist so configs keep parsing."""
+    """Names of the reference's advantage estimators (core_algos.py:88-109).  GRPO_PASSK and the two
+    optimal-token-baseline estimators are not implemented here; their names exist so configs keep
+    parsing, and looking them up raises the reference's "unknown estimator" error."""
 
     GAE = "gae"
     GRPO = "grpo"
@@ -181,6 +182,125 @@ def compute_grpo_vectorized_outcome_advantage(token_level_rewards: torch.Tensor,
                                               norm_adv_by_std_in_grpo: bool = True, config: Optional[Any] = None):
     """Vectorised twin (reference core_algos.py:333-357): std = sqrt(clamp(var, min=epsilon))."""
     return _grpo(token_level_rewards, response_mask, index, epsilon, norm_adv_by_std_in_grpo, std_mode=1)
+
+
+# ---- the other outcome estimators of the registry ----------------------------------------------
+_ADV = {"grpo": 0, "rloo": 1, "rloo_vectorized": 2, "mean_baseline": 3, "opo": 4, "gpg": 5}
+
+
+def _group_outcome(token_level_rewards, response_mask, index, estimator: str, epsilon=1e-6, f_norm=1.0,
+                   whiten_after=False):
+    """Score per response -> statistic of its prompt group -> one scalar per response -> scalar * mask
+    (``vamd_group_outcome_advantage``); ``whiten_after`` adds ``masked_whiten(.) * mask``."""
+    with torch.no_grad():
+        dev = _cabi.compute_device(token_level_rewards, response_mask)
+        r = _matrix(token_level_rewards, dev)
+        m, code = _mask_matrix(response_mask, dev, r.shape)
+        B, Lc = r.shape
+        ids, G = contiguous_group_ids(index)
+        if ids.numel() != B:
+            raise ValueError(f"index has {ids.numel()} entries for a batch of {B}")
+        ids = ids.to(dev)
+        adv = torch.empty_like(r)
+        Lb = _cabi.lib()
+        ws = _cabi.ticket_workspace(Lb.vamd_group_outcome_advantage_workspace_bytes(B, Lc, G), dev)
+        with torch.cuda.device(dev):
+            s = _cabi.stream_ptr(dev)
+            _cabi.check(Lb.vamd_group_outcome_advantage(r.data_ptr(), m.data_ptr(), code, ids.data_ptr(), B, Lc, G,
+                                                        _ADV[estimator], float(epsilon), 1, 0, float(f_norm),
+                                                        adv.data_ptr(), None, ws.data_ptr(), ws.numel(), s))
+            if whiten_after:
+                mom = verl_F._moments(adv, m, per_row=False)
+                verl_F._raise_on_tiny_mask(float(mom[0].item()))
+                stats = torch.empty(4, dtype=torch.float32, device=dev)
+                _cabi.check(Lb.vamd_whiten_stats(mom.data_ptr(), 1, stats.data_ptr(), s))
+                _cabi.check(Lb.vamd_affine_by_stats_masked(adv.data_ptr(), stats.data_ptr(), m.data_ptr(), code,
+                                                           adv.numel(), adv.data_ptr(), s))
+        out = adv.view(token_level_rewards.shape).to(token_level_rewards.device)
+        return out, out
+
+
+@register_adv_est(AdvantageEstimator.REINFORCE_PLUS_PLUS_BASELINE)
+def compute_reinforce_plus_plus_baseline_outcome_advantage(token_level_rewards: torch.Tensor,
+                                                           response_mask: torch.Tensor, index, epsilon: float = 1e-6,
+                                                           config: Optional[Any] = None, **kwargs):
+    """REINFORCE++ with a group-mean baseline (reference core_algos.py:421-474): score minus the
+    mean of its prompt group (0 for a single member), on the mask, whitened over all valid tokens,
+    on the mask again.  Returns one tensor twice."""
+    return _group_outcome(token_level_rewards, response_mask, index, "mean_baseline", epsilon, whiten_after=True)
+
+
+@register_adv_est(AdvantageEstimator.RLOO)
+def compute_rloo_outcome_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor, index,
+                                   epsilon: float = 1e-6, config: Optional[Any] = None, **kwargs):
+    """Leave-one-out baseline (reference core_algos.py:479-528); a single-member group keeps its score."""
+    return _group_outcome(token_level_rewards, response_mask, index, "rloo", epsilon)
+
+
+@register_adv_est(AdvantageEstimator.RLOO_VECTORIZED)
+def compute_rloo_vectorized_outcome_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor, index,
+                                              epsilon: float = 1e-6, config: Optional[Any] = None, **kwargs):
+    """Vectorised RLOO (reference core_algos.py:720-753); a single-member group gets 0."""
+    return _group_outcome(token_level_rewards, response_mask, index, "rloo_vectorized", epsilon)
+
+
+@register_adv_est(AdvantageEstimator.OPO)
+def compute_opo_outcome_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor, index,
+                                  epsilon: float = 1e-6, config: Optional[Any] = None, **kwargs):
+    """Length-weighted group baseline (reference core_algos.py:531-579)."""
+    return _group_outcome(token_level_rewards, response_mask, index, "opo", epsilon)
+
+
+@register_adv_est(AdvantageEstimator.GPG)
+def compute_gpg_outcome_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor, index,
+                                  epsilon: float = 1e-6, f_norm: float = 1.0, alpha: float = 1.0, config=None,
+                                  **kwargs):
+    """GPG (reference core_algos.py:657-717): ``alpha (score - group mean) / f_norm`` where ``alpha`` is
+    recomputed as ``batch / max(#{score != 0}, 1)`` whatever the argument says, as there (:697-698)."""
+    return _group_outcome(token_level_rewards, response_mask, index, "gpg", epsilon, f_norm=f_norm)
+
+
+def _returns_advantage(token_level_rewards, response_mask, mode: int, gamma: float, baselines=None):
+    with torch.no_grad():
+        dev = _cabi.compute_device(token_level_rewards, response_mask)
+        r = _matrix(token_level_rewards, dev)
+        m, code = _mask_matrix(response_mask, dev, r.shape)
+        B, Lc = r.shape
+        base = None
+        if baselines is not None:
+            base = _cabi.as_f32(baselines, dev).reshape(-1).contiguous()
+            assert base.numel() == B, f"reward_baselines has {base.numel()} entries for a batch of {B}"
+        adv = torch.empty_like(r)
+        ret = torch.empty_like(r)
+        mom = torch.empty(4, dtype=torch.float64, device=dev)
+        Lb = _cabi.lib()
+        ws = _cabi.ticket_workspace(Lb.vamd_returns_advantage_workspace_bytes(B, Lc), dev)
+        with torch.cuda.device(dev):
+            _cabi.check(Lb.vamd_returns_advantage(r.data_ptr(), m.data_ptr(), code, _cabi.ptr(base), B, Lc,
+                                                  float(gamma), mode, adv.data_ptr(), ret.data_ptr(), mom.data_ptr(),
+                                                  ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
+        if mode == 1:
+            verl_F._raise_on_tiny_mask(float(mom[0].item()))
+        shape, out_dev = token_level_rewards.shape, token_level_rewards.device
+        return adv.view(shape).to(out_dev), ret.view(shape).to(out_dev)
+
+
+@register_adv_est(AdvantageEstimator.REINFORCE_PLUS_PLUS)
+def compute_reinforce_plus_plus_outcome_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor,
+                                                  config: Optional[Any] = None, **kwargs):
+    """REINFORCE++ (reference core_algos.py:582-618): discounted return that restarts after a masked
+    step, whitened over the valid tokens and masked.  ``config.gamma`` is required, as there.
+    Returns ``(advantages, returns)``."""
+    assert config is not None
+    return _returns_advantage(token_level_rewards, response_mask, 1, float(config.gamma))
+
+
+@register_adv_est(AdvantageEstimator.REMAX)
+def compute_remax_outcome_advantage(token_level_rewards: torch.Tensor, reward_baselines: torch.Tensor,
+                                    response_mask: torch.Tensor, config: Optional[Any] = None, **kwargs):
+    """ReMax (reference core_algos.py:621-654): reverse cumulative sum of the masked rewards minus the
+    greedy-rollout baseline of the response on its mask.  Returns ``(advantages, returns)``."""
+    return _returns_advantage(token_level_rewards, response_mask, 0, 1.0, baselines=reward_baselines)
 
 
 # ---------------------------------------------------------------------------------------------
