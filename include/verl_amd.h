@@ -60,6 +60,13 @@ extern "C" {
 #define VAMD_ADV_OPO 4             /* s - sum(len s) / sum(len), len = response length */
 #define VAMD_ADV_GPG 5             /* alpha (s - mean) / f_norm, alpha = batch / max(#{s != 0}, 1) */
 
+/* policy-loss variants of the registry (core_algos.py:1159-1447, :1721-1779) */
+#define VAMD_PL_VANILLA 0 /* clipped PPO with the dual-clip floor */
+#define VAMD_PL_GPG 1     /* -log_prob A */
+#define VAMD_PL_CISPO 2   /* -sg(clip(ratio)) A log_prob */
+#define VAMD_PL_SAPO 3    /* -4/tau sigmoid(tau (ratio - 1)) A, tau by the sign of A */
+#define VAMD_PL_GSPO 4    /* clipped objective on the sequence-level importance ratio */
+
 /* token-level return recurrences (core_algos.py:582-654) */
 #define VAMD_RETURNS_REMAX 0        /* returns = reverse cumsum of r m; adv = returns - baseline_i m */
 #define VAMD_RETURNS_REINFORCE_PP 1 /* R_t = r_t + gamma c, c <- R_t m_t; adv = masked_whiten(R, m) m */
@@ -225,6 +232,19 @@ int vamd_policy_loss_forward(const float* old_log_prob, const float* log_prob, c
                              double batch_num_tokens, double global_batch_size, double loss_scale_factor,
                              float* out, float* grad_unscaled, float* coef_out, void* workspace,
                              size_t workspace_bytes, void* stream);
+/* The same pass for the other registered policy losses.  out[0..3] as above with the counters a variant
+ * does not define left at 0 (GPG: all three; SAPO: both clip fractions; CISPO / GSPO:
+ * pg_clipfrac_lower); ppo_kl of GSPO averages the unclamped log-ratio, as the reference does.  tau_pos /
+ * tau_neg are SAPO's; clip_c is only read by VAMD_PL_VANILLA.  GSPO runs a per-row pass over
+ * log_prob - old_log_prob first (its sequence-level ratio). */
+size_t vamd_policy_loss_variant_workspace_bytes(int64_t rows, int64_t cols);
+int vamd_policy_loss_variant_forward(int variant, const float* old_log_prob, const float* log_prob,
+                                     const float* advantages, const void* mask, int mask_dtype,
+                                     const float* is_weights, int64_t rows, int64_t cols, float clip_low,
+                                     float clip_high, float clip_c, float tau_pos, float tau_neg, int mode,
+                                     double dp_size, double batch_num_tokens, double global_batch_size,
+                                     double loss_scale_factor, float* out, float* grad_unscaled, float* coef_out,
+                                     void* workspace, size_t workspace_bytes, void* stream);
 int vamd_scale_rows(const float* g, const float* coef, const float* d_loss, float extra_scale, int64_t rows,
                     int64_t cols, float* out, void* stream);
 

@@ -55,4 +55,8 @@ from .losses import (  # noqa: F401
     kl_penalty_forward,
     kl_penalty,
     kl_straight_through,
+    policy_loss_gspo,
+    policy_loss_sapo,
+    policy_loss_gpg,
+    policy_loss_cispo,
 )

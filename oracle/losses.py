@@ -111,3 +111,67 @@ def kl_straight_through(logprob, ref_logprob, forward_score):
     """core_algos.py:1861-1866: value of ``forward_score``, gradient of k2."""
     backward_score = 0.5 * (logprob - ref_logprob).square()
     return backward_score - backward_score.detach() + forward_score.detach()
+
+
+# ---- other registered policy losses ------------------------------------------------------------
+def policy_loss_gspo(old_log_prob, log_prob, advantages, response_mask, clip_ratio_low=0.2, clip_ratio_high=0.2,
+                     rollout_is_weights=None, global_batch_info=None):
+    """GSPO, verl/trainer/ppo/core_algos.py:1253-1326: sequence-level ratio from the masked mean of the
+    token log-ratios (length clamped to >= 1), token-level gradient through ``log_prob - log_prob.detach()``,
+    log-ratio clamped at 10, clipped objective, always "seq-mean-token-mean".  Returns
+    ``(pg_loss, pg_clipfrac, ppo_kl, pg_clipfrac_lower = 0)``."""
+    d = log_prob - old_log_prob
+    lengths = torch.sum(response_mask, dim=-1).clamp(min=1)
+    seq = torch.sum(d * response_mask, dim=-1) / lengths
+    log_ratio = torch.clamp(log_prob - log_prob.detach() + seq.detach().unsqueeze(-1), max=10.0)
+    ratio = torch.exp(log_ratio)
+    l1 = -advantages * ratio
+    l2 = -advantages * torch.clamp(ratio, 1 - clip_ratio_low, 1 + clip_ratio_high)
+    losses = torch.maximum(l1, l2)
+    if rollout_is_weights is not None:
+        losses = losses * rollout_is_weights
+    pg_loss = agg_loss(losses, response_mask, "seq-mean-token-mean", **(global_batch_info or {}))
+    pg_clipfrac = masked_mean(torch.gt(l2, l1).float(), response_mask)
+    ppo_kl = masked_mean(-d, response_mask)
+    return pg_loss, pg_clipfrac, ppo_kl, torch.tensor(0.0)
+
+
+def policy_loss_sapo(old_log_prob, log_prob, advantages, response_mask, tau_pos, tau_neg,
+                     rollout_is_weights=None, global_batch_info=None):
+    """SAPO, core_algos.py:1329-1411: gate ``sigmoid(tau (ratio - 1)) 4 / tau`` with tau chosen by the sign of
+    the advantage, always "seq-mean-token-mean".  Returns ``(pg_loss, 0, ppo_kl, 0)``."""
+    tp = torch.as_tensor(tau_pos, dtype=advantages.dtype)
+    tn = torch.as_tensor(tau_neg, dtype=advantages.dtype)
+    k = torch.clamp(log_prob - old_log_prob, min=-20.0, max=20.0)
+    ratio = torch.exp(k)
+    taus = torch.where(advantages > 0, tp, tn)
+    gates = torch.sigmoid(taus * (ratio - 1.0)) * (4.0 / taus)
+    losses = -gates * advantages
+    if rollout_is_weights is not None:
+        losses = losses * rollout_is_weights
+    pg_loss = agg_loss(losses, response_mask, "seq-mean-token-mean", **(global_batch_info or {}))
+    return pg_loss, torch.tensor(0.0), masked_mean(-k, response_mask), torch.tensor(0.0)
+
+
+def policy_loss_gpg(log_prob, advantages, response_mask, loss_agg_mode="token-mean", rollout_is_weights=None,
+                    global_batch_info=None):
+    """GPG, core_algos.py:1414-1447: ``agg_loss(-log_prob * advantages)``; the reference returns no metrics."""
+    losses = -log_prob * advantages
+    if rollout_is_weights is not None:
+        losses = losses * rollout_is_weights
+    return agg_loss(losses, response_mask, loss_agg_mode, **(global_batch_info or {}))
+
+
+def policy_loss_cispo(old_log_prob, log_prob, advantages, response_mask, loss_agg_mode="token-mean",
+                      clip_ratio_low=0.2, clip_ratio_high=0.2, rollout_is_weights=None, global_batch_info=None):
+    """CISPO, core_algos.py:1721-1779: ``-sg(clamp(ratio)) * A * log_prob``; pg_clipfrac counts the tokens whose
+    ratio the clamp changed.  Returns ``(pg_loss, pg_clipfrac, ppo_kl, 0)``."""
+    k = torch.clamp(log_prob - old_log_prob, min=-20.0, max=20.0)
+    ratio = torch.exp(k)
+    clipped = torch.clamp(ratio, 1 - clip_ratio_low, 1 + clip_ratio_high)
+    losses = -clipped.detach() * advantages * log_prob
+    pg_clipfrac = masked_mean((ratio != clipped).float(), response_mask)
+    if rollout_is_weights is not None:
+        losses = losses * rollout_is_weights
+    pg_loss = agg_loss(losses, response_mask, loss_agg_mode, **(global_batch_info or {}))
+    return pg_loss, pg_clipfrac, masked_mean(-k, response_mask), torch.tensor(0.0)

@@ -442,6 +442,45 @@ def test_reinforce_plus_plus_and_remax(dev, shape, mdtype):
     assert CA.get_adv_estimator_fn("remax") is CA.compute_remax_outcome_advantage
 
 
+# ---- the other registered policy losses -----------------------------------------------------------------
+@pytest.mark.parametrize("variant", ["gpg", "cispo", "sapo", "gspo"])
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("with_isw", [False, True])
+def test_policy_loss_variants(dev, variant, mode, with_isw):
+    from verl_amd.trainer.ppo import core_algos as CA
+    g = torch.Generator().manual_seed(len(variant) * 7 + len(mode))
+    B, Lc = 12, 4200                                            # two column chunks with a ragged tail
+    mask, _ = _prefix_mask(B, Lc, g, lo=3)
+    mask[2] = 0                                                 # an empty response
+    old = torch.randn(B, Lc, generator=g) * 0.5 - 1
+    new = old + torch.randn(B, Lc, generator=g) * 0.2
+    new[0, 0] = old[0, 0] + 25.0                                # beyond the clamp of the log-ratio
+    new[1] = old[1] + 0.6                                       # a whole sequence outside GSPO's clip range
+    adv = torch.randn(B, Lc, generator=g)
+    isw = (torch.rand(B, Lc, generator=g) + 0.5) if with_isw else None
+    cfg = _cfg(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28, tau_pos=1.0, tau_neg=1.05)
+    nd = new.to(dev).requires_grad_(); no = new.clone().requires_grad_()
+    fn = getattr(CA, "compute_policy_loss_" + variant)
+    assert CA.get_policy_loss_fn(variant) is fn
+    loss, met = fn(old.to(dev), nd, adv.to(dev), mask.to(dev), mode, cfg, None if isw is None else isw.to(dev))
+    if variant == "gpg":
+        want = (O.policy_loss_gpg(no, adv, mask, mode, isw),)
+        assert met == {}
+    elif variant == "cispo":
+        want = O.policy_loss_cispo(old, no, adv, mask, mode, 0.2, 0.28, isw)
+    elif variant == "sapo":
+        want = O.policy_loss_sapo(old, no, adv, mask, 1.0, 1.05, isw)
+    else:
+        want = O.policy_loss_gspo(old, no, adv, mask, 0.2, 0.28, isw)
+    _close(loss, want[0], what=f"{variant} loss ({mode})")
+    if variant != "gpg":
+        assert abs(met["actor/pg_clipfrac"] - want[1].item()) < 1e-6, (met, want[1])
+        assert abs(met["actor/ppo_kl"] - want[2].item()) < 2e-6 * max(1.0, abs(want[2].item())), (met, want[2])
+        assert met["actor/pg_clipfrac_lower"] == 0.0
+    _close(torch.autograd.grad(loss * 2.0, nd)[0], torch.autograd.grad(want[0] * 2.0, no)[0], atol=1e-9,
+           what=f"d {variant} loss / d log_prob")
+
+
 # ---- KL penalty -------------------------------------------------------------------------------------
 @pytest.mark.parametrize("kind", ["kl", "k1", "abs", "mse", "k2", "low_var_kl", "k3"])
 def test_kl_penalty_elementwise(dev, kind):

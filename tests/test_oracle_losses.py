@@ -193,3 +193,55 @@ def test_kl_penalty_as_written_and_straight_through():
     want = 1 - torch.exp((b - a).detach())
     want[3] = 0.0                                   # ref - lp = 28 is clamped to 20: no gradient
     assert torch.allclose(g, want)
+
+
+def _policy_inputs(seed=0, B=4, Lc=9, dtype=torch.float64):
+    g = torch.Generator().manual_seed(seed)
+    old = torch.randn(B, Lc, generator=g, dtype=dtype) * 0.5 - 1
+    new = (old + torch.randn(B, Lc, generator=g, dtype=dtype) * 0.3).requires_grad_()
+    adv = torch.randn(B, Lc, generator=g, dtype=dtype)
+    mask = (torch.rand(B, Lc, generator=g) < 0.8).to(dtype)
+    mask[:, 0] = 1
+    return old, new, adv, mask
+
+
+def test_policy_loss_variants_closed_forms():
+    """Each variant against a scalar loop of its published formula, and its gradient against the hand derivative."""
+    old, new, adv, mask = _policy_inputs()
+    B, Lc = old.shape
+    # GPG: token-mean of -lp A; d/dlp = -A m / M
+    loss = L.policy_loss_gpg(new, adv, mask)
+    M_ = mask.sum()
+    assert torch.allclose(loss, (-(new * adv) * mask).sum() / M_)
+    g, = torch.autograd.grad(loss, new)
+    assert torch.allclose(g, -adv * mask / M_)
+    # CISPO: the clipped ratio is a constant factor
+    loss, cf, kl, _ = L.policy_loss_cispo(old, new, adv, mask, clip_ratio_low=0.2, clip_ratio_high=0.3)
+    r = torch.exp(new.detach() - old)
+    rc = r.clamp(0.8, 1.3)
+    assert torch.allclose(loss, (-(rc * adv * new.detach()) * mask).sum() / M_)
+    g, = torch.autograd.grad(loss, new)
+    assert torch.allclose(g, -rc * adv * mask / M_)
+    assert torch.allclose(cf, (((r < 0.8) | (r > 1.3)).double() * mask).sum() / (M_ + 1e-8))
+    assert torch.allclose(kl, (-(new.detach() - old) * mask).sum() / (M_ + 1e-8))
+    # SAPO: seq-mean-token-mean of -(4/tau) sigmoid(tau (r - 1)) A;  d/dlp = -4 A s (1 - s) r
+    loss, _, _, _ = L.policy_loss_sapo(old, new, adv, mask, tau_pos=1.0, tau_neg=1.05)
+    tau = torch.where(adv > 0, torch.tensor(1.0, dtype=torch.float64), torch.tensor(1.05, dtype=torch.float64))
+    sgm = torch.sigmoid(tau * (r - 1))
+    per_tok = -(4 / tau) * sgm * adv
+    rows = (per_tok * mask).sum(-1) / (mask.sum(-1) + 1e-8)
+    assert torch.allclose(loss, rows.mean())
+    g, = torch.autograd.grad(loss, new)
+    assert torch.allclose(g, (-4 * adv * sgm * (1 - sgm) * r) * mask / (mask.sum(-1, keepdim=True) + 1e-8) / B)
+    # GSPO: one ratio per sequence; with identical advantages along a row and no clipping the row loss is -A s_i
+    seq = ((new.detach() - old) * mask).sum(-1) / mask.sum(-1)
+    adv_row = adv[:, :1].expand(B, Lc).contiguous()
+    loss, cf, kl, low = L.policy_loss_gspo(old, new, adv_row, mask, clip_ratio_low=10.0, clip_ratio_high=10.0)
+    assert torch.allclose(loss, (-adv_row[:, 0] * torch.exp(seq)).mean()) and cf.item() == 0 and low.item() == 0
+    g, = torch.autograd.grad(loss, new)                # d/dlp_t = -A exp(s_i) m_t / M_i / B : token-level gradient
+    assert torch.allclose(g, (-adv_row * torch.exp(seq)[:, None]) * mask / (mask.sum(-1, keepdim=True) + 1e-8) / B)
+    # tight clip range: every token of a row with s_i outside the range and the "wrong" sign of A is clipped
+    loss, cf, _, _ = L.policy_loss_gspo(old, new, adv, mask, clip_ratio_low=1e-4, clip_ratio_high=1e-4)
+    rr = torch.exp(seq)[:, None].expand(B, Lc)
+    l1 = -adv * rr; l2 = -adv * rr.clamp(1 - 1e-4, 1 + 1e-4)
+    assert torch.allclose(cf, ((l2 > l1).double() * mask).sum() / (M_ + 1e-8))

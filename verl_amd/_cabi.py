@@ -67,6 +67,11 @@ SIGNATURES = {
     "vamd_policy_loss_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64,
                                          c_float, c_float, c_float, c_int, c_double, c_double, c_double, c_double,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "vamd_policy_loss_variant_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "vamd_policy_loss_variant_forward": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64,
+                                                 c_int64, c_float, c_float, c_float, c_float, c_float, c_int,
+                                                 c_double, c_double, c_double, c_double, c_void_p, c_void_p,
+                                                 c_void_p, c_void_p, c_size_t, c_void_p]),
     "vamd_scale_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int64, c_void_p, c_void_p]),
     "vamd_kl_penalty": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "vamd_kl_loss_workspace_bytes": (c_size_t, [c_int64, c_int64]),

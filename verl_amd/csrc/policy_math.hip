@@ -22,6 +22,7 @@ struct Work {
 // =============================================================================================
 template <bool VEC, class M>
 __global__ __launch_bounds__(kRcThreads) void moments_kernel(const float* __restrict__ values,
+                                                             const float* __restrict__ minus,
                                                              const M* __restrict__ mask, int64_t rows,
                                                              int64_t cols, int chunks, int per_row, Work wk,
                                                              double* __restrict__ out) {
@@ -30,6 +31,14 @@ __global__ __launch_bounds__(kRcThreads) void moments_kernel(const float* __rest
   const ChunkPos pos(row, chunk, cols);
   float x[kGroups][4], w[kGroups][4];
   load_groups<VEC>(values, pos, x);
+  if (minus) {  // moments of values - minus
+    float y[kGroups][4];
+    load_groups<VEC>(minus, pos, y);
+#pragma unroll
+    for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[g][e] -= y[g][e];
+  }
   load_mask_groups<VEC>(mask, pos, w);
   float s0 = 0, s1 = 0, s2 = 0, cnt = 0;
 #pragma unroll
@@ -194,7 +203,87 @@ __global__ __launch_bounds__(kRcThreads) void scale_rows_kernel(const float* __r
 // =============================================================================================
 struct PolicyParams {
   float ratio_lo, ratio_hi, clip_c;  // 1 - clip_low, 1 + clip_high, dual-clip constant
+  int variant;                       // VAMD_PL_*
+  float tau_pos, tau_neg;            // SAPO gate temperatures
+  const double* row_moments;         // GSPO: [rows][4], slot 0 = sum(m), slot 1 = sum((lp - old) m)
 };
+
+// Per-token loss, its derivative with respect to log_prob and the metric contributions of the
+// policy-loss variants (autograd conventions of PyTorch: maximum / minimum split ties 50/50,
+// clamp passes the gradient on its closed interval, detached factors carry none).
+//   VANILLA  clipped + dual-clip PPO                         core_algos.py:1159-1250
+//   GPG      -log_prob A                                     :1414-1447
+//   CISPO    -sg(clip(ratio)) A log_prob                     :1721-1779
+//   SAPO     -4/tau sigmoid(tau (ratio - 1)) A               :1329-1411
+//   GSPO     clipped objective on the sequence-level ratio   :1253-1326
+struct TokenLoss {
+  float loss, dloss, kl, cf, cfl;  // kl: -(clamped or raw) log-ratio; cf / cfl: 1 where the clip counters fire
+};
+
+__device__ __forceinline__ TokenLoss token_loss(const PolicyParams& pp, float old, float lp, float A, float seq_lr) {
+  TokenLoss t;
+  t.cf = 0.f;
+  t.cfl = 0.f;
+  const float d = lp - old;
+  const float k = fminf(fmaxf(d, -20.f), 20.f);
+  const float in_k = (d >= -20.f && d <= 20.f) ? 1.f : 0.f;
+  t.kl = -k;
+  switch (pp.variant) {
+    case VAMD_PL_GPG:
+      t.loss = -lp * A;
+      t.dloss = -A;
+      t.kl = 0.f;
+      break;
+    case VAMD_PL_CISPO: {
+      const float r = expf(k);
+      const float rc = fminf(fmaxf(r, pp.ratio_lo), pp.ratio_hi);
+      t.loss = -rc * A * lp;
+      t.dloss = -rc * A;
+      t.cf = r != rc ? 1.f : 0.f;
+    } break;
+    case VAMD_PL_SAPO: {
+      const float r = expf(k);
+      const float tau = A > 0.f ? pp.tau_pos : pp.tau_neg;
+      const float sg = 1.f / (1.f + expf(-tau * (r - 1.f)));
+      t.loss = -(sg * (4.f / tau)) * A;
+      t.dloss = -A * 4.f * sg * (1.f - sg) * r * in_k;
+    } break;
+    case VAMD_PL_GSPO: {
+      const float lr = fminf(seq_lr, 10.f);
+      const float pass = seq_lr <= 10.f ? 1.f : 0.f;
+      const float r = expf(lr);
+      const float l1 = -A * r;
+      const float rc = fminf(fmaxf(r, pp.ratio_lo), pp.ratio_hi);
+      const float l2 = -A * rc;
+      t.loss = fmaxf(l1, l2);
+      const float in_clip = (r >= pp.ratio_lo && r <= pp.ratio_hi) ? 1.f : 0.f;
+      const float g1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+      const float g2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+      t.dloss = (g1 + g2 * in_clip) * (-A * r) * pass;
+      t.cf = l2 > l1 ? 1.f : 0.f;
+      t.kl = -d;  // the metric uses the unclamped log-ratio (:1317)
+    } break;
+    default: {
+      const float r = expf(k);
+      const float l1 = -A * r;
+      const float rc = fminf(fmaxf(r, pp.ratio_lo), pp.ratio_hi);
+      const float l2 = -A * rc;
+      const float c1 = fmaxf(l1, l2);
+      const float l3 = -A * pp.clip_c;
+      const bool neg = A < 0.f;
+      t.loss = neg ? fminf(l3, c1) : c1;
+      t.cf = l2 > l1 ? 1.f : 0.f;
+      t.cfl = (c1 > l3 && neg) ? 1.f : 0.f;
+      const float in_clip = (r >= pp.ratio_lo && r <= pp.ratio_hi) ? 1.f : 0.f;
+      const float g1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+      const float g2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+      float dc1 = (g1 + g2 * in_clip) * (-A * r) * in_k;
+      if (neg) dc1 *= c1 < l3 ? 1.f : (c1 == l3 ? 0.5f : 0.f);
+      t.dloss = dc1;
+    } break;
+  }
+  return t;
+}
 
 template <bool VEC, class M, bool GRAD, bool ISW>
 __global__ __launch_bounds__(kRcThreads) void policy_kernel(
@@ -212,44 +301,27 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
   load_mask_groups<VEC>(mask, pos, w);
   if (ISW) load_groups<VEC>(isw, pos, iw);
   const bool token_mean = ap.mode == VAMD_AGG_TOKEN_MEAN;
+  float seq_lr = 0.f;
+  if (pp.variant == VAMD_PL_GSPO)  // sum((lp - old) m) / clamp(sum(m), min = 1)
+    seq_lr = (float)pp.row_moments[row * 4 + 1] / fmaxf((float)pp.row_moments[row * 4], 1.f);
   float s_loss = 0, s_m = 0, s_kl = 0, s_cf = 0, s_cfl = 0;
 #pragma unroll
   for (int g = 0; g < kGroups; ++g)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float A = a[g][e];
-      const float d = n[g][e] - o[g][e];
-      const float k = fminf(fmaxf(d, -20.f), 20.f);
-      const float r = expf(k);
-      const float l1 = -A * r;
-      const float rc = fminf(fmaxf(r, pp.ratio_lo), pp.ratio_hi);
-      const float l2 = -A * rc;
-      const float c1 = fmaxf(l1, l2);
-      const float l3 = -A * pp.clip_c;
-      const bool neg = A < 0.f;
-      float loss = neg ? fminf(l3, c1) : c1;
+      const TokenLoss t = token_loss(pp, o[g][e], n[g][e], a[g][e], seq_lr);
+      float loss = t.loss;
       if (ISW) loss *= iw[g][e];
       const float we = w[g][e];
       const bool in = we != 0.f;
       if (e < pos.valid[g]) {
         s_loss += ((token_mean && !in) ? 0.f : loss) * we;
         s_m += we;
-        s_kl += in ? -k * we : 0.f;
-        s_cf += (in && l2 > l1) ? we : 0.f;
-        s_cfl += (in && c1 > l3 && neg) ? we : 0.f;
+        s_kl += in ? t.kl * we : 0.f;
+        s_cf += in ? t.cf * we : 0.f;
+        s_cfl += in ? t.cfl * we : 0.f;
       }
-      if (GRAD) {
-        // autograd of maximum / minimum / clamp as PyTorch defines them (ties split 50/50,
-        // clamp passes the gradient on its closed interval)
-        const float in_k = (d >= -20.f && d <= 20.f) ? 1.f : 0.f;
-        const float in_clip = (r >= pp.ratio_lo && r <= pp.ratio_hi) ? 1.f : 0.f;
-        const float g1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
-        const float g2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
-        float dc1 = (g1 + g2 * in_clip) * (-A * r) * in_k;
-        if (neg) dc1 *= c1 < l3 ? 1.f : (c1 == l3 ? 0.5f : 0.f);
-        if (ISW) dc1 *= iw[g][e];
-        gr[g][e] = dc1 * we;
-      }
+      if (GRAD) gr[g][e] = (ISW ? t.dloss * iw[g][e] : t.dloss) * we;
     }
   if (GRAD) store_groups<VEC>(grad, pos, gr);
   __shared__ double smem[(5 + 3) * 4];
@@ -667,9 +739,20 @@ extern "C" size_t vamd_masked_moments_workspace_bytes(int64_t rows, int64_t cols
   return reduce_workspace_bytes(rows, cols, 4);
 }
 
+static int masked_moments_of_difference(const float* values, const float* minus, const void* mask, int mask_dtype,
+                                        int64_t rows, int64_t cols, int per_row, double* out, void* workspace,
+                                        size_t workspace_bytes, void* stream);
+
 extern "C" int vamd_masked_moments(const float* values, const void* mask, int mask_dtype, int64_t rows,
                                    int64_t cols, int per_row, double* out, void* workspace, size_t workspace_bytes,
                                    void* stream) {
+  return masked_moments_of_difference(values, nullptr, mask, mask_dtype, rows, cols, per_row, out, workspace,
+                                      workspace_bytes, stream);
+}
+
+static int masked_moments_of_difference(const float* values, const float* minus, const void* mask, int mask_dtype,
+                                        int64_t rows, int64_t cols, int per_row, double* out, void* workspace,
+                                        size_t workspace_bytes, void* stream) {
   int st = check_matrix("masked_moments", rows, cols);
   if (st != VAMD_OK) return st;
   VAMD_REQUIRE(values && mask && out, "masked_moments: null pointer");
@@ -681,10 +764,10 @@ extern "C" int vamd_masked_moments(const float* values, const void* mask, int ma
   const int chunks = (int)chunks_of(cols);
   const Work wk = carve_work(workspace);
   VAMD_MASK_DISPATCH(mask_dtype, M, {
-    const bool vec = can_vectorize(cols, {values}, mask, sizeof(M));
+    const bool vec = can_vectorize(cols, {values, minus}, mask, sizeof(M));
     VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((moments_kernel<V, M>), dim3((unsigned)(rows * chunks)),
-                                                 dim3(kRcThreads), 0, s, values, static_cast<const M*>(mask), rows,
-                                                 cols, chunks, per_row, wk, out));
+                                                 dim3(kRcThreads), 0, s, values, minus, static_cast<const M*>(mask),
+                                                 rows, cols, chunks, per_row, wk, out));
   });
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
@@ -802,10 +885,41 @@ extern "C" int vamd_policy_loss_forward(const float* old_log_prob, const float* 
   int st = check_matrix("policy_loss", rows, cols);
   if (st != VAMD_OK) return st;
   VAMD_REQUIRE(old_log_prob && log_prob && advantages && mask && out, "policy_loss: null pointer");
-  VAMD_REQUIRE(mode >= 0 && mode <= 3, "policy_loss: invalid mode %d", mode);
-  VAMD_REQUIRE(clip_c > 1.0f, "policy_loss: clip_ratio_c must be > 1.0, got %f", (double)clip_c);
-  VAMD_REQUIRE(!grad_unscaled || coef_out, "policy_loss: grad output needs coef_out");
   if (!workspace || workspace_bytes < vamd_policy_loss_workspace_bytes(rows, cols)) {
+    set_error("policy_loss: workspace too small");
+    return VAMD_EWORKSPACE;
+  }
+  // the vanilla loss never touches the per-row moments the general query reserves room for
+  return vamd_policy_loss_variant_forward(VAMD_PL_VANILLA, old_log_prob, log_prob, advantages, mask, mask_dtype,
+                                          is_weights, rows, cols, clip_low, clip_high, clip_c, 1.f, 1.f, mode,
+                                          dp_size, batch_num_tokens, global_batch_size, loss_scale_factor, out,
+                                          grad_unscaled, coef_out, workspace,
+                                          vamd_policy_loss_variant_workspace_bytes(rows, cols), stream);
+}
+
+extern "C" size_t vamd_policy_loss_variant_workspace_bytes(int64_t rows, int64_t cols) {
+  if (rows <= 0 || cols <= 0) return 0;
+  return reduce_workspace_bytes(rows, cols, 5) + align_up((size_t)rows * 4 * sizeof(double), 256);
+}
+
+extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_log_prob, const float* log_prob,
+                                                const float* advantages, const void* mask, int mask_dtype,
+                                                const float* is_weights, int64_t rows, int64_t cols, float clip_low,
+                                                float clip_high, float clip_c, float tau_pos, float tau_neg, int mode,
+                                                double dp_size, double batch_num_tokens, double global_batch_size,
+                                                double loss_scale_factor, float* out, float* grad_unscaled,
+                                                float* coef_out, void* workspace, size_t workspace_bytes,
+                                                void* stream) {
+  int st = check_matrix("policy_loss", rows, cols);
+  if (st != VAMD_OK) return st;
+  VAMD_REQUIRE(old_log_prob && log_prob && advantages && mask && out, "policy_loss: null pointer");
+  VAMD_REQUIRE(variant >= VAMD_PL_VANILLA && variant <= VAMD_PL_GSPO, "policy_loss: invalid variant %d", variant);
+  VAMD_REQUIRE(mode >= 0 && mode <= 3, "policy_loss: invalid mode %d", mode);
+  VAMD_REQUIRE(variant != VAMD_PL_VANILLA || clip_c > 1.0f, "policy_loss: clip_ratio_c must be > 1.0, got %f",
+               (double)clip_c);
+  VAMD_REQUIRE(variant != VAMD_PL_SAPO || (tau_pos != 0.f && tau_neg != 0.f), "policy_loss: SAPO needs non-zero tau");
+  VAMD_REQUIRE(!grad_unscaled || coef_out, "policy_loss: grad output needs coef_out");
+  if (!workspace || workspace_bytes < vamd_policy_loss_variant_workspace_bytes(rows, cols)) {
     set_error("policy_loss: workspace too small");
     return VAMD_EWORKSPACE;
   }
@@ -816,6 +930,17 @@ extern "C" int vamd_policy_loss_forward(const float* old_log_prob, const float* 
   pp.ratio_lo = (float)(1.0 - (double)clip_low);
   pp.ratio_hi = (float)(1.0 + (double)clip_high);
   pp.clip_c = clip_c;
+  pp.variant = variant;
+  pp.tau_pos = tau_pos;
+  pp.tau_neg = tau_neg;
+  pp.row_moments = nullptr;
+  if (variant == VAMD_PL_GSPO) {  // sequence-level log-ratio: per-row masked moments of log_prob - old_log_prob
+    double* row_moments = reinterpret_cast<double*>(static_cast<char*>(workspace) + reduce_workspace_bytes(rows, cols, 5));
+    st = masked_moments_of_difference(log_prob, old_log_prob, mask, mask_dtype, rows, cols, 1, row_moments, workspace,
+                                      reduce_workspace_bytes(rows, cols, 5), stream);
+    if (st != VAMD_OK) return st;
+    pp.row_moments = row_moments;
+  }
   const AggParams ap = make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor);
   const dim3 grid((unsigned)(rows * chunks)), block(kRcThreads);
 #define VAMD_PL(V, G, W)                                                                                     \
@@ -955,6 +1080,9 @@ extern "C" int vamd_grpo_advantage(const float* rewards, const void* mask, int m
                                    int64_t batch, int64_t length, int64_t n_groups, float epsilon, int norm_by_std,
                                    int std_mode, float* advantages, float* scores_out, void* workspace,
                                    size_t workspace_bytes, void* stream) {
+  int st = check_matrix("grpo", batch, length);
+  if (st != VAMD_OK) return st;
+  VAMD_REQUIRE(rewards && mask && group_ids && advantages && n_groups > 0, "grpo: bad argument");
   if (!workspace || workspace_bytes < vamd_grpo_workspace_bytes(batch, length, n_groups)) {
     set_error("grpo: workspace too small");
     return VAMD_EWORKSPACE;

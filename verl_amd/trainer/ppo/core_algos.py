@@ -369,7 +369,7 @@ def agg_loss(loss_mat: torch.Tensor, loss_mask: torch.Tensor, loss_agg_mode: str
 class _PolicyLoss(torch.autograd.Function):
     @staticmethod
     def forward(ctx, log_prob, old_log_prob, advantages, response_mask, is_weights, clip_low, clip_high, clip_c,
-                mode, dp_size, bnt, gbs, lsf):
+                mode, dp_size, bnt, gbs, lsf, variant=0, tau_pos=1.0, tau_neg=1.0):
         dev = _cabi.compute_device(log_prob, old_log_prob, advantages, response_mask)
         lp = _matrix(log_prob, dev)
         old = _matrix(old_log_prob, dev)
@@ -383,13 +383,13 @@ class _PolicyLoss(torch.autograd.Function):
         out = torch.empty(4, dtype=torch.float32, device=dev)
         coef = torch.empty(rows, dtype=torch.float32, device=dev)
         g = torch.empty_like(lp) if need_grad else None
-        ws = _cabi.ticket_workspace(Lb.vamd_policy_loss_workspace_bytes(rows, cols), dev)
+        ws = _cabi.ticket_workspace(Lb.vamd_policy_loss_variant_workspace_bytes(rows, cols), dev)
         with torch.cuda.device(dev):
-            _cabi.check(Lb.vamd_policy_loss_forward(old.data_ptr(), lp.data_ptr(), adv.data_ptr(), m.data_ptr(), code,
-                                                    _cabi.ptr(isw), rows, cols, clip_low, clip_high, clip_c, mode,
-                                                    dp_size, bnt, gbs, lsf, out.data_ptr(), _cabi.ptr(g),
-                                                    coef.data_ptr(), ws.data_ptr(), ws.numel(),
-                                                    _cabi.stream_ptr(dev)))
+            _cabi.check(Lb.vamd_policy_loss_variant_forward(variant, old.data_ptr(), lp.data_ptr(), adv.data_ptr(),
+                                                            m.data_ptr(), code, _cabi.ptr(isw), rows, cols, clip_low,
+                                                            clip_high, clip_c, tau_pos, tau_neg, mode, dp_size, bnt,
+                                                            gbs, lsf, out.data_ptr(), _cabi.ptr(g), coef.data_ptr(),
+                                                            ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
         if need_grad:
             ctx.save_for_backward(g, coef)
         ctx.in_shape = log_prob.shape
@@ -410,7 +410,7 @@ class _PolicyLoss(torch.autograd.Function):
             _cabi.check(_cabi.lib().vamd_scale_rows(g.data_ptr(), coef.data_ptr(), d.data_ptr(), 1.0, rows, cols,
                                                     res.data_ptr(), _cabi.stream_ptr(dev)))
         res = res.view(ctx.in_shape).to(device=ctx.in_device, dtype=ctx.in_dtype)
-        return (res,) + (None,) * 12
+        return (res,) + (None,) * 15
 
 
 def _cfg_get(config, key, default=None):
@@ -456,6 +456,74 @@ def compute_policy_loss_vanilla(old_log_prob: torch.Tensor, log_prob: torch.Tens
         "actor/pg_clipfrac_lower": vals[3],
     }
     return pg_loss, pg_metrics
+
+
+_PL = {"vanilla": 0, "gpg": 1, "cispo": 2, "sapo": 3, "gspo": 4}
+
+
+def _policy_loss_variant(variant, old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, config,
+                         rollout_is_weights, tau_pos=1.0, tau_neg=1.0, needs_clip=True):
+    clip_low = clip_high = 0.0
+    if needs_clip:
+        clip_ratio = config.clip_ratio
+        low = getattr(config, "clip_ratio_low", None)
+        high = getattr(config, "clip_ratio_high", None)
+        clip_low = low if low is not None else clip_ratio
+        clip_high = high if high is not None else clip_ratio
+    info = dict(getattr(config, "global_batch_info", None) or {})
+    pg_loss, out = _PolicyLoss.apply(
+        log_prob, old_log_prob, advantages, response_mask, rollout_is_weights, float(clip_low), float(clip_high), 3.0,
+        _agg_mode(loss_agg_mode), float(info.get("dp_size", 1)), _opt(info.get("batch_num_tokens")),
+        _opt(info.get("global_batch_size")), _opt(info.get("loss_scale_factor")), _PL[variant], float(tau_pos),
+        float(tau_neg))
+    vals = out.detach().tolist()
+    return pg_loss, {"actor/pg_clipfrac": vals[1], "actor/ppo_kl": vals[2], "actor/pg_clipfrac_lower": vals[3]}
+
+
+@register_policy_loss("gspo")
+def compute_policy_loss_gspo(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                             response_mask: torch.Tensor, loss_agg_mode: str = "seq-mean-token-mean",
+                             config: Optional[Any] = None, rollout_is_weights: torch.Tensor | None = None):
+    """GSPO (reference core_algos.py:1253-1326): the clipped objective on the sequence-level importance
+    ratio ``exp(min(mean_t(log_prob - old_log_prob), 10))`` with token-level gradients; always aggregated
+    as "seq-mean-token-mean" whatever ``loss_agg_mode`` says, as there (:1307-1309)."""
+    assert config is not None
+    return _policy_loss_variant("gspo", old_log_prob, log_prob, advantages, response_mask, "seq-mean-token-mean",
+                                config, rollout_is_weights)
+
+
+@register_policy_loss("sapo")
+def compute_policy_loss_sapo(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                             response_mask: torch.Tensor, loss_agg_mode: str = "seq-mean-token-mean",
+                             config: Optional[Any] = None, rollout_is_weights: torch.Tensor | None = None):
+    """SAPO (reference core_algos.py:1329-1411): ``-4/tau sigmoid(tau (ratio - 1)) A`` with ``config.tau_pos``
+    for positive and ``config.tau_neg`` for the other advantages; always "seq-mean-token-mean"."""
+    assert config is not None
+    return _policy_loss_variant("sapo", old_log_prob, log_prob, advantages, response_mask, "seq-mean-token-mean",
+                                config, rollout_is_weights, tau_pos=config.tau_pos, tau_neg=config.tau_neg,
+                                needs_clip=False)
+
+
+@register_policy_loss("gpg")
+def compute_policy_loss_gpg(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                            response_mask: torch.Tensor, loss_agg_mode: str = "token-mean",
+                            config: Optional[Any] = None, rollout_is_weights: torch.Tensor | None = None):
+    """GPG (reference core_algos.py:1414-1447): ``agg_loss(-log_prob A)``; returns an empty metrics dict."""
+    assert config is not None
+    pg_loss, _ = _policy_loss_variant("gpg", old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, config,
+                                      rollout_is_weights, needs_clip=False)
+    return pg_loss, {}
+
+
+@register_policy_loss("cispo")
+def compute_policy_loss_cispo(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                              response_mask: torch.Tensor, loss_agg_mode: str = "token-mean",
+                              config: Optional[Any] = None, rollout_is_weights: torch.Tensor | None = None):
+    """CISPO (reference core_algos.py:1721-1779): ``-sg(clip(ratio)) A log_prob``; ``actor/pg_clipfrac`` is the
+    share of valid tokens whose ratio was clipped."""
+    assert config is not None
+    return _policy_loss_variant("cispo", old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, config,
+                                rollout_is_weights)
 
 
 def compute_policy_loss(old_log_prob, log_prob, advantages, response_mask, cliprange=None, cliprange_low=None,
