@@ -429,66 +429,106 @@ struct GemmOutArgs {
   int64_t ld_out;
 };
 
+// Both gradient epilogues hand each 32 x 32 accumulator block through a 4 KB LDS patch private to the
+// wavefront (the 32 KB the pipeline leaves free), so that global accesses are whole 128-byte rows
+// of fp32 (64-byte rows of bf16) touched by 8 consecutive lanes instead of 16-byte pieces of 32
+// different rows.  After the exchange lane L holds columns 4 (L % 8) .. + 3 of rows 8 i + L / 8.
+struct BlockExchange {
+  char* stage;  // this wavefront's patch
+  int lr, lh, rd_row, rd_chunk;
+  __device__ __forceinline__ void init(char* lds_after_pipeline, const LanePos& p) {
+    stage = lds_after_pipeline + (threadIdx.x >> 6) * 4096;
+    lr = p.lr;
+    lh = p.lh;
+    rd_row = (threadIdx.x & 63) >> 3;
+    rd_chunk = threadIdx.x & 7;
+  }
+  __device__ __forceinline__ void run(const f32x16& blk, f32x4 (&out)[4]) const {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 v = {blk[4 * g], blk[4 * g + 1], blk[4 * g + 2], blk[4 * g + 3]};
+      *reinterpret_cast<f32x4*>(stage + lr * 128 + (((2 * g + lh) ^ ((lr >> 1) & 7)) << 4)) = v;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 8 * i + rd_row;
+      out[i] = *reinterpret_cast<const f32x4*>(stage + row * 128 + ((rd_chunk ^ ((row >> 1) & 7)) << 4));
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+};
+
 struct DHiddenEpi {
   LanePos p;
   const GemmOutArgs* a;
+  BlockExchange ex;
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const GemmOutArgs& A = *a;
+    const bool read_prev = A.mode == kAddF32 || A.mode == kFinalBf16AddPrev;
+    const bool to_f32 = A.mode == kStoreF32 || A.mode == kAddF32;
 #pragma unroll
-    for (int nb = 0; nb < kNB; ++nb) {
-      const int row = r0 + acc_row(p, nb);
-      if (row >= A.r_valid) continue;
+    for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
-      for (int mb = 0; mb < kMB; ++mb)
+      for (int mb = 0; mb < kMB; ++mb) {
+        f32x4 v[4];
+        ex.run(acc.a[mb][nb], v);
+        const int col = c0 + p.wc * 128 + mb * 32 + 4 * ex.rd_chunk;
+        if (col >= A.c_valid) continue;
+        const int row0 = r0 + p.wr * (kNB * 32) + nb * 32 + ex.rd_row;
+        f32x4 prev[4];
+        if (read_prev) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int col = c0 + p.wc * 128 + mb * 32 + 8 * g + 4 * p.lh;
-          if (col >= A.c_valid) continue;
-          f32x4 v = {acc.a[mb][nb][4 * g], acc.a[mb][nb][4 * g + 1], acc.a[mb][nb][4 * g + 2],
-                     acc.a[mb][nb][4 * g + 3]};
-          const int64_t off = (int64_t)row * A.ld_out + col;
-          if (A.mode == kStoreF32) {
-            *reinterpret_cast<f32x4*>(A.acc32 + off) = v;
-          } else if (A.mode == kAddF32) {
-            f32x4 o = *reinterpret_cast<const f32x4*>(A.acc32 + off);
-            *reinterpret_cast<f32x4*>(A.acc32 + off) = o + v;
-          } else {
-            if (A.mode == kFinalBf16AddPrev) v = v + *reinterpret_cast<const f32x4*>(A.acc32 + off);
-            *reinterpret_cast<u32x2*>(A.out + off) = pack_bf16x4(v[0], v[1], v[2], v[3]);
-          }
+          for (int i = 0; i < 4; ++i)
+            prev[i] = (row0 + 8 * i < A.r_valid)
+                          ? *reinterpret_cast<const f32x4*>(A.acc32 + (int64_t)(row0 + 8 * i) * A.ld_out + col)
+                          : f32x4{0.f, 0.f, 0.f, 0.f};
         }
-    }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int row = row0 + 8 * i;
+          if (row >= A.r_valid) continue;
+          f32x4 x = v[i];
+          if (read_prev) x = x + prev[i];
+          const int64_t off = (int64_t)row * A.ld_out + col;
+          if (to_f32) *reinterpret_cast<f32x4*>(A.acc32 + off) = x;
+          else *reinterpret_cast<u32x2*>(A.out + off) = pack_bf16x4(x[0], x[1], x[2], x[3]);
+        }
+      }
   }
 };
 
 struct DWeightEpi {
   LanePos p;
   const GemmOutArgs* a;
+  BlockExchange ex;
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const GemmOutArgs& A = *a;
 #pragma unroll
-    for (int nb = 0; nb < kNB; ++nb) {
-      const int row = r0 + acc_row(p, nb);
-      if (row >= A.r_valid) continue;
+    for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
-      for (int mb = 0; mb < kMB; ++mb)
+      for (int mb = 0; mb < kMB; ++mb) {
+        f32x4 v[4];
+        ex.run(acc.a[mb][nb], v);
+        const int col = c0 + p.wc * 128 + mb * 32 + 4 * ex.rd_chunk;
+        if (col >= A.c_valid) continue;
+        const int row0 = r0 + p.wr * (kNB * 32) + nb * 32 + ex.rd_row;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int col = c0 + p.wc * 128 + mb * 32 + 8 * g + 4 * p.lh;
-          if (col >= A.c_valid) continue;
-          float v0 = acc.a[mb][nb][4 * g], v1 = acc.a[mb][nb][4 * g + 1], v2 = acc.a[mb][nb][4 * g + 2],
-                v3 = acc.a[mb][nb][4 * g + 3];
+        for (int i = 0; i < 4; ++i) {
+          const int row = row0 + 8 * i;
+          if (row >= A.r_valid) continue;
+          f32x4 x = v[i];
           u32x2* dst = reinterpret_cast<u32x2*>(A.out + (int64_t)row * A.ld_out + col);
           if (A.mode == 1) {
             const u32x2 o = *dst;
-            v0 += bf16_bits_to_float(o[0] & 0xffffu);
-            v1 += bf16_bits_to_float(o[0] >> 16);
-            v2 += bf16_bits_to_float(o[1] & 0xffffu);
-            v3 += bf16_bits_to_float(o[1] >> 16);
+            x[0] += bf16_bits_to_float(o[0] & 0xffffu);
+            x[1] += bf16_bits_to_float(o[0] >> 16);
+            x[2] += bf16_bits_to_float(o[1] & 0xffffu);
+            x[3] += bf16_bits_to_float(o[1] >> 16);
           }
-          *dst = pack_bf16x4(v0, v1, v2, v3);
+          *dst = pack_bf16x4(x[0], x[1], x[2], x[3]);
         }
-    }
+      }
   }
 };
 
@@ -511,6 +551,7 @@ __global__ __launch_bounds__(kThreads) void lce_dgrad_kernel(GemmOutArgs gh, Gem
     DHiddenEpi epi;
     epi.p = pos;
     epi.a = &gh;
+    epi.ex.init(lds + kLdsBytes, pos);
     run_tiles<false, true>(gh.R, gh.C, gh.k_slabs, sched, epi, lds);
   }
   __syncthreads();
@@ -524,6 +565,7 @@ __global__ __launch_bounds__(kThreads) void lce_dgrad_kernel(GemmOutArgs gh, Gem
     DWeightEpi epi;
     epi.p = pos;
     epi.a = &gw;
+    epi.ex.init(lds + kLdsBytes, pos);
     run_tiles<true, true>(gw.R, gw.C, gw.k_slabs, sched, epi, lds);
   }
 }
@@ -546,7 +588,7 @@ static int ensure_lds_attributes() {
     if ((s = allow_big_lds(lce_forward_kernel<false>)) != VAMD_OK) { status = s; return; }
     if ((s = allow_big_lds(lce_forward_kernel<true>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) { status = s; return; }
     if ((s = allow_big_lds(lce_recompute_kernel)) != VAMD_OK) { status = s; return; }
-    if ((s = allow_big_lds(lce_dgrad_kernel)) != VAMD_OK) { status = s; return; }
+    if ((s = allow_big_lds(lce_dgrad_kernel, kLdsBytes + kCacheStageBytes)) != VAMD_OK) { status = s; return; }
   });
   return status;
 }
@@ -826,7 +868,7 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
       const int tiles = gh.r_tiles * gh.c_tiles + gw.r_tiles * gw.c_tiles;
       const int grid = tiles < cus ? tiles : cus;
       ScopedTiming tm(kTagDGrad, s);
-      hipLaunchKernelGGL(lce_dgrad_kernel, dim3(grid), dim3(kThreads), kLdsBytes, s, gh, gw);
+      hipLaunchKernelGGL(lce_dgrad_kernel, dim3(grid), dim3(kThreads), kLdsBytes + kCacheStageBytes, s, gh, gw);
     }
     VAMD_LAUNCH_CHECK();
   }
