@@ -96,12 +96,16 @@ int vamd_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream);
  *   same buffer to vamd_lce_backward replaces its logits-recompute GEMM by a streaming pass: a
  *   trade of 4 * n_tokens * vocab bytes of HBM (10 GB at 16384 x 152064) for a quarter of the
  *   step's matrix work.  Results do not depend on the choice beyond fp32 rounding of z.
+ *   sum_pi_squared: NULL, or [n_tokens] fp32 that receives sum_j softmax(z)_j^2
+ *   (calculate_sum_pi_squared_from_logits, verl/utils/torch_functional.py:680-694), carried as a
+ *   fifth running sum of the same online softmax; the reference cannot combine this statistic with
+ *   its fused kernels (verl/workers/actor/dp_actor.py:107-111).
  */
 size_t vamd_lce_forward_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab);
 int vamd_lce_forward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
                      int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs, float* entropy,
-                     float* lse, float* mean_z, float* logits_cache, void* workspace, size_t workspace_bytes,
-                     void* stream);
+                     float* lse, float* mean_z, float* logits_cache, float* sum_pi_squared, void* workspace,
+                     size_t workspace_bytes, void* stream);
 
 /* Backward: d_logits = [g_lp (onehot - p) - g_ent p (z - mean_z)] * rcp_temperature is formed
  * tile by tile from recomputed logits, never as a whole; d_hidden = d_logits . weight,

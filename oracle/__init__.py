@@ -32,6 +32,7 @@ from .masked import (  # noqa: F401
     masked_mean,
     masked_var,
     masked_whiten,
+    sum_pi_squared_from_logits,
 )
 from .advantages import (  # noqa: F401
     gae_advantage_return,

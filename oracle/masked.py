@@ -63,3 +63,9 @@ def masked_whiten(values, mask, shift_mean=True):
     if not shift_mean:
         out = out + mean
     return out
+
+
+def sum_pi_squared_from_logits(logits):
+    """``sum_j softmax(logits)_j ** 2`` as ``exp(logsumexp(2 z) - 2 logsumexp(z))``,
+    verl/utils/torch_functional.py:680-694."""
+    return torch.exp(torch.logsumexp(2.0 * logits, dim=-1) - 2.0 * torch.logsumexp(logits, dim=-1))

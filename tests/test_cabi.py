@@ -32,7 +32,7 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/verl_amd.h but not exported"
     assert sorted(_cabi.SIGNATURES) == declared, "ctypes prototypes and header disagree"
-    assert lib.vamd_abi_version() == 2
+    assert lib.vamd_abi_version() == 3
 
 
 def test_workspace_queries(lib):
@@ -50,7 +50,7 @@ def test_workspace_queries(lib):
 
 
 def test_argument_errors_are_reported_without_touching_the_gpu(lib):
-    rc = lib.vamd_lce_forward(None, None, None, 16, 100, 128, 1.0, None, None, None, None, None, None, 0, None)
+    rc = lib.vamd_lce_forward(None, None, None, 16, 100, 128, 1.0, None, None, None, None, None, None, None, 0, None)
     assert rc == -1 and b"multiple of 128" in lib.vamd_last_error()
     rc = lib.vamd_policy_loss_forward(None, None, None, None, 0, None, 4, 4, 0.2, 0.2, 3.0, 0, 1.0, -1.0, -1.0, -1.0,
                                       None, None, None, None, 0, None)

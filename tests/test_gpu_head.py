@@ -295,3 +295,24 @@ def test_benchmark_config_llama_head_token_chunked(dev):
     _close_bf16(torch.cat(dhs), want_dh, "d_hidden", e_dh)
     # d_weight passes through bf16 once per token chunk: one more half-ulp of the running value per accumulation
     _close_bf16(d_weight, want_dw, "d_weight accumulated over token chunks", e_dw + want_dw.abs())
+
+
+@pytest.mark.parametrize("n,h,v,T", [(1, 128, 128, 1.0), (300, 384, 1000, 0.7), (700, 256, 8192, 1.5), (2169, 896, 151936, 1.0)])
+def test_sum_pi_squared_from_the_head(dev, n, h, v, T):
+    """sum_j softmax(z)_j^2 carried by the forward pass next to log-prob and entropy; the other outputs are the
+    same numbers the plain forward gives."""
+    from verl_amd.utils.kernel import linear_cross_entropy as K
+    from oracle import masked as OM
+    hidden, weight, labels = _make(n, h, v, seed=3 * n + v, dist="normal" if v > 10000 else "uniform")
+    hd, wd, ld = hidden.to(dev), weight.to(dev), labels.to(dev)
+    lp, ent, pi2 = K.linear_cross_entropy_with_sum_pi_squared(hd, wd, ld, T)
+    lp0, ent0, _, _ = K.efficient_entropy_forward(hd, wd, ld, 0, T)
+    assert torch.equal(lp, lp0) and torch.equal(ent, ent0)
+    want = []
+    for lo in range(0, n, 512):
+        z = (hd[lo:lo + 512].float() @ wd.float().t()) / T
+        want.append(OM.sum_pi_squared_from_logits(z))
+    want = torch.cat(want)
+    assert pi2.shape == (n,) and pi2.dtype == torch.float32
+    assert (pi2 >= 1.0 / v - 1e-9).all() and (pi2 <= 1.0 + 1e-6).all()
+    assert torch.allclose(pi2, want, rtol=2e-3, atol=1e-9), ((pi2 - want).abs() / want).max().item()

@@ -299,3 +299,14 @@ def test_reinforce_plus_plus_and_remax_closed_forms():
     # ReMax with a mask: masked rewards do not count, masked positions still show the carried sum
     adv3, r3 = A.remax_outcome_advantage(r, base, m)
     assert torch.allclose(r3[:, 10], r3[:, 11]) and torch.allclose(adv3[:, 10], r3[:, 10])
+
+
+def test_sum_pi_squared_closed_forms():
+    z = torch.zeros(2, 50, dtype=torch.float64)
+    assert torch.allclose(M.sum_pi_squared_from_logits(z), torch.full((2,), 1 / 50, dtype=torch.float64))   # uniform
+    z = torch.tensor([[40.0, 0.0, 0.0]], dtype=torch.float64)
+    assert abs(M.sum_pi_squared_from_logits(z).item() - 1.0) < 1e-15                                          # one-hot
+    g = torch.Generator().manual_seed(0)
+    z = torch.randn(5, 33, generator=g, dtype=torch.float64) * 3
+    assert torch.allclose(M.sum_pi_squared_from_logits(z), (torch.softmax(z, -1) ** 2).sum(-1), rtol=1e-12)  # brute force
+    assert torch.allclose(M.sum_pi_squared_from_logits(z + 7.5), M.sum_pi_squared_from_logits(z), rtol=1e-12)  # shift

@@ -31,7 +31,7 @@ SIGNATURES = {
     "vamd_copy_bytes": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "vamd_lce_forward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "vamd_lce_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p,
-                                 c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+                                 c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "vamd_lce_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
     "vamd_lce_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int64,

@@ -73,6 +73,7 @@ struct FwdArgs {
   float rcp_t;       // 1 / temperature
   float4* partials;  // [splits][tok_tiles * 256] : (max2, sum, sum_y, label logit)
   float* z_cache;    // optional [n_tokens][vocab] fp32 logits / temperature, kept for the backward
+  float* pi2_partials;  // optional [splits][tok_tiles * 256] : sum of e^2 relative to the same max
 };
 
 struct SplitSched {
@@ -89,12 +90,14 @@ constexpr int kCacheStageBytes = (kThreads / 64) * 4096;  // one 32 x 32 fp32 bl
 // Per-lane online-softmax state for the kNB token slots (nb) the lane owns.  With CACHE the
 // scaled logits of every valid (token, vocabulary column) are also written out in fp32, so the
 // backward pass can form d_logits without repeating the GEMM.
-template <bool CACHE>
+// With PI2 a fifth running sum, sum_j e_j^2, is carried, from which sum_j softmax(z)_j^2 follows
+// (calculate_sum_pi_squared_from_logits, verl/utils/torch_functional.py:680-694).
+template <bool CACHE, bool PI2>
 struct FwdEpi {
   LanePos p;
   float scale2;
   int vocab;
-  float m[kNB], s[kNB], sy[kNB], zl[kNB];
+  float m[kNB], s[kNB], sy[kNB], zl[kNB], s2[kNB];
   int lab[kNB];
   float rcp_t;
   float* z_cache;  // CACHE: [n_tokens][vocab]
@@ -164,7 +167,7 @@ struct FwdEpi {
       }
       const float m_new = fmaxf(m[nb], ymax);
       const float resc = fast_exp2(m[nb] - m_new);
-      float s_ = s[nb] * resc, sy_ = sy[nb] * resc;
+      float s_ = s[nb] * resc, sy_ = sy[nb] * resc, s2_ = PI2 ? s2[nb] * resc * resc : 0.f;
 #pragma unroll
       for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
@@ -173,10 +176,12 @@ struct FwdEpi {
           const float e = fast_exp2(y - m_new);
           s_ += e;
           sy_ = fmaf(e, y, sy_);
+          if (PI2) s2_ = fmaf(e, e, s2_);
         }
       m[nb] = m_new;
       s[nb] = s_;
       sy[nb] = sy_;
+      if (PI2) s2[nb] = s2_;
     }
   }
 };
@@ -188,8 +193,18 @@ __device__ __forceinline__ void merge_state(float& m, float& s, float& sy, float
   sy = sy * a + sy2 * b;
   m = mm;
 }
+// the same with the squared sums q
+__device__ __forceinline__ void merge_state(float& m, float& s, float& sy, float& q, float m2, float s2, float sy2,
+                                            float q2) {
+  const float mm = fmaxf(m, m2);
+  const float a = fast_exp2(m - mm), b = fast_exp2(m2 - mm);
+  s = s * a + s2 * b;
+  sy = sy * a + sy2 * b;
+  q = q * a * a + q2 * b * b;
+  m = mm;
+}
 
-template <bool CACHE>
+template <bool CACHE, bool PI2>
 __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char lds[];
   // workgroup -> (token tile, vocabulary split); bands of 8 token tiles x all splits per XCD
@@ -208,7 +223,7 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
   sched.vt_begin = (int)(((int64_t)sp * a.voc_tiles) / a.splits);
   sched.vt_count = (int)(((int64_t)(sp + 1) * a.voc_tiles) / a.splits) - sched.vt_begin;
 
-  FwdEpi<CACHE> epi;
+  FwdEpi<CACHE, PI2> epi;
   epi.p = lane_pos();
   epi.scale2 = a.scale2;
   epi.vocab = a.vocab;
@@ -219,6 +234,7 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
     epi.s[nb] = 0.f;
     epi.sy[nb] = 0.f;
     epi.zl[nb] = 0.f;
+    epi.s2[nb] = 0.f;
     const int tok = sched.r0_ + acc_row(epi.p, nb);
     epi.lab[nb] = tok < a.n_tokens ? (int)a.labels[tok] : -1;
   }
@@ -236,46 +252,65 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
     const float s2 = __shfl_xor(epi.s[nb], 32, 64);
     const float sy2 = __shfl_xor(epi.sy[nb], 32, 64);
     const float z2 = __shfl_xor(epi.zl[nb], 32, 64);
-    merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], m2, s2, sy2);
+    if (PI2) {
+      const float q2 = __shfl_xor(epi.s2[nb], 32, 64);
+      merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], epi.s2[nb], m2, s2, sy2, q2);
+    } else {
+      merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], m2, s2, sy2);
+    }
     epi.zl[nb] += z2;
   }
   // ... then the two wavefronts that share a token quarter (wc = 0/1), through LDS (once every
   // wavefront's last slab transfers have landed).
   __syncthreads();
-  float4* red = reinterpret_cast<float4*>(lds);  // [2][256]
+  float4* red = reinterpret_cast<float4*>(lds);                     // [2][256]
+  float* redq = reinterpret_cast<float*>(lds + 2 * kTile * 16);    // [2][256] squared sums
   if (epi.p.lh == 0) {
 #pragma unroll
-    for (int nb = 0; nb < kNB; ++nb)
+    for (int nb = 0; nb < kNB; ++nb) {
       red[epi.p.wc * kTile + acc_row(epi.p, nb)] = make_float4(epi.m[nb], epi.s[nb], epi.sy[nb], epi.zl[nb]);
+      if (PI2) redq[epi.p.wc * kTile + acc_row(epi.p, nb)] = epi.s2[nb];
+    }
   }
   __syncthreads();
   if (threadIdx.x < kTile) {
     const int t = threadIdx.x;
     float4 x = red[t], y = red[kTile + t];
-    merge_state(x.x, x.y, x.z, y.x, y.y, y.z);
+    const int64_t slot = (int64_t)sp * a.tok_tiles * kTile + tn * kTile + t;
+    if (PI2) {
+      float q = redq[t];
+      merge_state(x.x, x.y, x.z, q, y.x, y.y, y.z, redq[kTile + t]);
+      a.pi2_partials[slot] = q;
+    } else {
+      merge_state(x.x, x.y, x.z, y.x, y.y, y.z);
+    }
     x.w += y.w;
-    a.partials[(int64_t)sp * a.tok_tiles * kTile + tn * kTile + t] = x;
+    a.partials[slot] = x;
   }
 }
 
 struct MergeArgs {
   const float4* partials;
+  const float* pi2_partials;  // null unless sum_pi_squared is wanted
   int splits, stride, n_tokens;
   float* logprobs;
   float* entropy;
   float* lse;
   float* mean_z;
+  float* sum_pi_squared;
 };
 
 __global__ __launch_bounds__(256) void lce_merge_kernel(MergeArgs a) {
   const int tok = blockIdx.x * 256 + threadIdx.x;
   if (tok >= a.n_tokens) return;
-  float m = kNegBig, s = 0.f, sy = 0.f, zl = 0.f;
+  float m = kNegBig, s = 0.f, sy = 0.f, zl = 0.f, q = 0.f;
   for (int sp = 0; sp < a.splits; ++sp) {
     const float4 x = a.partials[(int64_t)sp * a.stride + tok];
-    merge_state(m, s, sy, x.x, x.y, x.z);
+    if (a.pi2_partials) merge_state(m, s, sy, q, x.x, x.y, x.z, a.pi2_partials[(int64_t)sp * a.stride + tok]);
+    else merge_state(m, s, sy, x.x, x.y, x.z);
     zl += x.w;
   }
+  if (a.pi2_partials) a.sum_pi_squared[tok] = q / (s * s);
   const float lse = (m + log2f(s)) * kLn2;
   const float mz = (sy / s) * kLn2;
   a.lse[tok] = lse;
@@ -585,8 +620,10 @@ static int ensure_lds_attributes() {
   static int status = VAMD_OK;
   std::call_once(once, [] {
     int s;
-    if ((s = allow_big_lds(lce_forward_kernel<false>)) != VAMD_OK) { status = s; return; }
-    if ((s = allow_big_lds(lce_forward_kernel<true>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) { status = s; return; }
+    if ((s = allow_big_lds(lce_forward_kernel<false, false>)) != VAMD_OK) { status = s; return; }
+    if ((s = allow_big_lds(lce_forward_kernel<false, true>)) != VAMD_OK) { status = s; return; }
+    if ((s = allow_big_lds(lce_forward_kernel<true, false>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) { status = s; return; }
+    if ((s = allow_big_lds(lce_forward_kernel<true, true>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) { status = s; return; }
     if ((s = allow_big_lds(lce_recompute_kernel)) != VAMD_OK) { status = s; return; }
     if ((s = allow_big_lds(lce_dgrad_kernel, kLdsBytes + kCacheStageBytes)) != VAMD_OK) { status = s; return; }
   });
@@ -673,13 +710,14 @@ extern "C" size_t vamd_lce_forward_workspace_bytes(int64_t n_tokens, int64_t hid
   if (n_tokens <= 0 || vocab <= 0) return 0;
   const int64_t tok_tiles = ceil_div(n_tokens, kTile), voc_tiles = ceil_div(vocab, kTile);
   const int sp = fwd_splits(tok_tiles, voc_tiles);
-  return align_up((size_t)sp * tok_tiles * kTile * sizeof(float4), 256);
+  return align_up((size_t)sp * tok_tiles * kTile * sizeof(float4), 256) +
+         align_up((size_t)sp * tok_tiles * kTile * sizeof(float), 256);  // state + squared sums
 }
 
 extern "C" int vamd_lce_forward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
                                 int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs,
-                                float* entropy, float* lse, float* mean_z, float* logits_cache, void* workspace,
-                                size_t workspace_bytes, void* stream) {
+                                float* entropy, float* lse, float* mean_z, float* logits_cache,
+                                float* sum_pi_squared, void* workspace, size_t workspace_bytes, void* stream) {
   int st = check_head_shapes(n_tokens, hidden_size, vocab);
   if (st != VAMD_OK) return st;
   VAMD_REQUIRE(hidden && weight && labels && logprobs && entropy && lse && mean_z, "lce_forward: null pointer");
@@ -704,21 +742,32 @@ extern "C" int vamd_lce_forward(const void* hidden, const void* weight, const in
   a.scale2 = rcp_temperature * kLog2e;
   a.rcp_t = rcp_temperature;
   a.partials = static_cast<float4*>(workspace);
+  a.pi2_partials = sum_pi_squared
+                       ? reinterpret_cast<float*>(static_cast<char*>(workspace) +
+                                                  align_up((size_t)a.splits * a.tok_tiles * kTile * sizeof(float4), 256))
+                       : nullptr;
   a.z_cache = logits_cache;
   VAMD_REQUIRE(reinterpret_cast<uintptr_t>(logits_cache) % 16 == 0, "lce_forward: logits_cache must be 16-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
   {
     ScopedTiming tm(kTagForward, s);
-    if (logits_cache)
-      hipLaunchKernelGGL(lce_forward_kernel<true>, dim3(a.tok_tiles * a.splits), dim3(kThreads),
-                         kLdsBytes + kCacheStageBytes, s, a);
-    else
-      hipLaunchKernelGGL(lce_forward_kernel<false>, dim3(a.tok_tiles * a.splits), dim3(kThreads), kLdsBytes, s, a);
+    const dim3 grid(a.tok_tiles * a.splits), block(kThreads);
+    if (logits_cache) {
+      if (sum_pi_squared)
+        hipLaunchKernelGGL((lce_forward_kernel<true, true>), grid, block, kLdsBytes + kCacheStageBytes, s, a);
+      else
+        hipLaunchKernelGGL((lce_forward_kernel<true, false>), grid, block, kLdsBytes + kCacheStageBytes, s, a);
+    } else {
+      if (sum_pi_squared) hipLaunchKernelGGL((lce_forward_kernel<false, true>), grid, block, kLdsBytes, s, a);
+      else hipLaunchKernelGGL((lce_forward_kernel<false, false>), grid, block, kLdsBytes, s, a);
+    }
   }
   VAMD_LAUNCH_CHECK();
 
   MergeArgs m;
   m.partials = a.partials;
+  m.pi2_partials = a.pi2_partials;
+  m.sum_pi_squared = sum_pi_squared;
   m.splits = a.splits;
   m.stride = a.tok_tiles * kTile;
   m.n_tokens = (int)n_tokens;

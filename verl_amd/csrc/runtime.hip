@@ -55,5 +55,5 @@ extern "C" int vamd_copy_bytes(const void* src, void* dst, int64_t bytes, void* 
   return VAMD_OK;
 }
 
-extern "C" int vamd_abi_version(void) { return 2; }
+extern "C" int vamd_abi_version(void) { return 3; }
 extern "C" const char* vamd_last_error(void) { return vamd::g_error; }

@@ -50,12 +50,14 @@ def logits_cache_budget_bytes() -> int:
 
 
 def efficient_entropy_forward(hidden, weight, labels, reduction: int = 0, temperature: float = 1.0,
-                              dist_process_group=None, logits_cache: torch.Tensor | None = None):
+                              dist_process_group=None, logits_cache: torch.Tensor | None = None,
+                              sum_pi_squared: torch.Tensor | None = None):
     """Host side of the forward kernels (reference kernels.py:563-753).
 
     Returns ``(logprobs, entropy, lse, mean_z)``; the last two are the per-token statistics the
     backward pass needs (log-sum-exp and softmax-weighted mean of the scaled logits).
     ``logits_cache``: optional fp32 ``[tokens, vocab]`` tensor that receives the scaled logits.
+    ``sum_pi_squared``: optional fp32 ``[tokens]`` tensor that receives ``sum_j softmax(z)_j ** 2``.
     """
     if dist_process_group is not None:
         raise NotImplementedError("vocab-parallel process groups are not supported on this single-GPU path")
@@ -73,12 +75,15 @@ def efficient_entropy_forward(hidden, weight, labels, reduction: int = 0, temper
     if logits_cache is not None:
         assert logits_cache.shape == (n, v) and logits_cache.dtype == torch.float32
         assert logits_cache.is_contiguous() and logits_cache.device == dev
+    if sum_pi_squared is not None:
+        assert sum_pi_squared.shape == (n,) and sum_pi_squared.dtype == torch.float32
+        assert sum_pi_squared.is_contiguous() and sum_pi_squared.device == dev
     ws = _cabi.workspace(L.vamd_lce_forward_workspace_bytes(n, h, v), dev)
     with torch.cuda.device(dev):
         _cabi.check(L.vamd_lce_forward(hidden.data_ptr(), weight.data_ptr(), labels.data_ptr(), n, h, v,
                                        1.0 / temperature, logprobs.data_ptr(), entropy.data_ptr(), lse.data_ptr(),
-                                       mean_z.data_ptr(), _cabi.ptr(logits_cache), ws.data_ptr(), ws.numel(),
-                                       _cabi.stream_ptr(dev)))
+                                       mean_z.data_ptr(), _cabi.ptr(logits_cache), _cabi.ptr(sum_pi_squared),
+                                       ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
     if reduction == 1:
         logprobs = _sum_f32(logprobs)
     elif reduction == 2:
@@ -145,6 +150,24 @@ def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse,
                                         d_hidden.data_ptr(), d_weight.data_ptr(), int(accumulate), int(vocab_chunk), ws.data_ptr(),
                                         ws.numel(), _cabi.stream_ptr(dev)))
     return d_hidden, d_weight
+
+
+@torch.no_grad()
+def linear_cross_entropy_with_sum_pi_squared(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor,
+                                             temperature: float = 1.0):
+    """``(logprobs, entropy, sum_pi_squared)`` of the head in one pass, without gradients: what the
+    rollout-statistics pass of the actor needs when the optimal-token-baseline estimator is on
+    (reference verl/workers/actor/dp_actor.py:280-287 computes ``sum_pi_squared`` from materialised
+    logits with ``calculate_sum_pi_squared_from_logits``, verl/utils/torch_functional.py:680-694, and
+    refuses to combine it with its fused kernels, dp_actor.py:107-111).  Outputs are flat fp32
+    ``(num_tokens,)`` tensors."""
+    if hidden.dim() != 2:
+        hidden = hidden.view(-1, hidden.shape[-1])
+    if labels.dim() != 1:
+        labels = labels.view(-1)
+    pi2 = torch.empty((hidden.shape[0],), device=hidden.device, dtype=torch.float32)
+    logprobs, entropy, _, _ = efficient_entropy_forward(hidden, weight, labels, 0, temperature, sum_pi_squared=pi2)
+    return logprobs, entropy, pi2
 
 
 class LinearCrossEntropy(torch.autograd.Function):
