@@ -30,7 +30,7 @@ COPY_YARDSTICK_BYTES = 1 << 30
 # rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by the readings of the 1 GiB copy in the same run
 # (2048 and 1024 bytes per unit); see profiles/head_fwd_bwd_qwen7b_hbm_traffic.md.  Counters cannot be read
 # from inside this process, so the figure is recorded here and only reported for the shape it was measured on.
-MEASURED_TRAFFIC_BYTES = {"lce_dgrad_kernel": 6.42e9 + 0.357e9, "lce_forward_kernel": 31.48e9 + 9.972e9}
+MEASURED_TRAFFIC_BYTES = {"lce_dgrad_kernel": 6.52e9 + 0.353e9, "lce_forward_kernel": 34.03e9 + 9.971e9}
 GEMMS_PER_STEP = {"lce_forward_kernel": 1, "lce_recompute_kernel": 1, "lce_dgrad_kernel": 2}
 
 
