@@ -1,6 +1,7 @@
 """CPU-side checks of the boundary: the shared library loads, exports every symbol that
 include/verl_amd.h declares, answers its size queries, and the host wrappers refuse to run
 without a GPU instead of falling back."""
+import ctypes
 import os
 import re
 
@@ -98,3 +99,10 @@ def test_registries_and_host_logic_without_gpu():
     assert as_torch_index(["5", "6", "5"]).tolist() == [5, 6, 5]
     ids, G = contiguous_group_ids([10, 10, 7, 99])
     assert G == 3 and ids.tolist() == [1, 1, 0, 2]
+
+
+def test_backward_rejects_operands_beyond_32_bit_offsets(lib):
+    """The check runs before any GPU call: dummy non-null pointers are never dereferenced."""
+    p = ctypes.c_void_p(256)
+    rc = lib.vamd_lce_backward(p, p, p, 700000, 3584, 1024, 1.0, p, p, None, None, 0.0, None, p, p, 0, 0, p, 1 << 40, None)
+    assert rc == -1 and b"4 GiB" in lib.vamd_last_error()

@@ -804,6 +804,13 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
   VAMD_REQUIRE(hidden && weight && labels && lse && mean_z && d_hidden && d_weight, "lce_backward: null pointer");
   VAMD_REQUIRE(rcp_temperature > 0.f, "lce_backward: temperature must be positive");
   VAMD_REQUIRE(reinterpret_cast<uintptr_t>(logits_cache) % 16 == 0, "lce_backward: logits_cache must be 16-byte aligned");
+  {  // K-major operands are addressed with 32-bit byte offsets from their tile origin
+    const int64_t rows_padded = ceil_div(n_tokens, kTile) * kTile;
+    const int64_t row_pitch = dz_pitch(default_vocab_chunk(n_tokens, vocab, vocab_chunk));
+    VAMD_REQUIRE(n_tokens * hidden_size * 2 < (1ll << 32) && rows_padded * row_pitch * 2 < (1ll << 32),
+                 "lce_backward: hidden states (%lld x %lld) or the d_logits panel exceed 4 GiB; split the tokens into "
+                 "chunks and accumulate d_weight", (long long)n_tokens, (long long)hidden_size);
+  }
   const size_t need = vamd_lce_backward_workspace_bytes(n_tokens, hidden_size, vocab, vocab_chunk);
   if (!workspace || workspace_bytes < need) {
     set_error("lce_backward: workspace %zu bytes, need %zu", workspace_bytes, need);
