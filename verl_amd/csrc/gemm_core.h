@@ -47,7 +47,7 @@ constexpr int kWavesC = 2;                    // wavefronts along c
 constexpr int kThreads = 64 * kWavesR * kWavesC;
 constexpr int kNB = kTile / 32 / kWavesR;     // 32-row blocks per wavefront    (2)
 constexpr int kMB = kTile / 32 / kWavesC;     // 32-column blocks per wavefront (4)
-constexpr int kLoads = kTile * 8 / kThreads;  // 16-byte staging loads per lane per operand slab (4)
+constexpr int kLoads = kTile * 8 / kThreads;  // 16-byte memory -> LDS transfers per lane per operand slab (4)
 constexpr int kSlabBytes = kTile * kBK * 2;   // 32 KB
 constexpr int kLdsBytes = 4 * kSlabBytes;     // R,C x 2 stages = 128 KB
 static_assert(kNB == 2 && kMB == 4 && kLoads == 4, "slab_iter's slot schedule is written for this layout");

@@ -1,11 +1,13 @@
 // Fused vocab-projection log-prob / entropy head for gfx950.
 //
 // Forward : logits tiles are produced by the MFMA tile engine and consumed in registers by an
-//           online-softmax epilogue (running max, sum exp, sum z*exp, label logit per token);
-//           the [tokens, vocab] logits never reach memory.
-// Backward: logits tiles are recomputed, turned into d_logits tiles in registers and staged as
-//           one bf16 [tokens, vocab_chunk] panel; the same tile engine then forms
-//           d_hidden (+)= panel . W[chunk]  and  d_weight[chunk] = panel^T . hidden.
+//           online-softmax epilogue (running max, sum exp, sum z*exp, label logit and, on request,
+//           sum exp^2 per token).  The [tokens, vocab] logits are not needed afterwards; on request
+//           they are also written out in fp32 as a cache for the backward pass.
+// Backward: per vocabulary chunk, d_logits is formed as one bf16 [tokens, vocab_chunk] panel,
+//           either from the cached logits (a streaming pass) or from logits tiles recomputed by
+//           the tile engine; the same engine then forms
+//           d_hidden (+)= panel . W[chunk]  and  d_weight[chunk] = panel^T . hidden  in one launch.
 //
 // Arithmetic follows LinearCrossEntropy (verl/utils/kernel/linear_cross_entropy.py:40-116) /
 // efficient_entropy_forward+backward (verl/utils/kernel/kernels.py:563-753, :1512-1723): bf16
