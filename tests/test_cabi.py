@@ -106,3 +106,11 @@ def test_backward_rejects_operands_beyond_32_bit_offsets(lib):
     p = ctypes.c_void_p(256)
     rc = lib.vamd_lce_backward(p, p, p, 700000, 3584, 1024, 1.0, p, p, None, None, 0.0, None, p, p, 0, 0, p, 1 << 40, None)
     assert rc == -1 and b"4 GiB" in lib.vamd_last_error()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert res.returncode != 0 and "one GPU" in res.stderr and res.stdout.strip() == ""
