@@ -162,8 +162,16 @@ def test_reductions_3d_input_and_argument_errors(dev):
     wd = weight.to(dev).requires_grad_()
     ld = labels.view(b, s).to(dev)
     lp, ent = linear_cross_entropy(hd, wd, ld, 1.5, "none")
-    assert lp.shape == (b * s,) and ent.shape == (b * s,)                    # flat, like the reference
+    assert lp.shape == (b, s) and ent.shape == (b, s)                        # batch-shaped for batched input
     want_lp, want_ent, want_dh, want_dw = _oracle(hidden, weight, labels, 1.5, torch.ones(b * s), torch.zeros(b * s))
+    assert (lp.reshape(-1) - want_lp.to(dev)).abs().max().item() <= ATOL
+    assert (lp[:, -5:-1].reshape(-1) - want_lp.view(b, s)[:, -5:-1].reshape(-1).to(dev)).abs().max().item() <= ATOL
+    up = torch.randn(b, s, generator=torch.Generator().manual_seed(1)).to(dev)
+    dh_b, = torch.autograd.grad((lp * up).sum(), hd)                         # batch-shaped upstream gradients
+    lp_flat, _ = linear_cross_entropy(hd.view(b * s, h), wd, ld.view(-1), 1.5, "none")
+    assert lp_flat.shape == (b * s,)                                         # flat for 2-D input, like the reference op
+    dh_f, = torch.autograd.grad((lp_flat * up.view(-1)).sum(), hd)
+    assert torch.equal(dh_b, dh_f)
     lp_sum, _ = linear_cross_entropy(hd, wd, ld, 1.5, "sum")
     lp_mean, _ = linear_cross_entropy(hd, wd, ld, 1.5, "MEAN")
     assert lp_sum.dim() == 0 and abs(lp_sum.item() - want_lp.sum().item()) <= ATOL * b * s

@@ -175,9 +175,14 @@ class LinearCrossEntropy(torch.autograd.Function):
 
     hidden ``(..., hidden_size)`` bf16 -> flattened to ``(num_tokens, hidden_size)``;
     weight ``(vocab_size, hidden_size)`` bf16; labels ``(...)`` -> ``(num_tokens,)``.
-    Returns ``(logprobs, entropy)`` as FLAT fp32 ``(num_tokens,)`` tensors (``logprobs`` is a
-    scalar for ``reduction`` "sum" / "mean"), like the reference
-    (verl/utils/kernel/linear_cross_entropy.py:40-87).
+    Returns fp32 ``(logprobs, entropy)`` (``logprobs`` is a scalar for ``reduction`` "sum" /
+    "mean").  For 2-D ``hidden`` (the remove-padding path) they are ``(num_tokens,)`` like the
+    reference's fused op (verl/utils/kernel/linear_cross_entropy.py:40-87).  For ``hidden`` with
+    leading batch dimensions they keep those dimensions, like the reference's torch backend
+    (verl/utils/experimental/torch_functional.py:119-121): the padded caller slices them as
+    ``[:, -response_length - 1 : -1]`` (verl/workers/actor/dp_actor.py:362-363), which the flat
+    shape of the reference's fused op cannot serve, and the remove-padding caller's
+    ``squeeze(0)`` (:254) accepts either.
     """
 
     @staticmethod
@@ -203,11 +208,19 @@ class LinearCrossEntropy(torch.autograd.Function):
         ctx.REDUCTION = REDUCTION
         ctx.dist_process_group = dist_process_group
         ctx.temperature = temperature
+        if len(original_hidden_shape) != 2:
+            entropy = entropy.view(original_hidden_shape[:-1])
+            if REDUCTION == 0:
+                logprobs = logprobs.view(original_hidden_shape[:-1])
         return logprobs, entropy
 
     @staticmethod
     def backward(ctx, dlogprobs: torch.Tensor, dentropy: torch.Tensor):
         hidden, weight, labels, lse, mean_z, cache = ctx.saved_tensors
+        if dentropy is not None:
+            dentropy = dentropy.reshape(-1)
+        if dlogprobs is not None and ctx.REDUCTION == 0:
+            dlogprobs = dlogprobs.reshape(-1)
         d_hidden, d_weight = efficient_entropy_backward(
             dlogprobs, dentropy, hidden, weight, labels, lse, mean_z, ctx.REDUCTION, ctx.temperature,
             ctx.dist_process_group, logits_cache=cache)
