@@ -1,0 +1,117 @@
+"""One actor-update step composed the way the reference's callers compose it, through autograd, on the GPU path
+and on the oracle:
+
+  labels = roll(input_ids, -1)                                   verl/models/transformers/dense_common.py:172-175
+  log_prob, entropy = head(hidden, lm_head.weight, labels, T)    dense_common.py:179-185
+  response slice [:, -L-1:-1]                                    verl/workers/actor/dp_actor.py:362-363
+  old_log_prob = log_prob.detach() when on-policy                dp_actor.py:591-592
+  advantages = GRPO(token_level_rewards, response_mask, uid)     verl/trainer/ppo/ray_trainer.py:178-190
+  pg_loss, metrics = policy_loss_fn(...)                         dp_actor.py:608-616
+  policy_loss = pg_loss - entropy_coeff * agg_loss(entropy)      dp_actor.py:633-638
+  policy_loss += kl_loss_coef * agg_loss(kl_penalty(log_prob, ref_log_prob))   dp_actor.py:640-650
+  (policy_loss * loss_scale_factor).backward()                   dp_actor.py:652-660
+"""
+import types
+
+import numpy as np
+import pytest
+import torch
+
+import oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _cfg():
+    ns = types.SimpleNamespace(clip_ratio=0.2, clip_ratio_low=None, clip_ratio_high=None, clip_ratio_c=3.0,
+                               global_batch_info={})
+    ns.get = lambda k, d=None: getattr(ns, k, d)
+    return ns
+
+
+@pytest.mark.parametrize("mode", ["token-mean", "seq-mean-token-mean"])
+@pytest.mark.parametrize("on_policy", [True, False])
+def test_actor_update_step_matches_the_oracle_composition(dev, mode, on_policy):
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    g = torch.Generator().manual_seed(11)
+    B, S, Lr, H, V, T = 8, 96, 64, 256, 2048, 0.9
+    entropy_coeff, kl_coef, loss_scale = 0.01, 0.05, 0.5
+    input_ids = torch.randint(0, V, (B, S), generator=g)
+    hidden = (torch.randn(B, S, H, generator=g)).bfloat16()
+    weight = (torch.randn(V, H, generator=g) * 0.05).bfloat16()
+    lens = torch.randint(8, Lr + 1, (B,), generator=g)
+    mask = (torch.arange(Lr)[None, :] < lens[:, None]).float()
+    rewards = torch.zeros(B, Lr)
+    rewards[torch.arange(B), lens - 1] = torch.rand(B, generator=g)
+    uid = np.repeat(np.arange(B // 4), 4)
+    ref_lp = -torch.rand(B, Lr, generator=g) * 3
+    old_shift = torch.randn(B, Lr, generator=g) * 0.1
+    labels = torch.roll(input_ids, shifts=-1, dims=-1)
+
+    def run(head, algos, kl_fn, device):
+        h = hidden.to(device).requires_grad_()
+        w = weight.to(device).requires_grad_()
+        lp_full, ent_full = head(h, w, labels.to(device))
+        lp = lp_full[:, -Lr - 1:-1]
+        ent = ent_full[:, -Lr - 1:-1]
+        old = lp.detach() if on_policy else lp.detach() + old_shift.to(device)
+        m = mask.to(device)
+        adv, _ = algos["grpo"](rewards.to(device), m, uid)
+        pg_loss, clipfrac, ppo_kl = algos["policy"](old, lp, adv, m)
+        loss = pg_loss - entropy_coeff * algos["agg"](ent, m)
+        loss = loss + kl_coef * kl_fn(lp, ref_lp.to(device), m)
+        (loss * loss_scale).backward()
+        return dict(lp=lp.detach(), ent=ent.detach(), adv=adv, pg_loss=pg_loss.detach(), loss=loss.detach(),
+                    clipfrac=clipfrac, ppo_kl=ppo_kl, dh=h.grad, dw=w.grad)
+
+    def gpu_policy(old, lp, adv, m):
+        loss, met = CA.compute_policy_loss_vanilla(old_log_prob=old, log_prob=lp, advantages=adv, response_mask=m,
+                                                   loss_agg_mode=mode, config=_cfg(), rollout_is_weights=None)
+        return loss, met["actor/pg_clipfrac"], met["actor/ppo_kl"]
+
+    got = run(lambda h, w, y: linear_cross_entropy(h, w, y, T),
+              dict(grpo=CA.compute_grpo_outcome_advantage, policy=gpu_policy,
+                   agg=lambda x, m: CA.agg_loss(loss_mat=x, loss_mask=m, loss_agg_mode=mode)),
+              lambda lp, ref, m: CA.compute_kl_loss(lp, ref, m, "low_var_kl", mode), dev)
+
+    # oracle side: fp32 ground-truth head with retained upstream gradients
+    kept = {}
+
+    def oracle_head(h, w, y):
+        lp, ent = O.head_fp32_ground_truth(h.view(B * S, H), w, y.view(-1), T)
+        lp = lp.view(B, S); ent = ent.view(B, S)
+        lp.retain_grad(); ent.retain_grad()
+        kept["lp"], kept["ent"] = lp, ent
+        return lp, ent
+
+    def oracle_policy(old, lp, adv, m):
+        out = O.policy_loss_vanilla(old, lp, adv, m, mode)
+        return out[0], out[1].item(), out[2].item()
+
+    want = run(oracle_head,
+               dict(grpo=lambda r, m, i: O.grpo_outcome_advantage(r.clone(), m, i), policy=oracle_policy,
+                    agg=lambda x, m: O.agg_loss(x, m, mode)),
+               lambda lp, ref, m: O.agg_loss(O.kl_penalty(lp, ref, "low_var_kl"), m, mode), "cpu")
+
+    assert (got["lp"].cpu() - want["lp"]).abs().max().item() <= 2e-3
+    assert (got["ent"].cpu() - want["ent"]).abs().max().item() <= 2e-3
+    assert torch.allclose(got["adv"].cpu(), want["adv"], rtol=1e-5, atol=1e-6)
+    # the losses inherit the head's 2e-3 on log-prob / entropy through O(1) derivatives
+    assert abs(got["pg_loss"].item() - want["pg_loss"].item()) <= 2e-3
+    assert abs(got["loss"].item() - want["loss"].item()) <= 4e-3
+    assert abs(got["clipfrac"] - want["clipfrac"]) <= 2.0 / mask.sum().item() + 1e-6
+    assert abs(got["ppo_kl"] - want["ppo_kl"]) <= 2e-3
+    # gradients: the upstream gradients at the head are O(1 / tokens), so the bound is stated relative to the size
+    # of the products that form each entry (d_logits is staged in bf16, outputs are rounded to bf16)
+    g_lp = kept["lp"].grad.reshape(-1)
+    g_ent = kept["ent"].grad.reshape(-1)
+    _, _, ref_dh, ref_dw, e_dh, e_dw = O.head_fwd_bwd_chunked_fp32(hidden.view(B * S, H), weight, labels.view(-1), T, g_lp, g_ent)
+    # closed form == autograd of the ground truth (whose leaf gradients come back rounded to bf16)
+    assert torch.allclose(ref_dh, want["dh"].float().view(B * S, H), rtol=2.0 ** -7, atol=1e-9)
+    for name, got_g, ref_g, e in (("d_hidden", got["dh"].view(B * S, H), ref_dh, e_dh), ("d_weight", got["dw"], ref_dw, e_dw)):
+        err = (got_g.float().cpu() - ref_g).abs()
+        # the head ran on upstream gradients that differ from the oracle's by the 2e-3 of its own outputs: 1 % of E
+        bound = 2.0 ** -8 * ref_g.abs() + (2.0 ** -8 + 1e-2) * e + 1e-9
+        assert (err <= bound).all(), f"{name}: worst excess {(err - bound).max().item():.3e}"
+        assert err.pow(2).mean().sqrt().item() <= 0.02 * ref_g.pow(2).mean().sqrt().item() + 1e-9, name
