@@ -60,17 +60,17 @@ def cpu_baseline(n_cpu: int, h: int, v: int, temperature: float) -> dict:
     }
 
 
-def policy_math_rates(dev, with_cpu: bool) -> dict:
-    """The [B, L] kernels at B = 512, L = 4096 (BASELINE configs 3 and 4): microseconds per call from HIP events over
-    40 calls that rotate through 8 buffer sets (more than the 256 MB Infinity Cache), the algorithmic bytes of the
-    op, and the fraction of 8 TB/s that gives.  ``cpu_ms`` is the CPU oracle on one buffer set."""
+def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> dict:
+    """The [B, L] kernels (B = 512, L = 4096 are BASELINE configs 3 and 4): microseconds per call from HIP events
+    over 40 calls that rotate through 8 buffer sets (more than the 256 MB Infinity Cache), the algorithmic bytes of
+    the op, and the fraction of 8 TB/s that gives.  ``cpu_ms`` is the CPU oracle on one buffer set."""
     import torch
 
     import oracle as O
     from verl_amd import _cabi
 
     L = _cabi.lib()
-    B, Lc, nset = 512, 4096, 8
+    nset = 8
     BL = B * Lc
     g = torch.Generator(device=dev).manual_seed(0)
 
@@ -81,16 +81,17 @@ def policy_math_rates(dev, with_cpu: bool) -> dict:
         return dict(mask=mask, a=t(), b=t(), c=t(), o1=torch.empty(B, Lc, device=dev), o2=torch.empty(B, Lc, device=dev))
 
     sets = [mk() for _ in range(nset)]
-    ws = torch.zeros(1 << 22, dtype=torch.uint8, device=dev)
+    ws = torch.zeros(max(1 << 22, L.vamd_policy_loss_variant_workspace_bytes(B, Lc),
+                         L.vamd_group_outcome_advantage_workspace_bytes(B, Lc, n_groups)), dtype=torch.uint8, device=dev)
     out = torch.empty(8, device=dev)
     coef = torch.empty(B, device=dev)
     mom = torch.empty(4, dtype=torch.float64, device=dev)
-    gid = torch.arange(64, device=dev).repeat_interleave(8)
+    gid = torch.arange(n_groups, device=dev).repeat_interleave(B // n_groups)
     st = _cabi.stream_ptr(dev)
     P = lambda t: t.data_ptr()
     chk = _cabi.check
     ops = {
-        "grpo_advantage": (12 * BL, lambda s: chk(L.vamd_grpo_advantage(P(s["a"]), P(s["mask"]), 0, P(gid), B, Lc, 64, 1e-6, 1, 0, P(s["o1"]), None, P(ws), ws.numel(), st))),
+        "grpo_advantage": (12 * BL, lambda s: chk(L.vamd_grpo_advantage(P(s["a"]), P(s["mask"]), 0, P(gid), B, Lc, n_groups, 1e-6, 1, 0, P(s["o1"]), None, P(ws), ws.numel(), st))),
         "policy_loss_fwd": (16 * BL, lambda s: chk(L.vamd_policy_loss_forward(P(s["a"]), P(s["b"]), P(s["c"]), P(s["mask"]), 0, None, B, Lc, 0.2, 0.2, 3.0, 0, 1.0, -1.0, -1.0, -1.0, P(out), None, None, P(ws), ws.numel(), st))),
         "policy_loss_fwd_grad": (20 * BL, lambda s: chk(L.vamd_policy_loss_forward(P(s["a"]), P(s["b"]), P(s["c"]), P(s["mask"]), 0, None, B, Lc, 0.2, 0.2, 3.0, 0, 1.0, -1.0, -1.0, -1.0, P(out), P(s["o1"]), P(coef), P(ws), ws.numel(), st))),
         "gae_scan_whiten": (28 * BL, lambda s: chk(L.vamd_gae(P(s["a"]), P(s["b"]), P(s["mask"]), 0, B, Lc, 1.0, 0.95, 1, P(s["o1"]), P(s["o2"]), P(mom), P(ws), ws.numel(), st))),
@@ -220,6 +221,8 @@ def main() -> None:
     del hidden, weight
     torch.cuda.empty_cache()
     pm = policy_math_rates(dev, with_cpu=args.cpu_tokens > 0)
+    # the same kernels on 16 x larger tensors, where the fixed ~8 us of the single-launch reduction no longer dominates
+    pm_large = policy_math_rates(dev, with_cpu=False, B=2048, Lc=16384, n_groups=256)
 
     print(json.dumps({
         "metric": "tokens/s fwd+bwd logprob+entropy head @Qwen2.5-7B shape; MFMA util %",
@@ -243,6 +246,7 @@ def main() -> None:
         "roofline": roofline,
         "cpu_baseline": base,
         "policy_math_b512_l4096": pm,
+        "policy_math_b2048_l16384": pm_large,
     }))
 
 

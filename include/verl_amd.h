@@ -6,10 +6,11 @@
  *   - every function is asynchronous on `stream` (a hipStream_t passed as void*), allocates
  *     nothing and keeps no state between calls: scratch comes from the caller through
  *     (workspace, workspace_bytes); the matching *_workspace_bytes() gives the size needed;
- *   - the reductions (masked moments, agg_loss, policy / value loss, GRPO, GAE) finish inside one
- *     launch through a ticket counter in the FIRST 256 BYTES of their workspace: those bytes must
- *     be zero on entry and are zero again when the call has completed, so a caller may zero a
- *     buffer once and reuse it for calls that are ordered on one stream;
+ *   - the reductions (masked moments, agg_loss, policy / value / KL loss, the advantage
+ *     estimators) finish inside one launch through arrival counters in the FIRST
+ *     VAMD_TICKET_BYTES of their workspace: those bytes must be zero on entry and are zero again
+ *     when the call has completed, so a caller may zero a buffer once and reuse it for calls that
+ *     are ordered on one stream;
  *   - return value: 0 on success, a negative VAMD_E* code otherwise; vamd_last_error() returns a
  *     thread-local description of the last failure on the calling thread;
  *   - "mask" arguments come with a VAMD_MASK_* code naming their element type; the value used is
@@ -33,6 +34,8 @@ extern "C" {
 #define VAMD_EINVAL (-1)    /* bad shape / null pointer / unsupported option */
 #define VAMD_EWORKSPACE (-2) /* workspace missing or too small */
 #define VAMD_EHIP (-3)      /* a HIP runtime call failed; see vamd_last_error() */
+
+#define VAMD_TICKET_BYTES 16640 /* 65 arrival counters, 256 bytes apart */
 
 #define VAMD_MASK_F32 0
 #define VAMD_MASK_I64 1

@@ -44,10 +44,11 @@ def test_workspace_queries(lib):
     assert full < 1 << 30                                         # d_logits panel + fp32 d_hidden accumulator
     one = lib.vamd_lce_backward_workspace_bytes(256, 128, 1024, 0)
     assert one == 256 * (1024 + 128) * 2                          # a single padded panel, no accumulator
-    # single-launch reductions: 256-byte ticket header + one record of doubles per 4096-column chunk
-    assert lib.vamd_masked_moments_workspace_bytes(512, 4096) == 256 + 512 * 4 * 8
-    assert lib.vamd_policy_loss_workspace_bytes(512, 4097) == 256 + 512 * 2 * 5 * 8
-    assert lib.vamd_gae_workspace_bytes(512, 4096) >= 256 + 512 * 4 * 8
+    # single-launch reductions: arrival counters (VAMD_TICKET_BYTES) + one record of doubles per 4096-column chunk
+    ticket = 16640
+    assert lib.vamd_masked_moments_workspace_bytes(512, 4096) == ticket + 512 * 4 * 8
+    assert lib.vamd_policy_loss_workspace_bytes(512, 4097) == ticket + 512 * 2 * 5 * 8
+    assert lib.vamd_gae_workspace_bytes(512, 4096) >= ticket + 512 * 4 * 8
 
 
 def test_argument_errors_are_reported_without_touching_the_gpu(lib):

@@ -146,8 +146,8 @@ _ticket_ws: dict[tuple[int, int], torch.Tensor] = {}
 
 
 def ticket_workspace(nbytes: int, device: torch.device) -> torch.Tensor:
-    """Scratch for the single-launch reductions.  Their contract: the first 256 bytes (a ticket
-    counter) are zero on entry and zero again on exit, so one zero-initialised buffer per
+    """Scratch for the single-launch reductions.  Their contract: the first VAMD_TICKET_BYTES (arrival
+    counters) are zero on entry and zero again on exit, so one zero-initialised buffer per
     (device, stream) is kept and reused; kernels on one stream run in order and never share it."""
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr(device))
     need = max(int(nbytes), 4096)

@@ -19,7 +19,10 @@ namespace vamd {
 constexpr int kRcThreads = 256;
 constexpr int kChunk = 4096;  // columns per workgroup
 constexpr int kGroups = kChunk / (kRcThreads * 4);  // float4 groups per thread per input (4)
-constexpr size_t kTicketBytes = 256;
+constexpr int kTicketGroups = 64;   // first-level arrival counters
+constexpr int kTicketStride = 256;  // bytes between counters
+constexpr size_t kTicketBytes = (size_t)(kTicketGroups + 1) * kTicketStride;
+static_assert(kTicketBytes == VAMD_TICKET_BYTES, "the header documents the size of the counter area");
 
 inline int64_t chunks_of(int64_t cols) { return cols <= 0 ? 1 : (cols + kChunk - 1) / kChunk; }
 
@@ -135,17 +138,33 @@ __device__ __forceinline__ double peer_load(const double* p) {
 }
 // Ticket: true in exactly one workgroup of the launch, the one that arrives last.  Thread 0 must
 // have issued its peer_store()s before the call.  The last workgroup calls ticket_reset() when done.
-__device__ __forceinline__ bool last_block_arrives(unsigned* counter) {
-  __shared__ unsigned ticket;
+// Arrivals are counted in two levels -- workgroup b takes a ticket from counter 1 + b % G, and the
+// last arrival of each of the G counters takes one from counter 0 -- because same-address atomics
+// are served one after the other (about 15 ns each here): a single counter costs 8 us for 512
+// workgroups and bounds large launches, G = 64 counters on separate lines cost a few hundred ns.
+__device__ __forceinline__ unsigned ticket_groups() { return gridDim.x < (unsigned)kTicketGroups ? gridDim.x : (unsigned)kTicketGroups; }
+__device__ __forceinline__ bool last_block_arrives(unsigned* counters) {
+  __shared__ unsigned last;
   if (threadIdx.x == 0) {
+    const unsigned n = gridDim.x, G = ticket_groups();
+    const unsigned g = blockIdx.x % G;
+    const unsigned members = (n - g + G - 1) / G;
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    ticket = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned is_last = 0;
+    const unsigned t = __hip_atomic_fetch_add(counters + (1 + g) * (kTicketStride / 4), 1u, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+    if (t == members - 1) {
+      const unsigned t2 = __hip_atomic_fetch_add(counters, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      is_last = t2 == G - 1 ? 1u : 0u;
+    }
+    last = is_last;
   }
   __syncthreads();
-  return ticket == gridDim.x - 1;
+  return last != 0;
 }
-__device__ __forceinline__ void ticket_reset(unsigned* counter) {
-  if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ void ticket_reset(unsigned* counters) {
+  if (threadIdx.x <= ticket_groups())
+    __hip_atomic_store(counters + threadIdx.x * (kTicketStride / 4), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // (mean, rsqrt(var_unbiased + 1e-8), shift) from the masked moments sum(m), sum(v m), sum(v^2 m),
@@ -192,23 +211,36 @@ __device__ void finalize_agg(const double* __restrict__ partials, int64_t rows, 
   for (int i = 0; i <= NV; ++i) tot[i] = 0;
   double seq_mean_sum = 0;  // sum over kept rows of S_i / (M_i + 1e-8)
   double seq_sum = 0;       // sum over kept rows of S_i
-  for (int64_t r = threadIdx.x; r < rows; r += kRcThreads) {
-    double row[NV];
+  // two rows per trip so that their record loads (a round trip to the memory side each) overlap
+  for (int64_t r0 = threadIdx.x; r0 < rows; r0 += 2 * kRcThreads) {
+    const int64_t r1 = r0 + kRcThreads;
+    const bool has1 = r1 < rows;
+    double row[2][NV];
 #pragma unroll
-    for (int i = 0; i < NV; ++i) row[i] = 0;
+    for (int i = 0; i < NV; ++i) row[0][i] = row[1][i] = 0;
     for (int c = 0; c < chunks; ++c) {
-      double t[NV];  // issue the record's loads together, then add
+      double t[2][NV];
 #pragma unroll
-      for (int i = 0; i < NV; ++i) t[i] = peer_load(partials + (r * chunks + c) * NV + i);
+      for (int i = 0; i < NV; ++i) {
+        t[0][i] = peer_load(partials + (r0 * chunks + c) * NV + i);
+        t[1][i] = has1 ? peer_load(partials + (r1 * chunks + c) * NV + i) : 0.0;
+      }
 #pragma unroll
-      for (int i = 0; i < NV; ++i) row[i] += t[i];
+      for (int i = 0; i < NV; ++i) {
+        row[0][i] += t[0][i];
+        row[1][i] += t[1][i];
+      }
     }
 #pragma unroll
-    for (int i = 0; i < NV; ++i) tot[i] += row[i];
-    if (row[1] > 0) {
-      tot[NV] += 1;
-      seq_sum += row[0];
-      seq_mean_sum += (double)((float)row[0] / ((float)row[1] + 1e-8f));
+    for (int k = 0; k < 2; ++k) {
+      if (k == 1 && !has1) break;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) tot[i] += row[k][i];
+      if (row[k][1] > 0) {
+        tot[NV] += 1;
+        seq_sum += row[k][0];
+        seq_mean_sum += (double)((float)row[k][0] / ((float)row[k][1] + 1e-8f));
+      }
     }
   }
   double red[NV + 3];
