@@ -7,10 +7,11 @@
 //     nv' = a nv + b ,  g' = P nv + Q g + R           (a in {0,1})
 // and maps compose associatively, so the recurrence is a prefix "sum" over maps.  A row is cut
 // into segments of 1024 columns walked right to left; inside a segment each of the 256 threads
-// composes its 4 columns, a wavefront scan (shuffles) plus a 4-entry LDS pass yields every
-// thread's incoming state, and the thread then replays its 4 columns to emit the advantages.
-// Loads and stores are float4 and contiguous across the wavefront; the loads of four segments
-// are issued together so that memory latency is paid once per 4096 columns.  The workgroup that
+// composes its 4 columns, a wavefront scan (shuffles) plus an LDS pass over the wavefront totals
+// yields every thread's incoming state, and the thread then replays its 4 columns to emit the
+// advantages.  Loads and stores are float4 and contiguous across the wavefront; four segments are
+// loaded and scanned together, so memory latency, the shuffle chain and the workgroup barrier
+// are paid once per 4096 columns.  The workgroup that
 // finishes last folds the per-row masked moments and writes the whitening statistics, so the
 // whole estimator is two launches (scan, then the elementwise whitening).
 #include "rowchunk.h"
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(kRcThreads) void gae_scan_kernel(const float* __res
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int slot = kRcThreads - 1 - tid;  // thread 0 owns the right-most 4 columns of a segment
-  __shared__ Affine wave_tot[2][4];
+  __shared__ Affine wave_tot[2][kSegBatch][4];
   __shared__ float carry[2][2];
   if (tid == 0) {
     carry[0][0] = 0.f;  // nv
@@ -92,11 +93,14 @@ __global__ __launch_bounds__(kRcThreads) void gae_scan_kernel(const float* __res
         ldmask4<VEC>(mask, i, valid[b], w[b]);
       }
     }
+    // The segments of the batch are scanned together: their wavefront scans are independent (the
+    // shuffles of the four interleave), and one pass over the 16 wavefront totals in walk order
+    // then gives every thread the state entering its 4 columns of each segment.
+    Affine inc[kSegBatch], exc[kSegBatch];
 #pragma unroll
     for (int b = 0; b < kSegBatch; ++b) {
-      const int seg = top - b;
-      if (seg < 0) break;
-      // this thread's 4 columns as one map (right to left: e = 3 .. 0)
+      // this thread's 4 columns as one map (right to left: e = 3 .. 0); segments past the row start
+      // (seg < 0) hold zero masks and stay the identity
       Affine f = affine_identity();
 #pragma unroll
       for (int e = 3; e >= 0; --e) {
@@ -110,30 +114,50 @@ __global__ __launch_bounds__(kRcThreads) void gae_scan_kernel(const float* __res
           f = n;
         }
       }
-      // inclusive scan over the wavefront (lane order = walk order)
-      Affine inc = f;
+      inc[b] = f;
+    }
 #pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        const Affine nb = shfl_up_affine(inc, d);
-        if (lane >= d) inc = compose(inc, nb);
+    for (int d = 1; d < 64; d <<= 1) {
+#pragma unroll
+      for (int b = 0; b < kSegBatch; ++b) {
+        const Affine nb = shfl_up_affine(inc[b], d);
+        if (lane >= d) inc[b] = compose(inc[b], nb);
       }
-      if (lane == 63) wave_tot[par][wave] = inc;
-      Affine exc = shfl_up_affine(inc, 1);
-      if (lane == 0) exc = affine_identity();
-      __syncthreads();
-      // state entering this wavefront, then this thread
-      float nv = carry[par][0], g = carry[par][1];
-      for (int k = 0; k < wave; ++k) {
-        const Affine t = wave_tot[par][k];
+    }
+#pragma unroll
+    for (int b = 0; b < kSegBatch; ++b) {
+      if (lane == 63) wave_tot[par][b][wave] = inc[b];
+      exc[b] = shfl_up_affine(inc[b], 1);
+      if (lane == 0) exc[b] = affine_identity();
+    }
+    __syncthreads();
+    // walk the wavefront totals in order; remember the state where this thread's wavefront starts
+    float nv = carry[par][0], g = carry[par][1];
+    float nv_in[kSegBatch], g_in[kSegBatch];
+#pragma unroll
+    for (int b = 0; b < kSegBatch; ++b) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if (k == wave) {
+          nv_in[b] = nv;
+          g_in[b] = g;
+        }
+        const Affine t = wave_tot[par][b][k];
         const float nv2 = fmaf(t.a, nv, t.b);
         g = fmaf(t.P, nv, fmaf(t.Q, g, t.R));
         nv = nv2;
       }
-      {
-        const float nv2 = fmaf(exc.a, nv, exc.b);
-        g = fmaf(exc.P, nv, fmaf(exc.Q, g, exc.R));
-        nv = nv2;
-      }
+    }
+    if (tid == 0) {
+      carry[par ^ 1][0] = nv;
+      carry[par ^ 1][1] = g;
+    }
+#pragma unroll
+    for (int b = 0; b < kSegBatch; ++b) {
+      const int seg = top - b;
+      if (seg < 0) break;
+      nv = fmaf(exc[b].a, nv_in[b], exc[b].b);
+      g = fmaf(exc[b].P, nv_in[b], fmaf(exc[b].Q, g_in[b], exc[b].R));
       // replay the 4 columns
       float a_out[4], r_out[4];
 #pragma unroll
@@ -150,18 +174,13 @@ __global__ __launch_bounds__(kRcThreads) void gae_scan_kernel(const float* __res
         a_out[e] = g;
         r_out[e] = g + v[b][e];
       }
-      if (tid == kRcThreads - 1) {
-        carry[par ^ 1][0] = nv;
-        carry[par ^ 1][1] = g;
-      }
       if (valid[b] > 0) {
         const int64_t i = row * cols + (int64_t)seg * kSeg + slot * 4;
         st4<VEC>(adv, i, valid[b], a_out);
         st4<VEC>(ret, i, valid[b], r_out);
       }
-      __syncthreads();
-      par ^= 1;
     }
+    par ^= 1;
   }
   __shared__ double smem[16];
   double acc[4] = {m0, m1, m2, mc};
