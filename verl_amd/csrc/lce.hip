@@ -617,19 +617,25 @@ static int allow_big_lds(K kernel, int bytes = kLdsBytes) {
   return VAMD_OK;
 }
 
+// The kernels use more LDS than the default launch limit; the limit is a per-device function
+// attribute, so it is raised once on every device the library is used on.
 static int ensure_lds_attributes() {
-  static std::once_flag once;
-  static int status = VAMD_OK;
-  std::call_once(once, [] {
-    int s;
-    if ((s = allow_big_lds(lce_forward_kernel<false, false>)) != VAMD_OK) { status = s; return; }
-    if ((s = allow_big_lds(lce_forward_kernel<false, true>)) != VAMD_OK) { status = s; return; }
-    if ((s = allow_big_lds(lce_forward_kernel<true, false>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) { status = s; return; }
-    if ((s = allow_big_lds(lce_forward_kernel<true, true>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) { status = s; return; }
-    if ((s = allow_big_lds(lce_recompute_kernel)) != VAMD_OK) { status = s; return; }
-    if ((s = allow_big_lds(lce_dgrad_kernel, kLdsBytes + kCacheStageBytes)) != VAMD_OK) { status = s; return; }
-  });
-  return status;
+  static std::mutex mu;
+  static bool done[64];
+  int dev = 0;
+  VAMD_HIP(hipGetDevice(&dev));
+  VAMD_REQUIRE(dev >= 0 && dev < 64, "lce: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (done[dev]) return VAMD_OK;
+  int s;
+  if ((s = allow_big_lds(lce_forward_kernel<false, false>)) != VAMD_OK) return s;
+  if ((s = allow_big_lds(lce_forward_kernel<false, true>)) != VAMD_OK) return s;
+  if ((s = allow_big_lds(lce_forward_kernel<true, false>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) return s;
+  if ((s = allow_big_lds(lce_forward_kernel<true, true>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) return s;
+  if ((s = allow_big_lds(lce_recompute_kernel)) != VAMD_OK) return s;
+  if ((s = allow_big_lds(lce_dgrad_kernel, kLdsBytes + kCacheStageBytes)) != VAMD_OK) return s;
+  done[dev] = true;
+  return VAMD_OK;
 }
 
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
