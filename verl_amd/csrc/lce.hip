@@ -335,6 +335,36 @@ __device__ __forceinline__ u32x2 pack_bf16x4(float a, float b, float c, float d)
 
 __device__ __forceinline__ float bf16_bits_to_float(unsigned h) { return __uint_as_float(h << 16); }
 
+// The backward epilogues hand each 32 x 32 accumulator block through a 4 KB LDS patch private to the
+// wavefront (the 32 KB the pipeline leaves free), so that global accesses are whole 128-byte rows
+// of fp32 (64-byte rows of bf16) touched by 8 consecutive lanes instead of 16-byte pieces of 32
+// different rows.  After the exchange lane L holds columns 4 (L % 8) .. + 3 of rows 8 i + L / 8.
+struct BlockExchange {
+  char* stage;  // this wavefront's patch
+  int lr, lh, rd_row, rd_chunk;
+  __device__ __forceinline__ void init(char* lds_after_pipeline, const LanePos& p) {
+    stage = lds_after_pipeline + (threadIdx.x >> 6) * 4096;
+    lr = p.lr;
+    lh = p.lh;
+    rd_row = (threadIdx.x & 63) >> 3;
+    rd_chunk = threadIdx.x & 7;
+  }
+  __device__ __forceinline__ void run(const f32x16& blk, f32x4 (&out)[4]) const {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 v = {blk[4 * g], blk[4 * g + 1], blk[4 * g + 2], blk[4 * g + 3]};
+      *reinterpret_cast<f32x4*>(stage + lr * 128 + (((2 * g + lh) ^ ((lr >> 1) & 7)) << 4)) = v;
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 8 * i + rd_row;
+      out[i] = *reinterpret_cast<const f32x4*>(stage + row * 128 + ((rd_chunk ^ ((row >> 1) & 7)) << 4));
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+};
+
 struct RecomputeArgs {
   Operand hidden;  // R: [n_tokens][H]
   Operand weight;  // C: rows of this vocabulary chunk, x_extent = vocab - chunk_c0
@@ -355,6 +385,7 @@ struct RecomputeArgs {
 struct RecomputeEpi {
   LanePos p;
   const RecomputeArgs* a;
+  BlockExchange ex;
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const RecomputeArgs& A = *a;
 #pragma unroll
@@ -371,26 +402,29 @@ struct RecomputeEpi {
         rel = (int)A.labels[tok] - A.chunk_c0 - c0 - p.wc * 128;
       }
       const bool hit = __any(rel >= 0 && rel < 128);
-      uint16_t* out_row = A.dz + (int64_t)tok * A.dz_ld + c0;
 #pragma unroll
-      for (int mb = 0; mb < kMB; ++mb)
+      for (int mb = 0; mb < kMB; ++mb) {
+        f32x16 d;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          float d[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float x = acc.a[mb][nb][4 * g + e];
-            const float prob = fast_exp2(fmaf(x, A.scale2, -lse2));
-            const float u = fmaf(gent, fmaf(x, A.rcp_t, -mz), glp);  // g_lp/T + g_ent/T * (z - mean_z)
-            float dzv = -prob * u;
-            const int col = mb * 32 + 8 * g + 4 * p.lh + e;
-            if (hit) dzv += (col == rel) ? glp : 0.f;
-            const bool ok = live && (c0 + p.wc * 128 + col) < A.vocab_left;
-            d[e] = ok ? dzv : 0.f;
-          }
-          const int col0 = p.wc * 128 + mb * 32 + 8 * g + 4 * p.lh;
-          *reinterpret_cast<u32x2*>(out_row + col0) = pack_bf16x4(d[0], d[1], d[2], d[3]);
+        for (int v = 0; v < 16; ++v) {
+          const float x = acc.a[mb][nb][v];
+          const float prob = fast_exp2(fmaf(x, A.scale2, -lse2));
+          const float u = fmaf(gent, fmaf(x, A.rcp_t, -mz), glp);  // g_lp/T + g_ent/T * (z - mean_z)
+          float dzv = -prob * u;
+          const int col = mb * 32 + 8 * (v >> 2) + 4 * p.lh + (v & 3);
+          if (hit) dzv += (col == rel) ? glp : 0.f;
+          const bool ok = live && (c0 + p.wc * 128 + col) < A.vocab_left;
+          d[v] = ok ? dzv : 0.f;
         }
+        // every row of the panel is written, padding rows and columns as zeros
+        f32x4 o[4];
+        ex.run(d, o);
+        const int col0 = c0 + p.wc * 128 + mb * 32 + 4 * ex.rd_chunk;
+        const int64_t row0 = r0 + p.wr * (kNB * 32) + nb * 32 + ex.rd_row;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          *reinterpret_cast<u32x2*>(A.dz + (row0 + 8 * i) * A.dz_ld + col0) = pack_bf16x4(o[i][0], o[i][1], o[i][2], o[i][3]);
+      }
     }
   }
 };
@@ -405,6 +439,7 @@ __global__ __launch_bounds__(kThreads) void lce_recompute_kernel(RecomputeArgs a
   RecomputeEpi epi;
   epi.p = lane_pos();
   epi.a = &a;
+  epi.ex.init(lds + kLdsBytes, epi.p);
   run_tiles<false, false>(a.hidden, a.weight, a.k_slabs, sched, epi, lds);
 }
 
@@ -464,36 +499,6 @@ struct GemmOutArgs {
   float* acc32;          // fp32 accumulator [r_valid][ld_out] (d_hidden only)
   uint16_t* out;         // bf16 output
   int64_t ld_out;
-};
-
-// Both gradient epilogues hand each 32 x 32 accumulator block through a 4 KB LDS patch private to the
-// wavefront (the 32 KB the pipeline leaves free), so that global accesses are whole 128-byte rows
-// of fp32 (64-byte rows of bf16) touched by 8 consecutive lanes instead of 16-byte pieces of 32
-// different rows.  After the exchange lane L holds columns 4 (L % 8) .. + 3 of rows 8 i + L / 8.
-struct BlockExchange {
-  char* stage;  // this wavefront's patch
-  int lr, lh, rd_row, rd_chunk;
-  __device__ __forceinline__ void init(char* lds_after_pipeline, const LanePos& p) {
-    stage = lds_after_pipeline + (threadIdx.x >> 6) * 4096;
-    lr = p.lr;
-    lh = p.lh;
-    rd_row = (threadIdx.x & 63) >> 3;
-    rd_chunk = threadIdx.x & 7;
-  }
-  __device__ __forceinline__ void run(const f32x16& blk, f32x4 (&out)[4]) const {
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 v = {blk[4 * g], blk[4 * g + 1], blk[4 * g + 2], blk[4 * g + 3]};
-      *reinterpret_cast<f32x4*>(stage + lr * 128 + (((2 * g + lh) ^ ((lr >> 1) & 7)) << 4)) = v;
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = 8 * i + rd_row;
-      out[i] = *reinterpret_cast<const f32x4*>(stage + row * 128 + ((rd_chunk ^ ((row >> 1) & 7)) << 4));
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  }
 };
 
 struct DHiddenEpi {
@@ -632,7 +637,7 @@ static int ensure_lds_attributes() {
   if ((s = allow_big_lds(lce_forward_kernel<false, true>)) != VAMD_OK) return s;
   if ((s = allow_big_lds(lce_forward_kernel<true, false>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) return s;
   if ((s = allow_big_lds(lce_forward_kernel<true, true>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) return s;
-  if ((s = allow_big_lds(lce_recompute_kernel)) != VAMD_OK) return s;
+  if ((s = allow_big_lds(lce_recompute_kernel, kLdsBytes + kCacheStageBytes)) != VAMD_OK) return s;
   if ((s = allow_big_lds(lce_dgrad_kernel, kLdsBytes + kCacheStageBytes)) != VAMD_OK) return s;
   done[dev] = true;
   return VAMD_OK;
@@ -893,7 +898,7 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
         const int grid = tiles < cus ? tiles : cus;
         {
           ScopedTiming tm(kTagRecompute, s);
-          hipLaunchKernelGGL(lce_recompute_kernel, dim3(grid), dim3(kThreads), kLdsBytes, s, r);
+          hipLaunchKernelGGL(lce_recompute_kernel, dim3(grid), dim3(kThreads), kLdsBytes + kCacheStageBytes, s, r);
         }
         VAMD_LAUNCH_CHECK();
       }
