@@ -78,27 +78,61 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
         lens = torch.randint(64, Lc + 1, (B,), device=dev, generator=g)
         mask = (torch.arange(Lc, device=dev)[None, :] < lens[:, None]).float()
         t = lambda: torch.randn(B, Lc, device=dev, generator=g)
-        return dict(mask=mask, a=t(), b=t(), c=t(), o1=torch.empty(B, Lc, device=dev), o2=torch.empty(B, Lc, device=dev))
+        return dict(mask=mask, a=t(), b=t(), c=t(), o1=torch.empty(B, Lc, device=dev),
+                    o2=torch.empty(B, Lc, device=dev))
 
     sets = [mk() for _ in range(nset)]
-    ws = torch.zeros(max(1 << 22, L.vamd_policy_loss_variant_workspace_bytes(B, Lc),
-                         L.vamd_group_outcome_advantage_workspace_bytes(B, Lc, n_groups)), dtype=torch.uint8, device=dev)
+    ws_bytes = max(1 << 22, L.vamd_policy_loss_variant_workspace_bytes(B, Lc),
+                   L.vamd_group_outcome_advantage_workspace_bytes(B, Lc, n_groups))
+    ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
     out = torch.empty(8, device=dev)
     coef = torch.empty(B, device=dev)
     mom = torch.empty(4, dtype=torch.float64, device=dev)
     gid = torch.arange(n_groups, device=dev).repeat_interleave(B // n_groups)
     st = _cabi.stream_ptr(dev)
-    P = lambda t: t.data_ptr()
     chk = _cabi.check
+    wsp, wsn = ws.data_ptr(), ws.numel()
+    none3 = (-1.0, -1.0, -1.0)   # agg_loss: batch_num_tokens, global_batch_size, loss_scale_factor not given
+
+    def P(s, *names):
+        return tuple(s[n].data_ptr() for n in names)
+
+    def grpo(s):
+        chk(L.vamd_grpo_advantage(*P(s, "a", "mask"), 0, gid.data_ptr(), B, Lc, n_groups, 1e-6, 1, 0, *P(s, "o1"), None,
+                                  wsp, wsn, st))
+
+    def policy(s, grad):
+        outs = (*P(s, "o1"), coef.data_ptr()) if grad else (None, None)
+        chk(L.vamd_policy_loss_forward(*P(s, "a", "b", "c", "mask"), 0, None, B, Lc, 0.2, 0.2, 3.0, 0, 1.0, *none3,
+                                       out.data_ptr(), *outs, wsp, wsn, st))
+
+    def gae(s):
+        chk(L.vamd_gae(*P(s, "a", "b", "mask"), 0, B, Lc, 1.0, 0.95, 1, *P(s, "o1", "o2"), mom.data_ptr(), wsp, wsn, st))
+
+    def value(s):
+        chk(L.vamd_value_loss_forward(*P(s, "a", "b", "c", "mask"), 0, B, Lc, 0.5, 0, out.data_ptr(), *P(s, "o1"),
+                                      coef.data_ptr(), wsp, wsn, st))
+
+    def kl(s):
+        chk(L.vamd_kl_loss_forward(*P(s, "a", "b", "mask"), 0, B, Lc, 3, 0, 0, 1.0, *none3, out.data_ptr(), *P(s, "o1"),
+                                   coef.data_ptr(), wsp, wsn, st))
+
+    def moments(s):
+        chk(L.vamd_masked_moments(*P(s, "a", "mask"), 0, B, Lc, 0, mom.data_ptr(), wsp, wsn, st))
+
+    def copy(s):
+        chk(L.vamd_copy_bytes(*P(s, "a", "o1"), 4 * BL, st))
+
+    # name -> (algorithmic bytes per call, call)
     ops = {
-        "grpo_advantage": (12 * BL, lambda s: chk(L.vamd_grpo_advantage(P(s["a"]), P(s["mask"]), 0, P(gid), B, Lc, n_groups, 1e-6, 1, 0, P(s["o1"]), None, P(ws), ws.numel(), st))),
-        "policy_loss_fwd": (16 * BL, lambda s: chk(L.vamd_policy_loss_forward(P(s["a"]), P(s["b"]), P(s["c"]), P(s["mask"]), 0, None, B, Lc, 0.2, 0.2, 3.0, 0, 1.0, -1.0, -1.0, -1.0, P(out), None, None, P(ws), ws.numel(), st))),
-        "policy_loss_fwd_grad": (20 * BL, lambda s: chk(L.vamd_policy_loss_forward(P(s["a"]), P(s["b"]), P(s["c"]), P(s["mask"]), 0, None, B, Lc, 0.2, 0.2, 3.0, 0, 1.0, -1.0, -1.0, -1.0, P(out), P(s["o1"]), P(coef), P(ws), ws.numel(), st))),
-        "gae_scan_whiten": (28 * BL, lambda s: chk(L.vamd_gae(P(s["a"]), P(s["b"]), P(s["mask"]), 0, B, Lc, 1.0, 0.95, 1, P(s["o1"]), P(s["o2"]), P(mom), P(ws), ws.numel(), st))),
-        "value_loss_fwd_grad": (20 * BL, lambda s: chk(L.vamd_value_loss_forward(P(s["a"]), P(s["b"]), P(s["c"]), P(s["mask"]), 0, B, Lc, 0.5, 0, P(out), P(s["o1"]), P(coef), P(ws), ws.numel(), st))),
-        "kl_loss_fwd_grad": (16 * BL, lambda s: chk(L.vamd_kl_loss_forward(P(s["a"]), P(s["b"]), P(s["mask"]), 0, B, Lc, 3, 0, 0, 1.0, -1.0, -1.0, -1.0, P(out), P(s["o1"]), P(coef), P(ws), ws.numel(), st))),
-        "masked_moments": (8 * BL, lambda s: chk(L.vamd_masked_moments(P(s["a"]), P(s["mask"]), 0, B, Lc, 0, P(mom), P(ws), ws.numel(), st))),
-        "copy_yardstick": (8 * BL, lambda s: chk(L.vamd_copy_bytes(P(s["a"]), P(s["o1"]), 4 * BL, st))),
+        "grpo_advantage": (12 * BL, grpo),
+        "policy_loss_fwd": (16 * BL, lambda s: policy(s, False)),
+        "policy_loss_fwd_grad": (20 * BL, lambda s: policy(s, True)),
+        "gae_scan_whiten": (28 * BL, gae),
+        "value_loss_fwd_grad": (20 * BL, value),
+        "kl_loss_fwd_grad": (16 * BL, kl),
+        "masked_moments": (8 * BL, moments),
+        "copy_yardstick": (8 * BL, copy),
     }
     res = {}
     for name, (nbytes, fn) in ops.items():
@@ -113,7 +147,8 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
         e1.record()
         torch.cuda.synchronize()
         us = e0.elapsed_time(e1) / reps * 1e3
-        res[name] = {"us": us, "algorithmic_bytes": nbytes, "GBps": nbytes / us / 1e3, "frac_of_8TBps": nbytes / us / 1e3 / 8000.0}
+        gbps = nbytes / us / 1e3
+        res[name] = {"us": us, "algorithmic_bytes": nbytes, "GBps": gbps, "frac_of_8TBps": gbps / 8000.0}
     if with_cpu:
         s = {k: v.cpu() for k, v in sets[0].items()}
         idx = gid.cpu().numpy()
@@ -125,8 +160,10 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
 
         res["grpo_advantage"]["cpu_ms"] = cpu_ms(lambda: O.grpo_outcome_advantage(s["a"].clone(), s["mask"], idx))
         res["gae_scan_whiten"]["cpu_ms"] = cpu_ms(lambda: O.gae_advantage_return(s["a"], s["b"], s["mask"], 1.0, 0.95))
-        res["policy_loss_fwd"]["cpu_ms"] = cpu_ms(lambda: O.policy_loss_vanilla(s["a"], s["b"], s["c"], s["mask"], "token-mean"))
-        res["value_loss_fwd_grad"]["cpu_ms"] = cpu_ms(lambda: O.value_loss(s["a"], s["b"], s["c"], s["mask"], 0.5, "token-mean"))
+        res["policy_loss_fwd"]["cpu_ms"] = cpu_ms(
+            lambda: O.policy_loss_vanilla(s["a"], s["b"], s["c"], s["mask"], "token-mean"))
+        res["value_loss_fwd_grad"]["cpu_ms"] = cpu_ms(
+            lambda: O.value_loss(s["a"], s["b"], s["c"], s["mask"], 0.5, "token-mean"))
     return res
 
 

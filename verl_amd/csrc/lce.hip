@@ -423,7 +423,8 @@ struct RecomputeEpi {
         const int64_t row0 = r0 + p.wr * (kNB * 32) + nb * 32 + ex.rd_row;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          *reinterpret_cast<u32x2*>(A.dz + (row0 + 8 * i) * A.dz_ld + col0) = pack_bf16x4(o[i][0], o[i][1], o[i][2], o[i][3]);
+          *reinterpret_cast<u32x2*>(A.dz + (row0 + 8 * i) * A.dz_ld + col0) =
+              pack_bf16x4(o[i][0], o[i][1], o[i][2], o[i][3]);
       }
     }
   }

@@ -142,7 +142,9 @@ __device__ __forceinline__ double peer_load(const double* p) {
 // last arrival of each of the G counters takes one from counter 0 -- because same-address atomics
 // are served one after the other (about 15 ns each here): a single counter costs 8 us for 512
 // workgroups and bounds large launches, G = 64 counters on separate lines cost a few hundred ns.
-__device__ __forceinline__ unsigned ticket_groups() { return gridDim.x < (unsigned)kTicketGroups ? gridDim.x : (unsigned)kTicketGroups; }
+__device__ __forceinline__ unsigned ticket_groups() {
+  return gridDim.x < (unsigned)kTicketGroups ? gridDim.x : (unsigned)kTicketGroups;
+}
 __device__ __forceinline__ bool last_block_arrives(unsigned* counters) {
   __shared__ unsigned last;
   if (threadIdx.x == 0) {

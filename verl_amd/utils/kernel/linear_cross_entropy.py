@@ -147,8 +147,8 @@ def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse,
         _cabi.check(L.vamd_lce_backward(hidden.data_ptr(), weight.data_ptr(), labels.data_ptr(), n, h, v,
                                         1.0 / temperature, lse.data_ptr(), mean_z.data_ptr(), _cabi.ptr(dlogprobs),
                                         _cabi.ptr(dentropy), float(d_entropy_scalar), _cabi.ptr(logits_cache),
-                                        d_hidden.data_ptr(), d_weight.data_ptr(), int(accumulate), int(vocab_chunk), ws.data_ptr(),
-                                        ws.numel(), _cabi.stream_ptr(dev)))
+                                        d_hidden.data_ptr(), d_weight.data_ptr(), int(accumulate), int(vocab_chunk),
+                                        ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
     return d_hidden, d_weight
 
 
