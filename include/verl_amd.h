@@ -62,6 +62,8 @@ extern "C" {
 #define VAMD_ADV_MEAN_BASELINE 3   /* s - mean: REINFORCE++ baseline before its whitening */
 #define VAMD_ADV_OPO 4             /* s - sum(len s) / sum(len), len = response length */
 #define VAMD_ADV_GPG 5             /* alpha (s - mean) / f_norm, alpha = batch / max(#{s != 0}, 1) */
+#define VAMD_ADV_GRPO_PASSK 6      /* best response of a group: (max - second max) [/ (std + eps)]; others 0;
+                                      every group needs at least two responses (checked by the caller) */
 
 /* policy-loss variants of the registry (core_algos.py:1159-1447, :1721-1779) */
 #define VAMD_PL_VANILLA 0 /* clipped PPO with the dual-clip floor */

@@ -48,6 +48,7 @@ from .advantages import (  # noqa: F401
     gpg_outcome_advantage,
     reinforce_plus_plus_outcome_advantage,
     remax_outcome_advantage,
+    grpo_passk_outcome_advantage,
 )
 from .losses import (  # noqa: F401
     agg_loss,

@@ -300,3 +300,24 @@ def remax_outcome_advantage(token_level_rewards, reward_baselines, response_mask
     returns = (token_level_rewards * response_mask).flip(dims=[-1]).cumsum(dim=-1).flip(dims=[-1])
     advantages = returns - reward_baselines.unsqueeze(-1) * response_mask
     return advantages, returns
+
+
+@torch.no_grad()
+def grpo_passk_outcome_advantage(token_level_rewards, response_mask, index, epsilon=1e-6, norm_by_std=True):
+    """Pass@k, core_algos.py:360-418: per group the two largest scores (``torch.topk``); the response holding
+    the largest gets ``max - second max`` (divided by the group's unbiased std plus epsilon when
+    ``norm_by_std``), every other response 0; a group of fewer than two responses raises ``ValueError``."""
+    scores = token_level_rewards.sum(dim=-1)
+    advantages = torch.zeros_like(scores)
+    members = _group_members(scores, index)
+    for key, rows in members.items():
+        rewards = torch.stack([scores[i] for i in rows])
+        if rewards.numel() < 2:
+            raise ValueError(f"Pass@k requires at least 2 samples per group. Got {rewards.numel()} for group {key}.")
+        topk, topk_idx = torch.topk(rewards, 2)
+        advantage = topk[0] - topk[1]
+        if norm_by_std:
+            advantage = advantage / (torch.std(rewards) + epsilon)
+        advantages[rows[topk_idx[0].item()]] = advantage
+    advantages = advantages.unsqueeze(-1) * response_mask
+    return advantages, advantages

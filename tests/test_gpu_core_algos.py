@@ -409,6 +409,29 @@ def test_group_outcome_estimators_by_hand(dev):
         CA.compute_rloo_outcome_advantage(rewards.to(dev), mask.to(dev), index[:3])
 
 
+@pytest.mark.parametrize("batch_size,seq_len,num_groups,seed", GOLDEN["grpo_equivalence_grid"]["cases"])
+@pytest.mark.parametrize("norm", [True, False])
+def test_grpo_passk(dev, batch_size, seq_len, num_groups, seed, norm):
+    from verl_amd.trainer.ppo import core_algos as CA
+    torch.manual_seed(seed); random.seed(seed); np.random.seed(seed)
+    index = _make_group_index(batch_size, num_groups)
+    mask = _rand_mask(batch_size, seq_len)
+    rewards = torch.randn(batch_size, seq_len) * mask
+    cfg = _cfg(norm_adv_by_std_in_grpo=norm)
+    got, got2 = CA.compute_grpo_passk_outcome_advantage(rewards.to(dev), mask.to(dev), index, config=cfg)
+    want, _ = O.grpo_passk_outcome_advantage(rewards.clone(), mask, index, norm_by_std=norm)
+    assert got is got2
+    _close(got, want, atol=2e-5, what="pass@k")
+    assert torch.equal(got.cpu() != 0, want != 0)               # the same single response per group is rewarded
+    assert int((got.cpu().abs().sum(-1) != 0).sum()) == num_groups
+    lonely = index.copy(); lonely[0] = num_groups + 5
+    with pytest.raises(ValueError, match="at least 2 samples"):
+        CA.compute_grpo_passk_outcome_advantage(rewards.to(dev), mask.to(dev), lonely, config=cfg)
+    with pytest.raises(AssertionError):
+        CA.compute_grpo_passk_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    assert CA.get_adv_estimator_fn("grpo_passk") is CA.compute_grpo_passk_outcome_advantage
+
+
 @pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192)])
 @pytest.mark.parametrize("mdtype", [torch.float32, torch.int64])
 def test_reinforce_plus_plus_and_remax(dev, shape, mdtype):

@@ -310,3 +310,20 @@ def test_sum_pi_squared_closed_forms():
     z = torch.randn(5, 33, generator=g, dtype=torch.float64) * 3
     assert torch.allclose(M.sum_pi_squared_from_logits(z), (torch.softmax(z, -1) ** 2).sum(-1), rtol=1e-12)  # brute force
     assert torch.allclose(M.sum_pi_squared_from_logits(z + 7.5), M.sum_pi_squared_from_logits(z), rtol=1e-12)  # shift
+
+
+def test_grpo_passk_by_hand():
+    rewards, mask, _ = _scores_groups()                               # scores 3, 0.5, 6, 0, 6
+    index = np.array(["a", "a", "a", "b", "b"], dtype=object)         # groups {3, 0.5, 6} and {0, 6}
+    adv, adv2 = A.grpo_passk_outcome_advantage(rewards, mask, index, norm_by_std=False)
+    assert adv is adv2
+    assert torch.equal(adv[2], 3.0 * mask[2]) and torch.equal(adv[4], 6.0 * mask[4])      # max - second max
+    assert adv[[0, 1, 3]].abs().sum().item() == 0
+    adv, _ = A.grpo_passk_outcome_advantage(rewards, mask, index)
+    std_a = torch.tensor([3.0, 0.5, 6.0]).std()
+    assert torch.allclose(adv[2], 3.0 / (std_a + 1e-6) * mask[2])
+    assert torch.allclose(adv[4], 6.0 / (6.0 / math.sqrt(2) + 1e-6) * mask[4])
+    tied = rewards.clone(); tied[0] = tied[2]                         # best score held twice: the advantage is 0
+    assert A.grpo_passk_outcome_advantage(tied, mask, index)[0][:3].abs().sum().item() == 0
+    with pytest.raises(ValueError):
+        A.grpo_passk_outcome_advantage(rewards, mask, np.array(["a", "a", "a", "b", "c"], dtype=object))

@@ -521,6 +521,8 @@ struct GrpoArgs {
 //   MEAN_BASELINE    s - mean (REINFORCE++ baseline before its whitening)         :421-474
 //   OPO              s - sum(len s) / sum(len), len = response length             :531-579
 //   GPG              alpha (s - mean) / f_norm, alpha = rows / max(#{s != 0}, 1)  :657-717
+//   GRPO_PASSK       (max - second max) [/ (std + eps)] for the best response of a group, 0 for
+//                    the others                                                   :360-418
 // A single-member group has mean 0 (and std 1) in every estimator.
 // std_mode 0: unbiased torch.std; 1: sqrt(clamp(var, min=eps)) of group_mean_std.  Singleton
 // groups get mean 0, std 1 (core_algos.py:314-316, groupwise.py:215-221).
@@ -570,11 +572,38 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rowsum_kernel(const float* __
     }
   }
   __syncthreads();
-  if (ga.estimator == VAMD_ADV_GRPO) {
+  if (ga.estimator == VAMD_ADV_GRPO || ga.estimator == VAMD_ADV_GRPO_PASSK) {
     for (int64_t r = threadIdx.x; r < ga.rows; r += kRcThreads) {
       const int64_t g = ga.gid[r];
       const double d = (double)ga.scores[r] - g_sum[g] / (double)g_cnt[g];
       atomicAdd(&g_sq[g], d * d);
+    }
+    __syncthreads();
+  }
+  if (ga.estimator == VAMD_ADV_GRPO_PASSK) {
+    // one thread per group walks the responses in index order: best score (first index on ties,
+    // where the advantage is 0 anyway), runner-up, unbiased std; the group's entry of `mean`
+    // receives the advantage and the entry of `stdv` the index of the best response
+    __syncthreads();
+    for (int64_t g = threadIdx.x; g < ga.n_groups; g += kRcThreads) {
+      float best = -INFINITY, second = -INFINITY;
+      int64_t arg = -1;
+      for (int64_t r = 0; r < ga.rows; ++r) {
+        if (ga.gid[r] != g) continue;
+        const float sc = ga.scores[r];
+        if (sc > best) {
+          second = best;
+          best = sc;
+          arg = r;
+        } else if (sc > second) {
+          second = sc;
+        }
+      }
+      const int c = g_cnt[g];
+      float a = best - second;
+      if (ga.norm_by_std) a = a / ((float)sqrt(g_sq[g] / (double)(c - 1)) + ga.eps);
+      g_sum[g] = (double)a;
+      g_sq[g] = (double)arg;
     }
     __syncthreads();
   }
@@ -619,6 +648,9 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rowsum_kernel(const float* __
         break;
       case VAMD_ADV_GPG:
         out = alpha * (sc - (c > 1 ? (float)(g_sum[g] / (double)c) : 0.f)) / ga.f_norm;
+        break;
+      case VAMD_ADV_GRPO_PASSK:
+        out = (double)r == g_sq[g] ? (float)g_sum[g] : 0.f;
         break;
       default:  // VAMD_ADV_MEAN_BASELINE
         out = sc - (c > 1 ? (float)(g_sum[g] / (double)c) : 0.f);
@@ -1101,7 +1133,7 @@ extern "C" int vamd_group_outcome_advantage(const float* rewards, const void* ma
   int st = check_matrix("group_outcome_advantage", batch, length);
   if (st != VAMD_OK) return st;
   VAMD_REQUIRE(rewards && mask && group_ids && advantages && n_groups > 0, "group_outcome_advantage: bad argument");
-  VAMD_REQUIRE(estimator >= VAMD_ADV_GRPO && estimator <= VAMD_ADV_GPG, "group_outcome_advantage: invalid estimator %d",
+  VAMD_REQUIRE(estimator >= VAMD_ADV_GRPO && estimator <= VAMD_ADV_GRPO_PASSK, "group_outcome_advantage: invalid estimator %d",
                estimator);
   VAMD_REQUIRE(estimator == VAMD_ADV_GRPO || n_groups <= kGrpoLdsGroups,
                "group_outcome_advantage: estimators other than GRPO support at most %d groups", kGrpoLdsGroups);

@@ -185,11 +185,11 @@ def compute_grpo_vectorized_outcome_advantage(token_level_rewards: torch.Tensor,
 
 
 # ---- the other outcome estimators of the registry ----------------------------------------------
-_ADV = {"grpo": 0, "rloo": 1, "rloo_vectorized": 2, "mean_baseline": 3, "opo": 4, "gpg": 5}
+_ADV = {"grpo": 0, "rloo": 1, "rloo_vectorized": 2, "mean_baseline": 3, "opo": 4, "gpg": 5, "grpo_passk": 6}
 
 
 def _group_outcome(token_level_rewards, response_mask, index, estimator: str, epsilon=1e-6, f_norm=1.0,
-                   whiten_after=False):
+                   whiten_after=False, norm_by_std=True, min_group_size=1):
     """Score per response -> statistic of its prompt group -> one scalar per response -> scalar * mask
     (``vamd_group_outcome_advantage``); ``whiten_after`` adds ``masked_whiten(.) * mask``."""
     with torch.no_grad():
@@ -200,6 +200,13 @@ def _group_outcome(token_level_rewards, response_mask, index, estimator: str, ep
         ids, G = contiguous_group_ids(index)
         if ids.numel() != B:
             raise ValueError(f"index has {ids.numel()} entries for a batch of {B}")
+        if min_group_size > 1:
+            counts = torch.bincount(ids, minlength=G)
+            small = (counts < min_group_size).nonzero()
+            if small.numel():
+                where = (ids == small[0, 0]).nonzero()[0, 0].item()
+                raise ValueError(f"Pass@k requires at least 2 samples per group. Got {int(counts[small[0, 0]])} "
+                                 f"for group {index[where]}.")
         ids = ids.to(dev)
         adv = torch.empty_like(r)
         Lb = _cabi.lib()
@@ -207,7 +214,8 @@ def _group_outcome(token_level_rewards, response_mask, index, estimator: str, ep
         with torch.cuda.device(dev):
             s = _cabi.stream_ptr(dev)
             _cabi.check(Lb.vamd_group_outcome_advantage(r.data_ptr(), m.data_ptr(), code, ids.data_ptr(), B, Lc, G,
-                                                        _ADV[estimator], float(epsilon), 1, 0, float(f_norm),
+                                                        _ADV[estimator], float(epsilon), int(bool(norm_by_std)), 0,
+                                                        float(f_norm),
                                                         adv.data_ptr(), None, ws.data_ptr(), ws.numel(), s))
             if whiten_after:
                 mom = verl_F._moments(adv, m, per_row=False)
@@ -218,6 +226,20 @@ def _group_outcome(token_level_rewards, response_mask, index, estimator: str, ep
                                                            adv.numel(), adv.data_ptr(), s))
         out = adv.view(token_level_rewards.shape).to(token_level_rewards.device)
         return out, out
+
+
+@register_adv_est(AdvantageEstimator.GRPO_PASSK)
+def compute_grpo_passk_outcome_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor, index,
+                                         epsilon: float = 1e-6, norm_adv_by_std_in_grpo: bool = True,
+                                         config: Optional[Any] = None, **kwargs):
+    """Pass@k advantage (reference core_algos.py:360-418): only the best response of a prompt group gets a
+    non-zero advantage, ``max - second max`` of the group's scores, divided by ``std + epsilon`` when
+    ``config.get("norm_adv_by_std_in_grpo", True)`` (the argument of the same name is overridden by the
+    config, as there, :388).  Every group needs at least two responses (``ValueError`` otherwise)."""
+    assert config is not None
+    norm = _cfg_get(config, "norm_adv_by_std_in_grpo", True)
+    return _group_outcome(token_level_rewards, response_mask, index, "grpo_passk", epsilon, norm_by_std=norm,
+                          min_group_size=2)
 
 
 @register_adv_est(AdvantageEstimator.REINFORCE_PLUS_PLUS_BASELINE)
