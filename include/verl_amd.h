@@ -188,7 +188,6 @@ int vamd_grpo_advantage(const float* rewards, const void* mask, int mask_dtype, 
                         int std_mode, float* advantages, float* scores_out, void* workspace,
                         size_t workspace_bytes, void* stream);
 
-/* group_mean_std (verl/utils/groupwise.py:163-223): mean/std/count per group, singleton -> (0,1). */
 /* The group-normalised outcome estimators above behind one entry point; vamd_grpo_advantage is the
  * VAMD_ADV_GRPO case.  std_mode and norm_by_std only matter for GRPO, f_norm only for GPG.  Estimators
  * other than GRPO support at most 2048 groups.  The REINFORCE++-baseline estimator is
@@ -209,6 +208,26 @@ int vamd_returns_advantage(const float* rewards, const void* mask, int mask_dtyp
                            int64_t batch, int64_t length, float gamma, int mode, float* advantages, float* returns,
                            double* moments_out, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Optimal token baseline (compute_optimal_token_baseline_advantage, core_algos.py:756-873):
+ * returns = reverse cumulative sum of rewards * mask; W = forward cumulative sum of
+ * (1 - 2 exp(old_log_probs) + sum_pi_squared) [* is_weights^2] * mask; per prompt group and column
+ * baseline = sum(returns W mask) / (sum(W mask) + epsilon), 0 for a group of one;
+ * advantages = (returns - baseline) * mask.  The groups arrive as a row permutation: rows_by_group
+ * lists the rows of group 0 first (each group's rows in ascending order), group_offsets
+ * [n_groups + 1] delimits the groups.  tail_start (optional, [batch]): the baseline of row i counts as 0
+ * from column tail_start[i] on (the reference's handle_zero_tail, :858-868).  is_weights may be NULL.
+ * packed != 0 selects the multi-turn variant (compute_multi_turn_optimal_token_baseline_advantage,
+ * :876-1004): the k-th valid token of every trajectory shares baseline column k, tail_start counts in
+ * those packed columns, and rows_by_group must leave out the rows that have no valid token (their
+ * advantages are 0; n_groups may then be 0).  returns is always laid out like rewards. */
+size_t vamd_otb_advantage_workspace_bytes(int64_t batch, int64_t length, int packed);
+int vamd_otb_advantage(const float* rewards, const void* mask, int mask_dtype, const float* old_log_probs,
+                       const float* sum_pi_squared, const float* is_weights, const int64_t* rows_by_group,
+                       const int64_t* group_offsets, const int64_t* tail_start, int64_t batch, int64_t length,
+                       int64_t n_groups, int packed, float epsilon, float* advantages, float* returns,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+/* group_mean_std (verl/utils/groupwise.py:163-223): mean/std/count per group, singleton -> (0,1). */
 int vamd_group_mean_std(const float* scores, const int64_t* group_ids, int64_t n, int64_t n_groups, float eps,
                         float* mean, float* std, float* count, void* stream);
 

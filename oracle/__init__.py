@@ -49,6 +49,9 @@ from .advantages import (  # noqa: F401
     reinforce_plus_plus_outcome_advantage,
     remax_outcome_advantage,
     grpo_passk_outcome_advantage,
+    optimal_token_baseline_advantage,
+    multi_turn_optimal_token_baseline_advantage,
+    otb_brute_force_fp64,
 )
 from .losses import (  # noqa: F401
     agg_loss,

@@ -321,3 +321,145 @@ def grpo_passk_outcome_advantage(token_level_rewards, response_mask, index, epsi
         advantages[rows[topk_idx[0].item()]] = advantage
     advantages = advantages.unsqueeze(-1) * response_mask
     return advantages, advantages
+
+
+def _otb_streams(token_level_rewards, response_mask, old_log_probs, sum_pi_squared, rollout_is_weights):
+    """core_algos.py:809-822 (= :924-938): reward to go and the cumulative path-variance proxy."""
+    returns = (token_level_rewards * response_mask).flip(dims=[-1]).cumsum(dim=-1).flip(dims=[-1])
+    w = 1 - 2 * torch.exp(old_log_probs) + sum_pi_squared
+    if rollout_is_weights is not None:
+        w = w * (rollout_is_weights**2)
+    return returns, (w * response_mask).cumsum(dim=-1)
+
+
+def _otb_zero_tail(baselines, rows, lengths):
+    """core_algos.py:858-868 (= :983-993): when exactly one trajectory of the group is the longest, its
+    baseline is 0 from the second-longest length on."""
+    ordered = sorted(int(lengths[i]) for i in rows)
+    longest, second = ordered[-1], ordered[-2]
+    holders = [i for i in rows if int(lengths[i]) == longest]
+    if len(holders) == 1 and longest > second:
+        baselines[holders[0], second:] = 0.0
+
+
+@torch.no_grad()
+def optimal_token_baseline_advantage(token_level_rewards, response_mask, index, old_log_probs, sum_pi_squared,
+                                     rollout_is_weights=None, handle_zero_tail=False, epsilon=1e-8):
+    """core_algos.py:756-873: per prompt group and column, baseline = sum(G W m) / (sum(W m) + eps) over the
+    group's trajectories (none for a group of one); advantages = (G - baseline) * mask; returns
+    ``(advantages, returns)``."""
+    returns, w_cum = _otb_streams(token_level_rewards, response_mask, old_log_probs, sum_pi_squared,
+                                  rollout_is_weights)
+    members = defaultdict(list)
+    for i in range(token_level_rewards.shape[0]):
+        members[index[i]].append(i)
+    baselines = torch.zeros_like(returns)
+    lengths = response_mask.sum(dim=-1)
+    for rows in members.values():
+        if len(rows) == 1:
+            continue
+        sel = torch.tensor(rows)
+        num = (returns[sel] * w_cum[sel] * response_mask[sel]).sum(dim=0)
+        den = (w_cum[sel] * response_mask[sel]).sum(dim=0) + epsilon
+        baselines[sel] = (num / den).unsqueeze(0).expand(len(rows), -1)
+        if handle_zero_tail:
+            _otb_zero_tail(baselines, rows, lengths)
+    return (returns - baselines) * response_mask, returns
+
+
+@torch.no_grad()
+def multi_turn_optimal_token_baseline_advantage(token_level_rewards, response_mask, index, old_log_probs,
+                                                sum_pi_squared, rollout_is_weights=None, handle_zero_tail=True,
+                                                epsilon=1e-8):
+    """core_algos.py:876-1004: as above, but every trajectory's valid tokens are first packed to the left
+    (the k-th valid token of each trajectory shares baseline column k), trajectories with no valid token
+    leave their group, and the advantages are scattered back to the valid positions."""
+    returns, w_cum = _otb_streams(token_level_rewards, response_mask, old_log_probs, sum_pi_squared,
+                                  rollout_is_weights)
+    B = returns.shape[0]
+    lengths = response_mask.sum(dim=-1).long()
+    width = int(lengths.max().item()) if B > 0 else 0
+    packed_w = w_cum.new_zeros((B, width))
+    packed_g = torch.zeros_like(packed_w)
+    valid = response_mask.bool()
+    for i in range(B):
+        n = int(lengths[i])
+        packed_w[i, :n] = w_cum[i, valid[i]]
+        packed_g[i, :n] = returns[i, valid[i]]
+    members = defaultdict(list)
+    for i in range(B):
+        if int(lengths[i]) > 0:
+            members[index[i]].append(i)
+    baselines = torch.zeros_like(packed_g)
+    for rows in members.values():
+        if len(rows) == 1:
+            continue
+        sel = torch.tensor(rows)
+        b_star = (packed_g[sel] * packed_w[sel]).sum(dim=0) / (packed_w[sel].sum(dim=0) + epsilon)
+        baselines[sel] = b_star.to(baselines.dtype)
+        if handle_zero_tail:
+            _otb_zero_tail(baselines, rows, lengths)
+    packed_adv = packed_g - baselines
+    advantages = torch.zeros_like(returns)
+    for i in range(B):
+        n = int(lengths[i])
+        if n > 0:
+            advantages[i, valid[i]] = packed_adv[i, :n]
+    return advantages * response_mask, returns
+
+
+def otb_brute_force_fp64(rewards, mask, index, old_log_probs, sum_pi_squared, is_weights=None, packed=False,
+                         zero_tail=False, epsilon=1e-8):
+    """Scalar double-precision loops over Python lists written from the definition of the optimal token
+    baseline, B_k = sum_i G_ik W_ik / (sum_i W_ik + eps) with k the column (``packed=False``) or the rank of
+    the token among its trajectory's valid tokens (``packed=True``); pins the two functions above."""
+    import math
+    B, L = len(rewards), len(rewards[0])
+    G = [[0.0] * L for _ in range(B)]
+    W = [[0.0] * L for _ in range(B)]
+    slot = [[-1] * L for _ in range(B)]  # baseline column of each valid token
+    n_valid = [0] * B
+    for i in range(B):
+        acc = 0.0
+        for t in range(L - 1, -1, -1):
+            acc += rewards[i][t] * mask[i][t]
+            G[i][t] = acc
+        acc = 0.0
+        for t in range(L):
+            w = 1.0 - 2.0 * math.exp(old_log_probs[i][t]) + sum_pi_squared[i][t]
+            if is_weights is not None:
+                w *= is_weights[i][t] ** 2
+            acc += w * mask[i][t]
+            W[i][t] = acc
+            if mask[i][t] != 0:
+                slot[i][t] = n_valid[i] if packed else t
+                n_valid[i] += 1
+    groups = defaultdict(list)
+    for i in range(B):
+        if not packed or n_valid[i] > 0:
+            groups[index[i]].append(i)
+    adv = [[0.0] * L for _ in range(B)]
+    for rows in groups.values():
+        num = defaultdict(float)
+        den = defaultdict(float)
+        for i in rows:
+            for t in range(L):
+                if slot[i][t] >= 0:
+                    num[slot[i][t]] += G[i][t] * W[i][t] * mask[i][t]
+                    den[slot[i][t]] += W[i][t] * mask[i][t]
+        no_baseline_from = {i: L + 1 for i in rows}
+        if zero_tail and len(rows) > 1:
+            ordered = sorted(n_valid[i] for i in rows)
+            if ordered[-1] > ordered[-2]:
+                holder = [i for i in rows if n_valid[i] == ordered[-1]]
+                no_baseline_from[holder[0]] = ordered[-2]
+        for i in rows:
+            for t in range(L):
+                k = slot[i][t]
+                if k < 0:
+                    continue
+                b = 0.0
+                if len(rows) > 1 and k < no_baseline_from[i]:
+                    b = num[k] / (den[k] + epsilon)
+                adv[i][t] = (G[i][t] - b) * mask[i][t]
+    return adv, G

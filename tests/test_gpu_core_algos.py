@@ -465,6 +465,81 @@ def test_reinforce_plus_plus_and_remax(dev, shape, mdtype):
     assert CA.get_adv_estimator_fn("remax") is CA.compute_remax_outcome_advantage
 
 
+def _otb_inputs(B, Lc, seed, multi_turn, n_groups):
+    g = torch.Generator().manual_seed(seed)
+    rewards = torch.randn(B, Lc, generator=g)
+    if multi_turn:   # generated turns separated by masked tool output, of varying widths
+        turn = torch.randint(1, max(2, Lc // 6), (1,), generator=g).item()
+        mask = ((torch.arange(Lc)[None, :] + torch.randint(0, 2 * turn, (B, 1), generator=g)) // turn % 2 == 0).float()
+        mask = mask * _prefix_mask(B, Lc, g, lo=1)[0]
+        mask[B // 2] = 0                                         # a trajectory that generated nothing
+    else:
+        mask = _prefix_mask(B, Lc, g, lo=1)[0]
+    pi = torch.rand(B, Lc, generator=g).clamp_min(1e-4)
+    # a distribution's sum of squares lies between pi^2 and pi^2 + (1 - pi)^2
+    pi2 = pi * pi + torch.rand(B, Lc, generator=g) * (1 - pi) ** 2
+    isw = 0.5 + torch.rand(B, Lc, generator=g)
+    index = np.array([f"prompt-{i}" for i in torch.randint(0, n_groups, (B,), generator=g).tolist()], dtype=object)
+    index[-1] = "alone"                                          # a group of one
+    return rewards, mask, index, pi.log(), pi2, isw
+
+
+@pytest.mark.parametrize("shape,n_groups", [((4, 17), 2), ((16, 1024), 3), ((6, 4099), 2), ((64, 8192), 8)])
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.int64])
+@pytest.mark.parametrize("with_isw", [False, True])
+@pytest.mark.parametrize("zero_tail", [False, True])
+@pytest.mark.parametrize("multi_turn", [False, True])
+def test_optimal_token_baseline(dev, shape, n_groups, mdtype, with_isw, zero_tail, multi_turn):
+    from verl_amd.trainer.ppo import core_algos as CA
+    B, Lc = shape
+    r, m, index, lp, pi2, isw = _otb_inputs(B, Lc, Lc + B, multi_turn, n_groups)
+    w = isw if with_isw else None
+    fn = CA.compute_multi_turn_optimal_token_baseline_advantage if multi_turn else CA.compute_optimal_token_baseline_advantage
+    ref = O.multi_turn_optimal_token_baseline_advantage if multi_turn else O.optimal_token_baseline_advantage
+    adv, ret = fn(r.to(dev), m.to(dev).to(mdtype), index, lp.to(dev), pi2.to(dev),
+                  rollout_is_weights=None if w is None else w.to(dev), handle_zero_tail=zero_tail)
+    want_adv, want_ret = ref(r, m, index, lp, pi2, rollout_is_weights=w, handle_zero_tail=zero_tail)
+    adv64, ret64 = ref(r.double(), m.double(), index, lp.double(), pi2.double(),
+                       rollout_is_weights=None if w is None else w.double(), handle_zero_tail=zero_tail)
+    # the running sums are re-associated (and carried in double): hold them to the fp64 result as tightly as the
+    # reference's sequential fp32 cumsum holds
+    scale = max(1.0, ret64.abs().max().item())
+    for name, got, want32, want64 in (("returns", ret, want_ret, ret64), ("advantages", adv, want_adv, adv64)):
+        err_kernel = (got.cpu().double() - want64).abs().max().item()
+        err_oracle = (want32.double() - want64).abs().max().item()
+        assert err_kernel <= max(2 * err_oracle, 1e-5 * scale), (name, err_kernel, err_oracle, scale)
+    assert torch.equal(adv.cpu()[m == 0], torch.zeros_like(adv.cpu()[m == 0]))
+    lone = adv.cpu()[-1]                                         # a group of one keeps its returns
+    assert torch.allclose(lone, (ret.cpu() * m)[-1], rtol=0, atol=0)
+    name = "tir_optimal_token_baseline" if multi_turn else "optimal_token_baseline"
+    assert CA.get_adv_estimator_fn(name) is fn
+
+
+def test_optimal_token_baseline_consumes_the_head_sum_pi_squared(dev):
+    """sum_pi_squared as the head kernel produces it, log-probs from the same call, through the estimator."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy_with_sum_pi_squared
+    g = torch.Generator().manual_seed(3)
+    B, Lc, H, V = 8, 48, 128, 1024
+    hidden = torch.randn(B * Lc, H, generator=g).bfloat16()
+    weight = (torch.randn(V, H, generator=g) * 0.08).bfloat16()
+    labels = torch.randint(0, V, (B * Lc,), generator=g)
+    lp, _, pi2 = linear_cross_entropy_with_sum_pi_squared(hidden.to(dev), weight.to(dev), labels.to(dev), 1.0)
+    mask = _prefix_mask(B, Lc, g, lo=4)[0]
+    rewards = torch.randn(B, Lc, generator=g)
+    index = np.repeat(np.arange(B // 4), 4)
+    adv, ret = CA.compute_optimal_token_baseline_advantage(rewards.to(dev), mask.to(dev), index, lp.view(B, Lc),
+                                                           pi2.view(B, Lc))
+    logits = hidden.float() @ weight.float().t()
+    want_lp = torch.log_softmax(logits, -1).gather(-1, labels[:, None]).squeeze(-1)
+    want_pi2 = O.sum_pi_squared_from_logits(logits)
+    want_adv, want_ret = O.optimal_token_baseline_advantage(rewards, mask, index, want_lp.view(B, Lc),
+                                                            want_pi2.view(B, Lc))
+    _close(ret, want_ret, atol=1e-5 * want_ret.abs().max().item(), what="returns")
+    # the baseline is a ratio of sums of W, which inherits the head's 2e-3 on log-prob: O(1e-2) relative on W
+    assert (adv.cpu() - want_adv).abs().max().item() <= 2e-2 * want_ret.abs().max().item()
+
+
 # ---- the other registered policy losses -----------------------------------------------------------------
 @pytest.mark.parametrize("variant", ["gpg", "cispo", "sapo", "gspo"])
 @pytest.mark.parametrize("mode", MODES)

@@ -327,3 +327,78 @@ def test_grpo_passk_by_hand():
     assert A.grpo_passk_outcome_advantage(tied, mask, index)[0][:3].abs().sum().item() == 0
     with pytest.raises(ValueError):
         A.grpo_passk_outcome_advantage(rewards, mask, np.array(["a", "a", "a", "b", "c"], dtype=object))
+
+
+# ---- optimal token baseline ---------------------------------------------------------------------
+def _otb_case(seed, B, L, groups, multi_turn):
+    g = torch.Generator().manual_seed(seed)
+    rewards = torch.randn(B, L, generator=g, dtype=torch.float64)
+    if multi_turn:  # several generation turns with tool output (masked) between them
+        mask = (torch.rand(B, L, generator=g) < 0.6).double()
+        mask[0] = 0  # a trajectory with no valid token
+    else:
+        lens = torch.randint(1, L + 1, (B,), generator=g)
+        mask = (torch.arange(L)[None, :] < lens[:, None]).double()
+    old_lp = -torch.rand(B, L, generator=g, dtype=torch.float64) * 4
+    pi2 = torch.rand(B, L, generator=g, dtype=torch.float64)
+    isw = 0.5 + torch.rand(B, L, generator=g, dtype=torch.float64)
+    index = np.array([f"p{int(i)}" for i in torch.randint(0, groups, (B,), generator=g)], dtype=object)
+    return rewards, mask, index, old_lp, pi2, isw
+
+
+@pytest.mark.parametrize("seed,B,L,groups", [(0, 12, 17, 3), (1, 9, 8, 9), (2, 16, 33, 2)])
+@pytest.mark.parametrize("with_isw", [False, True])
+@pytest.mark.parametrize("zero_tail", [False, True])
+@pytest.mark.parametrize("multi_turn", [False, True])
+def test_optimal_token_baseline_against_fp64_brute_force(seed, B, L, groups, with_isw, zero_tail, multi_turn):
+    r, m, index, lp, pi2, isw = _otb_case(seed, B, L, groups, multi_turn)
+    w = isw if with_isw else None
+    want_adv, want_ret = A.otb_brute_force_fp64(r.tolist(), m.tolist(), index.tolist(), lp.tolist(), pi2.tolist(),
+                                                None if w is None else w.tolist(), packed=multi_turn,
+                                                zero_tail=zero_tail)
+    fn = A.multi_turn_optimal_token_baseline_advantage if multi_turn else A.optimal_token_baseline_advantage
+    adv, ret = fn(r, m, index, lp, pi2, rollout_is_weights=w, handle_zero_tail=zero_tail)
+    assert torch.allclose(ret, torch.tensor(want_ret, dtype=torch.float64), rtol=1e-12, atol=1e-12)
+    assert torch.allclose(adv, torch.tensor(want_adv, dtype=torch.float64), rtol=1e-9, atol=1e-9)
+
+
+def test_optimal_token_baseline_by_hand():
+    # two full-length responses of one prompt and a lone response of another; pi = 1/2 and sum pi^2 = 1/2 give
+    # w = 1/2 per token, so W = (1/2, 1) on both rows and the baseline is the plain mean of the returns
+    r = torch.tensor([[1.0, 2.0], [3.0, 0.0], [5.0, 7.0]])
+    m = torch.ones(3, 2)
+    lp = torch.full((3, 2), math.log(0.5))
+    pi2 = torch.full((3, 2), 0.5)
+    index = np.array(["a", "a", "b"], dtype=object)
+    adv, ret = A.optimal_token_baseline_advantage(r, m, index, lp, pi2)
+    assert ret.tolist() == [[3.0, 2.0], [3.0, 0.0], [12.0, 7.0]]
+    assert torch.allclose(adv, torch.tensor([[0.0, 1.0], [0.0, -1.0], [12.0, 7.0]]), atol=1e-6)
+    # unequal path variance: row 0 deterministic (w = 0), row 1 as before -> the baseline is row 1's return
+    lp0 = lp.clone(); lp0[0] = 0.0
+    pi20 = pi2.clone(); pi20[0] = 1.0
+    adv, _ = A.optimal_token_baseline_advantage(r, m, index, lp0, pi20)
+    assert torch.allclose(adv[:2], torch.tensor([[0.0, 2.0], [0.0, 0.0]]), atol=1e-6)
+    # the importance weights enter squared: doubling them on row 1 leaves a one-sided baseline unchanged
+    adv2, _ = A.optimal_token_baseline_advantage(r, m, index, lp0, pi20,
+                                                 rollout_is_weights=torch.tensor([[1.0, 1.0], [2.0, 2.0], [1.0, 1.0]]))
+    assert torch.allclose(adv2[:2], adv[:2], atol=1e-6)
+    # zero tail: row 1 shorter -> beyond its length the longest row keeps its return as the advantage
+    m2 = torch.tensor([[1.0, 1.0], [1.0, 0.0], [1.0, 1.0]])
+    adv3, ret3 = A.optimal_token_baseline_advantage(r, m2, index, lp, pi2, handle_zero_tail=True)
+    assert adv3[0, 1].item() == ret3[0, 1].item() == 2.0
+    adv4, _ = A.optimal_token_baseline_advantage(r, m2, index, lp, pi2, handle_zero_tail=False)
+    assert abs(adv4[0, 1].item()) < 1e-6  # alone in its column: the baseline equals its own return
+
+
+def test_multi_turn_optimal_token_baseline_packs_valid_tokens():
+    # with prefix masks the packed variant is the plain one
+    r, m, index, lp, pi2, _ = _otb_case(5, 10, 12, 3, multi_turn=False)
+    a, _ = A.optimal_token_baseline_advantage(r, m, index, lp, pi2)
+    b, _ = A.multi_turn_optimal_token_baseline_advantage(r, m, index, lp, pi2, handle_zero_tail=False)
+    assert torch.allclose(a, b, rtol=1e-12, atol=1e-12)
+    # inserting masked columns into the trajectories does not change the advantages of the valid tokens
+    L = m.shape[1]
+    wide = lambda x: torch.stack([x, torch.zeros_like(x)], dim=-1).reshape(x.shape[0], 2 * L)  # noqa: E731
+    c, _ = A.multi_turn_optimal_token_baseline_advantage(wide(r), wide(m), index, wide(lp), wide(pi2),
+                                                         handle_zero_tail=False)
+    assert torch.allclose(c[:, 0::2], b, rtol=1e-12, atol=1e-12) and (c[:, 1::2] == 0).all()

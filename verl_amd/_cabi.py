@@ -56,6 +56,10 @@ SIGNATURES = {
     "vamd_returns_advantage_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "vamd_returns_advantage": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_float, c_int,
                                        c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "vamd_otb_advantage_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int]),
+    "vamd_otb_advantage": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                   c_void_p, c_int64, c_int64, c_int64, c_int, c_float, c_void_p, c_void_p, c_void_p,
+                                   c_size_t, c_void_p]),
     "vamd_affine_by_stats_masked": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_void_p, c_void_p]),
     "vamd_group_mean_std": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_float, c_void_p, c_void_p, c_void_p,
                                     c_void_p]),

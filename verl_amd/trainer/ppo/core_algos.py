@@ -46,9 +46,7 @@ def get_policy_loss_fn(name):
 
 
 class AdvantageEstimator(str, Enum):
-    """Names of the reference's advantage estimators (core_algos.py:88-109).  GRPO_PASSK and the two
-    optimal-token-baseline estimators are not implemented here; their names exist so configs keep
-    parsing, and looking them up raises the reference's "unknown estimator" error."""
+    """Names of the reference's advantage estimators (core_algos.py:88-109); every one is registered below."""
 
     GAE = "gae"
     GRPO = "grpo"
@@ -323,6 +321,93 @@ def compute_remax_outcome_advantage(token_level_rewards: torch.Tensor, reward_ba
     """ReMax (reference core_algos.py:621-654): reverse cumulative sum of the masked rewards minus the
     greedy-rollout baseline of the response on its mask.  Returns ``(advantages, returns)``."""
     return _returns_advantage(token_level_rewards, response_mask, 0, 1.0, baselines=reward_baselines)
+
+
+def _optimal_token_baseline(token_level_rewards, response_mask, index, old_log_probs, sum_pi_squared,
+                            rollout_is_weights, handle_zero_tail, epsilon, packed):
+    """Both optimal-token-baseline estimators (``vamd_otb_advantage``).  The host part is the grouping: the
+    rows sorted by prompt, and, for ``handle_zero_tail``, the column from which the longest trajectory of
+    a group stands alone."""
+    with torch.no_grad():
+        dev = _cabi.compute_device(token_level_rewards, response_mask, old_log_probs, sum_pi_squared)
+        r = _matrix(token_level_rewards, dev)
+        m, code = _mask_matrix(response_mask, dev, r.shape)
+        lp = _matrix(old_log_probs, dev)
+        q = _matrix(sum_pi_squared, dev)
+        assert lp.shape == r.shape and q.shape == r.shape
+        isw = None
+        if rollout_is_weights is not None:
+            isw = _matrix(rollout_is_weights, dev)
+            assert isw.shape == r.shape
+        B, Lc = r.shape
+        ids, _ = contiguous_group_ids(index)
+        if ids.numel() != B:
+            raise ValueError(f"index has {ids.numel()} entries for a batch of {B}")
+        ids = ids.numpy()
+        lengths = None
+        if packed or handle_zero_tail:
+            lengths = verl_F._moments(r, m, per_row=True)[0].cpu().numpy().astype(np.int64)
+        rows = np.argsort(ids, kind="stable")
+        if packed:  # trajectories without a valid token leave their group
+            rows = rows[lengths[rows] > 0]
+        sorted_ids = ids[rows]
+        starts = np.flatnonzero(np.r_[True, sorted_ids[1:] != sorted_ids[:-1]]) if rows.size else np.zeros(0, np.int64)
+        offsets = np.r_[starts, rows.size].astype(np.int64)
+        G = len(offsets) - 1
+        tail = None
+        if handle_zero_tail:
+            tail = np.full(B, Lc, dtype=np.int64)
+            for g in range(G):
+                members = rows[offsets[g]:offsets[g + 1]]
+                if members.size < 2:
+                    continue
+                order = np.argsort(lengths[members], kind="stable")
+                longest, second = lengths[members[order[-1]]], lengths[members[order[-2]]]
+                if longest > second:
+                    tail[members[order[-1]]] = second
+            tail = torch.from_numpy(tail).to(dev)
+        rows_t = torch.from_numpy(rows.astype(np.int64)).to(dev) if G else None
+        offs_t = torch.from_numpy(offsets).to(dev) if G else None
+        adv = torch.empty_like(r)
+        ret = torch.empty_like(r)
+        Lb = _cabi.lib()
+        ws = _cabi.workspace(Lb.vamd_otb_advantage_workspace_bytes(B, Lc, int(packed)), dev)
+        with torch.cuda.device(dev):
+            _cabi.check(Lb.vamd_otb_advantage(r.data_ptr(), m.data_ptr(), code, lp.data_ptr(), q.data_ptr(),
+                                              _cabi.ptr(isw), _cabi.ptr(rows_t), _cabi.ptr(offs_t), _cabi.ptr(tail),
+                                              B, Lc, G, int(packed), float(epsilon), adv.data_ptr(), ret.data_ptr(),
+                                              ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
+        shape, out_dev = token_level_rewards.shape, token_level_rewards.device
+        return adv.view(shape).to(out_dev), ret.view(shape).to(out_dev)
+
+
+@register_adv_est(AdvantageEstimator.OPTIMAL_TOKEN_BASELINE)
+def compute_optimal_token_baseline_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor,
+                                             index: np.ndarray, old_log_probs: torch.Tensor,
+                                             sum_pi_squared: torch.Tensor, rollout_is_weights: torch.Tensor = None,
+                                             handle_zero_tail: bool = False, epsilon: float = 1e-8):
+    """Optimal token baseline (reference core_algos.py:756-873): per prompt group and column
+    ``B_t = sum(G_t W_t) / (sum(W_t) + epsilon)`` over the group's trajectories, with ``G`` the reward to go
+    and ``W`` the running sum of ``1 - 2 pi_t + sum pi^2`` (times the squared importance weights when given);
+    ``advantages = (G - B) * mask``, a lone trajectory keeps ``G``.  ``handle_zero_tail`` drops the baseline
+    of a group's single longest trajectory beyond the second-longest length.  ``sum_pi_squared`` is what
+    ``linear_cross_entropy_with_sum_pi_squared`` returns.  Returns ``(advantages, returns)``."""
+    return _optimal_token_baseline(token_level_rewards, response_mask, index, old_log_probs, sum_pi_squared,
+                                   rollout_is_weights, handle_zero_tail, epsilon, packed=False)
+
+
+@register_adv_est(AdvantageEstimator.TIR_OPTIMAL_TOKEN_BASELINE)
+def compute_multi_turn_optimal_token_baseline_advantage(token_level_rewards: torch.Tensor,
+                                                        response_mask: torch.Tensor, index: np.ndarray,
+                                                        old_log_probs: torch.Tensor, sum_pi_squared: torch.Tensor,
+                                                        rollout_is_weights: torch.Tensor = None,
+                                                        handle_zero_tail: bool = True, epsilon: float = 1e-8):
+    """Optimal token baseline for tool-integrated (multi-turn) rollouts (reference core_algos.py:876-1004):
+    the valid tokens of each trajectory are packed together first, so the k-th generated token of every
+    trajectory shares a baseline whatever tool output lies in between; trajectories without a valid token
+    do not count towards their group.  Returns ``(advantages, returns)``."""
+    return _optimal_token_baseline(token_level_rewards, response_mask, index, old_log_probs, sum_pi_squared,
+                                   rollout_is_weights, handle_zero_tail, epsilon, packed=True)
 
 
 # ---------------------------------------------------------------------------------------------
