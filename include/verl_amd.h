@@ -292,6 +292,16 @@ int vamd_value_loss_forward(const float* vpreds, const float* returns, const flo
 int vamd_kl_penalty(const float* logprob, const float* ref_logprob, int64_t n, int kind, int straight_through,
                     float* kld, float* grad, void* stream);
 
+/* apply_kl_penalty (verl/trainer/ppo/ray_trainer.py:70-109) without its controller update:
+ * kld = kl_penalty(logprob, ref_logprob) * mask; token_level_rewards = scores - beta * kld;
+ * current_kl[0] (1 device float) = mean over rows of masked_mean(kld, mask, axis=-1).  With
+ * kind = VAMD_KL_K1 and an all-ones mask the rewards are compute_rewards (core_algos.py:1009-1022). */
+size_t vamd_apply_kl_penalty_workspace_bytes(int64_t rows, int64_t cols);
+int vamd_apply_kl_penalty(const float* scores, const float* logprob, const float* ref_logprob, const void* mask,
+                          int mask_dtype, int64_t rows, int64_t cols, int kind, float beta,
+                          float* token_level_rewards, float* current_kl, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
 /* agg_loss(kl_penalty(logprob, ref_logprob), mask, mode) in one pass: the kl_loss of the actor
  * update (verl/workers/actor/dp_actor.py:640-646).  out[0] = kl_loss; grad_unscaled (optional) =
  * d kld / d logprob * mask, to be scaled by coef_out[row] and the upstream gradient with

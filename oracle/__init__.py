@@ -65,3 +65,8 @@ from .losses import (  # noqa: F401
     policy_loss_gpg,
     policy_loss_cispo,
 )
+from .trainer import (  # noqa: F401
+    apply_kl_penalty,
+    adaptive_kl_update,
+    compute_rewards,
+)

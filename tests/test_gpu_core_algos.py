@@ -704,3 +704,111 @@ def test_copy_bytes_is_exact(dev):
         _cabi.check(_cabi.lib().vamd_copy_bytes(src.data_ptr(), dst.data_ptr(), nbytes, _cabi.stream_ptr(dev)))
         assert torch.equal(src, dst)
     assert _cabi.lib().vamd_copy_bytes(src.data_ptr(), dst.data_ptr(), 24, _cabi.stream_ptr(dev)) == -1
+
+
+# ---- the trainer-side callers -------------------------------------------------------------------------
+class _Batch(dict):
+    """A dict with the two attributes of a TensorDict that the callers look at."""
+
+    @property
+    def batch_size(self):
+        return (next(iter(self.values())).shape[0],)
+
+
+def _data(batch, non_tensor=None):
+    return types.SimpleNamespace(batch=_Batch(batch), non_tensor_batch=non_tensor or {})
+
+
+@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192)])
+@pytest.mark.parametrize("kind", ["kl", "abs", "mse", "low_var_kl"])
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.int64, torch.bool])
+def test_kl_penalised_rewards(dev, shape, kind, mdtype):
+    from verl_amd.trainer.ppo import core_algos as CA
+    B, Lc = shape
+    g = torch.Generator().manual_seed(B * 7 + Lc)
+    scores = torch.randn(B, Lc, generator=g)
+    old = -torch.rand(B, Lc, generator=g) * 3
+    ref = old + torch.randn(B, Lc, generator=g) * 0.3
+    mask, _ = _prefix_mask(B, Lc, g, lo=1)
+    mask[0] = 0                                                  # an empty response
+    rewards, kl = CA.kl_penalised_rewards(scores.to(dev), old.to(dev), ref.to(dev), mask.to(dev).to(mdtype), 0.05, kind)
+    want_r, want_kl = O.apply_kl_penalty(scores, old, ref, mask, 0.05, kind)
+    _close(rewards, want_r, what="token_level_rewards")
+    assert torch.equal(rewards.cpu()[mask == 0], scores[mask == 0])
+    assert abs(kl.item() - want_kl) <= 1e-5 * max(1.0, abs(want_kl))
+
+
+def test_apply_kl_penalty_and_compute_rewards(dev):
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.trainer.ppo import ray_trainer as RT
+    g = torch.Generator().manual_seed(5)
+    B, Lc = 12, 300
+    scores = torch.randn(B, Lc, generator=g)
+    old = -torch.rand(B, Lc, generator=g) * 3
+    ref = old + torch.randn(B, Lc, generator=g) * 0.3
+    mask, _ = _prefix_mask(B, Lc, g, lo=1)
+    data = _data(dict(response_mask=mask.to(dev), token_level_scores=scores.to(dev), old_log_probs=old.to(dev),
+                      ref_log_prob=ref.to(dev)))
+    ctl = CA.AdaptiveKLController(init_kl_coef=0.1, target_kl=0.05, horizon=1000)
+    out, metrics = RT.apply_kl_penalty(data, ctl, kl_penalty="low_var_kl")
+    want_r, want_kl = O.apply_kl_penalty(scores, old, ref, mask, 0.1, "low_var_kl")
+    assert out is data
+    _close(data.batch["token_level_rewards"], want_r, what="token_level_rewards")
+    assert metrics["actor/reward_kl_penalty"] == pytest.approx(want_kl, rel=1e-5)
+    assert metrics["actor/reward_kl_penalty_coeff"] == 0.1
+    assert ctl.value == pytest.approx(O.adaptive_kl_update(0.1, want_kl, B, 0.05, 1000), rel=1e-6)
+    with pytest.raises(NotImplementedError):
+        RT.apply_kl_penalty(data, ctl, kl_penalty="full")
+    _close(CA.compute_rewards(scores.to(dev), old.to(dev), ref.to(dev), 0.3), O.compute_rewards(scores, old, ref, 0.3),
+           what="compute_rewards")
+
+
+def test_compute_advantage_dispatch(dev):
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.trainer.ppo import ray_trainer as RT
+    g = torch.Generator().manual_seed(9)
+    B, P, Lc = 8, 5, 40
+    rewards = torch.randn(B, Lc, generator=g)
+    values = torch.randn(B, Lc, generator=g)
+    mask, _ = _prefix_mask(B, Lc, g, lo=2)
+    attention = torch.cat([torch.ones(B, P), mask], dim=1)
+    uid = np.array([f"u{i // 4}" for i in range(B)], dtype=object)
+    pi = torch.rand(B, Lc, generator=g).clamp_min(1e-3)
+    batch = dict(token_level_rewards=rewards.to(dev), values=values.to(dev), attention_mask=attention.to(dev),
+                 responses=torch.zeros(B, Lc, dtype=torch.long, device=dev), old_log_probs=pi.log().to(dev),
+                 sum_pi_squared=(pi * pi + 0.5 * (1 - pi) ** 2).to(dev), reward_baselines=torch.randn(B, generator=g).to(dev))
+    cfg = _cfg(gamma=0.99, norm_adv_by_std_in_grpo=True)
+    cfg.get = lambda k, d=None: getattr(cfg, k, d)
+
+    def run(name, **kw):
+        # reward_baselines is only in the batch when ReMax put it there (every other estimator would reject it)
+        data = _data({k: v for k, v in batch.items() if k != "reward_baselines" or name == "remax"}, {"uid": uid})
+        out = RT.compute_advantage(data, CA.AdvantageEstimator(name), config=cfg, **kw)
+        assert out is data and torch.equal(data.batch["response_mask"].cpu(), mask)   # derived from attention_mask
+        return data.batch["advantages"].cpu(), data.batch["returns"].cpu()
+
+    m = mask
+    adv, ret = run("gae", gamma=0.99, lam=0.95)
+    want = O.gae_advantage_return(rewards, values, m, 0.99, 0.95)
+    _close(adv, want[0], atol=2e-5, what="gae adv"); _close(ret, want[1], atol=2e-5, what="gae ret")
+    adv, _ = run("grpo", norm_adv_by_std_in_grpo=False)
+    _close(adv, O.grpo_outcome_advantage(rewards.clone(), m, uid, norm_adv_by_std_in_grpo=False)[0], what="grpo")
+    adv, _ = run("rloo")
+    _close(adv, O.rloo_outcome_advantage(rewards.clone(), m, uid)[0], what="rloo")
+    adv, ret = run("remax")
+    want = O.remax_outcome_advantage(rewards, batch["reward_baselines"].cpu(), m)
+    _close(adv, want[0], atol=2e-5, what="remax adv"); _close(ret, want[1], atol=2e-5, what="remax ret")
+    adv, ret = run("reinforce_plus_plus")
+    _close(adv, O.reinforce_plus_plus_outcome_advantage(rewards, m, 0.99)[0], atol=2e-5, what="reinforce++")
+    for name, ref in (("optimal_token_baseline", O.optimal_token_baseline_advantage),
+                      ("tir_optimal_token_baseline", O.multi_turn_optimal_token_baseline_advantage)):
+        adv, ret = run(name)
+        want = ref(rewards, m, uid, batch["old_log_probs"].cpu(), batch["sum_pi_squared"].cpu())
+        _close(adv, want[0], atol=5e-5, what=name)
+    with pytest.raises(AssertionError, match="sum_pi_squared"):
+        data = _data({k: v for k, v in batch.items() if k not in ("sum_pi_squared", "reward_baselines")}, {"uid": uid})
+        RT.compute_advantage(data, CA.AdvantageEstimator.OPTIMAL_TOKEN_BASELINE, config=cfg)
+    cfg.use_pf_ppo = True
+    with pytest.raises(NotImplementedError):
+        RT.compute_advantage(_data(dict(batch), {"uid": uid}), CA.AdvantageEstimator.GAE, config=cfg)
+

@@ -494,6 +494,61 @@ __global__ __launch_bounds__(kRcThreads) void kl_loss_kernel(
   ticket_reset(wk.ticket);
 }
 
+// token_level_rewards = scores - beta * kld * mask and current_kl = mean over rows of
+// masked_mean(kld * mask, mask, axis=-1), the two things apply_kl_penalty derives from the KL estimate
+// (verl/trainer/ppo/ray_trainer.py:86-101), in one pass.
+template <bool VEC, class M>
+__global__ __launch_bounds__(kRcThreads) void kl_reward_kernel(
+    const float* __restrict__ scores, const float* __restrict__ logprob, const float* __restrict__ ref,
+    const M* __restrict__ mask, int64_t rows, int64_t cols, int chunks, int kind, float beta, Work wk,
+    float* __restrict__ rewards, float* __restrict__ current_kl) {
+  const int64_t row = blockIdx.x / chunks;
+  const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float sc[kGroups][4], lp[kGroups][4], rf[kGroups][4], w[kGroups][4];
+  load_groups<VEC>(scores, pos, sc);
+  load_groups<VEC>(logprob, pos, lp);
+  load_groups<VEC>(ref, pos, rf);
+  load_mask_groups<VEC>(mask, pos, w);
+  float s_kl = 0, s_m = 0;
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float kld, dk;
+      kl_point(kind, false, lp[g][e], rf[g][e], kld, dk);
+      const float we = w[g][e];
+      const float km = kld * we;
+      if (e < pos.valid[g]) {
+        s_kl += (we == 0.f ? 0.f : km) * we;  // masked_sum: where(mask, v, 0) * mask
+        s_m += we;
+      }
+      sc[g][e] = sc[g][e] - beta * km;
+    }
+  store_groups<VEC>(rewards, pos, sc);
+  __shared__ double smem[2 * 4];
+  double acc[2] = {s_kl, s_m};
+  block_sum<2, kRcThreads>(acc, smem);
+  if (threadIdx.x == 0) {
+    double* p = wk.partials + (int64_t)blockIdx.x * 2;
+    peer_store(p + 0, acc[0]); peer_store(p + 1, acc[1]);
+  }
+  if (!last_block_arrives(wk.ticket)) return;
+  double total = 0;
+  for (int64_t r = threadIdx.x; r < rows; r += kRcThreads) {
+    double S = 0, Ms = 0;
+    for (int c = 0; c < chunks; ++c) {
+      S += peer_load(wk.partials + (r * chunks + c) * 2);
+      Ms += peer_load(wk.partials + (r * chunks + c) * 2 + 1);
+    }
+    total += (double)((float)S / ((float)Ms + 1e-8f));
+  }
+  double t[1] = {total};
+  block_sum<1, kRcThreads>(t, smem);
+  if (threadIdx.x == 0) current_kl[0] = (float)(t[0] / (double)rows);
+  ticket_reset(wk.ticket);
+}
+
 // =============================================================================================
 // GRPO
 // =============================================================================================
@@ -1079,6 +1134,37 @@ extern "C" int vamd_kl_loss_forward(const float* logprob, const float* ref_logpr
     else { if (grad_unscaled) VAMD_KL(false, true); else VAMD_KL(false, false); }
   });
 #undef VAMD_KL
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
+
+extern "C" size_t vamd_apply_kl_penalty_workspace_bytes(int64_t rows, int64_t cols) {
+  return reduce_workspace_bytes(rows, cols, 2);
+}
+
+extern "C" int vamd_apply_kl_penalty(const float* scores, const float* logprob, const float* ref_logprob,
+                                     const void* mask, int mask_dtype, int64_t rows, int64_t cols, int kind,
+                                     float beta, float* token_level_rewards, float* current_kl, void* workspace,
+                                     size_t workspace_bytes, void* stream) {
+  int st = check_matrix("apply_kl_penalty", rows, cols);
+  if (st != VAMD_OK) return st;
+  VAMD_REQUIRE(scores && logprob && ref_logprob && mask && token_level_rewards && current_kl,
+               "apply_kl_penalty: null pointer");
+  VAMD_REQUIRE(kind >= VAMD_KL_K1 && kind <= VAMD_KL_K3, "apply_kl_penalty: invalid estimator %d", kind);
+  if (!workspace || workspace_bytes < vamd_apply_kl_penalty_workspace_bytes(rows, cols)) {
+    set_error("apply_kl_penalty: workspace too small");
+    return VAMD_EWORKSPACE;
+  }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int chunks = (int)chunks_of(cols);
+  const Work wk = carve_work(workspace);
+  VAMD_MASK_DISPATCH(mask_dtype, M, {
+    const bool vec = can_vectorize(cols, {scores, logprob, ref_logprob, token_level_rewards}, mask, sizeof(M));
+    VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((kl_reward_kernel<V, M>), dim3((unsigned)(rows * chunks)),
+                                                 dim3(kRcThreads), 0, s, scores, logprob, ref_logprob,
+                                                 static_cast<const M*>(mask), rows, cols, chunks, kind, beta, wk,
+                                                 token_level_rewards, current_kl));
+  });
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }

@@ -90,6 +90,41 @@ def get_adv_estimator_fn(name_or_enum):
     return ADV_ESTIMATOR_REGISTRY[name]
 
 
+class AdaptiveKLController:
+    """KL coefficient that tracks a target KL (reference core_algos.py:152-173): ``update`` multiplies
+    ``value`` by ``1 + clip(current_kl / target - 1, -0.2, 0.2) * n_steps / horizon``."""
+
+    def __init__(self, init_kl_coef, target_kl, horizon):
+        self.value = init_kl_coef
+        self.target = target_kl
+        self.horizon = horizon
+
+    def update(self, current_kl, n_steps):
+        error = min(max(current_kl / self.target - 1, -0.2), 0.2)
+        self.value *= 1 + error * n_steps / self.horizon
+
+
+class FixedKLController:
+    """Constant KL coefficient (reference core_algos.py:176-189); ``update`` does nothing."""
+
+    def __init__(self, kl_coef):
+        self.value = kl_coef
+
+    def update(self, current_kl, n_steps):
+        pass
+
+
+def get_kl_controller(kl_ctrl):
+    """Controller for ``kl_ctrl.type`` in {"fixed", "adaptive"} (reference core_algos.py:192-211)."""
+    if kl_ctrl.type == "fixed":
+        return FixedKLController(kl_coef=kl_ctrl.kl_coef)
+    if kl_ctrl.type == "adaptive":
+        assert kl_ctrl.horizon > 0, f"horizon must be larger than 0. Got {kl_ctrl.horizon}"
+        return AdaptiveKLController(init_kl_coef=kl_ctrl.kl_coef, target_kl=kl_ctrl.target_kl,
+                                    horizon=kl_ctrl.horizon)
+    raise NotImplementedError
+
+
 # ---------------------------------------------------------------------------------------------
 def _matrix(t: torch.Tensor, dev: torch.device) -> torch.Tensor:
     x = _cabi.as_f32(t, dev)
@@ -385,13 +420,15 @@ def _optimal_token_baseline(token_level_rewards, response_mask, index, old_log_p
 def compute_optimal_token_baseline_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor,
                                              index: np.ndarray, old_log_probs: torch.Tensor,
                                              sum_pi_squared: torch.Tensor, rollout_is_weights: torch.Tensor = None,
-                                             handle_zero_tail: bool = False, epsilon: float = 1e-8):
+                                             handle_zero_tail: bool = False, epsilon: float = 1e-8,
+                                             config: Optional[Any] = None):
     """Optimal token baseline (reference core_algos.py:756-873): per prompt group and column
     ``B_t = sum(G_t W_t) / (sum(W_t) + epsilon)`` over the group's trajectories, with ``G`` the reward to go
     and ``W`` the running sum of ``1 - 2 pi_t + sum pi^2`` (times the squared importance weights when given);
     ``advantages = (G - B) * mask``, a lone trajectory keeps ``G``.  ``handle_zero_tail`` drops the baseline
     of a group's single longest trajectory beyond the second-longest length.  ``sum_pi_squared`` is what
-    ``linear_cross_entropy_with_sum_pi_squared`` returns.  Returns ``(advantages, returns)``."""
+    ``linear_cross_entropy_with_sum_pi_squared`` returns.  ``config`` is accepted and unused (the trainer's
+    dispatcher passes it to every estimator).  Returns ``(advantages, returns)``."""
     return _optimal_token_baseline(token_level_rewards, response_mask, index, old_log_probs, sum_pi_squared,
                                    rollout_is_weights, handle_zero_tail, epsilon, packed=False)
 
@@ -401,7 +438,8 @@ def compute_multi_turn_optimal_token_baseline_advantage(token_level_rewards: tor
                                                         response_mask: torch.Tensor, index: np.ndarray,
                                                         old_log_probs: torch.Tensor, sum_pi_squared: torch.Tensor,
                                                         rollout_is_weights: torch.Tensor = None,
-                                                        handle_zero_tail: bool = True, epsilon: float = 1e-8):
+                                                        handle_zero_tail: bool = True, epsilon: float = 1e-8,
+                                                        config: Optional[Any] = None):
     """Optimal token baseline for tool-integrated (multi-turn) rollouts (reference core_algos.py:876-1004):
     the valid tokens of each trajectory are packed together first, so the k-th generated token of every
     trajectory shares a baseline whatever tool output lies in between; trajectories without a valid token
@@ -817,3 +855,35 @@ def compute_kl_loss(logprob: torch.Tensor, ref_logprob: torch.Tensor, response_m
     return _KlLoss.apply(logprob, ref_logprob, response_mask, _kl_kind(kl_penalty), bool(straight_through),
                          _agg_mode(loss_agg_mode), float(dp_size), _opt(batch_num_tokens), _opt(global_batch_size),
                          _opt(loss_scale_factor))
+
+
+def kl_penalised_rewards(token_level_scores: torch.Tensor, old_log_probs: torch.Tensor, ref_log_prob: torch.Tensor,
+                         response_mask: torch.Tensor, beta: float, kl_penalty: str = "kl"):
+    """The arithmetic of ``apply_kl_penalty`` (reference verl/trainer/ppo/ray_trainer.py:86-101) in one pass:
+    ``kld = kl_penalty(old_log_probs, ref_log_prob) * response_mask``, ``token_level_rewards =
+    token_level_scores - beta * kld`` and ``current_kl = mean_i masked_mean(kld_i, mask_i)``.  Returns
+    ``(token_level_rewards, current_kl)`` with ``current_kl`` a 0-d device tensor (no host sync here)."""
+    with torch.no_grad():
+        dev = _cabi.compute_device(token_level_scores, old_log_probs, ref_log_prob, response_mask)
+        sc = _matrix(token_level_scores, dev)
+        lp = _matrix(old_log_probs, dev)
+        rf = _matrix(ref_log_prob, dev)
+        assert sc.shape == lp.shape == rf.shape
+        m, code = _mask_matrix(response_mask, dev, sc.shape)
+        rows, cols = sc.shape
+        out = torch.empty_like(sc)
+        kl = torch.empty(1, dtype=torch.float32, device=dev)
+        Lb = _cabi.lib()
+        ws = _cabi.ticket_workspace(Lb.vamd_apply_kl_penalty_workspace_bytes(rows, cols), dev)
+        with torch.cuda.device(dev):
+            _cabi.check(Lb.vamd_apply_kl_penalty(sc.data_ptr(), lp.data_ptr(), rf.data_ptr(), m.data_ptr(), code,
+                                                 rows, cols, _kl_kind(kl_penalty), float(beta), out.data_ptr(),
+                                                 kl.data_ptr(), ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
+        out_dev = token_level_scores.device
+        return out.view(token_level_scores.shape).to(out_dev), kl[0].to(out_dev)
+
+
+def compute_rewards(token_level_scores, old_log_prob, ref_log_prob, kl_ratio):
+    """``token_level_scores - (old_log_prob - ref_log_prob) * kl_ratio`` (reference core_algos.py:1009-1022)."""
+    ones = torch.ones(token_level_scores.shape, dtype=torch.uint8, device=token_level_scores.device)
+    return kl_penalised_rewards(token_level_scores, old_log_prob, ref_log_prob, ones, kl_ratio, "kl")[0]
