@@ -232,6 +232,36 @@ int vamd_group_mean_std(const float* scores, const int64_t* group_ids, int64_t n
                         float* mean, float* std, float* count, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * compute_data_metrics (verl/trainer/ppo/metric_utils.py:81-225): every statistic of the step's batch
+ * in one launch.  The five [batch, response_length] fp32 tensors and response_mask are read once;
+ * attention_mask is [batch, prompt_length + response_length] (any VAMD_MASK_* element type) and gives
+ * the prompt and response lengths (:67-70).  values may be NULL (use_critic=False: the VAL_* slots
+ * and VF_EXPLAINED_VAR are then meaningless).  out: VAMD_DM_COUNT device doubles, indexed by the
+ * constants below.  Sequence scores/rewards are taken over non-aborted rows (response length != 0);
+ * means over an empty set come out as NaN, which the caller turns into the reference's exceptions.
+ */
+enum {
+  VAMD_DM_SCORE_MEAN = 0, VAMD_DM_SCORE_MAX, VAMD_DM_SCORE_MIN,
+  VAMD_DM_REWARD_MEAN, VAMD_DM_REWARD_MAX, VAMD_DM_REWARD_MIN,
+  VAMD_DM_ADV_MEAN, VAMD_DM_ADV_MAX, VAMD_DM_ADV_MIN,
+  VAMD_DM_RET_MEAN, VAMD_DM_RET_MAX, VAMD_DM_RET_MIN,
+  VAMD_DM_VAL_MEAN, VAMD_DM_VAL_MAX, VAMD_DM_VAL_MIN,
+  VAMD_DM_VF_EXPLAINED_VAR,
+  VAMD_DM_RESP_LEN_MEAN, VAMD_DM_RESP_LEN_MAX, VAMD_DM_RESP_LEN_MIN, VAMD_DM_RESP_LEN_CLIP,
+  VAMD_DM_RESP_LEN_NA_MEAN, VAMD_DM_RESP_LEN_NA_MAX, VAMD_DM_RESP_LEN_NA_MIN, VAMD_DM_RESP_LEN_NA_CLIP,
+  VAMD_DM_ABORTED_RATIO,
+  VAMD_DM_PROMPT_LEN_MEAN, VAMD_DM_PROMPT_LEN_MAX, VAMD_DM_PROMPT_LEN_MIN, VAMD_DM_PROMPT_LEN_CLIP,
+  VAMD_DM_VALID_TOKENS, /* number of response_mask != 0 elements */
+  VAMD_DM_NON_ABORTED,  /* number of rows with a non-zero response length */
+  VAMD_DM_COUNT
+};
+size_t vamd_data_metrics_workspace_bytes(int64_t batch, int64_t response_length);
+int vamd_data_metrics(const float* token_level_scores, const float* token_level_rewards, const float* advantages,
+                      const float* returns, const float* values, const void* response_mask, int mask_dtype,
+                      const void* attention_mask, int attention_dtype, int64_t batch, int64_t prompt_length,
+                      int64_t response_length, double* out, void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * agg_loss (core_algos.py:1025-1080), forward and backward.
  * out_loss: 1 device float.  coef_out [rows] floats: d loss / d loss_mat[i][t] = coef_out[i] *
  * (float)mask[i][t]; the backward entry point multiplies by the upstream scalar *d_loss.

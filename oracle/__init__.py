@@ -69,4 +69,5 @@ from .trainer import (  # noqa: F401
     apply_kl_penalty,
     adaptive_kl_update,
     compute_rewards,
+    compute_data_metrics,
 )

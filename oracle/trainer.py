@@ -32,3 +32,43 @@ def adaptive_kl_update(value, current_kl, n_steps, target, horizon):
 def compute_rewards(token_level_scores, old_log_prob, ref_log_prob, kl_ratio):
     """verl/trainer/ppo/core_algos.py:1009-1022."""
     return token_level_scores - (old_log_prob - ref_log_prob) * kl_ratio
+
+
+@torch.no_grad()
+def compute_data_metrics(batch, use_critic=True):
+    """verl/trainer/ppo/metric_utils.py:81-225 on a plain mapping of tensors (``batch[name]``); the
+    optional multi-turn entries of ``non_tensor_batch`` (:212-223) are host numpy reductions and are
+    left to the caller."""
+    width = batch["responses"].shape[-1]
+    attention = batch["attention_mask"]
+    prompt_length = attention[:, :-width].sum(-1).float()           # _compute_response_info, :67-70
+    response_length = attention[:, -width:].sum(-1).float()
+    max_prompt_length = attention[:, :-width].size(-1)
+    valid = batch["response_mask"].bool()
+    alive = response_length != 0
+    if int(alive.sum()) == 0:
+        raise ValueError("All samples are aborted, this should not happen.")
+    score = batch["token_level_scores"].sum(-1)[alive]
+    reward = batch["token_level_rewards"].sum(-1)[alive]
+    adv = batch["advantages"][valid]
+    ret = batch["returns"][valid]
+
+    def triple(prefix, x):
+        return {f"{prefix}/mean": x.mean().item(), f"{prefix}/max": x.max().item(), f"{prefix}/min": x.min().item()}
+
+    out = {}
+    out.update(triple("critic/score", score))
+    out.update(triple("critic/rewards", reward))
+    out.update(triple("critic/advantages", adv))
+    out.update(triple("critic/returns", ret))
+    if use_critic:
+        val = batch["values"][valid]
+        out.update(triple("critic/values", val))
+        out["critic/vf_explained_var"] = (1.0 - torch.var(ret - val) / (torch.var(ret) + 1e-5)).item()
+    for prefix, x, cap in (("response_length", response_length, width),
+                           ("response_length_non_aborted", response_length[alive], width),
+                           ("prompt_length", prompt_length, max_prompt_length)):
+        out.update(triple(prefix, x))
+        out[f"{prefix}/clip_ratio"] = (x == cap).float().mean().item()
+    out["response/aborted_ratio"] = (~alive).float().mean().item()
+    return out

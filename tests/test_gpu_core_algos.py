@@ -812,3 +812,66 @@ def test_compute_advantage_dispatch(dev):
     with pytest.raises(NotImplementedError):
         RT.compute_advantage(_data(dict(batch), {"uid": uid}), CA.AdvantageEstimator.GAE, config=cfg)
 
+
+def test_data_metrics_reference_mock_batch(dev):
+    from verl_amd.trainer.ppo.metric_utils import compute_data_metrics
+    case = GOLDEN["data_metrics"]
+    batch = {k: torch.tensor(case[k]).to(dev) for k in ("token_level_scores", "token_level_rewards", "advantages",
+                                                        "returns", "values", "attention_mask", "response_mask")}
+    batch["responses"] = torch.zeros(case["responses_shape"])
+    got = compute_data_metrics(_data(batch), use_critic=True)
+    want = {**case["expected"], **case["expected_by_hand"]}
+    assert set(got) == set(want)
+    for key, value in want.items():
+        assert got[key] == pytest.approx(value, rel=1e-5, abs=1e-5), key
+    without = compute_data_metrics(_data(batch), use_critic=False)
+    assert set(without) == set(want) - {"critic/values/mean", "critic/values/max", "critic/values/min",
+                                        "critic/vf_explained_var"}
+
+
+@pytest.mark.parametrize("shape,prompt", [((3, 17), 5), ((16, 1024), 256), ((5, 4099), 33), ((64, 8192), 1024)])
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.int64, torch.bool])
+@pytest.mark.parametrize("use_critic", [True, False])
+def test_data_metrics(dev, shape, prompt, mdtype, use_critic):
+    from verl_amd.trainer.ppo.metric_utils import compute_data_metrics
+    B, Lc = shape
+    g = torch.Generator().manual_seed(B + Lc + prompt)
+    attention_resp, lens = _prefix_mask(B, Lc, g, lo=1)
+    attention_resp[1] = 0                                        # an aborted sample
+    attention_resp[2] = 1                                        # one that hit the length limit
+    prompt_lens = torch.randint(1, prompt + 1, (B,), generator=g)
+    prompt_lens[0] = prompt
+    attention_prompt = (torch.arange(prompt)[None, :] >= (prompt - prompt_lens)[:, None]).float()   # left padded
+    attention = torch.cat([attention_prompt, attention_resp], dim=1).long()
+    holes = (torch.rand(B, Lc, generator=g) < 0.9).float()       # tool tokens: attended to, not trained on
+    response_mask = attention_resp * holes
+    batch = dict(token_level_scores=torch.randn(B, Lc, generator=g), token_level_rewards=torch.randn(B, Lc, generator=g),
+                 advantages=torch.randn(B, Lc, generator=g), returns=torch.randn(B, Lc, generator=g) + 0.5,
+                 values=torch.randn(B, Lc, generator=g) * 0.5 + 0.5, attention_mask=attention,
+                 response_mask=response_mask.to(mdtype), responses=torch.zeros(B, Lc, dtype=torch.long))
+    want = O.compute_data_metrics({**batch, "response_mask": response_mask}, use_critic=use_critic)
+    extra = {"__num_turns__": np.array([2, 4, 6]), "tool_call_counts": np.array([1, 1, 4])}
+    got = compute_data_metrics(_data({k: v.to(dev) for k, v in batch.items()}, extra), use_critic=use_critic)
+    assert got.pop("num_turns/mean") == 4 and got.pop("num_turns/min") == 2 and got.pop("num_turns/max") == 6
+    assert got.pop("tool_call_counts/mean") == 2 and got.pop("tool_call_counts/min") == 1 and got.pop("tool_call_counts/max") == 4
+    assert set(got) == set(want)
+    for key, value in want.items():
+        # extrema of stored values are exact; row sums, means and ratios are fp32 arithmetic in the reference
+        exact = key.endswith(("/max", "/min")) and not key.startswith(("critic/score", "critic/rewards"))
+        tol = dict(rel=0, abs=0) if exact else dict(rel=2e-5, abs=2e-5)
+        assert got[key] == pytest.approx(value, **tol), key
+
+
+def test_data_metrics_error_cases(dev):
+    from verl_amd.trainer.ppo.metric_utils import compute_data_metrics
+    B, P, Lc = 4, 3, 8
+    z = torch.zeros(B, Lc, device=dev)
+    batch = dict(token_level_scores=z, token_level_rewards=z, advantages=z, returns=z, values=z,
+                 responses=torch.zeros(B, Lc), response_mask=z,
+                 attention_mask=torch.cat([torch.ones(B, P), torch.zeros(B, Lc)], 1).long().to(dev))
+    with pytest.raises(ValueError, match="All samples are aborted"):
+        compute_data_metrics(_data(batch))
+    batch["attention_mask"] = torch.ones(B, P + Lc, dtype=torch.long, device=dev)
+    with pytest.raises(RuntimeError):
+        compute_data_metrics(_data(batch))                       # attended to, but no token in response_mask
+

@@ -56,3 +56,57 @@ def test_kl_controllers_worked_example():
     with pytest.raises(NotImplementedError):
         CA.get_kl_controller(types.SimpleNamespace(type="pid", kl_coef=0.2))
     assert math.isfinite(ctl.value)
+
+
+def test_data_metrics_reference_mock_batch():
+    from conftest import load_golden
+    case = load_golden()["data_metrics"]
+    batch = {k: torch.tensor(case[k]) for k in ("token_level_scores", "token_level_rewards", "advantages", "returns",
+                                                 "values", "attention_mask", "response_mask")}
+    batch["responses"] = torch.zeros(case["responses_shape"])
+    got = O.compute_data_metrics(batch, use_critic=True)
+    for key, want in {**case["expected"], **case["expected_by_hand"]}.items():
+        assert got[key] == pytest.approx(want, rel=1e-5, abs=1e-5), key
+    assert set(got) == set(case["expected"]) | set(case["expected_by_hand"])
+    without = O.compute_data_metrics(batch, use_critic=False)
+    for key in case["keys_without_critic_absent"]:
+        assert key not in without
+    assert set(without) == set(got) - {k for k in got if k.startswith("critic/values") or k == "critic/vf_explained_var"}
+
+
+def test_data_metrics_masks_lengths_and_aborted_rows_by_hand():
+    # row 0: prompt 1 of 2, response 3 of 3 but only 2 tokens in response_mask (a tool token in between);
+    # row 1: aborted (no response tokens); row 2: full prompt, response 1 of 3
+    batch = {
+        "attention_mask": torch.tensor([[0, 1, 1, 1, 1], [1, 1, 0, 0, 0], [1, 1, 1, 0, 0]]),
+        "response_mask": torch.tensor([[1, 0, 1], [0, 0, 0], [1, 0, 0]]),
+        "responses": torch.zeros(3, 3),
+        "token_level_scores": torch.tensor([[1.0, 10.0, 2.0], [100.0, 0.0, 0.0], [4.0, 0.0, 0.0]]),
+        "token_level_rewards": torch.tensor([[0.5, 0.0, 0.5], [9.0, 9.0, 9.0], [2.0, 0.0, 0.0]]),
+        "advantages": torch.tensor([[1.0, 50.0, -2.0], [50.0, 50.0, 50.0], [4.0, 50.0, 50.0]]),
+        "returns": torch.tensor([[1.0, -50.0, 2.0], [-50.0, -50.0, -50.0], [6.0, -50.0, -50.0]]),
+        "values": torch.tensor([[0.0, 7.0, 2.0], [7.0, 7.0, 7.0], [3.0, 7.0, 7.0]]),
+    }
+    got = O.compute_data_metrics(batch)
+    want = {
+        "critic/score/mean": (13.0 + 4.0) / 2, "critic/score/max": 13.0, "critic/score/min": 4.0,   # row 1 is left out
+        "critic/rewards/mean": 1.5, "critic/rewards/max": 2.0, "critic/rewards/min": 1.0,
+        "critic/advantages/mean": 1.0, "critic/advantages/max": 4.0, "critic/advantages/min": -2.0,
+        "critic/returns/mean": 3.0, "critic/returns/max": 6.0, "critic/returns/min": 1.0,
+        "critic/values/mean": 5.0 / 3, "critic/values/max": 3.0, "critic/values/min": 0.0,
+        # returns - values = (1, 0, 3): var 7/3; returns (1, 2, 6): var 7
+        "critic/vf_explained_var": 1.0 - (7.0 / 3) / (7.0 + 1e-5),
+        "response_length/mean": 4.0 / 3, "response_length/max": 3.0, "response_length/min": 0.0,
+        "response_length/clip_ratio": 1.0 / 3,
+        "response_length_non_aborted/mean": 2.0, "response_length_non_aborted/max": 3.0,
+        "response_length_non_aborted/min": 1.0, "response_length_non_aborted/clip_ratio": 0.5,
+        "response/aborted_ratio": 1.0 / 3,
+        "prompt_length/mean": 5.0 / 3, "prompt_length/max": 2.0, "prompt_length/min": 1.0,
+        "prompt_length/clip_ratio": 2.0 / 3,
+    }
+    assert set(got) == set(want)
+    for key, value in want.items():
+        assert got[key] == pytest.approx(value, rel=1e-5, abs=1e-6), key
+    batch["attention_mask"] = torch.tensor([[1, 1, 0, 0, 0]] * 3)
+    with pytest.raises(ValueError, match="aborted"):
+        O.compute_data_metrics(batch)

@@ -1,0 +1,257 @@
+// Per-step batch statistics of the trainer in one pass over the [batch, length] tensors.
+//
+// compute_data_metrics (verl/trainer/ppo/metric_utils.py:81-225) derives about thirty scalars from
+// six tensors with one masked_select / reduction / .item() each.  Here one launch reads every
+// tensor once: each (row, 4096-column chunk) workgroup leaves a record of partial sums and
+// extrema, and the workgroup that arrives last folds the records into per-row quantities
+// (sequence score and reward, prompt and response length) and then into the output vector, so
+// the host reads the whole set with a single copy.
+#include "rowchunk.h"
+
+namespace vamd {
+
+// record slots
+enum {
+  kDmScore = 0,   // sum of token_level_scores over the row chunk (unmasked, :105)
+  kDmReward,      // sum of token_level_rewards (unmasked, :106)
+  kDmRespLen,     // sum of attention_mask over the response columns (:69-70)
+  kDmPromptLen,   // sum of attention_mask over the prompt columns (chunk 0 only)
+  kDmValid,       // number of response_mask != 0 elements
+  kDmAdv, kDmRet, kDmRet2, kDmVal, kDmDiff, kDmDiff2,  // sums over the valid elements
+  kDmAdvMax, kDmAdvMin, kDmRetMax, kDmRetMin, kDmValMax, kDmValMin,
+  kDmRec
+};
+constexpr int kDmSums = kDmAdvMax;  // slots [0, kDmSums) add, the rest are extrema
+
+__device__ __forceinline__ double wave_max(double x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x = fmax(x, __shfl_xor(x, o, 64));
+  return x;
+}
+
+// Maximum of NV doubles per thread over the workgroup; result valid in thread 0.
+template <int NV, int NT>
+__device__ __forceinline__ void block_max(double (&v)[NV], double* smem /* NV * NT/64 doubles */) {
+  constexpr int NW = NT / 64;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    v[i] = wave_max(v[i]);
+    if (lane == 0) smem[i * NW + w] = v[i];
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      double s = smem[i * NW];
+      for (int j = 1; j < NW; ++j) s = fmax(s, smem[i * NW + j]);
+      v[i] = s;
+    }
+  }
+  __syncthreads();
+}
+
+struct DmArgs {
+  const float *scores, *rewards, *adv, *ret, *val;  // val may be null
+  int64_t rows, cols, prompt;                       // attention_mask is [rows][prompt + cols]
+  int chunks;
+  unsigned* ticket;
+  double* records;  // [rows * chunks][kDmRec]
+  double* out;      // [VAMD_DM_COUNT]
+};
+
+template <bool VEC, class M, class A>
+__global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, const M* __restrict__ mask,
+                                                                  const A* __restrict__ attention) {
+  const int64_t row = blockIdx.x / a.chunks;
+  const int chunk = blockIdx.x % a.chunks;
+  const ChunkPos pos(row, chunk, a.cols);
+  const double inf = __longlong_as_double(0x7ff0000000000000ll);
+  double s[kDmSums];
+#pragma unroll
+  for (int i = 0; i < kDmSums; ++i) s[i] = 0;
+  double hi[3] = {-inf, -inf, -inf}, lo[3] = {inf, inf, inf};  // adv, ret, val
+  {
+    float sc[kGroups][4], rw[kGroups][4], ad[kGroups][4], rt[kGroups][4], vl[kGroups][4], m[kGroups][4];
+    load_groups<VEC>(a.scores, pos, sc);
+    load_groups<VEC>(a.rewards, pos, rw);
+    load_groups<VEC>(a.adv, pos, ad);
+    load_groups<VEC>(a.ret, pos, rt);
+    if (a.val) load_groups<VEC>(a.val, pos, vl);
+    load_mask_groups<VEC>(mask, pos, m);
+    const int64_t att_row = row * (a.prompt + a.cols) + a.prompt;
+#pragma unroll
+    for (int k = 0; k < kGroups; ++k) {
+      const int64_t col = pos.idx[k] - row * a.cols;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (e >= pos.valid[k]) continue;
+        s[kDmScore] += (double)sc[k][e];
+        s[kDmReward] += (double)rw[k][e];
+        s[kDmRespLen] += (double)attention[att_row + col + e];
+        if (m[k][e] != 0.f) {
+          const double A_ = ad[k][e], R_ = rt[k][e];
+          s[kDmValid] += 1.0;
+          s[kDmAdv] += A_;
+          s[kDmRet] += R_;
+          s[kDmRet2] += R_ * R_;
+          hi[0] = fmax(hi[0], A_); lo[0] = fmin(lo[0], A_);
+          hi[1] = fmax(hi[1], R_); lo[1] = fmin(lo[1], R_);
+          if (a.val) {
+            const double V_ = vl[k][e];
+            const double D_ = (double)(rt[k][e] - vl[k][e]);  // the fp32 difference the reference forms (:143)
+            s[kDmVal] += V_;
+            s[kDmDiff] += D_;
+            s[kDmDiff2] += D_ * D_;
+            hi[2] = fmax(hi[2], V_); lo[2] = fmin(lo[2], V_);
+          }
+        }
+      }
+    }
+  }
+  if (chunk == 0) {
+    const int64_t p0 = row * (a.prompt + a.cols);
+    for (int64_t c = threadIdx.x; c < a.prompt; c += kRcThreads) s[kDmPromptLen] += (double)attention[p0 + c];
+  }
+  __shared__ double smem[24 * 4];
+  block_sum<kDmSums, kRcThreads>(s, smem);
+  double ext[6] = {hi[0], -lo[0], hi[1], -lo[1], hi[2], -lo[2]};
+  block_max<6, kRcThreads>(ext, smem);
+  if (threadIdx.x == 0) {
+    double* r = a.records + (int64_t)blockIdx.x * kDmRec;
+#pragma unroll
+    for (int i = 0; i < kDmSums; ++i) peer_store(r + i, s[i]);
+#pragma unroll
+    for (int i = 0; i < 6; ++i) peer_store(r + kDmSums + i, (i & 1) ? -ext[i] : ext[i]);
+  }
+  if (!last_block_arrives(a.ticket)) return;
+
+  // ---- fold: thread-strided over rows -------------------------------------------------------------
+  // sums: 0 n_non_aborted 1 score 2 reward 3 resp_len 4 resp_len==cols 5 resp_len (non-aborted)
+  //       6 resp_len==cols (non-aborted) 7 prompt_len 8 prompt_len==prompt
+  //       9.. the valid-element sums kDmValid .. kDmDiff2
+  constexpr int kElem = kDmSums - kDmValid;  // 7
+  double t[9 + kElem];
+#pragma unroll
+  for (int i = 0; i < 9 + kElem; ++i) t[i] = 0;
+  // maxima (minima negated): 0/1 score, 2/3 reward, 4/5 resp_len, 6/7 resp_len non-aborted, 8/9 prompt_len,
+  //                          10..15 adv, ret, val
+  double x[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) x[i] = -inf;
+  for (int64_t r = threadIdx.x; r < a.rows; r += kRcThreads) {
+    double row_s[5] = {0, 0, 0, 0, 0};
+    for (int c = 0; c < a.chunks; ++c) {
+      const double* rec = a.records + (r * a.chunks + c) * kDmRec;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) row_s[i] += peer_load(rec + i);
+#pragma unroll
+      for (int i = 0; i < kElem; ++i) t[9 + i] += peer_load(rec + kDmValid + i);
+#pragma unroll
+      for (int i = 0; i < 6; ++i) {
+        const double v = peer_load(rec + kDmSums + i);
+        x[10 + i] = fmax(x[10 + i], (i & 1) ? -v : v);
+      }
+    }
+    const double score = (double)(float)row_s[kDmScore], reward = (double)(float)row_s[kDmReward];
+    const double rl = row_s[kDmRespLen], pl = row_s[kDmPromptLen];
+    t[3] += rl;
+    t[4] += rl == (double)a.cols ? 1.0 : 0.0;
+    x[4] = fmax(x[4], rl); x[5] = fmax(x[5], -rl);
+    t[7] += pl;
+    t[8] += pl == (double)a.prompt ? 1.0 : 0.0;
+    x[8] = fmax(x[8], pl); x[9] = fmax(x[9], -pl);
+    if (rl != 0.0) {  // not aborted (:119-120)
+      t[0] += 1.0;
+      t[1] += score;
+      t[2] += reward;
+      x[0] = fmax(x[0], score); x[1] = fmax(x[1], -score);
+      x[2] = fmax(x[2], reward); x[3] = fmax(x[3], -reward);
+      t[5] += rl;
+      t[6] += rl == (double)a.cols ? 1.0 : 0.0;
+      x[6] = fmax(x[6], rl); x[7] = fmax(x[7], -rl);
+    }
+  }
+  block_sum<9 + kElem, kRcThreads>(t, smem);
+  block_max<16, kRcThreads>(x, smem);
+  if (threadIdx.x == 0) {
+    double* o = a.out;
+    const double B = (double)a.rows, na = t[0];
+    const double n = t[9 + 0], s_adv = t[9 + 1], s_ret = t[9 + 2], s_ret2 = t[9 + 3], s_val = t[9 + 4],
+                 s_d = t[9 + 5], s_d2 = t[9 + 6];
+    o[VAMD_DM_SCORE_MEAN] = t[1] / na;  o[VAMD_DM_SCORE_MAX] = x[0];  o[VAMD_DM_SCORE_MIN] = -x[1];
+    o[VAMD_DM_REWARD_MEAN] = t[2] / na; o[VAMD_DM_REWARD_MAX] = x[2]; o[VAMD_DM_REWARD_MIN] = -x[3];
+    o[VAMD_DM_ADV_MEAN] = s_adv / n;    o[VAMD_DM_ADV_MAX] = x[10];   o[VAMD_DM_ADV_MIN] = -x[11];
+    o[VAMD_DM_RET_MEAN] = s_ret / n;    o[VAMD_DM_RET_MAX] = x[12];   o[VAMD_DM_RET_MIN] = -x[13];
+    o[VAMD_DM_VAL_MEAN] = s_val / n;    o[VAMD_DM_VAL_MAX] = x[14];   o[VAMD_DM_VAL_MIN] = -x[15];
+    // torch.var: unbiased, NaN for a single element
+    const double var_d = (s_d2 - s_d * s_d / n) / (n - 1.0);
+    const double var_r = (s_ret2 - s_ret * s_ret / n) / (n - 1.0);
+    o[VAMD_DM_VF_EXPLAINED_VAR] = 1.0 - var_d / (var_r + 1e-5);
+    o[VAMD_DM_RESP_LEN_MEAN] = t[3] / B; o[VAMD_DM_RESP_LEN_MAX] = x[4]; o[VAMD_DM_RESP_LEN_MIN] = -x[5];
+    o[VAMD_DM_RESP_LEN_CLIP] = t[4] / B;
+    o[VAMD_DM_RESP_LEN_NA_MEAN] = t[5] / na; o[VAMD_DM_RESP_LEN_NA_MAX] = x[6]; o[VAMD_DM_RESP_LEN_NA_MIN] = -x[7];
+    o[VAMD_DM_RESP_LEN_NA_CLIP] = t[6] / na;
+    o[VAMD_DM_ABORTED_RATIO] = (B - na) / B;
+    o[VAMD_DM_PROMPT_LEN_MEAN] = t[7] / B; o[VAMD_DM_PROMPT_LEN_MAX] = x[8]; o[VAMD_DM_PROMPT_LEN_MIN] = -x[9];
+    o[VAMD_DM_PROMPT_LEN_CLIP] = t[8] / B;
+    o[VAMD_DM_VALID_TOKENS] = n;
+    o[VAMD_DM_NON_ABORTED] = na;
+  }
+  ticket_reset(a.ticket);
+}
+
+}  // namespace vamd
+
+using namespace vamd;
+
+extern "C" size_t vamd_data_metrics_workspace_bytes(int64_t batch, int64_t response_length) {
+  if (batch <= 0 || response_length <= 0) return 0;
+  return kTicketBytes + align_up((size_t)batch * chunks_of(response_length) * kDmRec * sizeof(double), 256);
+}
+
+extern "C" int vamd_data_metrics(const float* token_level_scores, const float* token_level_rewards,
+                                 const float* advantages, const float* returns, const float* values,
+                                 const void* response_mask, int mask_dtype, const void* attention_mask,
+                                 int attention_dtype, int64_t batch, int64_t prompt_length, int64_t response_length,
+                                 double* out, void* workspace, size_t workspace_bytes, void* stream) {
+  VAMD_REQUIRE(batch > 0 && response_length > 0 && prompt_length >= 0, "data_metrics: empty input");
+  VAMD_REQUIRE(batch * chunks_of(response_length) < (1ll << 31), "data_metrics: too many workgroups");
+  VAMD_REQUIRE(token_level_scores && token_level_rewards && advantages && returns && response_mask &&
+                   attention_mask && out,
+               "data_metrics: null pointer");
+  if (!workspace || workspace_bytes < vamd_data_metrics_workspace_bytes(batch, response_length)) {
+    set_error("data_metrics: workspace too small");
+    return VAMD_EWORKSPACE;
+  }
+  DmArgs a;
+  a.scores = token_level_scores; a.rewards = token_level_rewards; a.adv = advantages; a.ret = returns; a.val = values;
+  a.rows = batch; a.cols = response_length; a.prompt = prompt_length;
+  a.chunks = (int)chunks_of(response_length);
+  a.ticket = static_cast<unsigned*>(workspace);
+  a.records = reinterpret_cast<double*>(static_cast<char*>(workspace) + kTicketBytes);
+  a.out = out;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)(batch * a.chunks)), block(kRcThreads);
+#define VAMD_DM(A)                                                                                            \
+  VAMD_MASK_DISPATCH(mask_dtype, M, {                                                                          \
+    const bool vec = can_vectorize(response_length, {token_level_scores, token_level_rewards, advantages,      \
+                                                     returns, values}, response_mask, sizeof(M));              \
+    if (vec)                                                                                                   \
+      hipLaunchKernelGGL((data_metrics_kernel<true, M, A>), grid, block, 0, s, a,                              \
+                         static_cast<const M*>(response_mask), static_cast<const A*>(attention_mask));         \
+    else                                                                                                       \
+      hipLaunchKernelGGL((data_metrics_kernel<false, M, A>), grid, block, 0, s, a,                             \
+                         static_cast<const M*>(response_mask), static_cast<const A*>(attention_mask));         \
+  })
+  switch (attention_dtype) {
+    case VAMD_MASK_F32: VAMD_DM(float); break;
+    case VAMD_MASK_I64: VAMD_DM(int64_t); break;
+    case VAMD_MASK_U8: VAMD_DM(uint8_t); break;
+    case VAMD_MASK_I32: VAMD_DM(int32_t); break;
+    default: set_error("unknown mask dtype code %d", attention_dtype); return VAMD_EINVAL;
+  }
+#undef VAMD_DM
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
