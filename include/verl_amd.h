@@ -262,6 +262,40 @@ int vamd_data_metrics(const float* token_level_scores, const float* token_level_
                       int64_t response_length, double* out, void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Rollout-correction importance weights and off-policy diagnostics
+ * (verl/trainer/ppo/rollout_corr_helper.py: compute_rollout_correction_weights :481-598,
+ * compute_is_metrics :601-712, compute_offpolicy_metrics :835-937) in one pass over old_log_prob,
+ * rollout_log_prob and the (binary) response mask.
+ *   level VAMD_IS_NONE: metrics only.  rollout_log_prob may then be NULL, which leaves only
+ *     TRAINING_PPL, TRAINING_LOG_PPL and VALID_TOKENS defined.
+ *   level VAMD_IS_TOKEN: weights = min(exp(clamp(old - rollout, -20, 20)), threshold) * mask.
+ *   level VAMD_IS_SEQUENCE: one weight per row from the row's summed log ratio, broadcast over the mask.
+ * batch_normalize != 0 divides the weights by their batch mean (per token, or per non-empty sequence)
+ * when that mean exceeds 1e-8; IS_BATCH_NORM_FACTOR reports the divisor (1 when not applied).
+ * The IS_* metrics describe the weights before truncation, as in the reference.
+ * metrics: VAMD_RC_COUNT device doubles indexed by the constants below.
+ */
+#define VAMD_IS_NONE 0
+#define VAMD_IS_TOKEN 1
+#define VAMD_IS_SEQUENCE 2
+enum {
+  VAMD_RC_TRAINING_PPL = 0, VAMD_RC_TRAINING_LOG_PPL, VAMD_RC_KL, VAMD_RC_K3_KL, VAMD_RC_ROLLOUT_PPL,
+  VAMD_RC_ROLLOUT_LOG_PPL, VAMD_RC_LOG_PPL_DIFF, VAMD_RC_LOG_PPL_ABS_DIFF, VAMD_RC_LOG_PPL_DIFF_MAX,
+  VAMD_RC_LOG_PPL_DIFF_MIN, VAMD_RC_PPL_RATIO, VAMD_RC_CHI2_TOKEN, VAMD_RC_CHI2_SEQ,
+  VAMD_RC_IS_MEAN, VAMD_RC_IS_MAX, VAMD_RC_IS_MIN, VAMD_RC_IS_FRACTION_HIGH, VAMD_RC_IS_FRACTION_LOW,
+  VAMD_RC_IS_STD, VAMD_RC_IS_ESS, VAMD_RC_IS_SEQ_MEAN, VAMD_RC_IS_SEQ_STD, VAMD_RC_IS_SEQ_MAX,
+  VAMD_RC_IS_SEQ_MIN, VAMD_RC_IS_SEQ_MAX_DEVIATION, VAMD_RC_IS_SEQ_FRACTION_HIGH, VAMD_RC_IS_SEQ_FRACTION_LOW,
+  VAMD_RC_IS_BATCH_NORM_FACTOR,
+  VAMD_RC_VALID_TOKENS, /* number of mask != 0 elements */
+  VAMD_RC_COUNT
+};
+size_t vamd_rollout_correction_workspace_bytes(int64_t batch, int64_t length);
+int vamd_rollout_correction(const float* old_log_prob, const float* rollout_log_prob, const void* mask,
+                            int mask_dtype, int64_t batch, int64_t length, int level, float threshold,
+                            int batch_normalize, float* weights, double* metrics, void* workspace,
+                            size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * agg_loss (core_algos.py:1025-1080), forward and backward.
  * out_loss: 1 device float.  coef_out [rows] floats: d loss / d loss_mat[i][t] = coef_out[i] *
  * (float)mask[i][t]; the backward entry point multiplies by the upstream scalar *d_loss.

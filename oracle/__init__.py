@@ -71,3 +71,9 @@ from .trainer import (  # noqa: F401
     compute_rewards,
     compute_data_metrics,
 )
+from .rollout_corr import (  # noqa: F401
+    offpolicy_metrics,
+    is_metrics,
+    rollout_correction_weights,
+    rollout_correction_brute_force_fp64,
+)

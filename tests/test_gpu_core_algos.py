@@ -875,3 +875,88 @@ def test_data_metrics_error_cases(dev):
     with pytest.raises(RuntimeError):
         compute_data_metrics(_data(batch))                       # attended to, but no token in response_mask
 
+
+# ---- rollout correction -------------------------------------------------------------------------------
+def _rc_inputs(B, Lc, seed, spread):
+    g = torch.Generator().manual_seed(seed)
+    old = -torch.rand(B, Lc, generator=g) * 3
+    roll = old + torch.randn(B, Lc, generator=g) * spread
+    mask, _ = _prefix_mask(B, Lc, g, lo=1)
+    if B > 2:
+        mask[1] = 0                                              # an empty response
+    return old, roll, mask
+
+
+def _rc_check(got, want32, want64, what):
+    """Hold every metric to the fp64 evaluation as tightly as the reference's fp32 evaluation holds."""
+    assert set(got) == set(want32), (what, set(got) ^ set(want32))
+    for key in want32:
+        err = abs(got[key] - want64[key])
+        assert err <= max(2 * abs(want32[key] - want64[key]), 2e-5 * max(1.0, abs(want64[key]))), (what, key, got[key], want64[key])
+
+
+@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192)])
+@pytest.mark.parametrize("level,spread", [("token", 0.5), ("sequence", 0.02)])
+@pytest.mark.parametrize("normalize", [False, True])
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.int64])
+def test_rollout_correction_weights_and_metrics(dev, shape, level, spread, normalize, mdtype):
+    from verl_amd.trainer.ppo import rollout_corr_helper as RC
+    B, Lc = shape
+    old, roll, mask = _rc_inputs(B, Lc, B + Lc, spread)
+    proto, new_mask, metrics = RC.compute_rollout_correction_and_rejection_mask(
+        old.to(dev), roll.to(dev), mask.to(dev).to(mdtype), rollout_is=level, rollout_is_threshold=1.5,
+        rollout_is_batch_normalize=normalize)
+    w = proto.batch["rollout_is_weights"]
+    assert torch.equal(new_mask.cpu().float(), mask)
+
+    def oracle(dtype):
+        ww, m = O.rollout_correction_weights((old - roll).to(dtype), mask.to(dtype), level, 1.5, normalize)
+        m.update(O.offpolicy_metrics(old.to(dtype), roll.to(dtype), mask.to(dtype)))
+        return ww, m
+
+    w32, m32 = oracle(torch.float32)
+    w64, m64 = oracle(torch.float64)
+    _rc_check({k[len("rollout_corr/"):]: v for k, v in metrics.items()}, m32, m64, "unified")
+    assert all(k.startswith("rollout_corr/") for k in metrics)
+    err = (w.cpu().double() - w64).abs().max().item()
+    assert err <= max(2 * (w32.double() - w64).abs().max().item(), 1e-5), err
+    assert torch.equal(w.cpu()[mask == 0], torch.zeros_like(w.cpu()[mask == 0]))
+
+
+def test_rollout_correction_reference_literals_and_entry_points(dev):
+    from verl_amd.trainer.ppo import rollout_corr_helper as RC
+    case = GOLDEN["rollout_corr_mask_mode"]
+    old, roll, mask = (torch.tensor(case[k]).to(dev) for k in ("old_log_prob", "rollout_log_prob", "response_mask"))
+    proto, _, metrics = RC.compute_rollout_correction_and_rejection_mask(
+        old, roll, mask, rollout_is=case["rollout_is"], rollout_is_threshold=case["rollout_is_threshold"])
+    w = proto.batch["rollout_is_weights"].cpu()
+    assert abs(w[0, 0].item() - case["expected_weight_row0"]) <= case["atol"]
+    assert abs(w[1, 0].item() - case["expected_weight_row1"]) <= case["atol"]
+    names = GOLDEN["rollout_corr_metric_names"]
+    assert {f"rollout_corr/{k}" for k in names["is_metrics"] + names["offpolicy_metrics"]} <= set(metrics)
+    # IS disabled: no weights, the mask unchanged, the off-policy metrics still there (reference test :100-121)
+    proto, new_mask, metrics = RC.compute_rollout_correction_and_rejection_mask(old, roll, mask, rollout_is=None)
+    assert proto is None and torch.equal(new_mask, mask) and "rollout_corr/kl" in metrics
+    assert not any("rollout_is" in k for k in metrics)
+    # the two stand-alone functions
+    o, r, m = _rc_inputs(6, 50, 3, 0.4)
+    got = RC.compute_offpolicy_metrics(o.to(dev), r.to(dev), m.to(dev))
+    _rc_check(got, O.offpolicy_metrics(o, r, m), O.offpolicy_metrics(o.double(), r.double(), m.double()), "offpolicy")
+    assert set(RC.compute_offpolicy_metrics(o.to(dev), None, m.to(dev))) == set(names["offpolicy_metrics_without_rollout"])
+    w, got = RC.compute_rollout_correction_weights((o - r).to(dev), m.to(dev), "token", 2.0, True)
+    w32, m32 = O.rollout_correction_weights(o - r, m, "token", 2.0, True)
+    w64, m64 = O.rollout_correction_weights((o - r).double(), m.double(), "token", 2.0, True)
+    _rc_check(got, m32, m64, "weights")
+    assert (w.cpu().double() - w64).abs().max().item() <= 1e-5
+    with pytest.raises(ValueError, match="Invalid rollout_is"):
+        RC.compute_rollout_correction_weights((o - r).to(dev), m.to(dev), "geometric", 2.0)
+    with pytest.raises(ValueError, match="positive"):
+        RC.compute_rollout_correction_weights((o - r).to(dev), m.to(dev), "token", 0.0)
+    with pytest.raises(ValueError, match="at least one valid token"):
+        RC.compute_rollout_correction_weights((o - r).to(dev), torch.zeros_like(m).to(dev), "token", 2.0)
+    with pytest.raises(ValueError, match="does not match"):
+        RC.compute_rollout_correction_and_rejection_mask(o.to(dev), r[:, :-1].to(dev), m.to(dev))
+    with pytest.raises(NotImplementedError):
+        RC.compute_rollout_correction_and_rejection_mask(o.to(dev), r.to(dev), m.to(dev), rollout_rs="token_k1",
+                                                         rollout_rs_threshold="0.5_2.0")
+

@@ -62,6 +62,9 @@ SIGNATURES = {
     "vamd_data_metrics_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "vamd_data_metrics": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                   c_int64, c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "vamd_rollout_correction_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "vamd_rollout_correction": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_float, c_int,
+                                        c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "vamd_otb_advantage_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int]),
     "vamd_otb_advantage": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                    c_void_p, c_int64, c_int64, c_int64, c_int, c_float, c_void_p, c_void_p, c_void_p,

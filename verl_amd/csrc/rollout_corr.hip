@@ -1,0 +1,367 @@
+// Rollout-correction importance weights and off-policy diagnostics in one pass.
+//
+// compute_rollout_correction_weights + compute_is_metrics + compute_offpolicy_metrics
+// (verl/trainer/ppo/rollout_corr_helper.py:481-712, 835-937) evaluate about thirty masked reductions
+// over old_log_prob, rollout_log_prob and the response mask, each followed by .item().  Here every
+// (row, 4096-column chunk) workgroup reads the three tensors once, writes the truncated token-level
+// weights if those are asked for, and leaves a record of partial sums; the workgroup that arrives
+// last folds the records into per-sequence quantities and then into the metric vector.  Sequence-
+// level weights (one per row, known only after the fold) are broadcast by a second small launch, and
+// batch normalisation of token-level weights is a third.  The response mask is taken as binary.
+#include "rowchunk.h"
+
+namespace vamd {
+
+constexpr float kSafetyBound = 20.f;  // rollout_corr_helper.py:75
+
+enum {
+  kRcM = 0,    // sum of the mask
+  kRcOld,      // sum old_log_prob m
+  kRcRoll,     // sum rollout_log_prob m
+  kRcD,        // sum (old - rollout) m
+  kRcK3,       // sum (exp(d) - d - 1) m
+  kRcRho2,     // sum exp(clamp(d))^2 m
+  kRcW,        // token level: sum w m,  w = exp(clamp(d))
+  kRcC,        // sum clamp(w, 1/thr, thr) m
+  kRcC2,       // sum clamp(w, 1/thr, thr)^2 m
+  kRcTrunc,    // sum min(w, thr) m
+  kRcHigh,     // number of valid tokens with w > thr
+  kRcLow,      // number of valid tokens with w < 1/thr
+  kRcWMax,     // max w over the valid tokens
+  kRcWMinNeg,  // -(min w over the valid tokens)
+  kRcRec
+};
+constexpr int kRcSums = kRcWMax;
+
+struct RcArgs {
+  const float *old_lp, *roll_lp;  // roll_lp may be null: only the training perplexity is produced
+  int64_t rows, cols;
+  int chunks;
+  int level;  // VAMD_IS_*
+  float thr, lower;
+  int normalize;
+  float* weights;      // [rows][cols] or null
+  unsigned* ticket;
+  double* records;     // [rows * chunks][kRcRec]
+  float* row_weight;   // [rows]: sequence-level weight, truncated (and normalised)
+  float* factor;       // [1]: batch-normalisation divisor for the token-level weights (1 when not applied)
+  double* out;         // [VAMD_RC_COUNT]
+};
+
+__device__ __forceinline__ double wave_max_f64(double x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x = fmax(x, __shfl_xor(x, o, 64));
+  return x;
+}
+
+template <int NV, int NT>
+__device__ __forceinline__ void block_max_f64(double (&v)[NV], double* smem) {
+  constexpr int NW = NT / 64;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    v[i] = wave_max_f64(v[i]);
+    if (lane == 0) smem[i * NW + w] = v[i];
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      double s = smem[i * NW];
+      for (int j = 1; j < NW; ++j) s = fmax(s, smem[i * NW + j]);
+      v[i] = s;
+    }
+  }
+  __syncthreads();
+}
+
+template <bool VEC, class M>
+__global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, const M* __restrict__ mask) {
+  const int64_t row = blockIdx.x / a.chunks;
+  const int chunk = blockIdx.x % a.chunks;
+  const ChunkPos pos(row, chunk, a.cols);
+  const double inf = __longlong_as_double(0x7ff0000000000000ll);
+  float s[kRcSums];
+#pragma unroll
+  for (int i = 0; i < kRcSums; ++i) s[i] = 0.f;
+  float wmax = -__builtin_inff(), wmin = __builtin_inff();
+  {
+    float o[kGroups][4], r[kGroups][4], m[kGroups][4], wt[kGroups][4];
+    load_groups<VEC>(a.old_lp, pos, o);
+    if (a.roll_lp) load_groups<VEC>(a.roll_lp, pos, r);
+    load_mask_groups<VEC>(mask, pos, m);
+#pragma unroll
+    for (int k = 0; k < kGroups; ++k)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        wt[k][e] = 0.f;
+        if (e >= pos.valid[k] || m[k][e] == 0.f) continue;
+        s[kRcM] += 1.f;
+        s[kRcOld] += o[k][e];
+        if (!a.roll_lp) continue;
+        const float d = o[k][e] - r[k][e];
+        const float w = expf(fminf(fmaxf(d, -kSafetyBound), kSafetyBound));
+        s[kRcRoll] += r[k][e];
+        s[kRcD] += d;
+        s[kRcK3] += expf(d) - d - 1.f;
+        s[kRcRho2] += w * w;
+        if (a.level == VAMD_IS_TOKEN) {
+          const float c = fminf(fmaxf(w, a.lower), a.thr);
+          const float t = fminf(w, a.thr);
+          s[kRcW] += w;
+          s[kRcC] += c;
+          s[kRcC2] += c * c;
+          s[kRcTrunc] += t;
+          s[kRcHigh] += w > a.thr ? 1.f : 0.f;
+          s[kRcLow] += w < a.lower ? 1.f : 0.f;
+          wmax = fmaxf(wmax, w);
+          wmin = fminf(wmin, w);
+          wt[k][e] = t;
+        }
+      }
+    if (a.level == VAMD_IS_TOKEN && a.weights) store_groups<VEC>(a.weights, pos, wt);
+  }
+  __shared__ double smem[24 * 4];
+  double acc[kRcSums];
+#pragma unroll
+  for (int i = 0; i < kRcSums; ++i) acc[i] = s[i];
+  block_sum<kRcSums, kRcThreads>(acc, smem);
+  double ext[2] = {wmax, -(double)wmin};
+  block_max_f64<2, kRcThreads>(ext, smem);
+  if (threadIdx.x == 0) {
+    double* rec = a.records + (int64_t)blockIdx.x * kRcRec;
+#pragma unroll
+    for (int i = 0; i < kRcSums; ++i) peer_store(rec + i, acc[i]);
+    peer_store(rec + kRcWMax, ext[0]);
+    peer_store(rec + kRcWMinNeg, ext[1]);
+  }
+  if (!last_block_arrives(a.ticket)) return;
+
+  // ---- fold over rows -------------------------------------------------------------------------------
+  enum {
+    tM = 0, tD, tK3, tRho2, tW, tC, tC2, tTrunc, tHigh, tLow,         // token totals
+    tTrainPpl, tTrainLog, tRollPpl, tRollLog, tGap, tGapAbs, tRatio, tChiSeq,  // sums over rows
+    tSeq, tSeq2, tSeqHigh, tSeqLow,                                   // per-sequence mean weight
+    tLogHigh, tLogLow,                                                // sequence level: thresholds in log space
+    tAlive, tSeqTrunc,                                                // rows with tokens; their truncated weights
+    tN
+  };
+  enum { xGap = 0, xGapMinNeg, xW, xWMinNeg, xSeq, xSeqMinNeg, xDev, xLog, xLogMinNeg, xN };
+  double t[tN], x[xN];
+#pragma unroll
+  for (int i = 0; i < tN; ++i) t[i] = 0;
+#pragma unroll
+  for (int i = 0; i < xN; ++i) x[i] = -inf;
+  const float log_hi = logf(a.thr), log_lo = logf(a.lower);
+  const bool seq_level = a.level == VAMD_IS_SEQUENCE;
+  for (int64_t r = threadIdx.x; r < a.rows; r += kRcThreads) {
+    double f[kRcSums];
+#pragma unroll
+    for (int i = 0; i < kRcSums; ++i) f[i] = 0;
+    for (int c = 0; c < a.chunks; ++c) {
+      const double* rec = a.records + (r * a.chunks + c) * kRcRec;
+#pragma unroll
+      for (int i = 0; i < kRcSums; ++i) f[i] += peer_load(rec + i);
+      x[xW] = fmax(x[xW], peer_load(rec + kRcWMax));
+      x[xWMinNeg] = fmax(x[xWMinNeg], peer_load(rec + kRcWMinNeg));
+    }
+    const float Mi = (float)f[kRcM];
+    const float train = (float)f[kRcOld] / (Mi + 1e-8f);  // masked_mean(., axis=-1)
+    t[tM] += f[kRcM]; t[tD] += f[kRcD]; t[tK3] += f[kRcK3]; t[tRho2] += f[kRcRho2];
+    t[tTrainPpl] += (double)expf(-train);
+    t[tTrainLog] += (double)(-train);
+    if (Mi > 0.f) t[tAlive] += 1.0;
+    if (!a.roll_lp) continue;
+    const float roll = (float)f[kRcRoll] / (Mi + 1e-8f);
+    const float gap = roll - train;
+    const float dsum = (float)f[kRcD];
+    const float dsafe = fminf(fmaxf(dsum, -kSafetyBound), kSafetyBound);
+    t[tRollPpl] += (double)expf(-roll);
+    t[tRollLog] += (double)(-roll);
+    t[tGap] += (double)gap;
+    t[tGapAbs] += (double)fabsf(gap);
+    t[tRatio] += (double)expf(gap);
+    t[tChiSeq] += (double)expf(2.f * dsafe);
+    x[xGap] = fmax(x[xGap], (double)gap);
+    x[xGapMinNeg] = fmax(x[xGapMinNeg], -(double)gap);
+    float seq = 0.f;  // masked_mean(weights, axis=-1) of the untruncated weights
+    if (a.level == VAMD_IS_TOKEN) {
+      t[tW] += f[kRcW]; t[tC] += f[kRcC]; t[tC2] += f[kRcC2]; t[tTrunc] += f[kRcTrunc];
+      t[tHigh] += f[kRcHigh]; t[tLow] += f[kRcLow];
+      seq = (float)f[kRcW] / (Mi + 1e-8f);
+    } else if (seq_level) {
+      const float w = expf(dsafe);
+      const float c = fminf(fmaxf(w, a.lower), a.thr);
+      const float tr = fminf(w, a.thr);
+      t[tW] += (double)w * f[kRcM]; t[tC] += (double)c * f[kRcM]; t[tC2] += (double)c * (double)c * f[kRcM];
+      t[tLogHigh] += dsum > log_hi ? 1.0 : 0.0;
+      t[tLogLow] += dsum < log_lo ? 1.0 : 0.0;
+      x[xLog] = fmax(x[xLog], (double)dsum);
+      x[xLogMinNeg] = fmax(x[xLogMinNeg], -(double)dsum);
+      seq = w * Mi / (Mi + 1e-8f);
+      if (Mi > 0.f) t[tSeqTrunc] += (double)(tr * Mi / (Mi + 1e-8f));
+      a.row_weight[r] = tr;
+    }
+    if (a.level != VAMD_IS_NONE) {
+      t[tSeq] += (double)seq;
+      t[tSeq2] += (double)seq * (double)seq;
+      t[tSeqHigh] += seq > a.thr ? 1.0 : 0.0;
+      t[tSeqLow] += seq < a.lower ? 1.0 : 0.0;
+      x[xSeq] = fmax(x[xSeq], (double)seq);
+      x[xSeqMinNeg] = fmax(x[xSeqMinNeg], -(double)seq);
+      x[xDev] = fmax(x[xDev], (double)fabsf(seq - 1.f));
+    }
+  }
+  block_sum<tN, kRcThreads>(t, smem);
+  block_max_f64<xN, kRcThreads>(x, smem);
+  __shared__ float norm;
+  if (threadIdx.x == 0) {
+    double* o = a.out;
+    const double B = (double)a.rows, Mt = t[tM];
+    const double den = (double)((float)Mt + 1e-8f);  // masked_mean over everything
+    o[VAMD_RC_VALID_TOKENS] = Mt;
+    o[VAMD_RC_TRAINING_PPL] = t[tTrainPpl] / B;
+    o[VAMD_RC_TRAINING_LOG_PPL] = t[tTrainLog] / B;
+    o[VAMD_RC_KL] = -t[tD] / den;
+    o[VAMD_RC_K3_KL] = t[tK3] / den;
+    o[VAMD_RC_ROLLOUT_PPL] = t[tRollPpl] / B;
+    o[VAMD_RC_ROLLOUT_LOG_PPL] = t[tRollLog] / B;
+    o[VAMD_RC_LOG_PPL_DIFF] = t[tGap] / B;
+    o[VAMD_RC_LOG_PPL_ABS_DIFF] = t[tGapAbs] / B;
+    o[VAMD_RC_LOG_PPL_DIFF_MAX] = x[xGap];
+    o[VAMD_RC_LOG_PPL_DIFF_MIN] = -x[xGapMinNeg];
+    o[VAMD_RC_PPL_RATIO] = t[tRatio] / B;
+    o[VAMD_RC_CHI2_TOKEN] = t[tRho2] / den - 1.0;
+    o[VAMD_RC_CHI2_SEQ] = t[tChiSeq] / B - 1.0;
+    float divisor = 1.f;
+    if (a.level != VAMD_IS_NONE) {
+      const double mean_c = t[tC] / den, mean_c2 = t[tC2] / den;
+      o[VAMD_RC_IS_MEAN] = t[tW] / den;
+      if (seq_level) {
+        o[VAMD_RC_IS_MAX] = (double)expf(fminf((float)x[xLog], kSafetyBound));
+        o[VAMD_RC_IS_MIN] = (double)expf((float)(-x[xLogMinNeg]));
+        o[VAMD_RC_IS_FRACTION_HIGH] = t[tLogHigh] / B;
+        o[VAMD_RC_IS_FRACTION_LOW] = t[tLogLow] / B;
+      } else {
+        o[VAMD_RC_IS_MAX] = x[xW];
+        o[VAMD_RC_IS_MIN] = -x[xWMinNeg];
+        o[VAMD_RC_IS_FRACTION_HIGH] = t[tHigh] / den;
+        o[VAMD_RC_IS_FRACTION_LOW] = t[tLow] / den;
+      }
+      o[VAMD_RC_IS_STD] = Mt > 1.0 ? sqrt(fmax(mean_c2 - mean_c * mean_c, 0.0)) : 0.0;
+      o[VAMD_RC_IS_ESS] = (mean_c + 1e-8) * (mean_c + 1e-8) / mean_c2;
+      o[VAMD_RC_IS_SEQ_MEAN] = t[tSeq] / B;
+      o[VAMD_RC_IS_SEQ_STD] = B > 1.0 ? sqrt(fmax((t[tSeq2] - t[tSeq] * t[tSeq] / B) / (B - 1.0), 0.0)) : 0.0;
+      o[VAMD_RC_IS_SEQ_MAX] = x[xSeq];
+      o[VAMD_RC_IS_SEQ_MIN] = -x[xSeqMinNeg];
+      o[VAMD_RC_IS_SEQ_MAX_DEVIATION] = x[xDev];
+      o[VAMD_RC_IS_SEQ_FRACTION_HIGH] = t[tSeqHigh] / B;
+      o[VAMD_RC_IS_SEQ_FRACTION_LOW] = t[tSeqLow] / B;
+      o[VAMD_RC_IS_BATCH_NORM_FACTOR] = 1.0;
+      if (a.normalize) {
+        const double mean = seq_level ? t[tSeqTrunc] / fmax(t[tAlive], 1e-8) : t[tTrunc] / den;
+        if (mean > 1e-8) {
+          divisor = (float)mean;
+          o[VAMD_RC_IS_BATCH_NORM_FACTOR] = mean;
+        }
+      }
+    }
+    a.factor[0] = divisor;
+    norm = divisor;
+  }
+  __syncthreads();
+  if (seq_level && norm != 1.f)
+    for (int64_t r = threadIdx.x; r < a.rows; r += kRcThreads) a.row_weight[r] = a.row_weight[r] / norm;
+  ticket_reset(a.ticket);
+}
+
+// weights[i][t] = row_weight[i] * mask[i][t]
+template <bool VEC, class M>
+__global__ __launch_bounds__(kRcThreads) void rollout_broadcast_kernel(const float* __restrict__ row_weight,
+                                                                       const M* __restrict__ mask, int64_t cols,
+                                                                       int chunks, float* __restrict__ weights) {
+  const int64_t row = blockIdx.x / chunks;
+  const ChunkPos pos(row, blockIdx.x % chunks, cols);
+  float m[kGroups][4];
+  load_mask_groups<VEC>(mask, pos, m);
+  const float w = row_weight[row];
+#pragma unroll
+  for (int k = 0; k < kGroups; ++k)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) m[k][e] = m[k][e] != 0.f ? w : 0.f;
+  store_groups<VEC>(weights, pos, m);
+}
+
+// weights /= factor[0] (skipped when the factor is 1)
+__global__ __launch_bounds__(256) void rollout_divide_kernel(float* __restrict__ weights, int64_t n,
+                                                             const float* __restrict__ factor) {
+  const float f = factor[0];
+  if (f == 1.f) return;
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    if (i + e < n) weights[i + e] = weights[i + e] / f;
+}
+
+}  // namespace vamd
+
+using namespace vamd;
+
+extern "C" size_t vamd_rollout_correction_workspace_bytes(int64_t batch, int64_t length) {
+  if (batch <= 0 || length <= 0) return 0;
+  return kTicketBytes + align_up((size_t)batch * chunks_of(length) * kRcRec * sizeof(double), 256) +
+         align_up((size_t)batch * sizeof(float), 256) + 256;
+}
+
+extern "C" int vamd_rollout_correction(const float* old_log_prob, const float* rollout_log_prob, const void* mask,
+                                       int mask_dtype, int64_t batch, int64_t length, int level, float threshold,
+                                       int batch_normalize, float* weights, double* metrics, void* workspace,
+                                       size_t workspace_bytes, void* stream) {
+  VAMD_REQUIRE(batch > 0 && length > 0, "rollout_correction: empty input");
+  VAMD_REQUIRE(batch * chunks_of(length) < (1ll << 31), "rollout_correction: too many workgroups");
+  VAMD_REQUIRE(old_log_prob && mask && metrics, "rollout_correction: null pointer");
+  VAMD_REQUIRE(level >= VAMD_IS_NONE && level <= VAMD_IS_SEQUENCE, "rollout_correction: invalid level %d", level);
+  VAMD_REQUIRE(level == VAMD_IS_NONE || (rollout_log_prob && weights),
+               "rollout_correction: importance weights need rollout_log_prob and an output buffer");
+  VAMD_REQUIRE(level == VAMD_IS_NONE || threshold > 0.f, "rollout_correction: threshold must be positive");
+  if (!workspace || workspace_bytes < vamd_rollout_correction_workspace_bytes(batch, length)) {
+    set_error("rollout_correction: workspace too small");
+    return VAMD_EWORKSPACE;
+  }
+  RcArgs a;
+  a.old_lp = old_log_prob; a.roll_lp = rollout_log_prob;
+  a.rows = batch; a.cols = length; a.chunks = (int)chunks_of(length);
+  a.level = level; a.thr = threshold; a.lower = level == VAMD_IS_NONE ? 0.f : 1.0f / threshold;
+  a.normalize = batch_normalize;
+  a.weights = weights;
+  a.ticket = static_cast<unsigned*>(workspace);
+  Carver carve(static_cast<char*>(workspace) + kTicketBytes);
+  a.records = carve.take<double>((size_t)batch * a.chunks * kRcRec);
+  a.row_weight = carve.take<float>((size_t)batch);
+  a.factor = carve.take<float>(1);
+  a.out = metrics;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)(batch * a.chunks)), block(kRcThreads);
+  VAMD_MASK_DISPATCH(mask_dtype, M, {
+    const M* mk = static_cast<const M*>(mask);
+    const bool vec = can_vectorize(length, {old_log_prob, rollout_log_prob, weights}, mask, sizeof(M));
+    if (vec) {
+      hipLaunchKernelGGL((rollout_stats_kernel<true, M>), grid, block, 0, s, a, mk);
+      if (level == VAMD_IS_SEQUENCE)
+        hipLaunchKernelGGL((rollout_broadcast_kernel<true, M>), grid, block, 0, s, a.row_weight, mk, length, a.chunks,
+                           weights);
+    } else {
+      hipLaunchKernelGGL((rollout_stats_kernel<false, M>), grid, block, 0, s, a, mk);
+      if (level == VAMD_IS_SEQUENCE)
+        hipLaunchKernelGGL((rollout_broadcast_kernel<false, M>), grid, block, 0, s, a.row_weight, mk, length,
+                           a.chunks, weights);
+    }
+  });
+  if (level == VAMD_IS_TOKEN && batch_normalize) {
+    const int64_t n = batch * length;
+    hipLaunchKernelGGL(rollout_divide_kernel, dim3((unsigned)((n + 1023) / 1024)), dim3(256), 0, s, weights, n,
+                       a.factor);
+  }
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
