@@ -71,6 +71,8 @@ extern "C" {
 #define VAMD_PL_CISPO 2   /* -sg(clip(ratio)) A log_prob */
 #define VAMD_PL_SAPO 3    /* -4/tau sigmoid(tau (ratio - 1)) A, tau by the sign of A */
 #define VAMD_PL_GSPO 4    /* clipped objective on the sequence-level importance ratio */
+#define VAMD_PL_REINFORCE 5 /* -log_prob A; the KL metric is taken against old_log_prob = the rollout policy */
+#define VAMD_PL_GEO_MEAN 6  /* GMPO: -A_seq exp(mean_t of the sign-aware clipped log-ratio); mean over all rows */
 
 /* token-level return recurrences (core_algos.py:582-654) */
 #define VAMD_RETURNS_REMAX 0        /* returns = reverse cumsum of r m; adv = returns - baseline_i m */
@@ -328,7 +330,10 @@ int vamd_policy_loss_forward(const float* old_log_prob, const float* log_prob, c
  * does not define left at 0 (GPG: all three; SAPO: both clip fractions; CISPO / GSPO:
  * pg_clipfrac_lower); ppo_kl of GSPO averages the unclamped log-ratio, as the reference does.  tau_pos /
  * tau_neg are SAPO's; clip_c is only read by VAMD_PL_VANILLA.  GSPO runs a per-row pass over
- * log_prob - old_log_prob first (its sequence-level ratio). */
+ * log_prob - old_log_prob first (its sequence-level ratio).  REINFORCE (core_algos.py:1984-2061) reports
+ * only ppo_kl.  GEO_MEAN (:1635-1718) clips the log-ratio to [-clip_low, clip_high], runs a per-row pass
+ * for the geometric means (is_weights enter there, as exp(mean log(w + 1e-10))), ignores mode and the four
+ * agg_loss scalars (the loss is the mean over all rows) and reports all three metrics. */
 size_t vamd_policy_loss_variant_workspace_bytes(int64_t rows, int64_t cols);
 int vamd_policy_loss_variant_forward(int variant, const float* old_log_prob, const float* log_prob,
                                      const float* advantages, const void* mask, int mask_dtype,

@@ -64,6 +64,8 @@ from .losses import (  # noqa: F401
     policy_loss_sapo,
     policy_loss_gpg,
     policy_loss_cispo,
+    policy_loss_reinforce,
+    policy_loss_geo_mean,
 )
 from .trainer import (  # noqa: F401
     apply_kl_penalty,

@@ -175,3 +175,35 @@ def policy_loss_cispo(old_log_prob, log_prob, advantages, response_mask, loss_ag
         losses = losses * rollout_is_weights
     pg_loss = agg_loss(losses, response_mask, loss_agg_mode, **(global_batch_info or {}))
     return pg_loss, pg_clipfrac, masked_mean(-k, response_mask), torch.tensor(0.0)
+
+
+def policy_loss_reinforce(rollout_log_prob, log_prob, advantages, response_mask, loss_agg_mode="seq-mean-token-sum",
+                          rollout_is_weights=None, global_batch_info=None):
+    """REINFORCE with optional importance weights, verl/trainer/ppo/core_algos.py:1984-2061: returns
+    ``(pg_loss, ppo_kl)`` with the KL measured against the rollout policy."""
+    losses = -advantages * log_prob
+    if rollout_is_weights is not None:
+        losses = losses * rollout_is_weights
+    pg_loss = agg_loss(losses, response_mask, loss_agg_mode, **(global_batch_info or {}))
+    return pg_loss, masked_mean(-(log_prob - rollout_log_prob), response_mask)
+
+
+def policy_loss_geo_mean(old_log_prob, log_prob, advantages, response_mask, clip_ratio_low=0.2, clip_ratio_high=0.2,
+                         rollout_is_weights=None):
+    """GMPO, verl/trainer/ppo/core_algos.py:1635-1718: token log-ratios clipped to ``[-low, high]`` on the side
+    that the sign of the advantage makes pessimistic, their masked mean exponentiated into one ratio per
+    sequence, times the masked mean advantage; importance weights enter as their geometric mean per sequence;
+    plain mean over the sequences.  Returns ``(pg_loss, pg_clipfrac, ppo_kl, pg_clipfrac_lower)``."""
+    x = log_prob - old_log_prob
+    sgn = torch.sign(advantages)
+    clamped = torch.clamp(x, -clip_ratio_low, clip_ratio_high)
+    x_min = sgn * torch.min(sgn * x, sgn * clamped)
+    lengths = response_mask.sum(dim=-1)
+    ratio = torch.exp((x_min * response_mask).sum(dim=-1) / (lengths + 1e-8))
+    adv = (advantages * response_mask).sum(dim=-1) / (lengths + 1e-8)
+    losses = -adv * ratio
+    if rollout_is_weights is not None:
+        losses = losses * torch.exp((torch.log(rollout_is_weights + 1e-10) * response_mask).sum(dim=-1) / (lengths + 1e-8))
+    clipped = torch.ne(x, clamped)
+    return (torch.mean(losses), masked_mean((clipped * (advantages > 0)).float(), response_mask),
+            masked_mean(-x, response_mask), masked_mean((clipped * (advantages < 0)).float(), response_mask))

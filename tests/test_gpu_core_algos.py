@@ -579,6 +579,74 @@ def test_policy_loss_variants(dev, variant, mode, with_isw):
            what=f"d {variant} loss / d log_prob")
 
 
+@pytest.mark.parametrize("with_isw", [False, True])
+@pytest.mark.parametrize("shape", [(12, 4200), (5, 77), (32, 1024)])
+def test_policy_loss_geo_mean(dev, with_isw, shape):
+    from verl_amd.trainer.ppo import core_algos as CA
+    B, Lc = shape
+    g = torch.Generator().manual_seed(B + Lc)
+    mask, _ = _prefix_mask(B, Lc, g, lo=3)
+    mask[2] = 0                                                 # an empty response: loss 0, still counted in the mean
+    old = torch.randn(B, Lc, generator=g) * 0.5 - 1
+    new = old + torch.randn(B, Lc, generator=g) * 0.2           # about a third of the tokens beyond the clip range
+    adv = torch.randn(B, 1, generator=g).expand(B, Lc).contiguous()
+    adv[3] = 0                                                  # sign 0: no contribution, no gradient
+    adv[4] = torch.randn(Lc, generator=g)                       # token-level advantages of both signs in one row
+    isw = (torch.rand(B, Lc, generator=g) + 0.5) if with_isw else None
+    cfg = _cfg(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28)
+    nd = new.to(dev).requires_grad_(); no = new.clone().requires_grad_()
+    loss, met = CA.compute_policy_loss_geo_mean(old.to(dev), nd, adv.to(dev), mask.to(dev), "token-mean", cfg,
+                                                None if isw is None else isw.to(dev))
+    want = O.policy_loss_geo_mean(old, no, adv, mask, 0.2, 0.28, isw)
+    assert CA.get_policy_loss_fn("geo_mean") is CA.compute_policy_loss_geo_mean
+    _close(loss, want[0], what="geo_mean loss")
+    assert abs(met["actor/pg_clipfrac"] - want[1].item()) < 1e-6
+    assert abs(met["actor/ppo_kl"] - want[2].item()) < 2e-6 * max(1.0, abs(want[2].item()))
+    assert abs(met["actor/pg_clipfrac_lower"] - want[3].item()) < 1e-6
+    _close(torch.autograd.grad(loss * 2.0, nd)[0], torch.autograd.grad(want[0] * 2.0, no)[0], atol=1e-9,
+           what="d geo_mean loss / d log_prob")
+
+
+@pytest.mark.parametrize("loss_type", ["ppo_clip", "reinforce"])
+@pytest.mark.parametrize("rollout_is", [None, "token", "sequence"])
+@pytest.mark.parametrize("mode", ["token-mean", "seq-mean-token-sum"])
+def test_policy_loss_bypass_mode(dev, loss_type, rollout_is, mode):
+    from verl_amd.trainer.ppo import core_algos as CA
+    g = torch.Generator().manual_seed(21)
+    B, Lc = 10, 600
+    mask, _ = _prefix_mask(B, Lc, g, lo=3)
+    rollout = torch.randn(B, Lc, generator=g) * 0.5 - 1
+    new = rollout + torch.randn(B, Lc, generator=g) * (0.02 if rollout_is == "sequence" else 0.3)
+    adv = torch.randn(B, Lc, generator=g)
+    cfg = _cfg(clip_ratio=0.2)
+    cfg.policy_loss = {"rollout_correction": {"loss_type": loss_type, "rollout_is": rollout_is,
+                                              "rollout_is_threshold": 1.5, "rollout_is_batch_normalize": True}}
+    nd = new.to(dev).requires_grad_(); no = new.clone().requires_grad_()
+    loss, met = CA.compute_policy_loss_bypass_mode(rollout.to(dev), nd, adv.to(dev), mask.to(dev), mode, cfg)
+    w, rc_metrics = None, {}
+    if rollout_is is not None:
+        w, rc_metrics = O.rollout_correction_weights(new - rollout, mask, rollout_is, 1.5, True)
+    rc_metrics.update(O.offpolicy_metrics(new, rollout, mask))
+    if loss_type == "reinforce":
+        want_loss, want_kl = O.policy_loss_reinforce(rollout, no, adv, mask, mode, w)
+        assert set(met) == {"actor/ppo_kl"} | {f"rollout_corr/{k}" for k in rc_metrics}
+    else:
+        out = O.policy_loss_vanilla(rollout, no, adv, mask, mode)
+        want_loss, want_kl = out[0], out[2]
+        assert {"actor/pg_clipfrac", "actor/pg_clipfrac_lower"} <= set(met)
+    _close(loss, want_loss, what="bypass loss")
+    assert abs(met["actor/ppo_kl"] - want_kl.item()) < 2e-6 * max(1.0, abs(want_kl.item()))
+    for k, v in rc_metrics.items():
+        assert met[f"rollout_corr/{k}"] == pytest.approx(v, rel=2e-4, abs=2e-5), k
+    _close(torch.autograd.grad(loss, nd)[0], torch.autograd.grad(want_loss, no)[0], atol=1e-9, what="d bypass loss")
+    assert CA.get_policy_loss_fn("bypass_mode") is CA.compute_policy_loss_bypass_mode
+    with pytest.raises(ValueError, match="rollout_correction config not found"):
+        CA.compute_policy_loss_bypass_mode(rollout.to(dev), nd, adv.to(dev), mask.to(dev), mode, _cfg(clip_ratio=0.2))
+    cfg.policy_loss["rollout_correction"]["loss_type"] = "other"
+    with pytest.raises(ValueError, match="Invalid loss_type"):
+        CA.compute_policy_loss_bypass_mode(rollout.to(dev), nd, adv.to(dev), mask.to(dev), mode, cfg)
+
+
 # ---- KL penalty -------------------------------------------------------------------------------------
 @pytest.mark.parametrize("kind", ["kl", "k1", "abs", "mse", "k2", "low_var_kl", "k3"])
 def test_kl_penalty_elementwise(dev, kind):

@@ -245,3 +245,53 @@ def test_policy_loss_variants_closed_forms():
     rr = torch.exp(seq)[:, None].expand(B, Lc)
     l1 = -adv * rr; l2 = -adv * rr.clamp(1 - 1e-4, 1 + 1e-4)
     assert torch.allclose(cf, ((l2 > l1).double() * mask).sum() / (M_ + 1e-8))
+
+
+def test_reinforce_and_geo_mean_closed_forms():
+    old, new, adv, mask = _policy_inputs()
+    B, Lc = old.shape
+    M_ = mask.sum()
+    # REINFORCE: seq-mean-token-sum of -lp A w; the KL is measured against the first argument
+    w = torch.rand(B, Lc, dtype=torch.float64) + 0.5
+    loss, kl = L.policy_loss_reinforce(old, new, adv, mask, "seq-mean-token-sum", rollout_is_weights=w)
+    assert torch.allclose(loss, (-(new * adv * w) * mask).sum(-1).mean())
+    assert torch.allclose(kl, ((old - new.detach()) * mask).sum() / (M_ + 1e-8))
+    g, = torch.autograd.grad(loss, new)
+    assert torch.allclose(g, -adv * w * mask / B)
+    # GMPO against scalar loops written from the paper's objective: per sequence the geometric mean of the token
+    # ratios, each clipped only where clipping lowers the objective, times the mean advantage
+    lo, hi = 0.05, 0.1
+    loss, cf, kl, cfl = L.policy_loss_geo_mean(old, new, adv, mask, lo, hi, rollout_is_weights=w)
+    total, n_up, n_dn, dsum = 0.0, 0, 0, 0.0
+    grads = torch.zeros(B, Lc, dtype=torch.float64)
+    for i in range(B):
+        toks = [t for t in range(Lc) if mask[i, t] != 0]
+        logs, a_sum, w_logs, free = 0.0, 0.0, 0.0, []
+        for t in toks:
+            x = (new[i, t] - old[i, t]).item()
+            a = adv[i, t].item()
+            c = min(max(x, -lo), hi)
+            if a > 0:
+                k, is_free = min(x, c), x <= hi
+            elif a < 0:
+                k, is_free = max(x, c), x >= -lo
+            else:
+                k, is_free = 0.0, False
+            logs += k; a_sum += a; w_logs += math.log(w[i, t].item() + 1e-10); dsum -= x
+            n_up += (x != c and a > 0); n_dn += (x != c and a < 0)
+            free.append((t, is_free))
+        n = len(toks)
+        row = -(a_sum / n) * math.exp(logs / n) * math.exp(w_logs / n)
+        total += row / B
+        for t, is_free in free:
+            grads[i, t] = row / n / B if is_free else 0.0
+    assert loss.item() == pytest.approx(total, rel=1e-7)      # the reference adds 1e-8 to the lengths
+    assert cf.item() == pytest.approx(n_up / M_.item()) and cfl.item() == pytest.approx(n_dn / M_.item())
+    assert kl.item() == pytest.approx(dsum / M_.item(), rel=1e-9)
+    g, = torch.autograd.grad(loss, new)
+    assert torch.allclose(g, grads, rtol=1e-7, atol=1e-12)
+    # a wide clip range and one advantage per sequence: loss = -mean_i A_i exp(mean_t log-ratio)
+    adv_row = adv[:, :1].expand(B, Lc).contiguous()
+    loss, cf, _, cfl = L.policy_loss_geo_mean(old, new.detach(), adv_row, mask, 50.0, 50.0)
+    seq = ((new.detach() - old) * mask).sum(-1) / mask.sum(-1)
+    assert torch.allclose(loss, (-adv_row[:, 0] * torch.exp(seq)).mean()) and cf.item() == 0 and cfl.item() == 0

@@ -206,6 +206,8 @@ struct PolicyParams {
   int variant;                       // VAMD_PL_*
   float tau_pos, tau_neg;            // SAPO gate temperatures
   const double* row_moments;         // GSPO: [rows][4], slot 0 = sum(m), slot 1 = sum((lp - old) m)
+                                     // GEO_MEAN: [rows][chunks][4] partial sums of geo_rows_kernel
+  float nkl_lo, nkl_hi;              // GEO_MEAN: clip range of the log-ratio, (-clip_low, +clip_high)
 };
 
 // Per-token loss, its derivative with respect to log_prob and the metric contributions of the
@@ -216,6 +218,8 @@ struct PolicyParams {
 //   CISPO    -sg(clip(ratio)) A log_prob                     :1721-1779
 //   SAPO     -4/tau sigmoid(tau (ratio - 1)) A               :1329-1411
 //   GSPO     clipped objective on the sequence-level ratio   :1253-1326
+//   REINFORCE  -log_prob A, KL metric against the rollout policy (compute_policy_loss_reinforce) :1984-2061
+//   GEO_MEAN   -A_seq exp(mean_t clipped log-ratio) per sequence (GMPO)           :1635-1718
 struct TokenLoss {
   float loss, dloss, kl, cf, cfl;  // kl: -(clamped or raw) log-ratio; cf / cfl: 1 where the clip counters fire
 };
@@ -234,6 +238,23 @@ __device__ __forceinline__ TokenLoss token_loss(const PolicyParams& pp, float ol
       t.dloss = -A;
       t.kl = 0.f;
       break;
+    case VAMD_PL_REINFORCE:
+      t.loss = -lp * A;
+      t.dloss = -A;
+      t.kl = -d;
+      break;
+    case VAMD_PL_GEO_MEAN: {
+      // seq_lr carries q = -(A_seq ratio_seq w_seq) / (M + 1e-8): every valid token of the row holds the loss q
+      // (their sum is the sequence loss), and d loss / d log_prob is q where the token's log-ratio enters the
+      // geometric mean unclipped
+      const float c = fminf(fmaxf(d, pp.nkl_lo), pp.nkl_hi);
+      const float ind = A > 0.f ? (d <= pp.nkl_hi ? 1.f : 0.f) : (A < 0.f ? (d >= pp.nkl_lo ? 1.f : 0.f) : 0.f);
+      t.loss = seq_lr;
+      t.dloss = seq_lr * ind;
+      t.kl = -d;
+      t.cf = (d != c && A > 0.f) ? 1.f : 0.f;
+      t.cfl = (d != c && A < 0.f) ? 1.f : 0.f;
+    } break;
     case VAMD_PL_CISPO: {
       const float r = expf(k);
       const float rc = fminf(fmaxf(r, pp.ratio_lo), pp.ratio_hi);
@@ -285,6 +306,49 @@ __device__ __forceinline__ TokenLoss token_loss(const PolicyParams& pp, float ol
   return t;
 }
 
+// GMPO row sums (core_algos.py:1683-1704): per (row, chunk) the partial sums of the mask, of the sign-aware clipped
+// log-ratio, of the advantages and of log(is_weight + 1e-10), each times the mask.
+template <bool VEC, class M, bool ISW>
+__global__ __launch_bounds__(kRcThreads) void geo_rows_kernel(const float* __restrict__ old_lp,
+                                                              const float* __restrict__ lp,
+                                                              const float* __restrict__ adv,
+                                                              const M* __restrict__ mask,
+                                                              const float* __restrict__ isw, int64_t cols, int chunks,
+                                                              float lo, float hi, double* __restrict__ partials) {
+  const int64_t row = blockIdx.x / chunks;
+  const ChunkPos pos(row, blockIdx.x % chunks, cols);
+  float o[kGroups][4], n[kGroups][4], a[kGroups][4], w[kGroups][4], iw[kGroups][4];
+  load_groups<VEC>(old_lp, pos, o);
+  load_groups<VEC>(lp, pos, n);
+  load_groups<VEC>(adv, pos, a);
+  load_mask_groups<VEC>(mask, pos, w);
+  if (ISW) load_groups<VEC>(isw, pos, iw);
+  float s_m = 0, s_k = 0, s_a = 0, s_w = 0;
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (e >= pos.valid[g]) continue;
+      const float d = n[g][e] - o[g][e];
+      const float c = fminf(fmaxf(d, lo), hi);
+      const float A = a[g][e];
+      const float k = A > 0.f ? fminf(d, c) : (A < 0.f ? fmaxf(d, c) : 0.f);
+      const float we = w[g][e];
+      s_m += we;
+      s_k += k * we;
+      s_a += A * we;
+      if (ISW) s_w += logf(iw[g][e] + 1e-10f) * we;
+    }
+  __shared__ double smem[4 * 4];
+  double acc[4] = {s_m, s_k, s_a, s_w};
+  block_sum<4, kRcThreads>(acc, smem);
+  if (threadIdx.x == 0) {
+    double* p = partials + (int64_t)blockIdx.x * 4;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) p[i] = acc[i];
+  }
+}
+
 template <bool VEC, class M, bool GRAD, bool ISW>
 __global__ __launch_bounds__(kRcThreads) void policy_kernel(
     const float* __restrict__ old_lp, const float* __restrict__ lp, const float* __restrict__ adv,
@@ -304,6 +368,17 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
   float seq_lr = 0.f;
   if (pp.variant == VAMD_PL_GSPO)  // sum((lp - old) m) / clamp(sum(m), min = 1)
     seq_lr = (float)pp.row_moments[row * 4 + 1] / fmaxf((float)pp.row_moments[row * 4], 1.f);
+  if (pp.variant == VAMD_PL_GEO_MEAN) {
+    double r[4] = {0, 0, 0, 0};
+    for (int c = 0; c < chunks; ++c)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) r[i] += pp.row_moments[(row * chunks + c) * 4 + i];
+    const float den = (float)r[0] + 1e-8f;
+    const float ratio = expf((float)r[1] / den);
+    const float a_seq = (float)r[2] / den;
+    const float w_seq = expf((float)r[3] / den);  // 1 when no importance weights were given (sum of logs = 0)
+    seq_lr = -a_seq * ratio * w_seq / den;
+  }
   float s_loss = 0, s_m = 0, s_kl = 0, s_cf = 0, s_cfl = 0;
 #pragma unroll
   for (int g = 0; g < kGroups; ++g)
@@ -986,7 +1061,8 @@ extern "C" int vamd_policy_loss_forward(const float* old_log_prob, const float* 
 
 extern "C" size_t vamd_policy_loss_variant_workspace_bytes(int64_t rows, int64_t cols) {
   if (rows <= 0 || cols <= 0) return 0;
-  return reduce_workspace_bytes(rows, cols, 5) + align_up((size_t)rows * 4 * sizeof(double), 256);
+  // the reduction records, then per-row (GSPO) or per-(row, chunk) (GEO_MEAN) sums of the row pre-pass
+  return reduce_workspace_bytes(rows, cols, 5) + align_up((size_t)rows * chunks_of(cols) * 4 * sizeof(double), 256);
 }
 
 extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_log_prob, const float* log_prob,
@@ -1000,7 +1076,7 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
   int st = check_matrix("policy_loss", rows, cols);
   if (st != VAMD_OK) return st;
   VAMD_REQUIRE(old_log_prob && log_prob && advantages && mask && out, "policy_loss: null pointer");
-  VAMD_REQUIRE(variant >= VAMD_PL_VANILLA && variant <= VAMD_PL_GSPO, "policy_loss: invalid variant %d", variant);
+  VAMD_REQUIRE(variant >= VAMD_PL_VANILLA && variant <= VAMD_PL_GEO_MEAN, "policy_loss: invalid variant %d", variant);
   VAMD_REQUIRE(mode >= 0 && mode <= 3, "policy_loss: invalid mode %d", mode);
   VAMD_REQUIRE(variant != VAMD_PL_VANILLA || clip_c > 1.0f, "policy_loss: clip_ratio_c must be > 1.0, got %f",
                (double)clip_c);
@@ -1021,6 +1097,7 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
   pp.tau_pos = tau_pos;
   pp.tau_neg = tau_neg;
   pp.row_moments = nullptr;
+  pp.nkl_lo = pp.nkl_hi = 0.f;
   if (variant == VAMD_PL_GSPO) {  // sequence-level log-ratio: per-row masked moments of log_prob - old_log_prob
     double* row_moments = reinterpret_cast<double*>(static_cast<char*>(workspace) + reduce_workspace_bytes(rows, cols, 5));
     st = masked_moments_of_difference(log_prob, old_log_prob, mask, mask_dtype, rows, cols, 1, row_moments, workspace,
@@ -1028,8 +1105,28 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
     if (st != VAMD_OK) return st;
     pp.row_moments = row_moments;
   }
-  const AggParams ap = make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor);
+  AggParams ap = make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor);
   const dim3 grid((unsigned)(rows * chunks)), block(kRcThreads);
+  if (variant == VAMD_PL_GEO_MEAN) {
+    // the loss is the plain mean of the per-sequence losses over all rows (:1706): every valid token carries its
+    // row's loss / M, summed per row and divided by the number of rows
+    ap = make_agg(VAMD_AGG_SEQ_MEAN_TOKEN_SUM, 1.0, -1.0, (double)rows, -1.0);
+    pp.nkl_lo = -clip_low;
+    pp.nkl_hi = clip_high;
+    double* partials = reinterpret_cast<double*>(static_cast<char*>(workspace) + reduce_workspace_bytes(rows, cols, 5));
+    pp.row_moments = partials;
+#define VAMD_GEO(V, W)                                                                                            \
+  hipLaunchKernelGGL((geo_rows_kernel<V, M, W>), grid, block, 0, s, old_log_prob, log_prob, advantages, mk,       \
+                     is_weights, cols, chunks, pp.nkl_lo, pp.nkl_hi, partials)
+    VAMD_MASK_DISPATCH(mask_dtype, M, {
+      const bool vec = can_vectorize(cols, {old_log_prob, log_prob, advantages, is_weights}, mask, sizeof(M));
+      const M* mk = static_cast<const M*>(mask);
+      if (vec) { if (is_weights) VAMD_GEO(true, true); else VAMD_GEO(true, false); }
+      else { if (is_weights) VAMD_GEO(false, true); else VAMD_GEO(false, false); }
+    });
+#undef VAMD_GEO
+    is_weights = nullptr;  // already folded into the sequence loss
+  }
 #define VAMD_PL(V, G, W)                                                                                     \
   hipLaunchKernelGGL((policy_kernel<V, M, G, W>), grid, block, 0, s, old_log_prob, log_prob, advantages, mk, \
                      is_weights, rows, cols, chunks, pp, ap, wk, out, grad_unscaled, coef_out)

@@ -603,7 +603,7 @@ def compute_policy_loss_vanilla(old_log_prob: torch.Tensor, log_prob: torch.Tens
     return pg_loss, pg_metrics
 
 
-_PL = {"vanilla": 0, "gpg": 1, "cispo": 2, "sapo": 3, "gspo": 4}
+_PL = {"vanilla": 0, "gpg": 1, "cispo": 2, "sapo": 3, "gspo": 4, "reinforce": 5, "geo_mean": 6}
 
 
 def _policy_loss_variant(variant, old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, config,
@@ -669,6 +669,71 @@ def compute_policy_loss_cispo(old_log_prob: torch.Tensor, log_prob: torch.Tensor
     assert config is not None
     return _policy_loss_variant("cispo", old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, config,
                                 rollout_is_weights)
+
+
+@register_policy_loss("geo_mean")
+def compute_policy_loss_geo_mean(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                                 response_mask: torch.Tensor, loss_agg_mode: str = "token-mean",
+                                 config: Optional[Any] = None, rollout_is_weights: torch.Tensor | None = None):
+    """GMPO (reference core_algos.py:1635-1718): per sequence ``-mean_t(A) * exp(mean_t clipped log-ratio)``, the
+    log-ratio clipped to ``[-clip_ratio_low, clip_ratio_high]`` on the side the advantage's sign makes
+    pessimistic; importance weights enter as their geometric mean per sequence; the loss is the plain mean over
+    the sequences (``loss_agg_mode`` is not used, as there)."""
+    assert config is not None
+    return _policy_loss_variant("geo_mean", old_log_prob, log_prob, advantages, response_mask, "seq-mean-token-sum",
+                                config, rollout_is_weights)
+
+
+def compute_policy_loss_reinforce(rollout_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                                  response_mask: torch.Tensor, loss_agg_mode: str = "seq-mean-token-sum",
+                                  config: Optional[Any] = None, rollout_is_weights: Optional[torch.Tensor] = None):
+    """REINFORCE with optional importance weights (reference core_algos.py:1984-2061):
+    ``agg_loss(-A log_prob [w])``; ``actor/ppo_kl`` is measured against the rollout policy."""
+    assert config is not None, "ActorConfig must be provided for REINFORCE loss"
+    pg_loss, metrics = _policy_loss_variant("reinforce", rollout_log_prob, log_prob, advantages, response_mask,
+                                            loss_agg_mode, config, rollout_is_weights, needs_clip=False)
+    return pg_loss, {"actor/ppo_kl": metrics["actor/ppo_kl"]}
+
+
+@register_policy_loss("bypass_mode")
+def compute_policy_loss_bypass_mode(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                                    response_mask: torch.Tensor, loss_agg_mode: str = "token-mean",
+                                    config: Optional[Any] = None, rollout_is_weights: torch.Tensor | None = None):
+    """Bypass mode (reference core_algos.py:2064-2187): ``old_log_prob`` is the rollout policy's; the importance
+    weights ``pi_current / pi_rollout`` and the off-policy metrics are computed here from
+    ``config.policy_loss["rollout_correction"]`` (``loss_type`` "ppo_clip" or "reinforce", ``rollout_is``,
+    ``rollout_is_threshold``, ``rollout_is_batch_normalize``), then the clipped PPO loss (without the weights)
+    or the REINFORCE loss (with them) is returned with both sets of metrics.  ``rollout_is_weights`` is
+    ignored, as there.  ``rollout_rs`` raises ``NotImplementedError``."""
+    from .rollout_corr_helper import compute_rollout_correction_and_rejection_mask
+
+    assert config is not None, "config is required for bypass_mode loss"
+    rc = config.policy_loss.get("rollout_correction", None) if hasattr(config, "policy_loss") else None
+    if rc is None:
+        raise ValueError(
+            "rollout_correction config not found in policy_loss. "
+            "When using loss_mode='bypass_mode', ensure rollout_correction config is passed."
+        )
+    loss_type = rc.get("loss_type", "ppo_clip")
+    with torch.no_grad():
+        proto, effective_mask, rollout_metrics = compute_rollout_correction_and_rejection_mask(
+            old_log_prob=log_prob.detach(), rollout_log_prob=old_log_prob, response_mask=response_mask,
+            rollout_is=rc.get("rollout_is", None), rollout_is_threshold=rc.get("rollout_is_threshold", 2.0),
+            rollout_is_batch_normalize=rc.get("rollout_is_batch_normalize", False),
+            rollout_rs=rc.get("rollout_rs", None), rollout_rs_threshold=rc.get("rollout_rs_threshold", None))
+    weights = proto.batch["rollout_is_weights"] if proto else None
+    if loss_type == "reinforce":
+        pg_loss, pg_metrics = compute_policy_loss_reinforce(
+            rollout_log_prob=old_log_prob, log_prob=log_prob, advantages=advantages, response_mask=effective_mask,
+            loss_agg_mode=loss_agg_mode, config=config, rollout_is_weights=weights)
+    elif loss_type == "ppo_clip":
+        pg_loss, pg_metrics = compute_policy_loss_vanilla(
+            old_log_prob=old_log_prob, log_prob=log_prob, advantages=advantages, response_mask=effective_mask,
+            loss_agg_mode=loss_agg_mode, config=config, rollout_is_weights=None)
+    else:
+        raise ValueError(f"Invalid loss_type: {loss_type}. Must be 'reinforce' or 'ppo_clip'.")
+    pg_metrics.update(rollout_metrics)
+    return pg_loss, pg_metrics
 
 
 def compute_policy_loss(old_log_prob, log_prob, advantages, response_mask, cliprange=None, cliprange_low=None,
