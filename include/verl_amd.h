@@ -234,6 +234,20 @@ int vamd_group_mean_std(const float* scores, const int64_t* group_ids, int64_t n
                         float* mean, float* std, float* count, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Remove-padding output -> response window (verl/workers/actor/dp_actor.py:316-344: pad_input to
+ * [batch, seqlen], then the columns [-response_length - 1, -1)).  a / b / c: per-token values [nnz] in the
+ * order of indices (b, c optional); indices: the tokens' flat positions row * seqlen + col, ascending;
+ * out_*: [batch, response_length], every element written (0 where no token lies).  The gather is the
+ * backward direction: d_a[i] = d_out_a[row][j] for tokens inside the window, 0 for the others.
+ */
+int vamd_response_window_scatter(const float* a, const float* b, const float* c, const int64_t* indices,
+                                 int64_t nnz, int64_t batch, int64_t seqlen, int64_t response_length, float* out_a,
+                                 float* out_b, float* out_c, void* stream);
+int vamd_response_window_gather(const float* d_out_a, const float* d_out_b, const int64_t* indices, int64_t nnz,
+                                int64_t batch, int64_t seqlen, int64_t response_length, float* d_a, float* d_b,
+                                void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * compute_data_metrics (verl/trainer/ppo/metric_utils.py:81-225): every statistic of the step's batch
  * in one launch.  The five [batch, response_length] fp32 tensors and response_mask are read once;
  * attention_mask is [batch, prompt_length + response_length] (any VAMD_MASK_* element type) and gives

@@ -72,6 +72,7 @@ from .trainer import (  # noqa: F401
     adaptive_kl_update,
     compute_rewards,
     compute_data_metrics,
+    pad_to_response_window,
 )
 from .rollout_corr import (  # noqa: F401
     offpolicy_metrics,

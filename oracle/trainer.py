@@ -72,3 +72,11 @@ def compute_data_metrics(batch, use_critic=True):
         out[f"{prefix}/clip_ratio"] = (x == cap).float().mean().item()
     out["response/aborted_ratio"] = (~alive).float().mean().item()
     return out
+
+
+def pad_to_response_window(values, indices, batch, seqlen, response_length):
+    """``pad_input`` (scatter the per-token values to their flat positions in a zero ``(batch * seqlen)``
+    buffer) followed by the slice ``[:, -response_length - 1:-1]``, verl/workers/actor/dp_actor.py:316-344."""
+    full = torch.zeros(batch * seqlen, dtype=values.dtype)
+    full = full.index_put((indices,), values)
+    return full.view(batch, seqlen)[:, -response_length - 1:-1]

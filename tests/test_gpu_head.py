@@ -17,6 +17,7 @@ import pytest
 import torch
 
 from oracle import head as OH
+import oracle as O
 
 pytestmark = pytest.mark.gpu
 
@@ -324,3 +325,33 @@ def test_sum_pi_squared_from_the_head(dev, n, h, v, T):
     assert pi2.shape == (n,) and pi2.dtype == torch.float32
     assert (pi2 >= 1.0 / v - 1e-9).all() and (pi2 <= 1.0 + 1e-6).all()
     assert torch.allclose(pi2, want, rtol=2e-3, atol=1e-9), ((pi2 - want).abs() / want).max().item()
+
+
+@pytest.mark.parametrize("geometry", [(2, 5, 2), (8, 96, 64), (16, 1500, 1499), (4, 64, 1)])
+def test_pad_to_response_window(dev, geometry):
+    """The remove-padding outputs land in the response window exactly as pad_input + slice place them, and the
+    upstream gradients come back to the tokens (reference dp_actor.py:316-344)."""
+    from verl_amd.utils.kernel.response_window import pad_to_response_window
+    B, S, Lr = geometry
+    g = torch.Generator().manual_seed(B * S + Lr)
+    left = torch.randint(0, S // 2 + 1, (B,), generator=g)       # left padding of the prompt
+    right = torch.randint(0, S // 2, (B,), generator=g)          # right padding of the response
+    pos = torch.arange(S)[None, :]
+    attention = ((pos >= left[:, None]) & (pos < (S - right)[:, None])).long()
+    attention[0] = 1
+    indices = attention.flatten().nonzero().flatten()
+    nnz = indices.numel()
+    vals = [torch.randn(nnz, generator=g) for _ in range(3)]
+    dv = [v.to(dev).requires_grad_() for v in vals[:2]] + [vals[2].to(dev)]
+    got = pad_to_response_window(indices.to(dev), B, S, Lr, *dv)
+    assert len(got) == 3
+    ov = [v.clone().requires_grad_() for v in vals]
+    want = [O.pad_to_response_window(v, indices, B, S, Lr) for v in ov]
+    for a, b in zip(got, want):
+        assert a.shape == (B, Lr) and torch.equal(a.cpu(), b.detach())
+    up = [torch.randn(B, Lr, generator=g) for _ in range(2)]
+    (got[0] * up[0].to(dev)).sum().add((got[1] * up[1].to(dev)).sum()).backward()
+    (want[0] * up[0]).sum().add((want[1] * up[1]).sum()).backward()
+    assert torch.equal(dv[0].grad.cpu(), ov[0].grad) and torch.equal(dv[1].grad.cpu(), ov[1].grad)
+    only, = pad_to_response_window(indices.to(dev), B, S, Lr, vals[0].to(dev))
+    assert torch.equal(only.cpu(), want[0].detach())

@@ -110,3 +110,14 @@ def test_data_metrics_masks_lengths_and_aborted_rows_by_hand():
     batch["attention_mask"] = torch.tensor([[1, 1, 0, 0, 0]] * 3)
     with pytest.raises(ValueError, match="aborted"):
         O.compute_data_metrics(batch)
+
+
+def test_pad_to_response_window_by_hand():
+    # batch 2, seqlen 5, response 2: the window is columns 2 and 3 of each row
+    attention = torch.tensor([[0, 1, 1, 1, 1], [1, 1, 1, 0, 0]])
+    indices = attention.flatten().nonzero().flatten()            # 1 2 3 4 | 5 6 7
+    values = torch.tensor([10.0, 11.0, 12.0, 13.0, 20.0, 21.0, 22.0], requires_grad=True)
+    out = O.pad_to_response_window(values, indices, 2, 5, 2)
+    assert out.tolist() == [[11.0, 12.0], [22.0, 0.0]]
+    out.backward(torch.tensor([[1.0, 2.0], [3.0, 4.0]]))
+    assert values.grad.tolist() == [0.0, 1.0, 2.0, 0.0, 0.0, 0.0, 3.0]

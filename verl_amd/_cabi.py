@@ -65,6 +65,10 @@ SIGNATURES = {
     "vamd_rollout_correction_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "vamd_rollout_correction": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_float, c_int,
                                         c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "vamd_response_window_scatter": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                             c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "vamd_response_window_gather": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+                                            c_void_p, c_void_p, c_void_p]),
     "vamd_otb_advantage_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int]),
     "vamd_otb_advantage": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                    c_void_p, c_int64, c_int64, c_int64, c_int, c_float, c_void_p, c_void_p, c_void_p,
