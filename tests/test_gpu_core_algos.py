@@ -712,6 +712,39 @@ def test_kl_loss_fused(dev, mode, kind, mdtype):
     _close(torch.autograd.grad(got_st, ld2)[0], torch.autograd.grad(want_st, lo2)[0], atol=1e-7, what="straight-through grad")
 
 
+@pytest.mark.parametrize("mode", MODES)
+def test_losses_with_the_fold_in_its_own_launch(dev, mode):
+    """More (row, chunk) records than the last workgroup folds itself: the loss kernels leave the fold to a second
+    launch.  Same checks as the small shapes, on agg_loss, the policy loss, the value loss and the fused KL loss."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    B, Lc = 1500, 4100                                           # 3000 records
+    old, new, adv, mask = _policy_inputs(B, Lc, seed=5)
+    cfg = _cfg(clip_ratio=0.2, clip_ratio_high=0.28)
+    nd = new.to(dev).requires_grad_(); no = new.clone().requires_grad_()
+    loss, metrics = CA.compute_policy_loss_vanilla(old.to(dev), nd, adv.to(dev), mask.to(dev), mode, cfg)
+    w_loss, w_cf, w_kl, w_cfl = O.policy_loss_vanilla(old, no, adv, mask, mode, 0.2, 0.28, 3.0)
+    _close(loss, w_loss, what="pg_loss " + mode)
+    assert abs(metrics["actor/pg_clipfrac"] - w_cf.item()) <= 1e-6
+    assert abs(metrics["actor/ppo_kl"] - w_kl.item()) <= 1e-5 * abs(w_kl.item()) + 1e-6
+    assert abs(metrics["actor/pg_clipfrac_lower"] - w_cfl.item()) <= 1e-6
+    _close(torch.autograd.grad(loss, nd)[0], torch.autograd.grad(w_loss, no)[0], atol=1e-10, what="d pg_loss")
+    xd = adv.to(dev).requires_grad_(); xo = adv.clone().requires_grad_()
+    got = CA.agg_loss(xd, mask.to(dev), mode); want = O.agg_loss(xo, mask, mode)
+    _close(got, want, what="agg_loss " + mode)
+    _close(torch.autograd.grad(got, xd)[0], torch.autograd.grad(want, xo)[0], atol=1e-10, what="d agg_loss")
+    vd = new.to(dev).requires_grad_(); vo = new.clone().requires_grad_()
+    vl, vf = CA.compute_value_loss(vd, adv.to(dev), old.to(dev), mask.to(dev), 0.5, mode)
+    wl, wf = O.value_loss(vo, adv, old, mask, 0.5, mode)
+    _close(vl, wl, what="vf_loss " + mode)
+    assert abs(float(vf) - wf.item()) <= 1e-6
+    _close(torch.autograd.grad(vl, vd)[0], torch.autograd.grad(wl, vo)[0], atol=1e-10, what="d vf_loss")
+    kd = new.to(dev).requires_grad_(); ko = new.clone().requires_grad_()
+    kl = CA.compute_kl_loss(kd, old.to(dev), mask.to(dev), "low_var_kl", mode)
+    wk = O.agg_loss(O.kl_penalty(ko, old, "low_var_kl"), mask, mode)
+    _close(kl, wk, what="kl_loss " + mode)
+    _close(torch.autograd.grad(kl, kd)[0], torch.autograd.grad(wk, ko)[0], atol=1e-9, what="d kl_loss")
+
+
 # ---- the two benchmark configurations end to end --------------------------------------------------
 def test_benchmark_config_grpo_policy_loss(dev):
     """512 responses in 64 groups of 8, L = 4096, lengths U[64, 4096], Bernoulli(0.5) outcome reward

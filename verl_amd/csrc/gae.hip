@@ -50,7 +50,7 @@ constexpr int kSegBatch = 4;  // segments whose loads are issued together (48 Ki
 
 struct GaeWork {
   unsigned* ticket;   // workspace head: zero on entry, zero on exit
-  double* partials;   // [rows][4] masked moments of the raw advantages
+  double* partials;   // per row the 4 masked moments of the raw advantages; slot-major
 };
 
 template <bool VEC, class M>
@@ -186,15 +186,12 @@ __global__ __launch_bounds__(kRcThreads) void gae_scan_kernel(const float* __res
   double acc[4] = {m0, m1, m2, mc};
   block_sum<4, kRcThreads>(acc, smem);
   if (tid == 0) {
-    double* o = wk.partials + row * 4;
-    peer_store(o + 0, acc[0]); peer_store(o + 1, acc[1]); peer_store(o + 2, acc[2]); peer_store(o + 3, acc[3]);
+    store_record<4>(wk.partials, row, 0, rows, 1, acc);
   }
   if (!last_block_arrives(wk.ticket)) return;
   // the last row to finish folds the per-row moments and derives the whitening statistics
   double a[4] = {0, 0, 0, 0};
-  for (int64_t k = tid; k < rows; k += kRcThreads)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) a[i] += peer_load(wk.partials + k * 4 + i);
+  sum_records_strided<4>(wk.partials, rows, a);
   block_sum<4, kRcThreads>(a, smem);
   if (tid == 0) {
 #pragma unroll

@@ -3,9 +3,11 @@
 // compute_data_metrics (verl/trainer/ppo/metric_utils.py:81-225) derives about thirty scalars from
 // six tensors with one masked_select / reduction / .item() each.  Here one launch reads every
 // tensor once: each (row, 4096-column chunk) workgroup leaves a record of partial sums and
-// extrema, and the workgroup that arrives last folds the records into per-row quantities
-// (sequence score and reward, prompt and response length) and then into the output vector, so
-// the host reads the whole set with a single copy.
+// extrema.  A second, single-workgroup launch folds the records into per-row quantities (sequence
+// score and reward, prompt and response length) and then into the output vector, so the host
+// reads the whole set with a single copy.  The fold is a launch of its own because its registers
+// (a 17-slot record per row in flight, 32 running statistics) would otherwise be charged to every
+// wavefront of the streaming kernel.
 #include "rowchunk.h"
 
 namespace vamd {
@@ -18,7 +20,7 @@ enum {
   kDmPromptLen,   // sum of attention_mask over the prompt columns (chunk 0 only)
   kDmValid,       // number of response_mask != 0 elements
   kDmAdv, kDmRet, kDmRet2, kDmVal, kDmDiff, kDmDiff2,  // sums over the valid elements
-  kDmAdvMax, kDmAdvMin, kDmRetMax, kDmRetMin, kDmValMax, kDmValMin,
+  kDmAdvMax, kDmAdvMinNeg, kDmRetMax, kDmRetMinNeg, kDmValMax, kDmValMinNeg,  // minima are stored negated
   kDmRec
 };
 constexpr int kDmSums = kDmAdvMax;  // slots [0, kDmSums) add, the rest are extrema
@@ -55,8 +57,7 @@ struct DmArgs {
   const float *scores, *rewards, *adv, *ret, *val;  // val may be null
   int64_t rows, cols, prompt;                       // attention_mask is [rows][prompt + cols]
   int chunks;
-  unsigned* ticket;
-  double* records;  // [rows * chunks][kDmRec]
+  double* records;  // kDmRec slots per (row, chunk) workgroup, slot-major
   double* out;      // [VAMD_DM_COUNT]
 };
 
@@ -66,66 +67,74 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
   const int64_t row = blockIdx.x / a.chunks;
   const int chunk = blockIdx.x % a.chunks;
   const ChunkPos pos(row, chunk, a.cols);
-  const double inf = __longlong_as_double(0x7ff0000000000000ll);
-  double s[kDmSums];
+  // per-thread partials over its 16 elements in fp32 (exact counts, 1e-7 relative on the sums), widened below
+  float s[kDmSums];
 #pragma unroll
-  for (int i = 0; i < kDmSums; ++i) s[i] = 0;
-  double hi[3] = {-inf, -inf, -inf}, lo[3] = {inf, inf, inf};  // adv, ret, val
-  {
-    float sc[kGroups][4], rw[kGroups][4], ad[kGroups][4], rt[kGroups][4], vl[kGroups][4], m[kGroups][4];
-    load_groups<VEC>(a.scores, pos, sc);
-    load_groups<VEC>(a.rewards, pos, rw);
-    load_groups<VEC>(a.adv, pos, ad);
-    load_groups<VEC>(a.ret, pos, rt);
-    if (a.val) load_groups<VEC>(a.val, pos, vl);
-    load_mask_groups<VEC>(mask, pos, m);
-    const int64_t att_row = row * (a.prompt + a.cols) + a.prompt;
+  for (int i = 0; i < kDmSums; ++i) s[i] = 0.f;
+  float hi[3] = {-__builtin_inff(), -__builtin_inff(), -__builtin_inff()};  // adv, ret, val
+  float lo[3] = {__builtin_inff(), __builtin_inff(), __builtin_inff()};
+  const int64_t att_row = row * (a.prompt + a.cols) + a.prompt;
+#pragma unroll 2
+  for (int k = 0; k < kGroups; ++k) {
+    if (pos.valid[k] <= 0) continue;
+    float sc[4], rw[4], ad[4], rt[4], vl[4] = {0.f, 0.f, 0.f, 0.f}, m[4], at[4];
+    ld4<VEC>(a.scores, pos.idx[k], pos.valid[k], sc);
+    ld4<VEC>(a.rewards, pos.idx[k], pos.valid[k], rw);
+    ld4<VEC>(a.adv, pos.idx[k], pos.valid[k], ad);
+    ld4<VEC>(a.ret, pos.idx[k], pos.valid[k], rt);
+    if (a.val) ld4<VEC>(a.val, pos.idx[k], pos.valid[k], vl);
+    ldmask4<VEC>(mask, pos.idx[k], pos.valid[k], m);
+    ldmask4<VEC>(attention, att_row + (pos.idx[k] - row * a.cols), pos.valid[k], at);
 #pragma unroll
-    for (int k = 0; k < kGroups; ++k) {
-      const int64_t col = pos.idx[k] - row * a.cols;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (e >= pos.valid[k]) continue;
-        s[kDmScore] += (double)sc[k][e];
-        s[kDmReward] += (double)rw[k][e];
-        s[kDmRespLen] += (double)attention[att_row + col + e];
-        if (m[k][e] != 0.f) {
-          const double A_ = ad[k][e], R_ = rt[k][e];
-          s[kDmValid] += 1.0;
-          s[kDmAdv] += A_;
-          s[kDmRet] += R_;
-          s[kDmRet2] += R_ * R_;
-          hi[0] = fmax(hi[0], A_); lo[0] = fmin(lo[0], A_);
-          hi[1] = fmax(hi[1], R_); lo[1] = fmin(lo[1], R_);
-          if (a.val) {
-            const double V_ = vl[k][e];
-            const double D_ = (double)(rt[k][e] - vl[k][e]);  // the fp32 difference the reference forms (:143)
-            s[kDmVal] += V_;
-            s[kDmDiff] += D_;
-            s[kDmDiff2] += D_ * D_;
-            hi[2] = fmax(hi[2], V_); lo[2] = fmin(lo[2], V_);
-          }
+    for (int e = 0; e < 4; ++e) {
+      if (e >= pos.valid[k]) continue;
+      s[kDmScore] += sc[e];
+      s[kDmReward] += rw[e];
+      s[kDmRespLen] += at[e];
+      if (m[e] != 0.f) {
+        s[kDmValid] += 1.f;
+        s[kDmAdv] += ad[e];
+        s[kDmRet] += rt[e];
+        s[kDmRet2] += rt[e] * rt[e];
+        hi[0] = fmaxf(hi[0], ad[e]); lo[0] = fminf(lo[0], ad[e]);
+        hi[1] = fmaxf(hi[1], rt[e]); lo[1] = fminf(lo[1], rt[e]);
+        if (a.val) {
+          const float d = rt[e] - vl[e];  // the fp32 difference the reference forms (:143)
+          s[kDmVal] += vl[e];
+          s[kDmDiff] += d;
+          s[kDmDiff2] += d * d;
+          hi[2] = fmaxf(hi[2], vl[e]); lo[2] = fminf(lo[2], vl[e]);
         }
       }
     }
   }
   if (chunk == 0) {
     const int64_t p0 = row * (a.prompt + a.cols);
-    for (int64_t c = threadIdx.x; c < a.prompt; c += kRcThreads) s[kDmPromptLen] += (double)attention[p0 + c];
+    for (int64_t c = threadIdx.x; c < a.prompt; c += kRcThreads) s[kDmPromptLen] += (float)attention[p0 + c];
   }
-  __shared__ double smem[24 * 4];
-  block_sum<kDmSums, kRcThreads>(s, smem);
-  double ext[6] = {hi[0], -lo[0], hi[1], -lo[1], hi[2], -lo[2]};
+  __shared__ double smem[kDmSums * 4];
+  double acc[kDmSums];
+#pragma unroll
+  for (int i = 0; i < kDmSums; ++i) acc[i] = s[i];
+  block_sum<kDmSums, kRcThreads>(acc, smem);
+  double ext[6] = {hi[0], -(double)lo[0], hi[1], -(double)lo[1], hi[2], -(double)lo[2]};
   block_max<6, kRcThreads>(ext, smem);
   if (threadIdx.x == 0) {
-    double* r = a.records + (int64_t)blockIdx.x * kDmRec;
+    double rec[kDmRec];
 #pragma unroll
-    for (int i = 0; i < kDmSums; ++i) peer_store(r + i, s[i]);
+    for (int i = 0; i < kDmSums; ++i) rec[i] = acc[i];
 #pragma unroll
-    for (int i = 0; i < 6; ++i) peer_store(r + kDmSums + i, (i & 1) ? -ext[i] : ext[i]);
+    for (int i = 0; i < 6; ++i) rec[kDmSums + i] = ext[i];  // maxima, and minima negated
+    store_record<kDmRec>(a.records, row, chunk, a.rows, a.chunks, rec);  // read by the next launch
   }
-  if (!last_block_arrives(a.ticket)) return;
+}
 
+constexpr int kDmFoldThreads = 512;
+
+// One workgroup: records -> per-row quantities -> the output vector.
+__global__ __launch_bounds__(kDmFoldThreads) void data_metrics_fold_kernel(DmArgs a) {
+  const double inf = __longlong_as_double(0x7ff0000000000000ll);
+  __shared__ double smem[16 * (kDmFoldThreads / 64)];
   // ---- fold: thread-strided over rows -------------------------------------------------------------
   // sums: 0 n_non_aborted 1 score 2 reward 3 resp_len 4 resp_len==cols 5 resp_len (non-aborted)
   //       6 resp_len==cols (non-aborted) 7 prompt_len 8 prompt_len==prompt
@@ -139,20 +148,16 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
   double x[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) x[i] = -inf;
-  for (int64_t r = threadIdx.x; r < a.rows; r += kRcThreads) {
-    double row_s[5] = {0, 0, 0, 0, 0};
-    for (int c = 0; c < a.chunks; ++c) {
-      const double* rec = a.records + (r * a.chunks + c) * kDmRec;
+  for (int64_t r = threadIdx.x; r < a.rows; r += kDmFoldThreads) {
+    const int64_t rr[1] = {r};
+    const bool have[1] = {true};
+    double rec[1][kDmRec];
+    fold_row_records<kDmRec, kDmSums, 1, false>(a.records, rr, have, a.rows, a.chunks, rec);
+    const double* row_s = rec[0];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) row_s[i] += peer_load(rec + i);
+    for (int i = 0; i < kElem; ++i) t[9 + i] += rec[0][kDmValid + i];
 #pragma unroll
-      for (int i = 0; i < kElem; ++i) t[9 + i] += peer_load(rec + kDmValid + i);
-#pragma unroll
-      for (int i = 0; i < 6; ++i) {
-        const double v = peer_load(rec + kDmSums + i);
-        x[10 + i] = fmax(x[10 + i], (i & 1) ? -v : v);
-      }
-    }
+    for (int i = 0; i < 6; ++i) x[10 + i] = fmax(x[10 + i], rec[0][kDmSums + i]);
     const double score = (double)(float)row_s[kDmScore], reward = (double)(float)row_s[kDmReward];
     const double rl = row_s[kDmRespLen], pl = row_s[kDmPromptLen];
     t[3] += rl;
@@ -172,8 +177,8 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
       x[6] = fmax(x[6], rl); x[7] = fmax(x[7], -rl);
     }
   }
-  block_sum<9 + kElem, kRcThreads>(t, smem);
-  block_max<16, kRcThreads>(x, smem);
+  block_sum<9 + kElem, kDmFoldThreads>(t, smem);
+  block_max<16, kDmFoldThreads>(x, smem);
   if (threadIdx.x == 0) {
     double* o = a.out;
     const double B = (double)a.rows, na = t[0];
@@ -198,7 +203,6 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
     o[VAMD_DM_VALID_TOKENS] = n;
     o[VAMD_DM_NON_ABORTED] = na;
   }
-  ticket_reset(a.ticket);
 }
 
 }  // namespace vamd
@@ -207,7 +211,7 @@ using namespace vamd;
 
 extern "C" size_t vamd_data_metrics_workspace_bytes(int64_t batch, int64_t response_length) {
   if (batch <= 0 || response_length <= 0) return 0;
-  return kTicketBytes + align_up((size_t)batch * chunks_of(response_length) * kDmRec * sizeof(double), 256);
+  return align_up((size_t)batch * chunks_of(response_length) * kDmRec * sizeof(double), 256);
 }
 
 extern "C" int vamd_data_metrics(const float* token_level_scores, const float* token_level_rewards,
@@ -228,15 +232,15 @@ extern "C" int vamd_data_metrics(const float* token_level_scores, const float* t
   a.scores = token_level_scores; a.rewards = token_level_rewards; a.adv = advantages; a.ret = returns; a.val = values;
   a.rows = batch; a.cols = response_length; a.prompt = prompt_length;
   a.chunks = (int)chunks_of(response_length);
-  a.ticket = static_cast<unsigned*>(workspace);
-  a.records = reinterpret_cast<double*>(static_cast<char*>(workspace) + kTicketBytes);
+  a.records = static_cast<double*>(workspace);
   a.out = out;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)(batch * a.chunks)), block(kRcThreads);
 #define VAMD_DM(A)                                                                                            \
   VAMD_MASK_DISPATCH(mask_dtype, M, {                                                                          \
     const bool vec = can_vectorize(response_length, {token_level_scores, token_level_rewards, advantages,      \
-                                                     returns, values}, response_mask, sizeof(M));              \
+                                                     returns, values}, response_mask, sizeof(M)) &&            \
+                     prompt_length % 4 == 0 && aligned_to(attention_mask, 4 * sizeof(A));                      \
     if (vec)                                                                                                   \
       hipLaunchKernelGGL((data_metrics_kernel<true, M, A>), grid, block, 0, s, a,                              \
                          static_cast<const M*>(response_mask), static_cast<const A*>(attention_mask));         \
@@ -252,6 +256,7 @@ extern "C" int vamd_data_metrics(const float* token_level_scores, const float* t
     default: set_error("unknown mask dtype code %d", attention_dtype); return VAMD_EINVAL;
   }
 #undef VAMD_DM
+  hipLaunchKernelGGL(data_metrics_fold_kernel, dim3(1), dim3(kDmFoldThreads), 0, s, a);
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }

@@ -14,7 +14,7 @@ namespace vamd {
 
 struct Work {
   unsigned* ticket;  // workspace head: zero on entry, zero on exit
-  double* partials;  // [rows * chunks][NV]
+  double* partials;  // NV slots per (row, chunk) workgroup, slot-major (record_at)
 };
 
 // =============================================================================================
@@ -56,25 +56,24 @@ __global__ __launch_bounds__(kRcThreads) void moments_kernel(const float* __rest
   double acc[4] = {s0, s1, s2, cnt};
   block_sum<4, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
-    double* o = wk.partials + (int64_t)blockIdx.x * 4;
-    peer_store(o + 0, acc[0]); peer_store(o + 1, acc[1]); peer_store(o + 2, acc[2]); peer_store(o + 3, acc[3]);
+    store_record<4>(wk.partials, row, chunk, rows, chunks, acc);
   }
   if (!last_block_arrives(wk.ticket)) return;
   if (per_row) {
-    for (int64_t r = threadIdx.x; r < rows; r += kRcThreads) {
-      double a[4] = {0, 0, 0, 0};
-      for (int c = 0; c < chunks; ++c)
+    for (int64_t r0 = threadIdx.x; r0 < rows; r0 += 2 * kRcThreads) {
+      const int64_t rr[2] = {r0, r0 + kRcThreads};
+      const bool have[2] = {true, rr[1] < rows};
+      double a[2][4];
+      fold_row_records<4, 4, 2>(wk.partials, rr, have, rows, chunks, a);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) a[i] += peer_load(wk.partials + (r * chunks + c) * 4 + i);
+      for (int k = 0; k < 2; ++k)
+        if (have[k])
 #pragma unroll
-      for (int i = 0; i < 4; ++i) out[r * 4 + i] = a[i];
+          for (int i = 0; i < 4; ++i) out[rr[k] * 4 + i] = a[k][i];
     }
   } else {
     double a[4] = {0, 0, 0, 0};
-    const int64_t n = rows * chunks;
-    for (int64_t k = threadIdx.x; k < n; k += kRcThreads)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) a[i] += peer_load(wk.partials + k * 4 + i);
+    sum_records_strided<4>(wk.partials, rows * chunks, a);
     block_sum<4, kRcThreads>(a, smem);
     if (threadIdx.x == 0)
 #pragma unroll
@@ -122,9 +121,45 @@ __global__ __launch_bounds__(kRcThreads) void affine_masked_kernel(const float* 
 }
 
 // =============================================================================================
+// Folding the (row, chunk) records of the loss kernels.  Small launches let the workgroup that arrives last
+// do it (one launch in all); large ones leave it to a launch of its own: the fold's registers would otherwise
+// be charged to every wavefront of the streaming kernel and halve its occupancy.
+// =============================================================================================
+constexpr int kFoldThreads = 512;
+constexpr int64_t kInlineFoldRecords = 2048;  // up to this many (row, chunk) records the last workgroup folds
+
+enum { kEpiAgg, kEpiPolicy, kEpiValue, kEpiKl };
+
+template <int EPI, int NX>
+__device__ __forceinline__ void loss_epilogue(double loss, double msum, const double (&extra)[NX], float* __restrict__ out) {
+  const float denom = (float)msum + 1e-8f;  // masked_mean's denominator
+  if (EPI == kEpiPolicy) {
+    out[0] = (float)loss;
+    out[1] = (float)extra[1] / denom;  // pg_clipfrac
+    out[2] = (float)extra[0] / denom;  // ppo_kl
+    out[3] = (float)extra[NX > 2 ? 2 : 0] / denom;  // pg_clipfrac_lower
+  } else if (EPI == kEpiValue) {
+    out[0] = 0.5f * (float)loss;
+    out[1] = (float)extra[0] / denom;
+  } else {
+    out[0] = (float)loss;
+  }
+}
+
+template <int NV, int EPI>
+__global__ __launch_bounds__(kFoldThreads) void fold_loss_kernel(const double* __restrict__ records, int64_t rows,
+                                                                 int chunks, int64_t cols, AggParams ap,
+                                                                 float* __restrict__ coef, float* __restrict__ out) {
+  __shared__ double smem[(NV + 3) * (kFoldThreads / 64)];
+  double loss, msum, extra[NV > 2 ? NV - 2 : 1];
+  finalize_agg<NV, kFoldThreads, false>(records, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
+  if (threadIdx.x == 0) loss_epilogue<EPI>(loss, msum, extra, out);
+}
+
+// =============================================================================================
 // agg_loss forward / backward
 // =============================================================================================
-template <bool VEC, class M>
+template <bool VEC, class M, bool FOLD>
 __global__ __launch_bounds__(kRcThreads) void agg_kernel(const float* __restrict__ loss_mat,
                                                          const M* __restrict__ mask, int64_t rows, int64_t cols,
                                                          int chunks, AggParams ap, Work wk,
@@ -150,14 +185,15 @@ __global__ __launch_bounds__(kRcThreads) void agg_kernel(const float* __restrict
   double acc[2] = {s, m};
   block_sum<2, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
-    peer_store(wk.partials + (int64_t)blockIdx.x * 2, acc[0]);
-    peer_store(wk.partials + (int64_t)blockIdx.x * 2 + 1, acc[1]);
+    store_record<2>(wk.partials, row, chunk, rows, chunks, acc);
   }
-  if (!last_block_arrives(wk.ticket)) return;
-  double loss, msum, extra[1];
-  finalize_agg<2>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
-  if (threadIdx.x == 0) out_loss[0] = (float)loss;
-  ticket_reset(wk.ticket);
+  if constexpr (FOLD) {
+    if (!last_block_arrives(wk.ticket)) return;
+    double loss, msum, extra[1];
+    finalize_agg<2>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
+    if (threadIdx.x == 0) loss_epilogue<kEpiAgg>(loss, msum, extra, out_loss);
+    ticket_reset(wk.ticket);
+  }
 }
 
 // out[i][t] = coef[i] * (float)mask[i][t] * *d_loss
@@ -349,7 +385,7 @@ __global__ __launch_bounds__(kRcThreads) void geo_rows_kernel(const float* __res
   }
 }
 
-template <bool VEC, class M, bool GRAD, bool ISW>
+template <bool VEC, class M, bool GRAD, bool ISW, bool FOLD>
 __global__ __launch_bounds__(kRcThreads) void policy_kernel(
     const float* __restrict__ old_lp, const float* __restrict__ lp, const float* __restrict__ adv,
     const M* __restrict__ mask, const float* __restrict__ isw, int64_t rows, int64_t cols, int chunks,
@@ -403,27 +439,21 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
   double acc[5] = {s_loss, s_m, s_kl, s_cf, s_cfl};
   block_sum<5, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
-    double* p = wk.partials + (int64_t)blockIdx.x * 5;
-#pragma unroll
-    for (int i = 0; i < 5; ++i) peer_store(p + i, acc[i]);
+    store_record<5>(wk.partials, row, chunk, rows, chunks, acc);
   }
-  if (!last_block_arrives(wk.ticket)) return;
-  double loss, msum, extra[3];
-  finalize_agg<5>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
-  if (threadIdx.x == 0) {
-    const float denom = (float)msum + 1e-8f;  // masked_mean's denominator
-    out[0] = (float)loss;
-    out[1] = (float)extra[1] / denom;  // pg_clipfrac
-    out[2] = (float)extra[0] / denom;  // ppo_kl
-    out[3] = (float)extra[2] / denom;  // pg_clipfrac_lower
+  if constexpr (FOLD) {
+    if (!last_block_arrives(wk.ticket)) return;
+    double loss, msum, extra[3];
+    finalize_agg<5>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
+    if (threadIdx.x == 0) loss_epilogue<kEpiPolicy>(loss, msum, extra, out);
+    ticket_reset(wk.ticket);
   }
-  ticket_reset(wk.ticket);
 }
 
 // =============================================================================================
 // value loss (compute_value_loss, core_algos.py:1799-1838)
 // =============================================================================================
-template <bool VEC, class M, bool GRAD>
+template <bool VEC, class M, bool GRAD, bool FOLD>
 __global__ __launch_bounds__(kRcThreads) void value_kernel(
     const float* __restrict__ vpreds, const float* __restrict__ returns, const float* __restrict__ values,
     const M* __restrict__ mask, int64_t rows, int64_t cols, int chunks, float clip, AggParams ap, Work wk,
@@ -468,17 +498,15 @@ __global__ __launch_bounds__(kRcThreads) void value_kernel(
   double acc[3] = {s_loss, s_m, s_cf};
   block_sum<3, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
-    double* p = wk.partials + (int64_t)blockIdx.x * 3;
-    peer_store(p + 0, acc[0]); peer_store(p + 1, acc[1]); peer_store(p + 2, acc[2]);
+    store_record<3>(wk.partials, row, chunk, rows, chunks, acc);
   }
-  if (!last_block_arrives(wk.ticket)) return;
-  double loss, msum, extra[1];
-  finalize_agg<3>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
-  if (threadIdx.x == 0) {
-    out[0] = 0.5f * (float)loss;
-    out[1] = (float)extra[0] / ((float)msum + 1e-8f);
+  if constexpr (FOLD) {
+    if (!last_block_arrives(wk.ticket)) return;
+    double loss, msum, extra[1];
+    finalize_agg<3>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
+    if (threadIdx.x == 0) loss_epilogue<kEpiValue>(loss, msum, extra, out);
+    ticket_reset(wk.ticket);
   }
-  ticket_reset(wk.ticket);
 }
 
 // =============================================================================================
@@ -527,7 +555,7 @@ __global__ __launch_bounds__(256) void kl_elementwise_kernel(const float* __rest
 
 // agg_loss(kl_penalty(logprob, ref), mask, mode) in one pass, with the per-element gradient
 // (times the mask weight, before the per-row agg_loss coefficient) on request.
-template <bool VEC, class M, bool GRAD>
+template <bool VEC, class M, bool GRAD, bool FOLD>
 __global__ __launch_bounds__(kRcThreads) void kl_loss_kernel(
     const float* __restrict__ logprob, const float* __restrict__ ref, const M* __restrict__ mask, int64_t rows,
     int64_t cols, int chunks, int kind, int straight, AggParams ap, Work wk, float* __restrict__ out,
@@ -559,14 +587,15 @@ __global__ __launch_bounds__(kRcThreads) void kl_loss_kernel(
   double acc[2] = {s_loss, s_m};
   block_sum<2, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
-    double* p = wk.partials + (int64_t)blockIdx.x * 2;
-    peer_store(p + 0, acc[0]); peer_store(p + 1, acc[1]);
+    store_record<2>(wk.partials, row, chunk, rows, chunks, acc);
   }
-  if (!last_block_arrives(wk.ticket)) return;
-  double loss, msum, extra[1];
-  finalize_agg<2>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
-  if (threadIdx.x == 0) out[0] = (float)loss;
-  ticket_reset(wk.ticket);
+  if constexpr (FOLD) {
+    if (!last_block_arrives(wk.ticket)) return;
+    double loss, msum, extra[1];
+    finalize_agg<2>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
+    if (threadIdx.x == 0) loss_epilogue<kEpiKl>(loss, msum, extra, out);
+    ticket_reset(wk.ticket);
+  }
 }
 
 // token_level_rewards = scores - beta * kld * mask and current_kl = mean over rows of
@@ -605,18 +634,23 @@ __global__ __launch_bounds__(kRcThreads) void kl_reward_kernel(
   double acc[2] = {s_kl, s_m};
   block_sum<2, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
-    double* p = wk.partials + (int64_t)blockIdx.x * 2;
-    peer_store(p + 0, acc[0]); peer_store(p + 1, acc[1]);
+    store_record<2>(wk.partials, row, chunk, rows, chunks, acc);
   }
   if (!last_block_arrives(wk.ticket)) return;
   double total = 0;
-  for (int64_t r = threadIdx.x; r < rows; r += kRcThreads) {
-    double S = 0, Ms = 0;
-    for (int c = 0; c < chunks; ++c) {
-      S += peer_load(wk.partials + (r * chunks + c) * 2);
-      Ms += peer_load(wk.partials + (r * chunks + c) * 2 + 1);
+  for (int64_t r0 = threadIdx.x; r0 < rows; r0 += 4 * kRcThreads) {
+    int64_t rr[4];
+    bool have[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      rr[k] = r0 + (int64_t)k * kRcThreads;
+      have[k] = rr[k] < rows;
     }
-    total += (double)((float)S / ((float)Ms + 1e-8f));
+    double f[4][2];
+    fold_row_records<2, 2, 4>(wk.partials, rr, have, rows, chunks, f);
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+      if (have[k]) total += (double)((float)f[k][0] / ((float)f[k][1] + 1e-8f));
   }
   double t[1] = {total};
   block_sum<1, kRcThreads>(t, smem);
@@ -670,7 +704,7 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rowsum_kernel(const float* __
   __shared__ double smem[4];
   double acc[1] = {s};
   block_sum<1, kRcThreads>(acc, smem);
-  if (threadIdx.x == 0) peer_store(wk.partials + blockIdx.x, acc[0]);
+  if (threadIdx.x == 0) store_record<1>(wk.partials, row, chunk, ga.rows, chunks, acc);
   if (ga.n_groups > kGrpoLdsGroups) return;  // statistics come from the separate kernels below
   if (!last_block_arrives(wk.ticket)) return;
 
@@ -685,20 +719,32 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rowsum_kernel(const float* __
   __syncthreads();
   const bool opo = ga.estimator == VAMD_ADV_OPO;
   double nnz_local = 0;
-  for (int64_t r = threadIdx.x; r < ga.rows; r += kRcThreads) {
-    double t = 0;
-    for (int c = 0; c < chunks; ++c) t += peer_load(wk.partials + r * chunks + c);
-    const float sc = (float)t;
-    ga.scores[r] = sc;
-    nnz_local += sc != 0.f ? 1.0 : 0.0;
-    const int64_t g = ga.gid[r];
-    atomicAdd(&g_cnt[g], 1);
-    if (opo) {  // g_sum: sum(len * s), g_sq: sum(len)
-      const double len = ga.row_moments[r * 4];
-      atomicAdd(&g_sum[g], len * (double)sc);
-      atomicAdd(&g_sq[g], len);
-    } else {
-      atomicAdd(&g_sum[g], (double)sc);
+  for (int64_t r0 = threadIdx.x; r0 < ga.rows; r0 += 4 * kRcThreads) {
+    int64_t rr[4];
+    bool have[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      rr[k] = r0 + (int64_t)k * kRcThreads;
+      have[k] = rr[k] < ga.rows;
+    }
+    double row_sum[4][1];
+    fold_row_records<1, 1, 4>(wk.partials, rr, have, ga.rows, chunks, row_sum);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (!have[k]) break;
+      const int64_t r = rr[k];
+      const float sc = (float)row_sum[k][0];
+      ga.scores[r] = sc;
+      nnz_local += sc != 0.f ? 1.0 : 0.0;
+      const int64_t g = ga.gid[r];
+      atomicAdd(&g_cnt[g], 1);
+      if (opo) {  // g_sum: sum(len * s), g_sq: sum(len)
+        const double len = ga.row_moments[r * 4];
+        atomicAdd(&g_sum[g], len * (double)sc);
+        atomicAdd(&g_sq[g], len);
+      } else {
+        atomicAdd(&g_sum[g], (double)sc);
+      }
     }
   }
   __syncthreads();
@@ -797,7 +843,7 @@ __global__ void rowsum_finalize_kernel(const double* __restrict__ partials, int6
   const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (r >= rows) return;
   double s = 0;
-  for (int c = 0; c < chunks; ++c) s += partials[r * chunks + c];
+  for (int c = 0; c < chunks; ++c) s += partials[record_at(0, r, c, rows, chunks)];
   scores[r] = (float)s;
 }
 
@@ -991,12 +1037,25 @@ extern "C" int vamd_agg_loss_forward(const float* loss_mat, const void* mask, in
   const int chunks = (int)chunks_of(cols);
   const Work wk = carve_work(workspace);
   const AggParams ap = make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor);
+  bool sep = rows * chunks > kInlineFoldRecords;  // fold the records in a launch of their own
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(cols, {loss_mat}, mask, sizeof(M));
-    VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((agg_kernel<V, M>), dim3((unsigned)(rows * chunks)),
-                                                 dim3(kRcThreads), 0, s, loss_mat, static_cast<const M*>(mask),
-                                                 rows, cols, chunks, ap, wk, out_loss, coef_out));
+    const M* mk = static_cast<const M*>(mask);
+    const dim3 grid((unsigned)(rows * chunks)), block(kRcThreads);
+    if (vec && sep)
+      hipLaunchKernelGGL((agg_kernel<true, M, false>), grid, block, 0, s, loss_mat, mk, rows, cols, chunks, ap, wk,
+                         out_loss, coef_out);
+    else if (vec)
+      hipLaunchKernelGGL((agg_kernel<true, M, true>), grid, block, 0, s, loss_mat, mk, rows, cols, chunks, ap, wk,
+                         out_loss, coef_out);
+    else
+      hipLaunchKernelGGL((agg_kernel<false, M, true>), grid, block, 0, s, loss_mat, mk, rows, cols, chunks, ap, wk,
+                         out_loss, coef_out);
+    sep = sep && vec;
   });
+  if (sep)
+    hipLaunchKernelGGL((fold_loss_kernel<2, kEpiAgg>), dim3(1), dim3(kFoldThreads), 0, s, wk.partials, rows, chunks,
+                       cols, ap, coef_out, out_loss);
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }
@@ -1127,21 +1186,26 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
 #undef VAMD_GEO
     is_weights = nullptr;  // already folded into the sequence loss
   }
-#define VAMD_PL(V, G, W)                                                                                     \
-  hipLaunchKernelGGL((policy_kernel<V, M, G, W>), grid, block, 0, s, old_log_prob, log_prob, advantages, mk, \
+  bool sep = rows * chunks > kInlineFoldRecords;  // fold the records in a launch of their own
+#define VAMD_PL(V, G, W, F)                                                                                     \
+  hipLaunchKernelGGL((policy_kernel<V, M, G, W, F>), grid, block, 0, s, old_log_prob, log_prob, advantages, mk, \
                      is_weights, rows, cols, chunks, pp, ap, wk, out, grad_unscaled, coef_out)
+#define VAMD_PL_GW(V, F)                                                                             \
+  if (grad_unscaled) { if (is_weights) VAMD_PL(V, true, true, F); else VAMD_PL(V, true, false, F); } \
+  else { if (is_weights) VAMD_PL(V, false, true, F); else VAMD_PL(V, false, false, F); }
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(cols, {old_log_prob, log_prob, advantages, is_weights, grad_unscaled}, mask,
                                    sizeof(M));
     const M* mk = static_cast<const M*>(mask);
-    if (vec) {
-      if (grad_unscaled) { if (is_weights) VAMD_PL(true, true, true); else VAMD_PL(true, true, false); }
-      else { if (is_weights) VAMD_PL(true, false, true); else VAMD_PL(true, false, false); }
-    } else {
-      if (grad_unscaled) { if (is_weights) VAMD_PL(false, true, true); else VAMD_PL(false, true, false); }
-      else { if (is_weights) VAMD_PL(false, false, true); else VAMD_PL(false, false, false); }
-    }
+    sep = sep && vec;
+    if (sep) { VAMD_PL_GW(true, false) }
+    else if (vec) { VAMD_PL_GW(true, true) }
+    else { VAMD_PL_GW(false, true) }
   });
+  if (sep)
+    hipLaunchKernelGGL((fold_loss_kernel<5, kEpiPolicy>), dim3(1), dim3(kFoldThreads), 0, s, wk.partials, rows,
+                       chunks, cols, ap, coef_out, out);
+#undef VAMD_PL_GW
 #undef VAMD_PL
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
@@ -1170,15 +1234,21 @@ extern "C" int vamd_value_loss_forward(const float* vpreds, const float* returns
   const Work wk = carve_work(workspace);
   const AggParams ap = make_agg(mode, 1.0, -1.0, -1.0, -1.0);
   const dim3 grid((unsigned)(rows * chunks)), block(kRcThreads);
-#define VAMD_VL(V, G)                                                                                     \
-  hipLaunchKernelGGL((value_kernel<V, M, G>), grid, block, 0, s, vpreds, returns, values, mk, rows, cols, \
+  bool sep = rows * chunks > kInlineFoldRecords;
+#define VAMD_VL(V, G, F)                                                                                     \
+  hipLaunchKernelGGL((value_kernel<V, M, G, F>), grid, block, 0, s, vpreds, returns, values, mk, rows, cols, \
                      chunks, cliprange_value, ap, wk, out, grad_unscaled, coef_out)
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(cols, {vpreds, returns, values, grad_unscaled}, mask, sizeof(M));
     const M* mk = static_cast<const M*>(mask);
-    if (vec) { if (grad_unscaled) VAMD_VL(true, true); else VAMD_VL(true, false); }
-    else { if (grad_unscaled) VAMD_VL(false, true); else VAMD_VL(false, false); }
+    sep = sep && vec;
+    if (sep) { if (grad_unscaled) VAMD_VL(true, true, false); else VAMD_VL(true, false, false); }
+    else if (vec) { if (grad_unscaled) VAMD_VL(true, true, true); else VAMD_VL(true, false, true); }
+    else { if (grad_unscaled) VAMD_VL(false, true, true); else VAMD_VL(false, false, true); }
   });
+  if (sep)
+    hipLaunchKernelGGL((fold_loss_kernel<3, kEpiValue>), dim3(1), dim3(kFoldThreads), 0, s, wk.partials, rows, chunks,
+                       cols, ap, coef_out, out);
 #undef VAMD_VL
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
@@ -1221,15 +1291,21 @@ extern "C" int vamd_kl_loss_forward(const float* logprob, const float* ref_logpr
   const Work wk = carve_work(workspace);
   const AggParams ap = make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor);
   const dim3 grid((unsigned)(rows * chunks)), block(kRcThreads);
-#define VAMD_KL(V, G)                                                                                       \
-  hipLaunchKernelGGL((kl_loss_kernel<V, M, G>), grid, block, 0, s, logprob, ref_logprob, mk, rows, cols, chunks, \
+  bool sep = rows * chunks > kInlineFoldRecords;
+#define VAMD_KL(V, G, F)                                                                                       \
+  hipLaunchKernelGGL((kl_loss_kernel<V, M, G, F>), grid, block, 0, s, logprob, ref_logprob, mk, rows, cols, chunks, \
                      kind, straight_through, ap, wk, out, grad_unscaled, coef_out)
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(cols, {logprob, ref_logprob, grad_unscaled}, mask, sizeof(M));
     const M* mk = static_cast<const M*>(mask);
-    if (vec) { if (grad_unscaled) VAMD_KL(true, true); else VAMD_KL(true, false); }
-    else { if (grad_unscaled) VAMD_KL(false, true); else VAMD_KL(false, false); }
+    sep = sep && vec;
+    if (sep) { if (grad_unscaled) VAMD_KL(true, true, false); else VAMD_KL(true, false, false); }
+    else if (vec) { if (grad_unscaled) VAMD_KL(true, true, true); else VAMD_KL(true, false, true); }
+    else { if (grad_unscaled) VAMD_KL(false, true, true); else VAMD_KL(false, false, true); }
   });
+  if (sep)
+    hipLaunchKernelGGL((fold_loss_kernel<2, kEpiKl>), dim3(1), dim3(kFoldThreads), 0, s, wk.partials, rows, chunks,
+                       cols, ap, coef_out, out);
 #undef VAMD_KL
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;

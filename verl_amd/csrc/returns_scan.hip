@@ -33,7 +33,7 @@ constexpr int kRsBatch = 4;
 
 struct ReturnsWork {
   unsigned* ticket;  // workspace head: zero on entry, zero on exit
-  double* partials;  // [rows][3] sum(m), sum(R m), sum(R^2 m) with R zeroed outside the mask
+  double* partials;  // per row sum(m), sum(R m), sum(R^2 m) with R zeroed outside the mask; slot-major
 };
 
 template <bool VEC, class M, int MODE>
@@ -129,14 +129,11 @@ __global__ __launch_bounds__(kRcThreads) void returns_scan_kernel(const float* _
   double acc[3] = {m0, m1, m2};
   block_sum<3, kRcThreads>(acc, smem);
   if (tid == 0) {
-    double* o = wk.partials + row * 3;
-    peer_store(o + 0, acc[0]); peer_store(o + 1, acc[1]); peer_store(o + 2, acc[2]);
+    store_record<3>(wk.partials, row, 0, rows, 1, acc);
   }
   if (!last_block_arrives(wk.ticket)) return;
   double a[3] = {0, 0, 0};
-  for (int64_t k = tid; k < rows; k += kRcThreads)
-#pragma unroll
-    for (int i = 0; i < 3; ++i) a[i] += peer_load(wk.partials + k * 3 + i);
+  sum_records_strided<3>(wk.partials, rows, a);
   block_sum<3, kRcThreads>(a, smem);
   if (tid == 0) {
 #pragma unroll

@@ -4,10 +4,11 @@
 // (verl/trainer/ppo/rollout_corr_helper.py:481-712, 835-937) evaluate about thirty masked reductions
 // over old_log_prob, rollout_log_prob and the response mask, each followed by .item().  Here every
 // (row, 4096-column chunk) workgroup reads the three tensors once, writes the truncated token-level
-// weights if those are asked for, and leaves a record of partial sums; the workgroup that arrives
-// last folds the records into per-sequence quantities and then into the metric vector.  Sequence-
-// level weights (one per row, known only after the fold) are broadcast by a second small launch, and
-// batch normalisation of token-level weights is a third.  The response mask is taken as binary.
+// weights if those are asked for, and leaves a record of partial sums; a single-workgroup launch then
+// folds the records into per-sequence quantities and the metric vector (a launch of its own, so that
+// the fold's registers are not charged to every wavefront of the streaming kernel).  Sequence-level
+// weights (one per row, known only after the fold) are broadcast by a further small launch, as is the
+// batch normalisation of token-level weights.  The response mask is taken as binary.
 #include "rowchunk.h"
 
 namespace vamd {
@@ -41,8 +42,7 @@ struct RcArgs {
   float thr, lower;
   int normalize;
   float* weights;      // [rows][cols] or null
-  unsigned* ticket;
-  double* records;     // [rows * chunks][kRcRec]
+  double* records;     // kRcRec slots per (row, chunk) workgroup, slot-major
   float* row_weight;   // [rows]: sequence-level weight, truncated (and normalised)
   float* factor;       // [1]: batch-normalisation divisor for the token-level weights (1 when not applied)
   double* out;         // [VAMD_RC_COUNT]
@@ -80,7 +80,6 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
   const int64_t row = blockIdx.x / a.chunks;
   const int chunk = blockIdx.x % a.chunks;
   const ChunkPos pos(row, chunk, a.cols);
-  const double inf = __longlong_as_double(0x7ff0000000000000ll);
   float s[kRcSums];
 #pragma unroll
   for (int i = 0; i < kRcSums; ++i) s[i] = 0.f;
@@ -129,15 +128,21 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
   double ext[2] = {wmax, -(double)wmin};
   block_max_f64<2, kRcThreads>(ext, smem);
   if (threadIdx.x == 0) {
-    double* rec = a.records + (int64_t)blockIdx.x * kRcRec;
+    double rec[kRcRec];
 #pragma unroll
-    for (int i = 0; i < kRcSums; ++i) peer_store(rec + i, acc[i]);
-    peer_store(rec + kRcWMax, ext[0]);
-    peer_store(rec + kRcWMinNeg, ext[1]);
+    for (int i = 0; i < kRcSums; ++i) rec[i] = acc[i];
+    rec[kRcWMax] = ext[0];
+    rec[kRcWMinNeg] = ext[1];
+    store_record<kRcRec>(a.records, row, chunk, a.rows, a.chunks, rec);
   }
-  if (!last_block_arrives(a.ticket)) return;
+}
 
-  // ---- fold over rows -------------------------------------------------------------------------------
+constexpr int kRcFoldThreads = 512;
+
+// One workgroup: records -> per-sequence quantities -> the metric vector (and the per-row weights).
+__global__ __launch_bounds__(kRcFoldThreads) void rollout_fold_kernel(RcArgs a) {
+  const double inf = __longlong_as_double(0x7ff0000000000000ll);
+  __shared__ double smem[26 * (kRcFoldThreads / 64)];
   enum {
     tM = 0, tD, tK3, tRho2, tW, tC, tC2, tTrunc, tHigh, tLow,         // token totals
     tTrainPpl, tTrainLog, tRollPpl, tRollLog, tGap, tGapAbs, tRatio, tChiSeq,  // sums over rows
@@ -154,17 +159,14 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
   for (int i = 0; i < xN; ++i) x[i] = -inf;
   const float log_hi = logf(a.thr), log_lo = logf(a.lower);
   const bool seq_level = a.level == VAMD_IS_SEQUENCE;
-  for (int64_t r = threadIdx.x; r < a.rows; r += kRcThreads) {
-    double f[kRcSums];
-#pragma unroll
-    for (int i = 0; i < kRcSums; ++i) f[i] = 0;
-    for (int c = 0; c < a.chunks; ++c) {
-      const double* rec = a.records + (r * a.chunks + c) * kRcRec;
-#pragma unroll
-      for (int i = 0; i < kRcSums; ++i) f[i] += peer_load(rec + i);
-      x[xW] = fmax(x[xW], peer_load(rec + kRcWMax));
-      x[xWMinNeg] = fmax(x[xWMinNeg], peer_load(rec + kRcWMinNeg));
-    }
+  for (int64_t r = threadIdx.x; r < a.rows; r += kRcFoldThreads) {
+    const int64_t rr[1] = {r};
+    const bool have[1] = {true};
+    double rec[1][kRcRec];
+    fold_row_records<kRcRec, kRcSums, 1, false>(a.records, rr, have, a.rows, a.chunks, rec);
+    const double* f = rec[0];
+    x[xW] = fmax(x[xW], rec[0][kRcWMax]);
+    x[xWMinNeg] = fmax(x[xWMinNeg], rec[0][kRcWMinNeg]);
     const float Mi = (float)f[kRcM];
     const float train = (float)f[kRcOld] / (Mi + 1e-8f);  // masked_mean(., axis=-1)
     t[tM] += f[kRcM]; t[tD] += f[kRcD]; t[tK3] += f[kRcK3]; t[tRho2] += f[kRcRho2];
@@ -212,8 +214,9 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
       x[xDev] = fmax(x[xDev], (double)fabsf(seq - 1.f));
     }
   }
-  block_sum<tN, kRcThreads>(t, smem);
-  block_max_f64<xN, kRcThreads>(x, smem);
+  static_assert(tN <= 26, "smem is sized for 26 sums");
+  block_sum<tN, kRcFoldThreads>(t, smem);
+  block_max_f64<xN, kRcFoldThreads>(x, smem);
   __shared__ float norm;
   if (threadIdx.x == 0) {
     double* o = a.out;
@@ -271,8 +274,7 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
   }
   __syncthreads();
   if (seq_level && norm != 1.f)
-    for (int64_t r = threadIdx.x; r < a.rows; r += kRcThreads) a.row_weight[r] = a.row_weight[r] / norm;
-  ticket_reset(a.ticket);
+    for (int64_t r = threadIdx.x; r < a.rows; r += kRcFoldThreads) a.row_weight[r] = a.row_weight[r] / norm;
 }
 
 // weights[i][t] = row_weight[i] * mask[i][t]
@@ -309,7 +311,7 @@ using namespace vamd;
 
 extern "C" size_t vamd_rollout_correction_workspace_bytes(int64_t batch, int64_t length) {
   if (batch <= 0 || length <= 0) return 0;
-  return kTicketBytes + align_up((size_t)batch * chunks_of(length) * kRcRec * sizeof(double), 256) +
+  return align_up((size_t)batch * chunks_of(length) * kRcRec * sizeof(double), 256) +
          align_up((size_t)batch * sizeof(float), 256) + 256;
 }
 
@@ -334,8 +336,7 @@ extern "C" int vamd_rollout_correction(const float* old_log_prob, const float* r
   a.level = level; a.thr = threshold; a.lower = level == VAMD_IS_NONE ? 0.f : 1.0f / threshold;
   a.normalize = batch_normalize;
   a.weights = weights;
-  a.ticket = static_cast<unsigned*>(workspace);
-  Carver carve(static_cast<char*>(workspace) + kTicketBytes);
+  Carver carve(workspace);
   a.records = carve.take<double>((size_t)batch * a.chunks * kRcRec);
   a.row_weight = carve.take<float>((size_t)batch);
   a.factor = carve.take<float>(1);
@@ -345,14 +346,16 @@ extern "C" int vamd_rollout_correction(const float* old_log_prob, const float* r
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const M* mk = static_cast<const M*>(mask);
     const bool vec = can_vectorize(length, {old_log_prob, rollout_log_prob, weights}, mask, sizeof(M));
-    if (vec) {
+    if (vec)
       hipLaunchKernelGGL((rollout_stats_kernel<true, M>), grid, block, 0, s, a, mk);
-      if (level == VAMD_IS_SEQUENCE)
+    else
+      hipLaunchKernelGGL((rollout_stats_kernel<false, M>), grid, block, 0, s, a, mk);
+    hipLaunchKernelGGL(rollout_fold_kernel, dim3(1), dim3(kRcFoldThreads), 0, s, a);
+    if (level == VAMD_IS_SEQUENCE) {
+      if (vec)
         hipLaunchKernelGGL((rollout_broadcast_kernel<true, M>), grid, block, 0, s, a.row_weight, mk, length, a.chunks,
                            weights);
-    } else {
-      hipLaunchKernelGGL((rollout_stats_kernel<false, M>), grid, block, 0, s, a, mk);
-      if (level == VAMD_IS_SEQUENCE)
+      else
         hipLaunchKernelGGL((rollout_broadcast_kernel<false, M>), grid, block, 0, s, a.row_weight, mk, length,
                            a.chunks, weights);
     }

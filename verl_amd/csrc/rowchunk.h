@@ -169,6 +169,83 @@ __device__ __forceinline__ void ticket_reset(unsigned* counters) {
     __hip_atomic_store(counters + threadIdx.x * (kTicketStride / 4), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Records of the (row, chunk) workgroups are kept slot-major: slot i of workgroup (row, chunk) lives at
+// ((i * chunks + chunk) * rows + row).  The workgroup that folds them gives consecutive rows to consecutive threads,
+// so a wavefront's loads of one slot are 512 contiguous bytes; with one record per workgroup stored contiguously
+// they would be 64 separate cache lines, and the single CU doing the fold is bound by its request rate.
+__device__ __forceinline__ int64_t record_at(int slot, int64_t row, int chunk, int64_t rows, int chunks) {
+  return ((int64_t)slot * chunks + chunk) * rows + row;
+}
+
+// Thread 0 of workgroup (row, chunk) publishes its record.
+template <int NV>
+__device__ __forceinline__ void store_record(double* __restrict__ records, int64_t row, int chunk, int64_t rows,
+                                             int chunks, const double (&v)[NV]) {
+#pragma unroll
+  for (int i = 0; i < NV; ++i) peer_store(records + record_at(i, row, chunk, rows, chunks), v[i]);
+}
+
+// A record slot as the folding workgroup reads it: through the device-coherent path when the writers belong to
+// the same launch (COHERENT), as an ordinary load when the records come from an earlier launch.
+template <bool COHERENT>
+__device__ __forceinline__ double record_load(const double* p) {
+  if constexpr (COHERENT) return peer_load(p);
+  else return *p;
+}
+
+// Fold the chunk records of ROWS rows, slot by slot: slots [0, NSUM) add up, slots [NSUM, NV) take the maximum
+// (records hold minima negated).  Every record load is a round trip to the memory side, and the workgroup
+// doing the fold is the only one left running, so the loads of up to four chunks of every row of the trip are
+// issued together; the order of the additions (chunk 0 first) does not depend on that.
+template <int NV, int NSUM, int ROWS, bool COHERENT = true>
+__device__ __forceinline__ void fold_row_records(const double* __restrict__ records, const int64_t (&row)[ROWS],
+                                                 const bool (&have)[ROWS], int64_t rows, int chunks,
+                                                 double (&out)[ROWS][NV]) {
+  const double ninf = -__longlong_as_double(0x7ff0000000000000ll);
+#pragma unroll
+  for (int k = 0; k < ROWS; ++k)
+#pragma unroll
+    for (int i = 0; i < NV; ++i) out[k][i] = i < NSUM ? 0.0 : ninf;
+  for (int c0 = 0; c0 < chunks; c0 += 4) {
+    double t[ROWS][4][NV];
+#pragma unroll
+    for (int k = 0; k < ROWS; ++k)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const bool ok = have[k] && c0 + u < chunks;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+          t[k][u][i] = ok ? record_load<COHERENT>(records + record_at(i, row[k], c0 + u, rows, chunks))
+                          : (i < NSUM ? 0.0 : ninf);
+      }
+#pragma unroll
+    for (int k = 0; k < ROWS; ++k)
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int i = 0; i < NV; ++i) out[k][i] = i < NSUM ? out[k][i] + t[k][u][i] : fmax(out[k][i], t[k][u][i]);
+  }
+}
+
+// acc[i] += slot i of records tid, tid + 256, ... below n (n = rows * chunks records, slot-major), in that order,
+// four records in flight at a time.
+template <int NV>
+__device__ __forceinline__ void sum_records_strided(const double* __restrict__ records, int64_t n, double (&acc)[NV]) {
+  for (int64_t k0 = threadIdx.x; k0 < n; k0 += 4 * kRcThreads) {
+    double t[4][NV];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t k = k0 + (int64_t)u * kRcThreads;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) t[u][i] = k < n ? peer_load(records + (int64_t)i * n + k) : 0.0;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < NV; ++i) acc[i] += t[u][i];
+  }
+}
+
 // (mean, rsqrt(var_unbiased + 1e-8), shift) from the masked moments sum(m), sum(v m), sum(v^2 m),
 // following masked_mean / masked_var / masked_whiten (verl/utils/torch_functional.py:287-339).
 __device__ __forceinline__ void whiten_stats_from_moments(double s0, double s1, double s2, int shift_mean,
@@ -200,10 +277,10 @@ struct AggParams {
   double dp_size, batch_num_tokens, global_batch_size, loss_scale_factor;  // < 0 : None
 };
 
-// Called by ONE workgroup of 256 threads (the last one to arrive).  partials: [rows][chunks][NV] doubles with slot 0 =
+// Called by ONE workgroup of NT threads (the last one of the launch to arrive, or a launch of its own).  partials: slot-major records (record_at) with slot 0 =
 // sum(loss * w) and slot 1 = sum(w); slots >= 2 are summed over everything into extra[].
 // Writes loss (double, thread 0) and coef[rows].
-template <int NV>
+template <int NV, int NT = kRcThreads, bool COHERENT = true>
 __device__ void finalize_agg(const double* __restrict__ partials, int64_t rows, int chunks, int64_t cols,
                              const AggParams& ap, float* __restrict__ coef, double& loss_out, double& msum_out,
                              double (&extra)[NV > 2 ? NV - 2 : 1], double* smem) {
@@ -213,29 +290,15 @@ __device__ void finalize_agg(const double* __restrict__ partials, int64_t rows, 
   for (int i = 0; i <= NV; ++i) tot[i] = 0;
   double seq_mean_sum = 0;  // sum over kept rows of S_i / (M_i + 1e-8)
   double seq_sum = 0;       // sum over kept rows of S_i
-  // two rows per trip so that their record loads (a round trip to the memory side each) overlap
-  for (int64_t r0 = threadIdx.x; r0 < rows; r0 += 2 * kRcThreads) {
-    const int64_t r1 = r0 + kRcThreads;
-    const bool has1 = r1 < rows;
+  // two rows per trip, all their chunk records in flight together
+  for (int64_t r0 = threadIdx.x; r0 < rows; r0 += 2 * NT) {
+    const int64_t rr[2] = {r0, r0 + NT};
+    const bool have[2] = {true, rr[1] < rows};
     double row[2][NV];
-#pragma unroll
-    for (int i = 0; i < NV; ++i) row[0][i] = row[1][i] = 0;
-    for (int c = 0; c < chunks; ++c) {
-      double t[2][NV];
-#pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        t[0][i] = peer_load(partials + (r0 * chunks + c) * NV + i);
-        t[1][i] = has1 ? peer_load(partials + (r1 * chunks + c) * NV + i) : 0.0;
-      }
-#pragma unroll
-      for (int i = 0; i < NV; ++i) {
-        row[0][i] += t[0][i];
-        row[1][i] += t[1][i];
-      }
-    }
+    fold_row_records<NV, NV, 2, COHERENT>(partials, rr, have, rows, chunks, row);
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
-      if (k == 1 && !has1) break;
+      if (!have[k]) break;
 #pragma unroll
       for (int i = 0; i < NV; ++i) tot[i] += row[k][i];
       if (row[k][1] > 0) {
@@ -250,7 +313,7 @@ __device__ void finalize_agg(const double* __restrict__ partials, int64_t rows, 
   for (int i = 0; i <= NV; ++i) red[i] = tot[i];
   red[NV + 1] = seq_mean_sum;
   red[NV + 2] = seq_sum;
-  block_sum<NV + 3, kRcThreads>(red, smem);
+  block_sum<NV + 3, NT>(red, smem);
   __shared__ double bc[NV + 3];
   if (threadIdx.x == 0)
 #pragma unroll
@@ -278,15 +341,36 @@ __device__ void finalize_agg(const double* __restrict__ partials, int64_t rows, 
     } break;
   }
   if (coef) {
-    for (int64_t r = threadIdx.x; r < rows; r += kRcThreads) {
-      double c = c_all;
-      if (ap.mode == VAMD_AGG_SEQ_MEAN_TOKEN_SUM || ap.mode == VAMD_AGG_SEQ_MEAN_TOKEN_MEAN) {
-        double m = 0;
-        for (int k = 0; k < chunks; ++k) m += peer_load(partials + (r * chunks + k) * NV + 1);
-        c = 0;
-        if (m > 0) c = (ap.mode == VAMD_AGG_SEQ_MEAN_TOKEN_SUM ? 1.0 : 1.0 / (m + 1e-8)) * ap.dp_size / gbs;
+    const bool per_row = ap.mode == VAMD_AGG_SEQ_MEAN_TOKEN_SUM || ap.mode == VAMD_AGG_SEQ_MEAN_TOKEN_MEAN;
+    for (int64_t r0 = threadIdx.x; r0 < rows; r0 += 4 * NT) {
+      double m[4] = {0, 0, 0, 0};
+      if (per_row)  // the rows' mask sums again, all loads of the trip in flight together
+        for (int c0 = 0; c0 < chunks; c0 += 4) {
+          double t[4][4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              const int64_t r = r0 + (int64_t)k * NT;
+              t[k][u] = (r < rows && c0 + u < chunks)
+                            ? record_load<COHERENT>(partials + record_at(1, r, c0 + u, rows, chunks)) : 0.0;
+            }
+#pragma unroll
+          for (int k = 0; k < 4; ++k)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) m[k] += t[k][u];
+        }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int64_t r = r0 + (int64_t)k * NT;
+        if (r >= rows) break;
+        double c = c_all;
+        if (per_row) {
+          c = 0;
+          if (m[k] > 0) c = (ap.mode == VAMD_AGG_SEQ_MEAN_TOKEN_SUM ? 1.0 : 1.0 / (m[k] + 1e-8)) * ap.dp_size / gbs;
+        }
+        coef[r] = (float)c;
       }
-      coef[r] = (float)c;
     }
   }
   loss_out = loss;

@@ -59,7 +59,7 @@ def compute_data_metrics(batch, use_critic: bool = True) -> dict[str, Any]:
     prompt = attention.shape[1] - width
     out = torch.empty(len(_SLOTS), dtype=torch.float64, device=dev)
     Lb = _cabi.lib()
-    ws = _cabi.ticket_workspace(Lb.vamd_data_metrics_workspace_bytes(rows, width), dev)
+    ws = _cabi.workspace(Lb.vamd_data_metrics_workspace_bytes(rows, width), dev)
     with torch.cuda.device(dev):
         _cabi.check(Lb.vamd_data_metrics(tensors[0].data_ptr(), tensors[1].data_ptr(), tensors[2].data_ptr(),
                                          tensors[3].data_ptr(), _cabi.ptr(values), mask.data_ptr(), mcode,

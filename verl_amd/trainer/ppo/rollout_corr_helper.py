@@ -46,7 +46,7 @@ def _run(old_log_prob, rollout_log_prob, response_mask, level, threshold, batch_
         weights = torch.empty_like(old) if level else None
         out = torch.empty(len(_SLOTS), dtype=torch.float64, device=dev)
         Lb = _cabi.lib()
-        ws = _cabi.ticket_workspace(Lb.vamd_rollout_correction_workspace_bytes(rows, cols), dev)
+        ws = _cabi.workspace(Lb.vamd_rollout_correction_workspace_bytes(rows, cols), dev)
         with torch.cuda.device(dev):
             _cabi.check(Lb.vamd_rollout_correction(old.data_ptr(), _cabi.ptr(roll), mask.data_ptr(), code, rows, cols,
                                                    level, float(threshold or 0.0), int(bool(batch_normalize)),
