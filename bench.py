@@ -61,7 +61,7 @@ def cpu_baseline(n_cpu: int, h: int, v: int, temperature: float) -> dict:
 
 
 def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> dict:
-    """The [B, L] kernels (B = 512, L = 4096 are BASELINE configs 3 and 4): microseconds per call from HIP events
+    """The [B, L] kernels (B = 512, L = 4096 is the size of the GRPO / policy-loss and GAE benchmark configurations): microseconds per call from HIP events
     over 40 calls (best of three such loops) that rotate through 8 buffer sets (more than the 256 MB Infinity Cache), the algorithmic bytes of
     the op, and the fraction of 8 TB/s that gives.  ``cpu_ms`` is the CPU oracle on one buffer set."""
     import torch
@@ -212,7 +212,7 @@ def main() -> None:
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (every box here has one GPU; "
-              "the path shards by tokens, see DESIGN.md)", file=sys.stderr)
+              "across GPUs the path shards by tokens and needs no collective in its forward pass)", file=sys.stderr)
         sys.exit(2)
 
     import torch

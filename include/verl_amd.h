@@ -311,6 +311,27 @@ int vamd_rollout_correction(const float* old_log_prob, const float* rollout_log_
                             int batch_normalize, float* weights, double* metrics, void* workspace,
                             size_t workspace_bytes, void* stream);
 
+/* Rejection sampling of the rollout correction (compute_rollout_rejection_mask,
+ * rollout_corr_helper.py:163-357) as two streaming passes around a host step.  Records are doubles laid out
+ * [slot][chunk][row] with chunk count vamd_rollout_rs_chunks(length).
+ *   vamd_rollout_rs_row_stats: 6 slots per (row, chunk): number of valid tokens, sum of k1 = -r, of
+ *     k2 = r^2 / 2 and of k3 = exp(r) - 1 - r over them (r = old - rollout clamped to +-20), max k2, max k3
+ *     (-inf without a valid token).  The host folds the chunks, evaluates the sequence-level options and builds
+ *     row_keep [batch] (uint8).
+ *   vamd_rollout_rs_apply: new_mask = mask where row_keep and every token-level option keep the token, else 0,
+ *     in the mask's element type.  Token option j: estimators[j] in {0: k1, 1: k2, 2: k3}; k1 keeps
+ *     lower[j] <= k1 <= upper[j] (the logs of the ratio bounds), the others keep k <= upper[j].  The three
+ *     tables are host arrays of n_token_options (<= 3) entries.  Records: slot 0 = valid tokens the new mask
+ *     drops; then 8 slots per token option: sum, max, -min, count above upper, count below lower (k1 only), sum
+ *     and sum of squares of the value clamped to [lower or 0, upper], count rejected by this option. */
+int64_t vamd_rollout_rs_chunks(int64_t length);
+int vamd_rollout_rs_row_stats(const float* old_log_prob, const float* rollout_log_prob, const void* mask,
+                              int mask_dtype, int64_t batch, int64_t length, double* records, void* stream);
+int vamd_rollout_rs_apply(const float* old_log_prob, const float* rollout_log_prob, const void* mask, int mask_dtype,
+                          int64_t batch, int64_t length, const uint8_t* row_keep, int n_token_options,
+                          const int* estimators, const float* lower, const float* upper, void* new_mask,
+                          double* records, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * agg_loss (core_algos.py:1025-1080), forward and backward.
  * out_loss: 1 device float.  coef_out [rows] floats: d loss / d loss_mat[i][t] = coef_out[i] *

@@ -79,4 +79,7 @@ from .rollout_corr import (  # noqa: F401
     is_metrics,
     rollout_correction_weights,
     rollout_correction_brute_force_fp64,
+    rollout_rejection_mask,
+    parse_rs_thresholds,
+    RS_OPTIONS,
 )

@@ -159,3 +159,154 @@ def rollout_correction_brute_force_fp64(old, roll, mask, level, threshold):
                "rollout_is_eff_sample_size": tot["c"] ** 2 / (n * tot["c2"]),
                "rollout_is_std": math.sqrt(max(tot["c2"] / n - (tot["c"] / n) ** 2, 0.0))}
     return w, metrics
+
+
+# ---- rejection sampling (hard trust region) -----------------------------------------------------------------
+RS_OPTIONS = ("token_k1", "token_k2", "token_k3", "seq_sum_k1", "seq_sum_k2", "seq_sum_k3", "seq_mean_k1",
+              "seq_mean_k2", "seq_mean_k3", "seq_max_k2", "seq_max_k3")  # rollout_corr_helper.py:77-89
+
+
+def parse_rs_thresholds(options, spec):
+    """_parse_rollout_rs_thresholds, rollout_corr_helper.py:94-160: one threshold for all options or one per option;
+    a k1 option takes ``lower_upper`` (or ``upper`` alone, lower = 1 / upper), the others a single upper bound.
+    Returns ``{option: (lower or None, upper)}``."""
+    if spec is None:
+        raise ValueError("rollout_rs_threshold must be provided for rejection sampling.")
+    if isinstance(spec, (int, float)):
+        parts = [str(spec)]
+    elif isinstance(spec, str):
+        parts = [p.strip() for p in spec.split(",") if p.strip()]
+    else:
+        raise TypeError("rollout_rs_threshold must be a string or numeric value specifying per-option thresholds.")
+    if not parts:
+        raise ValueError("rollout_rs_threshold must contain at least one threshold value.")
+    if len(parts) not in (1, len(options)):
+        raise ValueError("rollout_rs_threshold expects either one threshold shared by all options or exactly "
+                         f"{len(options)} thresholds to match the provided rollout_rs options.")
+    if len(parts) == 1:
+        parts = parts * len(options)
+    out = {}
+    for option, part in zip(options, parts):
+        try:
+            if option.endswith("k1"):
+                lo, hi = part.split("_", 1) if "_" in part else (str(1.0 / float(part)), part)
+                lo, hi = float(lo), float(hi)
+            else:
+                if "_" in part:
+                    raise ValueError(f"rollout_rs_threshold for option '{option}' must provide a single upper bound "
+                                     f"without '_'. Received '{part}'.")
+                lo, hi = None, float(part)
+        except ValueError as exc:
+            if "single upper bound" in str(exc):
+                raise
+            raise ValueError(f"Invalid numeric threshold '{part}' for option '{option}'.") from exc
+        if hi <= 0 or (lo is not None and lo <= 0):
+            raise ValueError(f"Thresholds for option '{option}' must be positive, got {part}.")
+        out[option] = (lo, hi)
+    return out
+
+
+@torch.no_grad()
+def rs_metrics(option, stat, response_mask, seq_valid, level, per_sequence, upper, lower, apply_lower):
+    """compute_rs_metrics, rollout_corr_helper.py:360-478."""
+    if not response_mask.any():
+        raise ValueError("response_mask must contain at least one valid token (1).")
+    p = f"rollout_rs_{option}"
+    out = {}
+    valid = response_mask.bool()
+    seq = per_sequence if per_sequence is not None else masked_mean(stat, response_mask, axis=-1)
+    seq = seq[seq_valid]
+    by_sequence = level == "sequence" and seq.numel() > 0
+    out[f"{p}_mean"] = masked_mean(stat, response_mask).item()
+    if by_sequence:
+        out[f"{p}_max"], out[f"{p}_min"] = seq.max().item(), seq.min().item()
+        out[f"{p}_fraction_high"] = (seq > upper).float().mean().item()
+        out[f"{p}_fraction_low"] = (seq < lower).float().mean().item() if apply_lower else 0.0
+    else:
+        out[f"{p}_max"] = stat.masked_fill(~valid, float("-inf")).max().item()
+        out[f"{p}_min"] = stat.masked_fill(~valid, float("inf")).min().item()
+        out[f"{p}_fraction_high"] = masked_mean((stat > upper).float(), response_mask).item()
+        out[f"{p}_fraction_low"] = masked_mean((stat < lower).float(), response_mask).item() if apply_lower else 0.0
+    if response_mask.sum() > 1:
+        c = stat.clamp(min=lower if apply_lower else 0.0, max=upper)
+        var = masked_mean(c.square(), response_mask) - masked_mean(c, response_mask).square()
+        out[f"{p}_std"] = torch.sqrt(var.clamp(min=0.0)).item()
+    else:
+        out[f"{p}_std"] = 0.0
+    if seq.numel() > 0:
+        out[f"{p}_seq_mean"] = seq.mean().item()
+        out[f"{p}_seq_std"] = seq.std().item() if seq.numel() > 1 else 0.0
+        out[f"{p}_seq_max"] = seq.max().item()
+        out[f"{p}_seq_min"] = seq.min().item()
+        out[f"{p}_seq_max_deviation"] = seq.abs().max().item()
+        out[f"{p}_seq_fraction_high"] = (seq > upper).float().mean().item()
+        if apply_lower:
+            out[f"{p}_seq_fraction_low"] = (seq < lower).float().mean().item()
+    else:
+        for key in ("mean", "std", "max", "min", "max_deviation", "fraction_high", "fraction_low"):
+            out[f"{p}_seq_{key}"] = 0.0
+    return out
+
+
+@torch.no_grad()
+def rollout_rejection_mask(log_ratio, response_mask, rollout_rs="token_k1", rollout_rs_threshold=None):
+    """compute_rollout_rejection_mask, rollout_corr_helper.py:163-357: every requested option keeps a token (token
+    level) or a whole sequence (sum / mean / max of the token statistic) whose divergence estimate lies inside its
+    bounds; the masks multiply.  k1 = -log ratio with bounds ``[log lower, log upper]``, k2 = half the squared log
+    ratio, k3 = exp(r) - 1 - r, each with an upper bound; the log ratio is clamped to +-20 first.  Returns
+    ``(modified_response_mask, metrics)``."""
+    if rollout_rs is None or not isinstance(rollout_rs, str):
+        raise ValueError("rollout_rs must be a non-empty string (comma separated for multiple options).")
+    if rollout_rs_threshold is None:
+        raise ValueError("rollout_rs_threshold must be provided for rejection sampling.")
+    if log_ratio.shape[0] == 0:
+        return response_mask, {}
+    options = []
+    for opt in (o.strip() for o in rollout_rs.split(",")):
+        if not opt:
+            continue
+        if opt not in RS_OPTIONS:
+            raise ValueError(f"Invalid rollout_rs option: {opt}. Must be one of {sorted(RS_OPTIONS)}.")
+        if opt not in options:
+            options.append(opt)
+    if not options:
+        raise ValueError("rollout_rs must contain at least one valid option.")
+    bounds = parse_rs_thresholds(options, rollout_rs_threshold)
+    d = log_ratio.clamp(-SAFETY_BOUND, SAFETY_BOUND)
+    token = {"k1": -d, "k2": 0.5 * d**2, "k3": torch.exp(d) - 1.0 - d}
+    valid = response_mask.bool()
+    seq_valid = response_mask.sum(dim=-1) > 0
+    combined = torch.ones_like(response_mask, dtype=log_ratio.dtype)
+    metrics = {}
+    for opt in options:
+        scope, est = opt.rsplit("_", 1)
+        lower, upper = bounds[opt]
+        stat = token[est]
+        per_sequence = None
+        if scope == "seq_sum":
+            per_sequence = masked_sum(stat, response_mask, axis=-1)
+        elif scope == "seq_mean":
+            per_sequence = masked_mean(stat, response_mask, axis=-1)
+        elif scope == "seq_max":
+            top = stat.masked_fill(~valid, float("-inf")).max(dim=-1).values
+            per_sequence = torch.where(top == float("-inf"), torch.zeros_like(top), top)
+        if per_sequence is not None:
+            stat = per_sequence.unsqueeze(-1).expand_as(response_mask)
+        if est == "k1":
+            lo, hi, apply_lower = math.log(lower), math.log(upper), True
+            keep = (stat >= lo) & (stat <= hi)
+        else:
+            lo, hi, apply_lower = 0.0, upper, False
+            keep = stat <= hi
+        combined = combined * keep.to(log_ratio.dtype)
+        seq_keep = (~((~keep) & valid)).all(dim=-1)
+        metrics.update(rs_metrics(opt, stat, response_mask, seq_valid, "token" if scope == "token" else "sequence",
+                                  per_sequence, hi, lo, apply_lower))
+        metrics[f"rollout_rs_{opt}_masked_fraction"] = masked_mean(1 - keep.to(log_ratio.dtype), response_mask).item()
+        alive = seq_valid.float()
+        metrics[f"rollout_rs_{opt}_seq_masked_fraction"] = (
+            (((1.0 - seq_keep.to(log_ratio.dtype)) * alive).sum() / alive.sum()).item() if alive.sum() > 0 else 0.0)
+    metrics["rollout_rs_masked_fraction"] = masked_mean(1 - combined, response_mask).item()
+    final_keep = (combined > 0.5) & valid
+    metrics["rollout_rs_seq_masked_fraction"] = ((~final_keep) & valid).any(dim=-1).float().mean().item()
+    return (response_mask * combined).to(response_mask.dtype), metrics

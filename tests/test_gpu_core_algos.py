@@ -4,6 +4,7 @@ Tolerance (north star): advantages and losses within rtol 1e-5 in fp32; as in th
 equivalence tests an absolute floor of 1e-6 accompanies it (values that cancel to ~0).  Mask and
 index handling is checked bit-exactly (zeros stay exact zeros, group membership by label).
 """
+import math
 import random
 import types
 import uuid
@@ -1057,7 +1058,90 @@ def test_rollout_correction_reference_literals_and_entry_points(dev):
         RC.compute_rollout_correction_weights((o - r).to(dev), torch.zeros_like(m).to(dev), "token", 2.0)
     with pytest.raises(ValueError, match="does not match"):
         RC.compute_rollout_correction_and_rejection_mask(o.to(dev), r[:, :-1].to(dev), m.to(dev))
-    with pytest.raises(NotImplementedError):
-        RC.compute_rollout_correction_and_rejection_mask(o.to(dev), r.to(dev), m.to(dev), rollout_rs="token_k1",
-                                                         rollout_rs_threshold="0.5_2.0")
+    with pytest.raises(ValueError, match="rollout_rs_threshold must be explicitly provided"):
+        RC.compute_rollout_correction_and_rejection_mask(o.to(dev), r.to(dev), m.to(dev), rollout_rs="token_k1")
+
+
+_RS_CASES = [("token_k1", "0.8_1.3"), ("token_k2", 0.02), ("token_k3", 0.03), ("seq_sum_k1", "0.2_4.0"),
+             ("seq_sum_k2", 8.0), ("seq_sum_k3", 9.0), ("seq_mean_k1", 1.01), ("seq_mean_k2", 0.03),
+             ("seq_mean_k3", 0.033), ("seq_max_k2", 0.4), ("seq_max_k3", 0.6),
+             ("token_k1,seq_mean_k3,token_k2", "0.7_1.4,0.033,0.1"), ("seq_max_k2, token_k3 ,seq_sum_k1", "0.4,0.05,0.2_4.0")]
+
+
+@pytest.mark.parametrize("rollout_rs,threshold", _RS_CASES)
+@pytest.mark.parametrize("shape", [(9, 13), (24, 5000), (64, 1024)])
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.int64, torch.bool])
+def test_rollout_rejection_mask(dev, rollout_rs, threshold, shape, mdtype):
+    from verl_amd.trainer.ppo import rollout_corr_helper as RC
+    B, Lc = shape
+    g = torch.Generator().manual_seed(B * 31 + Lc + len(rollout_rs))
+    # per-sequence drift and spread vary, so that every option rejects some sequences and keeps others
+    d = torch.randn(B, Lc, generator=g) * (0.05 + 0.3 * torch.rand(B, 1, generator=g)) + 0.02 * torch.randn(B, 1, generator=g)
+    d = d / math.sqrt(Lc / 13)   if "seq_sum" in rollout_rs else d
+    d[0, 0] = 30.0                                               # beyond the safety clamp
+    mask = (torch.rand(B, Lc, generator=g) < 0.8).float()
+    mask[3] = 0                                                  # an empty sequence
+    new, metrics = RC.compute_rollout_rejection_mask(d.to(dev), mask.to(dev).to(mdtype), rollout_rs, threshold)
+    want32, m32 = O.rollout_rejection_mask(d, mask, rollout_rs, threshold)
+    want64, m64 = O.rollout_rejection_mask(d.double(), mask.double(), rollout_rs, threshold)
+    assert new.dtype == mdtype and new.shape == mask.shape
+    assert torch.equal(new.cpu().float(), want32), "the kept tokens differ"
+    _rc_check(metrics, m32, m64, rollout_rs)
+    assert metrics["rollout_rs_masked_fraction"] < 1             # something is kept
+    if Lc >= 1024:
+        assert metrics["rollout_rs_masked_fraction"] > 0         # and at these sizes every case rejects something
+
+
+def test_rollout_rejection_reference_literals_and_unified_entry(dev):
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.trainer.ppo import rollout_corr_helper as RC
+    case = GOLDEN["rollout_corr_mask_mode"]
+    old, roll, mask = (torch.tensor(case[k]).to(dev) for k in ("old_log_prob", "rollout_log_prob", "response_mask"))
+    proto, new, metrics = RC.compute_rollout_correction_and_rejection_mask(
+        old, roll, mask, rollout_is=case["rollout_is"], rollout_is_threshold=case["rollout_is_threshold"],
+        rollout_rs=case["rollout_rs"], rollout_rs_threshold=case["rollout_rs_threshold"])
+    w = proto.batch["rollout_is_weights"].cpu()
+    assert (w[0] > 0).all()                                      # rejection goes through the mask, not the weights
+    assert abs(w[0, 0].item() - case["expected_weight_row0"]) <= case["atol"]
+    assert (new[0] == case["expected_modified_mask_row0"]).all() and (new[1] == case["expected_modified_mask_row1"]).all()
+    assert abs(metrics["rollout_corr/rollout_rs_masked_fraction"] - case["expected_masked_fraction"]) < case["masked_fraction_atol"]
+    spec = GOLDEN["rollout_rs_options"]
+    g = torch.Generator().manual_seed(0)
+    B, Lc = spec["shape"]
+    o = torch.randn(B, Lc, generator=g); r = o + torch.randn(B, Lc, generator=g) * spec["noise_std"]
+    ones = torch.ones(B, Lc)
+    for option, threshold in spec["cases"] + [[spec["chained"]["rollout_rs"], spec["chained"]["rollout_rs_threshold"]]]:
+        _, new, metrics = RC.compute_rollout_correction_and_rejection_mask(o.to(dev), r.to(dev), ones.to(dev), rollout_rs=option,
+                                                                          rollout_rs_threshold=threshold)
+        want, wm = O.rollout_rejection_mask(o - r, ones, option, threshold)
+        assert torch.equal(new.cpu(), want)
+        for name in option.split(","):
+            assert "rollout_corr/" + spec["expected_key_template"].format(option=name) in metrics
+        assert {f"rollout_corr/{k}" for k in wm} <= set(metrics)
+    assert RC.SUPPORTED_ROLLOUT_RS_OPTIONS == set(O.RS_OPTIONS)
+    for rs, thr, err in (("token_k9", 1.0, ValueError), ("token_k2", "1_2", ValueError), ("token_k1,token_k2", "1,2,3", ValueError),
+                         ("token_k2", [1.0], TypeError), (" , ", 1.0, ValueError)):
+        with pytest.raises(err):
+            RC.compute_rollout_rejection_mask((o - r).to(dev), ones.to(dev), rs, thr)
+    with pytest.raises(ValueError, match="at least one valid token"):
+        RC.compute_rollout_rejection_mask((o - r).to(dev), torch.zeros(B, Lc, device=dev), "token_k2", 1.0)
+    # bypass mode with rejection: the loss sees the reduced mask
+    gen = torch.Generator().manual_seed(2)
+    B, Lc = 10, 300
+    m, _ = _prefix_mask(B, Lc, gen, lo=3)
+    rollout = torch.randn(B, Lc, generator=gen) * 0.5 - 1
+    new_lp = rollout + torch.randn(B, Lc, generator=gen) * 0.3
+    adv = torch.randn(B, Lc, generator=gen)
+    cfg = _cfg(clip_ratio=0.2)
+    cfg.policy_loss = {"rollout_correction": {"loss_type": "reinforce", "rollout_is": "token", "rollout_is_threshold": 2.0,
+                                              "rollout_rs": "token_k1", "rollout_rs_threshold": "0.7_1.5"}}
+    nd = new_lp.to(dev).requires_grad_(); no = new_lp.clone().requires_grad_()
+    loss, met = CA.compute_policy_loss_bypass_mode(rollout.to(dev), nd, adv.to(dev), m.to(dev), "seq-mean-token-sum", cfg)
+    w, _ = O.rollout_correction_weights(new_lp - rollout, m, "token", 2.0)
+    reduced, rs_m = O.rollout_rejection_mask(new_lp - rollout, m, "token_k1", "0.7_1.5")
+    want_loss, want_kl = O.policy_loss_reinforce(rollout, no, adv, reduced, "seq-mean-token-sum", w)
+    _close(loss, want_loss, what="bypass loss with rejection")
+    assert abs(met["actor/ppo_kl"] - want_kl.item()) < 2e-6 * max(1.0, abs(want_kl.item()))
+    assert met["rollout_corr/rollout_rs_masked_fraction"] == pytest.approx(rs_m["rollout_rs_masked_fraction"], rel=1e-5)
+    _close(torch.autograd.grad(loss, nd)[0], torch.autograd.grad(want_loss, no)[0], atol=1e-9, what="d bypass loss")
 

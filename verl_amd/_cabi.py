@@ -69,6 +69,10 @@ SIGNATURES = {
                                              c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "vamd_response_window_gather": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                             c_void_p, c_void_p, c_void_p]),
+    "vamd_rollout_rs_chunks": (c_int64, [c_int64]),
+    "vamd_rollout_rs_row_stats": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
+    "vamd_rollout_rs_apply": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int,
+                                      c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "vamd_otb_advantage_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int]),
     "vamd_otb_advantage": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                    c_void_p, c_int64, c_int64, c_int64, c_int, c_float, c_void_p, c_void_p, c_void_p,

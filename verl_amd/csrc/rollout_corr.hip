@@ -368,3 +368,223 @@ extern "C" int vamd_rollout_correction(const float* old_log_prob, const float* r
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }
+
+// =============================================================================================================
+// Rejection sampling (compute_rollout_rejection_mask, rollout_corr_helper.py:163-357).
+//
+// Two streaming passes with the decisions that need a whole sequence taken between them on the host, from a
+// [batch]-sized table: the first pass leaves, per (row, chunk), the sums and maxima of the three divergence
+// estimates k1 = -r, k2 = r^2 / 2, k3 = exp(r) - 1 - r (r = the log ratio clamped to +-20); the host folds the
+// chunks, evaluates the sequence-level options (sum / mean / max against their bounds) and hands back one keep flag
+// per row; the second pass applies the token-level options and that flag, writes the new mask in the element
+// type of the old one and leaves the per-(row, chunk) counts the token-level metrics are made of.
+// =============================================================================================================
+namespace vamd {
+
+enum { kRsCount = 0, kRsK1, kRsK2, kRsK3, kRsK2Max, kRsK3Max, kRsRowSlots };
+enum { kRsSum = 0, kRsMax, kRsMinNeg, kRsHigh, kRsLow, kRsClamp, kRsClamp2, kRsRejected, kRsOptionSlots };
+constexpr int kRsMaxTokenOptions = 3;
+
+__device__ __forceinline__ void rs_estimates(float old_lp, float roll_lp, float (&k)[3]) {
+  const float r = fminf(fmaxf(old_lp - roll_lp, -kSafetyBound), kSafetyBound);
+  k[0] = -r;
+  k[1] = 0.5f * r * r;
+  k[2] = expf(r) - 1.f - r;
+}
+
+template <bool VEC, class M>
+__global__ __launch_bounds__(kRcThreads) void rs_rows_kernel(const float* __restrict__ old_lp,
+                                                             const float* __restrict__ roll_lp,
+                                                             const M* __restrict__ mask, int64_t rows, int64_t cols,
+                                                             int chunks, double* __restrict__ records) {
+  const int64_t row = blockIdx.x / chunks;
+  const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float o[kGroups][4], r[kGroups][4], m[kGroups][4];
+  load_groups<VEC>(old_lp, pos, o);
+  load_groups<VEC>(roll_lp, pos, r);
+  load_mask_groups<VEC>(mask, pos, m);
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  float top[2] = {-__builtin_inff(), -__builtin_inff()};
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (e >= pos.valid[g] || m[g][e] == 0.f) continue;
+      float k[3];
+      rs_estimates(o[g][e], r[g][e], k);
+      s[0] += 1.f;
+      s[1] += k[0]; s[2] += k[1]; s[3] += k[2];
+      top[0] = fmaxf(top[0], k[1]);
+      top[1] = fmaxf(top[1], k[2]);
+    }
+  __shared__ double smem[4 * 4];
+  double acc[4] = {s[0], s[1], s[2], s[3]};
+  block_sum<4, kRcThreads>(acc, smem);
+  double ext[2] = {top[0], top[1]};
+  block_max_f64<2, kRcThreads>(ext, smem);
+  if (threadIdx.x == 0) {
+    const double rec[kRsRowSlots] = {acc[0], acc[1], acc[2], acc[3], ext[0], ext[1]};
+#pragma unroll
+    for (int i = 0; i < kRsRowSlots; ++i) records[record_at(i, row, chunk, rows, chunks)] = rec[i];
+  }
+}
+
+struct RsOptions {
+  int n;                                  // token-level options, 0..3
+  int estimator[kRsMaxTokenOptions];      // 0 k1, 1 k2, 2 k3
+  float lower[kRsMaxTokenOptions];        // keep rule and metric thresholds (k1: logs of the ratio bounds)
+  float upper[kRsMaxTokenOptions];
+  int two_sided[kRsMaxTokenOptions];      // k1: keep inside [lower, upper]; others: keep below upper
+};
+
+template <bool VEC, class M>
+__global__ __launch_bounds__(kRcThreads) void rs_apply_kernel(const float* __restrict__ old_lp,
+                                                              const float* __restrict__ roll_lp,
+                                                              const M* __restrict__ mask,
+                                                              const uint8_t* __restrict__ row_keep, int64_t rows,
+                                                              int64_t cols, int chunks, RsOptions opt,
+                                                              M* __restrict__ new_mask, double* __restrict__ records) {
+  const int64_t row = blockIdx.x / chunks;
+  const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float o[kGroups][4], r[kGroups][4], m[kGroups][4];
+  load_groups<VEC>(old_lp, pos, o);
+  load_groups<VEC>(roll_lp, pos, r);
+  load_mask_groups<VEC>(mask, pos, m);
+  const bool row_ok = row_keep[row] != 0;
+  float s[kRsMaxTokenOptions][kRsOptionSlots];
+#pragma unroll
+  for (int j = 0; j < kRsMaxTokenOptions; ++j)
+#pragma unroll
+    for (int i = 0; i < kRsOptionSlots; ++i) s[j][i] = (i == kRsMax || i == kRsMinNeg) ? -__builtin_inff() : 0.f;
+  float rejected = 0.f;
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g) {
+    M out[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float k[3];
+      rs_estimates(o[g][e], r[g][e], k);
+      bool keep = row_ok;
+      const bool in = e < pos.valid[g] && m[g][e] != 0.f;
+#pragma unroll
+      for (int j = 0; j < kRsMaxTokenOptions; ++j) {
+        if (j >= opt.n) break;
+        const float v = opt.estimator[j] == 0 ? k[0] : (opt.estimator[j] == 1 ? k[1] : k[2]);
+        const bool ok = opt.two_sided[j] ? (v >= opt.lower[j] && v <= opt.upper[j]) : (v <= opt.upper[j]);
+        keep = keep && ok;
+        if (in) {
+          const float c = fminf(fmaxf(v, opt.two_sided[j] ? opt.lower[j] : 0.f), opt.upper[j]);
+          s[j][kRsSum] += v;
+          s[j][kRsMax] = fmaxf(s[j][kRsMax], v);
+          s[j][kRsMinNeg] = fmaxf(s[j][kRsMinNeg], -v);
+          s[j][kRsHigh] += v > opt.upper[j] ? 1.f : 0.f;
+          s[j][kRsLow] += (opt.two_sided[j] && v < opt.lower[j]) ? 1.f : 0.f;
+          s[j][kRsClamp] += c;
+          s[j][kRsClamp2] += c * c;
+          s[j][kRsRejected] += ok ? 0.f : 1.f;
+        }
+      }
+      if (in && !keep) rejected += 1.f;
+      // response_mask * combined keep, in the mask's own element type; masked-out positions keep their 0
+      out[e] = keep ? static_cast<M>(m[g][e]) : static_cast<M>(0);
+    }
+    if (pos.valid[g] > 0) {
+      if constexpr (VEC) {
+        struct alignas(sizeof(M) * 4) Pack { M v[4]; };
+        Pack p;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) p.v[e] = out[e];
+        *reinterpret_cast<Pack*>(new_mask + pos.idx[g]) = p;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (e < pos.valid[g]) new_mask[pos.idx[g] + e] = out[e];
+      }
+    }
+  }
+  __shared__ double smem[8 * 4];
+  double rej[1] = {rejected};
+  block_sum<1, kRcThreads>(rej, smem);
+  if (threadIdx.x == 0) records[record_at(0, row, chunk, rows, chunks)] = rej[0];
+#pragma unroll
+  for (int j = 0; j < kRsMaxTokenOptions; ++j) {
+    if (j >= opt.n) break;
+    double sums[6] = {s[j][kRsSum], s[j][kRsHigh], s[j][kRsLow], s[j][kRsClamp], s[j][kRsClamp2], s[j][kRsRejected]};
+    block_sum<6, kRcThreads>(sums, smem);
+    double ext[2] = {s[j][kRsMax], s[j][kRsMinNeg]};
+    block_max_f64<2, kRcThreads>(ext, smem);
+    if (threadIdx.x == 0) {
+      const double rec[kRsOptionSlots] = {sums[0], ext[0], ext[1], sums[1], sums[2], sums[3], sums[4], sums[5]};
+#pragma unroll
+      for (int i = 0; i < kRsOptionSlots; ++i)
+        records[record_at(1 + j * kRsOptionSlots + i, row, chunk, rows, chunks)] = rec[i];
+    }
+  }
+}
+
+}  // namespace vamd
+
+extern "C" int64_t vamd_rollout_rs_chunks(int64_t length) { return chunks_of(length); }
+
+extern "C" int vamd_rollout_rs_row_stats(const float* old_log_prob, const float* rollout_log_prob, const void* mask,
+                                         int mask_dtype, int64_t batch, int64_t length, double* records,
+                                         void* stream) {
+  VAMD_REQUIRE(batch > 0 && length > 0, "rollout_rs_row_stats: empty input");
+  VAMD_REQUIRE(batch * chunks_of(length) < (1ll << 31), "rollout_rs_row_stats: too many workgroups");
+  VAMD_REQUIRE(old_log_prob && rollout_log_prob && mask && records, "rollout_rs_row_stats: null pointer");
+  const int chunks = (int)chunks_of(length);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)(batch * chunks)), block(kRcThreads);
+  VAMD_MASK_DISPATCH(mask_dtype, M, {
+    const M* mk = static_cast<const M*>(mask);
+    if (can_vectorize(length, {old_log_prob, rollout_log_prob}, mask, sizeof(M)))
+      hipLaunchKernelGGL((rs_rows_kernel<true, M>), grid, block, 0, s, old_log_prob, rollout_log_prob, mk, batch,
+                         length, chunks, records);
+    else
+      hipLaunchKernelGGL((rs_rows_kernel<false, M>), grid, block, 0, s, old_log_prob, rollout_log_prob, mk, batch,
+                         length, chunks, records);
+  });
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
+
+extern "C" int vamd_rollout_rs_apply(const float* old_log_prob, const float* rollout_log_prob, const void* mask,
+                                     int mask_dtype, int64_t batch, int64_t length, const uint8_t* row_keep,
+                                     int n_token_options, const int* estimators, const float* lower,
+                                     const float* upper, void* new_mask, double* records, void* stream) {
+  VAMD_REQUIRE(batch > 0 && length > 0, "rollout_rs_apply: empty input");
+  VAMD_REQUIRE(batch * chunks_of(length) < (1ll << 31), "rollout_rs_apply: too many workgroups");
+  VAMD_REQUIRE(old_log_prob && rollout_log_prob && mask && row_keep && new_mask && records,
+               "rollout_rs_apply: null pointer");
+  VAMD_REQUIRE(n_token_options >= 0 && n_token_options <= kRsMaxTokenOptions,
+               "rollout_rs_apply: at most %d token-level options", kRsMaxTokenOptions);
+  VAMD_REQUIRE(n_token_options == 0 || (estimators && lower && upper), "rollout_rs_apply: null option tables");
+  RsOptions opt;
+  opt.n = n_token_options;
+  for (int j = 0; j < kRsMaxTokenOptions; ++j) {
+    const bool have = j < n_token_options;
+    opt.estimator[j] = have ? estimators[j] : 0;
+    VAMD_REQUIRE(opt.estimator[j] >= 0 && opt.estimator[j] <= 2, "rollout_rs_apply: invalid estimator %d",
+                 opt.estimator[j]);
+    opt.lower[j] = have ? lower[j] : 0.f;
+    opt.upper[j] = have ? upper[j] : 0.f;
+    opt.two_sided[j] = opt.estimator[j] == 0;
+  }
+  const int chunks = (int)chunks_of(length);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)(batch * chunks)), block(kRcThreads);
+  VAMD_MASK_DISPATCH(mask_dtype, M, {
+    const M* mk = static_cast<const M*>(mask);
+    M* out = static_cast<M*>(new_mask);
+    if (can_vectorize(length, {old_log_prob, rollout_log_prob}, mask, sizeof(M)) && aligned_to(new_mask, sizeof(M) * 4))
+      hipLaunchKernelGGL((rs_apply_kernel<true, M>), grid, block, 0, s, old_log_prob, rollout_log_prob, mk, row_keep,
+                         batch, length, chunks, opt, out, records);
+    else
+      hipLaunchKernelGGL((rs_apply_kernel<false, M>), grid, block, 0, s, old_log_prob, rollout_log_prob, mk, row_keep,
+                         batch, length, chunks, opt, out, records);
+  });
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
