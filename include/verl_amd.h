@@ -311,6 +311,15 @@ int vamd_rollout_correction(const float* old_log_prob, const float* rollout_log_
                             int batch_normalize, float* weights, double* metrics, void* workspace,
                             size_t workspace_bytes, void* stream);
 
+/* Per-row sums for compute_variance_proxy_metrics (verl/trainer/ppo/metric_utils.py:306-412).  records: doubles
+ * [5][chunks][batch] with chunks = vamd_rollout_rs_chunks(length): number of valid tokens, sum of advantages,
+ * sum of w = 1 - 2 exp(old_log_prob) + sum_pi_squared (times is_weight^2 when is_weights is given), sum of the
+ * importance weights, sum of w / max(is_weight^2, 1e-10), each over the valid tokens.  is_weights may be NULL
+ * (slots 3 and 4 are then 0). */
+int vamd_variance_proxy_rows(const float* advantages, const float* old_log_probs, const float* sum_pi_squared,
+                             const float* is_weights, const void* mask, int mask_dtype, int64_t batch,
+                             int64_t length, double* records, void* stream);
+
 /* Rejection sampling of the rollout correction (compute_rollout_rejection_mask,
  * rollout_corr_helper.py:163-357) as two streaming passes around a host step.  Records are doubles laid out
  * [slot][chunk][row] with chunk count vamd_rollout_rs_chunks(length).

@@ -73,6 +73,7 @@ from .trainer import (  # noqa: F401
     compute_rewards,
     compute_data_metrics,
     pad_to_response_window,
+    variance_proxy_metrics,
 )
 from .rollout_corr import (  # noqa: F401
     offpolicy_metrics,

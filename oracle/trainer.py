@@ -10,7 +10,7 @@ import numpy as np
 import torch
 
 from .losses import kl_penalty
-from .masked import masked_mean
+from .masked import masked_mean, masked_sum
 
 
 @torch.no_grad()
@@ -80,3 +80,37 @@ def pad_to_response_window(values, indices, batch, seqlen, response_length):
     full = torch.zeros(batch * seqlen, dtype=values.dtype)
     full = full.index_put((indices,), values)
     return full.view(batch, seqlen)[:, -response_length - 1:-1]
+
+
+@torch.no_grad()
+def variance_proxy_metrics(batch, gradient_norm=None):
+    """compute_variance_proxy_metrics, verl/trainer/ppo/metric_utils.py:306-412, on a plain mapping: with
+    W(tau) = sum_t (1 - 2 pi_t + sum pi^2) and the mean advantage per trajectory, proxy 2 = E[A^2 W] (with
+    importance weights: E[rho^2 A^2 W_original]), proxy 1 = the squared gradient norm handed in, proxy 3 =
+    (proxy 2 - proxy 1) / (N - 1) floored at 0."""
+    out = {}
+    if "sum_pi_squared" not in batch or "old_log_probs" not in batch or "advantages" not in batch:
+        return out
+    w = 1 - 2 * torch.exp(batch["old_log_probs"]) + batch["sum_pi_squared"]
+    mask = batch["response_mask"]
+    isw = batch.get("rollout_is_weights", None)
+    if isw is not None:
+        w = w * isw**2
+    adv = masked_mean(batch["advantages"], mask, axis=-1)
+    w_sum = masked_sum(w, mask, axis=-1)
+    proxy1 = gradient_norm**2 if gradient_norm is not None else None
+    if isw is not None:
+        rho = masked_mean(isw, mask, axis=-1)
+        w_orig = masked_sum(w / torch.clamp(isw**2, min=1e-10), mask, axis=-1).clamp(min=0.0)
+        proxy2 = (rho**2 * adv**2 * w_orig).mean()
+    else:
+        proxy2 = (adv**2 * w_sum.clamp(min=0.0)).mean()
+    proxy3 = None
+    if proxy1 is not None and adv.shape[0] > 1:
+        proxy3 = max(0.0, ((proxy2 - proxy1) / (adv.shape[0] - 1)).item())
+    out["variance_proxy/proxy1_signal_strength"] = proxy1 if proxy1 is not None else 0.0
+    out["variance_proxy/proxy2_total_power"] = proxy2.item()
+    out["variance_proxy/proxy3_pure_noise"] = proxy3 if proxy3 is not None else 0.0
+    out["variance_proxy/expected_a_squared"] = (adv**2).mean().item()
+    out["variance_proxy/expected_w"] = w_sum.mean().item()
+    return out

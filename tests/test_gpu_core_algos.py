@@ -1145,3 +1145,46 @@ def test_rollout_rejection_reference_literals_and_unified_entry(dev):
     assert met["rollout_corr/rollout_rs_masked_fraction"] == pytest.approx(rs_m["rollout_rs_masked_fraction"], rel=1e-5)
     _close(torch.autograd.grad(loss, nd)[0], torch.autograd.grad(want_loss, no)[0], atol=1e-9, what="d bypass loss")
 
+
+@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192)])
+@pytest.mark.parametrize("with_isw", [False, True])
+@pytest.mark.parametrize("mdtype", [torch.float32, torch.int64])
+def test_variance_proxy_metrics(dev, shape, with_isw, mdtype):
+    from verl_amd.trainer.ppo.metric_utils import compute_variance_proxy_metrics
+    B, Lc = shape
+    g = torch.Generator().manual_seed(B + Lc)
+    pi = torch.rand(B, Lc, generator=g).clamp_min(1e-4)
+    batch = {"old_log_probs": pi.log(), "sum_pi_squared": pi * pi + torch.rand(B, Lc, generator=g) * (1 - pi) ** 2,
+             "advantages": torch.randn(B, 1, generator=g).expand(B, Lc).contiguous(),
+             "response_mask": _prefix_mask(B, Lc, g, lo=1)[0]}
+    batch["response_mask"][1] = 0                                # an empty trajectory
+    if with_isw:
+        batch["rollout_is_weights"] = (0.5 + torch.rand(B, Lc, generator=g)) * batch["response_mask"]
+    want = O.variance_proxy_metrics(batch, gradient_norm=0.3)
+    want64 = O.variance_proxy_metrics({k: v.double() for k, v in batch.items()}, gradient_norm=0.3)
+    on_dev = {k: (v.to(mdtype) if k == "response_mask" else v).to(dev) for k, v in batch.items()}
+    got = compute_variance_proxy_metrics(_data(on_dev), gradient_norm=0.3)
+    _rc_check(got, want, want64, "variance proxy")
+    assert compute_variance_proxy_metrics(_data({"advantages": on_dev["advantages"], "response_mask": on_dev["response_mask"]})) == {}
+
+
+def test_rollout_correction_batch_entry_points(dev):
+    from verl_amd.trainer.ppo import rollout_corr_helper as RC
+    o, r, m = _rc_inputs(8, 200, 5, 0.3)
+    data = _data(dict(old_log_probs=o.to(dev), rollout_log_probs=r.to(dev), response_mask=m.to(dev)))
+    cfg = {"rollout_is": "token", "rollout_is_threshold": 2.0, "rollout_rs": "token_k1", "rollout_rs_threshold": "0.6_1.6"}
+    out, metrics = RC.compute_rollout_correction_and_add_to_batch(data, cfg)
+    w, wm = O.rollout_correction_weights(o - r, m, "token", 2.0)
+    new, rm = O.rollout_rejection_mask(o - r, m, "token_k1", "0.6_1.6")
+    assert out is data and torch.equal(data.batch["response_mask"].cpu(), new)
+    _close(data.batch["rollout_is_weights"], w, what="weights")
+    assert {f"rollout_corr/{k}" for k in list(wm) + list(rm)} <= set(metrics)
+    data = _data(dict(old_log_probs=o.to(dev), rollout_log_probs=r.to(dev), response_mask=m.to(dev)))
+    RC.compute_rollout_correction_and_add_to_batch(data, {})
+    assert "rollout_is_weights" not in data.batch and torch.equal(data.batch["response_mask"].cpu(), m)
+    got = RC.compute_rollout_corr_metrics_from_logprobs(o.to(dev), r.to(dev), m.to(dev))
+    want = O.offpolicy_metrics(o, r, m)
+    assert set(got) == {f"rollout_corr/{k}" for k in want}
+    for k, v in want.items():
+        assert got[f"rollout_corr/{k}"] == pytest.approx(v, rel=1e-4, abs=1e-6), k
+

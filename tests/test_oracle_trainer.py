@@ -121,3 +121,24 @@ def test_pad_to_response_window_by_hand():
     assert out.tolist() == [[11.0, 12.0], [22.0, 0.0]]
     out.backward(torch.tensor([[1.0, 2.0], [3.0, 4.0]]))
     assert values.grad.tolist() == [0.0, 1.0, 2.0, 0.0, 0.0, 0.0, 3.0]
+
+
+def test_variance_proxy_by_hand():
+    # two trajectories; pi = 1/2 and sum pi^2 = 1/2 give w = 1/2 per token
+    batch = {"old_log_probs": torch.full((2, 3), math.log(0.5)), "sum_pi_squared": torch.full((2, 3), 0.5),
+             "advantages": torch.tensor([[2.0, 2.0, 9.0], [-1.0, -3.0, -2.0]]),
+             "response_mask": torch.tensor([[1.0, 1.0, 0.0], [1.0, 1.0, 1.0]])}
+    m = O.variance_proxy_metrics(batch, gradient_norm=0.5)
+    # A = (2, -2), W = (1, 1.5): E[A^2 W] = (4 + 6) / 2
+    assert m["variance_proxy/proxy2_total_power"] == pytest.approx(5.0)
+    assert m["variance_proxy/proxy1_signal_strength"] == 0.25
+    assert m["variance_proxy/proxy3_pure_noise"] == pytest.approx(4.75)
+    assert m["variance_proxy/expected_a_squared"] == pytest.approx(4.0) and m["variance_proxy/expected_w"] == pytest.approx(1.25)
+    # importance weights of 2 on the second trajectory: w carries rho^2, the proxy divides it out again and
+    # multiplies by the squared mean weight: (1 * 4 * 1 + 4 * 4 * 1.5) / 2
+    batch["rollout_is_weights"] = torch.tensor([[1.0, 1.0, 1.0], [2.0, 2.0, 2.0]])
+    m = O.variance_proxy_metrics(batch)
+    assert m["variance_proxy/proxy2_total_power"] == pytest.approx(14.0)
+    assert m["variance_proxy/expected_w"] == pytest.approx((1 + 6) / 2)
+    assert m["variance_proxy/proxy1_signal_strength"] == 0.0 and m["variance_proxy/proxy3_pure_noise"] == 0.0
+    assert O.variance_proxy_metrics({"advantages": batch["advantages"]}) == {}

@@ -69,6 +69,8 @@ SIGNATURES = {
                                              c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "vamd_response_window_gather": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                             c_void_p, c_void_p, c_void_p]),
+    "vamd_variance_proxy_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
+                                         c_void_p, c_void_p]),
     "vamd_rollout_rs_chunks": (c_int64, [c_int64]),
     "vamd_rollout_rs_row_stats": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_void_p]),
     "vamd_rollout_rs_apply": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_void_p, c_int,

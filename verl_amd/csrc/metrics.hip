@@ -205,9 +205,84 @@ __global__ __launch_bounds__(kDmFoldThreads) void data_metrics_fold_kernel(DmArg
   }
 }
 
+// Per-row sums behind compute_variance_proxy_metrics (verl/trainer/ppo/metric_utils.py:306-412):
+// slot 0 number of valid tokens, 1 sum of advantages, 2 sum of w = 1 - 2 exp(old_log_prob) + sum_pi_squared
+// (times is_weight^2 when importance weights are given), 3 sum of the importance weights,
+// 4 sum of w / max(is_weight^2, 1e-10), each over the valid tokens.  The [batch]-sized rest is host arithmetic.
+enum { kVpCount = 0, kVpAdv, kVpW, kVpIsw, kVpWOriginal, kVpSlots };
+
+template <bool VEC, class M, bool ISW>
+__global__ __launch_bounds__(kRcThreads) void variance_proxy_rows_kernel(const float* __restrict__ adv,
+                                                                         const float* __restrict__ old_lp,
+                                                                         const float* __restrict__ pi2,
+                                                                         const float* __restrict__ isw,
+                                                                         const M* __restrict__ mask, int64_t rows,
+                                                                         int64_t cols, int chunks,
+                                                                         double* __restrict__ records) {
+  const int64_t row = blockIdx.x / chunks;
+  const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float a[kGroups][4], lp[kGroups][4], q[kGroups][4], iw[kGroups][4], m[kGroups][4];
+  load_groups<VEC>(adv, pos, a);
+  load_groups<VEC>(old_lp, pos, lp);
+  load_groups<VEC>(pi2, pos, q);
+  if (ISW) load_groups<VEC>(isw, pos, iw);
+  load_mask_groups<VEC>(mask, pos, m);
+  float s[kVpSlots] = {0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (e >= pos.valid[g] || m[g][e] == 0.f) continue;
+      float w = 1.f - 2.f * expf(lp[g][e]) + q[g][e];
+      s[kVpCount] += 1.f;
+      s[kVpAdv] += a[g][e];
+      if (ISW) {
+        const float r2 = iw[g][e] * iw[g][e];
+        w = w * r2;
+        s[kVpIsw] += iw[g][e];
+        s[kVpWOriginal] += w / fmaxf(r2, 1e-10f);
+      }
+      s[kVpW] += w;
+    }
+  __shared__ double smem[kVpSlots * 4];
+  double acc[kVpSlots];
+#pragma unroll
+  for (int i = 0; i < kVpSlots; ++i) acc[i] = s[i];
+  block_sum<kVpSlots, kRcThreads>(acc, smem);
+  if (threadIdx.x == 0)
+#pragma unroll
+    for (int i = 0; i < kVpSlots; ++i) records[record_at(i, row, chunk, rows, chunks)] = acc[i];
+}
+
 }  // namespace vamd
 
 using namespace vamd;
+
+extern "C" int vamd_variance_proxy_rows(const float* advantages, const float* old_log_probs,
+                                        const float* sum_pi_squared, const float* is_weights, const void* mask,
+                                        int mask_dtype, int64_t batch, int64_t length, double* records,
+                                        void* stream) {
+  VAMD_REQUIRE(batch > 0 && length > 0, "variance_proxy_rows: empty input");
+  VAMD_REQUIRE(batch * chunks_of(length) < (1ll << 31), "variance_proxy_rows: too many workgroups");
+  VAMD_REQUIRE(advantages && old_log_probs && sum_pi_squared && mask && records, "variance_proxy_rows: null pointer");
+  const int chunks = (int)chunks_of(length);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)(batch * chunks)), block(kRcThreads);
+#define VAMD_VP(V, W)                                                                                            \
+  hipLaunchKernelGGL((variance_proxy_rows_kernel<V, M, W>), grid, block, 0, s, advantages, old_log_probs,        \
+                     sum_pi_squared, is_weights, mk, batch, length, chunks, records)
+  VAMD_MASK_DISPATCH(mask_dtype, M, {
+    const M* mk = static_cast<const M*>(mask);
+    const bool vec = can_vectorize(length, {advantages, old_log_probs, sum_pi_squared, is_weights}, mask, sizeof(M));
+    if (vec) { if (is_weights) VAMD_VP(true, true); else VAMD_VP(true, false); }
+    else { if (is_weights) VAMD_VP(false, true); else VAMD_VP(false, false); }
+  });
+#undef VAMD_VP
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
+
 
 extern "C" size_t vamd_data_metrics_workspace_bytes(int64_t batch, int64_t response_length) {
   if (batch <= 0 || response_length <= 0) return 0;

@@ -1,5 +1,6 @@
 """``compute_data_metrics`` of the reference (verl/trainer/ppo/metric_utils.py:81-225) as one kernel
-launch and one device-to-host copy instead of ~30 masked reductions with a ``.item()`` each.
+launch and one device-to-host copy instead of ~30 masked reductions with a ``.item()`` each, and
+``compute_variance_proxy_metrics`` (:306-412) as one pass that leaves per-trajectory sums for the host.
 
 ``batch`` is anything shaped like the reference's ``DataProto``: ``batch.batch`` maps names to
 tensors, ``batch.non_tensor_batch`` maps names to numpy arrays.
@@ -9,6 +10,7 @@ from __future__ import annotations
 import math
 from typing import Any
 
+import numpy as np
 import torch
 
 from ... import _cabi
@@ -83,3 +85,54 @@ def compute_data_metrics(batch, use_critic: bool = True) -> dict[str, Any]:
             metrics[f"{label}/max"] = extra[name].max()
             metrics[f"{label}/mean"] = extra[name].mean()
     return metrics
+
+
+def compute_variance_proxy_metrics(batch, gradient_norm: float = None) -> dict[str, float]:
+    """Gradient-variance proxies from the score-norm proxy ``W(tau) = sum_t (1 - 2 pi_t + sum pi^2)`` (reference
+    :306-412): ``proxy2_total_power = E[A^2 W]`` with ``A`` the trajectory's mean advantage (with
+    ``rollout_is_weights`` in the batch: ``E[rho^2 A^2 W_original]``), ``proxy1_signal_strength =
+    gradient_norm^2``, ``proxy3_pure_noise = max(0, (proxy2 - proxy1) / (N - 1))``, plus ``expected_a_squared``
+    and ``expected_w``.  Returns ``{}`` unless ``sum_pi_squared``, ``old_log_probs`` and ``advantages`` are in
+    the batch."""
+    b = batch.batch
+    if "sum_pi_squared" not in b or "old_log_probs" not in b or "advantages" not in b:
+        return {}
+    adv_t = b["advantages"]
+    dev = _cabi.compute_device(adv_t, b["response_mask"])
+    adv = _cabi.as_f32(adv_t, dev)
+    if adv.dim() == 1:
+        adv = adv.view(1, -1)
+    lp = _cabi.as_f32(b["old_log_probs"], dev).view(adv.shape)
+    pi2 = _cabi.as_f32(b["sum_pi_squared"], dev).view(adv.shape)
+    isw = _cabi.as_f32(b["rollout_is_weights"], dev).view(adv.shape) if "rollout_is_weights" in b else None
+    mask, code = _cabi.mask_code(b["response_mask"].detach().to(dev))
+    rows, cols = adv.shape
+    Lb = _cabi.lib()
+    chunks = int(Lb.vamd_rollout_rs_chunks(cols))
+    rec = torch.empty(5 * chunks * rows, dtype=torch.float64, device=dev)
+    with torch.cuda.device(dev):
+        _cabi.check(Lb.vamd_variance_proxy_rows(adv.data_ptr(), lp.data_ptr(), pi2.data_ptr(), _cabi.ptr(isw),
+                                                mask.data_ptr(), code, rows, cols, rec.data_ptr(),
+                                                _cabi.stream_ptr(dev)))
+    t = rec.cpu().numpy().reshape(5, chunks, rows).sum(axis=1)      # the one host sync
+    f32 = np.float32
+    n = t[0].astype(f32) + f32(1e-8)                                # masked_mean's denominator
+    a = t[1].astype(f32) / n
+    w_sum = t[2].astype(f32)
+    proxy1 = gradient_norm**2 if gradient_norm is not None else None
+    if isw is not None:
+        rho = t[3].astype(f32) / n
+        proxy2 = float((rho**2 * a**2 * np.maximum(t[4].astype(f32), 0)).mean())
+    else:
+        proxy2 = float((a**2 * np.maximum(w_sum, 0)).mean())
+    proxy3 = None
+    if proxy1 is not None and rows > 1:
+        proxy3 = max(0.0, (proxy2 - proxy1) / (rows - 1))
+    return {
+        "variance_proxy/proxy1_signal_strength": proxy1 if proxy1 is not None else 0.0,
+        "variance_proxy/proxy2_total_power": proxy2,
+        "variance_proxy/proxy3_pure_noise": proxy3 if proxy3 is not None else 0.0,
+        "variance_proxy/expected_a_squared": float((a**2).mean()),
+        "variance_proxy/expected_w": float(w_sum.mean()),
+    }
+

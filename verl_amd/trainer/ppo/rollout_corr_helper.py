@@ -355,3 +355,29 @@ def compute_rollout_rejection_mask(log_ratio: torch.Tensor, response_mask: torch
     multiply.  Returns ``(modified_response_mask, metrics)`` with the reference's ``rollout_rs_*`` metric names."""
     return _rejection(log_ratio, torch.zeros_like(log_ratio), response_mask, rollout_rs, rollout_rs_threshold)
 
+
+def compute_rollout_correction_and_add_to_batch(batch, rollout_corr_config):
+    """Run the rollout correction on ``batch.batch["old_log_probs" / "rollout_log_probs" / "response_mask"]``
+    with the settings of ``rollout_corr_config`` (``rollout_is``, ``rollout_is_threshold``,
+    ``rollout_is_batch_normalize``, ``rollout_rs``, ``rollout_rs_threshold``): ``response_mask`` is always
+    replaced by the mask after rejection, ``rollout_is_weights`` is added when ``rollout_is`` is set
+    (reference :940-994).  Returns ``(batch, metrics)``."""
+    proto, modified_response_mask, metrics = compute_rollout_correction_and_rejection_mask(
+        old_log_prob=batch.batch["old_log_probs"], rollout_log_prob=batch.batch["rollout_log_probs"],
+        response_mask=batch.batch["response_mask"], rollout_is=rollout_corr_config.get("rollout_is", None),
+        rollout_is_threshold=rollout_corr_config.get("rollout_is_threshold", 2.0),
+        rollout_is_batch_normalize=rollout_corr_config.get("rollout_is_batch_normalize", False),
+        rollout_rs=rollout_corr_config.get("rollout_rs", None),
+        rollout_rs_threshold=rollout_corr_config.get("rollout_rs_threshold", None))
+    batch.batch["response_mask"] = modified_response_mask
+    if proto is not None:
+        batch.batch["rollout_is_weights"] = proto.batch["rollout_is_weights"]
+    return batch, metrics
+
+
+def compute_rollout_corr_metrics_from_logprobs(log_prob: torch.Tensor, rollout_log_prob: torch.Tensor,
+                                               response_mask: torch.Tensor) -> dict[str, float]:
+    """The off-policy diagnostics of the current policy against the rollout policy, with the ``rollout_corr/``
+    prefix (reference :997-1031)."""
+    return {f"rollout_corr/{k}": v for k, v in compute_offpolicy_metrics(log_prob, rollout_log_prob, response_mask).items()}
+
