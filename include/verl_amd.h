@@ -386,6 +386,24 @@ int vamd_policy_loss_variant_forward(int variant, const float* old_log_prob, con
                                      double dp_size, double batch_num_tokens, double global_batch_size,
                                      double loss_scale_factor, float* out, float* grad_unscaled, float* coef_out,
                                      void* workspace, size_t workspace_bytes, void* stream);
+/* The two covariance-based policy losses.  kind 0 = KL-Cov (core_algos.py:1555-1632): -A ratio everywhere plus
+ * ppo_kl_coef |log ratio| on the max(1, int(n select_ratio)) valid tokens with the largest covariance
+ * (A - mean A)(log_prob - mean log_prob); out[2] is masked_mean(|log ratio|).  kind 1 = Clip-Cov (:1450-1552): the
+ * clipped surrogate (clip_low / clip_high) with min(max(int(select_ratio sum(mask)), 1), #candidates) tokens, drawn
+ * uniformly at random (seed) from the valid, unclipped tokens whose covariance lies strictly inside
+ * (cov_lb, cov_ub), contributing neither loss nor gradient; out[1] is their share of the valid tokens, out[2]
+ * masked_mean(-log ratio).  out[0] = loss, out[3] = 0.  selected_out (optional, rows * cols bytes) receives 1 for
+ * the selected tokens.  grad_unscaled / coef_out and the agg_loss scalars as for vamd_policy_loss_forward.  The
+ * workspace is plain scratch (no arrival counters); tokens whose selection key equals the threshold exactly share
+ * the remaining places in arrival order. */
+size_t vamd_policy_loss_cov_workspace_bytes(int64_t rows, int64_t cols);
+int vamd_policy_loss_cov_forward(int kind, const float* old_log_prob, const float* log_prob, const float* advantages,
+                                 const void* mask, int mask_dtype, const float* is_weights, int64_t rows,
+                                 int64_t cols, float clip_low, float clip_high, float cov_lb, float cov_ub,
+                                 double select_ratio, float ppo_kl_coef, uint64_t seed, int mode, double dp_size,
+                                 double batch_num_tokens, double global_batch_size, double loss_scale_factor,
+                                 float* out, float* grad_unscaled, float* coef_out, uint8_t* selected_out,
+                                 void* workspace, size_t workspace_bytes, void* stream);
 int vamd_scale_rows(const float* g, const float* coef, const float* d_loss, float extra_scale, int64_t rows,
                     int64_t cols, float* out, void* stream);
 

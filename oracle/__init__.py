@@ -66,6 +66,9 @@ from .losses import (  # noqa: F401
     policy_loss_cispo,
     policy_loss_reinforce,
     policy_loss_geo_mean,
+    policy_loss_kl_cov,
+    policy_loss_clip_cov,
+    clip_cov_candidates,
 )
 from .trainer import (  # noqa: F401
     apply_kl_penalty,

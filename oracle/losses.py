@@ -207,3 +207,73 @@ def policy_loss_geo_mean(old_log_prob, log_prob, advantages, response_mask, clip
     clipped = torch.ne(x, clamped)
     return (torch.mean(losses), masked_mean((clipped * (advantages > 0)).float(), response_mask),
             masked_mean(-x, response_mask), masked_mean((clipped * (advantages < 0)).float(), response_mask))
+
+
+def policy_loss_kl_cov(old_log_prob, log_prob, advantages, response_mask, loss_agg_mode="token-mean",
+                       kl_cov_ratio=0.0002, ppo_kl_coef=1.0, rollout_is_weights=None, global_batch_info=None):
+    """KL-Cov, verl/trainer/ppo/core_algos.py:1555-1632: the unclipped surrogate ``-A ratio`` everywhere, plus
+    ``ppo_kl_coef |log ratio|`` on the ``max(1, int(n kl_cov_ratio))`` valid tokens with the largest covariance
+    ``(A - mean A)(log_prob - mean log_prob)`` (plain means over the valid tokens).  Returns
+    ``(pg_loss, ppo_kl_abs, selected)`` with ``selected`` the boolean matrix of penalised tokens."""
+    x = log_prob - old_log_prob
+    ratio = torch.exp(x)
+    base = -advantages * ratio
+    with_kl = base + ppo_kl_coef * x.abs()
+    valid = response_mask > 0
+    selected = torch.zeros_like(valid)
+    adv_v = advantages[valid].detach().reshape(-1)
+    lp_v = log_prob[valid].detach().reshape(-1)
+    if min(kl_cov_ratio, adv_v.numel()) != 0:
+        cov = (adv_v - adv_v.mean()) * (lp_v - lp_v.mean())
+        k = max(1, int(cov.numel() * kl_cov_ratio))
+        top = torch.topk(cov, k, largest=True).indices
+        flat = torch.nonzero(valid.reshape(-1), as_tuple=True)[0][top]
+        selected.view(-1)[flat] = True
+    losses = torch.where(selected, with_kl, base)
+    if rollout_is_weights is not None:
+        losses = losses * rollout_is_weights
+    pg_loss = agg_loss(losses, response_mask, loss_agg_mode, **(global_batch_info or {}))
+    return pg_loss, masked_mean(x.abs(), response_mask), selected
+
+
+def clip_cov_candidates(old_log_prob, log_prob, advantages, response_mask, clip_ratio_low, clip_ratio_high,
+                        clip_cov_lb=1.0, clip_cov_ub=5.0, clip_cov_ratio=0.0002):
+    """The deterministic part of Clip-Cov's selection, core_algos.py:1502-1516: ``(candidates, clip_num)`` with
+    ``candidates`` the valid, not already clipped tokens whose covariance ``(A - masked_mean A)(log_prob -
+    masked_mean log_prob)`` lies strictly between the two bounds, and ``clip_num = max(int(ratio M), 1)``."""
+    ratio = torch.exp(log_prob - old_log_prob)
+    l1 = -advantages * ratio
+    l2 = -advantages * torch.clamp(ratio, 1 - clip_ratio_low, 1 + clip_ratio_high)
+    clipped = (l2 > l1) & (response_mask > 0)
+    cov = (advantages - masked_mean(advantages, response_mask)) * (log_prob - masked_mean(log_prob.detach(), response_mask))
+    cov = cov.detach().clone()
+    cov[response_mask == 0] = -torch.inf
+    cov[clipped] = -torch.inf
+    clip_num = max(int(clip_cov_ratio * response_mask.sum().item()), 1)
+    return (cov < clip_cov_ub) & (cov > clip_cov_lb) & (response_mask > 0), clip_num
+
+
+def policy_loss_clip_cov(old_log_prob, log_prob, advantages, response_mask, loss_agg_mode="token-mean",
+                         clip_ratio_low=0.2, clip_ratio_high=0.2, clip_cov_lb=1.0, clip_cov_ub=5.0,
+                         clip_cov_ratio=0.0002, rollout_is_weights=None, global_batch_info=None, dropped=None):
+    """Clip-Cov, core_algos.py:1450-1552: the clipped surrogate, with ``min(clip_num, #candidates)`` of the
+    candidates above, drawn uniformly at random, contributing neither loss nor gradient.  ``dropped`` (a boolean
+    matrix) replaces the random draw.  Returns ``(pg_loss, pg_clipfrac, ppo_kl, dropped)``."""
+    x = log_prob - old_log_prob
+    ratio = torch.exp(x)
+    l1 = -advantages * ratio
+    l2 = -advantages * torch.clamp(ratio, 1 - clip_ratio_low, 1 + clip_ratio_high)
+    if dropped is None:
+        cand, clip_num = clip_cov_candidates(old_log_prob, log_prob, advantages, response_mask, clip_ratio_low,
+                                             clip_ratio_high, clip_cov_lb, clip_cov_ub, clip_cov_ratio)
+        idx = torch.nonzero(cand)
+        dropped = torch.zeros_like(cand)
+        if len(idx) > 0:
+            idx = idx[torch.randperm(len(idx))[: min(clip_num, len(idx))]]
+            dropped[idx[:, 0], idx[:, 1]] = True
+    corr = (~dropped).to(l1.dtype)
+    losses = torch.maximum(l1, l2) * corr
+    if rollout_is_weights is not None:
+        losses = losses * rollout_is_weights
+    pg_loss = agg_loss(losses, response_mask, loss_agg_mode, **(global_batch_info or {}))
+    return pg_loss, masked_mean((corr == 0).float(), response_mask), masked_mean(-x, response_mask), dropped

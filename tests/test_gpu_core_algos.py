@@ -648,6 +648,97 @@ def test_policy_loss_bypass_mode(dev, loss_type, rollout_is, mode):
         CA.compute_policy_loss_bypass_mode(rollout.to(dev), nd, adv.to(dev), mask.to(dev), mode, cfg)
 
 
+def _cov_inputs(B, Lc, seed):
+    g = torch.Generator().manual_seed(seed)
+    mask, _ = _prefix_mask(B, Lc, g, lo=3)
+    mask[1] = 0
+    old = torch.randn(B, Lc, generator=g) * 0.5 - 1
+    new = old + torch.randn(B, Lc, generator=g) * 0.15
+    adv = torch.randn(B, Lc, generator=g)
+    return old, new, adv, mask, torch.rand(B, Lc, generator=g) + 0.5
+
+
+@pytest.mark.parametrize("shape", [(6, 40), (12, 4200), (300, 1024)])
+@pytest.mark.parametrize("mode", ["token-mean", "seq-mean-token-mean"])
+@pytest.mark.parametrize("with_isw", [False, True])
+def test_policy_loss_kl_cov(dev, shape, mode, with_isw):
+    from verl_amd.trainer.ppo import core_algos as CA
+    old, new, adv, mask, isw = _cov_inputs(*shape, seed=shape[1])
+    isw = isw if with_isw else None
+    cfg = _cfg(clip_ratio=0.2)
+    cfg.policy_loss = types.SimpleNamespace(kl_cov_ratio=0.002, ppo_kl_coef=0.7)
+    nd = new.to(dev).requires_grad_(); no = new.clone().requires_grad_()
+    loss, met = CA.compute_policy_loss_kl_cov(old.to(dev), nd, adv.to(dev), mask.to(dev), mode, cfg,
+                                              None if isw is None else isw.to(dev), return_selected=True)
+    want_loss, want_kl, want_sel = O.policy_loss_kl_cov(old, no, adv, mask, mode, 0.002, 0.7, isw)
+    k = max(1, int(mask.sum().item() * 0.002))
+    assert int(want_sel.sum()) == k and torch.equal(met["selected"].cpu(), want_sel), "the top-k tokens differ"
+    _close(loss, want_loss, what="kl_cov loss")
+    assert abs(met["actor/ppo_kl"] - want_kl.item()) < 2e-6 * max(1.0, want_kl.item())
+    _close(torch.autograd.grad(loss, nd)[0], torch.autograd.grad(want_loss, no)[0], atol=1e-9, what="d kl_cov loss")
+    assert CA.get_policy_loss_fn("kl_cov") is CA.compute_policy_loss_kl_cov
+    cfg.policy_loss = {}                                          # defaults: ratio 0.0002 -> at least one token
+    _, met = CA.compute_policy_loss_kl_cov(old.to(dev), new.to(dev), adv.to(dev), mask.to(dev), mode, cfg, return_selected=True)
+    assert int(met["selected"].sum()) == max(1, int(mask.sum().item() * 0.0002))
+
+
+@pytest.mark.parametrize("shape", [(6, 40), (12, 4200), (300, 1024)])
+@pytest.mark.parametrize("mode", ["token-mean", "seq-mean-token-sum"])
+@pytest.mark.parametrize("ratio", [0.01, 1.0])
+def test_policy_loss_clip_cov(dev, shape, mode, ratio):
+    from verl_amd.trainer.ppo import core_algos as CA
+    old, new, adv, mask, isw = _cov_inputs(*shape, seed=shape[0])
+    cfg = _cfg(clip_ratio=0.2, clip_ratio_high=0.25)
+    cfg.policy_loss = types.SimpleNamespace(clip_cov_ratio=ratio, clip_cov_lb=0.02, clip_cov_ub=1.5)
+    cand, clip_num = O.clip_cov_candidates(old, new, adv, mask, 0.2, 0.25, 0.02, 1.5, ratio)
+    nd = new.to(dev).requires_grad_(); no = new.clone().requires_grad_()
+    torch.manual_seed(7)
+    loss, met = CA.compute_policy_loss_clip_cov(old.to(dev), nd, adv.to(dev), mask.to(dev), mode, cfg, isw.to(dev),
+                                                return_selected=True)
+    dropped = met["selected"].cpu()
+    # the draw: the right number of tokens, all of them candidates; with ratio 1 every candidate goes
+    assert int(dropped.sum()) == min(clip_num, int(cand.sum())) and bool(cand[dropped].all())
+    if ratio == 1.0:
+        assert torch.equal(dropped, cand)
+    # given the draw, everything else is deterministic
+    want_loss, want_cf, want_kl, _ = O.policy_loss_clip_cov(old, no, adv, mask, mode, 0.2, 0.25, rollout_is_weights=isw,
+                                                            dropped=dropped)
+    _close(loss, want_loss, what="clip_cov loss")
+    assert abs(met["actor/pg_clipfrac"] - want_cf.item()) < 1e-6
+    assert abs(met["actor/ppo_kl"] - want_kl.item()) < 2e-6 * max(1.0, abs(want_kl.item()))
+    _close(torch.autograd.grad(loss, nd)[0], torch.autograd.grad(want_loss, no)[0], atol=1e-9, what="d clip_cov loss")
+    # the same seed gives the same draw, another seed another one (when there is a choice)
+    torch.manual_seed(7)
+    _, again = CA.compute_policy_loss_clip_cov(old.to(dev), new.to(dev), adv.to(dev), mask.to(dev), mode, cfg, return_selected=True)
+    assert torch.equal(again["selected"].cpu(), dropped)
+    if ratio < 1.0 and int(cand.sum()) > 4 * clip_num:
+        torch.manual_seed(8)
+        _, other = CA.compute_policy_loss_clip_cov(old.to(dev), new.to(dev), adv.to(dev), mask.to(dev), mode, cfg, return_selected=True)
+        assert not torch.equal(other["selected"].cpu(), dropped)
+    assert CA.get_policy_loss_fn("clip_cov") is CA.compute_policy_loss_clip_cov
+
+
+def test_clip_cov_draw_is_uniform(dev):
+    """Every candidate is dropped about equally often over many seeds (chi-square against the uniform law)."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    old, new, adv, mask, _ = _cov_inputs(4, 64, seed=1)
+    cfg = _cfg(clip_ratio=0.2)
+    cfg.policy_loss = types.SimpleNamespace(clip_cov_ratio=0.05, clip_cov_lb=0.0, clip_cov_ub=50.0)
+    cand, clip_num = O.clip_cov_candidates(old, new, adv, mask, 0.2, 0.2, 0.0, 50.0, 0.05)
+    n_cand = int(cand.sum())
+    assert n_cand > 3 * clip_num
+    counts = torch.zeros_like(cand, dtype=torch.float64)
+    trials = 400
+    args = (old.to(dev), new.to(dev), adv.to(dev), mask.to(dev), "token-mean", cfg)
+    for seed in range(trials):
+        torch.manual_seed(seed)
+        counts += CA.compute_policy_loss_clip_cov(*args, return_selected=True)[1]["selected"].cpu().double()
+    assert counts[~cand].sum() == 0
+    expected = trials * clip_num / n_cand
+    chi2 = ((counts[cand] - expected) ** 2 / expected).sum().item()
+    assert chi2 < n_cand + 6 * math.sqrt(2 * n_cand), (chi2, n_cand)      # mean n - 1, std sqrt(2 (n - 1))
+
+
 # ---- KL penalty -------------------------------------------------------------------------------------
 @pytest.mark.parametrize("kind", ["kl", "k1", "abs", "mse", "k2", "low_var_kl", "k3"])
 def test_kl_penalty_elementwise(dev, kind):

@@ -295,3 +295,62 @@ def test_reinforce_and_geo_mean_closed_forms():
     loss, cf, _, cfl = L.policy_loss_geo_mean(old, new.detach(), adv_row, mask, 50.0, 50.0)
     seq = ((new.detach() - old) * mask).sum(-1) / mask.sum(-1)
     assert torch.allclose(loss, (-adv_row[:, 0] * torch.exp(seq)).mean()) and cf.item() == 0 and cfl.item() == 0
+
+
+def test_kl_cov_and_clip_cov_against_scalar_loops():
+    old, new, adv, mask = _policy_inputs(seed=3, B=6, Lc=40)
+    B, Lc = old.shape
+    toks = [(i, t) for i in range(B) for t in range(Lc) if mask[i, t] != 0]
+    n = len(toks)
+    # KL-Cov: 5 % of the valid tokens, those with the largest covariance, carry the extra |log ratio| term
+    loss, kl_abs, selected = L.policy_loss_kl_cov(old, new, adv, mask, "token-mean", kl_cov_ratio=0.05, ppo_kl_coef=0.7)
+    ma = sum(adv[i, t].item() for i, t in toks) / n
+    ml = sum(new[i, t].item() for i, t in toks) / n
+    cov = {(i, t): (adv[i, t].item() - ma) * (new[i, t].item() - ml) for i, t in toks}
+    k = max(1, int(n * 0.05))
+    top = set(sorted(cov, key=cov.get, reverse=True)[:k])
+    assert {(i, t) for i, t in toks if selected[i, t]} == top and int(selected.sum()) == k
+    total = 0.0
+    for i, t in toks:
+        x = (new[i, t] - old[i, t]).item()
+        total += -adv[i, t].item() * math.exp(x) + (0.7 * abs(x) if (i, t) in top else 0.0)
+    assert loss.item() == pytest.approx(total / n, rel=1e-9)
+    assert kl_abs.item() == pytest.approx(sum(abs((new[i, t] - old[i, t]).item()) for i, t in toks) / n, rel=1e-7)
+    g, = torch.autograd.grad(loss, new)
+    i, t = next(iter(top))
+    x = (new[i, t] - old[i, t]).item()
+    assert g[i, t].item() == pytest.approx((-adv[i, t].item() * math.exp(x) + 0.7 * math.copysign(1, x)) / n, rel=1e-7)
+    assert L.policy_loss_kl_cov(old, new.detach(), adv, mask, kl_cov_ratio=1e-9)[2].sum() == 1       # at least one token
+
+    # Clip-Cov: the candidate band and clip_num by loops; the draw replaced by a fixed choice
+    cand, clip_num = L.clip_cov_candidates(old, new.detach(), adv, mask, 0.2, 0.25, clip_cov_lb=0.05, clip_cov_ub=2.0,
+                                           clip_cov_ratio=0.02)
+    want = set()
+    for i, t in toks:
+        r = math.exp((new[i, t] - old[i, t]).item())
+        a = adv[i, t].item()
+        clipped = -a * min(max(r, 0.8), 1.25) > -a * r
+        if not clipped and 0.05 < cov[(i, t)] < 2.0:
+            want.add((i, t))
+    # masked_mean adds 1e-8 to the count: the covariances agree to ~1e-9, the band membership exactly for this data
+    assert {(i, t) for i, t in toks if cand[i, t]} == want and clip_num == max(int(0.02 * n), 1)
+    dropped = torch.zeros_like(cand)
+    for i, t in list(want)[:clip_num]:
+        dropped[i, t] = True
+    loss, cf, kl, _ = L.policy_loss_clip_cov(old, new, adv, mask, "token-mean", 0.2, 0.25, dropped=dropped)
+    total = 0.0
+    for i, t in toks:
+        if dropped[i, t]:
+            continue
+        r = math.exp((new[i, t] - old[i, t]).item())
+        a = adv[i, t].item()
+        total += max(-a * r, -a * min(max(r, 0.8), 1.25))
+    assert loss.item() == pytest.approx(total / n, rel=1e-9)
+    assert cf.item() == pytest.approx(int(dropped.sum()) / n, rel=1e-6)
+    g, = torch.autograd.grad(loss, new)
+    assert (g[dropped] == 0).all()
+    # the random draw picks clip_num candidates, all inside the band
+    torch.manual_seed(0)
+    _, cf2, _, drawn = L.policy_loss_clip_cov(old, new.detach(), adv, mask, "token-mean", 0.2, 0.25, clip_cov_lb=0.05,
+                                              clip_cov_ub=2.0, clip_cov_ratio=0.02)
+    assert int(drawn.sum()) == min(clip_num, len(want)) and (cand[drawn]).all()

@@ -8,7 +8,7 @@ from __future__ import annotations
 import ctypes
 import os
 import threading
-from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_uint64, c_void_p
 
 import torch
 
@@ -69,6 +69,11 @@ SIGNATURES = {
                                              c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "vamd_response_window_gather": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
                                             c_void_p, c_void_p, c_void_p]),
+    "vamd_policy_loss_cov_workspace_bytes": (c_size_t, [c_int64, c_int64]),
+    "vamd_policy_loss_cov_forward": (c_int, [c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64,
+                                             c_int64, c_float, c_float, c_float, c_float, c_double, c_float, c_uint64,
+                                             c_int, c_double, c_double, c_double, c_double, c_void_p, c_void_p,
+                                             c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "vamd_variance_proxy_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
                                          c_void_p, c_void_p]),
     "vamd_rollout_rs_chunks": (c_int64, [c_int64]),

@@ -277,6 +277,16 @@ struct AggParams {
   double dp_size, batch_num_tokens, global_batch_size, loss_scale_factor;  // < 0 : None
 };
 
+inline AggParams make_agg_params(int mode, double dp, double bnt, double gbs, double lsf) {
+  AggParams a;
+  a.mode = mode;
+  a.dp_size = dp;
+  a.batch_num_tokens = bnt;
+  a.global_batch_size = gbs;
+  a.loss_scale_factor = lsf;
+  return a;
+}
+
 // Called by ONE workgroup of NT threads (the last one of the launch to arrive, or a launch of its own).  partials: slot-major records (record_at) with slot 0 =
 // sum(loss * w) and slot 1 = sum(w); slots >= 2 are summed over everything into extra[].
 // Writes loss (double, thread 0) and coef[rows].
@@ -377,6 +387,42 @@ __device__ void finalize_agg(const double* __restrict__ partials, int64_t rows, 
   msum_out = Msum;
 #pragma unroll
   for (int i = 2; i < NV; ++i) extra[i - 2] = bc[i];
+}
+
+// =============================================================================================
+// Folding the (row, chunk) records of the loss kernels.  Small launches let the workgroup that arrives last
+// do it (one launch in all); large ones leave it to a launch of its own: the fold's registers would otherwise
+// be charged to every wavefront of the streaming kernel and halve its occupancy.
+// =============================================================================================
+constexpr int kFoldThreads = 512;
+constexpr int64_t kInlineFoldRecords = 2048;  // up to this many (row, chunk) records the last workgroup folds
+
+enum { kEpiAgg, kEpiPolicy, kEpiValue, kEpiKl };
+
+template <int EPI, int NX>
+__device__ __forceinline__ void loss_epilogue(double loss, double msum, const double (&extra)[NX], float* __restrict__ out) {
+  const float denom = (float)msum + 1e-8f;  // masked_mean's denominator
+  if (EPI == kEpiPolicy) {
+    out[0] = (float)loss;
+    out[1] = (float)extra[1] / denom;  // pg_clipfrac
+    out[2] = (float)extra[0] / denom;  // ppo_kl
+    out[3] = (float)extra[NX > 2 ? 2 : 0] / denom;  // pg_clipfrac_lower
+  } else if (EPI == kEpiValue) {
+    out[0] = 0.5f * (float)loss;
+    out[1] = (float)extra[0] / denom;
+  } else {
+    out[0] = (float)loss;
+  }
+}
+
+template <int NV, int EPI>
+__global__ __launch_bounds__(kFoldThreads) void fold_loss_kernel(const double* __restrict__ records, int64_t rows,
+                                                                 int chunks, int64_t cols, AggParams ap,
+                                                                 float* __restrict__ coef, float* __restrict__ out) {
+  __shared__ double smem[(NV + 3) * (kFoldThreads / 64)];
+  double loss, msum, extra[NV > 2 ? NV - 2 : 1];
+  finalize_agg<NV, kFoldThreads, false>(records, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
+  if (threadIdx.x == 0) loss_epilogue<EPI>(loss, msum, extra, out);
 }
 
 }  // namespace vamd

@@ -671,6 +671,134 @@ def compute_policy_loss_cispo(old_log_prob: torch.Tensor, log_prob: torch.Tensor
                                 rollout_is_weights)
 
 
+class _CovLoss(torch.autograd.Function):
+    """The two covariance-selected losses (``vamd_policy_loss_cov_forward``)."""
+
+    @staticmethod
+    def forward(ctx, log_prob, old_log_prob, advantages, response_mask, is_weights, kind, clip_low, clip_high, cov_lb,
+                cov_ub, ratio, kl_coef, seed, mode, dp_size, bnt, gbs, lsf, want_selected):
+        dev = _cabi.compute_device(log_prob, old_log_prob, advantages, response_mask)
+        lp = _matrix(log_prob, dev)
+        old = _matrix(old_log_prob, dev)
+        adv = _matrix(advantages, dev)
+        assert lp.shape == old.shape == adv.shape
+        m, code = _mask_matrix(response_mask, dev, lp.shape)
+        isw = _matrix(is_weights, dev) if is_weights is not None else None
+        rows, cols = lp.shape
+        need_grad = ctx.needs_input_grad[0]
+        Lb = _cabi.lib()
+        out = torch.empty(4, dtype=torch.float32, device=dev)
+        coef = torch.empty(rows, dtype=torch.float32, device=dev)
+        g = torch.empty_like(lp) if need_grad else None
+        selected = torch.empty((rows, cols), dtype=torch.uint8, device=dev) if want_selected else None
+        ws = _cabi.workspace(Lb.vamd_policy_loss_cov_workspace_bytes(rows, cols), dev)
+        with torch.cuda.device(dev):
+            _cabi.check(Lb.vamd_policy_loss_cov_forward(kind, old.data_ptr(), lp.data_ptr(), adv.data_ptr(),
+                                                        m.data_ptr(), code, _cabi.ptr(isw), rows, cols, clip_low,
+                                                        clip_high, cov_lb, cov_ub, ratio, kl_coef, seed, mode,
+                                                        dp_size, bnt, gbs, lsf, out.data_ptr(), _cabi.ptr(g),
+                                                        coef.data_ptr(), _cabi.ptr(selected), ws.data_ptr(),
+                                                        ws.numel(), _cabi.stream_ptr(dev)))
+        if need_grad:
+            ctx.save_for_backward(g, coef)
+        ctx.in_shape = log_prob.shape
+        ctx.in_device = log_prob.device
+        ctx.in_dtype = log_prob.dtype
+        out = out.to(log_prob.device)
+        if selected is None:
+            selected = torch.empty(0, dtype=torch.uint8, device=log_prob.device)
+        else:
+            selected = selected.view(log_prob.shape).to(log_prob.device)
+        ctx.mark_non_differentiable(out, selected)
+        return out[0].clone(), out, selected
+
+    @staticmethod
+    def backward(ctx, d_loss, _d_out, _d_sel):
+        g, coef = ctx.saved_tensors
+        dev = g.device
+        rows, cols = g.shape
+        d = _cabi.as_f32(d_loss, dev).reshape(1)
+        res = torch.empty_like(g)
+        with torch.cuda.device(dev):
+            _cabi.check(_cabi.lib().vamd_scale_rows(g.data_ptr(), coef.data_ptr(), d.data_ptr(), 1.0, rows, cols,
+                                                    res.data_ptr(), _cabi.stream_ptr(dev)))
+        return (res.view(ctx.in_shape).to(device=ctx.in_device, dtype=ctx.in_dtype),) + (None,) * 18
+
+
+def _policy_loss_option(config, name, default):
+    """``config.policy_loss.<name>`` (attribute or mapping), ``default`` when absent or ``None``."""
+    pl = config.policy_loss
+    value = pl.get(name, None) if isinstance(pl, dict) else getattr(pl, name, None)
+    return default if value is None else value
+
+
+def _cov_loss(kind, old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, config, rollout_is_weights,
+              clip_low, clip_high, cov_lb, cov_ub, ratio, kl_coef, return_selected):
+    info = dict(getattr(config, "global_batch_info", None) or {})
+    # the draw of Clip-Cov follows torch's generator, so torch.manual_seed makes a step reproducible
+    seed = int(torch.randint(0, 2**62, (1,)).item()) if kind == 1 else 0
+    pg_loss, out, selected = _CovLoss.apply(
+        log_prob, old_log_prob, advantages, response_mask, rollout_is_weights, kind, float(clip_low), float(clip_high),
+        float(cov_lb), float(cov_ub), float(ratio), float(kl_coef), seed, _agg_mode(loss_agg_mode),
+        float(info.get("dp_size", 1)), _opt(info.get("batch_num_tokens")), _opt(info.get("global_batch_size")),
+        _opt(info.get("loss_scale_factor")), bool(return_selected))
+    return pg_loss, out.detach().tolist(), selected
+
+
+@register_policy_loss("clip_cov")
+def compute_policy_loss_clip_cov(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                                 response_mask: torch.Tensor, loss_agg_mode: str = "token-mean",
+                                 config: Optional[Any] = None, rollout_is_weights: torch.Tensor | None = None,
+                                 return_selected: bool = False):
+    """Clip-Cov (reference core_algos.py:1450-1552): the clipped surrogate, except that
+    ``min(max(int(clip_cov_ratio * sum(mask)), 1), #candidates)`` tokens drawn uniformly at random from the valid,
+    not already clipped tokens whose covariance ``(A - masked_mean A)(log_prob - masked_mean log_prob)`` lies
+    strictly between ``clip_cov_lb`` and ``clip_cov_ub`` contribute neither loss nor gradient;
+    ``actor/pg_clipfrac`` is their share of the valid tokens.  ``config.policy_loss`` supplies ``clip_cov_ratio``
+    (0.0002), ``clip_cov_lb`` (1.0), ``clip_cov_ub`` (5.0).  The draw is made on the device from a seed taken from
+    torch's default generator; with ``return_selected=True`` the metrics carry the boolean matrix of dropped tokens
+    under ``"selected"``."""
+    assert config is not None
+    assert config.policy_loss is not None
+    ratio = _policy_loss_option(config, "clip_cov_ratio", 0.0002)
+    clip_ratio = config.clip_ratio
+    low = getattr(config, "clip_ratio_low", None)
+    high = getattr(config, "clip_ratio_high", None)
+    assert ratio > 0, "clip_ratio should be larger than 0."
+    pg_loss, vals, selected = _cov_loss(1, old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, config,
+                                        rollout_is_weights, low if low is not None else clip_ratio,
+                                        high if high is not None else clip_ratio,
+                                        _policy_loss_option(config, "clip_cov_lb", 1.0),
+                                        _policy_loss_option(config, "clip_cov_ub", 5.0), ratio, 0.0, return_selected)
+    metrics = {"actor/pg_clipfrac": vals[1], "actor/ppo_kl": vals[2]}
+    if return_selected:
+        metrics["selected"] = selected.bool()
+    return pg_loss, metrics
+
+
+@register_policy_loss("kl_cov")
+def compute_policy_loss_kl_cov(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                               response_mask: torch.Tensor, loss_agg_mode: str = "token-mean",
+                               config: Optional[Any] = None, rollout_is_weights: torch.Tensor | None = None,
+                               return_selected: bool = False):
+    """KL-Cov (reference core_algos.py:1555-1632): ``-A ratio`` on every token plus ``ppo_kl_coef |log ratio|`` on
+    the ``max(1, int(n * kl_cov_ratio))`` valid tokens with the largest covariance ``(A - mean A)(log_prob - mean
+    log_prob)``; ``actor/ppo_kl`` is the masked mean of ``|log ratio|``.  ``config.policy_loss`` supplies
+    ``kl_cov_ratio`` (0.0002) and ``ppo_kl_coef`` (1.0).  The top-k runs on the device (the reference moves the
+    valid tokens to the CPU for it)."""
+    assert config is not None
+    assert config.policy_loss is not None
+    ratio = _policy_loss_option(config, "kl_cov_ratio", 0.0002)
+    assert ratio > 0, "kl_cov_ratio should be larger than 0."
+    pg_loss, vals, selected = _cov_loss(0, old_log_prob, log_prob, advantages, response_mask, loss_agg_mode, config,
+                                        rollout_is_weights, 0.0, 0.0, 0.0, 0.0, ratio,
+                                        _policy_loss_option(config, "ppo_kl_coef", 1.0), return_selected)
+    metrics = {"actor/ppo_kl": vals[2]}
+    if return_selected:
+        metrics["selected"] = selected.bool()
+    return pg_loss, metrics
+
+
 @register_policy_loss("geo_mean")
 def compute_policy_loss_geo_mean(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
                                  response_mask: torch.Tensor, loss_agg_mode: str = "token-mean",
