@@ -115,3 +115,78 @@ def test_actor_update_step_matches_the_oracle_composition(dev, mode, on_policy):
         bound = 2.0 ** -8 * ref_g.abs() + (2.0 ** -8 + 1e-2) * e + 1e-9
         assert (err <= bound).all(), f"{name}: worst excess {(err - bound).max().item():.3e}"
         assert err.pow(2).mean().sqrt().item() <= 0.02 * ref_g.pow(2).mean().sqrt().item() + 1e-9, name
+
+
+def test_remove_padding_actor_step_matches_the_oracle_composition(dev):
+    """The remove-padding variant of the step above (verl/workers/actor/dp_actor.py:147-344): the head runs on the
+    attended tokens only, labels are the rolled token stream, and log-prob / entropy / sum of squared probabilities
+    are placed into the response window before the losses."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy, linear_cross_entropy_with_sum_pi_squared
+    from verl_amd.utils.kernel.response_window import pad_to_response_window
+    g = torch.Generator().manual_seed(23)
+    B, P, Lr, H, V, T = 8, 32, 48, 256, 2048, 1.0
+    S = P + Lr
+    prompt_len = torch.randint(4, P + 1, (B,), generator=g)
+    resp_len = torch.randint(6, Lr + 1, (B,), generator=g)
+    pos = torch.arange(S)[None, :]
+    attention = ((pos >= (P - prompt_len)[:, None]) & (pos < (P + resp_len)[:, None])).long()     # left-padded prompts
+    response_mask = attention[:, -Lr:].float()
+    input_ids = torch.randint(0, V, (B, S), generator=g)
+    indices = attention.flatten().nonzero().flatten()
+    ids_rmpad = input_ids.flatten()[indices]
+    labels_rmpad = torch.roll(ids_rmpad, shifts=-1, dims=0)                                      # dp_actor.py:210
+    nnz = indices.numel()
+    hidden = torch.randn(nnz, H, generator=g).bfloat16()
+    weight = (torch.randn(V, H, generator=g) * 0.05).bfloat16()
+    rewards = torch.zeros(B, Lr); rewards[torch.arange(B), resp_len - 1] = torch.rand(B, generator=g)
+    uid = np.repeat(np.arange(B // 4), 4)
+    old_shift = torch.randn(B, Lr, generator=g) * 0.1
+
+    def step(head, window, algos, device):
+        h = hidden.to(device).requires_grad_()
+        w = weight.to(device).requires_grad_()
+        lp_flat, ent_flat = head(h, w, labels_rmpad.to(device))
+        lp, ent = window(lp_flat, ent_flat)
+        m = response_mask.to(device)
+        old = lp.detach() + old_shift.to(device) * m
+        adv, _ = algos["grpo"](rewards.to(device), m, uid)
+        pg_loss = algos["policy"](old, lp, adv, m)
+        loss = pg_loss - 0.01 * algos["agg"](ent, m)
+        loss.backward()
+        return dict(lp=lp.detach(), ent=ent.detach(), loss=loss.detach(), dh=h.grad, dw=w.grad)
+
+    cfg = _cfg()
+    got = step(lambda h, w, y: linear_cross_entropy(h, w, y, T),
+               lambda a, b: pad_to_response_window(indices.to(dev), B, S, Lr, a, b),
+               dict(grpo=CA.compute_grpo_outcome_advantage,
+                    policy=lambda old, lp, adv, m: CA.compute_policy_loss_vanilla(old, lp, adv, m, "token-mean", cfg)[0],
+                    agg=lambda x, m: CA.agg_loss(x, m, "token-mean")), dev)
+    kept = {}
+
+    def oracle_head(h, w, y):
+        lp, ent = O.head_fp32_ground_truth(h, w, y, T)
+        lp.retain_grad(); ent.retain_grad()
+        kept["lp"], kept["ent"] = lp, ent
+        return lp, ent
+
+    want = step(oracle_head,
+                lambda a, b: (O.pad_to_response_window(a, indices, B, S, Lr), O.pad_to_response_window(b, indices, B, S, Lr)),
+                dict(grpo=lambda r, m, i: O.grpo_outcome_advantage(r.clone(), m, i),
+                     policy=lambda old, lp, adv, m: O.policy_loss_vanilla(old, lp, adv, m, "token-mean")[0],
+                     agg=lambda x, m: O.agg_loss(x, m, "token-mean")), "cpu")
+    assert (got["lp"].cpu() - want["lp"]).abs().max().item() <= 2e-3
+    assert (got["ent"].cpu() - want["ent"]).abs().max().item() <= 2e-3
+    assert torch.equal(got["lp"].cpu()[response_mask == 0] == 0, want["lp"][response_mask == 0] == 0)
+    assert abs(got["loss"].item() - want["loss"].item()) <= 4e-3
+    _, _, ref_dh, ref_dw, e_dh, e_dw = O.head_fwd_bwd_chunked_fp32(hidden, weight, labels_rmpad, T, kept["lp"].grad, kept["ent"].grad)
+    for name, got_g, ref_g, e in (("d_hidden", got["dh"], ref_dh, e_dh), ("d_weight", got["dw"], ref_dw, e_dw)):
+        err = (got_g.float().cpu() - ref_g).abs()
+        bound = 2.0 ** -8 * ref_g.abs() + (2.0 ** -8 + 1e-2) * e + 1e-9
+        assert (err <= bound).all(), f"{name}: worst excess {(err - bound).max().item():.3e}"
+    # the third per-token output rides along in the same launch
+    lp3, ent3, pi2 = linear_cross_entropy_with_sum_pi_squared(hidden.to(dev), weight.to(dev), labels_rmpad.to(dev), T)
+    a, b, c = pad_to_response_window(indices.to(dev), B, S, Lr, lp3, ent3, pi2)
+    logits = hidden.float() @ weight.float().t()
+    want_pi2 = O.pad_to_response_window(O.sum_pi_squared_from_logits(logits), indices, B, S, Lr)
+    assert (c.cpu() - want_pi2).abs().max().item() <= 2e-3 and torch.equal(a.cpu(), got["lp"].cpu())
