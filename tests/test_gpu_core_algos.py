@@ -1279,3 +1279,63 @@ def test_rollout_correction_batch_entry_points(dev):
     for k, v in want.items():
         assert got[f"rollout_corr/{k}"] == pytest.approx(v, rel=1e-4, abs=1e-6), k
 
+
+def test_widened_entry_points_at_benchmark_size_properties(dev):
+    """B = 512, L = 4096 (the size of the policy-math benchmark configurations): properties that need no oracle."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.trainer.ppo import rollout_corr_helper as RC
+    from verl_amd.trainer.ppo.metric_utils import compute_data_metrics
+    B, Lc, n = 512, 4096, 8
+    g = torch.Generator(device=dev).manual_seed(0)
+    lens = torch.randint(64, Lc + 1, (B,), device=dev, generator=g)
+    mask = (torch.arange(Lc, device=dev)[None, :] < lens[:, None]).float()
+    uid = np.repeat(np.arange(B // n), n)
+    pi = torch.rand(B, Lc, device=dev, generator=g).clamp_min(1e-4)
+    pi2 = pi * pi + torch.rand(B, Lc, device=dev, generator=g) * (1 - pi) ** 2
+    rewards = torch.randn(B, Lc, device=dev, generator=g)
+    # optimal token baseline: with prefix masks the packed variant is the plain one; identical members of a group
+    # are their own baseline; the advantages of a group add up to zero under the weights W
+    a1, r1 = CA.compute_optimal_token_baseline_advantage(rewards, mask, uid, pi.log(), pi2)
+    a2, r2 = CA.compute_multi_turn_optimal_token_baseline_advantage(rewards, mask, uid, pi.log(), pi2, handle_zero_tail=False)
+    assert torch.equal(r1, r2) and torch.allclose(a1, a2, rtol=1e-6, atol=1e-6)
+    same = lambda x: x[::n].repeat_interleave(n, dim=0)          # every member of a group a copy of the first
+    a3, r3 = CA.compute_optimal_token_baseline_advantage(same(rewards), same(mask), uid, same(pi.log()), same(pi2))
+    assert a3.abs().max().item() <= 1e-4 * r3.abs().max().item()
+    W = ((1 - 2 * pi + pi2) * mask).cumsum(-1)
+    weighted = (a1 * W * mask).view(B // n, n, Lc).sum(1)
+    assert weighted.abs().max().item() <= 1e-3 * (r1.abs() * W).max().item()
+    # rollout correction: identical policies are neutral; infinite thresholds reject nothing; tight ones everything
+    lp = pi.log()
+    proto, new, m = RC.compute_rollout_correction_and_rejection_mask(lp, lp.clone(), mask, rollout_is="sequence",
+                                                                     rollout_is_threshold=2.0, rollout_rs="token_k3,seq_max_k2",
+                                                                     rollout_rs_threshold="1e9,1e9")
+    assert torch.equal(proto.batch["rollout_is_weights"], mask) and torch.equal(new, mask)
+    for key in ("kl", "k3_kl", "chi2_token", "chi2_seq", "rollout_rs_masked_fraction"):
+        assert abs(m["rollout_corr/" + key]) < 1e-6, key
+    assert m["rollout_corr/rollout_is_eff_sample_size"] == pytest.approx(1.0, abs=1e-6)
+    _, new, m = RC.compute_rollout_correction_and_rejection_mask(lp, lp + 0.5, mask, rollout_rs="seq_mean_k2", rollout_rs_threshold=0.1)
+    assert int(new.sum()) == 0 and m["rollout_corr/rollout_rs_masked_fraction"] == pytest.approx(1.0)
+    assert m["rollout_corr/rollout_rs_seq_mean_k2_mean"] == pytest.approx(0.125, rel=1e-5)
+    # KL-penalised rewards: linear in beta, and beta = 0 returns the scores
+    r0, kl0 = CA.kl_penalised_rewards(rewards, lp, lp - 0.3, mask, 0.0, "mse")
+    rb, klb = CA.kl_penalised_rewards(rewards, lp, lp - 0.3, mask, 0.2, "mse")
+    assert torch.equal(r0, rewards) and kl0.item() == pytest.approx(0.045, rel=1e-5) and klb.item() == kl0.item()
+    assert torch.allclose(rb, rewards - 0.2 * 0.045 * mask, rtol=1e-6, atol=1e-6)
+    # data metrics: lengths are exact counts; the score statistics of a constant tensor are that constant times L
+    attention = torch.cat([torch.ones(B, 16, device=dev), mask], 1).long()
+    dm = compute_data_metrics(_data(dict(token_level_scores=torch.full((B, Lc), 0.5, device=dev), token_level_rewards=rewards,
+                                         advantages=a1, returns=r1, values=r1 - 1.0, responses=torch.zeros(B, Lc),
+                                         attention_mask=attention, response_mask=mask)))
+    assert dm["response_length/mean"] == pytest.approx(lens.float().mean().item(), rel=1e-6)
+    assert dm["response_length/max"] == lens.max().item() and dm["response_length/min"] == lens.min().item()
+    assert dm["prompt_length/mean"] == 16 and dm["prompt_length/clip_ratio"] == 1.0
+    assert dm["critic/score/mean"] == pytest.approx(0.5 * Lc) and dm["critic/score/max"] == 0.5 * Lc
+    assert dm["critic/vf_explained_var"] == pytest.approx(1.0, abs=1e-4)       # returns - values is constant
+    # covariance losses: the number of selected tokens is the rule's, whatever the data
+    cfg = _cfg(clip_ratio=0.2)
+    cfg.policy_loss = {"kl_cov_ratio": 0.0002}
+    _, met = CA.compute_policy_loss_kl_cov(lp, lp + 0.1 * torch.randn(B, Lc, device=dev, generator=g), rewards, mask,
+                                           "token-mean", cfg, return_selected=True)
+    assert int(met["selected"].sum()) == max(1, int(mask.sum().item() * 0.0002))
+    assert not bool(met["selected"][mask == 0].any())
+
