@@ -93,7 +93,8 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
     group_offsets = torch.arange(0, B + 1, B // n_groups, device=dev)
     # scratch without arrival counters (these entry points overwrite all of it)
     ws_otb = torch.empty(max(L.vamd_otb_advantage_workspace_bytes(B, Lc, 0), L.vamd_data_metrics_workspace_bytes(B, Lc),
-                             L.vamd_rollout_correction_workspace_bytes(B, Lc)), dtype=torch.uint8, device=dev)
+                             L.vamd_rollout_correction_workspace_bytes(B, Lc),
+                             L.vamd_policy_loss_cov_workspace_bytes(B, Lc)), dtype=torch.uint8, device=dev)
     metrics = torch.empty(64, dtype=torch.float64, device=dev)
     attention = torch.ones(B, Lc, dtype=torch.int64, device=dev)      # no prompt columns: response part only
     st = _cabi.stream_ptr(dev)
@@ -149,6 +150,11 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
                                                0, 1.0, *none3, out.data_ptr(), *P(s, "o1"), coef.data_ptr(), wsp, wsn,
                                                st))
 
+    def kl_cov(s):
+        chk(L.vamd_policy_loss_cov_forward(0, *P(s, "a", "b", "c", "mask"), 0, None, B, Lc, 0.2, 0.2, 0.0, 0.0, 0.0002,
+                                           1.0, 0, 0, 1.0, *none3, out.data_ptr(), *P(s, "o1"), coef.data_ptr(), None,
+                                           ws_otb.data_ptr(), ws_otb.numel(), st))
+
     def copy(s):
         chk(L.vamd_copy_bytes(*P(s, "a", "o1"), 4 * BL, st))
 
@@ -166,6 +172,7 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
         "data_metrics": (24 * BL + 8 * BL, data_metrics),     # six fp32 tensors and the int64 attention mask
         "rollout_correction_token": (16 * BL, rollout_corr),
         "policy_loss_geo_mean_fwd_grad": (20 * BL, geo_mean),  # two passes over the inputs; one is the minimum
+        "policy_loss_kl_cov_fwd_grad": (20 * BL, kl_cov),      # statistics, keys, 3 histogram passes, loss: 12 launches
         "copy_yardstick": (8 * BL, copy),
     }
     res = {}
