@@ -210,6 +210,63 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
     return res
 
 
+def policy_math_chain(dev, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> dict:
+    """GRPO advantage -> policy loss with gradient -> GAE -> value loss with gradient, the per-step chain of the two
+    policy-math benchmark configurations, launched eagerly and replayed from one captured HIP graph (microseconds
+    per chain, best of three loops of 50)."""
+    import torch
+
+    from verl_amd import _cabi
+
+    L = _cabi.lib()
+    g = torch.Generator(device=dev).manual_seed(0)
+    f = lambda: torch.randn(B, Lc, device=dev, generator=g)
+    lens = torch.randint(64, Lc + 1, (B,), device=dev, generator=g)
+    mask = (torch.arange(Lc, device=dev)[None, :] < lens[:, None]).float()
+    rewards, old, values = f(), f() * 0.5 - 1, f()
+    new, vpreds = old + 0.05 * f(), values + 0.5 * f()
+    adv, grad, gae_adv, gae_ret, vgrad = (torch.empty(B, Lc, device=dev) for _ in range(5))
+    out, coef, mom = torch.empty(4, device=dev), torch.empty(B, device=dev), torch.empty(4, dtype=torch.float64, device=dev)
+    gid = torch.arange(n_groups, device=dev).repeat_interleave(B // n_groups)
+    ws = torch.zeros(max(1 << 22, L.vamd_group_outcome_advantage_workspace_bytes(B, Lc, n_groups),
+                         L.vamd_policy_loss_variant_workspace_bytes(B, Lc)), dtype=torch.uint8, device=dev)
+    chk, P = _cabi.check, (lambda t: t.data_ptr())
+
+    def chain():
+        st = _cabi.stream_ptr(dev)
+        chk(L.vamd_grpo_advantage(P(rewards), P(mask), 0, P(gid), B, Lc, n_groups, 1e-6, 1, 0, P(adv), None, P(ws),
+                                  ws.numel(), st))
+        chk(L.vamd_policy_loss_forward(P(old), P(new), P(adv), P(mask), 0, None, B, Lc, 0.2, 0.2, 3.0, 0, 1.0, -1.0, -1.0,
+                                       -1.0, P(out), P(grad), P(coef), P(ws), ws.numel(), st))
+        chk(L.vamd_gae(P(rewards), P(values), P(mask), 0, B, Lc, 1.0, 0.95, 1, P(gae_adv), P(gae_ret), P(mom), P(ws),
+                       ws.numel(), st))
+        chk(L.vamd_value_loss_forward(P(vpreds), P(gae_ret), P(values), P(mask), 0, B, Lc, 0.5, 0, P(out), P(vgrad),
+                                      P(coef), P(ws), ws.numel(), st))
+
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        chain()
+    torch.cuda.current_stream(dev).wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        chain()
+
+    def timed(fn, reps=50):
+        best = float("inf")
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) / reps * 1e3)
+        return best
+
+    return {"launches_per_chain": 6, "eager_us": timed(chain), "hip_graph_us": timed(graph.replay)}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -303,6 +360,7 @@ def main() -> None:
     pm = policy_math_rates(dev, with_cpu=args.cpu_tokens > 0)
     # the same kernels on 16 x larger tensors, where the fixed ~8 us of the single-launch reduction no longer dominates
     pm_large = policy_math_rates(dev, with_cpu=False, B=2048, Lc=16384, n_groups=256)
+    pm_chain = policy_math_chain(dev)
 
     print(json.dumps({
         "metric": "tokens/s fwd+bwd logprob+entropy head @Qwen2.5-7B shape; MFMA util %",
@@ -327,6 +385,7 @@ def main() -> None:
         "cpu_baseline": base,
         "policy_math_b512_l4096": pm,
         "policy_math_b2048_l16384": pm_large,
+        "policy_math_chain_b512_l4096": pm_chain,
     }))
 
 

@@ -1339,3 +1339,72 @@ def test_widened_entry_points_at_benchmark_size_properties(dev):
     assert int(met["selected"].sum()) == max(1, int(mask.sum().item() * 0.0002))
     assert not bool(met["selected"][mask == 0].any())
 
+
+def test_c_abi_chain_replays_from_a_hip_graph(dev):
+    """The library allocates nothing, clears nothing with memset and leaves its arrival counters at zero, so a chain
+    of entry points can be captured once and replayed: GRPO advantage -> policy loss with gradient -> GAE -> value
+    loss at the benchmark size, three replays on fresh data with eager work in between, each bit-equal to the eager
+    chain."""
+    from verl_amd import _cabi
+    Lb = _cabi.lib()
+    B, Lc, G = 512, 4096, 64
+    gen = torch.Generator(device=dev).manual_seed(1)
+    f = lambda: torch.empty(B, Lc, device=dev)
+    inp = dict(rewards=f(), mask=f(), old=f(), new=f(), values=f(), vpreds=f())
+    gid = torch.arange(G, device=dev).repeat_interleave(B // G)
+
+    def outputs():
+        return dict(adv=f(), grad=f(), out=torch.empty(4, device=dev), coef=torch.empty(B, device=dev), gae_adv=f(),
+                    gae_ret=f(), vgrad=f(), vout=torch.empty(2, device=dev), vcoef=torch.empty(B, device=dev),
+                    mom=torch.empty(4, dtype=torch.float64, device=dev))
+
+    ws = torch.zeros(max(Lb.vamd_group_outcome_advantage_workspace_bytes(B, Lc, G),
+                         Lb.vamd_policy_loss_variant_workspace_bytes(B, Lc), Lb.vamd_gae_workspace_bytes(B, Lc),
+                         Lb.vamd_value_loss_workspace_bytes(B, Lc)), dtype=torch.uint8, device=dev)
+
+    def chain(o):
+        st = _cabi.stream_ptr(dev)
+        P = lambda t: t.data_ptr()
+        _cabi.check(Lb.vamd_grpo_advantage(P(inp["rewards"]), P(inp["mask"]), 0, P(gid), B, Lc, G, 1e-6, 1, 0, P(o["adv"]),
+                                           None, P(ws), ws.numel(), st))
+        _cabi.check(Lb.vamd_policy_loss_forward(P(inp["old"]), P(inp["new"]), P(o["adv"]), P(inp["mask"]), 0, None, B, Lc,
+                                                0.2, 0.2, 3.0, 0, 1.0, -1.0, -1.0, -1.0, P(o["out"]), P(o["grad"]),
+                                                P(o["coef"]), P(ws), ws.numel(), st))
+        _cabi.check(Lb.vamd_gae(P(inp["rewards"]), P(inp["values"]), P(inp["mask"]), 0, B, Lc, 1.0, 0.95, 1, P(o["gae_adv"]),
+                                P(o["gae_ret"]), P(o["mom"]), P(ws), ws.numel(), st))
+        _cabi.check(Lb.vamd_value_loss_forward(P(inp["vpreds"]), P(o["gae_ret"]), P(inp["values"]), P(inp["mask"]), 0, B, Lc,
+                                               0.5, 0, P(o["vout"]), P(o["vgrad"]), P(o["vcoef"]), P(ws), ws.numel(), st))
+
+    def refill():
+        lens = torch.randint(64, Lc + 1, (B,), device=dev, generator=gen)
+        inp["mask"].copy_((torch.arange(Lc, device=dev)[None, :] < lens[:, None]).float())
+        inp["rewards"].zero_()
+        inp["rewards"][torch.arange(B, device=dev), lens - 1] = torch.rand(B, device=dev, generator=gen)
+        inp["old"].copy_(torch.randn(B, Lc, device=dev, generator=gen) * 0.5 - 1)
+        inp["new"].copy_(inp["old"] + torch.randn(B, Lc, device=dev, generator=gen) * 0.05)
+        inp["values"].copy_(torch.randn(B, Lc, device=dev, generator=gen))
+        inp["vpreds"].copy_(inp["values"] + torch.randn(B, Lc, device=dev, generator=gen) * 0.5)
+
+    refill()
+    captured = outputs()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        chain(captured)                                          # warm-up outside the capture
+    torch.cuda.current_stream(dev).wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        chain(captured)
+    for _ in range(3):
+        refill()
+        eager = outputs()
+        chain(eager)
+        torch.cuda.synchronize()
+        for t in captured.values():
+            t.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for name in eager:
+            assert torch.equal(captured[name], eager[name]), name
+        assert int(ws[:16640].to(torch.int32).sum()) == 0        # the arrival counters are back at zero
+
