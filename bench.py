@@ -158,6 +158,9 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
     def copy(s):
         chk(L.vamd_copy_bytes(*P(s, "a", "o1"), 4 * BL, st))
 
+    def sum4(s):
+        chk(L.vamd_sum4(*P(s, "a", "b", "c", "mask", "o1"), BL, st))
+
     # name -> (algorithmic bytes per call, call)
     ops = {
         "grpo_advantage": (12 * BL, grpo),
@@ -174,6 +177,7 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
         "policy_loss_geo_mean_fwd_grad": (20 * BL, geo_mean),  # two passes over the inputs; one is the minimum
         "policy_loss_kl_cov_fwd_grad": (20 * BL, kl_cov),      # statistics, keys, 3 histogram passes, loss: 12 launches
         "copy_yardstick": (8 * BL, copy),
+        "sum4_yardstick": (20 * BL, sum4),                    # four tensors in, one out: the traffic of a loss with gradient
     }
     res = {}
     for name, (nbytes, fn) in ops.items():

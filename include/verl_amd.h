@@ -85,6 +85,9 @@ const char* vamd_last_error(void);
  * (a multiple of 16, both pointers 16-byte aligned) from src to dst.  Profilers read its memory
  * counters next to those of the other kernels to turn counter units into bytes. */
 int vamd_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream);
+/* out[i] = a[i] + b[i] + c[i] + d[i] over n floats (n % 4 == 0, 16-byte aligned pointers): a second yardstick,
+ * the memory traffic of a fused loss kernel with its gradient and nothing else.  No counterpart in the reference. */
+int vamd_sum4(const float* a, const float* b, const float* c, const float* d, float* out, int64_t n, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Fused vocab-projection log-prob / entropy head.

@@ -56,33 +56,75 @@ __device__ __forceinline__ float mask_weight(M m) {
 }
 
 // ------------------------------------------------------------------------------------------
-// wavefront / workgroup sums in double (deterministic: fixed tree, no atomics)
-__device__ __forceinline__ double wave_sum(double x) {
+// wavefront / workgroup reductions in double (deterministic: fixed tree, no atomics).
+//
+// Every active wavefront calls these with all 64 lanes enabled.  The lane exchanges are data-parallel-primitive
+// moves inside the vector ALU (a few cycles each) for the steps within a row of 16 lanes, and four lane reads for
+// the rows; the same tree through the LDS crossbar (__shfl_xor) costs about a hundred cycles per dependent step,
+// which is what a workgroup pays when it is the last one running and nothing hides the latency.
+template <int CTRL>
+__device__ __forceinline__ double lane_exchange(double x) {
+  int lo = __double2loint(x), hi = __double2hiint(x);
+  lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, 0xF, 0xF, false);
+  hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, 0xF, 0xF, false);
+  return __hiloint2double(hi, lo);
+}
+__device__ __forceinline__ double lane_read(double x, int lane) {
+  return __hiloint2double(__builtin_amdgcn_readlane(__double2hiint(x), lane),
+                          __builtin_amdgcn_readlane(__double2loint(x), lane));
+}
+struct SumOp {
+  __device__ __forceinline__ double operator()(double a, double b) const { return a + b; }
+};
+struct MaxOp {
+  __device__ __forceinline__ double operator()(double a, double b) const { return fmax(a, b); }
+};
+// Reduce NV values per lane over the wavefront, step-major so the NV chains overlap; the result is in every lane.
+// Steps: partner lane ^ 1 and lane ^ 2 (quad permutes), then the mirrored half row and the mirrored row, whose
+// partners hold the same value as lane ^ 4 and lane ^ 8 would since a quad / half row is uniform by then.
+template <int NV, class Op>
+__device__ __forceinline__ void wave_reduce(double (&v)[NV], Op op) {
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
-  return x;
+  for (int i = 0; i < NV; ++i) v[i] = op(v[i], lane_exchange<0xB1>(v[i]));   // quad_perm [1,0,3,2]
+#pragma unroll
+  for (int i = 0; i < NV; ++i) v[i] = op(v[i], lane_exchange<0x4E>(v[i]));   // quad_perm [2,3,0,1]
+#pragma unroll
+  for (int i = 0; i < NV; ++i) v[i] = op(v[i], lane_exchange<0x141>(v[i]));  // row_half_mirror
+#pragma unroll
+  for (int i = 0; i < NV; ++i) v[i] = op(v[i], lane_exchange<0x140>(v[i]));  // row_mirror
+#pragma unroll
+  for (int i = 0; i < NV; ++i)
+    v[i] = op(op(lane_read(v[i], 0), lane_read(v[i], 16)), op(lane_read(v[i], 32), lane_read(v[i], 48)));
+}
+__device__ __forceinline__ double wave_sum(double x) {
+  double v[1] = {x};
+  wave_reduce<1>(v, SumOp());
+  return v[0];
 }
 
-// Sum NV doubles per thread over a workgroup of NT threads; result valid in thread 0.
-template <int NV, int NT>
-__device__ __forceinline__ void block_sum(double (&v)[NV], double* smem /* NV * NT/64 doubles */) {
+// Reduce NV doubles per thread over a workgroup of NT threads; result valid in thread 0.
+template <int NV, int NT, class Op>
+__device__ __forceinline__ void block_reduce(double (&v)[NV], double* smem /* NV * NT/64 doubles */, Op op) {
   constexpr int NW = NT / 64;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  wave_reduce<NV>(v, op);
+  if (lane == 0)
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    v[i] = wave_sum(v[i]);
-    if (lane == 0) smem[i * NW + w] = v[i];
-  }
+    for (int i = 0; i < NV; ++i) smem[i * NW + w] = v[i];
   __syncthreads();
   if (threadIdx.x == 0) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      double s = 0;
-      for (int j = 0; j < NW; ++j) s += smem[i * NW + j];
+      double s = smem[i * NW];
+      for (int j = 1; j < NW; ++j) s = op(s, smem[i * NW + j]);
       v[i] = s;
     }
   }
   __syncthreads();
+}
+template <int NV, int NT>
+__device__ __forceinline__ void block_sum(double (&v)[NV], double* smem) {
+  block_reduce<NV, NT>(v, smem, SumOp());
 }
 
 }  // namespace vamd

@@ -25,32 +25,10 @@ enum {
 };
 constexpr int kDmSums = kDmAdvMax;  // slots [0, kDmSums) add, the rest are extrema
 
-__device__ __forceinline__ double wave_max(double x) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) x = fmax(x, __shfl_xor(x, o, 64));
-  return x;
-}
-
 // Maximum of NV doubles per thread over the workgroup; result valid in thread 0.
 template <int NV, int NT>
 __device__ __forceinline__ void block_max(double (&v)[NV], double* smem /* NV * NT/64 doubles */) {
-  constexpr int NW = NT / 64;
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    v[i] = wave_max(v[i]);
-    if (lane == 0) smem[i * NW + w] = v[i];
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      double s = smem[i * NW];
-      for (int j = 1; j < NW; ++j) s = fmax(s, smem[i * NW + j]);
-      v[i] = s;
-    }
-  }
-  __syncthreads();
+  block_reduce<NV, NT>(v, smem, MaxOp());
 }
 
 struct DmArgs {

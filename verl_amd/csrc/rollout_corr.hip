@@ -48,31 +48,9 @@ struct RcArgs {
   double* out;         // [VAMD_RC_COUNT]
 };
 
-__device__ __forceinline__ double wave_max_f64(double x) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) x = fmax(x, __shfl_xor(x, o, 64));
-  return x;
-}
-
 template <int NV, int NT>
 __device__ __forceinline__ void block_max_f64(double (&v)[NV], double* smem) {
-  constexpr int NW = NT / 64;
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-#pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    v[i] = wave_max_f64(v[i]);
-    if (lane == 0) smem[i * NW + w] = v[i];
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      double s = smem[i * NW];
-      for (int j = 1; j < NW; ++j) s = fmax(s, smem[i * NW + j]);
-      v[i] = s;
-    }
-  }
-  __syncthreads();
+  block_reduce<NV, NT>(v, smem, MaxOp());
 }
 
 template <bool VEC, class M>
