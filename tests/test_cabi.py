@@ -45,9 +45,10 @@ def test_workspace_queries(lib):
     one = lib.vamd_lce_backward_workspace_bytes(256, 128, 1024, 0)
     assert one == 256 * (1024 + 128) * 2                          # a single padded panel, no accumulator
     # single-launch reductions: arrival counters (VAMD_TICKET_BYTES) + one record of doubles per 4096-column chunk
+    # + 64 records for the share totals of the two-level sum
     ticket = 16640
-    assert lib.vamd_masked_moments_workspace_bytes(512, 4096) == ticket + 512 * 4 * 8
-    assert lib.vamd_policy_loss_workspace_bytes(512, 4097) == ticket + 512 * 2 * 5 * 8
+    assert lib.vamd_masked_moments_workspace_bytes(512, 4096) == ticket + (512 + 64) * 4 * 8
+    assert lib.vamd_policy_loss_workspace_bytes(512, 4097) == ticket + (512 * 2 + 64) * 5 * 8
     assert lib.vamd_gae_workspace_bytes(512, 4096) >= ticket + 512 * 4 * 8
 
 

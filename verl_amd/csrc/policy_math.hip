@@ -58,8 +58,17 @@ __global__ __launch_bounds__(kRcThreads) void moments_kernel(const float* __rest
   if (threadIdx.x == 0) {
     store_record<4>(wk.partials, row, chunk, rows, chunks, acc);
   }
+  if (!per_row) {
+    double a[4];
+    if (!sum_all_records<4>(wk.ticket, wk.partials, rows, chunks, a, smem)) return;
+    if (threadIdx.x == 0)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[i] = a[i];
+    ticket_reset(wk.ticket);
+    return;
+  }
   if (!last_block_arrives(wk.ticket)) return;
-  if (per_row) {
+  {
     for (int64_t r0 = threadIdx.x; r0 < rows; r0 += 2 * kRcThreads) {
       const int64_t rr[2] = {r0, r0 + kRcThreads};
       const bool have[2] = {true, rr[1] < rows};
@@ -71,13 +80,6 @@ __global__ __launch_bounds__(kRcThreads) void moments_kernel(const float* __rest
 #pragma unroll
           for (int i = 0; i < 4; ++i) out[rr[k] * 4 + i] = a[k][i];
     }
-  } else {
-    double a[4] = {0, 0, 0, 0};
-    sum_records_strided<4>(wk.partials, rows * chunks, a);
-    block_sum<4, kRcThreads>(a, smem);
-    if (threadIdx.x == 0)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) out[i] = a[i];
   }
   ticket_reset(wk.ticket);
 }
@@ -625,7 +627,8 @@ __global__ __launch_bounds__(kRcThreads) void kl_reward_kernel(
 // =============================================================================================
 // GRPO
 // =============================================================================================
-constexpr int kGrpoLdsGroups = 2048;  // groups whose statistics fit the last workgroup's LDS
+constexpr int kGrpoLdsGroups = 2048;   // groups whose statistics fit one workgroup's LDS
+constexpr int kGrpoInlineGroups = 512;  // ... and the LDS of every workgroup of the streaming pass
 
 struct GrpoArgs {
   const int64_t* gid;
@@ -654,78 +657,115 @@ struct GrpoArgs {
 // A single-member group has mean 0 (and std 1) in every estimator.
 // std_mode 0: unbiased torch.std; 1: sqrt(clamp(var, min=eps)) of group_mean_std.  Singleton
 // groups get mean 0, std 1 (core_algos.py:314-316, groupwise.py:215-221).
-template <bool VEC>
-__global__ __launch_bounds__(kRcThreads) void grpo_rowsum_kernel(const float* __restrict__ x, int64_t cols,
-                                                                 int chunks, Work wk, GrpoArgs ga) {
-  const int64_t row = blockIdx.x / chunks;
-  const int chunk = blockIdx.x % chunks;
-  const ChunkPos pos(row, chunk, cols);
-  float v[kGroups][4];
-  load_groups<VEC>(x, pos, v);
-  float s = 0;
-#pragma unroll
-  for (int g = 0; g < kGroups; ++g) s += (v[g][0] + v[g][1]) + (v[g][2] + v[g][3]);
-  __shared__ double smem[4];
-  double acc[1] = {s};
-  block_sum<1, kRcThreads>(acc, smem);
-  if (threadIdx.x == 0) store_record<1>(wk.partials, row, chunk, ga.rows, chunks, acc);
-  if (ga.n_groups > kGrpoLdsGroups) return;  // statistics come from the separate kernels below
-  if (!last_block_arrives(wk.ticket)) return;
-
-  __shared__ int g_cnt[kGrpoLdsGroups];
-  __shared__ double g_sum[kGrpoLdsGroups];
-  __shared__ double g_sq[kGrpoLdsGroups];
-  for (int64_t g = threadIdx.x; g < ga.n_groups; g += kRcThreads) {
+// Scores, per-group statistics and the per-response scalar from the (row, chunk) row-sum records; run by one
+// workgroup of kRcThreads threads; g_cnt / g_sum / g_sq are LDS arrays of n_groups entries.
+template <bool COHERENT, int HELD, int NT, int EST = -1>
+__device__ __forceinline__ void grpo_scalars_from_records(const double* __restrict__ partials, int chunks,
+                                                          const GrpoArgs& ga, int* __restrict__ g_cnt,
+                                                          double* __restrict__ g_sum, double* __restrict__ g_sq) {
+  for (int64_t g = threadIdx.x; g < ga.n_groups; g += NT) {
     g_cnt[g] = 0;
     g_sum[g] = 0.0;
     g_sq[g] = 0.0;
   }
   __syncthreads();
-  const bool opo = ga.estimator == VAMD_ADV_OPO;
+  const int estimator = EST >= 0 ? EST : ga.estimator;  // a compile-time estimator drops the other branches
+  const bool opo = estimator == VAMD_ADV_OPO;
   double nnz_local = 0;
-  for (int64_t r0 = threadIdx.x; r0 < ga.rows; r0 += 4 * kRcThreads) {
-    int64_t rr[4];
-    bool have[4];
+  // One workgroup runs this with nothing else to hide its latency, so a thread takes HELD rows per trip with
+  // all their loads in flight, and when one trip covers the launch (rows <= HELD * NT) the rows' scores
+  // and group ids stay in registers for the passes below instead of being read back.
+  constexpr int64_t kTrip = (int64_t)HELD * NT;
+  const bool resident = ga.rows <= kTrip;
+  // Thread index -> row through a stride permutation: responses of one group usually sit next to each other,
+  // and 64 lanes adding to a handful of LDS addresses are served one lane after the other.  A prime stride that
+  // does not divide the row count is a bijection and sends neighbouring lanes to different groups.
+  // Index i = threadIdx.x + m * NT maps to row (i * stride) mod rows, walked by adding (NT * stride) mod rows.
+  const unsigned n_rows = (unsigned)ga.rows;
+  const unsigned stride = n_rows % 61 ? 61 : (n_rows % 59 ? 59 : 53);
+  const unsigned first_row = (threadIdx.x * stride) % n_rows, row_step = ((unsigned)NT * stride) % n_rows;
+  // rows of the HELD indices of a trip; `at` is the row of the trip's first index and moves on to the next trip
+  auto trip_rows = [&](unsigned& at, int64_t (&rk)[HELD]) {
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      rr[k] = r0 + (int64_t)k * kRcThreads;
-      have[k] = rr[k] < ga.rows;
+    for (int k = 0; k < HELD; ++k) {
+      rk[k] = at;
+      at += row_step;
+      if (at >= n_rows) at -= n_rows;
     }
-    double row_sum[4][1];
-    fold_row_records<1, 1, 4>(wk.partials, rr, have, ga.rows, chunks, row_sum);
+  };
+  float sc[HELD];
+  int gi[HELD];
+  unsigned at = first_row;
+  int64_t rk[HELD];
+  for (int64_t base = threadIdx.x; base < ga.rows; base += kTrip) {
+    double len[HELD];
+    trip_rows(at, rk);
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      if (!have[k]) break;
-      const int64_t r = rr[k];
-      const float sc = (float)row_sum[k][0];
-      ga.scores[r] = sc;
-      nnz_local += sc != 0.f ? 1.0 : 0.0;
-      const int64_t g = ga.gid[r];
-      atomicAdd(&g_cnt[g], 1);
+    for (int k = 0; k < HELD; ++k) {
+      const int64_t i = base + (int64_t)k * NT;
+      gi[k] = i < ga.rows ? (int)ga.gid[rk[k]] : 0;
+      len[k] = (opo && i < ga.rows) ? ga.row_moments[rk[k] * 4] : 0.0;
+    }
+    constexpr int kSub = HELD < 4 ? HELD : 4;  // rows whose chunk records are in flight together
+#pragma unroll
+    for (int h = 0; h < HELD; h += kSub) {
+      int64_t rr[kSub];
+      bool have[kSub];
+#pragma unroll
+      for (int k = 0; k < kSub; ++k) {
+        rr[k] = rk[h + k];
+        have[k] = base + (int64_t)(h + k) * NT < ga.rows;
+      }
+      double row_sum[kSub][1];
+      fold_row_records<1, 1, kSub, COHERENT>(partials, rr, have, ga.rows, chunks, row_sum);
+#pragma unroll
+      for (int k = 0; k < kSub; ++k) sc[h + k] = (float)row_sum[k][0];
+    }
+#pragma unroll
+    for (int k = 0; k < HELD; ++k) {
+      if (base + (int64_t)k * NT >= ga.rows) break;
+      ga.scores[rk[k]] = sc[k];
+      nnz_local += sc[k] != 0.f ? 1.0 : 0.0;
+      atomicAdd(&g_cnt[gi[k]], 1);
       if (opo) {  // g_sum: sum(len * s), g_sq: sum(len)
-        const double len = ga.row_moments[r * 4];
-        atomicAdd(&g_sum[g], len * (double)sc);
-        atomicAdd(&g_sq[g], len);
+        atomicAdd(&g_sum[gi[k]], len[k] * (double)sc[k]);
+        atomicAdd(&g_sq[gi[k]], len[k]);
       } else {
-        atomicAdd(&g_sum[g], (double)sc);
+        atomicAdd(&g_sum[gi[k]], (double)sc[k]);
       }
     }
   }
   __syncthreads();
-  if (ga.estimator == VAMD_ADV_GRPO || ga.estimator == VAMD_ADV_GRPO_PASSK) {
-    for (int64_t r = threadIdx.x; r < ga.rows; r += kRcThreads) {
-      const int64_t g = ga.gid[r];
-      const double d = (double)ga.scores[r] - g_sum[g] / (double)g_cnt[g];
-      atomicAdd(&g_sq[g], d * d);
+  // scores and group ids of the trip starting at `base`: still in registers, or read back
+  auto held_rows = [&](int64_t base) {
+    if (resident) return;  // rk[] is then still the one trip's
+    trip_rows(at, rk);
+#pragma unroll
+    for (int k = 0; k < HELD; ++k) {
+      const int64_t i = base + (int64_t)k * NT;
+      gi[k] = i < ga.rows ? (int)ga.gid[rk[k]] : 0;
+      sc[k] = i < ga.rows ? ga.scores[rk[k]] : 0.f;
+    }
+  };
+  if (estimator == VAMD_ADV_GRPO || estimator == VAMD_ADV_GRPO_PASSK) {
+    at = first_row;
+    for (int64_t base = threadIdx.x; base < ga.rows; base += kTrip) {
+      held_rows(base);
+#pragma unroll
+      for (int k = 0; k < HELD; ++k) {
+        if (base + (int64_t)k * NT >= ga.rows) break;
+        const double d = (double)sc[k] - g_sum[gi[k]] / (double)g_cnt[gi[k]];
+        atomicAdd(&g_sq[gi[k]], d * d);
+      }
     }
     __syncthreads();
   }
-  if (ga.estimator == VAMD_ADV_GRPO_PASSK) {
+  if (estimator == VAMD_ADV_GRPO_PASSK) {
     // one thread per group walks the responses in index order: best score (first index on ties,
     // where the advantage is 0 anyway), runner-up, unbiased std; the group's entry of `mean`
     // receives the advantage and the entry of `stdv` the index of the best response
     __syncthreads();
-    for (int64_t g = threadIdx.x; g < ga.n_groups; g += kRcThreads) {
+    for (int64_t g = threadIdx.x; g < ga.n_groups; g += NT) {
       float best = -INFINITY, second = -INFINITY;
       int64_t arg = -1;
       for (int64_t r = 0; r < ga.rows; ++r) {
@@ -748,57 +788,100 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rowsum_kernel(const float* __
     __syncthreads();
   }
   float alpha = 1.f;
-  if (ga.estimator == VAMD_ADV_GPG) {
-    __shared__ double nz_smem[4];
+  if (estimator == VAMD_ADV_GPG) {
+    __shared__ double nz_smem[NT / 64];
     __shared__ float alpha_bc;
     double acc1[1] = {nnz_local};
-    block_sum<1, kRcThreads>(acc1, nz_smem);
+    block_sum<1, NT>(acc1, nz_smem);
     if (threadIdx.x == 0) alpha_bc = (float)ga.rows / fmaxf((float)acc1[0], 1.f);
     __syncthreads();
     alpha = alpha_bc;
   }
-  for (int64_t r = threadIdx.x; r < ga.rows; r += kRcThreads) {
-    const int64_t g = ga.gid[r];
-    const int c = g_cnt[g];
-    const float sc = ga.scores[r];
-    float out;
-    switch (ga.estimator) {
-      case VAMD_ADV_GRPO: {
-        float mu = 0.f, sd = 1.f;
-        if (c > 1) {
-          const double var = g_sq[g] / (double)(c - 1);
-          mu = (float)(g_sum[g] / (double)c);
-          sd = ga.std_mode == 0 ? (float)sqrt(var) : sqrtf(fmaxf((float)var, ga.eps));
-        }
-        const float cen = sc - mu;
-        out = ga.norm_by_std ? cen / (sd + ga.eps) : cen;
-      } break;
-      case VAMD_ADV_RLOO:
-      case VAMD_ADV_RLOO_VECTORIZED: {
-        if (c > 1) {
-          const float mu = (float)(g_sum[g] / (double)c);
-          const float n = (float)c, n1 = (float)(c - 1);
-          out = sc * n / n1 - mu * n / n1;
-        } else {
-          out = ga.estimator == VAMD_ADV_RLOO ? sc : 0.f;
-        }
-      } break;
-      case VAMD_ADV_OPO:
-        out = c > 1 ? sc - (float)(g_sum[g] / g_sq[g]) : sc;
-        break;
-      case VAMD_ADV_GPG:
-        out = alpha * (sc - (c > 1 ? (float)(g_sum[g] / (double)c) : 0.f)) / ga.f_norm;
-        break;
-      case VAMD_ADV_GRPO_PASSK:
-        out = (double)r == g_sq[g] ? (float)g_sum[g] : 0.f;
-        break;
-      default:  // VAMD_ADV_MEAN_BASELINE
-        out = sc - (c > 1 ? (float)(g_sum[g] / (double)c) : 0.f);
-        break;
+  at = first_row;
+  for (int64_t base = threadIdx.x; base < ga.rows; base += kTrip) {
+    held_rows(base);
+#pragma unroll
+    for (int k = 0; k < HELD; ++k) {
+      if (base + (int64_t)k * NT >= ga.rows) break;
+      const int64_t r = rk[k];
+      const int g = gi[k];
+      const int c = g_cnt[g];
+      const float sck = sc[k];
+      float out;
+      switch (estimator) {
+        case VAMD_ADV_GRPO: {
+          float mu = 0.f, sd = 1.f;
+          if (c > 1) {
+            const double var = g_sq[g] / (double)(c - 1);
+            mu = (float)(g_sum[g] / (double)c);
+            sd = ga.std_mode == 0 ? (float)sqrt(var) : sqrtf(fmaxf((float)var, ga.eps));
+          }
+          const float cen = sck - mu;
+          out = ga.norm_by_std ? cen / (sd + ga.eps) : cen;
+        } break;
+        case VAMD_ADV_RLOO:
+        case VAMD_ADV_RLOO_VECTORIZED: {
+          if (c > 1) {
+            const float mu = (float)(g_sum[g] / (double)c);
+            const float n = (float)c, n1 = (float)(c - 1);
+            out = sck * n / n1 - mu * n / n1;
+          } else {
+            out = estimator == VAMD_ADV_RLOO ? sck : 0.f;
+          }
+        } break;
+        case VAMD_ADV_OPO:
+          out = c > 1 ? sck - (float)(g_sum[g] / g_sq[g]) : sck;
+          break;
+        case VAMD_ADV_GPG:
+          out = alpha * (sck - (c > 1 ? (float)(g_sum[g] / (double)c) : 0.f)) / ga.f_norm;
+          break;
+        case VAMD_ADV_GRPO_PASSK:
+          out = (double)r == g_sq[g] ? (float)g_sum[g] : 0.f;
+          break;
+        default:  // VAMD_ADV_MEAN_BASELINE
+          out = sck - (c > 1 ? (float)(g_sum[g] / (double)c) : 0.f);
+          break;
+      }
+      ga.scalars[r] = out;
     }
-    ga.scalars[r] = out;
   }
-  ticket_reset(wk.ticket);
+}
+
+// Small launches let the workgroup that arrives last run the statistics (TAIL); large ones leave them to a launch
+// of their own, whose registers and LDS are then not charged to every wavefront of the streaming pass.
+template <bool VEC, bool TAIL>
+__global__ __launch_bounds__(kRcThreads) void grpo_rowsum_kernel(const float* __restrict__ x, int64_t cols,
+                                                                 int chunks, Work wk, GrpoArgs ga) {
+  const int64_t row = blockIdx.x / chunks;
+  const int chunk = blockIdx.x % chunks;
+  const ChunkPos pos(row, chunk, cols);
+  float v[kGroups][4];
+  load_groups<VEC>(x, pos, v);
+  float s = 0;
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g) s += (v[g][0] + v[g][1]) + (v[g][2] + v[g][3]);
+  __shared__ double smem[4];
+  double acc[1] = {s};
+  block_sum<1, kRcThreads>(acc, smem);
+  if constexpr (TAIL) {
+    if (threadIdx.x == 0) store_record<1>(wk.partials, row, chunk, ga.rows, chunks, acc);
+    if (!last_block_arrives(wk.ticket)) return;
+    __shared__ int g_cnt[kGrpoInlineGroups];
+    __shared__ double g_sum[kGrpoInlineGroups], g_sq[kGrpoInlineGroups];
+    grpo_scalars_from_records<true, 4, kRcThreads>(wk.partials, chunks, ga, g_cnt, g_sum, g_sq);
+    ticket_reset(wk.ticket);
+  } else {
+    if (threadIdx.x == 0) wk.partials[record_at(0, row, chunk, ga.rows, chunks)] = acc[0];
+  }
+}
+
+constexpr int kGrpoTailThreads = 1024;
+template <int EST>
+__global__ __launch_bounds__(kGrpoTailThreads) void grpo_scalars_kernel_lds(const double* __restrict__ partials, int chunks,
+                                                                            GrpoArgs ga) {
+  __shared__ int g_cnt[kGrpoLdsGroups];
+  __shared__ double g_sum[kGrpoLdsGroups], g_sq[kGrpoLdsGroups];
+  grpo_scalars_from_records<false, 2, kGrpoTailThreads, EST>(partials, chunks, ga, g_cnt, g_sum, g_sq);
 }
 
 // ---- path for more groups than fit in LDS (and for group_mean_std itself) ----
@@ -883,7 +966,7 @@ static AggParams make_agg(int mode, double dp, double bnt, double gbs, double ls
 
 static size_t reduce_workspace_bytes(int64_t rows, int64_t cols, int nv) {
   if (rows <= 0 || cols <= 0) return 0;
-  return kTicketBytes + align_up((size_t)rows * chunks_of(cols) * nv * sizeof(double), 256);
+  return kTicketBytes + align_up(((size_t)rows * chunks_of(cols) + kShareSlots) * nv * sizeof(double), 256);
 }
 
 static Work carve_work(void* workspace) {
@@ -1388,8 +1471,24 @@ extern "C" int vamd_group_outcome_advantage(const float* rewards, const void* ma
   }
   {
     const bool vec = can_vectorize(length, {rewards}, nullptr, 0);
-    VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((grpo_rowsum_kernel<V>), dim3((unsigned)(batch * chunks)),
-                                                 dim3(kRcThreads), 0, s, rewards, length, chunks, wk, ga));
+    const bool lds_stats = n_groups <= kGrpoLdsGroups;
+    const dim3 grid((unsigned)(batch * chunks));
+    if (n_groups <= kGrpoInlineGroups && batch * chunks <= kInlineFoldRecords) {
+      VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((grpo_rowsum_kernel<V, true>), grid, dim3(kRcThreads), 0, s,
+                                                   rewards, length, chunks, wk, ga));
+    } else {
+      VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((grpo_rowsum_kernel<V, false>), grid, dim3(kRcThreads), 0, s,
+                                                   rewards, length, chunks, wk, ga));
+      if (lds_stats) {
+        VAMD_LAUNCH_CHECK();
+        if (estimator == VAMD_ADV_GRPO)
+          hipLaunchKernelGGL(grpo_scalars_kernel_lds<VAMD_ADV_GRPO>, dim3(1), dim3(kGrpoTailThreads), 0, s,
+                             wk.partials, chunks, ga);
+        else
+          hipLaunchKernelGGL(grpo_scalars_kernel_lds<-1>, dim3(1), dim3(kGrpoTailThreads), 0, s, wk.partials, chunks,
+                             ga);
+      }
+    }
     VAMD_LAUNCH_CHECK();
   }
   if (n_groups > kGrpoLdsGroups) {

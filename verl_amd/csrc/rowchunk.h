@@ -164,6 +164,33 @@ __device__ __forceinline__ bool last_block_arrives(unsigned* counters) {
   __syncthreads();
   return last != 0;
 }
+// The two levels taken apart, for launches whose last workgroup of each first-level counter has work to do
+// (folding that counter's share of the records) before it arrives at the second level.
+__device__ __forceinline__ bool share_last_arrives(unsigned* counters) {
+  __shared__ unsigned last;
+  if (threadIdx.x == 0) {
+    const unsigned n = gridDim.x, G = ticket_groups();
+    const unsigned g = blockIdx.x % G;
+    const unsigned members = (n - g + G - 1) / G;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const unsigned t = __hip_atomic_fetch_add(counters + (1 + g) * (kTicketStride / 4), 1u, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+    last = t == members - 1 ? 1u : 0u;
+  }
+  __syncthreads();
+  return last != 0;
+}
+// Called by the workgroups share_last_arrives() was true in, after thread 0 issued the peer_store()s of the share.
+__device__ __forceinline__ bool launch_last_arrives(unsigned* counters) {
+  __shared__ unsigned last;
+  if (threadIdx.x == 0) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const unsigned t = __hip_atomic_fetch_add(counters, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    last = t == ticket_groups() - 1 ? 1u : 0u;
+  }
+  __syncthreads();
+  return last != 0;
+}
 __device__ __forceinline__ void ticket_reset(unsigned* counters) {
   if (threadIdx.x <= ticket_groups())
     __hip_atomic_store(counters + threadIdx.x * (kTicketStride / 4), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -245,6 +272,58 @@ __device__ __forceinline__ void sum_records_strided(const double* __restrict__ r
       for (int i = 0; i < NV; ++i) acc[i] += t[u][i];
   }
 }
+
+// Sum of every slot over all n = rows * chunks records of the launch (slot-major, record_at).  Returns true in
+// exactly one workgroup, whose thread 0 then holds the totals.  Up to kOneLevelRecords records the workgroup that
+// arrives last adds them all; a larger launch would leave that one workgroup with dozens of dependent trips to
+// memory while the rest of the device idles, so there the last workgroup to arrive at each of the G first-level
+// counters adds the records of that counter's workgroups (b = g, g + G, ...: a fixed set, so the result does not
+// depend on the order of arrival) and publishes NV share totals behind the records, and the last of those G adds
+// the shares.  The shares of early counters are folded while later workgroups still stream.
+constexpr int64_t kOneLevelRecords = 4096;
+template <int NV>
+__device__ __forceinline__ bool sum_all_records(unsigned* counters, double* __restrict__ records, int64_t rows,
+                                                int chunks, double (&tot)[NV], double* smem /* NV * 4 */) {
+  const int64_t n = rows * chunks;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) tot[i] = 0;
+  if (n <= kOneLevelRecords) {
+    if (!last_block_arrives(counters)) return false;
+    sum_records_strided<NV>(records, n, tot);
+    block_sum<NV, kRcThreads>(tot, smem);
+    return true;
+  }
+  if (!share_last_arrives(counters)) return false;
+  const unsigned G = ticket_groups(), g = blockIdx.x % G;
+  const int64_t members = (n - g + G - 1) / G;
+  double* shares = records + n * NV;  // [NV][G]
+  for (int64_t m0 = threadIdx.x; m0 < members; m0 += 4 * kRcThreads) {
+    double t[4][NV];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t m = m0 + (int64_t)u * kRcThreads;
+      const int64_t b = g + m * G;  // the workgroup whose record this is
+      const int64_t k = (b % chunks) * rows + b / chunks;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) t[u][i] = m < members ? peer_load(records + (int64_t)i * n + k) : 0.0;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < NV; ++i) tot[i] += t[u][i];
+  }
+  block_sum<NV, kRcThreads>(tot, smem);
+  if (threadIdx.x == 0)
+#pragma unroll
+    for (int i = 0; i < NV; ++i) peer_store(shares + i * G + g, tot[i]);
+  if (!launch_last_arrives(counters)) return false;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) tot[i] = threadIdx.x < G ? peer_load(shares + i * G + threadIdx.x) : 0.0;
+  block_sum<NV, kRcThreads>(tot, smem);
+  return true;
+}
+// Doubles a record area needs behind its rows * chunks * nv record slots for sum_all_records().
+constexpr size_t kShareSlots = kTicketGroups;
 
 // (mean, rsqrt(var_unbiased + 1e-8), shift) from the masked moments sum(m), sum(v m), sum(v^2 m),
 // following masked_mean / masked_var / masked_whiten (verl/utils/torch_functional.py:287-339).
