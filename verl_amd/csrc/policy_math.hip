@@ -226,7 +226,11 @@ struct TokenLoss {
   float loss, dloss, kl, cf, cfl;  // kl: -(clamped or raw) log-ratio; cf / cfl: 1 where the clip counters fire
 };
 
+// VARIANT >= 0 fixes the variant at compile time: the per-token code is then straight-line and the 16 tokens of a
+// thread interleave; VARIANT = -1 reads it from pp (one branch per token, every variant's code in the kernel).
+template <int VARIANT>
 __device__ __forceinline__ TokenLoss token_loss(const PolicyParams& pp, float old, float lp, float A, float seq_lr) {
+  const int variant = VARIANT >= 0 ? VARIANT : pp.variant;
   TokenLoss t;
   t.cf = 0.f;
   t.cfl = 0.f;
@@ -234,7 +238,7 @@ __device__ __forceinline__ TokenLoss token_loss(const PolicyParams& pp, float ol
   const float k = fminf(fmaxf(d, -20.f), 20.f);
   const float in_k = (d >= -20.f && d <= 20.f) ? 1.f : 0.f;
   t.kl = -k;
-  switch (pp.variant) {
+  switch (variant) {
     case VAMD_PL_GPG:
       t.loss = -lp * A;
       t.dloss = -A;
@@ -351,7 +355,7 @@ __global__ __launch_bounds__(kRcThreads) void geo_rows_kernel(const float* __res
   }
 }
 
-template <bool VEC, class M, bool GRAD, bool ISW, bool FOLD>
+template <bool VEC, class M, bool GRAD, bool ISW, bool FOLD, int VARIANT>
 __global__ __launch_bounds__(kRcThreads) void policy_kernel(
     const float* __restrict__ old_lp, const float* __restrict__ lp, const float* __restrict__ adv,
     const M* __restrict__ mask, const float* __restrict__ isw, int64_t rows, int64_t cols, int chunks,
@@ -368,9 +372,10 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
   if (ISW) load_groups<VEC>(isw, pos, iw);
   const bool token_mean = ap.mode == VAMD_AGG_TOKEN_MEAN;
   float seq_lr = 0.f;
-  if (pp.variant == VAMD_PL_GSPO)  // sum((lp - old) m) / clamp(sum(m), min = 1)
+  const int variant = VARIANT >= 0 ? VARIANT : pp.variant;
+  if (variant == VAMD_PL_GSPO)  // sum((lp - old) m) / clamp(sum(m), min = 1)
     seq_lr = (float)pp.row_moments[row * 4 + 1] / fmaxf((float)pp.row_moments[row * 4], 1.f);
-  if (pp.variant == VAMD_PL_GEO_MEAN) {
+  if (variant == VAMD_PL_GEO_MEAN) {
     double r[4] = {0, 0, 0, 0};
     for (int c = 0; c < chunks; ++c)
 #pragma unroll
@@ -386,7 +391,7 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
   for (int g = 0; g < kGroups; ++g)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const TokenLoss t = token_loss(pp, o[g][e], n[g][e], a[g][e], seq_lr);
+      const TokenLoss t = token_loss<VARIANT>(pp, o[g][e], n[g][e], a[g][e], seq_lr);
       float loss = t.loss;
       if (ISW) loss *= iw[g][e];
       const float we = w[g][e];
@@ -1228,12 +1233,16 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
     is_weights = nullptr;  // already folded into the sequence loss
   }
   bool sep = rows * chunks > kInlineFoldRecords;  // fold the records in a launch of their own
-#define VAMD_PL(V, G, W, F)                                                                                     \
-  hipLaunchKernelGGL((policy_kernel<V, M, G, W, F>), grid, block, 0, s, old_log_prob, log_prob, advantages, mk, \
+  // the clipped PPO loss gets kernels of its own, the other variants share one with a per-token switch
+#define VAMD_PL_LAUNCH(V, G, W, F, K)                                                                              \
+  hipLaunchKernelGGL((policy_kernel<V, M, G, W, F, K>), grid, block, 0, s, old_log_prob, log_prob, advantages, mk, \
                      is_weights, rows, cols, chunks, pp, ap, wk, out, grad_unscaled, coef_out)
+#define VAMD_PL(V, G, W, F)                                                          \
+  if (variant == VAMD_PL_VANILLA) VAMD_PL_LAUNCH(V, G, W, F, VAMD_PL_VANILLA); \
+  else VAMD_PL_LAUNCH(V, G, W, F, -1)
 #define VAMD_PL_GW(V, F)                                                                             \
-  if (grad_unscaled) { if (is_weights) VAMD_PL(V, true, true, F); else VAMD_PL(V, true, false, F); } \
-  else { if (is_weights) VAMD_PL(V, false, true, F); else VAMD_PL(V, false, false, F); }
+  if (grad_unscaled) { if (is_weights) { VAMD_PL(V, true, true, F); } else { VAMD_PL(V, true, false, F); } } \
+  else { if (is_weights) { VAMD_PL(V, false, true, F); } else { VAMD_PL(V, false, false, F); } }
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(cols, {old_log_prob, log_prob, advantages, is_weights, grad_unscaled}, mask,
                                    sizeof(M));
@@ -1248,6 +1257,7 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
                        chunks, cols, ap, coef_out, out);
 #undef VAMD_PL_GW
 #undef VAMD_PL
+#undef VAMD_PL_LAUNCH
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }
