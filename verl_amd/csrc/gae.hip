@@ -7,10 +7,10 @@
 //     nv' = a nv + b ,  g' = P nv + Q g + R           (a in {0,1})
 // and maps compose associatively, so the recurrence is a prefix "sum" over maps.  A row is cut
 // into segments of 1024 columns walked right to left; inside a segment each of the 256 threads
-// composes its 4 columns, a wavefront scan (shuffles) plus an LDS pass over the wavefront totals
+// composes its 4 columns, a wavefront scan (lane exchanges) plus an LDS pass over the wavefront totals
 // yields every thread's incoming state, and the thread then replays its 4 columns to emit the
 // advantages.  Loads and stores are float4 and contiguous across the wavefront; four segments are
-// loaded and scanned together, so memory latency, the shuffle chain and the workgroup barrier
+// loaded and scanned together, so memory latency, the exchange chain and the workgroup barrier
 // are paid once per 4096 columns.  The workgroup that
 // finishes last folds the per-row masked moments and writes the whitening statistics, so the
 // whole estimator is two launches (scan, then the elementwise whitening).
@@ -35,14 +35,35 @@ __device__ __forceinline__ Affine compose(const Affine& later, const Affine& ear
   return o;
 }
 
-__device__ __forceinline__ Affine shfl_up_affine(const Affine& x, int d) {
+// Lane exchange inside the vector ALU (data-parallel primitives): a lane without a source in the pattern, or in a
+// row the mask leaves out, receives `none`.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_f32(float x, float none) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(none), __float_as_int(x), CTRL, ROW_MASK, 0xF, false));
+}
+// The map of the lane the pattern names, the identity where there is none (composing with it changes nothing,
+// so the scan needs no lane test).
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ Affine dpp_affine(const Affine& x) {
   Affine o;
-  o.a = __shfl_up(x.a, d, 64);
-  o.b = __shfl_up(x.b, d, 64);
-  o.P = __shfl_up(x.P, d, 64);
-  o.Q = __shfl_up(x.Q, d, 64);
-  o.R = __shfl_up(x.R, d, 64);
+  o.a = dpp_f32<CTRL, ROW_MASK>(x.a, 1.f);
+  o.b = dpp_f32<CTRL, ROW_MASK>(x.b, 0.f);
+  o.P = dpp_f32<CTRL, ROW_MASK>(x.P, 0.f);
+  o.Q = dpp_f32<CTRL, ROW_MASK>(x.Q, 1.f);
+  o.R = dpp_f32<CTRL, ROW_MASK>(x.R, 0.f);
   return o;
+}
+// Inclusive scan of the maps over the wavefront (lane 0 first): shifts by 1, 2, 4, 8 inside each row of 16 lanes,
+// then the last lane of row 0 / 2 into rows 1 / 3, then lane 31 into rows 2 and 3.
+__device__ __forceinline__ void wave_scan_step(Affine& x, int step) {
+  switch (step) {
+    case 0: x = compose(x, dpp_affine<0x111>(x)); break;       // row_shr:1
+    case 1: x = compose(x, dpp_affine<0x112>(x)); break;       // row_shr:2
+    case 2: x = compose(x, dpp_affine<0x114>(x)); break;       // row_shr:4
+    case 3: x = compose(x, dpp_affine<0x118>(x)); break;       // row_shr:8
+    case 4: x = compose(x, dpp_affine<0x142, 0xA>(x)); break;  // row_bcast:15 into rows 1 and 3
+    default: x = compose(x, dpp_affine<0x143, 0xC>(x)); break; // row_bcast:31 into rows 2 and 3
+  }
 }
 
 constexpr int kSeg = 1024;  // columns per segment = 256 threads x 4
@@ -94,7 +115,7 @@ __global__ __launch_bounds__(kRcThreads) void gae_scan_kernel(const float* __res
       }
     }
     // The segments of the batch are scanned together: their wavefront scans are independent (the
-    // shuffles of the four interleave), and one pass over the 16 wavefront totals in walk order
+    // exchanges of the four interleave), and one pass over the 16 wavefront totals in walk order
     // then gives every thread the state entering its 4 columns of each segment.
     Affine inc[kSegBatch], exc[kSegBatch];
 #pragma unroll
@@ -117,18 +138,14 @@ __global__ __launch_bounds__(kRcThreads) void gae_scan_kernel(const float* __res
       inc[b] = f;
     }
 #pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
+    for (int step = 0; step < 6; ++step) {
 #pragma unroll
-      for (int b = 0; b < kSegBatch; ++b) {
-        const Affine nb = shfl_up_affine(inc[b], d);
-        if (lane >= d) inc[b] = compose(inc[b], nb);
-      }
+      for (int b = 0; b < kSegBatch; ++b) wave_scan_step(inc[b], step);
     }
 #pragma unroll
     for (int b = 0; b < kSegBatch; ++b) {
       if (lane == 63) wave_tot[par][b][wave] = inc[b];
-      exc[b] = shfl_up_affine(inc[b], 1);
-      if (lane == 0) exc[b] = affine_identity();
+      exc[b] = dpp_affine<0x138>(inc[b]);  // wave_shr:1, the identity into lane 0
     }
     __syncthreads();
     // walk the wavefront totals in order; remember the state where this thread's wavefront starts
