@@ -75,15 +75,17 @@ __device__ __forceinline__ double lane_read(double x, int lane) {
 }
 struct SumOp {
   __device__ __forceinline__ double operator()(double a, double b) const { return a + b; }
+  __device__ __forceinline__ double identity() const { return 0.0; }
 };
 struct MaxOp {
   __device__ __forceinline__ double operator()(double a, double b) const { return fmax(a, b); }
+  __device__ __forceinline__ double identity() const { return -__longlong_as_double(0x7ff0000000000000ll); }
 };
 // Reduce NV values per lane over the wavefront, step-major so the NV chains overlap; the result is in every lane.
 // Steps: partner lane ^ 1 and lane ^ 2 (quad permutes), then the mirrored half row and the mirrored row, whose
 // partners hold the same value as lane ^ 4 and lane ^ 8 would since a quad / half row is uniform by then.
 template <int NV, class Op>
-__device__ __forceinline__ void wave_reduce(double (&v)[NV], Op op) {
+__device__ __forceinline__ void row_reduce(double (&v)[NV], Op op) {  // over each row of 16 lanes
 #pragma unroll
   for (int i = 0; i < NV; ++i) v[i] = op(v[i], lane_exchange<0xB1>(v[i]));   // quad_perm [1,0,3,2]
 #pragma unroll
@@ -92,6 +94,10 @@ __device__ __forceinline__ void wave_reduce(double (&v)[NV], Op op) {
   for (int i = 0; i < NV; ++i) v[i] = op(v[i], lane_exchange<0x141>(v[i]));  // row_half_mirror
 #pragma unroll
   for (int i = 0; i < NV; ++i) v[i] = op(v[i], lane_exchange<0x140>(v[i]));  // row_mirror
+}
+template <int NV, class Op>
+__device__ __forceinline__ void wave_reduce(double (&v)[NV], Op op) {
+  row_reduce<NV>(v, op);
 #pragma unroll
   for (int i = 0; i < NV; ++i)
     v[i] = op(op(lane_read(v[i], 0), lane_read(v[i], 16)), op(lane_read(v[i], 32), lane_read(v[i], 48)));
@@ -102,26 +108,27 @@ __device__ __forceinline__ double wave_sum(double x) {
   return v[0];
 }
 
-// Reduce NV doubles per thread over a workgroup of NT threads; result valid in thread 0.
+// Reduce NV doubles per thread over a workgroup of NT threads; result valid in thread 0.  The wavefront results
+// meet in LDS and the first wavefront combines them with one LDS read per value and a reduction over its first
+// row of lanes: a single thread reading them one after the other would wait out every LDS round trip.
 template <int NV, int NT, class Op>
 __device__ __forceinline__ void block_reduce(double (&v)[NV], double* smem /* NV * NT/64 doubles */, Op op) {
   constexpr int NW = NT / 64;
+  static_assert(NW <= 16, "the wavefront results are combined inside one row of 16 lanes");
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   wave_reduce<NV>(v, op);
   if (lane == 0)
 #pragma unroll
     for (int i = 0; i < NV; ++i) smem[i * NW + w] = v[i];
   __syncthreads();
-  if (threadIdx.x == 0) {
+  if (w == 0) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      double s = smem[i * NW];
-      for (int j = 1; j < NW; ++j) s = op(s, smem[i * NW + j]);
-      v[i] = s;
-    }
+    for (int i = 0; i < NV; ++i) v[i] = lane < NW ? smem[i * NW + lane] : op.identity();
+    row_reduce<NV>(v, op);
   }
   __syncthreads();
 }
+
 template <int NV, int NT>
 __device__ __forceinline__ void block_sum(double (&v)[NV], double* smem) {
   block_reduce<NV, NT>(v, smem, SumOp());

@@ -36,6 +36,8 @@ struct DmArgs {
   int64_t rows, cols, prompt;                       // attention_mask is [rows][prompt + cols]
   int chunks;
   double* records;  // kDmRec slots per (row, chunk) workgroup, slot-major
+  double* shares;   // per workgroup of the fold launch: its 16 sums and 16 maxima
+  unsigned* fold_counter;  // arrivals of the fold launch's workgroups; the streaming pass clears it
   double* out;      // [VAMD_DM_COUNT]
 };
 
@@ -44,6 +46,7 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
                                                                   const A* __restrict__ attention) {
   const int64_t row = blockIdx.x / a.chunks;
   const int chunk = blockIdx.x % a.chunks;
+  if (blockIdx.x == 0 && threadIdx.x == 0) a.fold_counter[0] = 0u;
   const ChunkPos pos(row, chunk, a.cols);
   // per-thread partials over its 16 elements in fp32 (exact counts, 1e-7 relative on the sums), widened below
   float s[kDmSums];
@@ -109,7 +112,8 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
 
 constexpr int kDmFoldThreads = 512;
 
-// One workgroup: records -> per-row quantities -> the output vector.
+// records -> per-row quantities -> the output vector: one row per thread, the workgroups' totals combined by the
+// last of them to finish.
 __global__ __launch_bounds__(kDmFoldThreads) void data_metrics_fold_kernel(DmArgs a) {
   const double inf = __longlong_as_double(0x7ff0000000000000ll);
   __shared__ double smem[16 * (kDmFoldThreads / 64)];
@@ -126,7 +130,8 @@ __global__ __launch_bounds__(kDmFoldThreads) void data_metrics_fold_kernel(DmArg
   double x[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) x[i] = -inf;
-  for (int64_t r = threadIdx.x; r < a.rows; r += kDmFoldThreads) {
+  for (int64_t r = (int64_t)blockIdx.x * kDmFoldThreads + threadIdx.x; r < a.rows;
+       r += (int64_t)gridDim.x * kDmFoldThreads) {
     const int64_t rr[1] = {r};
     const bool have[1] = {true};
     double rec[1][kDmRec];
@@ -157,6 +162,7 @@ __global__ __launch_bounds__(kDmFoldThreads) void data_metrics_fold_kernel(DmArg
   }
   block_sum<9 + kElem, kDmFoldThreads>(t, smem);
   block_max<16, kDmFoldThreads>(x, smem);
+  if (!fold_across_workgroups<9 + kElem, 16, kDmFoldThreads>(t, x, a.shares, a.fold_counter, smem)) return;
   if (threadIdx.x == 0) {
     double* o = a.out;
     const double B = (double)a.rows, na = t[0];
@@ -237,6 +243,12 @@ __global__ __launch_bounds__(kRcThreads) void variance_proxy_rows_kernel(const f
 
 using namespace vamd;
 
+// one row per thread of the fold launch, at most 256 workgroups
+static unsigned dm_fold_workgroups(int64_t batch) {
+  const int64_t n = (batch + kDmFoldThreads - 1) / kDmFoldThreads;
+  return (unsigned)(n < 1 ? 1 : (n > 256 ? 256 : n));
+}
+
 extern "C" int vamd_variance_proxy_rows(const float* advantages, const float* old_log_probs,
                                         const float* sum_pi_squared, const float* is_weights, const void* mask,
                                         int mask_dtype, int64_t batch, int64_t length, double* records,
@@ -264,7 +276,8 @@ extern "C" int vamd_variance_proxy_rows(const float* advantages, const float* ol
 
 extern "C" size_t vamd_data_metrics_workspace_bytes(int64_t batch, int64_t response_length) {
   if (batch <= 0 || response_length <= 0) return 0;
-  return align_up((size_t)batch * chunks_of(response_length) * kDmRec * sizeof(double), 256);
+  return align_up((size_t)batch * chunks_of(response_length) * kDmRec * sizeof(double), 256) +
+         align_up((size_t)dm_fold_workgroups(batch) * 32 * sizeof(double), 256) + 256;
 }
 
 extern "C" int vamd_data_metrics(const float* token_level_scores, const float* token_level_rewards,
@@ -285,7 +298,10 @@ extern "C" int vamd_data_metrics(const float* token_level_scores, const float* t
   a.scores = token_level_scores; a.rewards = token_level_rewards; a.adv = advantages; a.ret = returns; a.val = values;
   a.rows = batch; a.cols = response_length; a.prompt = prompt_length;
   a.chunks = (int)chunks_of(response_length);
-  a.records = static_cast<double*>(workspace);
+  Carver carve(workspace);
+  a.records = carve.take<double>((size_t)batch * a.chunks * kDmRec);
+  a.shares = carve.take<double>((size_t)dm_fold_workgroups(batch) * 32);
+  a.fold_counter = carve.take<unsigned>(1);
   a.out = out;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)(batch * a.chunks)), block(kRcThreads);
@@ -309,7 +325,7 @@ extern "C" int vamd_data_metrics(const float* token_level_scores, const float* t
     default: set_error("unknown mask dtype code %d", attention_dtype); return VAMD_EINVAL;
   }
 #undef VAMD_DM
-  hipLaunchKernelGGL(data_metrics_fold_kernel, dim3(1), dim3(kDmFoldThreads), 0, s, a);
+  hipLaunchKernelGGL(data_metrics_fold_kernel, dim3(dm_fold_workgroups(batch)), dim3(kDmFoldThreads), 0, s, a);
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }

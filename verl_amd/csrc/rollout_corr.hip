@@ -43,7 +43,9 @@ struct RcArgs {
   int normalize;
   float* weights;      // [rows][cols] or null
   double* records;     // kRcRec slots per (row, chunk) workgroup, slot-major
-  float* row_weight;   // [rows]: sequence-level weight, truncated (and normalised)
+  float* row_weight;   // [rows]: sequence-level weight, truncated (the broadcast divides by `factor`)
+  double* shares;      // per workgroup of the fold launch: its 26 sums and 9 maxima
+  unsigned* fold_counter;  // arrivals of the fold launch's workgroups; the streaming pass clears it
   float* factor;       // [1]: batch-normalisation divisor for the token-level weights (1 when not applied)
   double* out;         // [VAMD_RC_COUNT]
 };
@@ -57,6 +59,7 @@ template <bool VEC, class M>
 __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, const M* __restrict__ mask) {
   const int64_t row = blockIdx.x / a.chunks;
   const int chunk = blockIdx.x % a.chunks;
+  if (blockIdx.x == 0 && threadIdx.x == 0) a.fold_counter[0] = 0u;
   const ChunkPos pos(row, chunk, a.cols);
   float s[kRcSums];
 #pragma unroll
@@ -117,7 +120,8 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
 
 constexpr int kRcFoldThreads = 512;
 
-// One workgroup: records -> per-sequence quantities -> the metric vector (and the per-row weights).
+// records -> per-sequence quantities -> the metric vector (and the per-row weights): one row per thread, the
+// workgroups' totals combined by the last of them to finish.
 __global__ __launch_bounds__(kRcFoldThreads) void rollout_fold_kernel(RcArgs a) {
   const double inf = __longlong_as_double(0x7ff0000000000000ll);
   __shared__ double smem[26 * (kRcFoldThreads / 64)];
@@ -137,7 +141,8 @@ __global__ __launch_bounds__(kRcFoldThreads) void rollout_fold_kernel(RcArgs a) 
   for (int i = 0; i < xN; ++i) x[i] = -inf;
   const float log_hi = logf(a.thr), log_lo = logf(a.lower);
   const bool seq_level = a.level == VAMD_IS_SEQUENCE;
-  for (int64_t r = threadIdx.x; r < a.rows; r += kRcFoldThreads) {
+  for (int64_t r = (int64_t)blockIdx.x * kRcFoldThreads + threadIdx.x; r < a.rows;
+       r += (int64_t)gridDim.x * kRcFoldThreads) {
     const int64_t rr[1] = {r};
     const bool have[1] = {true};
     double rec[1][kRcRec];
@@ -195,7 +200,7 @@ __global__ __launch_bounds__(kRcFoldThreads) void rollout_fold_kernel(RcArgs a) 
   static_assert(tN <= 26, "smem is sized for 26 sums");
   block_sum<tN, kRcFoldThreads>(t, smem);
   block_max_f64<xN, kRcFoldThreads>(x, smem);
-  __shared__ float norm;
+  if (!fold_across_workgroups<tN, xN, kRcFoldThreads>(t, x, a.shares, a.fold_counter, smem)) return;
   if (threadIdx.x == 0) {
     double* o = a.out;
     const double B = (double)a.rows, Mt = t[tM];
@@ -248,23 +253,21 @@ __global__ __launch_bounds__(kRcFoldThreads) void rollout_fold_kernel(RcArgs a) 
       }
     }
     a.factor[0] = divisor;
-    norm = divisor;
   }
-  __syncthreads();
-  if (seq_level && norm != 1.f)
-    for (int64_t r = threadIdx.x; r < a.rows; r += kRcFoldThreads) a.row_weight[r] = a.row_weight[r] / norm;
 }
 
-// weights[i][t] = row_weight[i] * mask[i][t]
+// weights[i][t] = row_weight[i] / factor * mask[i][t]  (the division is skipped when the factor is 1)
 template <bool VEC, class M>
 __global__ __launch_bounds__(kRcThreads) void rollout_broadcast_kernel(const float* __restrict__ row_weight,
+                                                                       const float* __restrict__ factor,
                                                                        const M* __restrict__ mask, int64_t cols,
                                                                        int chunks, float* __restrict__ weights) {
   const int64_t row = blockIdx.x / chunks;
   const ChunkPos pos(row, blockIdx.x % chunks, cols);
   float m[kGroups][4];
   load_mask_groups<VEC>(mask, pos, m);
-  const float w = row_weight[row];
+  const float f = factor[0];
+  const float w = f != 1.f ? row_weight[row] / f : row_weight[row];
 #pragma unroll
   for (int k = 0; k < kGroups; ++k)
 #pragma unroll
@@ -287,10 +290,18 @@ __global__ __launch_bounds__(256) void rollout_divide_kernel(float* __restrict__
 
 using namespace vamd;
 
+// one row per thread of the fold launch, at most 256 workgroups, each leaving 26 sums and 9 maxima
+constexpr size_t kRcShareSlots = 26 + 9;
+static unsigned rc_fold_workgroups(int64_t batch) {
+  const int64_t n = (batch + kRcFoldThreads - 1) / kRcFoldThreads;
+  return (unsigned)(n < 1 ? 1 : (n > 256 ? 256 : n));
+}
+
 extern "C" size_t vamd_rollout_correction_workspace_bytes(int64_t batch, int64_t length) {
   if (batch <= 0 || length <= 0) return 0;
   return align_up((size_t)batch * chunks_of(length) * kRcRec * sizeof(double), 256) +
-         align_up((size_t)batch * sizeof(float), 256) + 256;
+         align_up((size_t)batch * sizeof(float), 256) + 256 +
+         align_up((size_t)rc_fold_workgroups(batch) * kRcShareSlots * sizeof(double), 256) + 256;
 }
 
 extern "C" int vamd_rollout_correction(const float* old_log_prob, const float* rollout_log_prob, const void* mask,
@@ -318,6 +329,8 @@ extern "C" int vamd_rollout_correction(const float* old_log_prob, const float* r
   a.records = carve.take<double>((size_t)batch * a.chunks * kRcRec);
   a.row_weight = carve.take<float>((size_t)batch);
   a.factor = carve.take<float>(1);
+  a.shares = carve.take<double>((size_t)rc_fold_workgroups(batch) * kRcShareSlots);
+  a.fold_counter = carve.take<unsigned>(1);
   a.out = metrics;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)(batch * a.chunks)), block(kRcThreads);
@@ -328,14 +341,14 @@ extern "C" int vamd_rollout_correction(const float* old_log_prob, const float* r
       hipLaunchKernelGGL((rollout_stats_kernel<true, M>), grid, block, 0, s, a, mk);
     else
       hipLaunchKernelGGL((rollout_stats_kernel<false, M>), grid, block, 0, s, a, mk);
-    hipLaunchKernelGGL(rollout_fold_kernel, dim3(1), dim3(kRcFoldThreads), 0, s, a);
+    hipLaunchKernelGGL(rollout_fold_kernel, dim3(rc_fold_workgroups(batch)), dim3(kRcFoldThreads), 0, s, a);
     if (level == VAMD_IS_SEQUENCE) {
       if (vec)
-        hipLaunchKernelGGL((rollout_broadcast_kernel<true, M>), grid, block, 0, s, a.row_weight, mk, length, a.chunks,
-                           weights);
-      else
-        hipLaunchKernelGGL((rollout_broadcast_kernel<false, M>), grid, block, 0, s, a.row_weight, mk, length,
+        hipLaunchKernelGGL((rollout_broadcast_kernel<true, M>), grid, block, 0, s, a.row_weight, a.factor, mk, length,
                            a.chunks, weights);
+      else
+        hipLaunchKernelGGL((rollout_broadcast_kernel<false, M>), grid, block, 0, s, a.row_weight, a.factor, mk,
+                           length, a.chunks, weights);
     }
   });
   if (level == VAMD_IS_TOKEN && batch_normalize) {

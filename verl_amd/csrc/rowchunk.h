@@ -325,6 +325,47 @@ __device__ __forceinline__ bool sum_all_records(unsigned* counters, double* __re
 // Doubles a record area needs behind its rows * chunks * nv record slots for sum_all_records().
 constexpr size_t kShareSlots = kTicketGroups;
 
+// Cross-workgroup step of a fold launch that gives every workgroup a share of the rows: on entry thread 0 of each
+// workgroup holds NS sums and NX maxima of its share; returns true in exactly one workgroup, whose thread 0 then
+// holds them over all shares (a launch of one workgroup returns at once).  shares: gridDim.x * (NS + NX) doubles;
+// counter: zero when the launch starts (the streaming pass before it clears it).
+template <int NS, int NX, int NT>
+__device__ __forceinline__ bool fold_across_workgroups(double (&t)[NS], double (&x)[NX], double* __restrict__ shares,
+                                                       unsigned* counter, double* smem /* max(NS, NX) * NT/64 */) {
+  const unsigned nb = gridDim.x;
+  if (nb == 1) return true;
+  __shared__ unsigned last;
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < NS; ++i) peer_store(shares + (size_t)i * nb + blockIdx.x, t[i]);
+#pragma unroll
+    for (int i = 0; i < NX; ++i) peer_store(shares + (size_t)(NS + i) * nb + blockIdx.x, x[i]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    last = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == nb - 1 ? 1u : 0u;
+  }
+  __syncthreads();
+  if (!last) return false;
+  const double ninf = -__longlong_as_double(0x7ff0000000000000ll);
+#pragma unroll
+  for (int i = 0; i < NS; ++i) t[i] = 0.0;
+#pragma unroll
+  for (int i = 0; i < NX; ++i) x[i] = ninf;
+  for (unsigned b = threadIdx.x; b < nb; b += NT) {
+    double ts[NS], xs[NX];
+#pragma unroll
+    for (int i = 0; i < NS; ++i) ts[i] = peer_load(shares + (size_t)i * nb + b);
+#pragma unroll
+    for (int i = 0; i < NX; ++i) xs[i] = peer_load(shares + (size_t)(NS + i) * nb + b);
+#pragma unroll
+    for (int i = 0; i < NS; ++i) t[i] += ts[i];
+#pragma unroll
+    for (int i = 0; i < NX; ++i) x[i] = fmax(x[i], xs[i]);
+  }
+  block_reduce<NS, NT>(t, smem, SumOp());
+  block_reduce<NX, NT>(x, smem, MaxOp());
+  return true;
+}
+
 // (mean, rsqrt(var_unbiased + 1e-8), shift) from the masked moments sum(m), sum(v m), sum(v^2 m),
 // following masked_mean / masked_var / masked_whiten (verl/utils/torch_functional.py:287-339).
 __device__ __forceinline__ void whiten_stats_from_moments(double s0, double s1, double s2, int shift_mean,
