@@ -57,7 +57,7 @@ def test_masked_mean_reference_vectors(dev, value, mask, want):
         assert torch.allclose(got.cpu(), torch.tensor(want), equal_nan=True)
 
 
-@pytest.mark.parametrize("shape", [(7, 33), (64, 4096), (3, 5000), (1, 100003)])
+@pytest.mark.parametrize("shape", [(7, 33), (64, 4096), (3, 5000), (1, 100003), (1100, 16000)])   # last: 4400 records
 @pytest.mark.parametrize("mdtype", [torch.float32, torch.int64, torch.bool, torch.int32])
 def test_masked_reductions(dev, shape, mdtype):
     from verl_amd.utils import torch_functional as F
@@ -431,6 +431,47 @@ def test_grpo_passk(dev, batch_size, seq_len, num_groups, seed, norm):
     with pytest.raises(AssertionError):
         CA.compute_grpo_passk_outcome_advantage(rewards.to(dev), mask.to(dev), index)
     assert CA.get_adv_estimator_fn("grpo_passk") is CA.compute_grpo_passk_outcome_advantage
+
+
+# (batch, length, groups, seed, shuffled): which statistics path a launch takes depends on the number of
+# (row, chunk) records, of groups and of rows
+_STAT_LAUNCH_CASES = [
+    (1500, 4100, 200, 7, True),     # 3000 records: statistics in a launch of their own, rows held in registers
+    (2500, 70, 300, 8, True),       # more rows than that launch holds: scores and group ids are read back
+    (1300, 90, 600, 9, True),       # few records but more groups than the streaming pass keeps LDS for
+    (1500, 100, 100, 10, True),     # same launch, more rows than its last workgroup holds
+    (122, 50, 10, 11, False),       # 61 divides the row count; responses of a group adjacent
+    (61 * 59, 40, 59, 12, False),   # so do 61 and 59
+    (512, 4096, 64, 13, False),     # the benchmark layout: 64 adjacent groups of 8
+]
+
+
+@pytest.mark.parametrize("batch_size,seq_len,num_groups,seed,shuffled", _STAT_LAUNCH_CASES)
+def test_group_estimators_on_every_statistics_path(dev, batch_size, seq_len, num_groups, seed, shuffled):
+    from verl_amd.trainer.ppo import core_algos as CA
+    torch.manual_seed(seed); random.seed(seed); np.random.seed(seed)
+    if shuffled:
+        index = _make_group_index(batch_size, num_groups)
+    else:
+        index = np.sort(_make_group_index(batch_size, num_groups))
+    mask = _rand_mask(batch_size, seq_len)
+    rewards = torch.randn(batch_size, seq_len) * mask
+    rewards[5] = 0
+    rd, md = rewards.to(dev), mask.to(dev)
+    got, _ = CA.compute_grpo_outcome_advantage(rd, md, index)
+    want, _ = O.grpo_outcome_advantage(rewards.clone(), mask, index)
+    _close(got, want, atol=2e-5, what="grpo")
+    assert torch.equal(got.cpu() == 0, want == 0)
+    for fn, oracle_fn, kw in _GROUP_ESTIMATORS:
+        got, _ = getattr(CA, fn)(rd, md, index, **kw)
+        want, _ = getattr(O, oracle_fn)(rewards.clone(), mask, index, **kw)
+        _close(got, want, atol=2e-5, what=fn)
+    for norm in (True, False):
+        cfg = _cfg(norm_adv_by_std_in_grpo=norm)
+        got, _ = CA.compute_grpo_passk_outcome_advantage(rd, md, index, config=cfg)
+        want, _ = O.grpo_passk_outcome_advantage(rewards.clone(), mask, index, norm_by_std=norm)
+        _close(got, want, atol=2e-5, what="pass@k")
+        assert torch.equal(got.cpu() != 0, want != 0)
 
 
 @pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192)])
@@ -1022,7 +1063,8 @@ def test_data_metrics_reference_mock_batch(dev):
                                         "critic/vf_explained_var"}
 
 
-@pytest.mark.parametrize("shape,prompt", [((3, 17), 5), ((16, 1024), 256), ((5, 4099), 33), ((64, 8192), 1024)])
+@pytest.mark.parametrize("shape,prompt", [((3, 17), 5), ((16, 1024), 256), ((5, 4099), 33), ((64, 8192), 1024),
+                                          ((1300, 300), 40)])              # the last: several fold workgroups
 @pytest.mark.parametrize("mdtype", [torch.float32, torch.int64, torch.bool])
 @pytest.mark.parametrize("use_critic", [True, False])
 def test_data_metrics(dev, shape, prompt, mdtype, use_critic):
@@ -1088,7 +1130,7 @@ def _rc_check(got, want32, want64, what):
         assert err <= max(2 * abs(want32[key] - want64[key]), 2e-5 * max(1.0, abs(want64[key]))), (what, key, got[key], want64[key])
 
 
-@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192)])
+@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192), (1300, 300)])
 @pytest.mark.parametrize("level,spread", [("token", 0.5), ("sequence", 0.02)])
 @pytest.mark.parametrize("normalize", [False, True])
 @pytest.mark.parametrize("mdtype", [torch.float32, torch.int64])
