@@ -78,6 +78,9 @@ extern "C" {
 #define VAMD_RETURNS_REMAX 0        /* returns = reverse cumsum of r m; adv = returns - baseline_i m */
 #define VAMD_RETURNS_REINFORCE_PP 1 /* R_t = r_t + gamma c, c <- R_t m_t; adv = masked_whiten(R, m) m */
 
+/* Bumped whenever an entry point changes its signature or a workspace its layout; a binding compares it with
+ * the header it was written against. */
+#define VAMD_ABI_VERSION 3
 int vamd_abi_version(void);
 const char* vamd_last_error(void);
 

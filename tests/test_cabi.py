@@ -33,7 +33,9 @@ def test_every_declared_symbol_is_exported_and_bound(lib):
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/verl_amd.h but not exported"
     assert sorted(_cabi.SIGNATURES) == declared, "ctypes prototypes and header disagree"
-    assert lib.vamd_abi_version() == 3
+    assert lib.vamd_abi_version() == _cabi.ABI_VERSION
+    header = open(os.path.join(os.path.dirname(__file__), "..", "include", "verl_amd.h")).read()
+    assert f"#define VAMD_ABI_VERSION {_cabi.ABI_VERSION}\n" in header
 
 
 def test_workspace_queries(lib):

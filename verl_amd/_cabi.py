@@ -117,6 +117,9 @@ def lib_path() -> str:
     return _LIB_PATH
 
 
+ABI_VERSION = 3  # VAMD_ABI_VERSION of include/verl_amd.h
+
+
 def load_library(path: str | None = None) -> ctypes.CDLL:
     """dlopen the library and attach prototypes.  Raises if it has not been built."""
     path = path or _LIB_PATH
@@ -130,6 +133,9 @@ def load_library(path: str | None = None) -> ctypes.CDLL:
         fn = getattr(lib, name)  # AttributeError names the missing symbol
         fn.restype = res
         fn.argtypes = args
+    if lib.vamd_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"{path} reports ABI version {lib.vamd_abi_version()}, these bindings are written for "
+                           f"{ABI_VERSION}: rebuild it with `python -m verl_amd.csrc.build`")
     return lib
 
 

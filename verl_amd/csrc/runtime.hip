@@ -84,5 +84,5 @@ extern "C" int vamd_sum4(const float* a, const float* b, const float* c, const f
   return VAMD_OK;
 }
 
-extern "C" int vamd_abi_version(void) { return 3; }
+extern "C" int vamd_abi_version(void) { return VAMD_ABI_VERSION; }
 extern "C" const char* vamd_last_error(void) { return vamd::g_error; }
