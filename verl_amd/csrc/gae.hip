@@ -35,12 +35,6 @@ __device__ __forceinline__ Affine compose(const Affine& later, const Affine& ear
   return o;
 }
 
-// Lane exchange inside the vector ALU (data-parallel primitives): a lane without a source in the pattern, or in a
-// row the mask leaves out, receives `none`.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float dpp_f32(float x, float none) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(none), __float_as_int(x), CTRL, ROW_MASK, 0xF, false));
-}
 // The map of the lane the pattern names, the identity where there is none (composing with it changes nothing,
 // so the scan needs no lane test).
 template <int CTRL, int ROW_MASK = 0xF>

@@ -10,7 +10,7 @@
 //
 // Two launches.  The first walks every row twice inside one workgroup -- right to left for the
 // returns, left to right for W -- as plain prefix sums carried in double (1024-column segments,
-// 4 columns per thread, wavefront shuffle scan plus the four wavefront totals through LDS).  The
+// 4 columns per thread, wavefront scan by lane exchanges plus the four wavefront totals through LDS).  The
 // second gives each (group, 4096-column chunk) to one workgroup, which adds up the group's rows
 // column by column in index order, forms the baseline and writes the advantages of those rows.
 // Nothing is reduced across workgroups, so neither launch needs arrival counters.
@@ -25,12 +25,6 @@
 namespace vamd {
 
 constexpr int kOtbSeg = 1024;
-
-__device__ __forceinline__ double shfl_up_f64(double x, int d) {
-  const unsigned long long u = __double_as_longlong(x);
-  const unsigned lo = __shfl_up((unsigned)u, d, 64), hi = __shfl_up((unsigned)(u >> 32), d, 64);
-  return __longlong_as_double(((unsigned long long)hi << 32) | lo);
-}
 
 // Running sum along one row in walk order (REVERSE: last column first).  load(col0, valid, v[4])
 // fills the 4 values at col0 .. col0 + 3 (0 beyond `valid`); store(col0, valid, out[4]) receives
@@ -57,12 +51,7 @@ __device__ __forceinline__ double row_running_sum(int64_t cols, double (*wave_to
       run += (double)v[e];
       inc[e] = run;
     }
-    double scan = run;  // inclusive scan of the thread totals over the wavefront
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-      const double nb = shfl_up_f64(scan, d);
-      if (lane >= d) scan += nb;
-    }
+    const double scan = wave_running_sum(run);  // inclusive scan of the thread totals over the wavefront
     if (lane == 63) wave_tot[par][wave] = scan;
     __syncthreads();
     double before = carry + (scan - run);

@@ -9,7 +9,7 @@
 // Both carry one value y leftwards through the affine step y' = a_t y + b_t
 // (ReMax: a = 1, b = r m, output y';  REINFORCE++: a = gamma m, b = r m, output r + gamma y), and
 // affine steps compose associatively, so a row is scanned like the GAE kernel scans its pairs:
-// 1024-column segments right to left, 4 columns per thread, a wavefront shuffle scan plus an LDS
+// 1024-column segments right to left, 4 columns per thread, a wavefront scan by lane exchanges plus an LDS
 // pass over the 4 wavefront totals, loads of four segments issued together.  The workgroup that
 // finishes last folds the per-row masked moments of the returns into whitening statistics; a second
 // streaming kernel forms the advantages.
@@ -85,15 +85,15 @@ __global__ __launch_bounds__(kRcThreads) void returns_scan_kernel(const float* _
           f = compose(s, f);
         }
       }
-      Step inc = f;
-#pragma unroll
-      for (int d = 1; d < 64; d <<= 1) {
-        const Step nb{__shfl_up(inc.a, d, 64), __shfl_up(inc.b, d, 64)};
-        if (lane >= d) inc = compose(inc, nb);
-      }
+      Step inc = f;  // inclusive scan over the wavefront; a lane without a source composes with the identity
+      inc = compose(inc, Step{dpp_f32<0x111>(inc.a, 1.f), dpp_f32<0x111>(inc.b, 0.f)});
+      inc = compose(inc, Step{dpp_f32<0x112>(inc.a, 1.f), dpp_f32<0x112>(inc.b, 0.f)});
+      inc = compose(inc, Step{dpp_f32<0x114>(inc.a, 1.f), dpp_f32<0x114>(inc.b, 0.f)});
+      inc = compose(inc, Step{dpp_f32<0x118>(inc.a, 1.f), dpp_f32<0x118>(inc.b, 0.f)});
+      inc = compose(inc, Step{dpp_f32<0x142, 0xA>(inc.a, 1.f), dpp_f32<0x142, 0xA>(inc.b, 0.f)});
+      inc = compose(inc, Step{dpp_f32<0x143, 0xC>(inc.a, 1.f), dpp_f32<0x143, 0xC>(inc.b, 0.f)});
       if (lane == 63) wave_tot[par][wave] = inc;
-      Step exc{__shfl_up(inc.a, 1, 64), __shfl_up(inc.b, 1, 64)};
-      if (lane == 0) exc = Step{1.f, 0.f};
+      const Step exc{dpp_f32<0x138>(inc.a, 1.f), dpp_f32<0x138>(inc.b, 0.f)};  // the lane before; identity into lane 0
       __syncthreads();
       float y = carry[par];
       for (int k = 0; k < wave; ++k) y = fmaf(wave_tot[par][k].a, y, wave_tot[par][k].b);

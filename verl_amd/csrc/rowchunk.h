@@ -196,6 +196,32 @@ __device__ __forceinline__ void ticket_reset(unsigned* counters) {
     __hip_atomic_store(counters + threadIdx.x * (kTicketStride / 4), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Lane exchange inside the vector ALU (data-parallel primitives): a lane without a source in the pattern, or in a
+// row the mask leaves out, receives `none`.  The wavefront scans use the shifts by 1, 2, 4, 8 inside a row of 16
+// lanes (0x111 .. 0x118), the last lane of rows 0 / 2 into rows 1 / 3 (0x142, row mask 0xA), lane 31 into rows 2
+// and 3 (0x143, row mask 0xC), and the shift by one lane over the whole wavefront (0x138); with `none` the identity
+// of the scanned operation no lane test is needed.
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dpp_f32(float x, float none) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(none), __float_as_int(x), CTRL, ROW_MASK, 0xF, false));
+}
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ double dpp_f64(double x, double none) {
+  const int lo = __builtin_amdgcn_update_dpp(__double2loint(none), __double2loint(x), CTRL, ROW_MASK, 0xF, false);
+  const int hi = __builtin_amdgcn_update_dpp(__double2hiint(none), __double2hiint(x), CTRL, ROW_MASK, 0xF, false);
+  return __hiloint2double(hi, lo);
+}
+// Inclusive running sum over the wavefront, lane 0 first.
+__device__ __forceinline__ double wave_running_sum(double x) {
+  x += dpp_f64<0x111>(x, 0.0);
+  x += dpp_f64<0x112>(x, 0.0);
+  x += dpp_f64<0x114>(x, 0.0);
+  x += dpp_f64<0x118>(x, 0.0);
+  x += dpp_f64<0x142, 0xA>(x, 0.0);
+  x += dpp_f64<0x143, 0xC>(x, 0.0);
+  return x;
+}
+
 // Records of the (row, chunk) workgroups are kept slot-major: slot i of workgroup (row, chunk) lives at
 // ((i * chunks + chunk) * rows + row).  The workgroup that folds them gives consecutive rows to consecutive threads,
 // so a wavefront's loads of one slot are 512 contiguous bytes; with one record per workgroup stored contiguously
