@@ -62,7 +62,8 @@ def cpu_baseline(n_cpu: int, h: int, v: int, temperature: float) -> dict:
 
 def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> dict:
     """The [B, L] kernels (B = 512, L = 4096 is the size of the GRPO / policy-loss and GAE benchmark configurations): microseconds per call from HIP events
-    over 40 calls (best of three such loops) that rotate through 8 buffer sets (more than the 256 MB Infinity Cache), the algorithmic bytes of
+    over 48 calls (best of three such loops) that rotate through 8 buffer sets, 16 at the smaller size (so that even the two-tensor ops
+    touch more than the 256 MB Infinity Cache before they come back to a set), the algorithmic bytes of
     the op, and the fraction of 8 TB/s that gives.  ``cpu_ms`` is the CPU oracle on one buffer set."""
     import torch
 
@@ -70,8 +71,8 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
     from verl_amd import _cabi
 
     L = _cabi.lib()
-    nset = 8
     BL = B * Lc
+    nset = 16 if BL * 4 * 2 * 8 < (300 << 20) else 8   # two fp32 tensors per set must add up to more than the cache
     g = torch.Generator(device=dev).manual_seed(0)
 
     def mk():
@@ -184,7 +185,7 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
         for s in sets:
             fn(s)
         torch.cuda.synchronize()
-        reps = 40
+        reps = 48
         us = float("inf")
         for _ in range(3):   # best of three timed loops: a host hiccup between launches shows up as GPU idle time
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
