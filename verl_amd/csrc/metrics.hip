@@ -34,8 +34,9 @@ __device__ __forceinline__ void block_max(double (&v)[NV], double* smem /* NV * 
 struct DmArgs {
   const float *scores, *rewards, *adv, *ret, *val;  // val may be null
   int64_t rows, cols, prompt;                       // attention_mask is [rows][prompt + cols]
-  int chunks;
-  double* records;  // kDmRec slots per (row, chunk) workgroup, slot-major
+  int chunks;       // records per row: spans of `span` 4096-column chunks
+  int span;
+  double* records;  // kDmRec slots per (row, span) workgroup, slot-major
   double* shares;   // per workgroup of the fold launch: its 16 sums and 16 maxima
   unsigned* fold_counter;  // arrivals of the fold launch's workgroups; the streaming pass clears it
   double* out;      // [VAMD_DM_COUNT]
@@ -47,14 +48,20 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
   const int64_t row = blockIdx.x / a.chunks;
   const int chunk = blockIdx.x % a.chunks;
   if (blockIdx.x == 0 && threadIdx.x == 0) a.fold_counter[0] = 0u;
-  const ChunkPos pos(row, chunk, a.cols);
-  // per-thread partials over its 16 elements in fp32 (exact counts, 1e-7 relative on the sums), widened below
-  float s[kDmSums];
+  // A workgroup walks a.span consecutive 4096-column chunks of its row and leaves one record (a.chunks counts
+  // those spans): the workgroup reduction of a record this wide costs more vector-ALU time than streaming one chunk.
+  double acc[kDmSums];
 #pragma unroll
-  for (int i = 0; i < kDmSums; ++i) s[i] = 0.f;
+  for (int i = 0; i < kDmSums; ++i) acc[i] = 0.0;
   float hi[3] = {-__builtin_inff(), -__builtin_inff(), -__builtin_inff()};  // adv, ret, val
   float lo[3] = {__builtin_inff(), __builtin_inff(), __builtin_inff()};
   const int64_t att_row = row * (a.prompt + a.cols) + a.prompt;
+  for (int u = 0; u < a.span; ++u) {
+  const ChunkPos pos(row, chunk * a.span + u, a.cols);
+  // per-thread partials over its 16 elements in fp32 (exact counts, 1e-7 relative on the sums), widened per chunk
+  float s[kDmSums];
+#pragma unroll
+  for (int i = 0; i < kDmSums; ++i) s[i] = 0.f;
 #pragma unroll 2
   for (int k = 0; k < kGroups; ++k) {
     if (pos.valid[k] <= 0) continue;
@@ -89,14 +96,16 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
       }
     }
   }
+#pragma unroll
+  for (int i = 0; i < kDmSums; ++i) acc[i] += (double)s[i];
+  }
   if (chunk == 0) {
     const int64_t p0 = row * (a.prompt + a.cols);
-    for (int64_t c = threadIdx.x; c < a.prompt; c += kRcThreads) s[kDmPromptLen] += (float)attention[p0 + c];
+    float prompt_len = 0.f;
+    for (int64_t c = threadIdx.x; c < a.prompt; c += kRcThreads) prompt_len += (float)attention[p0 + c];
+    acc[kDmPromptLen] += (double)prompt_len;
   }
   __shared__ double smem[kDmSums * 4];
-  double acc[kDmSums];
-#pragma unroll
-  for (int i = 0; i < kDmSums; ++i) acc[i] = s[i];
   block_sum<kDmSums, kRcThreads>(acc, smem);
   double ext[6] = {hi[0], -(double)lo[0], hi[1], -(double)lo[1], hi[2], -(double)lo[2]};
   block_max<6, kRcThreads>(ext, smem);
@@ -110,13 +119,15 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
   }
 }
 
-constexpr int kDmFoldThreads = 512;
+constexpr int kDmFoldThreads = 512;       // a batch of up to this many rows is folded by one workgroup
+constexpr int kDmFoldThreadsWide = 128;   // wider batches: one row per thread of many small workgroups, then their totals
 
 // records -> per-row quantities -> the output vector: one row per thread, the workgroups' totals combined by the
 // last of them to finish.
-__global__ __launch_bounds__(kDmFoldThreads) void data_metrics_fold_kernel(DmArgs a) {
+template <int NT>
+__global__ __launch_bounds__(NT) void data_metrics_fold_kernel(DmArgs a) {
   const double inf = __longlong_as_double(0x7ff0000000000000ll);
-  __shared__ double smem[16 * (kDmFoldThreads / 64)];
+  __shared__ double smem[16 * (NT / 64)];
   // ---- fold: thread-strided over rows -------------------------------------------------------------
   // sums: 0 n_non_aborted 1 score 2 reward 3 resp_len 4 resp_len==cols 5 resp_len (non-aborted)
   //       6 resp_len==cols (non-aborted) 7 prompt_len 8 prompt_len==prompt
@@ -130,8 +141,8 @@ __global__ __launch_bounds__(kDmFoldThreads) void data_metrics_fold_kernel(DmArg
   double x[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) x[i] = -inf;
-  for (int64_t r = (int64_t)blockIdx.x * kDmFoldThreads + threadIdx.x; r < a.rows;
-       r += (int64_t)gridDim.x * kDmFoldThreads) {
+  for (int64_t r = (int64_t)blockIdx.x * NT + threadIdx.x; r < a.rows;
+       r += (int64_t)gridDim.x * NT) {
     const int64_t rr[1] = {r};
     const bool have[1] = {true};
     double rec[1][kDmRec];
@@ -160,9 +171,9 @@ __global__ __launch_bounds__(kDmFoldThreads) void data_metrics_fold_kernel(DmArg
       x[6] = fmax(x[6], rl); x[7] = fmax(x[7], -rl);
     }
   }
-  block_sum<9 + kElem, kDmFoldThreads>(t, smem);
-  block_max<16, kDmFoldThreads>(x, smem);
-  if (!fold_across_workgroups<9 + kElem, 16, kDmFoldThreads>(t, x, a.shares, a.fold_counter, smem)) return;
+  block_sum<9 + kElem, NT>(t, smem);
+  block_max<16, NT>(x, smem);
+  if (!fold_across_workgroups<9 + kElem, 16, NT>(t, x, a.shares, a.fold_counter, smem)) return;
   if (threadIdx.x == 0) {
     double* o = a.out;
     const double B = (double)a.rows, na = t[0];
@@ -245,8 +256,9 @@ using namespace vamd;
 
 // one row per thread of the fold launch, at most 256 workgroups
 static unsigned dm_fold_workgroups(int64_t batch) {
-  const int64_t n = (batch + kDmFoldThreads - 1) / kDmFoldThreads;
-  return (unsigned)(n < 1 ? 1 : (n > 256 ? 256 : n));
+  if (batch <= kDmFoldThreads) return 1;
+  const int64_t n = (batch + kDmFoldThreadsWide - 1) / kDmFoldThreadsWide;
+  return (unsigned)(n > 256 ? 256 : n);
 }
 
 extern "C" int vamd_variance_proxy_rows(const float* advantages, const float* old_log_probs,
@@ -297,7 +309,8 @@ extern "C" int vamd_data_metrics(const float* token_level_scores, const float* t
   DmArgs a;
   a.scores = token_level_scores; a.rewards = token_level_rewards; a.adv = advantages; a.ret = returns; a.val = values;
   a.rows = batch; a.cols = response_length; a.prompt = prompt_length;
-  a.chunks = (int)chunks_of(response_length);
+  a.span = record_span(batch, (int)chunks_of(response_length));
+  a.chunks = ((int)chunks_of(response_length) + a.span - 1) / a.span;
   Carver carve(workspace);
   a.records = carve.take<double>((size_t)batch * a.chunks * kDmRec);
   a.shares = carve.take<double>((size_t)dm_fold_workgroups(batch) * 32);
@@ -325,7 +338,11 @@ extern "C" int vamd_data_metrics(const float* token_level_scores, const float* t
     default: set_error("unknown mask dtype code %d", attention_dtype); return VAMD_EINVAL;
   }
 #undef VAMD_DM
-  hipLaunchKernelGGL(data_metrics_fold_kernel, dim3(dm_fold_workgroups(batch)), dim3(kDmFoldThreads), 0, s, a);
+  if (dm_fold_workgroups(batch) == 1)
+    hipLaunchKernelGGL(data_metrics_fold_kernel<kDmFoldThreads>, dim3(1), dim3(kDmFoldThreads), 0, s, a);
+  else
+    hipLaunchKernelGGL(data_metrics_fold_kernel<kDmFoldThreadsWide>, dim3(dm_fold_workgroups(batch)),
+                       dim3(kDmFoldThreadsWide), 0, s, a);
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }

@@ -37,7 +37,8 @@ constexpr int kRcSums = kRcWMax;
 struct RcArgs {
   const float *old_lp, *roll_lp;  // roll_lp may be null: only the training perplexity is produced
   int64_t rows, cols;
-  int chunks;
+  int chunks;          // records per row: spans of `span` 4096-column chunks
+  int span;
   int level;  // VAMD_IS_*
   float thr, lower;
   int normalize;
@@ -60,12 +61,17 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
   const int64_t row = blockIdx.x / a.chunks;
   const int chunk = blockIdx.x % a.chunks;
   if (blockIdx.x == 0 && threadIdx.x == 0) a.fold_counter[0] = 0u;
-  const ChunkPos pos(row, chunk, a.cols);
-  float s[kRcSums];
+  // A workgroup walks a.span consecutive 4096-column chunks of its row and leaves one record (a.chunks counts
+  // those spans): the workgroup reduction of a record this wide costs more vector-ALU time than streaming one chunk.
+  double acc[kRcSums];
 #pragma unroll
-  for (int i = 0; i < kRcSums; ++i) s[i] = 0.f;
+  for (int i = 0; i < kRcSums; ++i) acc[i] = 0.0;
   float wmax = -__builtin_inff(), wmin = __builtin_inff();
-  {
+  for (int u = 0; u < a.span; ++u) {
+    const ChunkPos pos(row, chunk * a.span + u, a.cols);
+    float s[kRcSums];  // per-thread partials over 16 elements in fp32, widened after every chunk
+#pragma unroll
+    for (int i = 0; i < kRcSums; ++i) s[i] = 0.f;
     float o[kGroups][4], r[kGroups][4], m[kGroups][4], wt[kGroups][4];
     load_groups<VEC>(a.old_lp, pos, o);
     if (a.roll_lp) load_groups<VEC>(a.roll_lp, pos, r);
@@ -100,11 +106,10 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
         }
       }
     if (a.level == VAMD_IS_TOKEN && a.weights) store_groups<VEC>(a.weights, pos, wt);
+#pragma unroll
+    for (int i = 0; i < kRcSums; ++i) acc[i] += (double)s[i];
   }
   __shared__ double smem[24 * 4];
-  double acc[kRcSums];
-#pragma unroll
-  for (int i = 0; i < kRcSums; ++i) acc[i] = s[i];
   block_sum<kRcSums, kRcThreads>(acc, smem);
   double ext[2] = {wmax, -(double)wmin};
   block_max_f64<2, kRcThreads>(ext, smem);
@@ -118,13 +123,15 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
   }
 }
 
-constexpr int kRcFoldThreads = 512;
+constexpr int kRcFoldThreads = 512;       // a batch of up to this many rows is folded by one workgroup
+constexpr int kRcFoldThreadsWide = 128;   // wider batches: one row per thread of many small workgroups, then their totals
 
 // records -> per-sequence quantities -> the metric vector (and the per-row weights): one row per thread, the
 // workgroups' totals combined by the last of them to finish.
-__global__ __launch_bounds__(kRcFoldThreads) void rollout_fold_kernel(RcArgs a) {
+template <int NT>
+__global__ __launch_bounds__(NT) void rollout_fold_kernel(RcArgs a) {
   const double inf = __longlong_as_double(0x7ff0000000000000ll);
-  __shared__ double smem[26 * (kRcFoldThreads / 64)];
+  __shared__ double smem[26 * (NT / 64)];
   enum {
     tM = 0, tD, tK3, tRho2, tW, tC, tC2, tTrunc, tHigh, tLow,         // token totals
     tTrainPpl, tTrainLog, tRollPpl, tRollLog, tGap, tGapAbs, tRatio, tChiSeq,  // sums over rows
@@ -141,8 +148,8 @@ __global__ __launch_bounds__(kRcFoldThreads) void rollout_fold_kernel(RcArgs a) 
   for (int i = 0; i < xN; ++i) x[i] = -inf;
   const float log_hi = logf(a.thr), log_lo = logf(a.lower);
   const bool seq_level = a.level == VAMD_IS_SEQUENCE;
-  for (int64_t r = (int64_t)blockIdx.x * kRcFoldThreads + threadIdx.x; r < a.rows;
-       r += (int64_t)gridDim.x * kRcFoldThreads) {
+  for (int64_t r = (int64_t)blockIdx.x * NT + threadIdx.x; r < a.rows;
+       r += (int64_t)gridDim.x * NT) {
     const int64_t rr[1] = {r};
     const bool have[1] = {true};
     double rec[1][kRcRec];
@@ -198,9 +205,9 @@ __global__ __launch_bounds__(kRcFoldThreads) void rollout_fold_kernel(RcArgs a) 
     }
   }
   static_assert(tN <= 26, "smem is sized for 26 sums");
-  block_sum<tN, kRcFoldThreads>(t, smem);
-  block_max_f64<xN, kRcFoldThreads>(x, smem);
-  if (!fold_across_workgroups<tN, xN, kRcFoldThreads>(t, x, a.shares, a.fold_counter, smem)) return;
+  block_sum<tN, NT>(t, smem);
+  block_max_f64<xN, NT>(x, smem);
+  if (!fold_across_workgroups<tN, xN, NT>(t, x, a.shares, a.fold_counter, smem)) return;
   if (threadIdx.x == 0) {
     double* o = a.out;
     const double B = (double)a.rows, Mt = t[tM];
@@ -293,8 +300,9 @@ using namespace vamd;
 // one row per thread of the fold launch, at most 256 workgroups, each leaving 26 sums and 9 maxima
 constexpr size_t kRcShareSlots = 26 + 9;
 static unsigned rc_fold_workgroups(int64_t batch) {
-  const int64_t n = (batch + kRcFoldThreads - 1) / kRcFoldThreads;
-  return (unsigned)(n < 1 ? 1 : (n > 256 ? 256 : n));
+  if (batch <= kRcFoldThreads) return 1;
+  const int64_t n = (batch + kRcFoldThreadsWide - 1) / kRcFoldThreadsWide;
+  return (unsigned)(n > 256 ? 256 : n);
 }
 
 extern "C" size_t vamd_rollout_correction_workspace_bytes(int64_t batch, int64_t length) {
@@ -321,7 +329,9 @@ extern "C" int vamd_rollout_correction(const float* old_log_prob, const float* r
   }
   RcArgs a;
   a.old_lp = old_log_prob; a.roll_lp = rollout_log_prob;
-  a.rows = batch; a.cols = length; a.chunks = (int)chunks_of(length);
+  a.rows = batch; a.cols = length;
+  a.span = record_span(batch, (int)chunks_of(length));
+  a.chunks = ((int)chunks_of(length) + a.span - 1) / a.span;
   a.level = level; a.thr = threshold; a.lower = level == VAMD_IS_NONE ? 0.f : 1.0f / threshold;
   a.normalize = batch_normalize;
   a.weights = weights;
@@ -334,6 +344,8 @@ extern "C" int vamd_rollout_correction(const float* old_log_prob, const float* r
   a.out = metrics;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)(batch * a.chunks)), block(kRcThreads);
+  const int col_chunks = (int)chunks_of(length);  // the broadcast takes one 4096-column chunk per workgroup
+  const dim3 cols_grid((unsigned)(batch * col_chunks));
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const M* mk = static_cast<const M*>(mask);
     const bool vec = can_vectorize(length, {old_log_prob, rollout_log_prob, weights}, mask, sizeof(M));
@@ -341,14 +353,18 @@ extern "C" int vamd_rollout_correction(const float* old_log_prob, const float* r
       hipLaunchKernelGGL((rollout_stats_kernel<true, M>), grid, block, 0, s, a, mk);
     else
       hipLaunchKernelGGL((rollout_stats_kernel<false, M>), grid, block, 0, s, a, mk);
-    hipLaunchKernelGGL(rollout_fold_kernel, dim3(rc_fold_workgroups(batch)), dim3(kRcFoldThreads), 0, s, a);
+    if (rc_fold_workgroups(batch) == 1)
+      hipLaunchKernelGGL(rollout_fold_kernel<kRcFoldThreads>, dim3(1), dim3(kRcFoldThreads), 0, s, a);
+    else
+      hipLaunchKernelGGL(rollout_fold_kernel<kRcFoldThreadsWide>, dim3(rc_fold_workgroups(batch)),
+                         dim3(kRcFoldThreadsWide), 0, s, a);
     if (level == VAMD_IS_SEQUENCE) {
       if (vec)
-        hipLaunchKernelGGL((rollout_broadcast_kernel<true, M>), grid, block, 0, s, a.row_weight, a.factor, mk, length,
-                           a.chunks, weights);
+        hipLaunchKernelGGL((rollout_broadcast_kernel<true, M>), cols_grid, block, 0, s, a.row_weight, a.factor, mk,
+                           length, col_chunks, weights);
       else
-        hipLaunchKernelGGL((rollout_broadcast_kernel<false, M>), grid, block, 0, s, a.row_weight, a.factor, mk,
-                           length, a.chunks, weights);
+        hipLaunchKernelGGL((rollout_broadcast_kernel<false, M>), cols_grid, block, 0, s, a.row_weight, a.factor, mk,
+                           length, col_chunks, weights);
     }
   });
   if (level == VAMD_IS_TOKEN && batch_normalize) {

@@ -351,6 +351,14 @@ __device__ __forceinline__ bool sum_all_records(unsigned* counters, double* __re
 // Doubles a record area needs behind its rows * chunks * nv record slots for sum_all_records().
 constexpr size_t kShareSlots = kTicketGroups;
 
+// 4096-column chunks one workgroup of a wide-record statistics pass walks (1, 2 or 4): as many as leave the launch
+// a couple of thousand workgroups.
+inline int record_span(int64_t rows, int chunks) {
+  int span = 4;
+  while (span > 1 && (span > chunks || rows * ((chunks + span - 1) / span) < 2048)) span /= 2;
+  return span;
+}
+
 // Cross-workgroup step of a fold launch that gives every workgroup a share of the rows: on entry thread 0 of each
 // workgroup holds NS sums and NX maxima of its share; returns true in exactly one workgroup, whose thread 0 then
 // holds them over all shares (a launch of one workgroup returns at once).  shares: gridDim.x * (NS + NX) doubles;
