@@ -846,11 +846,13 @@ def test_kl_loss_fused(dev, mode, kind, mdtype):
 
 
 @pytest.mark.parametrize("mode", MODES)
-def test_losses_with_the_fold_in_its_own_launch(dev, mode):
-    """More (row, chunk) records than the last workgroup folds itself: the loss kernels leave the fold to a second
-    launch.  Same checks as the small shapes, on agg_loss, the policy loss, the value loss and the fused KL loss."""
+@pytest.mark.parametrize("B,Lc", [(1500, 4100), (1100, 16000)])   # 3000 and 4400 records
+def test_losses_with_the_fold_in_its_own_launch(dev, mode, B, Lc):
+    """More (row, chunk) records than the last workgroup folds itself: the loss kernels take the launch totals in
+    one level (up to 4096 records) or two (token-mean, seq-mean-token-sum-norm), or leave the per-row fold to a
+    second launch (the other two modes).  Same checks as the small shapes, on agg_loss, the policy loss, the value
+    loss and the fused KL loss."""
     from verl_amd.trainer.ppo import core_algos as CA
-    B, Lc = 1500, 4100                                           # 3000 records
     old, new, adv, mask = _policy_inputs(B, Lc, seed=5)
     cfg = _cfg(clip_ratio=0.2, clip_ratio_high=0.28)
     nd = new.to(dev).requires_grad_(); no = new.clone().requires_grad_()

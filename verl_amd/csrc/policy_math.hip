@@ -15,7 +15,45 @@ namespace vamd {
 struct Work {
   unsigned* ticket;  // workspace head: zero on entry, zero on exit
   double* partials;  // NV slots per (row, chunk) workgroup, slot-major (record_at)
+  int totals;        // loss kernels built without the fold: take the launch totals here (totals_epilogue)
 };
+
+// The loss kernels of a large launch carry no fold of their own (FOLD = false).  Two of the four agg_loss modes,
+// token-mean and seq-mean-token-sum-norm, need nothing but the launch totals, and those come cheaply in two
+// levels (sum_all_records: a few dozen registers, no per-row pass), so such a launch finishes here; the per-row
+// modes leave their records to fold_loss_kernel.  Same formulas as finalize_agg.
+template <int NV, int EPI>
+__device__ __forceinline__ void totals_epilogue(const Work& wk, int64_t rows, int chunks, int64_t cols,
+                                                const AggParams& ap, float* __restrict__ coef,
+                                                float* __restrict__ out, double* smem) {
+  double tot[NV];
+  if (!sum_all_records<NV>(wk.ticket, wk.partials, rows, chunks, tot, smem)) return;
+  __shared__ float c_all;
+  if (threadIdx.x == 0) {
+    double loss, c;
+    if (ap.mode == VAMD_AGG_TOKEN_MEAN) {
+      const double denom = ap.batch_num_tokens < 0 ? tot[1] : ap.batch_num_tokens;
+      loss = tot[0] / denom * ap.dp_size;
+      c = ap.dp_size / denom;
+    } else {
+      const double f = ap.loss_scale_factor < 0 ? (double)cols : ap.loss_scale_factor;
+      loss = tot[0] / f;
+      c = 1.0 / f;
+    }
+    double extra[NV > 2 ? NV - 2 : 1] = {};
+#pragma unroll
+    for (int i = 2; i < NV; ++i) extra[i - 2] = tot[i];
+    loss_epilogue<EPI>(loss, tot[1], extra, out);
+    c_all = (float)c;
+  }
+  __syncthreads();
+  if (coef)
+    for (int64_t r = threadIdx.x; r < rows; r += kRcThreads) coef[r] = c_all;
+  ticket_reset(wk.ticket);
+}
+inline bool totals_suffice(int mode) {
+  return mode == VAMD_AGG_TOKEN_MEAN || mode == VAMD_AGG_SEQ_MEAN_TOKEN_SUM_NORM;
+}
 
 // =============================================================================================
 // masked moments
@@ -159,6 +197,8 @@ __global__ __launch_bounds__(kRcThreads) void agg_kernel(const float* __restrict
     finalize_agg<2>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
     if (threadIdx.x == 0) loss_epilogue<kEpiAgg>(loss, msum, extra, out_loss);
     ticket_reset(wk.ticket);
+  } else {
+    if (wk.totals) totals_epilogue<2, kEpiAgg>(wk, rows, chunks, cols, ap, coef, out_loss, smem);
   }
 }
 
@@ -418,6 +458,8 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
     finalize_agg<5>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
     if (threadIdx.x == 0) loss_epilogue<kEpiPolicy>(loss, msum, extra, out);
     ticket_reset(wk.ticket);
+  } else {
+    if (wk.totals) totals_epilogue<5, kEpiPolicy>(wk, rows, chunks, cols, ap, coef, out, smem);
   }
 }
 
@@ -477,6 +519,8 @@ __global__ __launch_bounds__(kRcThreads) void value_kernel(
     finalize_agg<3>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
     if (threadIdx.x == 0) loss_epilogue<kEpiValue>(loss, msum, extra, out);
     ticket_reset(wk.ticket);
+  } else {
+    if (wk.totals) totals_epilogue<3, kEpiValue>(wk, rows, chunks, cols, ap, coef, out, smem);
   }
 }
 
@@ -566,6 +610,8 @@ __global__ __launch_bounds__(kRcThreads) void kl_loss_kernel(
     finalize_agg<2>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
     if (threadIdx.x == 0) loss_epilogue<kEpiKl>(loss, msum, extra, out);
     ticket_reset(wk.ticket);
+  } else {
+    if (wk.totals) totals_epilogue<2, kEpiKl>(wk, rows, chunks, cols, ap, coef, out, smem);
   }
 }
 
@@ -978,6 +1024,7 @@ static Work carve_work(void* workspace) {
   Work w;
   w.ticket = static_cast<unsigned*>(workspace);
   w.partials = reinterpret_cast<double*>(static_cast<char*>(workspace) + kTicketBytes);
+  w.totals = 0;
   return w;
 }
 
@@ -1081,9 +1128,10 @@ extern "C" int vamd_agg_loss_forward(const float* loss_mat, const void* mask, in
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int chunks = (int)chunks_of(cols);
-  const Work wk = carve_work(workspace);
+  Work wk = carve_work(workspace);
   const AggParams ap = make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor);
   bool sep = rows * chunks > kInlineFoldRecords;  // fold the records in a launch of their own
+  wk.totals = sep && totals_suffice(mode);        // ... unless the launch totals are all the mode needs
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(cols, {loss_mat}, mask, sizeof(M));
     const M* mk = static_cast<const M*>(mask);
@@ -1099,7 +1147,7 @@ extern "C" int vamd_agg_loss_forward(const float* loss_mat, const void* mask, in
                          out_loss, coef_out);
     sep = sep && vec;
   });
-  if (sep)
+  if (sep && !wk.totals)
     hipLaunchKernelGGL((fold_loss_kernel<2, kEpiAgg>), dim3(1), dim3(kFoldThreads), 0, s, wk.partials, rows, chunks,
                        cols, ap, coef_out, out_loss);
   VAMD_LAUNCH_CHECK();
@@ -1193,7 +1241,7 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int chunks = (int)chunks_of(cols);
-  const Work wk = carve_work(workspace);
+  Work wk = carve_work(workspace);
   PolicyParams pp;
   pp.ratio_lo = (float)(1.0 - (double)clip_low);
   pp.ratio_hi = (float)(1.0 + (double)clip_high);
@@ -1233,6 +1281,7 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
     is_weights = nullptr;  // already folded into the sequence loss
   }
   bool sep = rows * chunks > kInlineFoldRecords;  // fold the records in a launch of their own
+  wk.totals = sep && totals_suffice(ap.mode);     // ... unless the launch totals are all the mode needs
   // the clipped PPO loss gets kernels of its own, the other variants share one with a per-token switch
 #define VAMD_PL_LAUNCH(V, G, W, F, K)                                                                              \
   hipLaunchKernelGGL((policy_kernel<V, M, G, W, F, K>), grid, block, 0, s, old_log_prob, log_prob, advantages, mk, \
@@ -1252,7 +1301,7 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
     else if (vec) { VAMD_PL_GW(true, true) }
     else { VAMD_PL_GW(false, true) }
   });
-  if (sep)
+  if (sep && !wk.totals)
     hipLaunchKernelGGL((fold_loss_kernel<5, kEpiPolicy>), dim3(1), dim3(kFoldThreads), 0, s, wk.partials, rows,
                        chunks, cols, ap, coef_out, out);
 #undef VAMD_PL_GW
@@ -1282,10 +1331,11 @@ extern "C" int vamd_value_loss_forward(const float* vpreds, const float* returns
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int chunks = (int)chunks_of(cols);
-  const Work wk = carve_work(workspace);
+  Work wk = carve_work(workspace);
   const AggParams ap = make_agg(mode, 1.0, -1.0, -1.0, -1.0);
   const dim3 grid((unsigned)(rows * chunks)), block(kRcThreads);
   bool sep = rows * chunks > kInlineFoldRecords;
+  wk.totals = sep && totals_suffice(mode);
 #define VAMD_VL(V, G, F)                                                                                     \
   hipLaunchKernelGGL((value_kernel<V, M, G, F>), grid, block, 0, s, vpreds, returns, values, mk, rows, cols, \
                      chunks, cliprange_value, ap, wk, out, grad_unscaled, coef_out)
@@ -1297,7 +1347,7 @@ extern "C" int vamd_value_loss_forward(const float* vpreds, const float* returns
     else if (vec) { if (grad_unscaled) VAMD_VL(true, true, true); else VAMD_VL(true, false, true); }
     else { if (grad_unscaled) VAMD_VL(false, true, true); else VAMD_VL(false, false, true); }
   });
-  if (sep)
+  if (sep && !wk.totals)
     hipLaunchKernelGGL((fold_loss_kernel<3, kEpiValue>), dim3(1), dim3(kFoldThreads), 0, s, wk.partials, rows, chunks,
                        cols, ap, coef_out, out);
 #undef VAMD_VL
@@ -1339,10 +1389,11 @@ extern "C" int vamd_kl_loss_forward(const float* logprob, const float* ref_logpr
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int chunks = (int)chunks_of(cols);
-  const Work wk = carve_work(workspace);
+  Work wk = carve_work(workspace);
   const AggParams ap = make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor);
   const dim3 grid((unsigned)(rows * chunks)), block(kRcThreads);
   bool sep = rows * chunks > kInlineFoldRecords;
+  wk.totals = sep && totals_suffice(mode);
 #define VAMD_KL(V, G, F)                                                                                       \
   hipLaunchKernelGGL((kl_loss_kernel<V, M, G, F>), grid, block, 0, s, logprob, ref_logprob, mk, rows, cols, chunks, \
                      kind, straight_through, ap, wk, out, grad_unscaled, coef_out)
@@ -1354,7 +1405,7 @@ extern "C" int vamd_kl_loss_forward(const float* logprob, const float* ref_logpr
     else if (vec) { if (grad_unscaled) VAMD_KL(true, true, true); else VAMD_KL(true, false, true); }
     else { if (grad_unscaled) VAMD_KL(false, true, true); else VAMD_KL(false, false, true); }
   });
-  if (sep)
+  if (sep && !wk.totals)
     hipLaunchKernelGGL((fold_loss_kernel<2, kEpiKl>), dim3(1), dim3(kFoldThreads), 0, s, wk.partials, rows, chunks,
                        cols, ap, coef_out, out);
 #undef VAMD_KL
