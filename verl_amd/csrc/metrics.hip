@@ -57,47 +57,47 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
   float lo[3] = {__builtin_inff(), __builtin_inff(), __builtin_inff()};
   const int64_t att_row = row * (a.prompt + a.cols) + a.prompt;
   for (int u = 0; u < a.span; ++u) {
-  const ChunkPos pos(row, chunk * a.span + u, a.cols);
-  // per-thread partials over its 16 elements in fp32 (exact counts, 1e-7 relative on the sums), widened per chunk
-  float s[kDmSums];
+    const ChunkPos pos(row, chunk * a.span + u, a.cols);
+    // per-thread partials over its 16 elements in fp32 (exact counts, 1e-7 relative on the sums), widened per chunk
+    float s[kDmSums];
 #pragma unroll
-  for (int i = 0; i < kDmSums; ++i) s[i] = 0.f;
+    for (int i = 0; i < kDmSums; ++i) s[i] = 0.f;
 #pragma unroll 2
-  for (int k = 0; k < kGroups; ++k) {
-    if (pos.valid[k] <= 0) continue;
-    float sc[4], rw[4], ad[4], rt[4], vl[4] = {0.f, 0.f, 0.f, 0.f}, m[4], at[4];
-    ld4<VEC>(a.scores, pos.idx[k], pos.valid[k], sc);
-    ld4<VEC>(a.rewards, pos.idx[k], pos.valid[k], rw);
-    ld4<VEC>(a.adv, pos.idx[k], pos.valid[k], ad);
-    ld4<VEC>(a.ret, pos.idx[k], pos.valid[k], rt);
-    if (a.val) ld4<VEC>(a.val, pos.idx[k], pos.valid[k], vl);
-    ldmask4<VEC>(mask, pos.idx[k], pos.valid[k], m);
-    ldmask4<VEC>(attention, att_row + (pos.idx[k] - row * a.cols), pos.valid[k], at);
+    for (int k = 0; k < kGroups; ++k) {
+      if (pos.valid[k] <= 0) continue;
+      float sc[4], rw[4], ad[4], rt[4], vl[4] = {0.f, 0.f, 0.f, 0.f}, m[4], at[4];
+      ld4<VEC>(a.scores, pos.idx[k], pos.valid[k], sc);
+      ld4<VEC>(a.rewards, pos.idx[k], pos.valid[k], rw);
+      ld4<VEC>(a.adv, pos.idx[k], pos.valid[k], ad);
+      ld4<VEC>(a.ret, pos.idx[k], pos.valid[k], rt);
+      if (a.val) ld4<VEC>(a.val, pos.idx[k], pos.valid[k], vl);
+      ldmask4<VEC>(mask, pos.idx[k], pos.valid[k], m);
+      ldmask4<VEC>(attention, att_row + (pos.idx[k] - row * a.cols), pos.valid[k], at);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      if (e >= pos.valid[k]) continue;
-      s[kDmScore] += sc[e];
-      s[kDmReward] += rw[e];
-      s[kDmRespLen] += at[e];
-      if (m[e] != 0.f) {
-        s[kDmValid] += 1.f;
-        s[kDmAdv] += ad[e];
-        s[kDmRet] += rt[e];
-        s[kDmRet2] += rt[e] * rt[e];
-        hi[0] = fmaxf(hi[0], ad[e]); lo[0] = fminf(lo[0], ad[e]);
-        hi[1] = fmaxf(hi[1], rt[e]); lo[1] = fminf(lo[1], rt[e]);
-        if (a.val) {
-          const float d = rt[e] - vl[e];  // the fp32 difference the reference forms (:143)
-          s[kDmVal] += vl[e];
-          s[kDmDiff] += d;
-          s[kDmDiff2] += d * d;
-          hi[2] = fmaxf(hi[2], vl[e]); lo[2] = fminf(lo[2], vl[e]);
+      for (int e = 0; e < 4; ++e) {
+        if (e >= pos.valid[k]) continue;
+        s[kDmScore] += sc[e];
+        s[kDmReward] += rw[e];
+        s[kDmRespLen] += at[e];
+        if (m[e] != 0.f) {
+          s[kDmValid] += 1.f;
+          s[kDmAdv] += ad[e];
+          s[kDmRet] += rt[e];
+          s[kDmRet2] += rt[e] * rt[e];
+          hi[0] = fmaxf(hi[0], ad[e]); lo[0] = fminf(lo[0], ad[e]);
+          hi[1] = fmaxf(hi[1], rt[e]); lo[1] = fminf(lo[1], rt[e]);
+          if (a.val) {
+            const float d = rt[e] - vl[e];  // the fp32 difference the reference forms (:143)
+            s[kDmVal] += vl[e];
+            s[kDmDiff] += d;
+            s[kDmDiff2] += d * d;
+            hi[2] = fmaxf(hi[2], vl[e]); lo[2] = fminf(lo[2], vl[e]);
+          }
         }
       }
     }
-  }
 #pragma unroll
-  for (int i = 0; i < kDmSums; ++i) acc[i] += (double)s[i];
+    for (int i = 0; i < kDmSums; ++i) acc[i] += (double)s[i];
   }
   if (chunk == 0) {
     const int64_t p0 = row * (a.prompt + a.cols);
