@@ -27,8 +27,11 @@ struct CovState {
   unsigned k_rem;        // places left for keys equal to the prefix
   unsigned take_all;     // every candidate is selected
   unsigned tie_counter;  // tickets for keys equal to the threshold
-  unsigned hist[256];
+  // kHistCopies copies of the 256-bin histogram, workgroup b adding to copy b % kHistCopies: the keys of a
+  // launch fall into a handful of bins, and adds to one address are served one after the other
+  unsigned hist[64][256];
 };
+constexpr int kHistCopies = 64;
 
 struct CovArgs {
   const float *old_lp, *lp, *adv, *isw;
@@ -100,7 +103,7 @@ __global__ __launch_bounds__(256) void cov_prepare_kernel(CovArgs a) {
     for (int i = 0; i < 4; ++i) t[i] += a.stats[(int64_t)i * n + k];
   block_sum<4, 256>(t, smem);
   CovState* st = a.state;
-  st->hist[threadIdx.x] = 0;
+  for (int c = 0; c < kHistCopies; ++c) st->hist[c][threadIdx.x] = 0;
   if (threadIdx.x == 0) {
     const double msum = t[0], count = t[1];
     if (a.kind == kCovKl) {  // plain means over the valid tokens (:1604); k = max(1, int(n ratio)) (:1605)
@@ -164,7 +167,7 @@ __global__ __launch_bounds__(kRcThreads) void cov_keys_kernel(CovArgs a, const M
     }
   if (mine) atomicAdd(&cand, mine);
   __syncthreads();
-  if (hist[threadIdx.x]) atomicAdd(&a.state->hist[threadIdx.x], hist[threadIdx.x]);
+  if (hist[threadIdx.x]) atomicAdd(&a.state->hist[blockIdx.x % kHistCopies][threadIdx.x], hist[threadIdx.x]);
   if (threadIdx.x == 0 && cand) atomicAdd(&a.state->n_cand, cand);
 }
 
@@ -176,24 +179,40 @@ __global__ __launch_bounds__(256) void cov_hist_kernel(const unsigned* __restric
   __syncthreads();
   if (st->take_all || st->k == 0) return;
   const unsigned prefix = st->prefix >> (shift + 8);
-  const int64_t stride = (int64_t)gridDim.x * 256 * 4;
-  for (int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4; i < n; i += stride) {
+  auto count = [&](unsigned key) {
+    if (key != 0 && (key >> (shift + 8)) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+  };
+  // eight 16-byte loads per thread, all issued before the first key is looked at (the key plane is 256-byte aligned)
+  const uint4* __restrict__ keys4 = reinterpret_cast<const uint4*>(keys);
+  const int64_t n4 = n / 4;
+  const int64_t first = (int64_t)blockIdx.x * 256 * 8 + threadIdx.x;
+  uint4 v[8];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      if (i + e >= n) break;
-      const unsigned key = keys[i + e];
-      if (key != 0 && (key >> (shift + 8)) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
-    }
+  for (int u = 0; u < 8; ++u) {
+    const int64_t i = first + (int64_t)u * 256;
+    v[u] = i < n4 ? keys4[i] : make_uint4(0u, 0u, 0u, 0u);
   }
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    count(v[u].x);
+    count(v[u].y);
+    count(v[u].z);
+    count(v[u].w);
+  }
+  if (blockIdx.x == 0 && n4 * 4 + threadIdx.x < n) count(keys[n4 * 4 + threadIdx.x]);  // the last n % 4 keys
   __syncthreads();
-  if (hist[threadIdx.x]) atomicAdd(&st->hist[threadIdx.x], hist[threadIdx.x]);
+  if (hist[threadIdx.x]) atomicAdd(&st->hist[blockIdx.x % kHistCopies][threadIdx.x], hist[threadIdx.x]);
 }
 
 // One workgroup: the bin that holds the k_rem-th largest key of this pass becomes the next digit of the threshold.
 __global__ __launch_bounds__(256) void cov_pick_kernel(CovState* __restrict__ st, int shift) {
   __shared__ unsigned h[256];
-  h[threadIdx.x] = st->hist[threadIdx.x];
-  st->hist[threadIdx.x] = 0;
+  unsigned sum = 0;
+  for (int c = 0; c < kHistCopies; ++c) {
+    sum += st->hist[c][threadIdx.x];
+    st->hist[c][threadIdx.x] = 0;
+  }
+  h[threadIdx.x] = sum;
   __syncthreads();
   if (threadIdx.x != 0) return;
   if (shift == 24) {  // first pass: fix how many there are to take
@@ -320,6 +339,7 @@ extern "C" int vamd_policy_loss_cov_forward(int kind, const float* old_log_prob,
     set_error("policy_loss_cov: workspace too small");
     return VAMD_EWORKSPACE;
   }
+  VAMD_REQUIRE(aligned_to(workspace, 16), "policy_loss_cov: the workspace must be 16-byte aligned");
   CovArgs a;
   a.old_lp = old_log_prob; a.lp = log_prob; a.adv = advantages; a.isw = is_weights;
   a.rows = rows; a.cols = cols; a.chunks = (int)chunks_of(cols);
