@@ -22,7 +22,7 @@ enum { kCovKl = 0, kCovClip = 1 };
 struct CovState {
   float mean_a, mean_lp;
   unsigned k;            // tokens to select
-  unsigned n_cand;       // candidates (key != 0)
+  unsigned n_cand;       // candidates (key != 0): the total of the first histogram
   unsigned prefix;       // the digits of the threshold key found so far
   unsigned k_rem;        // places left for keys equal to the prefix
   unsigned take_all;     // every candidate is selected
@@ -131,9 +131,7 @@ __global__ __launch_bounds__(kRcThreads) void cov_keys_kernel(CovArgs a, const M
   const int chunk = blockIdx.x % a.chunks;
   const ChunkPos pos(row, chunk, a.cols);
   __shared__ unsigned hist[256];
-  __shared__ unsigned cand;
   hist[threadIdx.x] = 0;
-  if (threadIdx.x == 0) cand = 0;
   __syncthreads();
   float o[kGroups][4], lp[kGroups][4], A[kGroups][4], m[kGroups][4];
   load_groups<VEC>(a.lp, pos, lp);
@@ -141,7 +139,6 @@ __global__ __launch_bounds__(kRcThreads) void cov_keys_kernel(CovArgs a, const M
   load_mask_groups<VEC>(mask, pos, m);
   if (a.kind == kCovClip) load_groups<VEC>(a.old_lp, pos, o);
   const float mean_a = a.state->mean_a, mean_lp = a.state->mean_lp;
-  unsigned mine = 0;
 #pragma unroll
   for (int g = 0; g < kGroups; ++g)
 #pragma unroll
@@ -160,15 +157,10 @@ __global__ __launch_bounds__(kRcThreads) void cov_keys_kernel(CovArgs a, const M
         }
       }
       a.keys[pos.idx[g] + e] = key;
-      if (key != 0) {
-        ++mine;
-        atomicAdd(&hist[key >> 24], 1u);
-      }
+      if (key != 0) atomicAdd(&hist[key >> 24], 1u);
     }
-  if (mine) atomicAdd(&cand, mine);
   __syncthreads();
   if (hist[threadIdx.x]) atomicAdd(&a.state->hist[blockIdx.x % kHistCopies][threadIdx.x], hist[threadIdx.x]);
-  if (threadIdx.x == 0 && cand) atomicAdd(&a.state->n_cand, cand);
 }
 
 // Histogram of the byte at `shift` over the keys whose higher bytes equal the prefix.
@@ -204,33 +196,47 @@ __global__ __launch_bounds__(256) void cov_hist_kernel(const unsigned* __restric
   if (hist[threadIdx.x]) atomicAdd(&st->hist[blockIdx.x % kHistCopies][threadIdx.x], hist[threadIdx.x]);
 }
 
-// One workgroup: the bin that holds the k_rem-th largest key of this pass becomes the next digit of the threshold.
+// One workgroup: the bin that holds the k_rem-th largest key of this pass becomes the next digit of the threshold,
+// i.e. the largest bin b >= 1 with at least k_rem keys in bins b .. 255 (bin 0 when there is none).  The counts
+// from each bin upwards come from a 256-wide suffix scan in LDS rather than one thread walking the bins.
 __global__ __launch_bounds__(256) void cov_pick_kernel(CovState* __restrict__ st, int shift) {
-  __shared__ unsigned h[256];
+  __shared__ unsigned S[2][256];
+  __shared__ unsigned bin;
+  const unsigned t = threadIdx.x;
   unsigned sum = 0;
   for (int c = 0; c < kHistCopies; ++c) {
-    sum += st->hist[c][threadIdx.x];
-    st->hist[c][threadIdx.x] = 0;
+    sum += st->hist[c][t];
+    st->hist[c][t] = 0;
   }
-  h[threadIdx.x] = sum;
+  S[0][t] = sum;
+  if (t == 0) bin = 0;
   __syncthreads();
-  if (threadIdx.x != 0) return;
+  int p = 0;
+  for (unsigned d = 1; d < 256; d <<= 1, p ^= 1) {
+    S[p ^ 1][t] = S[p][t] + (t + d < 256 ? S[p][t + d] : 0u);
+    __syncthreads();
+  }
+  const unsigned* from = S[p];  // from[b]: keys in bins b .. 255
+  unsigned k_rem = st->k_rem;
   if (shift == 24) {  // first pass: fix how many there are to take
-    if (st->k >= st->n_cand) {
-      st->take_all = 1;  // fewer candidates than places (none selected when there are no candidates)
+    if (st->k >= from[0]) {
+      if (t == 0) {
+        st->n_cand = from[0];
+        st->take_all = 1;  // fewer candidates than places (none selected when there are no candidates)
+      }
       return;
     }
-    st->k_rem = st->k;
+    k_rem = st->k;
   }
   if (st->take_all || st->k == 0) return;
-  unsigned above = 0;
-  int b = 255;
-  for (; b > 0; --b) {
-    if (above + h[b] >= st->k_rem) break;
-    above += h[b];
+  if (t >= 1 && from[t] >= k_rem && (t == 255 || from[t + 1] < k_rem)) bin = t;
+  __syncthreads();
+  if (t == 0) {
+    const unsigned b = bin;
+    if (shift == 24) st->n_cand = from[0];
+    st->prefix |= b << shift;
+    st->k_rem = k_rem - (b == 255 ? 0u : from[b + 1]);
   }
-  st->prefix |= (unsigned)b << shift;
-  st->k_rem -= above;
 }
 
 template <bool VEC, class M, bool GRAD, bool ISW>
