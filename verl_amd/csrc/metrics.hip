@@ -119,8 +119,8 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
   }
 }
 
-constexpr int kDmFoldThreads = 512;       // a batch of up to this many rows is folded by one workgroup
-constexpr int kDmFoldThreadsWide = 128;   // wider batches: one row per thread of many small workgroups, then their totals
+constexpr int kFoldRows = 4;          // rows per thread and trip of the fold launch
+constexpr int kDmFoldThreads = 128;   // a workgroup of the fold launch takes up to kFoldRows * kDmFoldThreads rows
 
 // records -> per-row quantities -> the output vector: one row per thread, the workgroups' totals combined by the
 // last of them to finish.
@@ -141,34 +141,45 @@ __global__ __launch_bounds__(NT) void data_metrics_fold_kernel(DmArgs a) {
   double x[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) x[i] = -inf;
-  for (int64_t r = (int64_t)blockIdx.x * NT + threadIdx.x; r < a.rows;
-       r += (int64_t)gridDim.x * NT) {
-    const int64_t rr[1] = {r};
-    const bool have[1] = {true};
-    double rec[1][kDmRec];
-    fold_row_records<kDmRec, kDmSums, 1, false>(a.records, rr, have, a.rows, a.chunks, rec);
-    const double* row_s = rec[0];
+  // kFoldRows rows per thread and trip, their records in flight together: few wavefronts keep the workgroup
+  // reductions below short, and the loads of a trip are one round trip to memory whatever their number
+  for (int64_t r0 = (int64_t)blockIdx.x * NT * kFoldRows + threadIdx.x; r0 < a.rows;
+       r0 += (int64_t)gridDim.x * NT * kFoldRows) {
+    int64_t rr[kFoldRows];
+    bool have[kFoldRows];
 #pragma unroll
-    for (int i = 0; i < kElem; ++i) t[9 + i] += rec[0][kDmValid + i];
+    for (int k = 0; k < kFoldRows; ++k) {
+      rr[k] = r0 + (int64_t)k * NT;
+      have[k] = rr[k] < a.rows;
+    }
+    double rec[kFoldRows][kDmRec];
+    fold_row_records<kDmRec, kDmSums, kFoldRows, false, 1>(a.records, rr, have, a.rows, a.chunks, rec);
 #pragma unroll
-    for (int i = 0; i < 6; ++i) x[10 + i] = fmax(x[10 + i], rec[0][kDmSums + i]);
-    const double score = (double)(float)row_s[kDmScore], reward = (double)(float)row_s[kDmReward];
-    const double rl = row_s[kDmRespLen], pl = row_s[kDmPromptLen];
-    t[3] += rl;
-    t[4] += rl == (double)a.cols ? 1.0 : 0.0;
-    x[4] = fmax(x[4], rl); x[5] = fmax(x[5], -rl);
-    t[7] += pl;
-    t[8] += pl == (double)a.prompt ? 1.0 : 0.0;
-    x[8] = fmax(x[8], pl); x[9] = fmax(x[9], -pl);
-    if (rl != 0.0) {  // not aborted (:119-120)
-      t[0] += 1.0;
-      t[1] += score;
-      t[2] += reward;
-      x[0] = fmax(x[0], score); x[1] = fmax(x[1], -score);
-      x[2] = fmax(x[2], reward); x[3] = fmax(x[3], -reward);
-      t[5] += rl;
-      t[6] += rl == (double)a.cols ? 1.0 : 0.0;
-      x[6] = fmax(x[6], rl); x[7] = fmax(x[7], -rl);
+    for (int k = 0; k < kFoldRows; ++k) {
+      if (!have[k]) break;
+      const double* row_s = rec[k];
+#pragma unroll
+      for (int i = 0; i < kElem; ++i) t[9 + i] += rec[k][kDmValid + i];
+#pragma unroll
+      for (int i = 0; i < 6; ++i) x[10 + i] = fmax(x[10 + i], rec[k][kDmSums + i]);
+      const double score = (double)(float)row_s[kDmScore], reward = (double)(float)row_s[kDmReward];
+      const double rl = row_s[kDmRespLen], pl = row_s[kDmPromptLen];
+      t[3] += rl;
+      t[4] += rl == (double)a.cols ? 1.0 : 0.0;
+      x[4] = fmax(x[4], rl); x[5] = fmax(x[5], -rl);
+      t[7] += pl;
+      t[8] += pl == (double)a.prompt ? 1.0 : 0.0;
+      x[8] = fmax(x[8], pl); x[9] = fmax(x[9], -pl);
+      if (rl != 0.0) {  // not aborted (:119-120)
+        t[0] += 1.0;
+        t[1] += score;
+        t[2] += reward;
+        x[0] = fmax(x[0], score); x[1] = fmax(x[1], -score);
+        x[2] = fmax(x[2], reward); x[3] = fmax(x[3], -reward);
+        t[5] += rl;
+        t[6] += rl == (double)a.cols ? 1.0 : 0.0;
+        x[6] = fmax(x[6], rl); x[7] = fmax(x[7], -rl);
+      }
     }
   }
   block_sum<9 + kElem, NT>(t, smem);
@@ -254,11 +265,11 @@ __global__ __launch_bounds__(kRcThreads) void variance_proxy_rows_kernel(const f
 
 using namespace vamd;
 
-// one row per thread of the fold launch, at most 256 workgroups
+// workgroups of the fold launch (at most 256)
 static unsigned dm_fold_workgroups(int64_t batch) {
-  if (batch <= kDmFoldThreads) return 1;
-  const int64_t n = (batch + kDmFoldThreadsWide - 1) / kDmFoldThreadsWide;
-  return (unsigned)(n > 256 ? 256 : n);
+  const int64_t per = (int64_t)kFoldRows * kDmFoldThreads;
+  const int64_t n = (batch + per - 1) / per;
+  return (unsigned)(n < 1 ? 1 : (n > 256 ? 256 : n));
 }
 
 extern "C" int vamd_variance_proxy_rows(const float* advantages, const float* old_log_probs,
@@ -338,11 +349,8 @@ extern "C" int vamd_data_metrics(const float* token_level_scores, const float* t
     default: set_error("unknown mask dtype code %d", attention_dtype); return VAMD_EINVAL;
   }
 #undef VAMD_DM
-  if (dm_fold_workgroups(batch) == 1)
-    hipLaunchKernelGGL(data_metrics_fold_kernel<kDmFoldThreads>, dim3(1), dim3(kDmFoldThreads), 0, s, a);
-  else
-    hipLaunchKernelGGL(data_metrics_fold_kernel<kDmFoldThreadsWide>, dim3(dm_fold_workgroups(batch)),
-                       dim3(kDmFoldThreadsWide), 0, s, a);
+  hipLaunchKernelGGL(data_metrics_fold_kernel<kDmFoldThreads>, dim3(dm_fold_workgroups(batch)), dim3(kDmFoldThreads),
+                     0, s, a);
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }

@@ -123,8 +123,8 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
   }
 }
 
-constexpr int kRcFoldThreads = 512;       // a batch of up to this many rows is folded by one workgroup
-constexpr int kRcFoldThreadsWide = 128;   // wider batches: one row per thread of many small workgroups, then their totals
+constexpr int kFoldRows = 4;          // rows per thread and trip of the fold launch
+constexpr int kRcFoldThreads = 128;   // a workgroup of the fold launch takes up to kFoldRows * kRcFoldThreads rows
 
 // records -> per-sequence quantities -> the metric vector (and the per-row weights): one row per thread, the
 // workgroups' totals combined by the last of them to finish.
@@ -148,60 +148,72 @@ __global__ __launch_bounds__(NT) void rollout_fold_kernel(RcArgs a) {
   for (int i = 0; i < xN; ++i) x[i] = -inf;
   const float log_hi = logf(a.thr), log_lo = logf(a.lower);
   const bool seq_level = a.level == VAMD_IS_SEQUENCE;
-  for (int64_t r = (int64_t)blockIdx.x * NT + threadIdx.x; r < a.rows;
-       r += (int64_t)gridDim.x * NT) {
-    const int64_t rr[1] = {r};
-    const bool have[1] = {true};
-    double rec[1][kRcRec];
-    fold_row_records<kRcRec, kRcSums, 1, false>(a.records, rr, have, a.rows, a.chunks, rec);
-    const double* f = rec[0];
-    x[xW] = fmax(x[xW], rec[0][kRcWMax]);
-    x[xWMinNeg] = fmax(x[xWMinNeg], rec[0][kRcWMinNeg]);
-    const float Mi = (float)f[kRcM];
-    const float train = (float)f[kRcOld] / (Mi + 1e-8f);  // masked_mean(., axis=-1)
-    t[tM] += f[kRcM]; t[tD] += f[kRcD]; t[tK3] += f[kRcK3]; t[tRho2] += f[kRcRho2];
-    t[tTrainPpl] += (double)expf(-train);
-    t[tTrainLog] += (double)(-train);
-    if (Mi > 0.f) t[tAlive] += 1.0;
-    if (!a.roll_lp) continue;
-    const float roll = (float)f[kRcRoll] / (Mi + 1e-8f);
-    const float gap = roll - train;
-    const float dsum = (float)f[kRcD];
-    const float dsafe = fminf(fmaxf(dsum, -kSafetyBound), kSafetyBound);
-    t[tRollPpl] += (double)expf(-roll);
-    t[tRollLog] += (double)(-roll);
-    t[tGap] += (double)gap;
-    t[tGapAbs] += (double)fabsf(gap);
-    t[tRatio] += (double)expf(gap);
-    t[tChiSeq] += (double)expf(2.f * dsafe);
-    x[xGap] = fmax(x[xGap], (double)gap);
-    x[xGapMinNeg] = fmax(x[xGapMinNeg], -(double)gap);
-    float seq = 0.f;  // masked_mean(weights, axis=-1) of the untruncated weights
-    if (a.level == VAMD_IS_TOKEN) {
-      t[tW] += f[kRcW]; t[tC] += f[kRcC]; t[tC2] += f[kRcC2]; t[tTrunc] += f[kRcTrunc];
-      t[tHigh] += f[kRcHigh]; t[tLow] += f[kRcLow];
-      seq = (float)f[kRcW] / (Mi + 1e-8f);
-    } else if (seq_level) {
-      const float w = expf(dsafe);
-      const float c = fminf(fmaxf(w, a.lower), a.thr);
-      const float tr = fminf(w, a.thr);
-      t[tW] += (double)w * f[kRcM]; t[tC] += (double)c * f[kRcM]; t[tC2] += (double)c * (double)c * f[kRcM];
-      t[tLogHigh] += dsum > log_hi ? 1.0 : 0.0;
-      t[tLogLow] += dsum < log_lo ? 1.0 : 0.0;
-      x[xLog] = fmax(x[xLog], (double)dsum);
-      x[xLogMinNeg] = fmax(x[xLogMinNeg], -(double)dsum);
-      seq = w * Mi / (Mi + 1e-8f);
-      if (Mi > 0.f) t[tSeqTrunc] += (double)(tr * Mi / (Mi + 1e-8f));
-      a.row_weight[r] = tr;
+  // kFoldRows rows per thread and trip, their records in flight together: few wavefronts keep the workgroup
+  // reductions below short, and the loads of a trip are one round trip to memory whatever their number
+  for (int64_t r0 = (int64_t)blockIdx.x * NT * kFoldRows + threadIdx.x; r0 < a.rows;
+       r0 += (int64_t)gridDim.x * NT * kFoldRows) {
+    int64_t rr[kFoldRows];
+    bool have[kFoldRows];
+#pragma unroll
+    for (int k = 0; k < kFoldRows; ++k) {
+      rr[k] = r0 + (int64_t)k * NT;
+      have[k] = rr[k] < a.rows;
     }
-    if (a.level != VAMD_IS_NONE) {
-      t[tSeq] += (double)seq;
-      t[tSeq2] += (double)seq * (double)seq;
-      t[tSeqHigh] += seq > a.thr ? 1.0 : 0.0;
-      t[tSeqLow] += seq < a.lower ? 1.0 : 0.0;
-      x[xSeq] = fmax(x[xSeq], (double)seq);
-      x[xSeqMinNeg] = fmax(x[xSeqMinNeg], -(double)seq);
-      x[xDev] = fmax(x[xDev], (double)fabsf(seq - 1.f));
+    double rec[kFoldRows][kRcRec];
+    fold_row_records<kRcRec, kRcSums, kFoldRows, false, 1>(a.records, rr, have, a.rows, a.chunks, rec);
+#pragma unroll
+    for (int k = 0; k < kFoldRows; ++k) {
+      if (!have[k]) break;
+      const int64_t r = rr[k];
+      const double* f = rec[k];
+      x[xW] = fmax(x[xW], rec[k][kRcWMax]);
+      x[xWMinNeg] = fmax(x[xWMinNeg], rec[k][kRcWMinNeg]);
+      const float Mi = (float)f[kRcM];
+      const float train = (float)f[kRcOld] / (Mi + 1e-8f);  // masked_mean(., axis=-1)
+      t[tM] += f[kRcM]; t[tD] += f[kRcD]; t[tK3] += f[kRcK3]; t[tRho2] += f[kRcRho2];
+      t[tTrainPpl] += (double)expf(-train);
+      t[tTrainLog] += (double)(-train);
+      if (Mi > 0.f) t[tAlive] += 1.0;
+      if (!a.roll_lp) continue;
+      const float roll = (float)f[kRcRoll] / (Mi + 1e-8f);
+      const float gap = roll - train;
+      const float dsum = (float)f[kRcD];
+      const float dsafe = fminf(fmaxf(dsum, -kSafetyBound), kSafetyBound);
+      t[tRollPpl] += (double)expf(-roll);
+      t[tRollLog] += (double)(-roll);
+      t[tGap] += (double)gap;
+      t[tGapAbs] += (double)fabsf(gap);
+      t[tRatio] += (double)expf(gap);
+      t[tChiSeq] += (double)expf(2.f * dsafe);
+      x[xGap] = fmax(x[xGap], (double)gap);
+      x[xGapMinNeg] = fmax(x[xGapMinNeg], -(double)gap);
+      float seq = 0.f;  // masked_mean(weights, axis=-1) of the untruncated weights
+      if (a.level == VAMD_IS_TOKEN) {
+        t[tW] += f[kRcW]; t[tC] += f[kRcC]; t[tC2] += f[kRcC2]; t[tTrunc] += f[kRcTrunc];
+        t[tHigh] += f[kRcHigh]; t[tLow] += f[kRcLow];
+        seq = (float)f[kRcW] / (Mi + 1e-8f);
+      } else if (seq_level) {
+        const float w = expf(dsafe);
+        const float c = fminf(fmaxf(w, a.lower), a.thr);
+        const float tr = fminf(w, a.thr);
+        t[tW] += (double)w * f[kRcM]; t[tC] += (double)c * f[kRcM]; t[tC2] += (double)c * (double)c * f[kRcM];
+        t[tLogHigh] += dsum > log_hi ? 1.0 : 0.0;
+        t[tLogLow] += dsum < log_lo ? 1.0 : 0.0;
+        x[xLog] = fmax(x[xLog], (double)dsum);
+        x[xLogMinNeg] = fmax(x[xLogMinNeg], -(double)dsum);
+        seq = w * Mi / (Mi + 1e-8f);
+        if (Mi > 0.f) t[tSeqTrunc] += (double)(tr * Mi / (Mi + 1e-8f));
+        a.row_weight[r] = tr;
+      }
+      if (a.level != VAMD_IS_NONE) {
+        t[tSeq] += (double)seq;
+        t[tSeq2] += (double)seq * (double)seq;
+        t[tSeqHigh] += seq > a.thr ? 1.0 : 0.0;
+        t[tSeqLow] += seq < a.lower ? 1.0 : 0.0;
+        x[xSeq] = fmax(x[xSeq], (double)seq);
+        x[xSeqMinNeg] = fmax(x[xSeqMinNeg], -(double)seq);
+        x[xDev] = fmax(x[xDev], (double)fabsf(seq - 1.f));
+      }
     }
   }
   static_assert(tN <= 26, "smem is sized for 26 sums");
@@ -297,12 +309,12 @@ __global__ __launch_bounds__(256) void rollout_divide_kernel(float* __restrict__
 
 using namespace vamd;
 
-// one row per thread of the fold launch, at most 256 workgroups, each leaving 26 sums and 9 maxima
+// workgroups of the fold launch (at most 256), each leaving 26 sums and 9 maxima
 constexpr size_t kRcShareSlots = 26 + 9;
 static unsigned rc_fold_workgroups(int64_t batch) {
-  if (batch <= kRcFoldThreads) return 1;
-  const int64_t n = (batch + kRcFoldThreadsWide - 1) / kRcFoldThreadsWide;
-  return (unsigned)(n > 256 ? 256 : n);
+  const int64_t per = (int64_t)kFoldRows * kRcFoldThreads;
+  const int64_t n = (batch + per - 1) / per;
+  return (unsigned)(n < 1 ? 1 : (n > 256 ? 256 : n));
 }
 
 extern "C" size_t vamd_rollout_correction_workspace_bytes(int64_t batch, int64_t length) {
@@ -353,11 +365,8 @@ extern "C" int vamd_rollout_correction(const float* old_log_prob, const float* r
       hipLaunchKernelGGL((rollout_stats_kernel<true, M>), grid, block, 0, s, a, mk);
     else
       hipLaunchKernelGGL((rollout_stats_kernel<false, M>), grid, block, 0, s, a, mk);
-    if (rc_fold_workgroups(batch) == 1)
-      hipLaunchKernelGGL(rollout_fold_kernel<kRcFoldThreads>, dim3(1), dim3(kRcFoldThreads), 0, s, a);
-    else
-      hipLaunchKernelGGL(rollout_fold_kernel<kRcFoldThreadsWide>, dim3(rc_fold_workgroups(batch)),
-                         dim3(kRcFoldThreadsWide), 0, s, a);
+    hipLaunchKernelGGL(rollout_fold_kernel<kRcFoldThreads>, dim3(rc_fold_workgroups(batch)), dim3(kRcFoldThreads), 0,
+                       s, a);
     if (level == VAMD_IS_SEQUENCE) {
       if (vec)
         hipLaunchKernelGGL((rollout_broadcast_kernel<true, M>), cols_grid, block, 0, s, a.row_weight, a.factor, mk,

@@ -248,9 +248,9 @@ __device__ __forceinline__ double record_load(const double* p) {
 
 // Fold the chunk records of ROWS rows, slot by slot: slots [0, NSUM) add up, slots [NSUM, NV) take the maximum
 // (records hold minima negated).  Every record load is a round trip to the memory side, and the workgroup
-// doing the fold is the only one left running, so the loads of up to four chunks of every row of the trip are
+// doing the fold is the only one left running, so the loads of up to FLIGHT chunks of every row of the trip are
 // issued together; the order of the additions (chunk 0 first) does not depend on that.
-template <int NV, int NSUM, int ROWS, bool COHERENT = true>
+template <int NV, int NSUM, int ROWS, bool COHERENT = true, int FLIGHT = 4>
 __device__ __forceinline__ void fold_row_records(const double* __restrict__ records, const int64_t (&row)[ROWS],
                                                  const bool (&have)[ROWS], int64_t rows, int chunks,
                                                  double (&out)[ROWS][NV]) {
@@ -259,12 +259,12 @@ __device__ __forceinline__ void fold_row_records(const double* __restrict__ reco
   for (int k = 0; k < ROWS; ++k)
 #pragma unroll
     for (int i = 0; i < NV; ++i) out[k][i] = i < NSUM ? 0.0 : ninf;
-  for (int c0 = 0; c0 < chunks; c0 += 4) {
-    double t[ROWS][4][NV];
+  for (int c0 = 0; c0 < chunks; c0 += FLIGHT) {
+    double t[ROWS][FLIGHT][NV];
 #pragma unroll
     for (int k = 0; k < ROWS; ++k)
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < FLIGHT; ++u) {
         const bool ok = have[k] && c0 + u < chunks;
 #pragma unroll
         for (int i = 0; i < NV; ++i)
@@ -274,7 +274,7 @@ __device__ __forceinline__ void fold_row_records(const double* __restrict__ reco
 #pragma unroll
     for (int k = 0; k < ROWS; ++k)
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < FLIGHT; ++u)
 #pragma unroll
         for (int i = 0; i < NV; ++i) out[k][i] = i < NSUM ? out[k][i] + t[k][u][i] : fmax(out[k][i], t[k][u][i]);
   }
