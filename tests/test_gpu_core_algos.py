@@ -206,6 +206,29 @@ def test_grpo_reference_grid(dev, batch_size, seq_len, num_groups, seed):
     _close(a4, want4, atol=1e-5, what="grpo without std")
 
 
+def test_grpo_nearly_equal_scores_are_held_to_fp64(dev):
+    """Two-member groups whose scores nearly coincide: (s - mean) / (std + eps) divides rounding noise by a tiny
+    std, and the reference's own fp32 mean / std is then 1e-4 away from the exact value.  The kernel carries the
+    group statistics in double and must be no further from the fp64 evaluation than the fp32 restatement is."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    g = torch.Generator().manual_seed(11)
+    B, L = 700, 130
+    base = torch.randn(B // 2, generator=g) * 3
+    scores = torch.stack([base, base + torch.randn(B // 2, generator=g) * 0.02], dim=1).reshape(B)   # pairs 0.02 apart
+    mask, lens = _prefix_mask(B, L, g, lo=1)
+    rewards = torch.zeros(B, L)
+    rewards[torch.arange(B), lens - 1] = scores
+    rewards[:, 0] += torch.randn(B, generator=g) * 1e-3
+    index = np.repeat(np.arange(B // 2), 2)
+    got, _ = CA.compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    w32, _ = O.grpo_outcome_advantage(rewards.clone(), mask, index)
+    w64, _ = O.grpo_outcome_advantage(rewards.double(), mask.double(), index)
+    err = (got.cpu().double() - w64).abs().max().item()
+    err32 = (w32.double() - w64).abs().max().item()
+    assert err32 > 1e-5                      # the case is ill-conditioned for fp32
+    assert err <= max(err32, 1e-5), (err, err32)
+
+
 def test_grpo_singletons_equal_scores_and_group_mean_std(dev):
     from verl_amd.trainer.ppo import core_algos as CA
     from verl_amd.utils.groupwise import as_torch_index, group_mean_std
