@@ -857,43 +857,45 @@ __device__ __forceinline__ void grpo_scalars_from_records(const double* __restri
       const int64_t r = rk[k];
       const int g = gi[k];
       const int c = g_cnt[g];
-      const float sck = sc[k];
-      float out;
+      // The scores are fp32 like the reference's, everything after them is evaluated in double and rounded once:
+      // rounding the group mean to fp32 before the subtraction would cost 1e-4 of the advantage in a group whose
+      // scores nearly coincide.
+      const double sck = (double)sc[k];
+      const double mean = c > 1 ? g_sum[g] / (double)c : 0.0;
+      double out;
       switch (estimator) {
         case VAMD_ADV_GRPO: {
-          float mu = 0.f, sd = 1.f;
+          double sd = 1.0;
           if (c > 1) {
             const double var = g_sq[g] / (double)(c - 1);
-            mu = (float)(g_sum[g] / (double)c);
-            sd = ga.std_mode == 0 ? (float)sqrt(var) : sqrtf(fmaxf((float)var, ga.eps));
+            sd = ga.std_mode == 0 ? sqrt(var) : sqrt(fmax(var, (double)ga.eps));
           }
-          const float cen = sck - mu;
-          out = ga.norm_by_std ? cen / (sd + ga.eps) : cen;
+          const double cen = sck - mean;
+          out = ga.norm_by_std ? cen / (sd + (double)ga.eps) : cen;
         } break;
         case VAMD_ADV_RLOO:
         case VAMD_ADV_RLOO_VECTORIZED: {
           if (c > 1) {
-            const float mu = (float)(g_sum[g] / (double)c);
-            const float n = (float)c, n1 = (float)(c - 1);
-            out = sck * n / n1 - mu * n / n1;
+            const double n = (double)c, n1 = (double)(c - 1);
+            out = sck * n / n1 - mean * n / n1;
           } else {
-            out = estimator == VAMD_ADV_RLOO ? sck : 0.f;
+            out = estimator == VAMD_ADV_RLOO ? sck : 0.0;
           }
         } break;
         case VAMD_ADV_OPO:
-          out = c > 1 ? sck - (float)(g_sum[g] / g_sq[g]) : sck;
+          out = c > 1 ? sck - g_sum[g] / g_sq[g] : sck;
           break;
         case VAMD_ADV_GPG:
-          out = alpha * (sck - (c > 1 ? (float)(g_sum[g] / (double)c) : 0.f)) / ga.f_norm;
+          out = (double)alpha * (sck - mean) / (double)ga.f_norm;
           break;
         case VAMD_ADV_GRPO_PASSK:
-          out = (double)r == g_sq[g] ? (float)g_sum[g] : 0.f;
+          out = (double)r == g_sq[g] ? g_sum[g] : 0.0;
           break;
         default:  // VAMD_ADV_MEAN_BASELINE
-          out = sck - (c > 1 ? (float)(g_sum[g] / (double)c) : 0.f);
+          out = sck - mean;
           break;
       }
-      ga.scalars[r] = out;
+      ga.scalars[r] = (float)out;
     }
   }
 }
