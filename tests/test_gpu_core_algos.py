@@ -206,6 +206,30 @@ def test_grpo_reference_grid(dev, batch_size, seq_len, num_groups, seed):
     _close(a4, want4, atol=1e-5, what="grpo without std")
 
 
+def test_grpo_with_more_groups_than_one_workgroup_holds(dev):
+    """More than 2048 groups: row sums, one thread per group for the statistics, one per response for the scalar."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    torch.manual_seed(21); random.seed(21); np.random.seed(21)
+    B, L, G = 5200, 37, 2400
+    index = _make_group_index(B, G)
+    mask = _rand_mask(B, L)
+    rewards = torch.randn(B, L) * mask
+    # with 2400 mostly two-member groups some pairs of scores nearly tie, and there the fp32 rounding of a score
+    # decides the advantage (in the reference too): compare the rows of groups whose scores are at least 0.01 apart
+    scores = rewards.double().sum(-1).numpy()
+    spread = np.array([np.ptp(scores[index == gidx]) for gidx in range(G)])
+    rows = torch.from_numpy(spread[index] > 1e-2)
+    assert rows.float().mean() > 0.95
+    for fn, of in ((CA.compute_grpo_outcome_advantage, O.grpo_outcome_advantage),
+                   (CA.compute_grpo_vectorized_outcome_advantage, O.grpo_vectorized_outcome_advantage)):
+        got, _ = fn(rewards.to(dev), mask.to(dev), index)
+        w32, _ = of(rewards.clone(), mask, index)
+        w64, _ = of(rewards.double(), mask.double(), index)
+        err = (got.cpu().double() - w64)[rows].abs().max().item()
+        assert err <= max(2 * (w32.double() - w64)[rows].abs().max().item(), 2e-5), err
+        assert torch.equal(got.cpu() == 0, w32 == 0)
+
+
 def test_grpo_nearly_equal_scores_are_held_to_fp64(dev):
     """Two-member groups whose scores nearly coincide: (s - mean) / (std + eps) divides rounding noise by a tiny
     std, and the reference's own fp32 mean / std is then 1e-4 away from the exact value.  The kernel carries the

@@ -691,8 +691,8 @@ struct GrpoArgs {
   const double* row_moments;  // OPO: [rows][4] per-row masked moments, slot 0 = response length
   float* scores;   // [rows] scratch
   float* scalars;  // [rows] out: normalised scalar per response
-  float* mean;     // [n_groups] (only used by the large-group-count path)
-  float* stdv;
+  double* mean;    // [n_groups] (only used by the large-group-count path)
+  double* stdv;
 };
 
 // Row sums of the rewards (the mask is NOT applied, core_algos.py:303); the last workgroup turns
@@ -947,10 +947,12 @@ __global__ void rowsum_finalize_kernel(const double* __restrict__ partials, int6
   scores[r] = (float)s;
 }
 
-// One thread per group: count, mean, std over the group's members in index order.
+// One thread per group: count, mean, std over the group's members in index order; written as fp32 for
+// group_mean_std itself and in double for the GRPO path, which subtracts and divides in double.
+template <class T>
 __global__ void group_stats_kernel(const float* __restrict__ scores, const int64_t* __restrict__ gid, int64_t n,
-                                   int64_t n_groups, float eps, int std_mode, float* __restrict__ mean,
-                                   float* __restrict__ stdv, float* __restrict__ count) {
+                                   int64_t n_groups, float eps, int std_mode, T* __restrict__ mean,
+                                   T* __restrict__ stdv, float* __restrict__ count) {
   const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (g >= n_groups) return;
   double s = 0;
@@ -960,7 +962,7 @@ __global__ void group_stats_kernel(const float* __restrict__ scores, const int64
       s += scores[i];
       ++c;
     }
-  float mu = 0.f, sd = 1.f;
+  double mu = 0.0, sd = 1.0;
   if (c > 1) {
     const double m = s / (double)c;
     double q = 0;
@@ -970,22 +972,23 @@ __global__ void group_stats_kernel(const float* __restrict__ scores, const int64
         q += d * d;
       }
     const double var = q / (double)(c - 1);
-    mu = (float)m;
-    sd = std_mode == 0 ? (float)sqrt(var) : sqrtf(fmaxf((float)var, eps));
+    mu = m;
+    if (std_mode == 0) sd = sqrt(var);
+    else sd = sizeof(T) == sizeof(double) ? sqrt(fmax(var, (double)eps)) : (double)sqrtf(fmaxf((float)var, eps));
   }
-  mean[g] = mu;
-  stdv[g] = sd;
+  mean[g] = (T)mu;
+  stdv[g] = (T)sd;
   if (count) count[g] = (float)c;
 }
 
 __global__ void grpo_scalars_kernel(const float* __restrict__ scores, const int64_t* __restrict__ gid, int64_t n,
-                                    const float* __restrict__ mean, const float* __restrict__ stdv, float eps,
+                                    const double* __restrict__ mean, const double* __restrict__ stdv, float eps,
                                     int norm_by_std, float* __restrict__ scalars) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= n) return;
   const int64_t g = gid[i];
-  const float c = scores[i] - mean[g];
-  scalars[i] = norm_by_std ? c / (stdv[g] + eps) : c;
+  const double c = (double)scores[i] - mean[g];
+  scalars[i] = (float)(norm_by_std ? c / (stdv[g] + (double)eps) : c);
 }
 
 // adv[i][t] = scalars[i] * (float)mask[i][t]
@@ -1451,14 +1454,14 @@ extern "C" size_t vamd_grpo_workspace_bytes(int64_t batch, int64_t length, int64
   if (batch <= 0 || length <= 0 || n_groups <= 0) return 0;
   size_t b = reduce_workspace_bytes(batch, length, 1);
   b += 2 * align_up((size_t)batch * sizeof(float), 256);     // scores, scalars
-  b += 2 * align_up((size_t)n_groups * sizeof(float), 256);  // mean, std (large-group-count path)
+  b += 2 * align_up((size_t)n_groups * sizeof(double), 256);  // mean, std (large-group-count path)
   return b;
 }
 
 extern "C" int vamd_group_mean_std(const float* scores, const int64_t* group_ids, int64_t n, int64_t n_groups,
                                    float eps, float* mean, float* std, float* count, void* stream) {
   VAMD_REQUIRE(scores && group_ids && mean && std && n > 0 && n_groups > 0, "group_mean_std: bad argument");
-  hipLaunchKernelGGL(group_stats_kernel, dim3((unsigned)((n_groups + 63) / 64)), dim3(64), 0,
+  hipLaunchKernelGGL(group_stats_kernel<float>, dim3((unsigned)((n_groups + 63) / 64)), dim3(64), 0,
                      static_cast<hipStream_t>(stream), scores, group_ids, n, n_groups, eps, 1, mean, std, count);
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
@@ -1522,8 +1525,8 @@ extern "C" int vamd_group_outcome_advantage(const float* rewards, const void* ma
   ga.scores = carve.take<float>((size_t)batch);
   float* scalars = carve.take<float>((size_t)batch);
   ga.scalars = scores_out ? scores_out : scalars;
-  ga.mean = carve.take<float>((size_t)n_groups);
-  ga.stdv = carve.take<float>((size_t)n_groups);
+  ga.mean = carve.take<double>((size_t)n_groups);
+  ga.stdv = carve.take<double>((size_t)n_groups);
   ga.row_moments = nullptr;
   if (opo) {  // response lengths: per-row masked moments of the rewards, slot 0 = sum(mask)
     double* row_moments = carve.take<double>((size_t)batch * 4);
@@ -1558,7 +1561,7 @@ extern "C" int vamd_group_outcome_advantage(const float* rewards, const void* ma
     hipLaunchKernelGGL(rowsum_finalize_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, wk.partials,
                        batch, chunks, ga.scores);
     VAMD_LAUNCH_CHECK();
-    hipLaunchKernelGGL(group_stats_kernel, dim3((unsigned)((n_groups + 63) / 64)), dim3(64), 0, s, ga.scores,
+    hipLaunchKernelGGL(group_stats_kernel<double>, dim3((unsigned)((n_groups + 63) / 64)), dim3(64), 0, s, ga.scores,
                        group_ids, batch, n_groups, epsilon, std_mode, ga.mean, ga.stdv, (float*)nullptr);
     VAMD_LAUNCH_CHECK();
     hipLaunchKernelGGL(grpo_scalars_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, ga.scores,
