@@ -92,7 +92,8 @@ def test_masked_edge_cases(dev):
 
 
 # ---- GAE ----------------------------------------------------------------------------------------
-@pytest.mark.parametrize("B,L", [(1, 2), (3, 7), (3, 64), (5, 1023), (4, 1024), (3, 1025), (2, 4100), (16, 4096)])
+@pytest.mark.parametrize("B,L", [(1, 2), (3, 7), (3, 64), (5, 1023), (4, 1024), (3, 1025), (2, 4100), (16, 4096),
+                                 (1300, 70)])      # the last: more rows than one trip of the statistics fold
 @pytest.mark.parametrize("gamma,lam", [(1.0, 0.95), (0.99, 0.9), (0.95, 0.5)])
 def test_gae_against_oracle(dev, B, L, gamma, lam):
     from verl_amd.trainer.ppo.core_algos import compute_gae_advantage_return
@@ -521,7 +522,7 @@ def test_group_estimators_on_every_statistics_path(dev, batch_size, seq_len, num
         assert torch.equal(got.cpu() != 0, want != 0)
 
 
-@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192)])
+@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192), (1300, 70)])
 @pytest.mark.parametrize("mdtype", [torch.float32, torch.int64])
 def test_reinforce_plus_plus_and_remax(dev, shape, mdtype):
     from verl_amd.trainer.ppo import core_algos as CA
@@ -1002,7 +1003,7 @@ def _data(batch, non_tensor=None):
     return types.SimpleNamespace(batch=_Batch(batch), non_tensor_batch=non_tensor or {})
 
 
-@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192)])
+@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192), (1300, 70)])
 @pytest.mark.parametrize("kind", ["kl", "abs", "mse", "low_var_kl"])
 @pytest.mark.parametrize("mdtype", [torch.float32, torch.int64, torch.bool])
 def test_kl_penalised_rewards(dev, shape, kind, mdtype):
@@ -1328,7 +1329,7 @@ def test_rollout_rejection_reference_literals_and_unified_entry(dev):
     _close(torch.autograd.grad(loss, nd)[0], torch.autograd.grad(want_loss, no)[0], atol=1e-9, what="d bypass loss")
 
 
-@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192)])
+@pytest.mark.parametrize("shape", [(3, 17), (16, 1024), (5, 4099), (64, 8192), (1300, 70)])
 @pytest.mark.parametrize("with_isw", [False, True])
 @pytest.mark.parametrize("mdtype", [torch.float32, torch.int64])
 def test_variance_proxy_metrics(dev, shape, with_isw, mdtype):
