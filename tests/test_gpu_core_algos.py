@@ -979,6 +979,45 @@ def test_benchmark_config_gae_value_policy_loss(dev):
 
 
 @pytest.mark.gpu
+def test_sliced_inputs_give_the_same_results(dev):
+    """The trainer hands over response-window slices of longer tensors: strided views must give what their
+    contiguous copies give, bit for bit, and gradients must arrive on the view's base."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.utils import torch_functional as F
+    B, L, pad = 9, 1030, 5
+    g = torch.Generator().manual_seed(4)
+    wide = lambda: torch.randn(B, L + 2 * pad, generator=g).to(dev)
+    old_w, new_w, adv_w, val_w = wide(), wide(), wide(), wide()
+    lens = torch.randint(1, L + 1, (B,), generator=g)
+    mask_w = torch.zeros(B, L + 2 * pad)
+    mask_w[:, pad:pad + L] = (torch.arange(L)[None, :] < lens[:, None]).float()
+    mask_w = mask_w.to(dev)
+    cut = lambda t: t[:, pad:pad + L]
+    old, new, adv, val, mask = (cut(t) for t in (old_w, new_w, adv_w, val_w, mask_w))
+    assert not new.is_contiguous()
+    c = lambda t: t.contiguous()
+    assert torch.equal(F.masked_mean(new, mask), F.masked_mean(c(new), c(mask)))
+    assert torch.equal(F.masked_whiten(new, mask), F.masked_whiten(c(new), c(mask)))
+    a1, r1 = CA.compute_gae_advantage_return(adv * mask, val, mask, 0.99, 0.95)
+    a2, r2 = CA.compute_gae_advantage_return(c(adv * mask), c(val), c(mask), 0.99, 0.95)
+    assert torch.equal(a1, a2) and torch.equal(r1, r2)
+    index = np.arange(B) % 3
+    g1, _ = CA.compute_grpo_outcome_advantage(adv * mask, mask, index)
+    g2, _ = CA.compute_grpo_outcome_advantage(c(adv * mask), c(mask), index)
+    assert torch.equal(g1, g2)
+    base = new_w.clone().requires_grad_()
+    leaf = new.contiguous().clone().requires_grad_()
+    l1, _ = CA.compute_policy_loss_vanilla(old, cut(base), adv, mask, "token-mean", _cfg())
+    l2, _ = CA.compute_policy_loss_vanilla(c(old), leaf, c(adv), c(mask), "token-mean", _cfg())
+    assert torch.equal(l1, l2)
+    gb, = torch.autograd.grad(l1, base)
+    gl, = torch.autograd.grad(l2, leaf)
+    assert torch.equal(cut(gb), gl) and float(gb[:, :pad].abs().max()) == 0 and float(gb[:, pad + L:].abs().max()) == 0
+    v1, _ = CA.compute_value_loss(new, adv, val, mask, 0.5, "seq-mean-token-mean")
+    v2, _ = CA.compute_value_loss(c(new), c(adv), c(val), c(mask), 0.5, "seq-mean-token-mean")
+    assert torch.equal(v1, v2)
+
+
 def test_copy_bytes_is_exact(dev):
     """The measurement yardstick copies every byte, including a tail shorter than one grid stride."""
     from verl_amd import _cabi
