@@ -1018,6 +1018,27 @@ def test_sliced_inputs_give_the_same_results(dev):
     assert torch.equal(v1, v2)
 
 
+def test_two_streams_keep_their_own_counters(dev):
+    """The single-launch reductions keep arrival counters in a workspace; calls issued on two streams run
+    concurrently and must not share one."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.utils import torch_functional as F
+    old, new, adv, mask = (t.to(dev) for t in _policy_inputs(300, 4096, seed=9))
+    want_loss, _ = CA.compute_policy_loss_vanilla(old, new, adv, mask, "seq-mean-token-mean", _cfg())
+    want_mean = F.masked_mean(adv, mask)
+    a, b = torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev)
+    a.wait_stream(torch.cuda.current_stream(dev)); b.wait_stream(torch.cuda.current_stream(dev))
+    got = []
+    for _ in range(20):
+        with torch.cuda.stream(a):
+            got.append(("loss", CA.compute_policy_loss_vanilla(old, new, adv, mask, "seq-mean-token-mean", _cfg())[0]))
+        with torch.cuda.stream(b):
+            got.append(("mean", F.masked_mean(adv, mask)))
+    a.synchronize(); b.synchronize()
+    for kind, value in got:
+        assert torch.equal(value, want_loss if kind == "loss" else want_mean), kind
+
+
 def test_copy_bytes_is_exact(dev):
     """The measurement yardstick copies every byte, including a tail shorter than one grid stride."""
     from verl_amd import _cabi
