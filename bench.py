@@ -212,6 +212,14 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
             lambda: O.policy_loss_vanilla(s["a"], s["b"], s["c"], s["mask"], "token-mean"))
         res["value_loss_fwd_grad"]["cpu_ms"] = cpu_ms(
             lambda: O.value_loss(s["a"], s["b"], s["c"], s["mask"], 0.5, "token-mean"))
+        res["kl_loss_fwd_grad"]["cpu_ms"] = cpu_ms(
+            lambda: O.agg_loss(O.kl_penalty(s["a"], s["b"], "low_var_kl"), s["mask"], "token-mean"))
+        res["masked_moments"]["cpu_ms"] = cpu_ms(lambda: O.masked_var(s["a"], s["mask"]))
+        res["apply_kl_penalty"]["cpu_ms"] = cpu_ms(
+            lambda: O.apply_kl_penalty(s["c"], s["a"], s["b"], s["mask"], 0.05, "kl"))
+        res["rollout_correction_token"]["cpu_ms"] = cpu_ms(
+            lambda: (O.rollout_correction_weights(s["a"] - s["b"], s["mask"], "token", 2.0, False),
+                     O.offpolicy_metrics(s["a"], s["b"], s["mask"])))
     return res
 
 
