@@ -129,6 +129,40 @@ __device__ __forceinline__ void block_reduce(double (&v)[NV], double* smem /* NV
   __syncthreads();
 }
 
+// The same for a dozen values or more per thread.  Carrying every value through every exchange step costs
+// NV x 6 dependent double operations per wavefront; here the wavefront stages its 64 x NV values in LDS and lane j
+// adds up value j over the 64 lanes (in lane order), NV lanes at a time, so the chain is 64 additions whatever NV
+// is.  stage: NT/64 * NV * kWidePitch doubles; the pitch of 65 keeps the lanes' rows on different banks and its
+// last column takes the wavefront's result.  Result valid in thread 0.
+constexpr int kWidePitch = 65;
+template <int NV, int NT, class Op>
+__device__ __forceinline__ void block_reduce_wide(double (&v)[NV], double* stage, Op op) {
+  static_assert(NV <= 64, "one lane per value");
+  constexpr int NW = NT / 64;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  double* mine = stage + (size_t)w * NV * kWidePitch;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) mine[i * kWidePitch + lane] = v[i];
+  __syncthreads();
+  if (lane < NV) {
+    const double* row = mine + lane * kWidePitch;
+    double s = row[0];
+#pragma unroll 8
+    for (int l = 1; l < 64; ++l) s = op(s, row[l]);
+    mine[lane * kWidePitch + 64] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      double r = stage[i * kWidePitch + 64];
+      for (int j = 1; j < NW; ++j) r = op(r, stage[(size_t)j * NV * kWidePitch + i * kWidePitch + 64]);
+      v[i] = r;
+    }
+  }
+  __syncthreads();
+}
+
 template <int NV, int NT>
 __device__ __forceinline__ void block_sum(double (&v)[NV], double* smem) {
   block_reduce<NV, NT>(v, smem, SumOp());

@@ -42,7 +42,9 @@ struct DmArgs {
   double* out;      // [VAMD_DM_COUNT]
 };
 
-template <bool VEC, class M, class A>
+// WIDE: the 17-value workgroup reduction through an LDS staging area (block_reduce_wide), which shortens the tail
+// of a launch of one round of workgroups; its 23 KB per workgroup would cost a larger launch its occupancy.
+template <bool VEC, class M, class A, bool WIDE>
 __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, const M* __restrict__ mask,
                                                                   const A* __restrict__ attention) {
   const int64_t row = blockIdx.x / a.chunks;
@@ -105,10 +107,15 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
     for (int64_t c = threadIdx.x; c < a.prompt; c += kRcThreads) prompt_len += (float)attention[p0 + c];
     acc[kDmPromptLen] += (double)prompt_len;
   }
-  __shared__ double smem[kDmSums * 4];
-  block_sum<kDmSums, kRcThreads>(acc, smem);
+  __shared__ double stage[WIDE ? 4 * kDmSums * kWidePitch : kDmSums * 4];
   double ext[6] = {hi[0], -(double)lo[0], hi[1], -(double)lo[1], hi[2], -(double)lo[2]};
-  block_max<6, kRcThreads>(ext, smem);
+  if constexpr (WIDE) {
+    block_reduce_wide<kDmSums, kRcThreads>(acc, stage, SumOp());
+    block_reduce_wide<6, kRcThreads>(ext, stage, MaxOp());
+  } else {
+    block_sum<kDmSums, kRcThreads>(acc, stage);
+    block_max<6, kRcThreads>(ext, stage);
+  }
   if (threadIdx.x == 0) {
     double rec[kDmRec];
 #pragma unroll
@@ -127,7 +134,7 @@ constexpr int kDmFoldThreads = 128;   // a workgroup of the fold launch takes up
 template <int NT>
 __global__ __launch_bounds__(NT) void data_metrics_fold_kernel(DmArgs a) {
   const double inf = __longlong_as_double(0x7ff0000000000000ll);
-  __shared__ double smem[16 * (NT / 64)];
+  __shared__ double stage[(NT / 64) * 16 * kWidePitch];
   // ---- fold: thread-strided over rows -------------------------------------------------------------
   // sums: 0 n_non_aborted 1 score 2 reward 3 resp_len 4 resp_len==cols 5 resp_len (non-aborted)
   //       6 resp_len==cols (non-aborted) 7 prompt_len 8 prompt_len==prompt
@@ -182,9 +189,9 @@ __global__ __launch_bounds__(NT) void data_metrics_fold_kernel(DmArgs a) {
       }
     }
   }
-  block_sum<9 + kElem, NT>(t, smem);
-  block_max<16, NT>(x, smem);
-  if (!fold_across_workgroups<9 + kElem, 16, NT>(t, x, a.shares, a.fold_counter, smem)) return;
+  block_reduce_wide<9 + kElem, NT>(t, stage, SumOp());
+  block_reduce_wide<16, NT>(x, stage, MaxOp());
+  if (!fold_across_workgroups<9 + kElem, 16, NT>(t, x, a.shares, a.fold_counter, stage)) return;
   if (threadIdx.x == 0) {
     double* o = a.out;
     const double B = (double)a.rows, na = t[0];
@@ -329,16 +336,20 @@ extern "C" int vamd_data_metrics(const float* token_level_scores, const float* t
   a.out = out;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)(batch * a.chunks)), block(kRcThreads);
+  const bool wide = batch * a.chunks <= 1024;  // one round of workgroups at six per CU
 #define VAMD_DM(A)                                                                                            \
   VAMD_MASK_DISPATCH(mask_dtype, M, {                                                                          \
     const bool vec = can_vectorize(response_length, {token_level_scores, token_level_rewards, advantages,      \
                                                      returns, values}, response_mask, sizeof(M)) &&            \
                      prompt_length % 4 == 0 && aligned_to(attention_mask, 4 * sizeof(A));                      \
-    if (vec)                                                                                                   \
-      hipLaunchKernelGGL((data_metrics_kernel<true, M, A>), grid, block, 0, s, a,                              \
+    if (vec && wide)                                                                                           \
+      hipLaunchKernelGGL((data_metrics_kernel<true, M, A, true>), grid, block, 0, s, a,                        \
+                         static_cast<const M*>(response_mask), static_cast<const A*>(attention_mask));         \
+    else if (vec)                                                                                              \
+      hipLaunchKernelGGL((data_metrics_kernel<true, M, A, false>), grid, block, 0, s, a,                       \
                          static_cast<const M*>(response_mask), static_cast<const A*>(attention_mask));         \
     else                                                                                                       \
-      hipLaunchKernelGGL((data_metrics_kernel<false, M, A>), grid, block, 0, s, a,                             \
+      hipLaunchKernelGGL((data_metrics_kernel<false, M, A, false>), grid, block, 0, s, a,                      \
                          static_cast<const M*>(response_mask), static_cast<const A*>(attention_mask));         \
   })
   switch (attention_dtype) {

@@ -131,7 +131,7 @@ constexpr int kRcFoldThreads = 128;   // a workgroup of the fold launch takes up
 template <int NT>
 __global__ __launch_bounds__(NT) void rollout_fold_kernel(RcArgs a) {
   const double inf = __longlong_as_double(0x7ff0000000000000ll);
-  __shared__ double smem[26 * (NT / 64)];
+  __shared__ double stage[(NT / 64) * 26 * kWidePitch];
   enum {
     tM = 0, tD, tK3, tRho2, tW, tC, tC2, tTrunc, tHigh, tLow,         // token totals
     tTrainPpl, tTrainLog, tRollPpl, tRollLog, tGap, tGapAbs, tRatio, tChiSeq,  // sums over rows
@@ -216,10 +216,10 @@ __global__ __launch_bounds__(NT) void rollout_fold_kernel(RcArgs a) {
       }
     }
   }
-  static_assert(tN <= 26, "smem is sized for 26 sums");
-  block_sum<tN, NT>(t, smem);
-  block_max_f64<xN, NT>(x, smem);
-  if (!fold_across_workgroups<tN, xN, NT>(t, x, a.shares, a.fold_counter, smem)) return;
+  static_assert(tN <= 26 && xN <= 26, "the staging area is sized for 26 values");
+  block_reduce_wide<tN, NT>(t, stage, SumOp());
+  block_reduce_wide<xN, NT>(x, stage, MaxOp());
+  if (!fold_across_workgroups<tN, xN, NT>(t, x, a.shares, a.fold_counter, stage)) return;
   if (threadIdx.x == 0) {
     double* o = a.out;
     const double B = (double)a.rows, Mt = t[tM];

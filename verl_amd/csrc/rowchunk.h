@@ -365,7 +365,8 @@ inline int record_span(int64_t rows, int chunks) {
 // counter: zero when the launch starts (the streaming pass before it clears it).
 template <int NS, int NX, int NT>
 __device__ __forceinline__ bool fold_across_workgroups(double (&t)[NS], double (&x)[NX], double* __restrict__ shares,
-                                                       unsigned* counter, double* smem /* max(NS, NX) * NT/64 */) {
+                                                       unsigned* counter,
+                                                       double* stage /* as block_reduce_wide, max(NS, NX) values */) {
   const unsigned nb = gridDim.x;
   if (nb == 1) return true;
   __shared__ unsigned last;
@@ -395,8 +396,8 @@ __device__ __forceinline__ bool fold_across_workgroups(double (&t)[NS], double (
 #pragma unroll
     for (int i = 0; i < NX; ++i) x[i] = fmax(x[i], xs[i]);
   }
-  block_reduce<NS, NT>(t, smem, SumOp());
-  block_reduce<NX, NT>(x, smem, MaxOp());
+  block_reduce_wide<NS, NT>(t, stage, SumOp());
+  block_reduce_wide<NX, NT>(x, stage, MaxOp());
   return true;
 }
 
