@@ -11,7 +11,7 @@
 // Two launches.  The first walks every row twice inside one workgroup -- right to left for the
 // returns, left to right for W -- as plain prefix sums carried in double (1024-column segments,
 // 4 columns per thread, wavefront scan by lane exchanges plus the four wavefront totals through LDS).  The
-// second gives each (group, 4096-column chunk) to one workgroup, which adds up the group's rows
+// second gives each (group, 1024-column segment) to one workgroup, which adds up the group's rows
 // column by column in index order, forms the baseline and writes the advantages of those rows.
 // Nothing is reduced across workgroups, so neither launch needs arrival counters.
 //
@@ -162,73 +162,89 @@ struct OtbGroups {
   const int64_t* row_len;        // packed rows: columns below row_len[row] are valid and the mask is not read
 };
 
+// Mask of the 4 columns at `col` of `row`: read, or implied by the row's packed length.
 template <bool VEC, class M>
-__device__ __forceinline__ void otb_mask_groups(const M* __restrict__ mask, const OtbGroups& gr, int64_t row,
-                                                int64_t cols, const ChunkPos& pos, float (&m)[kGroups][4]) {
+__device__ __forceinline__ void otb_mask4(const M* __restrict__ mask, const OtbGroups& gr, int64_t row, int64_t cols,
+                                          int64_t col, int valid, float (&m)[4]) {
   if (gr.row_len) {
     const int64_t n = gr.row_len[row];
 #pragma unroll
-    for (int k = 0; k < kGroups; ++k)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) m[k][e] = (e < pos.valid[k] && pos.idx[k] - row * cols + e < n) ? 1.f : 0.f;
+    for (int e = 0; e < 4; ++e) m[e] = (e < valid && col + e < n) ? 1.f : 0.f;
   } else {
-    load_mask_groups<VEC>(mask, pos, m);
+    ldmask4<VEC>(mask, row * cols + col, valid, m);
   }
 }
 
+constexpr int kOtbRows = 4;  // rows of a group whose loads are in flight together
+
+// One workgroup per (group, 1024-column segment), a thread per 4 columns: the group's rows are added up in index
+// order, kOtbRows of them in flight at a time (a group is a handful of rows, so the launch needs narrow segments to
+// fill the device, and a thread walking the rows one load at a time would wait out every trip to memory).
 // `adv` may be `returns` itself (each thread overwrites only what it has just read).
 template <bool VEC, class M>
 __global__ __launch_bounds__(kRcThreads) void otb_baseline_kernel(const float* returns,
                                                                   const float* __restrict__ w_cum,
                                                                   const M* __restrict__ mask, OtbGroups gr,
-                                                                  int64_t cols, int chunks, float eps, float* adv) {
-  const int64_t g = blockIdx.x / chunks;
-  const int chunk = blockIdx.x % chunks;
+                                                                  int64_t cols, int segs, float eps, float* adv) {
+  const int64_t g = blockIdx.x / segs;
+  const int64_t col = (int64_t)(blockIdx.x % segs) * kOtbSeg + threadIdx.x * 4;
+  const int64_t left = cols - col;
+  const int valid = left >= 4 ? 4 : (left > 0 ? (int)left : 0);
+  if (valid == 0) return;
   const int64_t first = gr.group_offsets[g], last = gr.group_offsets[g + 1];
-  float num[kGroups][4], den[kGroups][4];
-#pragma unroll
-  for (int k = 0; k < kGroups; ++k)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) num[k][e] = den[k][e] = 0.f;
+  float num[4] = {0.f, 0.f, 0.f, 0.f}, den[4] = {0.f, 0.f, 0.f, 0.f};
   if (last - first > 1) {
-    for (int64_t i = first; i < last; ++i) {
-      const int64_t row = gr.rows_by_group[i];
-      const ChunkPos pos(row, chunk, cols);
-      float R[kGroups][4], W[kGroups][4], m[kGroups][4];
-      load_groups<VEC>(returns, pos, R);
-      load_groups<VEC>(w_cum, pos, W);
-      otb_mask_groups<VEC>(mask, gr, row, cols, pos, m);
+    for (int64_t i0 = first; i0 < last; i0 += kOtbRows) {
+      float R[kOtbRows][4], W[kOtbRows][4], m[kOtbRows][4];
 #pragma unroll
-      for (int k = 0; k < kGroups; ++k)
+      for (int k = 0; k < kOtbRows; ++k) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (m[k][e] != 0.f) {  // packed rows hold no defined value beyond their length
-            num[k][e] += R[k][e] * W[k][e] * m[k][e];
-            den[k][e] += W[k][e] * m[k][e];
-          }
+        for (int e = 0; e < 4; ++e) R[k][e] = W[k][e] = m[k][e] = 0.f;
+        if (i0 + k < last) {
+          const int64_t row = gr.rows_by_group[i0 + k];
+          ld4<VEC>(returns, row * cols + col, valid, R[k]);
+          ld4<VEC>(w_cum, row * cols + col, valid, W[k]);
+          otb_mask4<VEC>(mask, gr, row, cols, col, valid, m[k]);
         }
+      }
+#pragma unroll
+      for (int k = 0; k < kOtbRows; ++k)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (m[k][e] != 0.f) {  // packed rows hold no defined value beyond their length
+            num[e] += R[k][e] * W[k][e] * m[k][e];
+            den[e] += W[k][e] * m[k][e];
+          }
     }
 #pragma unroll
-    for (int k = 0; k < kGroups; ++k)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) num[k][e] = num[k][e] / (den[k][e] + eps);  // the baseline
+    for (int e = 0; e < 4; ++e) num[e] = num[e] / (den[e] + eps);  // the baseline
   }
-  for (int64_t i = first; i < last; ++i) {
-    const int64_t row = gr.rows_by_group[i];
-    const ChunkPos pos(row, chunk, cols);
-    const int64_t cut = gr.tail_start ? gr.tail_start[row] : cols;
-    float R[kGroups][4], m[kGroups][4];
-    load_groups<VEC>(returns, pos, R);
-    otb_mask_groups<VEC>(mask, gr, row, cols, pos, m);
+  for (int64_t i0 = first; i0 < last; i0 += kOtbRows) {
+    float R[kOtbRows][4], m[kOtbRows][4];
+    int64_t row[kOtbRows], cut[kOtbRows];
 #pragma unroll
-    for (int k = 0; k < kGroups; ++k)
+    for (int k = 0; k < kOtbRows; ++k) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) R[k][e] = m[k][e] = 0.f;
+      row[k] = -1;
+      cut[k] = 0;
+      if (i0 + k < last) {
+        row[k] = gr.rows_by_group[i0 + k];
+        cut[k] = gr.tail_start ? gr.tail_start[row[k]] : cols;
+        ld4<VEC>(returns, row[k] * cols + col, valid, R[k]);
+        otb_mask4<VEC>(mask, gr, row[k], cols, col, valid, m[k]);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kOtbRows; ++k) {
+      if (row[k] < 0) break;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int64_t col = pos.idx[k] - row * cols + e;
-        const float b = col < cut ? num[k][e] : 0.f;
+        const float b = col + e < cut[k] ? num[e] : 0.f;
         R[k][e] = m[k][e] != 0.f ? (R[k][e] - b) * m[k][e] : 0.f;
       }
-    store_groups<VEC>(adv, pos, R);
+      st4<VEC>(adv, row[k] * cols + col, valid, R[k]);
+    }
   }
 }
 
@@ -269,7 +285,7 @@ extern "C" int vamd_otb_advantage(const float* rewards, const void* mask, int ma
                                   int64_t length, int64_t n_groups, int packed, float epsilon, float* advantages,
                                   float* returns, void* workspace, size_t workspace_bytes, void* stream) {
   VAMD_REQUIRE(batch > 0 && length > 0 && n_groups >= 0, "otb_advantage: empty input");
-  VAMD_REQUIRE(batch * chunks_of(length) < (1ll << 31) && n_groups * chunks_of(length) < (1ll << 31),
+  VAMD_REQUIRE(batch * chunks_of(length) < (1ll << 31) && n_groups * ((length + kOtbSeg - 1) / kOtbSeg) < (1ll << 31),
                "otb_advantage: too many workgroups");
   VAMD_REQUIRE(length < (1ll << 24), "otb_advantage: rows longer than 2^24 - 1 columns are not supported");
   VAMD_REQUIRE(rewards && mask && old_log_probs && sum_pi_squared && advantages && returns,
@@ -293,7 +309,8 @@ extern "C" int vamd_otb_advantage(const float* rewards, const void* mask, int ma
   }
   const int chunks = (int)chunks_of(length);
   const OtbGroups gr{rows_by_group, group_offsets, tail_start, pk.row_len};
-  const dim3 threads(kRcThreads), per_row((unsigned)batch), per_group((unsigned)(n_groups * chunks)),
+  const int segs = (int)((length + kOtbSeg - 1) / kOtbSeg);  // 1024-column segments of the baseline pass
+  const dim3 threads(kRcThreads), per_row((unsigned)batch), per_group((unsigned)(n_groups * segs)),
       per_chunk((unsigned)(batch * chunks));
 #define VAMD_OTB(V, W)                                                                                              \
   do {                                                                                                              \
@@ -302,14 +319,14 @@ extern "C" int vamd_otb_advantage(const float* rewards, const void* mask, int ma
                          sum_pi_squared, is_weights, length, returns, w_cum, pk);                                   \
       if (n_groups > 0)                                                                                             \
         hipLaunchKernelGGL((otb_baseline_kernel<V, M>), per_group, threads, 0, s, pk.g, pk.w, mk, gr, length,        \
-                           chunks, epsilon, pk.g);                                                                  \
+                           segs, epsilon, pk.g);                                                                    \
       hipLaunchKernelGGL((otb_unpack_kernel<V, M>), per_chunk, threads, 0, s, pk.g, pk.rank, mk, length, chunks,     \
                          advantages);                                                                               \
     } else {                                                                                                        \
       hipLaunchKernelGGL((otb_scan_kernel<V, M, W, false>), per_row, threads, 0, s, rewards, mk, old_log_probs,      \
                          sum_pi_squared, is_weights, length, returns, w_cum, pk);                                   \
       hipLaunchKernelGGL((otb_baseline_kernel<V, M>), per_group, threads, 0, s, returns, w_cum, mk, gr, length,      \
-                         chunks, epsilon, advantages);                                                              \
+                         segs, epsilon, advantages);                                                                \
     }                                                                                                               \
   } while (0)
   VAMD_MASK_DISPATCH(mask_dtype, M, {
