@@ -120,6 +120,21 @@ int vamd_lce_forward(const void* hidden, const void* weight, const int64_t* labe
                      float* lse, float* mean_z, float* logits_cache, float* sum_pi_squared, void* workspace,
                      size_t workspace_bytes, void* stream);
 
+/* The forward pass for callers that cannot allocate device memory or hand over a workspace: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments, arithmetic and results as vamd_lce_forward without a logits cache; the
+ * softmax partials of the (token tile, vocabulary split) workgroups go to a buffer built into the library
+ * (VAMD_LCE_STATIC_MAX_TOKENS * 20 + 512 bytes of device memory, held by every GPU the library is
+ * used on until the process ends).  n_tokens above VAMD_LCE_STATIC_MAX_TOKENS is refused with VAMD_EINVAL.
+ * The call allocates nothing and records no memset.  All calls on one GPU share the one buffer: calls on
+ * different streams of the same GPU that may overlap race on it; calls ordered on one stream do not.
+ * The first call on a device looks up the buffer's address and raises the kernels' LDS limit, so make it
+ * before a capture begins. */
+#define VAMD_LCE_STATIC_MAX_TOKENS 65536
+int vamd_lce_forward_static(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
+                            int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs,
+                            float* entropy, float* lse, float* mean_z, float* sum_pi_squared, void* stream);
+
 /* Backward: d_logits = [g_lp (onehot - p) - g_ent p (z - mean_z)] * rcp_temperature is formed
  * tile by tile from recomputed logits, never as a whole; d_hidden = d_logits . weight,
  * d_weight = d_logits^T . hidden, both accumulated in fp32 and rounded to bf16 once.

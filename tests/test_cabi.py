@@ -118,3 +118,9 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert res.returncode != 0 and "one GPU" in res.stderr and res.stdout.strip() == ""
+
+
+def test_static_forward_refuses_sizes_beyond_its_buffer_before_any_gpu_call(lib):
+    # the pointers are never dereferenced: the size check precedes every HIP call
+    rc = lib.vamd_lce_forward_static(1, 1, 1, 65536 + 1, 128, 256, 1.0, 1, 1, 1, 1, None, None)
+    assert rc == -1 and b"at most 65536 tokens" in lib.vamd_last_error()

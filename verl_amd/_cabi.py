@@ -33,6 +33,8 @@ SIGNATURES = {
     "vamd_lce_forward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "vamd_lce_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "vamd_lce_forward_static": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p,
+                                        c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "vamd_lce_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
     "vamd_lce_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int64,

@@ -728,20 +728,12 @@ extern "C" size_t vamd_lce_forward_workspace_bytes(int64_t n_tokens, int64_t hid
          align_up((size_t)sp * tok_tiles * kTile * sizeof(float), 256);  // state + squared sums
 }
 
-extern "C" int vamd_lce_forward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
-                                int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs,
-                                float* entropy, float* lse, float* mean_z, float* logits_cache,
-                                float* sum_pi_squared, void* workspace, size_t workspace_bytes, void* stream) {
-  int st = check_head_shapes(n_tokens, hidden_size, vocab);
-  if (st != VAMD_OK) return st;
-  VAMD_REQUIRE(hidden && weight && labels && logprobs && entropy && lse && mean_z, "lce_forward: null pointer");
-  VAMD_REQUIRE(rcp_temperature > 0.f, "lce_forward: temperature must be positive");
-  const size_t need = vamd_lce_forward_workspace_bytes(n_tokens, hidden_size, vocab);
-  if (!workspace || workspace_bytes < need) {
-    set_error("lce_forward: workspace %zu bytes, need %zu", workspace_bytes, need);
-    return VAMD_EWORKSPACE;
-  }
-  if ((st = ensure_lds_attributes()) != VAMD_OK) return st;
+// Forward launches shared by the two entry points; `workspace` holds at least
+// vamd_lce_forward_workspace_bytes() bytes and the arguments have been checked.
+static int lce_forward_launch(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
+                              int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs,
+                              float* entropy, float* lse, float* mean_z, float* logits_cache, float* sum_pi_squared,
+                              void* workspace, void* stream) {
 
   FwdArgs a;
   a.hidden = Operand{static_cast<const uint16_t*>(hidden), hidden_size, (int)n_tokens, (int)hidden_size};
@@ -795,6 +787,82 @@ extern "C" int vamd_lce_forward(const void* hidden, const void* weight, const in
   }
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
+}
+
+static int check_forward_args(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
+                              int64_t hidden_size, int64_t vocab, float rcp_temperature, const float* logprobs,
+                              const float* entropy, const float* lse, const float* mean_z) {
+  int st = check_head_shapes(n_tokens, hidden_size, vocab);
+  if (st != VAMD_OK) return st;
+  VAMD_REQUIRE(hidden && weight && labels && logprobs && entropy && lse && mean_z, "lce_forward: null pointer");
+  VAMD_REQUIRE(rcp_temperature > 0.f, "lce_forward: temperature must be positive");
+  return VAMD_OK;
+}
+
+extern "C" int vamd_lce_forward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
+                                int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs,
+                                float* entropy, float* lse, float* mean_z, float* logits_cache,
+                                float* sum_pi_squared, void* workspace, size_t workspace_bytes, void* stream) {
+  int st = check_forward_args(hidden, weight, labels, n_tokens, hidden_size, vocab, rcp_temperature, logprobs, entropy,
+                              lse, mean_z);
+  if (st != VAMD_OK) return st;
+  const size_t need = vamd_lce_forward_workspace_bytes(n_tokens, hidden_size, vocab);
+  if (!workspace || workspace_bytes < need) {
+    set_error("lce_forward: workspace %zu bytes, need %zu", workspace_bytes, need);
+    return VAMD_EWORKSPACE;
+  }
+  if ((st = ensure_lds_attributes()) != VAMD_OK) return st;
+  return lce_forward_launch(hidden, weight, labels, n_tokens, hidden_size, vocab, rcp_temperature, logprobs, entropy,
+                            lse, mean_z, logits_cache, sum_pi_squared, workspace, stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// The forward pass for callers that cannot allocate: the per-(token tile, vocabulary split)
+// softmax partials live in a file-scope device array instead of a caller workspace.  Every GPU
+// holds its own copy of the array at its own address; the address is looked up once per device.
+// The array's name is only a host-side handle for that lookup: launches and copies use the
+// looked-up pointer.
+namespace vamd {
+constexpr size_t kStaticScratchBytes = (size_t)VAMD_LCE_STATIC_MAX_TOKENS * (sizeof(float4) + sizeof(float)) + 512;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static int static_scratch_pointer(void** out) {
+  static std::mutex mu;
+  static void* ptr_by_device[64];
+  int dev = 0;
+  VAMD_HIP(hipGetDevice(&dev));
+  VAMD_REQUIRE(dev >= 0 && dev < 64, "lce: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr_by_device[dev]) {
+    void* p = nullptr;
+    VAMD_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    VAMD_REQUIRE(p != nullptr, "lce: the static scratch array has no device address");
+    ptr_by_device[dev] = p;
+  }
+  *out = ptr_by_device[dev];
+  return VAMD_OK;
+}
+}  // namespace vamd
+
+extern "C" int vamd_lce_forward_static(const void* hidden, const void* weight, const int64_t* labels,
+                                       int64_t n_tokens, int64_t hidden_size, int64_t vocab, float rcp_temperature,
+                                       float* logprobs, float* entropy, float* lse, float* mean_z,
+                                       float* sum_pi_squared, void* stream) {
+  int st = check_forward_args(hidden, weight, labels, n_tokens, hidden_size, vocab, rcp_temperature, logprobs, entropy,
+                              lse, mean_z);
+  if (st != VAMD_OK) return st;
+  const size_t need = vamd_lce_forward_workspace_bytes(n_tokens, hidden_size, vocab);
+  VAMD_REQUIRE(n_tokens <= VAMD_LCE_STATIC_MAX_TOKENS && need <= kStaticScratchBytes,
+               "lce_forward_static: %lld tokens need %zu bytes of scratch; the built-in buffer serves at most %d "
+               "tokens (%zu bytes): use vamd_lce_forward with a caller workspace",
+               (long long)n_tokens, need, (int)VAMD_LCE_STATIC_MAX_TOKENS, kStaticScratchBytes);
+  if ((st = ensure_lds_attributes()) != VAMD_OK) return st;
+  void* ws = nullptr;
+  if ((st = static_scratch_pointer(&ws)) != VAMD_OK) return st;
+  // Every partial the merge kernel reads is written by the forward kernel of the same call, so
+  // nothing in the buffer has to start at zero and a previous call's contents do not matter.
+  return lce_forward_launch(hidden, weight, labels, n_tokens, hidden_size, vocab, rcp_temperature, logprobs, entropy,
+                            lse, mean_z, nullptr, sum_pi_squared, ws, stream);
 }
 
 extern "C" size_t vamd_lce_backward_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab,
