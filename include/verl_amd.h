@@ -80,7 +80,7 @@ extern "C" {
 
 /* Bumped whenever an entry point changes its signature or a workspace its layout; a binding compares it with
  * the header it was written against. */
-#define VAMD_ABI_VERSION 3
+#define VAMD_ABI_VERSION 4
 int vamd_abi_version(void);
 const char* vamd_last_error(void);
 
@@ -99,8 +99,8 @@ int vamd_sum4(const float* a, const float* b, const float* c, const float* d, fl
  * verl/utils/kernel/kernels.py:563-753 and :1512-1723).
  *
  *   hidden [n_tokens, hidden_size] bf16 row-major, weight [vocab, hidden_size] bf16 row-major,
- *   labels [n_tokens] int64 in [0, vocab).  hidden_size % 128 == 0 (kernels.py:593),
- *   vocab % 8 == 0.
+ *   labels [n_tokens] int64 in [0, vocab).  hidden_size % 128 == 0 (kernels.py:593); any vocab
+ *   (the vocabulary tail is masked as the reference does); a logits cache needs vocab % 8 == 0.
  *   z = hidden . weight^T * rcp_temperature ; logprobs = z[label] - lse(z) ;
  *   entropy = lse(z) - sum softmax(z) z.
  *   lse[n] and mean_z[n] (= sum softmax(z) z) are saved for the backward pass in place of the
@@ -135,29 +135,48 @@ int vamd_lce_forward_static(const void* hidden, const void* weight, const int64_
                             int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs,
                             float* entropy, float* lse, float* mean_z, float* sum_pi_squared, void* stream);
 
-/* Backward: d_logits = [g_lp (onehot - p) - g_ent p (z - mean_z)] * rcp_temperature is formed
- * tile by tile from recomputed logits, never as a whole; d_hidden = d_logits . weight,
+/* Backward: d_logits = [g_lp (onehot - p) - g_ent p (z - mean_z)] * rcp_temperature is formed one
+ * vocabulary chunk at a time as a bf16 [n_pad, vocab_chunk] panel in the workspace -- from logits
+ * recomputed tile by tile on the matrix cores (logits_cache == NULL: no [n_tokens, vocab] tensor ever
+ * exists, as in the reference, kernels.py:1374-1509) or from the cache the forward call filled (a
+ * streaming pass instead of the recompute GEMM) -- and consumed by d_hidden = d_logits . weight and
  * d_weight = d_logits^T . hidden, both accumulated in fp32 and rounded to bf16 once.
  *   d_logprobs [n] fp32 or NULL (treated as zeros);
  *   d_entropy  [n] fp32 or NULL, in which case the constant d_entropy_scalar is used for every
  *   token (an entropy-bonus coefficient folded into the backward pass);
  *   d_hidden [n, hidden_size] bf16 out; d_weight [vocab, hidden_size] bf16 out.
- *   accumulate_d_weight != 0 adds into d_weight instead of overwriting it (token-chunked use).
+ *   d_weight_mode says where this call's weight gradient goes (token-chunked callers sum several calls):
+ *     VAMD_DW_STORE            d_weight = bf16(g)                                (d_weight_acc32 unused)
+ *     VAMD_DW_ADD_BF16         d_weight = bf16(d_weight + g): one bf16 rounding of the running sum per call,
+ *                              what `weight.grad += d_weight` does in the reference's bf16 training
+ *     VAMD_DW_F32_STORE        d_weight_acc32 = g                                (d_weight may be NULL)
+ *     VAMD_DW_F32_ADD          d_weight_acc32 += g                               (d_weight may be NULL)
+ *     VAMD_DW_F32_ADD_FINISH   d_weight_acc32 += g; d_weight = bf16(d_weight_acc32): the sum over all token
+ *                              chunks is rounded once
+ *   d_weight_acc32: [vocab, hidden_size] fp32, 16-byte aligned, for the three F32 modes.
  * vocab_chunk = 0 lets the library choose how many vocabulary columns of d_logits are staged
  * at a time (the workspace holds one [n_pad, vocab_chunk] bf16 panel plus an fp32 d_hidden
  * accumulator); pass the same value to the workspace query.
  */
+#define VAMD_DW_STORE 0
+#define VAMD_DW_ADD_BF16 1
+#define VAMD_DW_F32_STORE 2
+#define VAMD_DW_F32_ADD 3
+#define VAMD_DW_F32_ADD_FINISH 4
 size_t vamd_lce_backward_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab, int64_t vocab_chunk);
 int vamd_lce_backward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
                       int64_t hidden_size, int64_t vocab, float rcp_temperature, const float* lse,
                       const float* mean_z, const float* d_logprobs, const float* d_entropy, float d_entropy_scalar,
-                      const float* logits_cache, void* d_hidden, void* d_weight, int accumulate_d_weight,
-                      int64_t vocab_chunk, void* workspace, size_t workspace_bytes, void* stream);
+                      const float* logits_cache, void* d_hidden, void* d_weight, int d_weight_mode,
+                      float* d_weight_acc32, int64_t vocab_chunk, void* workspace, size_t workspace_bytes,
+                      void* stream);
 
 /* Benchmark aid (no counterpart in the reference): with timing enabled, every head kernel
  * launch of the process is bracketed by HIP events on its stream.  vamd_lce_timing_collect
  * waits for them and adds up milliseconds and launch counts per kernel, indexed
- * 0 forward, 1 merge, 2 d_logits panel (recompute GEMM or cached-logits pass), 3 gradient GEMMs (d_hidden + d_weight) (arrays of 4). */
+ * 0 forward, 1 merge, 2 d_logits panel from recomputed logits (the recompute GEMM), 3 gradient GEMMs
+ * (d_hidden + d_weight), 4 d_logits panel from cached logits (arrays of VAMD_LCE_TIMING_KERNELS). */
+#define VAMD_LCE_TIMING_KERNELS 5
 int vamd_lce_timing_enable(int on);
 int vamd_lce_timing_collect(double* ms_by_kernel_host, int64_t* launches_by_kernel_host);
 

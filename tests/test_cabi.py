@@ -108,8 +108,16 @@ def test_registries_and_host_logic_without_gpu():
 def test_backward_rejects_operands_beyond_32_bit_offsets(lib):
     """The check runs before any GPU call: dummy non-null pointers are never dereferenced."""
     p = ctypes.c_void_p(256)
-    rc = lib.vamd_lce_backward(p, p, p, 700000, 3584, 1024, 1.0, p, p, None, None, 0.0, None, p, p, 0, 0, p, 1 << 40, None)
+    rc = lib.vamd_lce_backward(p, p, p, 700000, 3584, 1024, 1.0, p, p, None, None, 0.0, None, p, p, 0, None, 0, p, 1 << 40, None)
     assert rc == -1 and b"4 GiB" in lib.vamd_last_error()
+    # fp32 accumulation of the weight gradient needs its buffer; an unknown mode is refused
+    rc = lib.vamd_lce_backward(p, p, p, 256, 128, 1024, 1.0, p, p, None, None, 0.0, None, p, None, 3, None, 0, p, 1 << 40, None)
+    assert rc == -1 and b"d_weight_acc32" in lib.vamd_last_error()
+    rc = lib.vamd_lce_backward(p, p, p, 256, 128, 1024, 1.0, p, p, None, None, 0.0, None, p, p, 7, None, 0, p, 1 << 40, None)
+    assert rc == -1 and b"d_weight_mode" in lib.vamd_last_error()
+    # a vocabulary that is not a multiple of 8 is served, but not together with a logits cache
+    rc = lib.vamd_lce_forward(p, p, p, 256, 128, 1001, 1.0, p, p, p, p, p, None, p, 1 << 30, None)
+    assert rc == -1 and b"multiple of 8" in lib.vamd_last_error()
 
 
 def test_bench_refuses_more_than_one_gpu():

@@ -27,8 +27,8 @@ BF16_HALF_ULP = 2.0 ** -8
 
 @pytest.fixture(params=["recompute", "logits_cache"])
 def backward_mode(request, monkeypatch):
-    """Autograd tests run twice: with the fp32 logits cache (default) and with it switched off, which makes the
-    backward pass recompute the logits."""
+    """Autograd tests run twice: with the backward pass recomputing the logits (the default) and with the opt-in
+    fp32 logits cache."""
     monkeypatch.setenv("VAMD_LCE_LOGITS_CACHE_GB", "0" if request.param == "recompute" else "16")
     return request.param
 
@@ -191,10 +191,10 @@ def test_reductions_3d_input_and_argument_errors(dev):
         linear_cross_entropy(hd[..., :64], wd[:, :64], ld, 1.5, "none")      # non-contiguous / H % 128
 
 
-@pytest.mark.parametrize("case", [1, 2, 3])
+@pytest.mark.parametrize("case", [0, 1, 2, 3, 4])
 def test_reference_test_shapes_fwd_bwd(dev, backward_mode, case):
-    """Three of the five (N, H, V) cases of the reference's own test (the ragged-N ones that fit a quick run),
-    bf16 upstream grads as there; ground truth evaluated in fp32 on the GPU."""
+    """The five (N, H, V) cases of the reference's own test (tests/utils/test_linear_cross_entropy.py:112-143),
+    its input distributions and bf16 upstream grads; ground truth evaluated in fp32 on the GPU."""
     from conftest import load_golden
     fx = load_golden()["head_shapes"]
     n, h, v = (fx["cases"][case][k] for k in ("num_tokens", "hidden_size", "vocab"))
@@ -235,9 +235,23 @@ def test_benchmark_config_7b_head_full_size(dev):
     assert (ent - want_ent).abs().max().item() <= ATOL
     _close_bf16(dh, want_dh, "d_hidden", e_dh)
     _close_bf16(dw, want_dw, "d_weight", e_dw)
-    # typical (not worst-case) agreement: the rms error stays far below the bound
-    assert (dw.float() - want_dw).pow(2).mean().sqrt().item() < 1.5e-3
-    assert (dh.float() - want_dh).pow(2).mean().sqrt().item() < 1.5e-3
+    # measured errors against the strict 2e-3 (printed with -s; the gradients' share beyond 2e-3 is the bf16
+    # rounding of the outputs and of the staged d_logits, which the bound above spells out)
+    errs = {"logprob": (lp - want_lp).abs().max().item(), "entropy": (ent - want_ent).abs().max().item(),
+            "d_hidden": (dh.float() - want_dh).abs().max().item(), "d_weight": (dw.float() - want_dw).abs().max().item()}
+    rms = {"d_hidden": (dh.float() - want_dh).pow(2).mean().sqrt().item(),
+           "d_weight": (dw.float() - want_dw).pow(2).mean().sqrt().item()}
+    frac_over = {"d_hidden": ((dh.float() - want_dh).abs() > ATOL).float().mean().item(),
+                 "d_weight": ((dw.float() - want_dw).abs() > ATOL).float().mean().item()}
+    print(f"\nC2 recompute: max abs err {errs}; rms {rms}; share of elements beyond 2e-3 {frac_over}; "
+          f"max |d_hidden| {want_dh.abs().max().item():.3e}, max |d_weight| {want_dw.abs().max().item():.3e}")
+    # typical (not worst-case) agreement: the rms error stays below half a bf16 ulp (2**-8) of the rms gradient,
+    # i.e. on average the result is as close as its own output format allows
+    rel = {"d_hidden": rms["d_hidden"] / want_dh.pow(2).mean().sqrt().item(),
+           "d_weight": rms["d_weight"] / want_dw.pow(2).mean().sqrt().item()}
+    print(f"C2 recompute: rms error / rms gradient {rel}")
+    assert rel["d_hidden"] < BF16_HALF_ULP and rel["d_weight"] < BF16_HALF_ULP, rel
+    assert errs["logprob"] < 1e-4 and errs["entropy"] < 1e-4 and errs["d_hidden"] < ATOL, errs
     del want_dw, want_dh, e_dw, e_dh
     # sum_j dz_j = 0 for every token  =>  the vocabulary-axis sum of d_weight vanishes (bf16 rounding of 152064 rows)
     # (each of the ~16384 label rows carries its own bf16 rounding error, so the sum is noise of relative size ~1e-5)
@@ -256,6 +270,8 @@ def test_benchmark_config_7b_head_full_size(dev):
     dh_c, dw_c = K.efficient_entropy_backward(g_lp, None, hidden, weight, labels, lse_c, mz_c, 0, T,
                                               d_entropy_scalar=0.001, logits_cache=cache)
     del cache
+    print(f"C2 logits cache vs recompute: max abs diff d_hidden {(dh_c.float() - dh.float()).abs().max().item():.3e}, "
+          f"d_weight {(dw_c.float() - dw.float()).abs().max().item():.3e}")
     _close_bf16(dh_c, dh.float(), "d_hidden cached vs recomputed")
     _close_bf16(dw_c, dw.float(), "d_weight cached vs recomputed")
     assert (dh_c.float() - dh.float()).pow(2).mean().sqrt().item() < 1e-4
@@ -276,34 +292,119 @@ def test_benchmark_config_small_head_forward_only(dev):
 
 
 def test_benchmark_config_llama_head_token_chunked(dev):
-    """Llama-3.1-8B head shape (H=4096, V=128256, T=0.7) processed in 8192-token chunks with the weight gradient
-    accumulated across chunks and the entropy coefficient 0.001 passed as a scalar folded into the backward; two
-    chunks of the configuration's eight keep the test short.  One chunk goes through the logits cache, the other
-    through the recompute path."""
+    """Llama-3.1-8B head shape at long-rollout scale (N=65536, H=4096, V=128256, T=0.7) processed in eight
+    8192-token chunks, the entropy coefficient 0.001 passed as a scalar folded into the backward.  The weight
+    gradient is summed over the eight chunks in fp32 and rounded to bf16 once, so it is held to the same bound as
+    a single call.  Alternating chunks go through the logits cache and through the recompute path.  The same sum
+    kept in bf16 (one rounding of the running sum per chunk, what ``weight.grad +=`` does in bf16 training) is run
+    beside it and must stay within one extra half-ulp of the running value per accumulation."""
     from verl_amd.utils.kernel import linear_cross_entropy as K
-    n, h, v, T, chunk = 16384, 4096, 128256, 0.7, 8192
+    n, h, v, T, chunk = 65536, 4096, 128256, 0.7, 8192
     g = torch.Generator(device=dev).manual_seed(5)
     hidden = torch.randn(n, h, device=dev, generator=g).bfloat16()
     weight = (torch.randn(v, h, device=dev, generator=g) * 0.02).bfloat16()
     labels = torch.randint(0, v, (n,), device=dev, generator=g)
     g_lp = torch.randn(n, device=dev, generator=g)
-    d_weight = torch.zeros_like(weight)
+    acc32 = torch.empty(v, h, device=dev, dtype=torch.float32)
+    d_weight_bf16_sum = torch.zeros_like(weight)
     lps, ents, dhs = [], [], []
+    d_weight = None
+    n_chunks = n // chunk
     for ci, lo in enumerate(range(0, n, chunk)):
         sl = slice(lo, lo + chunk)
-        cache = torch.empty(chunk, v, device=dev) if ci == 0 else None
+        cache = torch.empty(chunk, v, device=dev) if ci % 2 == 0 else None
         lp, ent, lse, mz = K.efficient_entropy_forward(hidden[sl], weight, labels[sl], 0, T, logits_cache=cache)
-        dh, _ = K.efficient_entropy_backward(g_lp[sl], None, hidden[sl], weight, labels[sl], lse, mz, 0, T,
-                                             d_entropy_scalar=0.001, d_weight_out=d_weight, logits_cache=cache)
+        step = "first" if ci == 0 else ("last" if ci == n_chunks - 1 else "middle")
+        dh, dw = K.efficient_entropy_backward(g_lp[sl], None, hidden[sl], weight, labels[sl], lse, mz, 0, T,
+                                              d_entropy_scalar=0.001, logits_cache=cache,
+                                              d_weight_acc32=acc32, acc32_step=step)
+        assert (dw is None) == (step != "last")
+        d_weight = dw
+        dh2, _ = K.efficient_entropy_backward(g_lp[sl], None, hidden[sl], weight, labels[sl], lse, mz, 0, T,
+                                              d_entropy_scalar=0.001, logits_cache=cache,
+                                              d_weight_out=d_weight_bf16_sum)
+        assert torch.equal(dh, dh2)
         lps.append(lp); ents.append(ent); dhs.append(dh)
         del cache
+    del acc32
     want_lp, want_ent, want_dh, want_dw, e_dh, e_dw = _oracle_with_scale(
         hidden, weight, labels, T, g_lp, torch.full((n,), 0.001, device=dev), dev)
     assert (torch.cat(lps) - want_lp).abs().max().item() <= ATOL
     assert (torch.cat(ents) - want_ent).abs().max().item() <= ATOL
     _close_bf16(torch.cat(dhs), want_dh, "d_hidden", e_dh)
-    # d_weight passes through bf16 once per token chunk: one more half-ulp of the running value per accumulation
-    _close_bf16(d_weight, want_dw, "d_weight accumulated over token chunks", e_dw + want_dw.abs())
+    _close_bf16(d_weight, want_dw, "d_weight summed over 8 token chunks in fp32", e_dw)
+    # the bf16 running sum: each of the 7 additions rounds a value no larger than the final one in magnitude plus
+    # what is still to come; bound it by half an ulp of (|want| + E) per accumulation
+    _close_bf16(d_weight_bf16_sum, want_dw, "d_weight summed over 8 token chunks in bf16",
+                e_dw + (n_chunks - 1) * (want_dw.abs() + e_dw))
+    err32 = (d_weight.float() - want_dw).abs().max().item()
+    err16 = (d_weight_bf16_sum.float() - want_dw).abs().max().item()
+    print(f"\nC5 d_weight max abs err: fp32 accumulation {err32:.3e}, bf16 accumulation {err16:.3e}; "
+          f"max |d_weight| {want_dw.abs().max().item():.3e}")
+
+
+def test_weight_gradient_fp32_accumulation_small(dev):
+    """Three token chunks summed in fp32 equal one call over all tokens up to the final bf16 rounding."""
+    from verl_amd.utils.kernel import linear_cross_entropy as K
+    n, h, v, T = 900, 256, 3000, 1.3
+    hidden, weight, labels = _make(n, h, v, seed=17, dist="normal")
+    hd, wd, ld = hidden.to(dev), weight.to(dev), labels.to(dev)
+    g_lp = torch.randn(n, generator=torch.Generator().manual_seed(2)).to(dev)
+    g_ent = torch.full((n,), 0.01, device=dev)
+    acc32 = torch.full((v, h), float("nan"), device=dev)        # "first" must overwrite, not add
+    out = torch.empty_like(wd)
+    for step, sl in (("first", slice(0, 300)), ("middle", slice(300, 650)), ("last", slice(650, 900))):
+        _, _, lse, mz = K.efficient_entropy_forward(hd[sl], wd, ld[sl], 0, T)
+        _, dw = K.efficient_entropy_backward(g_lp[sl], g_ent[sl], hd[sl], wd, ld[sl], lse, mz, 0, T,
+                                             d_weight_acc32=acc32, acc32_step=step, d_weight_out=out, vocab_chunk=1024)
+    assert dw is out
+    _, _, want_dh, want_dw, e_dh, e_dw = _oracle_with_scale(hidden, weight, labels, T, g_lp.cpu(), g_ent.cpu(), "cpu")
+    _close_bf16(out, want_dw, "d_weight (fp32 accumulation, 3 chunks)", e_dw)
+    assert torch.equal(out, acc32.bfloat16())
+
+
+@pytest.mark.parametrize("n,h,v", [(130, 128, 1001), (257, 256, 257), (64, 128, 7), (300, 128, 4099)])
+def test_vocabulary_not_a_multiple_of_eight(dev, n, h, v):
+    """The vocabulary tail is masked, as in the reference (kernels.py masks ragged V); forward and backward."""
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    hidden, weight, labels = _make(n, h, v, seed=n + v)
+    g = torch.Generator().manual_seed(v)
+    g_lp, g_ent = torch.randn(n, generator=g), torch.randn(n, generator=g) * 0.1
+    hd = hidden.to(dev).requires_grad_(); wd = weight.to(dev).requires_grad_()
+    lp, ent = linear_cross_entropy(hd, wd, labels.to(dev), 1.2)
+    dh, dw = torch.autograd.grad((lp, ent), (hd, wd), (g_lp.to(dev), g_ent.to(dev)))
+    want_lp, want_ent, want_dh, want_dw, e_dh, e_dw = _oracle_with_scale(hidden, weight, labels, 1.2, g_lp, g_ent, "cpu")
+    assert (lp.cpu() - want_lp).abs().max().item() <= ATOL and (ent.cpu() - want_ent).abs().max().item() <= ATOL
+    _close_bf16(dh, want_dh, "d_hidden", e_dh)
+    _close_bf16(dw, want_dw, "d_weight", e_dw)
+
+
+def test_forward_without_grad_keeps_no_logits(dev, monkeypatch):
+    """Under torch.no_grad() (the actor's compute_log_prob) no [tokens, vocab] tensor is allocated even when the
+    weight requires grad and the logits cache is switched on."""
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    monkeypatch.setenv("VAMD_LCE_LOGITS_CACHE_GB", "16")
+    n, h, v = 4096, 256, 32768
+    hidden, weight, labels = _make(n, h, v, seed=1)
+    hd, wd, ld = hidden.to(dev), weight.to(dev).requires_grad_(), labels.to(dev)
+    torch.cuda.synchronize(); torch.cuda.reset_peak_memory_stats(dev)
+    base = torch.cuda.memory_allocated(dev)
+    with torch.no_grad():
+        lp, ent = linear_cross_entropy(hd, wd, ld, 1.0)
+    torch.cuda.synchronize()
+    assert torch.cuda.max_memory_allocated(dev) - base < 4 * n * v // 8
+    assert not lp.requires_grad
+    # with grad mode on and the cache switched on, the same call does keep the logits
+    torch.cuda.reset_peak_memory_stats(dev)
+    lp2, _ = linear_cross_entropy(hd, wd, ld, 1.0)
+    assert torch.cuda.max_memory_allocated(dev) - base >= 4 * n * v and torch.equal(lp2.detach(), lp)
+    # and by default (cache off) it does not
+    monkeypatch.setenv("VAMD_LCE_LOGITS_CACHE_GB", "0")
+    del lp2
+    torch.cuda.synchronize(); torch.cuda.reset_peak_memory_stats(dev)
+    base = torch.cuda.memory_allocated(dev)
+    lp3, _ = linear_cross_entropy(hd, wd, ld, 1.0)
+    assert torch.cuda.max_memory_allocated(dev) - base < 4 * n * v // 8 and lp3.requires_grad
 
 
 @pytest.mark.parametrize("n,h,v,T", [(1, 128, 128, 1.0), (300, 384, 1000, 0.7), (700, 256, 8192, 1.5), (2169, 896, 151936, 1.0)])

@@ -17,6 +17,9 @@ _lock = threading.Lock()
 _lib = None
 
 MASK_F32, MASK_I64, MASK_U8, MASK_I32 = 0, 1, 2, 3
+# d_weight_mode of vamd_lce_backward (VAMD_DW_*)
+DW_STORE, DW_ADD_BF16, DW_F32_STORE, DW_F32_ADD, DW_F32_ADD_FINISH = 0, 1, 2, 3, 4
+LCE_TIMING_KERNELS = 5
 AGG_MODES = {
     "token-mean": 0,
     "seq-mean-token-sum": 1,
@@ -37,8 +40,8 @@ SIGNATURES = {
                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "vamd_lce_backward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
     "vamd_lce_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p,
-                                  c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_int64,
-                                  c_void_p, c_size_t, c_void_p]),
+                                  c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                  c_int64, c_void_p, c_size_t, c_void_p]),
     "vamd_lce_timing_enable": (c_int, [c_int]),
     "vamd_lce_timing_collect": (c_int, [c_void_p, c_void_p]),
     "vamd_masked_moments_workspace_bytes": (c_size_t, [c_int64, c_int64]),
@@ -119,7 +122,7 @@ def lib_path() -> str:
     return _LIB_PATH
 
 
-ABI_VERSION = 3  # VAMD_ABI_VERSION of include/verl_amd.h
+ABI_VERSION = 4  # VAMD_ABI_VERSION of include/verl_amd.h
 
 
 def load_library(path: str | None = None) -> ctypes.CDLL:

@@ -32,7 +32,7 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // Optional per-kernel timing for benchmarks: when enabled, every head kernel launch (from any
 // thread: autograd runs backward on its own) is bracketed by a pair of HIP events on the launch
 // stream.
-enum : int { kTagForward = 0, kTagMerge = 1, kTagRecompute = 2, kTagDGrad = 3, kNumTags = 4 };
+enum : int { kTagForward = 0, kTagMerge = 1, kTagRecompute = 2, kTagDGrad = 3, kTagDLogits = 4, kNumTags = 5 };
 struct TimedLaunch {
   int tag;
   hipEvent_t start, stop;
@@ -496,8 +496,8 @@ struct GemmOutArgs {
   Operand R, C;
   int k_slabs, r_tiles, c_tiles;
   int r_valid, c_valid;  // rows / cols of the output that exist
-  int mode;              // d_hidden: one of the enum above; d_weight: 0 = overwrite, 1 = accumulate
-  float* acc32;          // fp32 accumulator [r_valid][ld_out] (d_hidden only)
+  int mode;              // d_hidden: one of the enum above; d_weight: a VAMD_DW_* value
+  float* acc32;          // fp32 accumulator [r_valid][ld_out]
   uint16_t* out;         // bf16 output
   int64_t ld_out;
 };
@@ -561,13 +561,19 @@ struct DWeightEpi {
           const int row = row0 + 8 * i;
           if (row >= A.r_valid) continue;
           f32x4 x = v[i];
-          u32x2* dst = reinterpret_cast<u32x2*>(A.out + (int64_t)row * A.ld_out + col);
-          if (A.mode == 1) {
+          const int64_t off = (int64_t)row * A.ld_out + col;
+          u32x2* dst = reinterpret_cast<u32x2*>(A.out + off);
+          if (A.mode == VAMD_DW_ADD_BF16) {
             const u32x2 o = *dst;
             x[0] += bf16_bits_to_float(o[0] & 0xffffu);
             x[1] += bf16_bits_to_float(o[0] >> 16);
             x[2] += bf16_bits_to_float(o[1] & 0xffffu);
             x[3] += bf16_bits_to_float(o[1] >> 16);
+          } else if (A.mode >= VAMD_DW_F32_STORE) {
+            f32x4* acc = reinterpret_cast<f32x4*>(A.acc32 + off);
+            if (A.mode != VAMD_DW_F32_STORE) x = x + *acc;
+            *acc = x;
+            if (A.mode != VAMD_DW_F32_ADD_FINISH) continue;
           }
           *dst = pack_bf16x4(x[0], x[1], x[2], x[3]);
         }
@@ -659,16 +665,20 @@ static int fwd_splits(int64_t tok_tiles, int64_t voc_tiles) {
   return (int)sp;
 }
 
-static int check_head_shapes(int64_t n, int64_t h, int64_t v) {
+// Any vocabulary size is served; only the fp32 logits cache, whose rows are read and written 32 bytes at a time,
+// needs a multiple of 8.
+static int check_head_shapes(int64_t n, int64_t h, int64_t v, const void* logits_cache) {
   VAMD_REQUIRE(n > 0 && h > 0 && v > 0, "lce: empty problem n=%lld h=%lld v=%lld", (long long)n, (long long)h,
                (long long)v);
   VAMD_REQUIRE(h % 128 == 0, "lce: hidden_size %lld must be a multiple of 128", (long long)h);
-  VAMD_REQUIRE(v % 8 == 0 && v >= 8, "lce: vocab %lld must be a multiple of 8", (long long)v);
+  VAMD_REQUIRE(!logits_cache || v % 8 == 0, "lce: a logits cache needs a vocab that is a multiple of 8, got %lld",
+               (long long)v);
   VAMD_REQUIRE(n < (1ll << 30) && v < (1ll << 30), "lce: n_tokens / vocab too large");
+  VAMD_REQUIRE(reinterpret_cast<uintptr_t>(logits_cache) % 16 == 0, "lce: logits_cache must be 16-byte aligned");
   return VAMD_OK;
 }
 
-static int64_t default_vocab_chunk(int64_t n_tokens, int64_t vocab, int64_t requested) {
+static int64_t default_vocab_chunk(int64_t n_tokens, int64_t hidden_size, int64_t vocab, int64_t requested) {
   const int64_t n_pad = ceil_div(n_tokens, kTile) * kTile;
   const int64_t v_pad = ceil_div(vocab, kTile) * kTile;
   int64_t cv = requested;
@@ -681,6 +691,9 @@ static int64_t default_vocab_chunk(int64_t n_tokens, int64_t vocab, int64_t requ
     cv = budget / (n_pad * 2) / kTile * kTile;
   }
   cv = ceil_div(cv, kTile) * kTile;
+  // the weight rows of a chunk are walked with 32-bit byte offsets from the chunk's first row
+  const int64_t cap = ((1ll << 32) - 1) / (hidden_size * 2) / kTile * kTile;
+  if (cv > cap) cv = cap;
   if (cv < kTile) cv = kTile;
   if (cv > v_pad) cv = v_pad;
   return cv;
@@ -753,7 +766,6 @@ static int lce_forward_launch(const void* hidden, const void* weight, const int6
                                                   align_up((size_t)a.splits * a.tok_tiles * kTile * sizeof(float4), 256))
                        : nullptr;
   a.z_cache = logits_cache;
-  VAMD_REQUIRE(reinterpret_cast<uintptr_t>(logits_cache) % 16 == 0, "lce_forward: logits_cache must be 16-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
   {
     ScopedTiming tm(kTagForward, s);
@@ -791,8 +803,8 @@ static int lce_forward_launch(const void* hidden, const void* weight, const int6
 
 static int check_forward_args(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
                               int64_t hidden_size, int64_t vocab, float rcp_temperature, const float* logprobs,
-                              const float* entropy, const float* lse, const float* mean_z) {
-  int st = check_head_shapes(n_tokens, hidden_size, vocab);
+                              const float* entropy, const float* lse, const float* mean_z, const float* logits_cache) {
+  int st = check_head_shapes(n_tokens, hidden_size, vocab, logits_cache);
   if (st != VAMD_OK) return st;
   VAMD_REQUIRE(hidden && weight && labels && logprobs && entropy && lse && mean_z, "lce_forward: null pointer");
   VAMD_REQUIRE(rcp_temperature > 0.f, "lce_forward: temperature must be positive");
@@ -804,7 +816,7 @@ extern "C" int vamd_lce_forward(const void* hidden, const void* weight, const in
                                 float* entropy, float* lse, float* mean_z, float* logits_cache,
                                 float* sum_pi_squared, void* workspace, size_t workspace_bytes, void* stream) {
   int st = check_forward_args(hidden, weight, labels, n_tokens, hidden_size, vocab, rcp_temperature, logprobs, entropy,
-                              lse, mean_z);
+                              lse, mean_z, logits_cache);
   if (st != VAMD_OK) return st;
   const size_t need = vamd_lce_forward_workspace_bytes(n_tokens, hidden_size, vocab);
   if (!workspace || workspace_bytes < need) {
@@ -849,7 +861,7 @@ extern "C" int vamd_lce_forward_static(const void* hidden, const void* weight, c
                                        float* logprobs, float* entropy, float* lse, float* mean_z,
                                        float* sum_pi_squared, void* stream) {
   int st = check_forward_args(hidden, weight, labels, n_tokens, hidden_size, vocab, rcp_temperature, logprobs, entropy,
-                              lse, mean_z);
+                              lse, mean_z, nullptr);
   if (st != VAMD_OK) return st;
   const size_t need = vamd_lce_forward_workspace_bytes(n_tokens, hidden_size, vocab);
   VAMD_REQUIRE(n_tokens <= VAMD_LCE_STATIC_MAX_TOKENS && need <= kStaticScratchBytes,
@@ -869,7 +881,7 @@ extern "C" size_t vamd_lce_backward_workspace_bytes(int64_t n_tokens, int64_t hi
                                                     int64_t vocab_chunk) {
   if (n_tokens <= 0 || vocab <= 0 || hidden_size <= 0) return 0;
   const int64_t n_pad = ceil_div(n_tokens, kTile) * kTile;
-  const int64_t cv = default_vocab_chunk(n_tokens, vocab, vocab_chunk);
+  const int64_t cv = default_vocab_chunk(n_tokens, hidden_size, vocab, vocab_chunk);
   size_t bytes = align_up((size_t)n_pad * dz_pitch(cv) * 2, 256);
   if (cv < ceil_div(vocab, kTile) * kTile) bytes += align_up((size_t)n_tokens * hidden_size * 4, 256);
   return bytes;
@@ -879,16 +891,24 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
                                  int64_t hidden_size, int64_t vocab, float rcp_temperature, const float* lse,
                                  const float* mean_z, const float* d_logprobs, const float* d_entropy,
                                  float d_entropy_scalar, const float* logits_cache, void* d_hidden, void* d_weight,
-                                 int accumulate_d_weight, int64_t vocab_chunk, void* workspace,
+                                 int d_weight_mode, float* d_weight_acc32, int64_t vocab_chunk, void* workspace,
                                  size_t workspace_bytes, void* stream) {
-  int st = check_head_shapes(n_tokens, hidden_size, vocab);
+  int st = check_head_shapes(n_tokens, hidden_size, vocab, logits_cache);
   if (st != VAMD_OK) return st;
-  VAMD_REQUIRE(hidden && weight && labels && lse && mean_z && d_hidden && d_weight, "lce_backward: null pointer");
+  VAMD_REQUIRE(hidden && weight && labels && lse && mean_z && d_hidden, "lce_backward: null pointer");
   VAMD_REQUIRE(rcp_temperature > 0.f, "lce_backward: temperature must be positive");
-  VAMD_REQUIRE(reinterpret_cast<uintptr_t>(logits_cache) % 16 == 0, "lce_backward: logits_cache must be 16-byte aligned");
+  VAMD_REQUIRE(d_weight_mode >= VAMD_DW_STORE && d_weight_mode <= VAMD_DW_F32_ADD_FINISH,
+               "lce_backward: unknown d_weight_mode %d", d_weight_mode);
+  {
+    const bool writes_bf16 = d_weight_mode <= VAMD_DW_ADD_BF16 || d_weight_mode == VAMD_DW_F32_ADD_FINISH;
+    const bool uses_f32 = d_weight_mode >= VAMD_DW_F32_STORE;
+    VAMD_REQUIRE(!writes_bf16 || d_weight, "lce_backward: d_weight_mode %d writes d_weight, which is null", d_weight_mode);
+    VAMD_REQUIRE(!uses_f32 || (d_weight_acc32 && reinterpret_cast<uintptr_t>(d_weight_acc32) % 16 == 0),
+                 "lce_backward: d_weight_mode %d needs a 16-byte aligned d_weight_acc32", d_weight_mode);
+  }
   {  // K-major operands are addressed with 32-bit byte offsets from their tile origin
     const int64_t rows_padded = ceil_div(n_tokens, kTile) * kTile;
-    const int64_t row_pitch = dz_pitch(default_vocab_chunk(n_tokens, vocab, vocab_chunk));
+    const int64_t row_pitch = dz_pitch(default_vocab_chunk(n_tokens, hidden_size, vocab, vocab_chunk));
     VAMD_REQUIRE(n_tokens * hidden_size * 2 < (1ll << 32) && rows_padded * row_pitch * 2 < (1ll << 32),
                  "lce_backward: hidden states (%lld x %lld) or the d_logits panel exceed 4 GiB; split the tokens into "
                  "chunks and accumulate d_weight", (long long)n_tokens, (long long)hidden_size);
@@ -904,7 +924,7 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
 
   const int tok_tiles = (int)ceil_div(n_tokens, kTile);
   const int64_t n_pad = (int64_t)tok_tiles * kTile;
-  const int64_t cv = default_vocab_chunk(n_tokens, vocab, vocab_chunk);
+  const int64_t cv = default_vocab_chunk(n_tokens, hidden_size, vocab, vocab_chunk);
   const int n_chunks = (int)ceil_div(vocab, cv);
   Carver carve(workspace);
   const int64_t pitch = dz_pitch(cv);
@@ -937,7 +957,7 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
       d.dz = dz;
       d.dz_ld = (int)pitch;
       {
-        ScopedTiming tm(kTagRecompute, s);
+        ScopedTiming tm(kTagDLogits, s);
         hipLaunchKernelGGL(lce_dlogits_kernel, dim3((unsigned)n_pad, (unsigned)ceil_div(d.chunk_cols, 2048)), dim3(256),
                            0, s, d);
       }
@@ -998,9 +1018,9 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
     gw.c_tiles = h_tiles;
     gw.r_valid = (int)cols;
     gw.c_valid = (int)hidden_size;
-    gw.mode = accumulate_d_weight ? 1 : 0;
-    gw.acc32 = nullptr;
-    gw.out = static_cast<uint16_t*>(d_weight) + c0 * hidden_size;
+    gw.mode = d_weight_mode;
+    gw.acc32 = d_weight_acc32 ? d_weight_acc32 + c0 * hidden_size : nullptr;
+    gw.out = d_weight ? static_cast<uint16_t*>(d_weight) + c0 * hidden_size : nullptr;
     gw.ld_out = hidden_size;
     {
       const int tiles = gh.r_tiles * gh.c_tiles + gw.r_tiles * gw.c_tiles;

@@ -4,11 +4,12 @@ Drop-in for ``verl.utils.kernel.linear_cross_entropy`` (reference
 verl/utils/kernel/linear_cross_entropy.py:38-119): same class name, ``forward`` / ``backward``
 signatures, argument checks and return tuple.  The arithmetic runs in ``libverl_amd.so``
 (``vamd_lce_forward`` / ``vamd_lce_backward``): bf16 MFMA logits tiles with an in-register online
-softmax.  The ``[tokens, vocab]`` logits are never needed; when a backward pass will follow and
-``4 * tokens * vocab`` bytes fit the budget below, the forward pass keeps them in fp32 so that the
-backward pass skips its logits-recompute GEMM (a quarter of the step's matrix work) -- HBM is the
-cheap resource on a 288 GB part.  ``VAMD_LCE_LOGITS_CACHE_GB`` sets the budget (default 16,
-0 turns the cache off); results are the same either way.
+softmax.  The ``[tokens, vocab]`` logits are never materialised: the backward pass recomputes them
+tile by tile, as the reference does.  Opt-in trade for a 288 GB part: with
+``VAMD_LCE_LOGITS_CACHE_GB=<budget>`` in the environment (default 0 = off), a forward pass that a
+backward pass will follow keeps the logits in fp32 when ``4 * tokens * vocab`` bytes fit the budget,
+and the backward pass then skips its logits-recompute GEMM (a quarter of the step's matrix work).
+Results are the same either way up to one fp32 rounding of the logits.
 """
 from __future__ import annotations
 
@@ -41,12 +42,12 @@ def _check_inputs(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tens
     assert hidden.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16, (
         f"the MI355X head computes on bf16 inputs, got {hidden.dtype} / {weight.dtype}"
     )
-    assert weight.shape[0] % 8 == 0, "vocab size must be a multiple of 8"
 
 
 def logits_cache_budget_bytes() -> int:
-    """Largest fp32 logits cache the autograd path may allocate (``VAMD_LCE_LOGITS_CACHE_GB``, default 16)."""
-    return int(float(os.environ.get("VAMD_LCE_LOGITS_CACHE_GB", "16")) * (1 << 30))
+    """Largest fp32 logits cache the autograd path may allocate: ``VAMD_LCE_LOGITS_CACHE_GB`` GiB, default 0
+    (no cache: the backward pass recomputes the logits)."""
+    return int(float(os.environ.get("VAMD_LCE_LOGITS_CACHE_GB", "0")) * (1 << 30))
 
 
 def efficient_entropy_forward(hidden, weight, labels, reduction: int = 0, temperature: float = 1.0,
@@ -102,14 +103,20 @@ def _sum_f32(x: torch.Tensor) -> torch.Tensor:
 def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse, mean_z, reduction: int = 0,
                                temperature: float = 1.0, dist_process_group=None, d_entropy_scalar: float = 0.0,
                                d_weight_out: torch.Tensor | None = None, vocab_chunk: int = 0,
-                               logits_cache: torch.Tensor | None = None):
+                               logits_cache: torch.Tensor | None = None,
+                               d_weight_acc32: torch.Tensor | None = None, acc32_step: str | None = None):
     """Host side of the backward kernels (reference kernels.py:1512-1723).
 
     ``dlogprobs`` / ``dentropy`` may be ``None`` (no contribution).  ``d_entropy_scalar`` adds a
-    constant upstream entropy gradient for every token without materialising it.  When
-    ``d_weight_out`` is given the weight gradient is ACCUMULATED into it (token-chunked use).
+    constant upstream entropy gradient for every token without materialising it.
     ``logits_cache``: the tensor the forward call filled, if any (skips the recompute GEMM).
-    Returns ``(d_hidden, d_weight)`` in ``hidden.dtype``.
+    Token-chunked callers sum the weight gradient of several calls, in one of two ways:
+    ``d_weight_out`` (bf16) alone is ADDED to in bf16, one rounding of the running sum per call, like
+    ``weight.grad +=`` in bf16 training; with ``d_weight_acc32`` (fp32 ``[vocab, hidden]``) the sum is kept
+    in fp32 and ``acc32_step`` says which call this is: ``"first"`` (store), ``"middle"`` (add) or ``"last"``
+    (add, then write the sum, rounded once, to ``d_weight_out`` or a fresh tensor).
+    Returns ``(d_hidden, d_weight)`` in ``hidden.dtype``; ``d_weight`` is ``None`` for the "first" and
+    "middle" steps of an fp32 accumulation.
     """
     if dist_process_group is not None:
         raise NotImplementedError("vocab-parallel process groups are not supported on this single-GPU path")
@@ -139,16 +146,25 @@ def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse,
         labels = labels.to(torch.int64)
     L = _cabi.lib()
     d_hidden = torch.empty_like(hidden)
-    accumulate = d_weight_out is not None
-    d_weight = d_weight_out if accumulate else torch.empty_like(weight)
-    assert d_weight.shape == weight.shape and d_weight.dtype == weight.dtype and d_weight.is_contiguous()
+    if d_weight_acc32 is not None:
+        assert acc32_step in ("first", "middle", "last"), "acc32_step must be 'first', 'middle' or 'last'"
+        assert d_weight_acc32.shape == weight.shape and d_weight_acc32.dtype == torch.float32
+        assert d_weight_acc32.is_contiguous() and d_weight_acc32.device == dev
+        mode = {"first": _cabi.DW_F32_STORE, "middle": _cabi.DW_F32_ADD, "last": _cabi.DW_F32_ADD_FINISH}[acc32_step]
+        d_weight = (d_weight_out if d_weight_out is not None else torch.empty_like(weight)) if acc32_step == "last" else None
+    else:
+        assert acc32_step is None, "acc32_step needs d_weight_acc32"
+        mode = _cabi.DW_ADD_BF16 if d_weight_out is not None else _cabi.DW_STORE
+        d_weight = d_weight_out if d_weight_out is not None else torch.empty_like(weight)
+    if d_weight is not None:
+        assert d_weight.shape == weight.shape and d_weight.dtype == weight.dtype and d_weight.is_contiguous()
     ws = _cabi.workspace(L.vamd_lce_backward_workspace_bytes(n, h, v, vocab_chunk), dev)
     with torch.cuda.device(dev):
         _cabi.check(L.vamd_lce_backward(hidden.data_ptr(), weight.data_ptr(), labels.data_ptr(), n, h, v,
                                         1.0 / temperature, lse.data_ptr(), mean_z.data_ptr(), _cabi.ptr(dlogprobs),
                                         _cabi.ptr(dentropy), float(d_entropy_scalar), _cabi.ptr(logits_cache),
-                                        d_hidden.data_ptr(), d_weight.data_ptr(), int(accumulate), int(vocab_chunk),
-                                        ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
+                                        d_hidden.data_ptr(), _cabi.ptr(d_weight), mode, _cabi.ptr(d_weight_acc32),
+                                        int(vocab_chunk), ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
     return d_hidden, d_weight
 
 
@@ -188,7 +204,9 @@ class LinearCrossEntropy(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor,
                 temperature: typing.Optional[float] = 1.0, reduction: typing.Optional[str] = "none",
-                dist_process_group: typing.Optional[dist.ProcessGroup] = None):
+                dist_process_group: typing.Optional[dist.ProcessGroup] = None, grad_mode: bool = True):
+        # grad_mode: whether autograd was recording when the caller invoked the op.  Inside forward() grad mode is
+        # always off and ctx.needs_input_grad only mirrors requires_grad, so the wrapper below passes it in.
         assert isinstance(temperature, float), f"temperature must be a float, but got {type(temperature)}"
         assert isinstance(reduction, str), f"reduction must be a str, but got {type(reduction)}"
         REDUCTION = get_entropy_reduction_enum_number(reduction.lower())
@@ -199,7 +217,8 @@ class LinearCrossEntropy(torch.autograd.Function):
             labels = labels.view(-1)
         cache = None
         n_tokens, vocab = hidden.shape[0], weight.shape[0]
-        if (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]) and 4 * n_tokens * vocab <= logits_cache_budget_bytes():
+        backward_follows = grad_mode and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
+        if backward_follows and vocab % 8 == 0 and 4 * n_tokens * vocab <= logits_cache_budget_bytes():
             cache = torch.empty((n_tokens, vocab), device=hidden.device, dtype=torch.float32)
         logprobs, entropy, lse, mean_z = efficient_entropy_forward(
             hidden, weight, labels, REDUCTION, temperature, dist_process_group, logits_cache=cache)
@@ -225,7 +244,14 @@ class LinearCrossEntropy(torch.autograd.Function):
             dlogprobs, dentropy, hidden, weight, labels, lse, mean_z, ctx.REDUCTION, ctx.temperature,
             ctx.dist_process_group, logits_cache=cache)
         d_hidden = d_hidden.view(ctx.original_hidden_shape)
-        return (d_hidden, d_weight, None, None, None, None)
+        return (d_hidden, d_weight, None, None, None, None, None)
 
 
-linear_cross_entropy = LinearCrossEntropy.apply
+def linear_cross_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor,
+                         temperature: typing.Optional[float] = 1.0, reduction: typing.Optional[str] = "none",
+                         dist_process_group: typing.Optional[dist.ProcessGroup] = None):
+    """``LinearCrossEntropy.apply`` with the reference's positional signature
+    (verl/utils/kernel/linear_cross_entropy.py:119).  A forward pass under ``torch.no_grad()`` (the actor's
+    ``compute_log_prob``) keeps nothing for a backward pass, whatever ``requires_grad`` says."""
+    return LinearCrossEntropy.apply(hidden, weight, labels, temperature, reduction, dist_process_group,
+                                    torch.is_grad_enabled())
