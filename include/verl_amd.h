@@ -181,6 +181,36 @@ int vamd_lce_timing_enable(int on);
 int vamd_lce_timing_collect(double* ms_by_kernel_host, int64_t* launches_by_kernel_host);
 
 /* ------------------------------------------------------------------------------------------
+ * Per-token log-prob / entropy from materialised logits: the unfused definitions the actor uses when the
+ * fused head is off.  logprobs_from_logits / _v2 / _naive (verl/utils/torch_functional.py:72-100, :148-200),
+ * entropy_from_logits / entropy_from_logits_with_chunking (:224-263).
+ *   logits [n_rows, vocab] with row pitch ld (elements), element type VAMD_DT_*; arithmetic in fp32;
+ *   labels [n_rows] int64 in [0, vocab) (may be NULL when logprobs is NULL).
+ *   logprobs = z[label] - lse(z); entropy = lse(z) - sum softmax(z) z; lse and mean_z (= sum softmax(z) z) are
+ *   what the backward pass needs.  Every output is fp32 [n_rows] and may be NULL if not wanted.
+ * One pass over the logits (online softmax), no workspace. */
+#define VAMD_DT_F32 0
+#define VAMD_DT_BF16 1
+#define VAMD_DT_F16 2
+int vamd_row_softmax_stats(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t ld,
+                           const int64_t* labels, float* logprobs, float* entropy, float* lse, float* mean_z,
+                           void* stream);
+/* d_logits = d_logprobs (onehot(label) - p) - d_entropy p (z - mean_z), p = exp(z - lse): what autograd hands back
+ * through log_softmax + gather (logprobs_from_logits_naive) and through logsumexp - sum softmax * z
+ * (entropy_from_logits).  d_logprobs / d_entropy: fp32 [n_rows], either may be NULL (no contribution);
+ * d_logits has the element type of logits and row pitch ld_out, and may be the logits buffer itself (in place, the
+ * reference's inplace_backward). */
+int vamd_row_softmax_backward(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t ld,
+                              const int64_t* labels, const float* lse, const float* mean_z, const float* d_logprobs,
+                              const float* d_entropy, void* d_logits, int64_t ld_out, void* stream);
+/* clip_by_value (verl/utils/torch_functional.py:203-221): out = max(min(x, hi), lo) over n fp32 elements, and its
+ * gradients with torch's rule for binary min / max (the selected operand takes the gradient, equal operands half
+ * each); d_x / d_lo / d_hi may be NULL. */
+int vamd_clip_by_value(const float* x, const float* lo, const float* hi, int64_t n, float* out, void* stream);
+int vamd_clip_by_value_backward(const float* x, const float* lo, const float* hi, const float* grad_out, int64_t n,
+                                float* d_x, float* d_lo, float* d_hi, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Masked reductions: verl/utils/torch_functional.py:266-339.
  * vamd_masked_moments writes out[0..3] (double): sum(m), sum(where(m,v,0)*m),
  * sum(where(m,v,0)^2*m), count(m != 0)  -- the sufficient statistics of masked_sum / masked_mean /

@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
 LIB_DIR = os.path.join(PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libverl_amd.so")
-SOURCES = ["runtime.hip", "lce.hip", "policy_math.hip", "gae.hip", "returns_scan.hip", "otb.hip", "metrics.hip", "rollout_corr.hip", "response_window.hip", "cov_select.hip"]
+SOURCES = ["runtime.hip", "lce.hip", "policy_math.hip", "gae.hip", "returns_scan.hip", "otb.hip", "metrics.hip", "rollout_corr.hip", "response_window.hip", "cov_select.hip", "row_softmax.hip"]
 HEADERS = ["common.h", "gemm_core.h", "rowchunk.h", os.path.join("..", "..", "include", "verl_amd.h")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

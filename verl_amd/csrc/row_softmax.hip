@@ -1,0 +1,323 @@
+// Per-token log-prob / entropy from MATERIALISED logits, and clip_by_value: the unfused definitions the actor
+// uses when the fused head is off (verl/utils/torch_functional.py:72-100 logprobs_from_logits, :148-200 _naive / _v2,
+// :224-263 entropy_from_logits / _with_chunking, :203-221 clip_by_value).
+//
+// Forward: one pass over a row of logits with an online softmax (running max, sum e, sum e*z per thread, merged over
+// the workgroup), one workgroup per row, 16-byte loads, four of them in flight per thread.  Algorithmic traffic: the
+// logits once.  Backward: elementwise over [rows, vocab], d_logits = g_lp (onehot - p) - g_ent p (z - mean_z) with
+// p = exp(z - lse): logits in, gradient out (in place if the caller passes the same buffer).
+#include "common.h"
+
+namespace vamd {
+namespace {
+
+constexpr int kRowThreads = 256;
+constexpr int kInFlight = 4;  // 16-byte loads a thread issues before it consumes them
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kNegBig = -1.0e30f;
+
+struct F32 { using type = float; static constexpr int kVec = 4; };
+struct BF16 { using type = uint16_t; static constexpr int kVec = 8; };
+struct F16 { using type = _Float16; static constexpr int kVec = 8; };
+
+__device__ __forceinline__ float to_float(float x, F32) { return x; }
+__device__ __forceinline__ float to_float(uint16_t x, BF16) { return __uint_as_float((unsigned)x << 16); }
+__device__ __forceinline__ float to_float(_Float16 x, F16) { return (float)x; }
+__device__ __forceinline__ float from_float(float x, F32) { return x; }
+__device__ __forceinline__ uint16_t from_float(float x, BF16) {
+  const __bf16 b = (__bf16)x;  // round to nearest even
+  return __builtin_bit_cast(uint16_t, b);
+}
+__device__ __forceinline__ _Float16 from_float(float x, F16) { return (_Float16)x; }
+
+template <class D>
+struct alignas(16) Pack {
+  typename D::type v[D::kVec];
+};
+
+// Load the D::kVec elements starting at column c of a row (those at or beyond `cols` read as `fill`).
+template <class D, bool VEC>
+__device__ __forceinline__ void load_group(const typename D::type* __restrict__ row, int64_t c, int64_t cols,
+                                           float fill, float (&x)[D::kVec]) {
+  if (VEC && c + D::kVec <= cols) {
+    const Pack<D> p = *reinterpret_cast<const Pack<D>*>(row + c);
+#pragma unroll
+    for (int e = 0; e < D::kVec; ++e) x[e] = to_float(p.v[e], D());
+  } else {
+#pragma unroll
+    for (int e = 0; e < D::kVec; ++e) x[e] = (c + e < cols) ? to_float(row[c + e], D()) : fill;
+  }
+}
+
+template <class D, bool VEC>
+__device__ __forceinline__ void store_group(typename D::type* __restrict__ row, int64_t c, int64_t cols,
+                                            const float (&x)[D::kVec]) {
+  if (VEC && c + D::kVec <= cols) {
+    Pack<D> p;
+#pragma unroll
+    for (int e = 0; e < D::kVec; ++e) p.v[e] = from_float(x[e], D());
+    *reinterpret_cast<Pack<D>*>(row + c) = p;
+  } else {
+#pragma unroll
+    for (int e = 0; e < D::kVec; ++e)
+      if (c + e < cols) row[c + e] = from_float(x[e], D());
+  }
+}
+
+__device__ __forceinline__ void merge(float& m, float& s, float& sz, float m2, float s2, float sz2) {
+  const float mm = fmaxf(m, m2);
+  const float a = __builtin_amdgcn_exp2f(m - mm), b = __builtin_amdgcn_exp2f(m2 - mm);
+  s = s * a + s2 * b;
+  sz = sz * a + sz2 * b;
+  m = mm;
+}
+
+struct StatsArgs {
+  const void* logits;
+  int64_t ld;
+  const int64_t* labels;
+  int64_t cols;
+  float* logprobs;
+  float* entropy;
+  float* lse;
+  float* mean_z;
+};
+
+template <class D, bool VEC>
+__global__ __launch_bounds__(kRowThreads) void row_softmax_stats_kernel(StatsArgs a) {
+  using T = typename D::type;
+  constexpr int G = D::kVec;
+  const int64_t r = blockIdx.x;
+  const T* __restrict__ row = static_cast<const T*>(a.logits) + r * a.ld;
+  // running state in the log2 domain: m = max of z log2(e), s = sum 2^(y - m), sz = sum 2^(y - m) z
+  float m = kNegBig, s = 0.f, sz = 0.f;
+  const int64_t stride = (int64_t)kRowThreads * G;
+  for (int64_t c0 = (int64_t)threadIdx.x * G; c0 < a.cols; c0 += stride * kInFlight) {
+    float x[kInFlight][G];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) {
+      const int64_t c = c0 + u * stride;
+      if (c < a.cols) load_group<D, VEC>(row, c, a.cols, kNegBig, x[u]);
+      else
+#pragma unroll
+        for (int e = 0; e < G; ++e) x[u][e] = kNegBig;
+    }
+    float gmax = kNegBig;
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u)
+#pragma unroll
+      for (int e = 0; e < G; ++e) gmax = fmaxf(gmax, x[u][e]);
+    gmax *= kLog2e;
+    if (gmax > m) {
+      const float resc = __builtin_amdgcn_exp2f(m - gmax);
+      s *= resc;
+      sz *= resc;
+      m = gmax;
+    }
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u)
+#pragma unroll
+      for (int e = 0; e < G; ++e) {
+        const float z = x[u][e];
+        const float ex = __builtin_amdgcn_exp2f(fmaf(z, kLog2e, -m));  // padding: 2^(-1e30 ...) = 0
+        s += ex;
+        sz = fmaf(ex, z, sz);  // padding: 0 * -1e30; a true -inf logit gives NaN, as softmax(z) * z does
+      }
+  }
+  // wavefront, then workgroup
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) {
+    const float m2 = __shfl_xor(m, off, 64), s2 = __shfl_xor(s, off, 64), sz2 = __shfl_xor(sz, off, 64);
+    merge(m, s, sz, m2, s2, sz2);
+  }
+  __shared__ float red[3][kRowThreads / 64];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  if (lane == 0) {
+    red[0][w] = m;
+    red[1][w] = s;
+    red[2][w] = sz;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int j = 1; j < kRowThreads / 64; ++j) merge(m, s, sz, red[0][j], red[1][j], red[2][j]);
+    const float lse = (m + log2f(s)) * kLn2;
+    const float mz = sz / s;
+    if (a.lse) a.lse[r] = lse;
+    if (a.mean_z) a.mean_z[r] = mz;
+    if (a.entropy) a.entropy[r] = lse - mz;
+    if (a.logprobs) a.logprobs[r] = to_float(row[a.labels[r]], D()) - lse;
+  }
+}
+
+struct BackwardArgs {
+  const void* logits;
+  int64_t ld;
+  const int64_t* labels;  // needed with d_logprobs
+  const float* lse;
+  const float* mean_z;    // needed with d_entropy
+  const float* d_logprobs;
+  const float* d_entropy;
+  void* d_logits;
+  int64_t ld_out;
+  int64_t cols;
+  int chunks;
+};
+
+// one workgroup per (row, chunk of kRowThreads * G * kInFlight columns)
+template <class D, bool VEC>
+__global__ __launch_bounds__(kRowThreads) void row_softmax_backward_kernel(BackwardArgs a) {
+  using T = typename D::type;
+  constexpr int G = D::kVec;
+  const int64_t r = blockIdx.x / a.chunks;
+  const int chunk = blockIdx.x % a.chunks;
+  const T* __restrict__ row = static_cast<const T*>(a.logits) + r * a.ld;
+  T* __restrict__ out = static_cast<T*>(a.d_logits) + r * a.ld_out;
+  const float lse2 = a.lse[r] * kLog2e;
+  const float glp = a.d_logprobs ? a.d_logprobs[r] : 0.f;
+  const float gent = a.d_entropy ? a.d_entropy[r] : 0.f;
+  const float mz = a.d_entropy ? a.mean_z[r] : 0.f;
+  const int64_t label = a.d_logprobs ? a.labels[r] : -1;
+  const int64_t stride = (int64_t)kRowThreads * G;
+  const int64_t c0 = (int64_t)chunk * stride * kInFlight + (int64_t)threadIdx.x * G;
+  float x[kInFlight][G];
+#pragma unroll
+  for (int u = 0; u < kInFlight; ++u) {
+    const int64_t c = c0 + u * stride;
+    if (c < a.cols) load_group<D, VEC>(row, c, a.cols, 0.f, x[u]);
+  }
+#pragma unroll
+  for (int u = 0; u < kInFlight; ++u) {
+    const int64_t c = c0 + u * stride;
+    if (c >= a.cols) continue;
+#pragma unroll
+    for (int e = 0; e < G; ++e) {
+      const float z = x[u][e];
+      const float p = __builtin_amdgcn_exp2f(fmaf(z, kLog2e, -lse2));
+      const float t = fmaf(gent, z - mz, glp);  // g_lp + g_ent (z - mean_z)
+      x[u][e] = -p * t + ((c + e == label) ? glp : 0.f);
+    }
+    store_group<D, VEC>(out, c, a.cols, x[u]);
+  }
+}
+
+// out = max(min(x, hi), lo)
+__global__ __launch_bounds__(256) void clip_kernel(const float* __restrict__ x, const float* __restrict__ lo,
+                                                   const float* __restrict__ hi, int64_t n, float* __restrict__ out) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    out[i] = fmaxf(fminf(x[i], hi[i]), lo[i]);
+}
+
+// Gradients of max(min(x, hi), lo) the way torch's binary min / max hand them out: the smaller (larger) operand
+// takes the gradient, equal operands take half each.
+__global__ __launch_bounds__(256) void clip_backward_kernel(const float* __restrict__ x, const float* __restrict__ lo,
+                                                            const float* __restrict__ hi, const float* __restrict__ g,
+                                                            int64_t n, float* __restrict__ dx, float* __restrict__ dlo,
+                                                            float* __restrict__ dhi) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const float xv = x[i], l = lo[i], h = hi[i], gv = g[i];
+    const float a = fminf(xv, h);
+    const float a_x = xv < h ? 1.f : (xv == h ? 0.5f : 0.f);  // d min(x, hi) / dx; the rest goes to hi
+    const float o_a = a > l ? 1.f : (a == l ? 0.5f : 0.f);    // d max(a, lo) / da; the rest goes to lo
+    if (dx) dx[i] = gv * o_a * a_x;
+    if (dhi) dhi[i] = gv * o_a * (1.f - a_x);
+    if (dlo) dlo[i] = gv * (1.f - o_a);
+  }
+}
+
+template <class D>
+bool rows_vectorizable(const void* base, int64_t ld) {
+  return reinterpret_cast<uintptr_t>(base) % 16 == 0 && (ld * (int64_t)sizeof(typename D::type)) % 16 == 0;
+}
+
+int check_rows(const char* what, const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t ld) {
+  VAMD_REQUIRE(logits != nullptr, "%s: null logits", what);
+  VAMD_REQUIRE(dtype >= VAMD_DT_F32 && dtype <= VAMD_DT_F16, "%s: unknown element type code %d", what, dtype);
+  VAMD_REQUIRE(n_rows > 0 && vocab > 0 && ld >= vocab, "%s: bad shape rows=%lld vocab=%lld ld=%lld", what,
+               (long long)n_rows, (long long)vocab, (long long)ld);
+  VAMD_REQUIRE(n_rows < (1ll << 31), "%s: too many rows", what);
+  return VAMD_OK;
+}
+
+}  // namespace
+}  // namespace vamd
+
+using namespace vamd;
+
+#define VAMD_DTYPE_DISPATCH(code, D, ...)                  \
+  switch (code) {                                          \
+    case VAMD_DT_F32: { using D = F32; __VA_ARGS__; } break;   \
+    case VAMD_DT_BF16: { using D = BF16; __VA_ARGS__; } break; \
+    default: { using D = F16; __VA_ARGS__; } break;            \
+  }
+
+extern "C" int vamd_row_softmax_stats(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t ld,
+                                      const int64_t* labels, float* logprobs, float* entropy, float* lse,
+                                      float* mean_z, void* stream) {
+  int st = check_rows("row_softmax_stats", logits, dtype, n_rows, vocab, ld);
+  if (st != VAMD_OK) return st;
+  VAMD_REQUIRE((logprobs == nullptr) || labels, "row_softmax_stats: logprobs need labels");
+  VAMD_REQUIRE(logprobs || entropy || lse || mean_z, "row_softmax_stats: no output requested");
+  StatsArgs a{logits, ld, labels, vocab, logprobs, entropy, lse, mean_z};
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  VAMD_DTYPE_DISPATCH(dtype, D, {
+    if (rows_vectorizable<D>(logits, ld))
+      hipLaunchKernelGGL((row_softmax_stats_kernel<D, true>), dim3((unsigned)n_rows), dim3(kRowThreads), 0, s, a);
+    else
+      hipLaunchKernelGGL((row_softmax_stats_kernel<D, false>), dim3((unsigned)n_rows), dim3(kRowThreads), 0, s, a);
+  });
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
+
+extern "C" int vamd_row_softmax_backward(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t ld,
+                                         const int64_t* labels, const float* lse, const float* mean_z,
+                                         const float* d_logprobs, const float* d_entropy, void* d_logits,
+                                         int64_t ld_out, void* stream) {
+  int st = check_rows("row_softmax_backward", logits, dtype, n_rows, vocab, ld);
+  if (st != VAMD_OK) return st;
+  VAMD_REQUIRE(d_logits && ld_out >= vocab && lse, "row_softmax_backward: bad output or missing lse");
+  VAMD_REQUIRE(d_logprobs || d_entropy, "row_softmax_backward: no upstream gradient");
+  VAMD_REQUIRE(!d_logprobs || labels, "row_softmax_backward: d_logprobs needs labels");
+  VAMD_REQUIRE(!d_entropy || mean_z, "row_softmax_backward: d_entropy needs mean_z");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  VAMD_DTYPE_DISPATCH(dtype, D, {
+    const int64_t per_wg = (int64_t)kRowThreads * D::kVec * kInFlight;
+    const int64_t chunks = (vocab + per_wg - 1) / per_wg;
+    VAMD_REQUIRE(n_rows * chunks < (1ll << 31), "row_softmax_backward: too many workgroups");
+    BackwardArgs a{logits, ld, labels, lse, mean_z, d_logprobs, d_entropy, d_logits, ld_out, vocab, (int)chunks};
+    const dim3 grid((unsigned)(n_rows * chunks));
+    if (rows_vectorizable<D>(logits, ld) && rows_vectorizable<D>(d_logits, ld_out))
+      hipLaunchKernelGGL((row_softmax_backward_kernel<D, true>), grid, dim3(kRowThreads), 0, s, a);
+    else
+      hipLaunchKernelGGL((row_softmax_backward_kernel<D, false>), grid, dim3(kRowThreads), 0, s, a);
+  });
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
+
+static unsigned flat_grid(int64_t n) {
+  int64_t blocks = (n + 255) / 256;
+  const int64_t cap = (int64_t)device_cu_count() * 16;
+  return (unsigned)(blocks < cap ? blocks : cap);
+}
+
+extern "C" int vamd_clip_by_value(const float* x, const float* lo, const float* hi, int64_t n, float* out,
+                                  void* stream) {
+  VAMD_REQUIRE(x && lo && hi && out && n > 0, "clip_by_value: bad argument");
+  hipLaunchKernelGGL(clip_kernel, dim3(flat_grid(n)), dim3(256), 0, static_cast<hipStream_t>(stream), x, lo, hi, n, out);
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
+
+extern "C" int vamd_clip_by_value_backward(const float* x, const float* lo, const float* hi, const float* grad_out,
+                                           int64_t n, float* d_x, float* d_lo, float* d_hi, void* stream) {
+  VAMD_REQUIRE(x && lo && hi && grad_out && n > 0 && (d_x || d_lo || d_hi), "clip_by_value_backward: bad argument");
+  hipLaunchKernelGGL(clip_backward_kernel, dim3(flat_grid(n)), dim3(256), 0, static_cast<hipStream_t>(stream), x, lo,
+                     hi, grad_out, n, d_x, d_lo, d_hi);
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}

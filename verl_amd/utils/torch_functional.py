@@ -1,14 +1,185 @@
-"""Masked reductions on MI355X: drop-ins for ``masked_sum`` / ``masked_mean`` / ``masked_var`` /
-``masked_whiten`` of the reference (verl/utils/torch_functional.py:266-339).
+"""Drop-ins for the tensor helpers of the reference's ``verl/utils/torch_functional.py`` on MI355X:
 
-Inputs may live on the CPU (they are staged to the current GPU and the result is returned on
-the CPU) or on a GPU.  Values are computed in fp32 with fp64 accumulation of the partial sums.
+* the per-token definitions on materialised logits the actor uses when the fused head is off --
+  ``logprobs_from_logits`` / ``_v2`` / ``_naive`` (reference :72-100, :148-200), ``entropy_from_logits`` /
+  ``entropy_from_logits_with_chunking`` (:224-263) -- as one online-softmax pass per row
+  (``vamd_row_softmax_stats``) with an elementwise backward (``vamd_row_softmax_backward``), and ``clip_by_value``
+  (:203-221);
+* the masked reductions ``masked_sum`` / ``masked_mean`` / ``masked_var`` / ``masked_whiten`` (:266-339).
+
+Inputs of the masked reductions may live on the CPU (they are staged to the current GPU and the result is
+returned on the CPU) or on a GPU.  Values are computed in fp32 with fp64 accumulation of the partial sums.
 """
 from __future__ import annotations
+
+import math
 
 import torch
 
 from .. import _cabi
+
+_ROW_DTYPES = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 2}   # VAMD_DT_*
+
+
+def _logit_rows(logits: torch.Tensor):
+    """``logits`` as a 2-D ``[rows, vocab]`` view with unit stride along the vocabulary, and its row pitch."""
+    assert logits.is_cuda, "the logits must live on the GPU: there is no CPU fallback"
+    assert logits.dtype in _ROW_DTYPES, f"logits must be fp32, bf16 or fp16, got {logits.dtype}"
+    assert logits.dim() >= 1 and logits.numel() > 0
+    vocab = logits.shape[-1]
+    rows = logits.reshape(-1, vocab)
+    if rows.stride(-1) != 1 or (rows.shape[0] > 1 and rows.stride(0) < vocab):
+        rows = rows.contiguous()
+    return rows, (rows.stride(0) if rows.shape[0] > 1 else vocab)
+
+
+def _row_stats(rows, ld, labels, want_logprobs: bool, want_entropy: bool, want_mean_z: bool):
+    n, vocab = rows.shape
+    dev = rows.device
+    f = lambda want: torch.empty(n, dtype=torch.float32, device=dev) if want else None
+    logprobs, entropy, lse, mean_z = f(want_logprobs), f(want_entropy), f(True), f(want_mean_z)
+    with torch.cuda.device(dev):
+        _cabi.check(_cabi.lib().vamd_row_softmax_stats(
+            rows.data_ptr(), _ROW_DTYPES[rows.dtype], n, vocab, ld, _cabi.ptr(labels), _cabi.ptr(logprobs),
+            _cabi.ptr(entropy), lse.data_ptr(), _cabi.ptr(mean_z), _cabi.stream_ptr(dev)))
+    return logprobs, entropy, lse, mean_z
+
+
+def _row_backward(rows, ld, labels, lse, mean_z, d_logprobs, d_entropy, in_place: bool):
+    n, vocab = rows.shape
+    dev = rows.device
+    out = rows if in_place else torch.empty((n, vocab), dtype=rows.dtype, device=dev)
+    ld_out = ld if in_place else vocab
+    g = lambda t: None if t is None else t.detach().reshape(-1).to(device=dev, dtype=torch.float32).contiguous()
+    d_logprobs, d_entropy = g(d_logprobs), g(d_entropy)
+    with torch.cuda.device(dev):
+        _cabi.check(_cabi.lib().vamd_row_softmax_backward(
+            rows.data_ptr(), _ROW_DTYPES[rows.dtype], n, vocab, ld, _cabi.ptr(labels), lse.data_ptr(),
+            _cabi.ptr(mean_z), _cabi.ptr(d_logprobs), _cabi.ptr(d_entropy), out.data_ptr(), ld_out,
+            _cabi.stream_ptr(dev)))
+    return out
+
+
+class _LogProbsFromLogits(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, labels, inplace_backward: bool):
+        assert labels.shape == logits.shape[:-1], f"labels {tuple(labels.shape)} do not match logits {tuple(logits.shape)}"
+        rows, ld = _logit_rows(logits)
+        lab = labels.reshape(-1).to(device=rows.device, dtype=torch.int64).contiguous()
+        logprobs, _, lse, _ = _row_stats(rows, ld, lab, True, False, False)
+        ctx.save_for_backward(rows, lab, lse)
+        ctx.ld, ctx.shape = ld, logits.shape
+        # writing the gradient over the logits needs the rows to BE the caller's storage
+        ctx.in_place = (bool(inplace_backward) and rows.data_ptr() == logits.data_ptr() and logits.is_contiguous()
+                        and not (logits.is_leaf and logits.requires_grad))   # never overwrite a parameter
+        return logprobs.to(logits.dtype).view(logits.shape[:-1])
+
+    @staticmethod
+    def backward(ctx, g):
+        rows, lab, lse = ctx.saved_tensors
+        d = _row_backward(rows, ctx.ld, lab, lse, None, g, None, ctx.in_place)
+        return d.view(ctx.shape), None, None
+
+
+class _EntropyFromLogits(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, fp32_output: bool):
+        rows, ld = _logit_rows(logits)
+        _, entropy, lse, mean_z = _row_stats(rows, ld, None, False, True, True)
+        ctx.save_for_backward(rows, lse, mean_z)
+        ctx.ld, ctx.shape = ld, logits.shape
+        if not fp32_output:
+            entropy = entropy.to(logits.dtype)
+        return entropy.view(logits.shape[:-1])
+
+    @staticmethod
+    def backward(ctx, g):
+        rows, lse, mean_z = ctx.saved_tensors
+        d = _row_backward(rows, ctx.ld, None, lse, mean_z, None, g, False)
+        return d.view(ctx.shape), None
+
+
+def logprobs_from_logits(logits: torch.Tensor, labels: torch.Tensor, inplace_backward: bool = True) -> torch.Tensor:
+    """Log-probability of ``labels`` under ``softmax(logits)``, shape ``logits.shape[:-1]``, dtype of ``logits``
+    (reference torch_functional.py:72-100).  With ``inplace_backward`` the backward pass writes the gradient over
+    the logits, as the reference's flash-attn path does: pass ``False`` when the logits are used again."""
+    return _LogProbsFromLogits.apply(logits, labels, inplace_backward)
+
+
+def logprobs_from_logits_naive(logits: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
+    """``log_softmax`` + gather (reference torch_functional.py:148-163)."""
+    return _LogProbsFromLogits.apply(logits, labels, False)
+
+
+def logprobs_from_logits_v2(logits: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
+    """``logits[label] - logsumexp(logits)`` row by row (reference torch_functional.py:166-200); fp32 arithmetic for
+    every input dtype, one rounding to the dtype of ``logits`` at the end."""
+    return _LogProbsFromLogits.apply(logits, labels, False)
+
+
+def entropy_from_logits(logits: torch.Tensor) -> torch.Tensor:
+    """``logsumexp(logits) - sum(softmax(logits) * logits)`` (reference torch_functional.py:224-238), dtype of
+    ``logits``."""
+    return _EntropyFromLogits.apply(logits, False)
+
+
+def entropy_from_logits_with_chunking(logits: torch.Tensor, chunk_size: int = 2048) -> torch.Tensor:
+    """The same in fp32 whatever the dtype of ``logits`` (reference torch_functional.py:241-263).  ``chunk_size``
+    is accepted for the signature: the kernel walks a row at a time and holds no ``[chunk, vocab]`` temporaries."""
+    return _EntropyFromLogits.apply(logits, True)
+
+
+class _ClipByValue(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, tensor_min, tensor_max):
+        dev = _cabi.compute_device(x, tensor_min, tensor_max)
+        to = lambda t: torch.as_tensor(t, dtype=torch.float32, device=dev)
+        shape = torch.broadcast_shapes(*(tuple(torch.as_tensor(t).shape) for t in (x, tensor_min, tensor_max)))
+        xs, lo, hi = (to(t).expand(shape).contiguous() for t in (x, tensor_min, tensor_max))
+        out = torch.empty_like(xs)
+        if xs.numel():
+            with torch.cuda.device(dev):
+                _cabi.check(_cabi.lib().vamd_clip_by_value(xs.data_ptr(), lo.data_ptr(), hi.data_ptr(), xs.numel(),
+                                                           out.data_ptr(), _cabi.stream_ptr(dev)))
+        ctx.save_for_backward(xs, lo, hi)
+        ctx.meta = [(tuple(t.shape), t.dtype, t.device) if isinstance(t, torch.Tensor) else None
+                    for t in (x, tensor_min, tensor_max)]
+        dtypes = [t.dtype for t in (x, tensor_min, tensor_max) if isinstance(t, torch.Tensor)]
+        dtype = torch.float32
+        if dtypes:   # what torch.max(torch.min(x, hi), lo) would return for same-rank tensors
+            dtype = dtypes[0]
+            for d in dtypes[1:]:
+                dtype = torch.promote_types(dtype, d)
+            if not dtype.is_floating_point:
+                dtype = torch.float32
+        return out.to(device=x.device if isinstance(x, torch.Tensor) else dev, dtype=dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        xs, lo, hi = ctx.saved_tensors
+        dev = xs.device
+        gs = g.detach().to(device=dev, dtype=torch.float32).expand(xs.shape).contiguous()
+        need = ctx.needs_input_grad
+        outs = [torch.empty_like(xs) if need[i] and ctx.meta[i] is not None else None for i in range(3)]
+        if xs.numel() and any(o is not None for o in outs):
+            with torch.cuda.device(dev):
+                _cabi.check(_cabi.lib().vamd_clip_by_value_backward(
+                    xs.data_ptr(), lo.data_ptr(), hi.data_ptr(), gs.data_ptr(), xs.numel(), _cabi.ptr(outs[0]),
+                    _cabi.ptr(outs[1]), _cabi.ptr(outs[2]), _cabi.stream_ptr(dev)))
+        res = []
+        for o, meta in zip(outs, ctx.meta):
+            if o is None:
+                res.append(None)
+            else:
+                shape, dtype, device = meta
+                res.append(o.sum_to_size(shape).to(device=device, dtype=dtype))
+        return tuple(res)
+
+
+def clip_by_value(x: torch.Tensor, tensor_min: torch.Tensor, tensor_max: torch.Tensor) -> torch.Tensor:
+    """``max(min(x, tensor_max), tensor_min)`` with tensor bounds that broadcast against ``x`` (reference
+    torch_functional.py:203-221), differentiable in all three arguments with torch's tie rule."""
+    return _ClipByValue.apply(x, tensor_min, tensor_max)
 
 
 def _as_matrix(values: torch.Tensor, mask: torch.Tensor, dev: torch.device):
@@ -35,27 +206,83 @@ def _moments(values: torch.Tensor, mask: torch.Tensor, per_row: bool) -> torch.T
     return out.t() if per_row else out
 
 
+def _normalise_axis(axis, ndim: int):
+    """``None`` or the sorted tuple of reduced dimensions."""
+    if axis is None:
+        return None
+    dims = (axis,) if isinstance(axis, int) else tuple(axis)
+    dims = tuple(sorted(d % ndim for d in dims)) if ndim else ()
+    assert len(set(dims)) == len(dims), f"duplicate dimension in axis={axis}"
+    return dims
+
+
+class _MaskedReduce(torch.autograd.Function):
+    """``masked_sum`` / ``masked_mean`` over any set of dimensions.  The reduced dimensions are moved last and the
+    tensor is seen as ``[kept, reduced]``, which the row-wise moments kernel reduces; the gradient is
+    ``mask * upstream`` (``/ (mask.sum + 1e-8)`` for the mean), one row-scaling kernel."""
+
+    @staticmethod
+    def forward(ctx, values, mask, dims, mean: bool):
+        ndim = values.dim()
+        dev = _cabi.compute_device(values, mask)
+        if dims is None:
+            # all elements: keep the tensor's own [leading, last] matrix shape, which spreads the launch over rows
+            perm, kept_shape = tuple(range(ndim)), ()
+            cols = values.shape[-1] if ndim else 1
+            rows = values.numel() // cols
+        else:
+            kept = tuple(d for d in range(ndim) if d not in dims)
+            perm = kept + dims
+            kept_shape = tuple(values.shape[d] for d in kept)
+            rows = math.prod(kept_shape)
+            cols = math.prod(values.shape[d] for d in dims)
+        v = _cabi.as_f32(values, dev).permute(perm).reshape(rows, cols).contiguous()
+        m, _ = _cabi.mask_code(mask.detach().to(dev).permute(perm).reshape(rows, cols))
+        mom = _moments(v, m, per_row=dims is not None)              # fp64: [4, rows], or [4] for all elements
+        total = mom[1].to(torch.float32)
+        denom = mom[0].to(torch.float32) + 1e-8 if mean else None
+        out = total / denom if mean else total
+        ctx.save_for_backward(m, denom)
+        ctx.geometry = (perm, tuple(values.shape), rows, cols, values.dtype, values.device)
+        out_dtype = torch.result_type(values, mask)
+        if not out_dtype.is_floating_point:
+            out_dtype = torch.float32
+        return out.view(kept_shape).to(device=values.device, dtype=out_dtype)
+
+    @staticmethod
+    def backward(ctx, g):
+        m, denom = ctx.saved_tensors
+        perm, shape, rows, cols, dtype, device = ctx.geometry
+        dev = m.device
+        coef = g.detach().to(device=dev, dtype=torch.float32).reshape(-1)   # one per kept row, or one in all
+        if denom is not None:
+            coef = coef / denom
+        coef = coef.expand(rows).contiguous()
+        weights = m if m.dtype == torch.float32 else m.to(torch.float32)   # d masked_sum / d values = mask
+        one = torch.ones(1, dtype=torch.float32, device=dev)
+        res = torch.empty((rows, cols), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            _cabi.check(_cabi.lib().vamd_scale_rows(weights.data_ptr(), coef.data_ptr(), one.data_ptr(), 1.0, rows,
+                                                    cols, res.data_ptr(), _cabi.stream_ptr(dev)))
+        inverse = [0] * len(perm)
+        for i, d in enumerate(perm):
+            inverse[d] = i
+        res = res.view([shape[d] for d in perm]).permute(inverse)
+        return res.to(device=device, dtype=dtype), None, None, None
+
+
 def _reduce(values, mask, axis, mean: bool):
-    if values.requires_grad:
-        raise NotImplementedError("verl_amd masked reductions are forward-only; detach the input or use agg_loss")
-    if values.numel() == 0:
-        raise ValueError("masked reduction of an empty tensor")
-    ndim = values.dim()
-    if axis is not None and not (axis in (-1, ndim - 1) or (ndim == 1 and axis == 0)):
-        raise NotImplementedError("verl_amd masked reductions support axis=None and the last axis")
-    dev = _cabi.compute_device(values, mask)
-    v, m, _ = _as_matrix(values, mask, dev)
-    mom = _moments(v, m, per_row=axis is not None and ndim > 1)
-    s = mom[1].to(torch.float32)
-    if mean:
-        s = s / (mom[0].to(torch.float32) + 1e-8)
-    if axis is not None and ndim > 1:
-        s = s.view(values.shape[:-1])
-    return s.to(values.device)
+    assert values.shape == mask.shape, f"values {tuple(values.shape)} and mask {tuple(mask.shape)} differ"
+    dims = _normalise_axis(axis, values.dim())
+    if values.numel() == 0:   # a sum over nothing is 0, and 0 / (0 + 1e-8) is 0
+        kept = () if dims is None else tuple(s for d, s in enumerate(values.shape) if d not in dims)
+        return torch.zeros(kept, dtype=torch.float32, device=values.device)
+    return _MaskedReduce.apply(values, mask, dims, mean)
 
 
 def masked_sum(values: torch.Tensor, mask: torch.Tensor, axis=None) -> torch.Tensor:
-    """sum(where(mask.bool(), values, 0) * mask) (reference torch_functional.py:266-284)."""
+    """sum(where(mask.bool(), values, 0) * mask) over ``axis`` (an int, a tuple of ints or ``None`` for all
+    elements), differentiable in ``values`` (reference torch_functional.py:266-284)."""
     return _reduce(values, mask, axis, mean=False)
 
 
@@ -79,7 +306,11 @@ def _raise_on_tiny_mask(mask_sum: float) -> None:
 
 
 def masked_var(values: torch.Tensor, mask: torch.Tensor, unbiased: bool = True) -> torch.Tensor:
-    """Two-pass masked variance with Bessel's factor (reference torch_functional.py:304-319)."""
+    """Masked variance with Bessel's factor (reference torch_functional.py:304-319).  The reference centres by
+    the mean in a second fp32 pass; here one pass accumulates count, sum and sum of squares in fp64 and the
+    variance is ``(S2 - 2 mean S1 + mean^2 S0) / S0`` evaluated in fp64.  With fp32 inputs the cancellation
+    costs a relative error of about ``(mean / std)^2 * 1e-16``: below fp32 resolution while ``|mean| / std``
+    stays under about 1e4."""
     _, mom, _ = _global_moments(values, mask)
     s0, s1, s2, _ = (x for x in mom.to("cpu").tolist())
     mean = torch.tensor(s1, dtype=torch.float32) / (torch.tensor(s0, dtype=torch.float32) + 1e-8)
