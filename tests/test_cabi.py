@@ -5,6 +5,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 import torch
 
@@ -101,8 +102,20 @@ def test_registries_and_host_logic_without_gpu():
     g = as_torch_index(["a", "b", "a", "c", "0042", 42])
     assert g.tolist()[4] != g.tolist()[5] and len(torch.unique(g)) == 5
     assert as_torch_index(["5", "6", "5"]).tolist() == [5, 6, 5]
-    ids, G = contiguous_group_ids([10, 10, 7, 99])
-    assert G == 3 and ids.tolist() == [1, 1, 0, 2]
+    assert as_torch_index(torch.tensor([1.0, 2.0, 1.0])).tolist() == [1, 2, 1]
+    assert as_torch_index(np.array([3, 3, 7])).tolist() == [3, 3, 7]
+    assert as_torch_index(np.array([True, False])).tolist() == [1, 0]
+    assert as_torch_index(np.array([1.5, 2.5, 1.5])).tolist() == [1, 2, 1]          # numpy floats: integer cast
+    t = as_torch_index(torch.tensor([1.5, 2.5, 1.5]))                               # tensor floats: opaque labels
+    assert t.tolist() == [0, 1, 0]
+    ids, G = contiguous_group_ids([10, 10, 7, 99])                                  # ids in order of first appearance
+    assert G == 3 and ids.tolist() == [0, 0, 1, 2]
+    ids, G = contiguous_group_ids(np.array(["u-1", "u-2", "u-1", 5, 5.0], dtype=object))
+    assert G == 3 and ids.tolist() == [0, 1, 0, 2, 2]                               # Python equality: 5 == 5.0
+    ids, G = contiguous_group_ids(["0042", 42, "x"])
+    assert G == 3
+    ids, G = contiguous_group_ids(["0042", "42", "7"], vectorized=True)             # numeric strings coincide there
+    assert G == 2 and ids.tolist() == [0, 0, 1]
 
 
 def test_backward_rejects_operands_beyond_32_bit_offsets(lib):
@@ -132,3 +145,27 @@ def test_static_forward_refuses_sizes_beyond_its_buffer_before_any_gpu_call(lib)
     # the pointers are never dereferenced: the size check precedes every HIP call
     rc = lib.vamd_lce_forward_static(1, 1, 1, 65536 + 1, 128, 256, 1.0, 1, 1, 1, 1, None, None)
     assert rc == -1 and b"at most 65536 tokens" in lib.vamd_last_error()
+
+
+def test_as_torch_index_agrees_with_the_oracle_restatement():
+    """The product's label handling is written differently from the oracle's line-by-line restatement of
+    verl/utils/groupwise.py:91-160; both must give the same ids on every kind of label."""
+    import uuid
+
+    from oracle import advantages as A
+    from verl_amd.utils.groupwise import as_torch_index
+    rng = np.random.default_rng(0)
+    uuids = [str(uuid.UUID(int=int(x))) for x in rng.integers(0, 2**62, 9)]
+    cases = [
+        torch.tensor([3, 1, 3, 2]), torch.tensor([3, 1, 3], dtype=torch.int32), torch.tensor([True, False, True]),
+        torch.tensor([1.0, 2.0, 1.0]), torch.tensor([1.0, 2.0000001, 1.0]), torch.tensor([0.5, 1.5, 0.5]),
+        torch.tensor([1.0, 2.0], dtype=torch.bfloat16), torch.tensor([[1, 2], [2, 1]]),
+        np.array([3, 3, 7]), np.array([1.0, 2.0, 1.0]), np.array([1.5, 2.5, 1.5]), np.array([True, False]),
+        np.array(["5", "6", "5"]), np.array(uuids * 2, dtype=object), ["a", "b", "a", "c", "0042", 42],
+        ["5", "6", "5"], [3, 1, 3], (1.0, 2.0), np.array([[1, 2], [2, 1]]), [("a", 1), ("b", 2), ("a", 1)],
+    ]
+    for case in cases:
+        want = A.as_torch_index(case)
+        got = as_torch_index(case)
+        assert got.dtype == torch.long and got.dim() == 1
+        assert torch.equal(got, want.cpu()), f"{case!r}: {got.tolist()} vs {want.tolist()}"

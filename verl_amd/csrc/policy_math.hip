@@ -733,7 +733,8 @@ __device__ __forceinline__ void grpo_scalars_from_records(const double* __restri
   // does not divide the row count is a bijection and sends neighbouring lanes to different groups.
   // Index i = threadIdx.x + m * NT maps to row (i * stride) mod rows, walked by adding (NT * stride) mod rows.
   const unsigned n_rows = (unsigned)ga.rows;
-  const unsigned stride = n_rows % 61 ? 61 : (n_rows % 59 ? 59 : 53);
+  // (a row count divisible by 61, 59 and 53 at once -- a multiple of 190747 -- walks the rows in order instead)
+  const unsigned stride = n_rows % 61 ? 61 : (n_rows % 59 ? 59 : (n_rows % 53 ? 53 : 1));
   const unsigned first_row = (threadIdx.x * stride) % n_rows, row_step = ((unsigned)NT * stride) % n_rows;
   // rows of the HELD indices of a trip; `at` is the row of the trip's first index and moves on to the next trip
   auto trip_rows = [&](unsigned& at, int64_t (&rk)[HELD]) {

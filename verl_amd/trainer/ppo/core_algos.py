@@ -179,7 +179,7 @@ def _grpo(token_level_rewards, response_mask, index, epsilon, norm_adv_by_std_in
         r = _matrix(token_level_rewards, dev)
         m, code = _mask_matrix(response_mask, dev, r.shape)
         B, Lc = r.shape
-        ids, G = contiguous_group_ids(index)
+        ids, G = contiguous_group_ids(index, vectorized=std_mode == 1)
         if ids.numel() != B:
             raise ValueError(f"index has {ids.numel()} entries for a batch of {B}")
         ids = ids.to(dev)
@@ -230,7 +230,7 @@ def _group_outcome(token_level_rewards, response_mask, index, estimator: str, ep
         r = _matrix(token_level_rewards, dev)
         m, code = _mask_matrix(response_mask, dev, r.shape)
         B, Lc = r.shape
-        ids, G = contiguous_group_ids(index)
+        ids, G = contiguous_group_ids(index, vectorized=estimator == "rloo_vectorized")
         if ids.numel() != B:
             raise ValueError(f"index has {ids.numel()} entries for a batch of {B}")
         if min_group_size > 1:

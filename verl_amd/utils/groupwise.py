@@ -16,66 +16,84 @@ from .. import _cabi
 __all__ = ["as_torch_index", "group_mean_std"]
 
 
-def _labels_to_numpy(x: Any) -> np.ndarray:
+_INT_TENSORS = (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8, torch.bool)
+
+
+def _flat_labels(index: Any) -> tuple[np.ndarray, bool]:
+    """1-D numpy view of the labels and whether they came from a torch tensor (the reference treats non-integral
+    float TENSORS as opaque labels but hands non-integral float ARRAYS to numpy's integer cast)."""
+    if isinstance(index, torch.Tensor):
+        t = index.detach().reshape(-1).cpu()
+        if t.dtype.is_floating_point:
+            t = t.to(torch.float64)
+        return t.numpy(), True
     try:
-        arr = np.asarray(x)
+        arr = np.asarray(index)
     except Exception:
         try:
-            arr = np.array(list(x), dtype=object)
+            arr = np.array(list(index), dtype=object)
         except Exception:
-            arr = np.array([x], dtype=object)
-    return arr.reshape(-1)
+            arr = np.array([index], dtype=object)
+    return arr.reshape(-1), False
 
 
-def _factorise(arr: np.ndarray) -> np.ndarray:
+def _ids_if_numeric(arr: np.ndarray, from_torch: bool) -> Optional[np.ndarray]:
+    """int64 ids when the labels ARE numbers: integers and booleans as they are, floats within 1e-6 of an integer
+    rounded, and -- for non-tensor input -- anything numpy can cast to int64 (numeric strings such as "0042")."""
+    if arr.dtype != object and (np.issubdtype(arr.dtype, np.integer) or arr.dtype == np.bool_):
+        return arr.astype(np.int64, copy=False)
+    if arr.dtype != object and np.issubdtype(arr.dtype, np.floating):
+        nearest = np.rint(arr.astype(np.float64, copy=False))
+        if np.allclose(arr, nearest, rtol=0.0, atol=1e-6):
+            return nearest.astype(np.int64)
+    if from_torch:
+        return None
     try:
-        _, inv = np.unique(arr, return_inverse=True)
-    except Exception:  # unorderable mixed types: compare their string forms
-        _, inv = np.unique(np.array([str(v) for v in arr], dtype=object), return_inverse=True)
-    return inv.astype(np.int64, copy=False)
+        return arr.astype(np.int64)
+    except Exception:
+        return None
+
+
+def _ids_by_sorted_rank(arr: np.ndarray, from_torch: bool) -> np.ndarray:
+    """Rank of each label among the sorted distinct labels (``np.unique``), on their string forms when the labels
+    cannot be ordered against each other or came from a float tensor."""
+    labels = np.array([str(v) for v in arr.tolist()], dtype=object) if from_torch else arr.astype(object, copy=False)
+    try:
+        inverse = np.unique(labels, return_inverse=True)[1]
+    except Exception:
+        inverse = np.unique(np.array([str(v) for v in labels], dtype=object), return_inverse=True)[1]
+    return np.asarray(inverse, dtype=np.int64).reshape(-1)
 
 
 def as_torch_index(index: Any, device: torch.device | str | None = None) -> torch.Tensor:
-    """Group labels -> 1-D ``torch.long`` ids, following the reference's rules
-    (verl/utils/groupwise.py:91-160): integer tensors / arrays pass through unchanged, floats
-    within 1e-6 of integers are rounded, numeric strings are coerced, anything else (UUID strings,
-    mixed types) is factorised with ``np.unique(return_inverse=True)``.  The result stays on the
-    CPU unless ``device`` is given."""
-    target = torch.device(device) if device is not None else torch.device("cpu")
+    """Group labels -> 1-D ``torch.long`` ids with the results of the reference's ``as_torch_index``
+    (verl/utils/groupwise.py:91-160): numeric labels keep their value, every other kind of label (UUID strings,
+    mixed types) gets its rank among the distinct labels.  The result stays on the CPU unless ``device`` is given."""
+    arr, from_torch = _flat_labels(index)
+    ids = _ids_if_numeric(arr, from_torch)
+    if ids is None:
+        ids = _ids_by_sorted_rank(arr, from_torch)
+    out = torch.from_numpy(np.ascontiguousarray(ids))
+    return out if device is None else out.to(torch.device(device))
+
+
+def contiguous_group_ids(index: Any, vectorized: bool = False) -> tuple[torch.Tensor, int]:
+    """Labels -> ids ``0..G-1`` in order of first appearance (CPU int64) and ``G``.  Group membership is decided
+    by Python equality of the labels, as in the reference's ``id2score[index[i]]`` dictionaries
+    (verl/trainer/ppo/core_algos.py:305-312); nothing downstream depends on which id a group gets.
+    ``vectorized``: membership as the reference's vectorised estimators see it, i.e. equality of the
+    ``as_torch_index`` values (there the labels "0042" and 42 are one group)."""
+    if vectorized:
+        index = as_torch_index(index)
     if isinstance(index, torch.Tensor):
-        flat = index.reshape(-1)
-        if flat.dtype in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8, torch.bool):
-            return flat.to(device=target, dtype=torch.long)
-        if flat.dtype.is_floating_point:
-            f64 = flat.to(torch.float64)
-            rounded = torch.round(f64)
-            if torch.allclose(f64, rounded, rtol=0.0, atol=1e-6):
-                return rounded.to(device=target, dtype=torch.long)
-        arr = np.array([str(v.item()) for v in flat], dtype=object)
+        labels = index.detach().reshape(-1).cpu().tolist()
+    elif isinstance(index, np.ndarray):
+        labels = index.reshape(-1).tolist()
     else:
-        arr = _labels_to_numpy(index)
-        if arr.dtype != object and np.issubdtype(arr.dtype, np.integer):
-            return torch.from_numpy(arr.astype(np.int64, copy=False)).to(target)
-        if arr.dtype != object and np.issubdtype(arr.dtype, np.floating):
-            a64 = arr.astype(np.float64, copy=False)
-            rounded = np.rint(a64)
-            if np.allclose(a64, rounded, rtol=0.0, atol=1e-6):
-                return torch.from_numpy(rounded.astype(np.int64)).to(target)
-        try:
-            return torch.from_numpy(arr.astype(np.int64)).to(target)
-        except Exception:
-            pass
-        if arr.dtype != object:
-            arr = arr.astype(object)
-    return torch.from_numpy(_factorise(arr)).to(target)
-
-
-def contiguous_group_ids(index: Any) -> tuple[torch.Tensor, int]:
-    """Ids remapped to 0..G-1 (CPU int64) and G.  Membership is what matters downstream, so
-    integer labels that ``as_torch_index`` passes through are factorised here as well."""
-    ids = as_torch_index(index).cpu().numpy()
-    uniq, inv = np.unique(ids, return_inverse=True)
-    return torch.from_numpy(inv.astype(np.int64, copy=False).reshape(-1)), int(len(uniq))
+        labels = list(index)
+    table: dict = {}
+    ids = np.fromiter((table.setdefault(k, len(table)) for k in labels), dtype=np.int64, count=len(labels))
+    return torch.from_numpy(ids), len(table)
 
 
 @torch.no_grad()
