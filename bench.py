@@ -23,7 +23,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
-KERNEL_NAMES = ["lce_forward_kernel", "lce_merge_kernel", "lce_recompute_kernel", "lce_dgrad_kernel"]
+KERNEL_NAMES = ["lce_forward_kernel", "lce_merge_kernel", "lce_recompute_kernel", "lce_dgrad_kernel", "lce_dlogits_kernel"]
 # MFMA GEMMs of 2*N*V*H flops each that a kernel performs per step
 COPY_YARDSTICK_BYTES = 1 << 30
 # L2 <-> fabric bytes of one full-chunk launch (16384 vocabulary columns) of each kernel at this workload:
@@ -60,7 +60,7 @@ def cpu_baseline(n_cpu: int, h: int, v: int, temperature: float) -> dict:
     }
 
 
-def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> dict:
+def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_groups: int = 64, only=None) -> dict:
     """The [B, L] kernels (B = 512, L = 4096 is the size of the GRPO / policy-loss and GAE benchmark configurations): microseconds per call from HIP events
     over 48 calls (best of three such loops) that rotate through 8 buffer sets, 16 at the smaller size (so that even the two-tensor ops
     touch more than the 256 MB Infinity Cache before they come back to a set), the algorithmic bytes of
@@ -88,7 +88,7 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
     ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
     out = torch.empty(8, device=dev)
     coef = torch.empty(B, device=dev)
-    mom = torch.empty(4, dtype=torch.float64, device=dev)
+    mom = torch.empty(8, dtype=torch.float64, device=dev)
     gid = torch.arange(n_groups, device=dev).repeat_interleave(B // n_groups)
     rows_by_group = torch.arange(B, device=dev)                       # gid is already sorted
     group_offsets = torch.arange(0, B + 1, B // n_groups, device=dev)
@@ -182,6 +182,8 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
     }
     res = {}
     for name, (nbytes, fn) in ops.items():
+        if only is not None and name not in only:
+            continue
         for s in sets:
             fn(s)
         torch.cuda.synchronize()
@@ -239,7 +241,7 @@ def policy_math_chain(dev, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> 
     rewards, old, values = f(), f() * 0.5 - 1, f()
     new, vpreds = old + 0.05 * f(), values + 0.5 * f()
     adv, grad, gae_adv, gae_ret, vgrad = (torch.empty(B, Lc, device=dev) for _ in range(5))
-    out, coef, mom = torch.empty(4, device=dev), torch.empty(B, device=dev), torch.empty(4, dtype=torch.float64, device=dev)
+    out, coef, mom = torch.empty(4, device=dev), torch.empty(B, device=dev), torch.empty(8, dtype=torch.float64, device=dev)
     gid = torch.arange(n_groups, device=dev).repeat_interleave(B // n_groups)
     ws = torch.zeros(max(1 << 22, L.vamd_group_outcome_advantage_workspace_bytes(B, Lc, n_groups),
                          L.vamd_policy_loss_variant_workspace_bytes(B, Lc)), dtype=torch.uint8, device=dev)
@@ -280,12 +282,312 @@ def policy_math_chain(dev, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> 
     return {"launches_per_chain": 6, "eager_us": timed(chain), "hip_graph_us": timed(graph.replay)}
 
 
+def policy_math_python_path(dev, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> dict:
+    """The same operations called the way the trainer calls them -- through the functions of
+    ``verl_amd.trainer.ppo.core_algos`` / ``verl_amd.utils.torch_functional`` with torch tensors on the GPU --
+    so that argument checks, output allocation, ctypes marshalling and the host synchronisations the interfaces
+    require (Python-float metrics) are all inside the figure: wall-clock microseconds per call over 200 calls that
+    end in one device synchronisation (best of three loops)."""
+    import numpy as np
+    import torch
+
+    import verl_amd.utils.torch_functional as VF
+    from verl_amd.trainer.ppo import core_algos as CA
+
+    g = torch.Generator(device=dev).manual_seed(0)
+    f = lambda: torch.randn(B, Lc, device=dev, generator=g)
+    lens = torch.randint(64, Lc + 1, (B,), device=dev, generator=g)
+    mask = (torch.arange(Lc, device=dev)[None, :] < lens[:, None]).float()
+    rewards, old, values = f(), f() * 0.5 - 1, f()
+    new, vpreds = (old + 0.05 * f()).requires_grad_(), (values + 0.5 * f()).requires_grad_()
+    adv, returns = f(), f()
+    index = np.repeat(np.arange(n_groups), B // n_groups)
+
+    class Cfg:
+        clip_ratio, clip_ratio_low, clip_ratio_high, global_batch_info = 0.2, None, None, {}
+
+        @staticmethod
+        def get(key, default=None):
+            return default
+
+    def policy_fwd():
+        with torch.no_grad():
+            CA.compute_policy_loss_vanilla(old, new, adv, mask, "token-mean", Cfg)
+
+    def policy_fwd_bwd():
+        loss, _ = CA.compute_policy_loss_vanilla(old, new, adv, mask, "token-mean", Cfg)
+        torch.autograd.grad(loss, new)
+
+    def value_fwd_bwd():
+        loss, _ = CA.compute_value_loss(vpreds, returns, values, mask, 0.5, "token-mean")
+        torch.autograd.grad(loss, vpreds)
+
+    ops = {
+        "grpo_advantage": lambda: CA.compute_grpo_outcome_advantage(rewards, mask, index),
+        "policy_loss_fwd": policy_fwd,
+        "policy_loss_fwd_grad": policy_fwd_bwd,
+        "gae_scan_whiten": lambda: CA.compute_gae_advantage_return(rewards, values, mask, 1.0, 0.95),
+        "value_loss_fwd_grad": value_fwd_bwd,
+        "masked_mean": lambda: VF.masked_mean(values, mask),
+        "masked_whiten": lambda: VF.masked_whiten(values, mask),
+        "agg_loss_token_mean": lambda: CA.agg_loss(values, mask, "token-mean"),
+    }
+    res = {}
+    for name, fn in ops.items():
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            t0 = time.perf_counter()
+            for _ in range(200):
+                fn()
+            torch.cuda.synchronize()
+            best = min(best, (time.perf_counter() - t0) / 200 * 1e6)
+        res[name] = {"us_per_call": best}
+    return res
+
+
+def _sclk_sampler():
+    """Background reader of the shader clock (rocm-smi), for the ceiling probe: returns (stop, samples)."""
+    import subprocess
+    import threading
+
+    samples, stop = [], threading.Event()
+
+    def run():
+        while not stop.is_set():
+            try:
+                out = subprocess.run(["rocm-smi", "--showclocks", "--json"], capture_output=True, text=True, timeout=5).stdout
+                txt = json.loads(out).get("card0", {}).get("sclk clock speed:", "")
+                mhz = int("".join(c for c in txt if c.isdigit()) or 0)
+                if mhz:
+                    samples.append((time.time(), mhz))
+            except Exception:
+                pass
+            stop.wait(0.15)
+
+    th = threading.Thread(target=run, daemon=True)
+    th.start()
+    return stop, samples
+
+
+def mfma_ceiling_probe(dev, n: int, h: int, v: int, seconds: float = 1.5) -> dict:
+    """Where the matrix pipes top out on THIS board and data: the head's forward kernel and the vendor GEMM
+    (torch.matmul -> hipBLASLt) at the three operand layouts of the step (logits NT, d_hidden NN, d_weight TN,
+    one 16384-column vocabulary chunk each), on all-zero operands and on the benchmark's random operands, each run
+    back to back for `seconds` with the shader clock read beside it.  Zeros draw the least power, so the clock
+    stays at its maximum there; the random figures are what power management leaves."""
+    import torch
+
+    from verl_amd import _cabi
+
+    L = _cabi.lib()
+    st = _cabi.stream_ptr(dev)
+    g = torch.Generator(device=dev).manual_seed(0)
+    labels = torch.randint(0, v, (n,), device=dev, generator=g)
+    outs = [torch.empty(n, device=dev) for _ in range(4)]
+    ws = torch.empty(L.vamd_lce_forward_workspace_bytes(n, h, v), dtype=torch.uint8, device=dev)
+    vc = 16384
+    stop, samples = _sclk_sampler()
+    res = {}
+
+    def run_for(fn, flops):
+        fn()
+        torch.cuda.synchronize()
+        t_begin = time.time()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 0
+        e0.record()
+        while time.time() - t_begin < seconds:
+            for _ in range(4):
+                fn()
+            reps += 4
+            torch.cuda.synchronize()
+        e1.record()
+        torch.cuda.synchronize()
+        t_end = time.time()
+        ms = e0.elapsed_time(e1) / reps
+        clk = [m for (t, m) in samples if t_begin + 0.4 * (t_end - t_begin) <= t <= t_end]
+        return {"ms": ms, "PFLOPs": flops / ms / 1e12, "sclk_MHz": (sum(clk) / len(clk)) if clk else None}
+
+    for kind in ("zeros", "random"):
+        if kind == "zeros":
+            hid = torch.zeros(n, h, device=dev, dtype=torch.bfloat16)
+            w = torch.zeros(v, h, device=dev, dtype=torch.bfloat16)
+        else:
+            hid = torch.randn(n, h, device=dev, generator=g).bfloat16()
+            w = (torch.randn(v, h, device=dev, generator=g) * 0.02).bfloat16()
+
+        def fwd():
+            _cabi.check(L.vamd_lce_forward(hid.data_ptr(), w.data_ptr(), labels.data_ptr(), n, h, v, 1.0,
+                                           *(o.data_ptr() for o in outs), None, None, ws.data_ptr(), ws.numel(), st))
+
+        wc = w[:vc]
+        z = torch.empty(n, vc, device=dev, dtype=torch.bfloat16)
+        dh = torch.empty(n, h, device=dev, dtype=torch.bfloat16)
+        dw = torch.empty(vc, h, device=dev, dtype=torch.bfloat16)
+        res[kind] = {
+            "lce_forward_kernel": run_for(fwd, 2.0 * n * v * h),
+            "vendor_gemm_NT_logits": run_for(lambda: torch.matmul(hid, wc.t(), out=z), 2.0 * n * vc * h),
+        }
+        if kind == "random":
+            z.normal_(generator=g)
+        res[kind]["vendor_gemm_NN_d_hidden"] = run_for(lambda: torch.matmul(z, wc, out=dh), 2.0 * n * vc * h)
+        res[kind]["vendor_gemm_TN_d_weight"] = run_for(lambda: torch.matmul(z.t(), hid, out=dw), 2.0 * n * vc * h)
+        del hid, w, wc, z, dh, dw
+    stop.set()
+    res["note"] = ("ms per call; PFLOP/s on 2*M*N*K; sclk from rocm-smi over the second half of each run "
+                   "(None when rocm-smi is unavailable); vendor GEMMs on one 16384-column vocabulary chunk")
+    return res
+
+
+def time_head_mode(step, steps: int, warmup: int, n: int, dev) -> dict:
+    """Wall-clock milliseconds per forward+backward step and the peak device memory the step adds."""
+    import torch
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats(dev)
+    base = torch.cuda.memory_allocated(dev)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    return {"ms_per_step": dt / steps * 1e3, "tokens_per_s": n * steps / dt,
+            "peak_step_memory_bytes": torch.cuda.max_memory_allocated(dev) - base}
+
+
+def head_kernel_times(L, step, prof_steps: int) -> dict:
+    """Per-kernel durations from HIP events recorded on the launch stream around every head kernel launch."""
+    from verl_amd import _cabi
+
+    L.vamd_lce_timing_enable(1)
+    for _ in range(prof_steps):
+        step()
+    ms = (ctypes.c_double * len(KERNEL_NAMES))()
+    cnt = (ctypes.c_int64 * len(KERNEL_NAMES))()
+    _cabi.check(L.vamd_lce_timing_collect(ms, cnt))
+    L.vamd_lce_timing_enable(0)
+    kernels = {}
+    for i, name in enumerate(KERNEL_NAMES):
+        if cnt[i]:
+            kernels[name] = {"ms_per_step": ms[i] / prof_steps, "launches_per_step": cnt[i] / prof_steps,
+                             "avg_ms": ms[i] / cnt[i]}
+    return kernels
+
+
+def other_head_configs(dev, steps: int) -> dict:
+    """BASELINE configs[0] (Qwen2.5-0.5B head shape, forward only) and configs[4] (Llama-3-8B head shape, 65536
+    tokens as eight 8192-token chunks, T = 0.7, entropy coefficient folded into the backward, weight gradient summed
+    over the chunks in fp32), timed end to end through the host mirror."""
+    import torch
+
+    from verl_amd.utils.kernel import linear_cross_entropy as K
+
+    g = torch.Generator(device=dev).manual_seed(3)
+    res = {}
+    n, h, v = 2048, 896, 151936
+    hid = torch.randn(n, h, device=dev, generator=g).bfloat16()
+    w = (torch.randn(v, h, device=dev, generator=g) * 0.02).bfloat16()
+    lab = torch.randint(0, v, (n,), device=dev, generator=g)
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps * 1e3
+
+    with torch.no_grad():
+        ms = timed(lambda: K.linear_cross_entropy(hid, w, lab, 1.0), 20)
+    res["qwen0.5b_forward_only"] = {"n_tokens": n, "hidden_size": h, "vocab": v, "ms": ms, "tokens_per_s": n / ms * 1e3,
+                                    "PFLOPs_algorithmic": 2.0 * n * v * h / ms / 1e12}
+    del hid, w, lab
+    n, h, v, T, chunk = 65536, 4096, 128256, 0.7, 8192
+    hid = torch.randn(n, h, device=dev, generator=g).bfloat16()
+    w = (torch.randn(v, h, device=dev, generator=g) * 0.02).bfloat16()
+    lab = torch.randint(0, v, (n,), device=dev, generator=g)
+    g_lp = torch.randn(n, device=dev, generator=g)
+    acc32 = torch.empty(v, h, device=dev, dtype=torch.float32)
+    d_weight = torch.empty_like(w)
+    n_chunks = n // chunk
+
+    def long_rollout():
+        for ci in range(n_chunks):
+            sl = slice(ci * chunk, (ci + 1) * chunk)
+            _, _, lse, mz = K.efficient_entropy_forward(hid[sl], w, lab[sl], 0, T)
+            K.efficient_entropy_backward(g_lp[sl], None, hid[sl], w, lab[sl], lse, mz, 0, T, d_entropy_scalar=0.001,
+                                         d_weight_acc32=acc32, d_weight_out=d_weight,
+                                         acc32_step="first" if ci == 0 else ("last" if ci == n_chunks - 1 else "middle"))
+
+    ms = timed(long_rollout, max(1, min(steps, 3)))
+    res["llama8b_long_rollout_fwd_bwd"] = {"n_tokens": n, "hidden_size": h, "vocab": v, "temperature": T,
+                                           "token_chunk": chunk, "ms": ms, "tokens_per_s": n / ms * 1e3,
+                                           "PFLOPs_algorithmic": 6.0 * n * v * h / ms / 1e12,
+                                           "mode": "recompute, fp32 d_weight accumulation over the 8 chunks"}
+    return res
+
+
+def unfused_logits_rates(dev) -> dict:
+    """The per-token definitions on materialised logits (row-wise online softmax): microseconds, algorithmic bytes
+    (the logits once forward; logits in + gradient out backward) and the fraction of 8 TB/s, at 4096 tokens of the
+    Qwen2.5-7B vocabulary.  Two buffer sets alternate so that a call never finds its rows in the Infinity Cache."""
+    import torch
+
+    from verl_amd import _cabi
+
+    L = _cabi.lib()
+    n, v = 4096, 152064
+    st = _cabi.stream_ptr(dev)
+    res = {}
+    for name, dtype, code, esz in (("bf16", torch.bfloat16, 1, 2), ("fp32", torch.float32, 0, 4)):
+        sets = [torch.randn(n, v, device=dev, dtype=dtype) for _ in range(2)]
+        grads = [torch.empty(n, v, device=dev, dtype=dtype) for _ in range(2)]
+        labels = torch.randint(0, v, (n,), device=dev)
+        f = [torch.empty(n, device=dev) for _ in range(4)]
+        g_lp = torch.randn(n, device=dev)
+
+        def fwd(i):
+            _cabi.check(L.vamd_row_softmax_stats(sets[i].data_ptr(), code, n, v, v, labels.data_ptr(), f[0].data_ptr(),
+                                                 f[1].data_ptr(), f[2].data_ptr(), f[3].data_ptr(), st))
+
+        def bwd(i):
+            _cabi.check(L.vamd_row_softmax_backward(sets[i].data_ptr(), code, n, v, v, labels.data_ptr(), f[2].data_ptr(),
+                                                    f[3].data_ptr(), g_lp.data_ptr(), g_lp.data_ptr(),
+                                                    grads[i].data_ptr(), v, st))
+
+        for label, fn, nbytes in (("forward", fwd, n * v * esz), ("backward", bwd, 2 * n * v * esz)):
+            fn(0); fn(1)
+            torch.cuda.synchronize()
+            best = float("inf")
+            for _ in range(3):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for i in range(8):
+                    fn(i % 2)
+                e1.record()
+                torch.cuda.synchronize()
+                best = min(best, e0.elapsed_time(e1) / 8 * 1e3)
+            res[f"{name}_{label}"] = {"us": best, "algorithmic_bytes": nbytes, "GBps": nbytes / best / 1e3,
+                                      "frac_of_8TBps": nbytes / best / 1e3 / 8000.0}
+        del sets, grads
+    res["shape"] = {"n_tokens": n, "vocab": v}
+    return res
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--cpu-tokens", type=int, default=8192, help="token sample for the CPU baseline (0 = skip)")
+    ap.add_argument("--head-only", action="store_true",
+                    help="only the headline workload and its per-kernel timing (what the profiler runs trace)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (every box here has one GPU; "
@@ -321,33 +623,21 @@ def main() -> None:
     torch.cuda.synchronize()
     del src, dst
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
-    tokens_per_s = n * args.steps / dt
-
-    # per-kernel durations from HIP events on the launch stream (a separate, untimed pass)
-    L.vamd_lce_timing_enable(1)
+    # The headline is the mode the library ships as its default (whatever VAMD_LCE_LOGITS_CACHE_GB says in this
+    # process's environment; unset = no cache, the backward pass recomputes the logits).
+    default_cached = 4 * n * v <= logits_cache_budget_bytes()
+    head = time_head_mode(step, args.steps, args.warmup, n, dev)
+    ms_per_step, tokens_per_s = head["ms_per_step"], head["tokens_per_s"]
     prof_steps = max(1, min(args.steps, 5))
-    for _ in range(prof_steps):
-        step()
-    ms = (ctypes.c_double * len(KERNEL_NAMES))()
-    cnt = (ctypes.c_int64 * len(KERNEL_NAMES))()
-    _cabi.check(L.vamd_lce_timing_collect(ms, cnt))
-    L.vamd_lce_timing_enable(0)
-    kernels = {}
-    for i, name in enumerate(KERNEL_NAMES):
-        if cnt[i]:
-            kernels[name] = {"ms_per_step": ms[i] / prof_steps, "launches_per_step": cnt[i] / prof_steps,
-                             "avg_ms": ms[i] / cnt[i]}
+    kernels = head_kernel_times(L, step, prof_steps)
+
     gemm_flops = 2.0 * n * v * h
-    cached = 4 * n * v <= logits_cache_budget_bytes()   # backward forms d_logits from cached logits: no recompute GEMM
+    peak = PEAK_BF16_TFLOPS * 1e12
+
+    def fractions(ms, cached):
+        return {"step_algorithmic_frac": 6.0 * gemm_flops / 2.0 / (ms * 1e-3) / peak,
+                "step_hardware_frac": (6.0 if cached else 8.0) * gemm_flops / 2.0 / (ms * 1e-3) / peak}
+
     dom = max((k for k in kernels if k in GEMMS_PER_STEP), key=lambda k: kernels[k]["ms_per_step"])
     d = kernels[dom]
     flops_per_launch = GEMMS_PER_STEP[dom] * gemm_flops / d["launches_per_step"]
@@ -359,23 +649,31 @@ def main() -> None:
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_BF16_TFLOPS,
-        "traffic": MEASURED_TRAFFIC_BYTES.get(dom) if cached else None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
         "flops_per_launch": flops_per_launch,
         "avg_launch_ms": d["avg_ms"],
-        "step_algorithmic_frac": 6.0 * n * v * h / (ms_per_step * 1e-3) / (PEAK_BF16_TFLOPS * 1e12),
-        "step_hardware_frac": (6.0 if cached else 8.0) * n * v * h / (ms_per_step * 1e-3) / (PEAK_BF16_TFLOPS * 1e12),
+        **fractions(ms_per_step, default_cached),
         "kernels": kernels,
     }
 
-    base = cpu_baseline(args.cpu_tokens, h, v, T) if args.cpu_tokens > 0 else None
-    del hidden, weight
-    torch.cuda.empty_cache()
-    pm = policy_math_rates(dev, with_cpu=args.cpu_tokens > 0)
-    # the same kernels on 16 x larger tensors, where the fixed ~8 us of the single-launch reduction no longer dominates
-    pm_large = policy_math_rates(dev, with_cpu=False, B=2048, Lc=16384, n_groups=256)
-    pm_chain = policy_math_chain(dev)
+    # the other mode beside it, same process, same tensors
+    modes = {}
+    this_mode = "logits_cache" if default_cached else "recompute"
+    modes[this_mode] = {**head, **fractions(ms_per_step, default_cached), "default": True}
+    saved_env = os.environ.get("VAMD_LCE_LOGITS_CACHE_GB")
+    os.environ["VAMD_LCE_LOGITS_CACHE_GB"] = "0" if default_cached else "16"
+    other = time_head_mode(step, args.steps, args.warmup, n, dev)
+    other_kernels = head_kernel_times(L, step, prof_steps)
+    modes["recompute" if default_cached else "logits_cache"] = {
+        **other, **fractions(other["ms_per_step"], not default_cached), "default": False,
+        "kernels": other_kernels,
+        "enable": "VAMD_LCE_LOGITS_CACHE_GB=0" if default_cached else "VAMD_LCE_LOGITS_CACHE_GB=16"}
+    if saved_env is None:
+        del os.environ["VAMD_LCE_LOGITS_CACHE_GB"]
+    else:
+        os.environ["VAMD_LCE_LOGITS_CACHE_GB"] = saved_env
 
-    print(json.dumps({
+    line = {
         "metric": "tokens/s fwd+bwd logprob+entropy head @Qwen2.5-7B shape; MFMA util %",
         "value": tokens_per_s,
         "unit": "tokens/s",
@@ -392,14 +690,33 @@ def main() -> None:
                                "(BASELINE configs[1])",
                    "n_tokens": n, "hidden_size": h, "vocab": v, "temperature": T,
                    "upstream": "dlogprob ~ N(0,1) fp32, dentropy = 0.001",
-                   "fp32_logits_cache_bytes": 4 * n * v if 4 * n * v <= logits_cache_budget_bytes() else 0},
-        "mfma_util_pct": 100.0 * roofline["step_hardware_frac"],
+                   "backward": "logits cache" if default_cached else "recomputes the logits (no [tokens, vocab] tensor)",
+                   "fp32_logits_cache_bytes": 4 * n * v if default_cached else 0},
+        # algorithmic-or-recompute flops of the step over the 2.5 PFLOP/s peak: what share of the matrix pipes' peak
+        # the step's own arithmetic amounts to.  It is not a hardware counter.
+        "step_hardware_flops_pct_of_peak": 100.0 * roofline["step_hardware_frac"],
         "roofline": roofline,
-        "cpu_baseline": base,
-        "policy_math_b512_l4096": pm,
-        "policy_math_b2048_l16384": pm_large,
-        "policy_math_chain_b512_l4096": pm_chain,
-    }))
+        "head_modes": modes,
+    }
+    if args.head_only:
+        print(json.dumps(line))
+        return
+
+    line["cpu_baseline"] = cpu_baseline(args.cpu_tokens, h, v, T) if args.cpu_tokens > 0 else None
+    del hidden, weight
+    torch.cuda.empty_cache()
+    line["mfma_ceiling_probe"] = mfma_ceiling_probe(dev, n, h, v)
+    torch.cuda.empty_cache()
+    line["head_other_configs"] = other_head_configs(dev, args.steps)
+    torch.cuda.empty_cache()
+    line["unfused_logits_rows"] = unfused_logits_rates(dev)
+    torch.cuda.empty_cache()
+    line["policy_math_b512_l4096"] = policy_math_rates(dev, with_cpu=args.cpu_tokens > 0)
+    line["policy_math_python_path_b512_l4096"] = policy_math_python_path(dev)
+    # the same kernels on 16 x larger tensors, where the fixed ~8 us of the single-launch reduction no longer dominates
+    line["policy_math_b2048_l16384"] = policy_math_rates(dev, with_cpu=False, B=2048, Lc=16384, n_groups=256)
+    line["policy_math_chain_b512_l4096"] = policy_math_chain(dev)
+    print(json.dumps(line))
 
 
 if __name__ == "__main__":

@@ -236,10 +236,15 @@ int vamd_affine_by_stats(const float* values, const float* stats, int64_t n, flo
 /* ------------------------------------------------------------------------------------------
  * GAE: compute_gae_advantage_return (verl/trainer/ppo/core_algos.py:214-262).
  * rewards, values [B, L] fp32, mask [B, L]; advantages (whitened) and returns [B, L] fp32 out.
- * The recurrence is evaluated as a chunked associative scan of affine maps; masked steps carry
- * the state.  whiten == 0 leaves the raw advantages (the value before :261).
- * moments_out (4 doubles, may be NULL) receives the masked moments of the raw advantages so the
- * host can raise masked_var's M in {0,1} error.
+ * The recurrence is evaluated as a chunked associative scan (a most-recent-valid-value scan for the
+ * bootstrap value, then a one-variable affine scan for the advantage); masked steps carry the state.
+ * whiten == 0 leaves the raw advantages (the value before :261).  With whiten != 0 the whole estimator is one
+ * launch whose workgroups meet once (the grid is capped at what the device holds at a time): the masked
+ * moments are folded, and every workgroup whitens what it produced.
+ * moments_out (5 doubles, may be NULL) receives the masked moments of the raw advantages (sum m, sum g m,
+ * sum g^2 m, count) so the host can raise masked_var's M in {0,1} error; moments_out[4] is 0, or 1 if the
+ * workgroups' bounded wait for each other ran out (the advantages are then left raw; VAMD_GATE_SPIN_LIMIT in the
+ * environment overrides the bound).
  */
 size_t vamd_gae_workspace_bytes(int64_t batch, int64_t length);
 int vamd_gae(const float* rewards, const float* values, const void* mask, int mask_dtype, int64_t batch,
@@ -253,6 +258,9 @@ int vamd_gae(const float* rewards, const float* values, const void* mask, int ma
  * groupwise.as_torch_index does).  std_mode 0: unbiased torch.std (loop form); 1:
  * sqrt(clamp(var, min=eps)) (vectorised form).  scores_out [B] (may be NULL) receives the
  * normalised scalar per response.
+ * Up to 2048 (row, 4096-column) pieces and 512 groups the estimator is one launch whose workgroups meet once
+ * (bounded wait, as in vamd_gae); a workgroup whose wait runs out stores NaN advantages.  Larger inputs take a
+ * row-sum launch, a statistics launch and a broadcast launch.
  */
 size_t vamd_grpo_workspace_bytes(int64_t batch, int64_t length, int64_t n_groups);
 int vamd_grpo_advantage(const float* rewards, const void* mask, int mask_dtype, const int64_t* group_ids,

@@ -108,14 +108,18 @@ def test_registries_and_host_logic_without_gpu():
     assert as_torch_index(np.array([1.5, 2.5, 1.5])).tolist() == [1, 2, 1]          # numpy floats: integer cast
     t = as_torch_index(torch.tensor([1.5, 2.5, 1.5]))                               # tensor floats: opaque labels
     assert t.tolist() == [0, 1, 0]
-    ids, G = contiguous_group_ids([10, 10, 7, 99])                                  # ids in order of first appearance
+    ids, G = contiguous_group_ids([10, 10, 7, 99])                                  # a list: ids by first appearance
     assert G == 3 and ids.tolist() == [0, 0, 1, 2]
+    ids, G = contiguous_group_ids(np.array([10, 10, 7, 99]))                        # integers: ids by sorted label
+    assert G == 3 and ids.tolist() == [1, 1, 0, 2]
+    ids, G = contiguous_group_ids(torch.tensor([[3, 3], [1, 3]]))
+    assert G == 2 and ids.tolist() == [1, 1, 0, 1]
     ids, G = contiguous_group_ids(np.array(["u-1", "u-2", "u-1", 5, 5.0], dtype=object))
     assert G == 3 and ids.tolist() == [0, 1, 0, 2, 2]                               # Python equality: 5 == 5.0
     ids, G = contiguous_group_ids(["0042", 42, "x"])
     assert G == 3
     ids, G = contiguous_group_ids(["0042", "42", "7"], vectorized=True)             # numeric strings coincide there
-    assert G == 2 and ids.tolist() == [0, 0, 1]
+    assert G == 2 and ids.tolist() == [1, 1, 0]                                     # integers again: by sorted label
 
 
 def test_backward_rejects_operands_beyond_32_bit_offsets(lib):

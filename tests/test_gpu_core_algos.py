@@ -134,6 +134,74 @@ def test_gae_gamma_lambda_one_long_rows_vs_fp64(dev):
     _close(adv, adv64.float(), rtol=1e-5, atol=2e-5, what="whitened advantages vs fp64")
 
 
+@pytest.mark.parametrize("B,L", [(3000, 300), (5, 9000), (1500, 4100), (700, 4096), (2, 3), (1100, 37)])
+def test_gae_single_launch_paths(dev, B, L):
+    """The one-launch estimator on every route through it: more rows than the device holds workgroups (a workgroup
+    walks several rows and whitens them from memory), rows longer than one batch of segments, and a single row per
+    workgroup whose advantages wait in registers.  Masks with holes; compared with the fp64 evaluation of the
+    reference recurrence."""
+    from verl_amd.trainer.ppo.core_algos import compute_gae_advantage_return
+    g = torch.Generator().manual_seed(B * 7 + L)
+    r = torch.randn(B, L, generator=g)
+    v = torch.randn(B, L, generator=g)
+    m = (torch.rand(B, L, generator=g) < 0.8).float()
+    m[0] = 0
+    m[-1, : max(1, L // 2)] = 1
+    adv, ret = compute_gae_advantage_return(r.to(dev), v.to(dev), m.to(dev), 0.99, 0.95)
+    want_adv, want_ret = O.gae_advantage_return(r.double(), v.double(), m.double(), 0.99, 0.95)
+    scale = want_ret.abs().max().item()
+    assert (ret.cpu().double() - want_ret).abs().max().item() <= 2e-5 * scale
+    assert (adv.cpu().double() - want_adv).abs().max().item() <= 2e-5 * want_adv.abs().max().item()
+
+
+def test_gae_bounded_wait_runs_out_without_hanging(dev, monkeypatch):
+    """With the poll limit forced to zero the workgroups do not wait for the whitening statistics: every one of them
+    still exits, the host is told (RuntimeError), the arrival counters are back at zero and the next call is right."""
+    from verl_amd import _cabi
+    from verl_amd.trainer.ppo.core_algos import compute_gae_advantage_return
+    B, L = 512, 4096
+    g = torch.Generator().manual_seed(3)
+    r, v = torch.randn(B, L, generator=g).to(dev), torch.randn(B, L, generator=g).to(dev)
+    m = torch.ones(B, L, device=dev)
+    monkeypatch.setenv("VAMD_GATE_SPIN_LIMIT", "0")
+    with pytest.raises(RuntimeError, match="bounded wait"):
+        compute_gae_advantage_return(r, v, m, 1.0, 0.95)
+    torch.cuda.synchronize()
+    ws = _cabi.ticket_workspace(4096, dev)
+    assert int(ws[:16640].to(torch.int32).sum()) == 0
+    monkeypatch.delenv("VAMD_GATE_SPIN_LIMIT")
+    adv, ret = compute_gae_advantage_return(r, v, m, 1.0, 0.95)
+    want_adv, want_ret = O.gae_advantage_return(r.cpu().double(), v.cpu().double(), m.cpu().double(), 1.0, 0.95)
+    assert (adv.cpu().double() - want_adv).abs().max().item() <= 2e-5 * want_adv.abs().max().item()
+
+
+def test_grpo_single_launch_bounded_wait_runs_out_without_hanging(dev, monkeypatch):
+    """The one-launch GRPO estimator with its poll limit forced to zero: every workgroup exits, those that did not
+    see the statistics store NaN (never a wrong advantage), the counters are back at zero and the next call is
+    right."""
+    from verl_amd import _cabi
+    from verl_amd.trainer.ppo.core_algos import compute_grpo_outcome_advantage
+    B, L = 512, 4096
+    g = torch.Generator().manual_seed(5)
+    rewards = torch.zeros(B, L)
+    rewards[:, -1] = torch.bernoulli(torch.full((B,), 0.5), generator=g)
+    mask = torch.ones(B, L)
+    index = np.repeat(np.arange(B // 8), 8)
+    want, _ = O.grpo_outcome_advantage(rewards.clone(), mask, index)
+    monkeypatch.setenv("VAMD_GATE_SPIN_LIMIT", "0")
+    adv, _ = compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    torch.cuda.synchronize()
+    got = adv.cpu()
+    bad = torch.isnan(got)
+    assert bad.any(), "with no waiting allowed some workgroup must have given up"
+    assert torch.allclose(got[~bad], want[~bad], rtol=1e-5, atol=1e-6)
+    ws = _cabi.ticket_workspace(4096, dev)
+    assert int(ws[:16640].to(torch.int32).sum()) == 0
+    monkeypatch.delenv("VAMD_GATE_SPIN_LIMIT")
+    adv, _ = compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    assert torch.allclose(adv.cpu(), want, rtol=1e-5, atol=1e-6)
+
+
 def test_gae_multi_turn_fixture_and_errors(dev):
     from verl_amd.trainer.ppo.core_algos import compute_gae_advantage_return
     random.seed(0)
@@ -1508,7 +1576,7 @@ def test_c_abi_chain_replays_from_a_hip_graph(dev):
     def outputs():
         return dict(adv=f(), grad=f(), out=torch.empty(4, device=dev), coef=torch.empty(B, device=dev), gae_adv=f(),
                     gae_ret=f(), vgrad=f(), vout=torch.empty(2, device=dev), vcoef=torch.empty(B, device=dev),
-                    mom=torch.empty(4, dtype=torch.float64, device=dev))
+                    mom=torch.empty(5, dtype=torch.float64, device=dev))
 
     ws = torch.zeros(max(Lb.vamd_group_outcome_advantage_workspace_bytes(B, Lc, G),
                          Lb.vamd_policy_loss_variant_workspace_bytes(B, Lc), Lb.vamd_gae_workspace_bytes(B, Lc),

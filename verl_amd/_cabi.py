@@ -177,7 +177,29 @@ def compute_device(*tensors: torch.Tensor) -> torch.device:
 
 
 def stream_ptr(device: torch.device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """hipStream_t of torch's current stream on `device`, as an integer (one C call, no Stream object)."""
+    index = device.index
+    if index is None:
+        index = torch.cuda.current_device()
+    return torch._C._cuda_getCurrentRawStream(index)
+
+
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(device: torch.device):
+    """Context that makes `device` current for the library call inside it; free when it already is."""
+    if device.index is None or device.index == torch._C._cuda_getDevice():
+        return _NO_GUARD
+    return torch.cuda.device(device)
 
 
 def ptr(t: torch.Tensor | None):
@@ -208,20 +230,31 @@ def ticket_workspace(nbytes: int, device: torch.device) -> torch.Tensor:
 
 def mask_code(mask: torch.Tensor) -> tuple[torch.Tensor, int]:
     """Contiguous mask in one of the element types the kernels read, with its VAMD_MASK_* code."""
-    if mask.dtype == torch.float32:
+    dt = mask.dtype
+    if dt is torch.float32:
         code = MASK_F32
-    elif mask.dtype == torch.int64:
+    elif dt is torch.int64:
         code = MASK_I64
-    elif mask.dtype in (torch.bool, torch.uint8):
+    elif dt is torch.bool or dt is torch.uint8:
         code = MASK_U8
-    elif mask.dtype == torch.int32:
+    elif dt is torch.int32:
         code = MASK_I32
     else:  # fp16 / bf16 / fp64 / int8 / int16: exact in fp32 for 0/1 masks
         mask = mask.to(torch.float32)
         code = MASK_F32
-    return mask.contiguous(), code
+    return (mask if mask.is_contiguous() else mask.contiguous()), code
 
 
 def as_f32(t: torch.Tensor, device: torch.device) -> torch.Tensor:
-    """fp32, contiguous, on `device` (a no-op for tensors that already are)."""
+    """fp32, contiguous, on `device`, detached (the tensor itself when it already is all that: the kernels only
+    take its address)."""
+    if t.dtype is torch.float32 and t.device == device and t.is_contiguous():
+        return t.detach() if t.requires_grad else t
     return t.detach().to(device=device, dtype=torch.float32).contiguous()
+
+
+def on_device(t: torch.Tensor, device: torch.device) -> torch.Tensor:
+    """`t` detached on `device` (itself when it already is)."""
+    if t.device == device:
+        return t.detach() if t.requires_grad else t
+    return t.detach().to(device)

@@ -48,6 +48,12 @@ struct Carver {
 };
 
 int device_cu_count();
+// Workgroups of `threads` threads of `kernel` (no dynamic LDS) that the current device holds at the same time:
+// the grid limit of kernels whose workgroups wait for each other.  Cached per (device, kernel).
+int resident_workgroups(const void* kernel, int threads);
+// Poll limit of the launch-wide rendezvous: VAMD_GATE_SPIN_LIMIT in the environment (tests set 0 to force the
+// timed-out path), else `standard`.
+unsigned gate_spin_limit(unsigned standard);
 
 // mask element -> (weight, member) following masked_sum: weight = (float)m, member = m != 0
 template <class M>

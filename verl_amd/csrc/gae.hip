@@ -1,215 +1,303 @@
-// Generalised Advantage Estimation as a chunked associative scan (one workgroup per sequence).
+// Generalised Advantage Estimation as a chunked associative scan.
 //
-// Reference: compute_gae_advantage_return, verl/trainer/ppo/core_algos.py:214-262.  Walking a
-// row from its last column to its first, a valid step maps the carried state (nv, g) to
-//     nv' = v_t ,   g' = (r_t - v_t) + gamma * nv + gamma*lam * g ,
-// and a masked step leaves it unchanged.  Every step is therefore an affine map
-//     nv' = a nv + b ,  g' = P nv + Q g + R           (a in {0,1})
-// and maps compose associatively, so the recurrence is a prefix "sum" over maps.  A row is cut
-// into segments of 1024 columns walked right to left; inside a segment each of the 256 threads
-// composes its 4 columns, a wavefront scan (lane exchanges) plus an LDS pass over the wavefront totals
-// yields every thread's incoming state, and the thread then replays its 4 columns to emit the
-// advantages.  Loads and stores are float4 and contiguous across the wavefront; four segments are
-// loaded and scanned together, so memory latency, the exchange chain and the workgroup barrier
-// are paid once per 4096 columns.  The workgroup that
-// finishes last folds the per-row masked moments and writes the whitening statistics, so the
-// whole estimator is two launches (scan, then the elementwise whitening).
+// Reference: compute_gae_advantage_return, verl/trainer/ppo/core_algos.py:214-262.  Walking a row from its last
+// column to its first, a valid step maps the carried state (nv, g) to
+//     nv' = v_t ,   g' = (r_t - v_t + gamma nv) + gamma*lam g ,
+// and a masked step leaves it unchanged.  The two halves of the state are scanned one after the other, which keeps
+// what the lanes exchange small:
+//   1. nv entering a column is the value at the nearest valid column to its right: a "most recent flagged value"
+//      scan.  Inside a wavefront it is one ballot, one count-leading-zeros and one lane read; across the 16
+//      (segment, wavefront) pieces of a batch the first 16 lanes of wavefront 0 do the same once.
+//   2. with nv known, delta_t = r_t - v_t + gamma nv_t is data, and g' = gamma*lam g + delta_t (valid) / g (masked)
+//      is a one-variable affine map (Q, R): composing two of them is a multiply and a fused multiply-add.  A
+//      wavefront scans its 64 lane maps with six lane-exchange steps; wavefront 0 scans the 16 piece totals.
+// A row is cut into segments of 1024 columns (256 threads x 4) walked right to left, four segments per batch
+// with all their loads issued together; every thread then replays its 4 columns per segment to emit the advantages.
+//
+// With whitening the whole estimator is ONE launch: every workgroup keeps a record of the masked moments of its
+// rows, the workgroup that arrives last folds them into (mean, rstd) and opens the gate the others wait at, and
+// each workgroup then whitens what it produced -- from registers when it owns a single row of at most 4096 columns
+// (the advantages are then written once), from its own freshly written rows otherwise.
 #include "rowchunk.h"
 
 namespace vamd {
 
-struct Affine {
-  float a, b, P, Q, R;
-};
-
-__device__ __forceinline__ Affine affine_identity() { return Affine{1.f, 0.f, 0.f, 1.f, 0.f}; }
-
-// later o earlier : apply `earlier` first
-__device__ __forceinline__ Affine compose(const Affine& later, const Affine& earlier) {
-  Affine o;
-  o.a = later.a * earlier.a;
-  o.b = fmaf(later.a, earlier.b, later.b);
-  o.P = fmaf(later.P, earlier.a, later.Q * earlier.P);
-  o.Q = later.Q * earlier.Q;
-  o.R = fmaf(later.P, earlier.b, fmaf(later.Q, earlier.R, later.R));
-  return o;
-}
-
-// The map of the lane the pattern names, the identity where there is none (composing with it changes nothing,
-// so the scan needs no lane test).
-template <int CTRL, int ROW_MASK = 0xF>
-__device__ __forceinline__ Affine dpp_affine(const Affine& x) {
-  Affine o;
-  o.a = dpp_f32<CTRL, ROW_MASK>(x.a, 1.f);
-  o.b = dpp_f32<CTRL, ROW_MASK>(x.b, 0.f);
-  o.P = dpp_f32<CTRL, ROW_MASK>(x.P, 0.f);
-  o.Q = dpp_f32<CTRL, ROW_MASK>(x.Q, 1.f);
-  o.R = dpp_f32<CTRL, ROW_MASK>(x.R, 0.f);
-  return o;
-}
-// Inclusive scan of the maps over the wavefront (lane 0 first): shifts by 1, 2, 4, 8 inside each row of 16 lanes,
-// then the last lane of row 0 / 2 into rows 1 / 3, then lane 31 into rows 2 and 3.
-__device__ __forceinline__ void wave_scan_step(Affine& x, int step) {
-  switch (step) {
-    case 0: x = compose(x, dpp_affine<0x111>(x)); break;       // row_shr:1
-    case 1: x = compose(x, dpp_affine<0x112>(x)); break;       // row_shr:2
-    case 2: x = compose(x, dpp_affine<0x114>(x)); break;       // row_shr:4
-    case 3: x = compose(x, dpp_affine<0x118>(x)); break;       // row_shr:8
-    case 4: x = compose(x, dpp_affine<0x142, 0xA>(x)); break;  // row_bcast:15 into rows 1 and 3
-    default: x = compose(x, dpp_affine<0x143, 0xC>(x)); break; // row_bcast:31 into rows 2 and 3
-  }
-}
-
-constexpr int kSeg = 1024;  // columns per segment = 256 threads x 4
-constexpr int kSegBatch = 4;  // segments whose loads are issued together (48 KiB in flight per workgroup)
+constexpr int kSeg = 1024;       // columns per segment = 256 threads x 4
+constexpr int kSegBatch = 4;     // segments whose loads are issued together (48 KiB in flight per workgroup)
+constexpr int kPieces = kSegBatch * (kRcThreads / 64);  // (segment, wavefront) pieces of a batch, in walk order
+static_assert(kPieces == 16, "wavefront 0 scans the piece totals inside one row of 16 lanes");
 
 struct GaeWork {
   unsigned* ticket;   // workspace head: zero on entry, zero on exit
-  double* partials;   // per row the 4 masked moments of the raw advantages; slot-major
+  double* partials;   // per workgroup the 4 masked moments of the raw advantages; slot-major
 };
 
-template <bool VEC, class M>
-__global__ __launch_bounds__(kRcThreads) void gae_scan_kernel(const float* __restrict__ rewards,
-                                                              const float* __restrict__ values,
-                                                              const M* __restrict__ mask, int64_t rows, int64_t cols,
-                                                              float gamma, float gl, float* __restrict__ adv,
-                                                              float* __restrict__ ret, GaeWork wk,
-                                                              double* __restrict__ moments, float* __restrict__ stats) {
-  const int64_t row = blockIdx.x;
+// g -> Q g + R
+struct Lin {
+  float Q, R;
+};
+// later o earlier : apply `earlier` first
+__device__ __forceinline__ Lin lin_after(const Lin& later, const Lin& earlier) {
+  return Lin{later.Q * earlier.Q, fmaf(later.Q, earlier.R, later.R)};
+}
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ Lin dpp_lin(const Lin& x) {  // the identity where the pattern names no lane
+  return Lin{dpp_f32<CTRL, ROW_MASK>(x.Q, 1.f), dpp_f32<CTRL, ROW_MASK>(x.R, 0.f)};
+}
+__device__ __forceinline__ void row_scan_lin(Lin& x) {  // inclusive, inside each row of 16 lanes
+  x = lin_after(x, dpp_lin<0x111>(x));  // row_shr:1
+  x = lin_after(x, dpp_lin<0x112>(x));  // row_shr:2
+  x = lin_after(x, dpp_lin<0x114>(x));  // row_shr:4
+  x = lin_after(x, dpp_lin<0x118>(x));  // row_shr:8
+}
+__device__ __forceinline__ void wave_scan_lin_tail(Lin& x) {  // rows -> whole wavefront
+  x = lin_after(x, dpp_lin<0x142, 0xA>(x));  // row_bcast:15 into rows 1 and 3
+  x = lin_after(x, dpp_lin<0x143, 0xC>(x));  // row_bcast:31 into rows 2 and 3
+}
+
+// Among the lanes below `lane` whose bit is set in `flags`, the highest; -1 if none.
+__device__ __forceinline__ int nearest_flagged_below(unsigned long long flags, int lane) {
+  const unsigned long long lower = flags & ((1ull << lane) - 1ull);
+  return lower ? 63 - __clzll((long long)lower) : -1;
+}
+
+struct GaeArgs {
+  const float* rewards;
+  const float* values;
+  const void* mask;
+  int64_t rows, cols;
+  float gamma, gl;
+  float* adv;
+  float* ret;
+  GaeWork wk;
+  double* moments;  // [5]: sum m, sum g m, sum g^2 m, count, 1.0 if the rendezvous timed out
+  float* stats;     // [4]: mean, rstd, shift
+  unsigned spin_limit;
+};
+
+template <bool VEC, class M, bool WHITEN>
+__global__ __launch_bounds__(kRcThreads) void gae_kernel(GaeArgs a) {
+  const M* __restrict__ mask = static_cast<const M*>(a.mask);
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int slot = kRcThreads - 1 - tid;  // thread 0 owns the right-most 4 columns of a segment
-  __shared__ Affine wave_tot[2][kSegBatch][4];
-  __shared__ float carry[2][2];
-  if (tid == 0) {
-    carry[0][0] = 0.f;  // nv
-    carry[0][1] = 0.f;  // g
-  }
-  float m0 = 0, m1 = 0, m2 = 0, mc = 0;  // masked moments of the raw advantages
+  __shared__ float nv_piece_val[kPieces], nv_in_piece[kPieces], g_in_piece[kPieces];
+  __shared__ unsigned nv_piece_flag[kPieces];
+  __shared__ Lin piece_total[kPieces];
+  __shared__ float carry[2];  // nv, g entering the batch
+  const float gamma = a.gamma, gl = a.gl;
+  const int64_t cols = a.cols;
   const int nseg = (int)((cols + kSeg - 1) / kSeg);
-  int par = 0;
-  __syncthreads();
-  for (int top = nseg - 1; top >= 0; top -= kSegBatch) {
-    // issue every load of up to kSegBatch segments before touching any of them
-    float r[kSegBatch][4], v[kSegBatch][4], w[kSegBatch][4];
-    int valid[kSegBatch];
-#pragma unroll
-    for (int b = 0; b < kSegBatch; ++b) {
-      const int seg = top - b;
-      const int64_t c = (int64_t)seg * kSeg + slot * 4;
-      const int64_t left = cols - c;
-      valid[b] = seg < 0 ? 0 : (left >= 4 ? 4 : (left > 0 ? (int)left : 0));
-#pragma unroll
-      for (int e = 0; e < 4; ++e) r[b][e] = v[b][e] = w[b][e] = 0.f;
-      if (valid[b] > 0) {
-        const int64_t i = row * cols + c;
-        ld4<VEC>(rewards, i, valid[b], r[b]);
-        ld4<VEC>(values, i, valid[b], v[b]);
-        ldmask4<VEC>(mask, i, valid[b], w[b]);
-      }
-    }
-    // The segments of the batch are scanned together: their wavefront scans are independent (the
-    // exchanges of the four interleave), and one pass over the 16 wavefront totals in walk order
-    // then gives every thread the state entering its 4 columns of each segment.
-    Affine inc[kSegBatch], exc[kSegBatch];
-#pragma unroll
-    for (int b = 0; b < kSegBatch; ++b) {
-      // this thread's 4 columns as one map (right to left: e = 3 .. 0); segments past the row start
-      // (seg < 0) hold zero masks and stay the identity
-      Affine f = affine_identity();
-#pragma unroll
-      for (int e = 3; e >= 0; --e) {
-        if (w[b][e] != 0.f) {
-          Affine n;
-          n.a = 0.f;
-          n.b = v[b][e];
-          n.P = fmaf(gl, f.P, gamma * f.a);
-          n.Q = gl * f.Q;
-          n.R = fmaf(gamma, f.b, fmaf(gl, f.R, r[b][e] - v[b][e]));
-          f = n;
-        }
-      }
-      inc[b] = f;
-    }
-#pragma unroll
-    for (int step = 0; step < 6; ++step) {
-#pragma unroll
-      for (int b = 0; b < kSegBatch; ++b) wave_scan_step(inc[b], step);
-    }
-#pragma unroll
-    for (int b = 0; b < kSegBatch; ++b) {
-      if (lane == 63) wave_tot[par][b][wave] = inc[b];
-      exc[b] = dpp_affine<0x138>(inc[b]);  // wave_shr:1, the identity into lane 0
-    }
+  // a workgroup that owns one row of a single batch keeps its advantages in registers across the rendezvous
+  const bool held = WHITEN && gridDim.x == a.rows && nseg <= kSegBatch;
+  const bool streaming = streams_past_caches(a.rows * cols);
+  float keep[kSegBatch][4];
+  float m0 = 0, m1 = 0, m2 = 0, mc = 0;  // masked moments of the raw advantages
+
+  for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
     __syncthreads();
-    // walk the wavefront totals in order; remember the state where this thread's wavefront starts
-    float nv = carry[par][0], g = carry[par][1];
-    float nv_in[kSegBatch], g_in[kSegBatch];
+    if (tid == 0) carry[0] = carry[1] = 0.f;
+    for (int top = nseg - 1; top >= 0; top -= kSegBatch) {
+      // issue every load of up to kSegBatch segments before touching any of them
+      float r[kSegBatch][4], v[kSegBatch][4], w[kSegBatch][4];
+      int valid[kSegBatch];
 #pragma unroll
-    for (int b = 0; b < kSegBatch; ++b) {
+      for (int b = 0; b < kSegBatch; ++b) {
+        const int seg = top - b;
+        const int64_t c = (int64_t)seg * kSeg + slot * 4;
+        const int64_t left = cols - c;
+        valid[b] = seg < 0 ? 0 : (left >= 4 ? 4 : (left > 0 ? (int)left : 0));
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        if (k == wave) {
-          nv_in[b] = nv;
-          g_in[b] = g;
+        for (int e = 0; e < 4; ++e) r[b][e] = v[b][e] = w[b][e] = 0.f;
+        if (valid[b] > 0) {
+          const int64_t i = row * cols + c;
+          ld4<VEC>(a.rewards, i, valid[b], r[b], streaming);
+          ld4<VEC>(a.values, i, valid[b], v[b], streaming);
+          ldmask4<VEC>(mask, i, valid[b], w[b], streaming);
         }
-        const Affine t = wave_tot[par][b][k];
-        const float nv2 = fmaf(t.a, nv, t.b);
-        g = fmaf(t.P, nv, fmaf(t.Q, g, t.R));
-        nv = nv2;
       }
-    }
-    if (tid == 0) {
-      carry[par ^ 1][0] = nv;
-      carry[par ^ 1][1] = g;
-    }
+      // ---- 1. nv: the value the thread leaves behind (its lowest valid column), and who is nearest before it
+      float left_val[kSegBatch];
+      int src_lane[kSegBatch];
 #pragma unroll
-    for (int b = 0; b < kSegBatch; ++b) {
-      const int seg = top - b;
-      if (seg < 0) break;
-      nv = fmaf(exc[b].a, nv_in[b], exc[b].b);
-      g = fmaf(exc[b].P, nv_in[b], fmaf(exc[b].Q, g_in[b], exc[b].R));
-      // replay the 4 columns
-      float a_out[4], r_out[4];
+      for (int b = 0; b < kSegBatch; ++b) {
+        bool any = false;
+        float val = 0.f;
 #pragma unroll
-      for (int e = 3; e >= 0; --e) {
-        if (w[b][e] != 0.f) {
-          const float delta = r[b][e] + gamma * nv - v[b][e];
-          g = fmaf(gl, g, delta);
-          nv = v[b][e];
-          m1 += g * w[b][e];
-          m2 += g * g * w[b][e];
-          mc += 1.f;
+        for (int e = 3; e >= 0; --e) {  // selects, not branches: a wavefront's lanes disagree about every column
+          const bool on = w[b][e] != 0.f;
+          any = any || on;
+          val = on ? v[b][e] : val;
         }
-        m0 += w[b][e];
-        a_out[e] = g;
-        r_out[e] = g + v[b][e];
+        left_val[b] = val;
+        const unsigned long long flags = __ballot(any);
+        src_lane[b] = nearest_flagged_below(flags, lane);
+        if (lane == 0) {
+          nv_piece_flag[b * 4 + wave] = flags != 0ull;
+          // the wavefront's last word: its highest flagged lane
+          nv_piece_val[b * 4 + wave] = 0.f;
+        }
+        const int top_lane = flags ? 63 - __clzll((long long)flags) : 0;
+        const float wave_val = __shfl(val, top_lane, 64);
+        if (lane == 0 && flags) nv_piece_val[b * 4 + wave] = wave_val;
       }
-      if (valid[b] > 0) {
-        const int64_t i = row * cols + (int64_t)seg * kSeg + slot * 4;
-        st4<VEC>(adv, i, valid[b], a_out);
-        st4<VEC>(ret, i, valid[b], r_out);
+      __syncthreads();
+      if (wave == 0) {  // nv entering each piece: the nearest flagged piece before it, else the batch's carry
+        const bool mine = lane < kPieces;
+        const bool flagged = mine && nv_piece_flag[mine ? lane : 0] != 0u;
+        const float val = mine ? nv_piece_val[lane] : 0.f;
+        const unsigned long long flags = __ballot(flagged);
+        const int src = nearest_flagged_below(flags, lane);
+        const float from = __shfl(val, src < 0 ? 0 : src, 64);
+        const float c_nv = carry[0];
+        if (mine) nv_in_piece[lane] = src < 0 ? c_nv : from;
+        if (lane == kPieces - 1) carry[0] = flagged ? val : (src < 0 ? c_nv : from);
+      }
+      __syncthreads();
+      // ---- 2. g: the thread's 4 columns as one map; delta replaces the reward in place
+      Lin inc[kSegBatch], exc[kSegBatch];
+#pragma unroll
+      for (int b = 0; b < kSegBatch; ++b) {
+        const float from_lane = __shfl(left_val[b], src_lane[b] < 0 ? 0 : src_lane[b], 64);
+        float nv = src_lane[b] < 0 ? nv_in_piece[b * 4 + wave] : from_lane;
+        Lin f{1.f, 0.f};
+#pragma unroll
+        for (int e = 3; e >= 0; --e) {
+          const bool on = w[b][e] != 0.f;
+          const float delta = fmaf(gamma, nv, r[b][e] - v[b][e]);
+          f.R = on ? fmaf(gl, f.R, delta) : f.R;
+          f.Q = on ? f.Q * gl : f.Q;
+          nv = on ? v[b][e] : nv;
+          r[b][e] = delta;  // read again only where the column is valid
+        }
+        inc[b] = f;
+      }
+#pragma unroll
+      for (int b = 0; b < kSegBatch; ++b) row_scan_lin(inc[b]);
+#pragma unroll
+      for (int b = 0; b < kSegBatch; ++b) wave_scan_lin_tail(inc[b]);
+#pragma unroll
+      for (int b = 0; b < kSegBatch; ++b) {
+        if (lane == 63) piece_total[b * 4 + wave] = inc[b];
+        exc[b] = dpp_lin<0x138>(inc[b]);  // wave_shr:1, the identity into lane 0
+      }
+      __syncthreads();
+      if (wave == 0) {  // g entering each piece
+        Lin t = lane < kPieces ? piece_total[lane] : Lin{1.f, 0.f};
+        row_scan_lin(t);
+        const Lin before = dpp_lin<0x111>(t);  // exclusive: the pieces before this one
+        const float c_g = carry[1];
+        if (lane < kPieces) g_in_piece[lane] = fmaf(before.Q, c_g, before.R);
+        if (lane == kPieces - 1) carry[1] = fmaf(t.Q, c_g, t.R);
+      }
+      __syncthreads();
+#pragma unroll
+      for (int b = 0; b < kSegBatch; ++b) {
+        const int seg = top - b;
+        if (seg < 0) break;
+        float g = fmaf(exc[b].Q, g_in_piece[b * 4 + wave], exc[b].R);
+        float a_out[4], r_out[4];
+#pragma unroll
+        for (int e = 3; e >= 0; --e) {
+          const bool on = w[b][e] != 0.f;
+          g = on ? fmaf(gl, g, r[b][e]) : g;
+          const float gw = on ? g * w[b][e] : 0.f;
+          m1 += gw;
+          m2 = fmaf(g, gw, m2);
+          mc += on ? 1.f : 0.f;
+          m0 += w[b][e];
+          a_out[e] = g;
+          r_out[e] = g + v[b][e];
+        }
+        if (valid[b] > 0) {
+          const int64_t i = row * cols + (int64_t)seg * kSeg + slot * 4;
+          st4<VEC>(a.ret, i, valid[b], r_out, streaming);
+          if (!held) {
+            st4<VEC>(a.adv, i, valid[b], a_out, streaming && !WHITEN);  // with WHITEN: read back after the rendezvous
+          }
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) keep[b][e] = a_out[e];
       }
     }
-    par ^= 1;
   }
+
   __shared__ double smem[16];
   double acc[4] = {m0, m1, m2, mc};
   block_sum<4, kRcThreads>(acc, smem);
-  if (tid == 0) {
-    store_record<4>(wk.partials, row, 0, rows, 1, acc);
-  }
-  if (!last_block_arrives(wk.ticket)) return;
-  // the last row to finish folds the per-row moments and derives the whitening statistics
-  double a[4] = {0, 0, 0, 0};
-  sum_records_strided<4>(wk.partials, rows, a);
-  block_sum<4, kRcThreads>(a, smem);
-  if (tid == 0) {
+  if (tid == 0) store_record<4>(a.wk.partials, blockIdx.x, 0, gridDim.x, 1, acc);
+  const bool last = last_block_arrives(a.wk.ticket);
+  if (last) {  // fold the workgroups' moments, derive the whitening statistics
+    double t[4] = {0, 0, 0, 0};
+    sum_records_strided<4>(a.wk.partials, gridDim.x, t);
+    block_sum<4, kRcThreads>(t, smem);
+    if (tid == 0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) moments[i] = a[i];
-    whiten_stats_from_moments(a[0], a[1], a[2], 1, stats);
+      for (int i = 0; i < 4; ++i) a.moments[i] = t[i];
+      float st[3];
+      whiten_stats_from_moments(t[0], t[1], t[2], 1, st);
+#pragma unroll
+      for (int i = 0; i < 3; ++i) peer_store_f32(a.stats + i, st[i]);
+      if (WHITEN) gate_release(a.wk.ticket);  // waits for the stores above before it opens the gate
+    }
+    __syncthreads();  // the other threads of this workgroup read the statistics next
   }
-  ticket_reset(wk.ticket);
+  if (!WHITEN) {
+    if (last) {
+      if (tid == 0) a.moments[4] = 0.0;
+      ticket_reset(a.wk.ticket);
+    }
+    return;
+  }
+  const bool open = last || gate_wait(a.wk.ticket, a.spin_limit);
+  if (open) {
+    const float mean = peer_load_f32(a.stats), rstd = peer_load_f32(a.stats + 1);
+    if (held) {
+#pragma unroll
+      for (int b = 0; b < kSegBatch; ++b) {
+        const int seg = nseg - 1 - b;
+        const int64_t c = (int64_t)seg * kSeg + slot * 4;
+        const int64_t left = cols - c;
+        const int n_ok = seg < 0 ? 0 : (left >= 4 ? 4 : (left > 0 ? (int)left : 0));
+        if (n_ok <= 0) continue;
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = (keep[b][e] - mean) * rstd;
+        st4<VEC>(a.adv, (int64_t)blockIdx.x * cols + c, n_ok, o, streaming);
+      }
+    } else {  // every thread revisits the 4-column groups it wrote itself
+      for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x)
+        for (int64_t c = (int64_t)slot * 4; c < cols; c += (int64_t)kRcThreads * 4 * 4) {
+          float x[4][4];
+          int n_ok[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int64_t cu = c + (int64_t)u * kRcThreads * 4;
+            const int64_t left = cols - cu;
+            n_ok[u] = left >= 4 ? 4 : (left > 0 ? (int)left : 0);
+            if (n_ok[u] > 0) ld4<VEC>(a.adv, row * cols + cu, n_ok[u], x[u], false);
+          }
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            if (n_ok[u] <= 0) continue;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[u][e] = (x[u][e] - mean) * rstd;
+            st4<VEC>(a.adv, row * cols + c + (int64_t)u * kRcThreads * 4, n_ok[u], x[u], streaming);
+          }
+        }
+    }
+  } else if (held) {  // timed out: leave the raw advantages, the host is told through moments[4]
+#pragma unroll
+    for (int b = 0; b < kSegBatch; ++b) {
+      const int seg = nseg - 1 - b;
+      const int64_t c = (int64_t)seg * kSeg + slot * 4;
+      const int64_t left = cols - c;
+      const int n_ok = seg < 0 ? 0 : (left >= 4 ? 4 : (left > 0 ? (int)left : 0));
+      if (n_ok > 0) st4<VEC>(a.adv, (int64_t)blockIdx.x * cols + c, n_ok, keep[b], streaming);
+    }
+  }
+  const unsigned verdict = gate_depart(a.wk.ticket);
+  if (verdict != 0 && tid == 0) a.moments[4] = verdict > 1 ? 1.0 : 0.0;
 }
 
 }  // namespace vamd
@@ -232,24 +320,44 @@ extern "C" int vamd_gae(const float* rewards, const float* values, const void* m
     return VAMD_EWORKSPACE;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  GaeWork wk;
-  wk.ticket = static_cast<unsigned*>(workspace);
+  GaeArgs a;
+  a.wk.ticket = static_cast<unsigned*>(workspace);
   Carver carve(static_cast<char*>(workspace) + kTicketBytes);
-  wk.partials = carve.take<double>((size_t)batch * 4);
-  double* moments = carve.take<double>(4);
-  float* stats = carve.take<float>(4);
-  double* mom = moments_out ? moments_out : moments;
-  const float gl = (float)((double)gamma * (double)lam);
+  a.wk.partials = carve.take<double>((size_t)batch * 4);
+  double* moments = carve.take<double>(8);
+  a.stats = carve.take<float>(4);
+  a.moments = moments_out ? moments_out : moments;
+  a.rewards = rewards;
+  a.values = values;
+  a.mask = mask;
+  a.rows = batch;
+  a.cols = length;
+  a.gamma = gamma;
+  a.gl = (float)((double)gamma * (double)lam);
+  a.adv = advantages;
+  a.ret = returns;
+  a.spin_limit = gate_spin_limit(kGateSpinLimit);
+  // The workgroups wait for each other before whitening, so the grid never exceeds what the device holds at once;
+  // beyond that a workgroup walks several rows.
+  auto launch = [&](auto kernel) -> int {
+    int64_t grid = batch;
+    if (whiten) {
+      const int64_t cap = resident_workgroups(reinterpret_cast<const void*>(kernel), kRcThreads);
+      if (grid > cap) grid = cap;
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kRcThreads), 0, s, a);
+    return VAMD_OK;
+  };
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(length, {rewards, values, advantages, returns}, mask, sizeof(M));
-    if (vec)
-      hipLaunchKernelGGL((gae_scan_kernel<true, M>), dim3((unsigned)batch), dim3(kRcThreads), 0, s, rewards, values,
-                         static_cast<const M*>(mask), batch, length, gamma, gl, advantages, returns, wk, mom, stats);
-    else
-      hipLaunchKernelGGL((gae_scan_kernel<false, M>), dim3((unsigned)batch), dim3(kRcThreads), 0, s, rewards, values,
-                         static_cast<const M*>(mask), batch, length, gamma, gl, advantages, returns, wk, mom, stats);
+    if (whiten) {
+      if (vec) launch(gae_kernel<true, M, true>);
+      else launch(gae_kernel<false, M, true>);
+    } else {
+      if (vec) launch(gae_kernel<true, M, false>);
+      else launch(gae_kernel<false, M, false>);
+    }
   });
   VAMD_LAUNCH_CHECK();
-  if (whiten) return vamd_affine_by_stats(advantages, stats, batch * length, advantages, stream);
   return VAMD_OK;
 }

@@ -28,11 +28,34 @@ inline int64_t chunks_of(int64_t cols) { return cols <= 0 ? 1 : (cols + kChunk -
 
 inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
+// Streaming hint.  A launch of this many workgroups (4096 columns each: 128 MB per fp32 tensor) touches more than the
+// caches hold, so nothing it reads or writes will be found there again: its loads and stores are issued non-temporal,
+// which on this part is worth 7 - 9 % of HBM bandwidth (two-tensor read 6.3 -> 6.9 TB/s, four-in one-out
+// 5.5 -> 6.2 TB/s at 128 MB per tensor).  Smaller launches keep the default policy: their tensors (8 MB at the
+// benchmark size) are usually still cached from the kernel that produced them, and are read again by the next one.
+// The test is uniform over the launch, so it costs one scalar branch per access.
+// Kernels whose grid is not one workgroup per 4096 columns pass the flag themselves (streams_past_caches(elements)).
+constexpr unsigned kStreamingGrid = 8192;
+__device__ __forceinline__ bool launch_streams_past_caches() { return gridDim.x >= kStreamingGrid; }
+__device__ __forceinline__ bool streams_past_caches(int64_t elements) {
+  return elements >= (int64_t)kStreamingGrid * 4096;
+}
+
+typedef float nt_f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned nt_u32x4 __attribute__((ext_vector_type(4)));
+
 template <bool VEC>
-__device__ __forceinline__ void ld4(const float* __restrict__ p, int64_t i, int valid, float (&x)[4]) {
+__device__ __forceinline__ void ld4(const float* __restrict__ p, int64_t i, int valid, float (&x)[4],
+                                    bool streaming = launch_streams_past_caches()) {
   if constexpr (VEC) {
-    const float4 v = *reinterpret_cast<const float4*>(p + i);
-    x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    // the two loads are kept apart on purpose (a branch, not a select): merged into one they lose the hint
+    if (streaming) {
+      const nt_f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const nt_f32x4*>(p + i));
+      x[0] = v[0]; x[1] = v[1]; x[2] = v[2]; x[3] = v[3];
+    } else {
+      const float4 v = *reinterpret_cast<const float4*>(p + i);
+      x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    }
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e) x[e] = e < valid ? p[i + e] : 0.f;
@@ -40,22 +63,48 @@ __device__ __forceinline__ void ld4(const float* __restrict__ p, int64_t i, int 
 }
 
 template <bool VEC>
-__device__ __forceinline__ void st4(float* __restrict__ p, int64_t i, int valid, const float (&x)[4]) {
+__device__ __forceinline__ void st4(float* __restrict__ p, int64_t i, int valid, const float (&x)[4],
+                                    bool streaming = launch_streams_past_caches()) {
   if constexpr (VEC) {
-    *reinterpret_cast<float4*>(p + i) = make_float4(x[0], x[1], x[2], x[3]);
+    if (streaming) {  // kept apart from the default store by type, or the two are merged and the hint is lost
+      const nt_u32x4 v = {__float_as_uint(x[0]), __float_as_uint(x[1]), __float_as_uint(x[2]), __float_as_uint(x[3])};
+      __builtin_nontemporal_store(v, reinterpret_cast<nt_u32x4*>(p + i));
+    } else {
+      *reinterpret_cast<float4*>(p + i) = make_float4(x[0], x[1], x[2], x[3]);
+    }
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e)
       if (e < valid) p[i + e] = x[e];
   }
 }
-
 // mask -> float weights; elements past `valid` read as 0 (excluded)
 template <bool VEC, class M>
-__device__ __forceinline__ void ldmask4(const M* __restrict__ p, int64_t i, int valid, float (&w)[4]) {
+__device__ __forceinline__ void ldmask4(const M* __restrict__ p, int64_t i, int valid, float (&w)[4],
+                                        bool streaming = launch_streams_past_caches()) {
   if constexpr (VEC) {
     struct alignas(sizeof(M) * 4) Pack { M v[4]; };
-    const Pack k = *reinterpret_cast<const Pack*>(p + i);
+    Pack k;
+    if (streaming) {
+      if constexpr (sizeof(M) == 4 && static_cast<M>(0.5f) != static_cast<M>(0)) {  // fp32 mask: load as integers
+        const nt_u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const nt_u32x4*>(p + i));
+        k = __builtin_bit_cast(Pack, raw);
+      } else if constexpr (sizeof(M) == 4) {  // int32 mask: load as floats (a type the default path does not use)
+        const nt_f32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const nt_f32x4*>(p + i));
+        k = __builtin_bit_cast(Pack, raw);
+      } else if constexpr (sizeof(M) == 8) {
+        struct Two { nt_u32x4 lo, hi; };
+        Two raw;
+        raw.lo = __builtin_nontemporal_load(reinterpret_cast<const nt_u32x4*>(p + i));
+        raw.hi = __builtin_nontemporal_load(reinterpret_cast<const nt_u32x4*>(p + i) + 1);
+        k = __builtin_bit_cast(Pack, raw);
+      } else {
+        const unsigned raw = __builtin_nontemporal_load(reinterpret_cast<const unsigned*>(p + i));
+        k = __builtin_bit_cast(Pack, raw);
+      }
+    } else {
+      k = *reinterpret_cast<const Pack*>(p + i);
+    }
 #pragma unroll
     for (int e = 0; e < 4; ++e) w[e] = static_cast<float>(k.v[e]);
   } else {
@@ -194,6 +243,80 @@ __device__ __forceinline__ bool launch_last_arrives(unsigned* counters) {
 __device__ __forceinline__ void ticket_reset(unsigned* counters) {
   if (threadIdx.x <= ticket_groups())
     __hip_atomic_store(counters + threadIdx.x * (kTicketStride / 4), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Rendezvous of a whole launch, for kernels that need a launch-wide result (whitening statistics, group
+// statistics) before their last pass and would otherwise pay a second launch for it -- which costs as much as
+// streaming 8 MB does.  REQUIREMENT: every workgroup of the launch is resident at the same time; the host side
+// caps the grid at what the device holds (resident_workgroups) and lets workgroups loop over rows beyond that.
+//   arrival   : last_block_arrives() as above; the workgroup it is true in computes the result, publishes it with
+//               device-coherent stores and calls gate_release();
+//   waiting   : the others poll the release word in gate_wait(), at most spin_limit times (a sleep between
+//               polls), so that every wavefront exits whatever happens; false = timed out;
+//   departure : every workgroup calls gate_depart() last; the final one to leave zeroes the counter area, so the
+//               workspace contract (zero on entry, zero on exit) holds, and reports whether anyone timed out.
+// The words live inside the counter area: departures at word 16 of each counter's 256-byte slot, the release flag
+// at word 32 and the timed-out flag at word 48 of slot 0.
+constexpr int kDepartWord = 16, kReleaseWord = 32, kTimedOutWord = 48;
+constexpr unsigned kGateSpinLimit = 1u << 22;  // polls of about half a microsecond: seconds, not forever
+
+__device__ __forceinline__ void gate_release(unsigned* counters) {  // thread 0, after its peer stores
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __hip_atomic_store(counters + kReleaseWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ bool gate_wait(unsigned* counters, unsigned spin_limit) {
+  __shared__ unsigned released;
+  if (threadIdx.x == 0) {
+    unsigned seen = 0;
+    for (unsigned spins = 0;; ++spins) {
+      seen = __hip_atomic_load(counters + kReleaseWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (seen != 0 || spins >= spin_limit) break;
+      __builtin_amdgcn_s_sleep(4);
+    }
+    if (seen == 0) __hip_atomic_store(counters + kTimedOutWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    released = seen;
+  }
+  __syncthreads();
+  return released != 0;
+}
+// Returns, in the workgroup that leaves last only, 1 + (someone timed out); 0 everywhere else.
+__device__ __forceinline__ unsigned gate_depart(unsigned* counters) {
+  __shared__ unsigned verdict;
+  if (threadIdx.x == 0) {
+    const unsigned n = gridDim.x, G = ticket_groups();
+    const unsigned g = blockIdx.x % G;
+    const unsigned members = (n - g + G - 1) / G;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    unsigned v = 0;
+    const unsigned t = __hip_atomic_fetch_add(counters + (1 + g) * (kTicketStride / 4) + kDepartWord, 1u,
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (t == members - 1) {
+      const unsigned t2 = __hip_atomic_fetch_add(counters + kDepartWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (t2 == G - 1)
+        v = 1u + __hip_atomic_load(counters + kTimedOutWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    verdict = v;
+  }
+  __syncthreads();
+  if (verdict != 0) {
+    if (threadIdx.x <= ticket_groups()) {
+      unsigned* slot = counters + threadIdx.x * (kTicketStride / 4);
+      __hip_atomic_store(slot, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(slot + kDepartWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (threadIdx.x == 0) {
+      __hip_atomic_store(counters + kReleaseWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(counters + kTimedOutWord, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  return verdict;
+}
+__device__ __forceinline__ void peer_store_f32(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float peer_load_f32(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Lane exchange inside the vector ALU (data-parallel primitives): a lane without a source in the pattern, or in a

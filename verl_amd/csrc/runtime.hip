@@ -1,7 +1,10 @@
 // Library-wide pieces of the C ABI: version, thread-local error text, cached device facts.
 #include <stdarg.h>
+#include <stdlib.h>
 
+#include <map>
 #include <mutex>
+#include <utility>
 
 #include "common.h"
 
@@ -31,24 +34,65 @@ int device_cu_count() {
   return cached[dev];
 }
 
+int resident_workgroups(const void* kernel, int threads) {
+  static std::mutex mu;
+  static std::map<std::pair<int, const void*>, int> cache;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = cache.find({dev, kernel});
+  if (it != cache.end()) return it->second;
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || per_cu < 1) per_cu = 1;
+  int cus = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 1;
+  const int n = per_cu * cus;
+  cache[{dev, kernel}] = n;
+  return n;
+}
+
+unsigned gate_spin_limit(unsigned standard) {
+  if (const char* e = getenv("VAMD_GATE_SPIN_LIMIT")) {
+    char* end = nullptr;
+    const unsigned long v = strtoul(e, &end, 10);
+    if (end != e) return (unsigned)v;
+  }
+  return standard;
+}
+
 // Plain streaming copy, 16 bytes per lane and grid-stride: the yardstick the memory counters of
-// the other kernels are scaled by.
-__global__ __launch_bounds__(256) void copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, int64_t n16) {
+// the other kernels are scaled by.  STREAM: non-temporal loads and stores, the policy the [B, L] kernels use for
+// tensors beyond the caches.
+typedef unsigned ys_u32x4 __attribute__((ext_vector_type(4)));
+typedef float ys_f32x4 __attribute__((ext_vector_type(4)));
+template <bool STREAM>
+__global__ __launch_bounds__(256) void copy_kernel(const ys_u32x4* __restrict__ src, ys_u32x4* __restrict__ dst, int64_t n16) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) {
+    if (STREAM) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+    else dst[i] = src[i];
+  }
 }
 
 // out = a + b + c + d, 16 bytes per lane from each input: the traffic of a fused loss kernel with its gradient
 // (four tensors in, one out) without any of its arithmetic or its reduction, as a second yardstick.
-__global__ __launch_bounds__(256) void sum4_kernel(const float4* __restrict__ a, const float4* __restrict__ b,
-                                                   const float4* __restrict__ c, const float4* __restrict__ d,
-                                                   float4* __restrict__ out, int64_t n4) {
+template <bool STREAM>
+__global__ __launch_bounds__(256) void sum4_kernel(const ys_f32x4* __restrict__ a, const ys_f32x4* __restrict__ b,
+                                                   const ys_f32x4* __restrict__ c, const ys_f32x4* __restrict__ d,
+                                                   ys_f32x4* __restrict__ out, int64_t n4) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += stride) {
-    const float4 x = a[i], y = b[i], z = c[i], w = d[i];
-    out[i] = make_float4(x.x + y.x + z.x + w.x, x.y + y.y + z.y + w.y, x.z + y.z + z.z + w.z, x.w + y.w + z.w + w.w);
+    if (STREAM) {
+      const ys_f32x4 x = __builtin_nontemporal_load(a + i), y = __builtin_nontemporal_load(b + i),
+                     z = __builtin_nontemporal_load(c + i), w = __builtin_nontemporal_load(d + i);
+      __builtin_nontemporal_store(x + y + z + w, out + i);
+    } else {
+      out[i] = a[i] + b[i] + c[i] + d[i];
+    }
   }
 }
+
+constexpr int64_t kStreamingBytes = 128ll << 20;  // per tensor: the size from which the [B, L] kernels stream
 
 }  // namespace vamd
 
@@ -61,8 +105,12 @@ extern "C" int vamd_copy_bytes(const void* src, void* dst, int64_t bytes, void* 
   int64_t blocks = (n16 + 255) / 256;
   const int64_t cap = (int64_t)device_cu_count() * 16;
   if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL(copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const uint4*)src,
-                     (uint4*)dst, n16);
+  if (bytes >= kStreamingBytes)
+    hipLaunchKernelGGL(copy_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const ys_u32x4*)src, (ys_u32x4*)dst, n16);
+  else
+    hipLaunchKernelGGL(copy_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const ys_u32x4*)src, (ys_u32x4*)dst, n16);
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }
@@ -78,8 +126,12 @@ extern "C" int vamd_sum4(const float* a, const float* b, const float* c, const f
   int64_t blocks = (n4 + 255) / 256;
   const int64_t cap = (int64_t)device_cu_count() * 16;
   if (blocks > cap) blocks = cap;
-  hipLaunchKernelGGL(sum4_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const float4*)a,
-                     (const float4*)b, (const float4*)c, (const float4*)d, (float4*)out, n4);
+  if (n * 4 >= kStreamingBytes)
+    hipLaunchKernelGGL(sum4_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const ys_f32x4*)a, (const ys_f32x4*)b, (const ys_f32x4*)c, (const ys_f32x4*)d, (ys_f32x4*)out, n4);
+  else
+    hipLaunchKernelGGL(sum4_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const ys_f32x4*)a, (const ys_f32x4*)b, (const ys_f32x4*)c, (const ys_f32x4*)d, (ys_f32x4*)out, n4);
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
 }

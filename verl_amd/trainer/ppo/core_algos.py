@@ -135,7 +135,7 @@ def _matrix(t: torch.Tensor, dev: torch.device) -> torch.Tensor:
 
 
 def _mask_matrix(mask: torch.Tensor, dev: torch.device, shape) -> tuple[torch.Tensor, int]:
-    m, code = _cabi.mask_code(mask.detach().to(dev))
+    m, code = _cabi.mask_code(_cabi.on_device(mask, dev))
     if m.dim() == 1:
         m = m.view(1, -1)
     assert tuple(m.shape) == tuple(shape), f"mask shape {tuple(mask.shape)} does not match {tuple(shape)}"
@@ -161,14 +161,18 @@ def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torc
         B, Lc = r.shape
         adv = torch.empty_like(r)
         ret = torch.empty_like(r)
-        mom = torch.empty(4, dtype=torch.float64, device=dev)
+        mom = torch.empty(5, dtype=torch.float64, device=dev)
         Lb = _cabi.lib()
         ws = _cabi.ticket_workspace(Lb.vamd_gae_workspace_bytes(B, Lc), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_gae(r.data_ptr(), v.data_ptr(), m.data_ptr(), code, B, Lc, float(gamma), float(lam),
                                     1, adv.data_ptr(), ret.data_ptr(), mom.data_ptr(), ws.data_ptr(), ws.numel(),
                                     _cabi.stream_ptr(dev)))
-        verl_F._raise_on_tiny_mask(float(mom[0].item()))
+        mom_host = mom.tolist()
+        verl_F._raise_on_tiny_mask(mom_host[0])
+        if mom_host[4] != 0.0:
+            raise RuntimeError("vamd_gae: the workgroups' bounded wait for the whitening statistics ran out; "
+                               "the advantages were left unwhitened")
         out_dev = token_level_rewards.device
         return adv.view(token_level_rewards.shape).to(out_dev), ret.view(token_level_rewards.shape).to(out_dev)
 
@@ -186,7 +190,7 @@ def _grpo(token_level_rewards, response_mask, index, epsilon, norm_adv_by_std_in
         adv = torch.empty_like(r)
         Lb = _cabi.lib()
         ws = _cabi.ticket_workspace(Lb.vamd_grpo_workspace_bytes(B, Lc, G), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_grpo_advantage(r.data_ptr(), m.data_ptr(), code, ids.data_ptr(), B, Lc, G,
                                                float(epsilon), int(bool(norm_adv_by_std_in_grpo)), std_mode,
                                                adv.data_ptr(), None, ws.data_ptr(), ws.numel(),
@@ -244,7 +248,7 @@ def _group_outcome(token_level_rewards, response_mask, index, estimator: str, ep
         adv = torch.empty_like(r)
         Lb = _cabi.lib()
         ws = _cabi.ticket_workspace(Lb.vamd_group_outcome_advantage_workspace_bytes(B, Lc, G), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             s = _cabi.stream_ptr(dev)
             _cabi.check(Lb.vamd_group_outcome_advantage(r.data_ptr(), m.data_ptr(), code, ids.data_ptr(), B, Lc, G,
                                                         _ADV[estimator], float(epsilon), int(bool(norm_by_std)), 0,
@@ -330,7 +334,7 @@ def _returns_advantage(token_level_rewards, response_mask, mode: int, gamma: flo
         mom = torch.empty(4, dtype=torch.float64, device=dev)
         Lb = _cabi.lib()
         ws = _cabi.ticket_workspace(Lb.vamd_returns_advantage_workspace_bytes(B, Lc), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_returns_advantage(r.data_ptr(), m.data_ptr(), code, _cabi.ptr(base), B, Lc,
                                                   float(gamma), mode, adv.data_ptr(), ret.data_ptr(), mom.data_ptr(),
                                                   ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
@@ -407,7 +411,7 @@ def _optimal_token_baseline(token_level_rewards, response_mask, index, old_log_p
         ret = torch.empty_like(r)
         Lb = _cabi.lib()
         ws = _cabi.workspace(Lb.vamd_otb_advantage_workspace_bytes(B, Lc, int(packed)), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_otb_advantage(r.data_ptr(), m.data_ptr(), code, lp.data_ptr(), q.data_ptr(),
                                               _cabi.ptr(isw), _cabi.ptr(rows_t), _cabi.ptr(offs_t), _cabi.ptr(tail),
                                               B, Lc, G, int(packed), float(epsilon), adv.data_ptr(), ret.data_ptr(),
@@ -473,7 +477,7 @@ class _AggLoss(torch.autograd.Function):
         out = torch.empty((), dtype=torch.float32, device=dev)
         coef = torch.empty(rows, dtype=torch.float32, device=dev)
         ws = _cabi.ticket_workspace(Lb.vamd_agg_loss_workspace_bytes(rows, cols), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_agg_loss_forward(x.data_ptr(), m.data_ptr(), code, rows, cols, mode, dp_size, bnt,
                                                  gbs, lsf, out.data_ptr(), coef.data_ptr(), ws.data_ptr(),
                                                  ws.numel(), _cabi.stream_ptr(dev)))
@@ -491,7 +495,7 @@ class _AggLoss(torch.autograd.Function):
         rows, cols = m.shape
         g = torch.empty((rows, cols), dtype=torch.float32, device=dev)
         d = _cabi.as_f32(d_loss, dev).reshape(1)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(_cabi.lib().vamd_agg_loss_backward(d.data_ptr(), coef.data_ptr(), m.data_ptr(), ctx.code,
                                                            rows, cols, g.data_ptr(), _cabi.stream_ptr(dev)))
         g = g.view(ctx.in_shape).to(device=ctx.in_device, dtype=ctx.in_dtype)
@@ -529,7 +533,7 @@ class _PolicyLoss(torch.autograd.Function):
         coef = torch.empty(rows, dtype=torch.float32, device=dev)
         g = torch.empty_like(lp) if need_grad else None
         ws = _cabi.ticket_workspace(Lb.vamd_policy_loss_variant_workspace_bytes(rows, cols), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_policy_loss_variant_forward(variant, old.data_ptr(), lp.data_ptr(), adv.data_ptr(),
                                                             m.data_ptr(), code, _cabi.ptr(isw), rows, cols, clip_low,
                                                             clip_high, clip_c, tau_pos, tau_neg, mode, dp_size, bnt,
@@ -551,7 +555,7 @@ class _PolicyLoss(torch.autograd.Function):
         rows, cols = g.shape
         d = _cabi.as_f32(d_loss, dev).reshape(1)
         res = torch.empty_like(g)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(_cabi.lib().vamd_scale_rows(g.data_ptr(), coef.data_ptr(), d.data_ptr(), 1.0, rows, cols,
                                                     res.data_ptr(), _cabi.stream_ptr(dev)))
         res = res.view(ctx.in_shape).to(device=ctx.in_device, dtype=ctx.in_dtype)
@@ -692,7 +696,7 @@ class _CovLoss(torch.autograd.Function):
         g = torch.empty_like(lp) if need_grad else None
         selected = torch.empty((rows, cols), dtype=torch.uint8, device=dev) if want_selected else None
         ws = _cabi.workspace(Lb.vamd_policy_loss_cov_workspace_bytes(rows, cols), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_policy_loss_cov_forward(kind, old.data_ptr(), lp.data_ptr(), adv.data_ptr(),
                                                         m.data_ptr(), code, _cabi.ptr(isw), rows, cols, clip_low,
                                                         clip_high, cov_lb, cov_ub, ratio, kl_coef, seed, mode,
@@ -719,7 +723,7 @@ class _CovLoss(torch.autograd.Function):
         rows, cols = g.shape
         d = _cabi.as_f32(d_loss, dev).reshape(1)
         res = torch.empty_like(g)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(_cabi.lib().vamd_scale_rows(g.data_ptr(), coef.data_ptr(), d.data_ptr(), 1.0, rows, cols,
                                                     res.data_ptr(), _cabi.stream_ptr(dev)))
         return (res.view(ctx.in_shape).to(device=ctx.in_device, dtype=ctx.in_dtype),) + (None,) * 18
@@ -899,7 +903,7 @@ class _ValueLoss(torch.autograd.Function):
         coef = torch.empty(rows, dtype=torch.float32, device=dev)
         g = torch.empty_like(vp) if need_grad else None
         ws = _cabi.ticket_workspace(Lb.vamd_value_loss_workspace_bytes(rows, cols), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_value_loss_forward(vp.data_ptr(), ret.data_ptr(), val.data_ptr(), m.data_ptr(), code,
                                                    rows, cols, cliprange_value, mode, out.data_ptr(), _cabi.ptr(g),
                                                    coef.data_ptr(), ws.data_ptr(), ws.numel(),
@@ -920,7 +924,7 @@ class _ValueLoss(torch.autograd.Function):
         rows, cols = g.shape
         d = _cabi.as_f32(d_loss, dev).reshape(1)
         res = torch.empty_like(g)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(_cabi.lib().vamd_scale_rows(g.data_ptr(), coef.data_ptr(), d.data_ptr(), 0.5, rows, cols,
                                                     res.data_ptr(), _cabi.stream_ptr(dev)))
         res = res.view(ctx.in_shape).to(device=ctx.in_device, dtype=ctx.in_dtype)
@@ -959,7 +963,7 @@ class _KlPenalty(torch.autograd.Function):
         need_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
         kld = torch.empty_like(lp)
         g = torch.empty_like(lp) if need_grad else None
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(_cabi.lib().vamd_kl_penalty(lp.data_ptr(), ref.data_ptr(), lp.numel(), kind,
                                                     int(straight_through), kld.data_ptr(), _cabi.ptr(g),
                                                     _cabi.stream_ptr(dev)))
@@ -1009,7 +1013,7 @@ class _KlLoss(torch.autograd.Function):
         coef = torch.empty(rows, dtype=torch.float32, device=dev)
         g = torch.empty_like(lp) if need_grad else None
         ws = _cabi.ticket_workspace(Lb.vamd_kl_loss_workspace_bytes(rows, cols), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_kl_loss_forward(lp.data_ptr(), ref.data_ptr(), m.data_ptr(), code, rows, cols, kind,
                                                 int(straight_through), mode, dp, bnt, gbs, lsf, out.data_ptr(),
                                                 _cabi.ptr(g), coef.data_ptr(), ws.data_ptr(), ws.numel(),
@@ -1028,7 +1032,7 @@ class _KlLoss(torch.autograd.Function):
         rows, cols = g.shape
         d = _cabi.as_f32(d_loss, dev).reshape(1)
         res = torch.empty_like(g)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(_cabi.lib().vamd_scale_rows(g.data_ptr(), coef.data_ptr(), d.data_ptr(), 1.0, rows, cols,
                                                     res.data_ptr(), _cabi.stream_ptr(dev)))
         res = res.view(ctx.in_shape).to(device=ctx.in_device, dtype=ctx.in_dtype)
@@ -1068,7 +1072,7 @@ def kl_penalised_rewards(token_level_scores: torch.Tensor, old_log_probs: torch.
         kl = torch.empty(1, dtype=torch.float32, device=dev)
         Lb = _cabi.lib()
         ws = _cabi.ticket_workspace(Lb.vamd_apply_kl_penalty_workspace_bytes(rows, cols), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_apply_kl_penalty(sc.data_ptr(), lp.data_ptr(), rf.data_ptr(), m.data_ptr(), code,
                                                  rows, cols, _kl_kind(kl_penalty), float(beta), out.data_ptr(),
                                                  kl.data_ptr(), ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))

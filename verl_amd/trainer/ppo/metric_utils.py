@@ -62,7 +62,7 @@ def compute_data_metrics(batch, use_critic: bool = True) -> dict[str, Any]:
     out = torch.empty(len(_SLOTS), dtype=torch.float64, device=dev)
     Lb = _cabi.lib()
     ws = _cabi.workspace(Lb.vamd_data_metrics_workspace_bytes(rows, width), dev)
-    with torch.cuda.device(dev):
+    with _cabi.device_guard(dev):
         _cabi.check(Lb.vamd_data_metrics(tensors[0].data_ptr(), tensors[1].data_ptr(), tensors[2].data_ptr(),
                                          tensors[3].data_ptr(), _cabi.ptr(values), mask.data_ptr(), mcode,
                                          attention.data_ptr(), acode, rows, prompt, width, out.data_ptr(),
@@ -110,7 +110,7 @@ def compute_variance_proxy_metrics(batch, gradient_norm: float = None) -> dict[s
     Lb = _cabi.lib()
     chunks = int(Lb.vamd_rollout_rs_chunks(cols))
     rec = torch.empty(5 * chunks * rows, dtype=torch.float64, device=dev)
-    with torch.cuda.device(dev):
+    with _cabi.device_guard(dev):
         _cabi.check(Lb.vamd_variance_proxy_rows(adv.data_ptr(), lp.data_ptr(), pi2.data_ptr(), _cabi.ptr(isw),
                                                 mask.data_ptr(), code, rows, cols, rec.data_ptr(),
                                                 _cabi.stream_ptr(dev)))

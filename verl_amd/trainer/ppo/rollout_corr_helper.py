@@ -44,14 +44,14 @@ def _run(old_log_prob, rollout_log_prob, response_mask, level, threshold, batch_
         roll = None
         if rollout_log_prob is not None:
             roll = _cabi.as_f32(rollout_log_prob, dev).view(old.shape)
-        mask, code = _cabi.mask_code(response_mask.detach().to(dev))
+        mask, code = _cabi.mask_code(_cabi.on_device(response_mask, dev))
         mask = mask.view(old.shape)
         rows, cols = old.shape
         weights = torch.empty_like(old) if level else None
         out = torch.empty(len(_SLOTS), dtype=torch.float64, device=dev)
         Lb = _cabi.lib()
         ws = _cabi.workspace(Lb.vamd_rollout_correction_workspace_bytes(rows, cols), dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_rollout_correction(old.data_ptr(), _cabi.ptr(roll), mask.data_ptr(), code, rows, cols,
                                                    level, float(threshold or 0.0), int(bool(batch_normalize)),
                                                    _cabi.ptr(weights), out.data_ptr(), ws.data_ptr(), ws.numel(),
@@ -244,7 +244,7 @@ def _rejection(old_log_prob, rollout_log_prob, response_mask, rollout_rs, rollou
         if old.dim() == 1:
             old = old.view(1, -1)
         roll = _cabi.as_f32(rollout_log_prob, dev).view(old.shape)
-        mask, code = _cabi.mask_code(response_mask.detach().to(dev))
+        mask, code = _cabi.mask_code(_cabi.on_device(response_mask, dev))
         mask = mask.view(old.shape)
         rows, cols = old.shape
         Lb = _cabi.lib()
@@ -252,7 +252,7 @@ def _rejection(old_log_prob, rollout_log_prob, response_mask, rollout_rs, rollou
         stream = _cabi.stream_ptr(dev)
         # pass 1: per-sequence sums and maxima of the three estimates
         rec = torch.empty(6 * chunks * rows, dtype=torch.float64, device=dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_rollout_rs_row_stats(old.data_ptr(), roll.data_ptr(), mask.data_ptr(), code, rows, cols,
                                                      rec.data_ptr(), stream))
         table = _records(rec, 6, chunks, rows)                 # host sync 1
@@ -298,7 +298,7 @@ def _rejection(old_log_prob, rollout_log_prob, response_mask, rollout_rs, rollou
         est_arr = (ctypes.c_int * 3)(*[_ESTIMATOR[t[1]] for t in token_opts], *([0] * (3 - n_tok)))
         lo_arr = (ctypes.c_float * 3)(*[t[2] for t in token_opts], *([0.0] * (3 - n_tok)))
         hi_arr = (ctypes.c_float * 3)(*[t[3] for t in token_opts], *([0.0] * (3 - n_tok)))
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(Lb.vamd_rollout_rs_apply(old.data_ptr(), roll.data_ptr(), mask.data_ptr(), code, rows, cols,
                                                  keep_dev.data_ptr(), n_tok, ctypes.addressof(est_arr),
                                                  ctypes.addressof(lo_arr), ctypes.addressof(hi_arr),

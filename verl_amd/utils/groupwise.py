@@ -78,7 +78,7 @@ def as_torch_index(index: Any, device: torch.device | str | None = None) -> torc
 
 
 def contiguous_group_ids(index: Any, vectorized: bool = False) -> tuple[torch.Tensor, int]:
-    """Labels -> ids ``0..G-1`` in order of first appearance (CPU int64) and ``G``.  Group membership is decided
+    """Labels -> ids ``0..G-1`` (CPU int64) and ``G``.  Group membership is decided
     by Python equality of the labels, as in the reference's ``id2score[index[i]]`` dictionaries
     (verl/trainer/ppo/core_algos.py:305-312); nothing downstream depends on which id a group gets.
     ``vectorized``: membership as the reference's vectorised estimators see it, i.e. equality of the
@@ -86,14 +86,16 @@ def contiguous_group_ids(index: Any, vectorized: bool = False) -> tuple[torch.Te
     if vectorized:
         index = as_torch_index(index)
     if isinstance(index, torch.Tensor):
-        labels = index.detach().reshape(-1).cpu().tolist()
-    elif isinstance(index, np.ndarray):
-        labels = index.reshape(-1).tolist()
-    else:
-        labels = list(index)
+        index = index.detach().reshape(-1).cpu().numpy()
+    if isinstance(index, np.ndarray) and index.dtype.kind in "iub":
+        # plain integers: equality is integer equality, and numpy factorises them without a Python loop (the ids then
+        # follow the sorted labels instead of their first appearance, which no caller can tell apart)
+        uniq, inverse = np.unique(index.reshape(-1), return_inverse=True)
+        return torch.from_numpy(np.ascontiguousarray(inverse.reshape(-1), dtype=np.int64)), int(uniq.size)
+    labels = index.reshape(-1).tolist() if isinstance(index, np.ndarray) else list(index)
     table: dict = {}
-    ids = np.fromiter((table.setdefault(k, len(table)) for k in labels), dtype=np.int64, count=len(labels))
-    return torch.from_numpy(ids), len(table)
+    ids = [table.setdefault(k, len(table)) for k in labels]
+    return torch.tensor(ids, dtype=torch.int64), len(table)
 
 
 @torch.no_grad()
@@ -122,7 +124,7 @@ def group_mean_std(scores: torch.Tensor, gidx: torch.Tensor, eps: float = 1e-6,
     mean = torch.empty(G, dtype=torch.float32, device=dev)
     std = torch.empty(G, dtype=torch.float32, device=dev)
     cnt = torch.empty(G, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _cabi.device_guard(dev):
         _cabi.check(_cabi.lib().vamd_group_mean_std(s.data_ptr(), g.data_ptr(), s.numel(), G, float(eps),
                                                     mean.data_ptr(), std.data_ptr(), cnt.data_ptr(),
                                                     _cabi.stream_ptr(dev)))

@@ -80,7 +80,7 @@ def efficient_entropy_forward(hidden, weight, labels, reduction: int = 0, temper
         assert sum_pi_squared.shape == (n,) and sum_pi_squared.dtype == torch.float32
         assert sum_pi_squared.is_contiguous() and sum_pi_squared.device == dev
     ws = _cabi.workspace(L.vamd_lce_forward_workspace_bytes(n, h, v), dev)
-    with torch.cuda.device(dev):
+    with _cabi.device_guard(dev):
         _cabi.check(L.vamd_lce_forward(hidden.data_ptr(), weight.data_ptr(), labels.data_ptr(), n, h, v,
                                        1.0 / temperature, logprobs.data_ptr(), entropy.data_ptr(), lse.data_ptr(),
                                        mean_z.data_ptr(), _cabi.ptr(logits_cache), _cabi.ptr(sum_pi_squared),
@@ -159,7 +159,7 @@ def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse,
     if d_weight is not None:
         assert d_weight.shape == weight.shape and d_weight.dtype == weight.dtype and d_weight.is_contiguous()
     ws = _cabi.workspace(L.vamd_lce_backward_workspace_bytes(n, h, v, vocab_chunk), dev)
-    with torch.cuda.device(dev):
+    with _cabi.device_guard(dev):
         _cabi.check(L.vamd_lce_backward(hidden.data_ptr(), weight.data_ptr(), labels.data_ptr(), n, h, v,
                                         1.0 / temperature, lse.data_ptr(), mean_z.data_ptr(), _cabi.ptr(dlogprobs),
                                         _cabi.ptr(dentropy), float(d_entropy_scalar), _cabi.ptr(logits_cache),

@@ -23,7 +23,7 @@ class _ResponseWindow(torch.autograd.Function):
             assert t is None or t.numel() == nnz, f"{t.numel()} values for {nnz} token positions"
         outs = [None if t is None else torch.empty((batch, response_length), dtype=torch.float32, device=dev)
                 for t in vals]
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(_cabi.lib().vamd_response_window_scatter(
                 _cabi.ptr(vals[0]), _cabi.ptr(vals[1]), _cabi.ptr(vals[2]), idx.data_ptr(), nnz, batch, seqlen,
                 response_length, _cabi.ptr(outs[0]), _cabi.ptr(outs[1]), _cabi.ptr(outs[2]), _cabi.stream_ptr(dev)))
@@ -45,7 +45,7 @@ class _ResponseWindow(torch.autograd.Function):
             pair = todo[first:first + 2]
             src = [_cabi.as_f32(grads[k], dev).view(batch, width) for k in pair] + [None]
             dst = [torch.empty(nnz, dtype=torch.float32, device=dev) for _ in pair] + [None]
-            with torch.cuda.device(dev):
+            with _cabi.device_guard(dev):
                 _cabi.check(_cabi.lib().vamd_response_window_gather(
                     _cabi.ptr(src[0]), _cabi.ptr(src[1]), idx.data_ptr(), nnz, batch, seqlen, width,
                     _cabi.ptr(dst[0]), _cabi.ptr(dst[1]), _cabi.stream_ptr(dev)))

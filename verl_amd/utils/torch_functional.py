@@ -38,7 +38,7 @@ def _row_stats(rows, ld, labels, want_logprobs: bool, want_entropy: bool, want_m
     dev = rows.device
     f = lambda want: torch.empty(n, dtype=torch.float32, device=dev) if want else None
     logprobs, entropy, lse, mean_z = f(want_logprobs), f(want_entropy), f(True), f(want_mean_z)
-    with torch.cuda.device(dev):
+    with _cabi.device_guard(dev):
         _cabi.check(_cabi.lib().vamd_row_softmax_stats(
             rows.data_ptr(), _ROW_DTYPES[rows.dtype], n, vocab, ld, _cabi.ptr(labels), _cabi.ptr(logprobs),
             _cabi.ptr(entropy), lse.data_ptr(), _cabi.ptr(mean_z), _cabi.stream_ptr(dev)))
@@ -52,7 +52,7 @@ def _row_backward(rows, ld, labels, lse, mean_z, d_logprobs, d_entropy, in_place
     ld_out = ld if in_place else vocab
     g = lambda t: None if t is None else t.detach().reshape(-1).to(device=dev, dtype=torch.float32).contiguous()
     d_logprobs, d_entropy = g(d_logprobs), g(d_entropy)
-    with torch.cuda.device(dev):
+    with _cabi.device_guard(dev):
         _cabi.check(_cabi.lib().vamd_row_softmax_backward(
             rows.data_ptr(), _ROW_DTYPES[rows.dtype], n, vocab, ld, _cabi.ptr(labels), lse.data_ptr(),
             _cabi.ptr(mean_z), _cabi.ptr(d_logprobs), _cabi.ptr(d_entropy), out.data_ptr(), ld_out,
@@ -138,7 +138,7 @@ class _ClipByValue(torch.autograd.Function):
         xs, lo, hi = (to(t).expand(shape).contiguous() for t in (x, tensor_min, tensor_max))
         out = torch.empty_like(xs)
         if xs.numel():
-            with torch.cuda.device(dev):
+            with _cabi.device_guard(dev):
                 _cabi.check(_cabi.lib().vamd_clip_by_value(xs.data_ptr(), lo.data_ptr(), hi.data_ptr(), xs.numel(),
                                                            out.data_ptr(), _cabi.stream_ptr(dev)))
         ctx.save_for_backward(xs, lo, hi)
@@ -162,7 +162,7 @@ class _ClipByValue(torch.autograd.Function):
         need = ctx.needs_input_grad
         outs = [torch.empty_like(xs) if need[i] and ctx.meta[i] is not None else None for i in range(3)]
         if xs.numel() and any(o is not None for o in outs):
-            with torch.cuda.device(dev):
+            with _cabi.device_guard(dev):
                 _cabi.check(_cabi.lib().vamd_clip_by_value_backward(
                     xs.data_ptr(), lo.data_ptr(), hi.data_ptr(), gs.data_ptr(), xs.numel(), _cabi.ptr(outs[0]),
                     _cabi.ptr(outs[1]), _cabi.ptr(outs[2]), _cabi.stream_ptr(dev)))
@@ -185,7 +185,7 @@ def clip_by_value(x: torch.Tensor, tensor_min: torch.Tensor, tensor_max: torch.T
 def _as_matrix(values: torch.Tensor, mask: torch.Tensor, dev: torch.device):
     assert values.shape == mask.shape, f"values {tuple(values.shape)} and mask {tuple(mask.shape)} differ"
     v = _cabi.as_f32(values, dev)
-    m, code = _cabi.mask_code(mask.detach().to(dev))
+    m, code = _cabi.mask_code(_cabi.on_device(mask, dev))
     cols = v.shape[-1] if v.dim() >= 1 and v.numel() > 0 else 1
     rows = v.numel() // max(cols, 1)
     return v.view(rows, cols), m.view(rows, cols), code
@@ -200,7 +200,7 @@ def _moments(values: torch.Tensor, mask: torch.Tensor, per_row: bool) -> torch.T
     out = torch.empty((rows, 4) if per_row else (4,), dtype=torch.float64, device=dev)
     mk, code = _cabi.mask_code(mask)
     ws = _cabi.ticket_workspace(L.vamd_masked_moments_workspace_bytes(rows, cols), dev)
-    with torch.cuda.device(dev):
+    with _cabi.device_guard(dev):
         _cabi.check(L.vamd_masked_moments(values.data_ptr(), mk.data_ptr(), code, rows, cols, int(per_row),
                                           out.data_ptr(), ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
     return out.t() if per_row else out
@@ -261,7 +261,7 @@ class _MaskedReduce(torch.autograd.Function):
         weights = m if m.dtype == torch.float32 else m.to(torch.float32)   # d masked_sum / d values = mask
         one = torch.ones(1, dtype=torch.float32, device=dev)
         res = torch.empty((rows, cols), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _cabi.device_guard(dev):
             _cabi.check(_cabi.lib().vamd_scale_rows(weights.data_ptr(), coef.data_ptr(), one.data_ptr(), 1.0, rows,
                                                     cols, res.data_ptr(), _cabi.stream_ptr(dev)))
         inverse = [0] * len(perm)
@@ -330,7 +330,7 @@ def masked_whiten(values: torch.Tensor, mask: torch.Tensor, shift_mean: bool = T
     L = _cabi.lib()
     stats = torch.empty(4, dtype=torch.float32, device=dev)
     out = torch.empty_like(v)
-    with torch.cuda.device(dev):
+    with _cabi.device_guard(dev):
         s = _cabi.stream_ptr(dev)
         _cabi.check(L.vamd_whiten_stats(mom.data_ptr(), int(shift_mean), stats.data_ptr(), s))
         _cabi.check(L.vamd_affine_by_stats(v.data_ptr(), stats.data_ptr(), v.numel(), out.data_ptr(), s))
