@@ -115,6 +115,12 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
         chk(L.vamd_policy_loss_forward(*P(s, "a", "b", "c", "mask"), 0, None, B, Lc, 0.2, 0.2, 3.0, 0, 1.0, *none3,
                                        out.data_ptr(), *outs, wsp, wsn, st))
 
+    one = torch.ones(1, device=dev)
+
+    def policy_autograd(s):   # what autograd runs: the forward kernel, then the gradient scaled by the upstream scalar
+        policy(s, True)
+        chk(L.vamd_scale_rows(*P(s, "o1"), coef.data_ptr(), one.data_ptr(), 1.0, B, Lc, *P(s, "o2"), st))
+
     def gae(s):
         chk(L.vamd_gae(*P(s, "a", "b", "mask"), 0, B, Lc, 1.0, 0.95, 1, *P(s, "o1", "o2"), mom.data_ptr(), wsp, wsn, st))
 
@@ -167,6 +173,7 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
         "grpo_advantage": (12 * BL, grpo),
         "policy_loss_fwd": (16 * BL, lambda s: policy(s, False)),
         "policy_loss_fwd_grad": (20 * BL, lambda s: policy(s, True)),
+        "policy_loss_fwd_bwd_as_autograd_runs_it": (28 * BL, policy_autograd),   # + read the gradient, write it scaled
         "gae_scan_whiten": (28 * BL, gae),
         "value_loss_fwd_grad": (20 * BL, value),
         "kl_loss_fwd_grad": (16 * BL, kl),
@@ -226,8 +233,8 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
 
 
 def policy_math_chain(dev, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> dict:
-    """GRPO advantage -> policy loss with gradient -> GAE -> value loss with gradient, the per-step chain of the two
-    policy-math benchmark configurations, launched eagerly and replayed from one captured HIP graph (microseconds
+    """GRPO advantage -> policy loss with gradient -> GAE with whitening -> value loss with gradient (one launch
+    each), the per-step chain of the two policy-math benchmark configurations, launched eagerly and replayed from one captured HIP graph (microseconds
     per chain, best of three loops of 50)."""
     import torch
 
@@ -279,7 +286,7 @@ def policy_math_chain(dev, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> 
             best = min(best, e0.elapsed_time(e1) / reps * 1e3)
         return best
 
-    return {"launches_per_chain": 6, "eager_us": timed(chain), "hip_graph_us": timed(graph.replay)}
+    return {"launches_per_chain": 4, "eager_us": timed(chain), "hip_graph_us": timed(graph.replay)}
 
 
 def policy_math_python_path(dev, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> dict:

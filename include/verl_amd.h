@@ -220,6 +220,14 @@ int vamd_clip_by_value_backward(const float* x, const float* lo, const float* hi
 size_t vamd_masked_moments_workspace_bytes(int64_t rows, int64_t cols);
 int vamd_masked_moments(const float* values, const void* mask, int mask_dtype, int64_t rows, int64_t cols,
                         int per_row, double* out, void* workspace, size_t workspace_bytes, void* stream);
+/* The same reduction with the results the callers are after derived in the same launch (each output may be NULL):
+ * moments as above; sum = masked_sum; mean = masked_mean = sum / (sum(mask) + 1e-8); denom = sum(mask) + 1e-8
+ * (fp32, [rows] with per_row != 0, else [1]); whiten_stats [4] = (mean, rsqrt(unbiased var + 1e-8), shift) of
+ * masked_whiten over the whole input (per_row must be 0), ready for vamd_affine_by_stats.  Same workspace as
+ * vamd_masked_moments. */
+int vamd_masked_reduce(const float* values, const void* mask, int mask_dtype, int64_t rows, int64_t cols,
+                       int per_row, double* moments, float* sum, float* mean, float* denom, float* whiten_stats,
+                       int shift_mean, void* workspace, size_t workspace_bytes, void* stream);
 
 /* out[i] = (values[i] - stats[0]) * stats[1] + stats[2], stats being three DEVICE floats
  * (mean, rsqrt(var + 1e-8), re-added mean or 0): the elementwise half of masked_whiten

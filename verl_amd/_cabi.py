@@ -51,6 +51,8 @@ SIGNATURES = {
     "vamd_clip_by_value": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "vamd_clip_by_value_backward": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p,
                                             c_void_p, c_void_p]),
+    "vamd_masked_reduce": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p,
+                                   c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
     "vamd_masked_moments_workspace_bytes": (c_size_t, [c_int64, c_int64]),
     "vamd_masked_moments": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int, c_void_p, c_void_p,
                                     c_size_t, c_void_p]),

@@ -58,12 +58,32 @@ inline bool totals_suffice(int mode) {
 // =============================================================================================
 // masked moments
 // =============================================================================================
+// Where the folded moments go: the four doubles (per row or for the whole launch) and, derived from them in the
+// same launch, the fp32 results the callers are after.
+struct MomentOuts {
+  double* moments;  // [rows][4] or [4]; may be null
+  float* sum;       // [rows] or [1]: masked_sum
+  float* mean;      // [rows] or [1]: masked_mean = sum / (sum(mask) + 1e-8)
+  float* denom;     // [rows] or [1]: sum(mask) + 1e-8 (what the gradient of masked_mean divides by)
+  float* whiten;    // [4], whole launch only: mean, rsqrt(var + 1e-8), shift
+  int shift_mean;
+};
+__device__ __forceinline__ void write_moment_outs(const MomentOuts& o, int64_t at, const double (&a)[4]) {
+  if (o.moments)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o.moments[at * 4 + i] = a[i];
+  const float denom = (float)a[0] + 1e-8f;
+  if (o.sum) o.sum[at] = (float)a[1];
+  if (o.mean) o.mean[at] = (float)a[1] / denom;
+  if (o.denom) o.denom[at] = denom;
+}
+
 template <bool VEC, class M>
 __global__ __launch_bounds__(kRcThreads) void moments_kernel(const float* __restrict__ values,
                                                              const float* __restrict__ minus,
                                                              const M* __restrict__ mask, int64_t rows,
                                                              int64_t cols, int chunks, int per_row, Work wk,
-                                                             double* __restrict__ out) {
+                                                             MomentOuts out) {
   const int64_t row = blockIdx.x / chunks;
   const int chunk = blockIdx.x % chunks;
   const ChunkPos pos(row, chunk, cols);
@@ -99,9 +119,10 @@ __global__ __launch_bounds__(kRcThreads) void moments_kernel(const float* __rest
   if (!per_row) {
     double a[4];
     if (!sum_all_records<4>(wk.ticket, wk.partials, rows, chunks, a, smem)) return;
-    if (threadIdx.x == 0)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) out[i] = a[i];
+    if (threadIdx.x == 0) {
+      write_moment_outs(out, 0, a);
+      if (out.whiten) whiten_stats_from_moments(a[0], a[1], a[2], out.shift_mean, out.whiten);
+    }
     ticket_reset(wk.ticket);
     return;
   }
@@ -114,9 +135,7 @@ __global__ __launch_bounds__(kRcThreads) void moments_kernel(const float* __rest
       fold_row_records<4, 4, 2>(wk.partials, rr, have, rows, chunks, a);
 #pragma unroll
       for (int k = 0; k < 2; ++k)
-        if (have[k])
-#pragma unroll
-          for (int i = 0; i < 4; ++i) out[rr[k] * 4 + i] = a[k][i];
+        if (have[k]) write_moment_outs(out, rr[k], a[k]);
     }
   }
   ticket_reset(wk.ticket);
@@ -1091,22 +1110,35 @@ extern "C" size_t vamd_masked_moments_workspace_bytes(int64_t rows, int64_t cols
 }
 
 static int masked_moments_of_difference(const float* values, const float* minus, const void* mask, int mask_dtype,
-                                        int64_t rows, int64_t cols, int per_row, double* out, void* workspace,
+                                        int64_t rows, int64_t cols, int per_row, MomentOuts out, void* workspace,
                                         size_t workspace_bytes, void* stream);
 
 extern "C" int vamd_masked_moments(const float* values, const void* mask, int mask_dtype, int64_t rows,
                                    int64_t cols, int per_row, double* out, void* workspace, size_t workspace_bytes,
                                    void* stream) {
-  return masked_moments_of_difference(values, nullptr, mask, mask_dtype, rows, cols, per_row, out, workspace,
+  VAMD_REQUIRE(out, "masked_moments: null pointer");
+  return masked_moments_of_difference(values, nullptr, mask, mask_dtype, rows, cols, per_row,
+                                      MomentOuts{out, nullptr, nullptr, nullptr, nullptr, 1}, workspace,
+                                      workspace_bytes, stream);
+}
+
+extern "C" int vamd_masked_reduce(const float* values, const void* mask, int mask_dtype, int64_t rows, int64_t cols,
+                                  int per_row, double* moments, float* sum, float* mean, float* denom,
+                                  float* whiten_stats, int shift_mean, void* workspace, size_t workspace_bytes,
+                                  void* stream) {
+  VAMD_REQUIRE(moments || sum || mean || denom || whiten_stats, "masked_reduce: no output requested");
+  VAMD_REQUIRE(!(per_row && whiten_stats), "masked_reduce: whitening statistics are taken over the whole input");
+  return masked_moments_of_difference(values, nullptr, mask, mask_dtype, rows, cols, per_row,
+                                      MomentOuts{moments, sum, mean, denom, whiten_stats, shift_mean}, workspace,
                                       workspace_bytes, stream);
 }
 
 static int masked_moments_of_difference(const float* values, const float* minus, const void* mask, int mask_dtype,
-                                        int64_t rows, int64_t cols, int per_row, double* out, void* workspace,
+                                        int64_t rows, int64_t cols, int per_row, MomentOuts out, void* workspace,
                                         size_t workspace_bytes, void* stream) {
   int st = check_matrix("masked_moments", rows, cols);
   if (st != VAMD_OK) return st;
-  VAMD_REQUIRE(values && mask && out, "masked_moments: null pointer");
+  VAMD_REQUIRE(values && mask, "masked_moments: null pointer");
   if (!workspace || workspace_bytes < vamd_masked_moments_workspace_bytes(rows, cols)) {
     set_error("masked_moments: workspace too small");
     return VAMD_EWORKSPACE;
@@ -1303,7 +1335,8 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
   pp.nkl_lo = pp.nkl_hi = 0.f;
   if (variant == VAMD_PL_GSPO) {  // sequence-level log-ratio: per-row masked moments of log_prob - old_log_prob
     double* row_moments = reinterpret_cast<double*>(static_cast<char*>(workspace) + reduce_workspace_bytes(rows, cols, 5));
-    st = masked_moments_of_difference(log_prob, old_log_prob, mask, mask_dtype, rows, cols, 1, row_moments, workspace,
+    st = masked_moments_of_difference(log_prob, old_log_prob, mask, mask_dtype, rows, cols, 1,
+                                      MomentOuts{row_moments, nullptr, nullptr, nullptr, nullptr, 1}, workspace,
                                       reduce_workspace_bytes(rows, cols, 5), stream);
     if (st != VAMD_OK) return st;
     pp.row_moments = row_moments;

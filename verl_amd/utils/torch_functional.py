@@ -216,6 +216,51 @@ def _normalise_axis(axis, ndim: int):
     return dims
 
 
+def _reduce_geometry(values, dims):
+    """(perm, kept_shape, rows, cols) that turn ``values`` into the [kept, reduced] matrix of a reduction."""
+    ndim = values.dim()
+    if dims is None:
+        # all elements: keep the tensor's own [leading, last] matrix shape, which spreads the launch over rows
+        cols = values.shape[-1] if ndim else 1
+        return None, (), values.numel() // cols, cols
+    kept = tuple(d for d in range(ndim) if d not in dims)
+    perm = kept + dims
+    if perm == tuple(range(ndim)):
+        perm = None                      # the reduced dimensions are already the trailing ones
+    kept_shape = tuple(values.shape[d] for d in kept)
+    return perm, kept_shape, math.prod(kept_shape), math.prod(values.shape[d] for d in dims)
+
+
+def _masked_reduce_forward(values, mask, dims, mean: bool, want_denom: bool):
+    """One launch: fp32 masked sum or mean over ``dims`` (and the mean's denominator for the backward pass)."""
+    dev = _cabi.compute_device(values, mask)
+    perm, kept_shape, rows, cols = _reduce_geometry(values, dims)
+    v = _cabi.as_f32(values, dev)
+    m = _cabi.on_device(mask, dev)
+    if perm is not None:
+        v, m = v.permute(perm), m.permute(perm)
+    v = v.reshape(rows, cols)
+    m, code = _cabi.mask_code(m.reshape(rows, cols))
+    if not v.is_contiguous():
+        v = v.contiguous()
+    per_row = dims is not None
+    out = torch.empty(rows if per_row else 1, dtype=torch.float32, device=dev)
+    denom = torch.empty_like(out) if (mean and want_denom) else None
+    L = _cabi.lib()
+    ws = _cabi.ticket_workspace(L.vamd_masked_moments_workspace_bytes(rows, cols), dev)
+    with _cabi.device_guard(dev):
+        _cabi.check(L.vamd_masked_reduce(v.data_ptr(), m.data_ptr(), code, rows, cols, int(per_row), None,
+                                         None if mean else out.data_ptr(), out.data_ptr() if mean else None,
+                                         _cabi.ptr(denom), None, 1, ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
+    out_dtype = torch.result_type(values, mask)
+    if not out_dtype.is_floating_point:
+        out_dtype = torch.float32
+    res = out.view(kept_shape)
+    if res.dtype != out_dtype or res.device != values.device:
+        res = res.to(device=values.device, dtype=out_dtype)
+    return res, m, denom, (perm, tuple(values.shape), rows, cols, values.dtype, values.device)
+
+
 class _MaskedReduce(torch.autograd.Function):
     """``masked_sum`` / ``masked_mean`` over any set of dimensions.  The reduced dimensions are moved last and the
     tensor is seen as ``[kept, reduced]``, which the row-wise moments kernel reduces; the gradient is
@@ -223,31 +268,10 @@ class _MaskedReduce(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, values, mask, dims, mean: bool):
-        ndim = values.dim()
-        dev = _cabi.compute_device(values, mask)
-        if dims is None:
-            # all elements: keep the tensor's own [leading, last] matrix shape, which spreads the launch over rows
-            perm, kept_shape = tuple(range(ndim)), ()
-            cols = values.shape[-1] if ndim else 1
-            rows = values.numel() // cols
-        else:
-            kept = tuple(d for d in range(ndim) if d not in dims)
-            perm = kept + dims
-            kept_shape = tuple(values.shape[d] for d in kept)
-            rows = math.prod(kept_shape)
-            cols = math.prod(values.shape[d] for d in dims)
-        v = _cabi.as_f32(values, dev).permute(perm).reshape(rows, cols).contiguous()
-        m, _ = _cabi.mask_code(mask.detach().to(dev).permute(perm).reshape(rows, cols))
-        mom = _moments(v, m, per_row=dims is not None)              # fp64: [4, rows], or [4] for all elements
-        total = mom[1].to(torch.float32)
-        denom = mom[0].to(torch.float32) + 1e-8 if mean else None
-        out = total / denom if mean else total
+        res, m, denom, geometry = _masked_reduce_forward(values, mask, dims, mean, want_denom=True)
         ctx.save_for_backward(m, denom)
-        ctx.geometry = (perm, tuple(values.shape), rows, cols, values.dtype, values.device)
-        out_dtype = torch.result_type(values, mask)
-        if not out_dtype.is_floating_point:
-            out_dtype = torch.float32
-        return out.view(kept_shape).to(device=values.device, dtype=out_dtype)
+        ctx.geometry = geometry
+        return res
 
     @staticmethod
     def backward(ctx, g):
@@ -264,10 +288,13 @@ class _MaskedReduce(torch.autograd.Function):
         with _cabi.device_guard(dev):
             _cabi.check(_cabi.lib().vamd_scale_rows(weights.data_ptr(), coef.data_ptr(), one.data_ptr(), 1.0, rows,
                                                     cols, res.data_ptr(), _cabi.stream_ptr(dev)))
-        inverse = [0] * len(perm)
-        for i, d in enumerate(perm):
-            inverse[d] = i
-        res = res.view([shape[d] for d in perm]).permute(inverse)
+        if perm is None:
+            res = res.view(shape)
+        else:
+            inverse = [0] * len(perm)
+            for i, d in enumerate(perm):
+                inverse[d] = i
+            res = res.view([shape[d] for d in perm]).permute(inverse)
         return res.to(device=device, dtype=dtype), None, None, None
 
 
@@ -277,7 +304,9 @@ def _reduce(values, mask, axis, mean: bool):
     if values.numel() == 0:   # a sum over nothing is 0, and 0 / (0 + 1e-8) is 0
         kept = () if dims is None else tuple(s for d, s in enumerate(values.shape) if d not in dims)
         return torch.zeros(kept, dtype=torch.float32, device=values.device)
-    return _MaskedReduce.apply(values, mask, dims, mean)
+    if values.requires_grad and torch.is_grad_enabled():
+        return _MaskedReduce.apply(values, mask, dims, mean)
+    return _masked_reduce_forward(values, mask, dims, mean, want_denom=False)[0]   # nothing to record: no autograd node
 
 
 def masked_sum(values: torch.Tensor, mask: torch.Tensor, axis=None) -> torch.Tensor:
@@ -324,14 +353,20 @@ def masked_var(values: torch.Tensor, mask: torch.Tensor, unbiased: bool = True) 
 
 
 def masked_whiten(values: torch.Tensor, mask: torch.Tensor, shift_mean: bool = True) -> torch.Tensor:
-    """(values - mean) * rsqrt(var + 1e-8) on every element (reference torch_functional.py:322-339)."""
-    v, mom, dev = _global_moments(values, mask)
-    _raise_on_tiny_mask(float(mom[0].item()))
+    """(values - mean) * rsqrt(var + 1e-8) on every element (reference torch_functional.py:322-339): one launch for
+    the masked moments and the statistics, one for the elementwise pass."""
+    dev = _cabi.compute_device(values, mask)
+    v, m, code = _as_matrix(values, mask, dev)
+    rows, cols = v.shape
     L = _cabi.lib()
+    mom = torch.empty(4, dtype=torch.float64, device=dev)
     stats = torch.empty(4, dtype=torch.float32, device=dev)
     out = torch.empty_like(v)
+    ws = _cabi.ticket_workspace(L.vamd_masked_moments_workspace_bytes(rows, cols), dev)
     with _cabi.device_guard(dev):
         s = _cabi.stream_ptr(dev)
-        _cabi.check(L.vamd_whiten_stats(mom.data_ptr(), int(shift_mean), stats.data_ptr(), s))
+        _cabi.check(L.vamd_masked_reduce(v.data_ptr(), m.data_ptr(), code, rows, cols, 0, mom.data_ptr(), None, None,
+                                         None, stats.data_ptr(), int(shift_mean), ws.data_ptr(), ws.numel(), s))
         _cabi.check(L.vamd_affine_by_stats(v.data_ptr(), stats.data_ptr(), v.numel(), out.data_ptr(), s))
+    _raise_on_tiny_mask(mom[0].item())   # the reference raises here too; the pass above is already queued
     return out.view(values.shape).to(values.device)
