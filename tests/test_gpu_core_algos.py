@@ -299,6 +299,28 @@ def test_grpo_with_more_groups_than_one_workgroup_holds(dev):
         assert torch.equal(got.cpu() == 0, w32 == 0)
 
 
+@pytest.mark.parametrize("B,L", [(96, 9000), (1800, 700), (2100, 5000), (40, 70000)])
+@pytest.mark.parametrize("mask_kind", ["float01", "weights", "bool", "int64"])
+def test_grpo_mask_kinds_over_chunked_and_shared_rows(dev, B, L, mask_kind):
+    """Rows of several chunks, workgroups that own several rows, rows too long to keep their mask between the two
+    passes; masks of every dtype, and a float mask with weights other than 0 and 1, which the reference multiplies
+    through like any other value."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    g = torch.Generator().manual_seed(B + L)
+    index = np.asarray([i % max(B // 6, 1) for i in range(B)], dtype=np.int64)
+    mask01 = (torch.rand(B, L, generator=g) < 0.7).float()
+    mask01[:, 0] = 1.0
+    rewards = torch.randn(B, L, generator=g) * mask01 * 0.1
+    if mask_kind == "weights":
+        mask = mask01 * torch.tensor([0.5, 1.0, 2.0])[torch.randint(0, 3, (B, L), generator=g)]
+    else:
+        mask = {"float01": mask01, "bool": mask01.bool(), "int64": mask01.long()}[mask_kind]
+    want, _ = O.grpo_outcome_advantage(rewards.clone(), mask.float(), index)
+    got, _ = CA.compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    _close(got, want, what=f"grpo {mask_kind} {B}x{L}")
+    assert torch.equal(got.cpu() == 0, want == 0)
+
+
 def test_grpo_nearly_equal_scores_are_held_to_fp64(dev):
     """Two-member groups whose scores nearly coincide: (s - mean) / (std + eps) divides rounding noise by a tiny
     std, and the reference's own fp32 mean / std is then 1e-4 away from the exact value.  The kernel carries the

@@ -51,6 +51,14 @@ int device_cu_count();
 // Workgroups of `threads` threads of `kernel` (no dynamic LDS) that the current device holds at the same time:
 // the grid limit of kernels whose workgroups wait for each other.  Cached per (device, kernel).
 int resident_workgroups(const void* kernel, int threads);
+// Grid for `items` units of work on a kernel whose workgroups wait for each other: at most `resident`, and chosen so
+// that every workgroup walks the same number of items (2048 items on 1536 resident workgroups: 1024 x 2, not
+// 1536 of which a third walk two).
+inline int64_t balanced_waiting_grid(int64_t items, int64_t resident) {
+  if (items <= resident) return items;
+  const int64_t passes = (items + resident - 1) / resident;
+  return (items + passes - 1) / passes;
+}
 // Poll limit of the launch-wide rendezvous: VAMD_GATE_SPIN_LIMIT in the environment (tests set 0 to force the
 // timed-out path), else `standard`.
 unsigned gate_spin_limit(unsigned standard);

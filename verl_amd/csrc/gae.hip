@@ -341,10 +341,7 @@ extern "C" int vamd_gae(const float* rewards, const float* values, const void* m
   // beyond that a workgroup walks several rows.
   auto launch = [&](auto kernel) -> int {
     int64_t grid = batch;
-    if (whiten) {
-      const int64_t cap = resident_workgroups(reinterpret_cast<const void*>(kernel), kRcThreads);
-      if (grid > cap) grid = cap;
-    }
+    if (whiten) grid = balanced_waiting_grid(batch, resident_workgroups(reinterpret_cast<const void*>(kernel), kRcThreads));
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kRcThreads), 0, s, a);
     return VAMD_OK;
   };

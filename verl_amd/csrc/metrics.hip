@@ -58,6 +58,7 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
   float hi[3] = {-__builtin_inff(), -__builtin_inff(), -__builtin_inff()};  // adv, ret, val
   float lo[3] = {__builtin_inff(), __builtin_inff(), __builtin_inff()};
   const int64_t att_row = row * (a.prompt + a.cols) + a.prompt;
+  const bool streaming = streams_past_caches(a.rows * a.cols);  // the grid counts spans of chunks, not chunks
   for (int u = 0; u < a.span; ++u) {
     const ChunkPos pos(row, chunk * a.span + u, a.cols);
     // per-thread partials over its 16 elements in fp32 (exact counts, 1e-7 relative on the sums), widened per chunk
@@ -68,13 +69,13 @@ __global__ __launch_bounds__(kRcThreads) void data_metrics_kernel(DmArgs a, cons
     for (int k = 0; k < kGroups; ++k) {
       if (pos.valid[k] <= 0) continue;
       float sc[4], rw[4], ad[4], rt[4], vl[4] = {0.f, 0.f, 0.f, 0.f}, m[4], at[4];
-      ld4<VEC>(a.scores, pos.idx[k], pos.valid[k], sc);
-      ld4<VEC>(a.rewards, pos.idx[k], pos.valid[k], rw);
-      ld4<VEC>(a.adv, pos.idx[k], pos.valid[k], ad);
-      ld4<VEC>(a.ret, pos.idx[k], pos.valid[k], rt);
-      if (a.val) ld4<VEC>(a.val, pos.idx[k], pos.valid[k], vl);
-      ldmask4<VEC>(mask, pos.idx[k], pos.valid[k], m);
-      ldmask4<VEC>(attention, att_row + (pos.idx[k] - row * a.cols), pos.valid[k], at);
+      ld4<VEC>(a.scores, pos.idx[k], pos.valid[k], sc, streaming);
+      ld4<VEC>(a.rewards, pos.idx[k], pos.valid[k], rw, streaming);
+      ld4<VEC>(a.adv, pos.idx[k], pos.valid[k], ad, streaming);
+      ld4<VEC>(a.ret, pos.idx[k], pos.valid[k], rt, streaming);
+      if (a.val) ld4<VEC>(a.val, pos.idx[k], pos.valid[k], vl, streaming);
+      ldmask4<VEC>(mask, pos.idx[k], pos.valid[k], m, streaming);
+      ldmask4<VEC>(attention, att_row + (pos.idx[k] - row * a.cols), pos.valid[k], at, streaming);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         if (e >= pos.valid[k]) continue;

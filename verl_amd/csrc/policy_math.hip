@@ -924,19 +924,27 @@ __device__ __forceinline__ void grpo_scalars_from_records(const double* __restri
 
 // Small launches let the workgroup that arrives last run the statistics (TAIL); large ones leave them to a launch
 // of their own, whose registers and LDS are then not charged to every wavefront of the streaming pass.
+// `chunks` counts the records per row: a workgroup walks `span` consecutive 4096-column chunks (1 for small
+// launches; for launches of thousands of rows the whole row, so that the records stay few enough for the statistics
+// to run in the same launch).
 template <bool VEC, bool TAIL>
 __global__ __launch_bounds__(kRcThreads) void grpo_rowsum_kernel(const float* __restrict__ x, int64_t cols,
-                                                                 int chunks, Work wk, GrpoArgs ga) {
+                                                                 int chunks, int span, Work wk, GrpoArgs ga) {
   const int64_t row = blockIdx.x / chunks;
   const int chunk = blockIdx.x % chunks;
-  const ChunkPos pos(row, chunk, cols);
-  float v[kGroups][4];
-  load_groups<VEC>(x, pos, v);
-  float s = 0;
+  const bool streaming = streams_past_caches(ga.rows * cols);
+  double total = 0.0;
+  for (int u = 0; u < span; ++u) {
+    const ChunkPos pos(row, chunk * span + u, cols);
+    float v[kGroups][4];
+    load_groups<VEC>(x, pos, v, streaming);
+    float s = 0;
 #pragma unroll
-  for (int g = 0; g < kGroups; ++g) s += (v[g][0] + v[g][1]) + (v[g][2] + v[g][3]);
+    for (int g = 0; g < kGroups; ++g) s += (v[g][0] + v[g][1]) + (v[g][2] + v[g][3]);
+    total += (double)s;
+  }
   __shared__ double smem[4];
-  double acc[1] = {s};
+  double acc[1] = {total};
   block_sum<1, kRcThreads>(acc, smem);
   if constexpr (TAIL) {
     if (threadIdx.x == 0) store_record<1>(wk.partials, row, chunk, ga.rows, chunks, acc);
@@ -990,6 +998,167 @@ __global__ __launch_bounds__(kRcThreads) void grpo_single_launch_kernel(const fl
     for (int e = 0; e < 4; ++e) w[g][e] = open ? w[g][e] * a : a;
   store_groups<VEC>(out, pos, w);
   gate_depart(wk.ticket);
+}
+
+// GRPO proper, up to a few thousand responses, in one launch WITHOUT a serial statistics step: workgroup b owns rows
+// b, b + grid, ...  Pass 1 leaves every row's score (the unmasked row sum, fp32 like the reference's) in memory;
+// the workgroups then meet once (the last arrival opens the gate at once: there is nothing to fold); in pass 2 each
+// workgroup finds the other members of its row's group by comparing the group ids (a few KB, cache-resident),
+// takes the group's mean and unbiased standard deviation from their scores in double, and streams scalar * mask.
+// Every workgroup repeats a little arithmetic, none waits for a single workgroup to do all of it.  A workgroup that
+// owns at most kGrpoHeldSlots chunks keeps its mask as bits in LDS across the meeting and only stores afterwards.
+constexpr int kGrpoHeldSlots = 32;  // chunks of one workgroup whose mask bits stay in LDS (16 KB)
+struct GrpoRowsArgs {
+  const float* rewards;
+  const void* mask;
+  const int64_t* gid;
+  int64_t rows, cols;
+  int chunks;
+  float eps;
+  int norm_by_std, std_mode;
+  float* scores;   // [rows] scratch, written and read through the device-coherent path
+  float* scalars;  // [rows] optional out
+  float* out;
+  unsigned* ticket;
+  unsigned spin_limit;
+};
+
+constexpr int64_t kGrpoRowsLimit = 32 * kRcThreads;  // one membership bit per thread for every 256 responses
+// Bit k set: response k * 256 + threadIdx.x belongs to the group of `row` (no bits for a row past the end).
+__device__ __forceinline__ unsigned grpo_member_bits(const int64_t* __restrict__ gid, int64_t rows, int64_t row) {
+  unsigned bits = 0;
+  if (row < rows) {
+    const int64_t g = gid[row];
+    for (int k = 0; (int64_t)k * kRcThreads + threadIdx.x < rows; ++k)
+      bits |= (gid[(int64_t)k * kRcThreads + threadIdx.x] == g ? 1u : 0u) << k;
+  }
+  return bits;
+}
+
+template <bool VEC, class M>
+__global__ __launch_bounds__(kRcThreads) void grpo_rows_kernel(GrpoRowsArgs a) {
+  const M* __restrict__ mask = static_cast<const M*>(a.mask);
+  const bool streaming = streams_past_caches(a.rows * a.cols);
+  // One bit per mask element this workgroup owns, kept in LDS across the meeting when they fit, so that pass 2 only
+  // stores.  A thread that met a mask value other than 0 and 1 reads its mask again instead.
+  static_assert(kGroups * 4 <= 16, "one 16-bit word per thread and chunk");
+  __shared__ unsigned short held_bits[kGrpoHeldSlots * kRcThreads];
+  const int64_t own_rows = (a.rows - blockIdx.x + gridDim.x - 1) / gridDim.x;
+  const bool held = own_rows * a.chunks <= kGrpoHeldSlots;
+  bool binary = true;
+  int slot = 0;
+  __shared__ double smem[6 * (kRcThreads / 64)];
+  __shared__ double bc[2];
+  float w[kGroups][4];
+  for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
+    double total = 0.0;
+    for (int c = 0; c < a.chunks; ++c) {
+      const ChunkPos pos(row, c, a.cols);
+      float v[kGroups][4];
+      load_groups<VEC>(a.rewards, pos, v, streaming);
+      if (held) {
+        load_mask_groups<VEC>(mask, pos, w, streaming);
+        unsigned bits = 0;
+#pragma unroll
+        for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float m = w[g][e];
+            bits |= (m != 0.f ? 1u : 0u) << (g * 4 + e);
+            binary = binary && (m == 0.f || m == 1.f);
+          }
+        held_bits[slot * kRcThreads + threadIdx.x] = (unsigned short)bits;
+        ++slot;
+      }
+      float s = 0;
+#pragma unroll
+      for (int g = 0; g < kGroups; ++g) s += (v[g][0] + v[g][1]) + (v[g][2] + v[g][3]);
+      total += (double)s;
+    }
+    double acc[1] = {total};
+    block_sum<1, kRcThreads>(acc, smem);
+    if (threadIdx.x == 0) peer_store_f32(a.scores + row, (float)acc[0]);
+  }
+  // Which responses share a group with this workgroup's first two rows does not depend on the scores: thread t notes
+  // it for responses t, t + 256, ... (one bit each, kGrpoRowsLimit / 256 of them) while the others are still summing.
+  unsigned member[2];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) member[r] = grpo_member_bits(a.gid, a.rows, (int64_t)blockIdx.x + (int64_t)r * gridDim.x);
+  const bool last = last_block_arrives(a.ticket);  // waits for this workgroup's stores first
+  if (last && threadIdx.x == 0) gate_release(a.ticket);
+  const bool open = last || gate_wait(a.ticket, a.spin_limit);
+  slot = 0;
+  // two rows at a time: their group statistics share one pass over the scores and one workgroup reduction
+  for (int64_t base = blockIdx.x; base < a.rows; base += 2 * (int64_t)gridDim.x) {
+    float scalar[2] = {__int_as_float(0x7fc00000), __int_as_float(0x7fc00000)};  // a wait that ran out stores NaN
+    if (open) {
+      if (base != blockIdx.x)
+#pragma unroll
+        for (int r = 0; r < 2; ++r) member[r] = grpo_member_bits(a.gid, a.rows, base + (int64_t)r * gridDim.x);
+      // count, sum and sum of squares of (score - own score) over the group: differences of fp32 scores are exact
+      // in double, and shifted by the row's own score the one-pass variance loses nothing to cancellation
+      double own[2], cs[6];
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int64_t row = base + (int64_t)r * gridDim.x;
+        own[r] = row < a.rows ? (double)peer_load_f32(a.scores + row) : 0.0;
+        cs[3 * r] = cs[3 * r + 1] = cs[3 * r + 2] = 0.0;
+        for (unsigned bits = member[r]; bits; bits &= bits - 1) {
+          const int64_t i = (int64_t)(__ffs(bits) - 1) * kRcThreads + threadIdx.x;
+          const double d = (double)peer_load_f32(a.scores + i) - own[r];
+          cs[3 * r] += 1.0;
+          cs[3 * r + 1] += d;
+          cs[3 * r + 2] += d * d;
+        }
+      }
+      block_sum<6, kRcThreads>(cs, smem);
+      if (threadIdx.x == 0) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+          const int64_t row = base + (int64_t)r * gridDim.x;
+          if (row >= a.rows) continue;
+          // scores are fp32 like the reference's; everything after them is evaluated in double and rounded once
+          const double cnt = cs[3 * r], s1 = cs[3 * r + 1], s2 = cs[3 * r + 2];
+          double cen = own[r], sd = 1.0;  // a group of one: mean 0, std 1
+          if (cnt > 1.0) {
+            cen = -s1 / cnt;
+            const double var = fmax(s2 - s1 * s1 / cnt, 0.0) / (cnt - 1.0);
+            sd = a.std_mode == 0 ? sqrt(var) : sqrt(fmax(var, (double)a.eps));
+          }
+          bc[r] = a.norm_by_std ? cen / (sd + (double)a.eps) : cen;
+          if (a.scalars) a.scalars[row] = (float)bc[r];
+        }
+      }
+      __syncthreads();
+      scalar[0] = (float)bc[0];
+      scalar[1] = (float)bc[1];
+      __syncthreads();
+    }
+#pragma unroll
+    for (int r = 0; r < 2; ++r) {
+      const int64_t row = base + (int64_t)r * gridDim.x;
+      if (row >= a.rows) break;
+      for (int c = 0; c < a.chunks; ++c) {
+        const ChunkPos pos(row, c, a.cols);
+        if (held && binary) {
+          const unsigned bits = held_bits[slot * kRcThreads + threadIdx.x];
+#pragma unroll
+          for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[g][e] = (bits >> (g * 4 + e)) & 1u ? 1.f : 0.f;
+        } else {
+          load_mask_groups<VEC>(mask, pos, w, streaming);
+        }
+        ++slot;
+#pragma unroll
+        for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[g][e] = open ? w[g][e] * scalar[r] : scalar[r];
+        store_groups<VEC>(a.out, pos, w, streaming);
+      }
+    }
+  }
+  gate_depart(a.ticket);
 }
 
 constexpr int kGrpoTailThreads = 1024;
@@ -1613,6 +1782,34 @@ extern "C" int vamd_group_outcome_advantage(const float* rewards, const void* ma
                              reduce_workspace_bytes(batch, length, 4), stream);
     if (st != VAMD_OK) return st;
   }
+  if (estimator == VAMD_ADV_GRPO && batch <= kGrpoRowsLimit) {
+    GrpoRowsArgs ra;
+    ra.rewards = rewards;
+    ra.mask = mask;
+    ra.gid = group_ids;
+    ra.rows = batch;
+    ra.cols = length;
+    ra.chunks = chunks;
+    ra.eps = epsilon;
+    ra.norm_by_std = norm_by_std;
+    ra.std_mode = std_mode;
+    ra.scores = ga.scores;
+    ra.scalars = scores_out;
+    ra.out = advantages;
+    ra.ticket = wk.ticket;
+    ra.spin_limit = gate_spin_limit(kGateSpinLimit);
+    VAMD_MASK_DISPATCH(mask_dtype, M, {
+      const bool vec = can_vectorize(length, {rewards, advantages}, mask, sizeof(M));
+      auto go = [&](auto kernel) {
+        const int64_t grid = balanced_waiting_grid(batch, resident_workgroups(reinterpret_cast<const void*>(kernel), kRcThreads));
+        hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kRcThreads), 0, s, ra);
+      };
+      if (vec) go(grpo_rows_kernel<true, M>);
+      else go(grpo_rows_kernel<false, M>);
+    });
+    VAMD_LAUNCH_CHECK();
+    return VAMD_OK;
+  }
   if (n_groups <= kGrpoInlineGroups && batch * chunks <= kInlineFoldRecords) {
     // one launch, if the device holds every workgroup of it at the same time
     bool launched = false;
@@ -1633,31 +1830,34 @@ extern "C" int vamd_group_outcome_advantage(const float* rewards, const void* ma
       return VAMD_OK;
     }
   }
+  // records per row of the row-sum pass: one per chunk, or one per row once there are enough rows to fill the device
+  const int span = (batch >= 1024 && chunks > 1) ? chunks : 1;
+  const int rec_chunks = (chunks + span - 1) / span;
   {
     const bool vec = can_vectorize(length, {rewards}, nullptr, 0);
     const bool lds_stats = n_groups <= kGrpoLdsGroups;
-    const dim3 grid((unsigned)(batch * chunks));
-    if (n_groups <= kGrpoInlineGroups && batch * chunks <= kInlineFoldRecords) {
+    const dim3 grid((unsigned)(batch * rec_chunks));
+    if (n_groups <= kGrpoInlineGroups && batch * rec_chunks <= kInlineFoldRecords) {
       VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((grpo_rowsum_kernel<V, true>), grid, dim3(kRcThreads), 0, s,
-                                                   rewards, length, chunks, wk, ga));
+                                                   rewards, length, rec_chunks, span, wk, ga));
     } else {
       VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((grpo_rowsum_kernel<V, false>), grid, dim3(kRcThreads), 0, s,
-                                                   rewards, length, chunks, wk, ga));
+                                                   rewards, length, rec_chunks, span, wk, ga));
       if (lds_stats) {
         VAMD_LAUNCH_CHECK();
         if (estimator == VAMD_ADV_GRPO)
           hipLaunchKernelGGL(grpo_scalars_kernel_lds<VAMD_ADV_GRPO>, dim3(1), dim3(kGrpoTailThreads), 0, s,
-                             wk.partials, chunks, ga);
+                             wk.partials, rec_chunks, ga);
         else
-          hipLaunchKernelGGL(grpo_scalars_kernel_lds<-1>, dim3(1), dim3(kGrpoTailThreads), 0, s, wk.partials, chunks,
-                             ga);
+          hipLaunchKernelGGL(grpo_scalars_kernel_lds<-1>, dim3(1), dim3(kGrpoTailThreads), 0, s, wk.partials,
+                             rec_chunks, ga);
       }
     }
     VAMD_LAUNCH_CHECK();
   }
   if (n_groups > kGrpoLdsGroups) {
     hipLaunchKernelGGL(rowsum_finalize_kernel, dim3((unsigned)((batch + 255) / 256)), dim3(256), 0, s, wk.partials,
-                       batch, chunks, ga.scores);
+                       batch, rec_chunks, ga.scores);
     VAMD_LAUNCH_CHECK();
     hipLaunchKernelGGL(group_stats_kernel<double>, dim3((unsigned)((n_groups + 63) / 64)), dim3(64), 0, s, ga.scores,
                        group_ids, batch, n_groups, epsilon, std_mode, ga.mean, ga.stdv, (float*)nullptr);

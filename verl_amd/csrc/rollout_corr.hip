@@ -73,9 +73,10 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
 #pragma unroll
     for (int i = 0; i < kRcSums; ++i) s[i] = 0.f;
     float o[kGroups][4], r[kGroups][4], m[kGroups][4], wt[kGroups][4];
-    load_groups<VEC>(a.old_lp, pos, o);
-    if (a.roll_lp) load_groups<VEC>(a.roll_lp, pos, r);
-    load_mask_groups<VEC>(mask, pos, m);
+    const bool streaming = streams_past_caches(a.rows * a.cols);  // the grid counts spans of chunks, not chunks
+    load_groups<VEC>(a.old_lp, pos, o, streaming);
+    if (a.roll_lp) load_groups<VEC>(a.roll_lp, pos, r, streaming);
+    load_mask_groups<VEC>(mask, pos, m, streaming);
 #pragma unroll
     for (int k = 0; k < kGroups; ++k)
 #pragma unroll
@@ -105,7 +106,7 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
           wt[k][e] = t;
         }
       }
-    if (a.level == VAMD_IS_TOKEN && a.weights) store_groups<VEC>(a.weights, pos, wt);
+    if (a.level == VAMD_IS_TOKEN && a.weights) store_groups<VEC>(a.weights, pos, wt, streaming);
 #pragma unroll
     for (int i = 0; i < kRcSums; ++i) acc[i] += (double)s[i];
   }

@@ -142,11 +142,12 @@ struct ChunkPos {
 };
 
 template <bool VEC>
-__device__ __forceinline__ void load_groups(const float* __restrict__ p, const ChunkPos& pos, float (&x)[kGroups][4]) {
+__device__ __forceinline__ void load_groups(const float* __restrict__ p, const ChunkPos& pos, float (&x)[kGroups][4],
+                                            bool streaming = launch_streams_past_caches()) {
 #pragma unroll
   for (int g = 0; g < kGroups; ++g) {
     if (pos.valid[g] > 0) {
-      ld4<VEC>(p, pos.idx[g], pos.valid[g], x[g]);
+      ld4<VEC>(p, pos.idx[g], pos.valid[g], x[g], streaming);
     } else {
 #pragma unroll
       for (int e = 0; e < 4; ++e) x[g][e] = 0.f;
@@ -155,11 +156,12 @@ __device__ __forceinline__ void load_groups(const float* __restrict__ p, const C
 }
 
 template <bool VEC, class M>
-__device__ __forceinline__ void load_mask_groups(const M* __restrict__ p, const ChunkPos& pos, float (&w)[kGroups][4]) {
+__device__ __forceinline__ void load_mask_groups(const M* __restrict__ p, const ChunkPos& pos, float (&w)[kGroups][4],
+                                                 bool streaming = launch_streams_past_caches()) {
 #pragma unroll
   for (int g = 0; g < kGroups; ++g) {
     if (pos.valid[g] > 0) {
-      ldmask4<VEC>(p, pos.idx[g], pos.valid[g], w[g]);
+      ldmask4<VEC>(p, pos.idx[g], pos.valid[g], w[g], streaming);
     } else {
 #pragma unroll
       for (int e = 0; e < 4; ++e) w[g][e] = 0.f;
@@ -168,10 +170,11 @@ __device__ __forceinline__ void load_mask_groups(const M* __restrict__ p, const 
 }
 
 template <bool VEC>
-__device__ __forceinline__ void store_groups(float* __restrict__ p, const ChunkPos& pos, const float (&x)[kGroups][4]) {
+__device__ __forceinline__ void store_groups(float* __restrict__ p, const ChunkPos& pos, const float (&x)[kGroups][4],
+                                             bool streaming = launch_streams_past_caches()) {
 #pragma unroll
   for (int g = 0; g < kGroups; ++g)
-    if (pos.valid[g] > 0) st4<VEC>(p, pos.idx[g], pos.valid[g], x[g]);
+    if (pos.valid[g] > 0) st4<VEC>(p, pos.idx[g], pos.valid[g], x[g], streaming);
 }
 
 // Publishing a record to the workgroup that will fold it, without a device-wide fence (an

@@ -44,6 +44,12 @@ int resident_workgroups(const void* kernel, int threads) {
   if (it != cache.end()) return it->second;
   int per_cu = 0;
   if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || per_cu < 1) per_cu = 1;
+  // The runtime's figure follows vector registers and LDS; a kernel with close to a hundred scalar registers was
+  // seen to fit one wavefront per SIMD fewer than it says (2048 workgroups of 256 threads did not all become
+  // resident, 1792 would have).  Waiting kernels must never overestimate, so two waves per SIMD are held back.
+  const int waves_per_wg = (threads + 63) / 64;
+  const int cap = (6 * 4) / waves_per_wg;  // 6 of the 8 wavefront slots of each of the 4 SIMDs
+  if (cap >= 1 && per_cu > cap) per_cu = cap;
   int cus = 0;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 1;
   const int n = per_cu * cus;
