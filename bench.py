@@ -30,7 +30,10 @@ COPY_YARDSTICK_BYTES = 1 << 30
 # rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by the readings of the 1 GiB copy in the same run
 # (2048 and 1024 bytes per unit); see profiles/head_fwd_bwd_qwen7b_hbm_traffic.md.  Counters cannot be read
 # from inside this process, so the figure is recorded here and only reported for the shape it was measured on.
-MEASURED_TRAFFIC_BYTES = {"lce_dgrad_kernel": 6.52e9 + 0.353e9, "lce_forward_kernel": 34.03e9 + 9.971e9}
+MEASURED_TRAFFIC_BYTES = {"lce_dgrad_kernel": 6.547e9 + 0.353e9,      # per full chunk, either backward mode
+                          "lce_forward_kernel": 26.22e9 + 0.004e9,   # without the logits cache (the default)
+                          "lce_forward_kernel_with_cache": 33.39e9 + 9.974e9,
+                          "lce_recompute_kernel": 2.826e9 + 0.611e9, "lce_dlogits_kernel": 1.124e9 + 0.537e9}
 GEMMS_PER_STEP = {"lce_forward_kernel": 1, "lce_recompute_kernel": 1, "lce_dgrad_kernel": 2}
 
 
@@ -355,24 +358,35 @@ def policy_math_python_path(dev, B: int = 512, Lc: int = 4096, n_groups: int = 6
     return res
 
 
+def _read_sclk_mhz():
+    """Current shader clock in MHz from the driver's sysfs table (the line marked '*'), or None."""
+    import glob
+
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")):
+        try:
+            for ln in open(path).read().splitlines():
+                if ln.rstrip().endswith("*"):
+                    digits = "".join(c for c in ln.split(":", 1)[1] if c.isdigit())
+                    if digits:
+                        return int(digits)
+        except (OSError, IndexError):
+            continue
+    return None
+
+
 def _sclk_sampler():
-    """Background reader of the shader clock (rocm-smi), for the ceiling probe: returns (stop, samples)."""
-    import subprocess
+    """Background reader of the shader clock, for the ceiling probe: returns (stop, samples).  Reads sysfs, starts no
+    other program."""
     import threading
 
     samples, stop = [], threading.Event()
 
     def run():
         while not stop.is_set():
-            try:
-                out = subprocess.run(["rocm-smi", "--showclocks", "--json"], capture_output=True, text=True, timeout=5).stdout
-                txt = json.loads(out).get("card0", {}).get("sclk clock speed:", "")
-                mhz = int("".join(c for c in txt if c.isdigit()) or 0)
-                if mhz:
-                    samples.append((time.time(), mhz))
-            except Exception:
-                pass
-            stop.wait(0.15)
+            mhz = _read_sclk_mhz()
+            if mhz:
+                samples.append((time.time(), mhz))
+            stop.wait(0.05)
 
     th = threading.Thread(target=run, daemon=True)
     th.start()
@@ -444,8 +458,8 @@ def mfma_ceiling_probe(dev, n: int, h: int, v: int, seconds: float = 1.5) -> dic
         res[kind]["vendor_gemm_TN_d_weight"] = run_for(lambda: torch.matmul(z.t(), hid, out=dw), 2.0 * n * vc * h)
         del hid, w, wc, z, dh, dw
     stop.set()
-    res["note"] = ("ms per call; PFLOP/s on 2*M*N*K; sclk from rocm-smi over the second half of each run "
-                   "(None when rocm-smi is unavailable); vendor GEMMs on one 16384-column vocabulary chunk")
+    res["note"] = ("ms per call; PFLOP/s on 2*M*N*K; sclk from the driver's sysfs table over the second half of each "
+                   "run (None when it cannot be read); vendor GEMMs on one 16384-column vocabulary chunk")
     return res
 
 
@@ -595,6 +609,10 @@ def main() -> None:
     ap.add_argument("--cpu-tokens", type=int, default=8192, help="token sample for the CPU baseline (0 = skip)")
     ap.add_argument("--head-only", action="store_true",
                     help="only the headline workload and its per-kernel timing (what the profiler runs trace)")
+    ap.add_argument("--ceiling-only", action="store_true",
+                    help="only the matrix-pipe ceiling probe (zeros against random operands, vendor GEMMs beside "
+                         "the forward kernel): what a counter pass for the shader clock runs")
+    ap.add_argument("--ceiling-seconds", type=float, default=1.5, help="how long the probe keeps each kernel running")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (every box here has one GPU; "
@@ -610,6 +628,9 @@ def main() -> None:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     n, h, v, T = 16384, 3584, 152064, 1.0
+    if args.ceiling_only:
+        print(json.dumps({"mfma_ceiling_probe": mfma_ceiling_probe(dev, n, h, v, seconds=args.ceiling_seconds)}))
+        return
     g = torch.Generator(device=dev).manual_seed(0)
     hidden = torch.randn(n, h, device=dev, generator=g).bfloat16().requires_grad_()
     weight = (torch.randn(v, h, device=dev, generator=g) * 0.02).bfloat16().requires_grad_()
@@ -712,7 +733,7 @@ def main() -> None:
     line["cpu_baseline"] = cpu_baseline(args.cpu_tokens, h, v, T) if args.cpu_tokens > 0 else None
     del hidden, weight
     torch.cuda.empty_cache()
-    line["mfma_ceiling_probe"] = mfma_ceiling_probe(dev, n, h, v)
+    line["mfma_ceiling_probe"] = mfma_ceiling_probe(dev, n, h, v, seconds=args.ceiling_seconds)
     torch.cuda.empty_cache()
     line["head_other_configs"] = other_head_configs(dev, args.steps)
     torch.cuda.empty_cache()

@@ -1065,7 +1065,12 @@ def test_benchmark_config_gae_value_policy_loss(dev):
     old = torch.randn(B, L, generator=g) * 0.5 - 1
     new = old + torch.randn(B, L, generator=g) * 0.05
     loss, _ = CA.compute_policy_loss_vanilla(old.to(dev), new.to(dev), adv, mask.to(dev), "token-mean", _cfg())
-    _close(loss, O.policy_loss_vanilla(old, new, want_adv, mask, "token-mean")[0], rtol=1e-4, what="pg_loss")
+    # the loss kernel itself: against the restatement on the very advantages it was given
+    _close(loss, O.policy_loss_vanilla(old, new, adv.cpu(), mask, "token-mean")[0], rtol=1e-5, what="pg_loss")
+    # the chain: whitened advantages average to zero, so the loss is what is left of a million cancelling terms and
+    # inherits the advantages' own difference from the sequential fp32 scan, weighted by a ratio that stays below 1.5
+    want_loss = O.policy_loss_vanilla(old, new, want_adv, mask, "token-mean")[0]
+    assert abs(loss.item() - want_loss.item()) <= 1.5 * (adv.cpu() - want_adv).abs().max().item() + 1e-7
 
 
 @pytest.mark.gpu
