@@ -134,11 +134,12 @@ def test_gae_gamma_lambda_one_long_rows_vs_fp64(dev):
     _close(adv, adv64.float(), rtol=1e-5, atol=2e-5, what="whitened advantages vs fp64")
 
 
-@pytest.mark.parametrize("B,L", [(3000, 300), (5, 9000), (1500, 4100), (700, 4096), (2, 3), (1100, 37)])
+@pytest.mark.parametrize("B,L", [(3000, 300), (5, 9000), (1500, 4100), (700, 4096), (2, 3), (1100, 37), (1200, 20000),
+                                 (2500, 9000), (6, 40000)])
 def test_gae_single_launch_paths(dev, B, L):
     """The one-launch estimator on every route through it: more rows than the device holds workgroups (a workgroup
-    walks several rows and whitens them from memory), rows longer than one batch of segments, and a single row per
-    workgroup whose advantages wait in registers.  Masks with holes; compared with the fp64 evaluation of the
+    walks several rows), rows longer than one batch of segments, workgroups whose batches all wait on chip (registers,
+    LDS) and workgroups that whiten most of theirs from memory, row lengths that leave the first batch ragged.  Masks with holes; compared with the fp64 evaluation of the
     reference recurrence."""
     from verl_amd.trainer.ppo.core_algos import compute_gae_advantage_return
     g = torch.Generator().manual_seed(B * 7 + L)
@@ -173,6 +174,38 @@ def test_gae_bounded_wait_runs_out_without_hanging(dev, monkeypatch):
     adv, ret = compute_gae_advantage_return(r, v, m, 1.0, 0.95)
     want_adv, want_ret = O.gae_advantage_return(r.cpu().double(), v.cpu().double(), m.cpu().double(), 1.0, 0.95)
     assert (adv.cpu().double() - want_adv).abs().max().item() <= 2e-5 * want_adv.abs().max().item()
+
+
+@pytest.mark.parametrize("B,L", [(512, 4096), (1500, 9000), (3, 30000)])
+def test_gae_bounded_wait_leaves_every_advantage_raw_or_whitened(dev, monkeypatch, B, L):
+    """The same forced time-out through the C ABI, where the outputs can be looked at: returns are right, and every
+    advantage is either the raw one (its workgroup gave up) or the whitened one (it found the gate open) -- whether it
+    waited in registers, in LDS or in memory -- and the fifth moment says that a wait ran out."""
+    from verl_amd import _cabi
+    g = torch.Generator().manual_seed(B + L)
+    r, v = torch.randn(B, L, generator=g), torch.randn(B, L, generator=g)
+    m = (torch.rand(B, L, generator=g) < 0.9).float()
+    want_adv, want_ret = O.gae_advantage_return(r.double(), v.double(), m.double(), 0.99, 0.95)
+    raw = want_ret - v.double()                      # returns = raw advantages + values
+    rd, vd, md = r.to(dev), v.to(dev), m.to(dev)
+    adv, ret = torch.empty_like(rd), torch.empty_like(rd)
+    mom = torch.empty(5, dtype=torch.float64, device=dev)
+    Lb = _cabi.lib()
+    ws = _cabi.ticket_workspace(Lb.vamd_gae_workspace_bytes(B, L), dev)
+    monkeypatch.setenv("VAMD_GATE_SPIN_LIMIT", "0")
+    _cabi.check(Lb.vamd_gae(rd.data_ptr(), vd.data_ptr(), md.data_ptr(), _cabi.MASK_F32, B, L, 0.99, 0.95, 1,
+                            adv.data_ptr(), ret.data_ptr(), mom.data_ptr(), ws.data_ptr(), ws.numel(),
+                            _cabi.stream_ptr(dev)))
+    torch.cuda.synchronize()
+    monkeypatch.delenv("VAMD_GATE_SPIN_LIMIT")
+    assert int(ws[:16640].to(torch.int32).sum()) == 0
+    scale = want_ret.abs().max().item()
+    assert (ret.cpu().double() - want_ret).abs().max().item() <= 2e-5 * scale
+    got = adv.cpu().double()
+    off = torch.minimum((got - raw).abs(), (got - want_adv).abs())
+    assert off.max().item() <= 2e-5 * max(scale, want_adv.abs().max().item())
+    if ((got - want_adv).abs() > 1e-3).any():       # some advantage was left raw: the host must have been told
+        assert mom[4].item() != 0.0
 
 
 def test_grpo_single_launch_bounded_wait_runs_out_without_hanging(dev, monkeypatch):

@@ -16,8 +16,8 @@
 //
 // With whitening the whole estimator is ONE launch: every workgroup keeps a record of the masked moments of its
 // rows, the workgroup that arrives last folds them into (mean, rstd) and opens the gate the others wait at, and
-// each workgroup then whitens what it produced -- from registers when it owns a single row of at most 4096 columns
-// (the advantages are then written once), from its own freshly written rows otherwise.
+// each workgroup then whitens what it produced.  The last three batches a workgroup walked wait on chip (one in
+// registers, two in LDS) and are written once, whitened; earlier batches were stored raw and are read back.
 #include "rowchunk.h"
 
 namespace vamd {
@@ -88,8 +88,15 @@ __global__ __launch_bounds__(kRcThreads) void gae_kernel(GaeArgs a) {
   const float gamma = a.gamma, gl = a.gl;
   const int64_t cols = a.cols;
   const int nseg = (int)((cols + kSeg - 1) / kSeg);
-  // a workgroup that owns one row of a single batch keeps its advantages in registers across the rendezvous
-  const bool held = WHITEN && gridDim.x == a.rows && nseg <= kSegBatch;
+  // With whitening, the advantages of the last batches a workgroup walks stay on chip across the rendezvous (the very
+  // last in registers, the kLdsHeld before it in LDS, each thread its own columns): they are neither stored raw nor
+  // read back.  At 512 x 4096 that is everything; at 2048 x 16384 on 1024 workgroups three batches of eight.
+  constexpr int kLdsHeld = 2;
+  __shared__ float4 lds_keep[WHITEN ? kLdsHeld * kSegBatch : 1][kRcThreads];
+  const int batches_per_row = (nseg + kSegBatch - 1) / kSegBatch;
+  const int64_t own_rows = (a.rows - blockIdx.x + gridDim.x - 1) / gridDim.x;
+  const int64_t last_batch = own_rows * batches_per_row - 1;
+  int64_t batch_no = 0;
   const bool streaming = streams_past_caches(a.rows * cols);
   float keep[kSegBatch][4];
   float m0 = 0, m1 = 0, m2 = 0, mc = 0;  // masked moments of the raw advantages
@@ -97,7 +104,9 @@ __global__ __launch_bounds__(kRcThreads) void gae_kernel(GaeArgs a) {
   for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
     __syncthreads();
     if (tid == 0) carry[0] = carry[1] = 0.f;
-    for (int top = nseg - 1; top >= 0; top -= kSegBatch) {
+    for (int top = nseg - 1; top >= 0; top -= kSegBatch, ++batch_no) {
+      const int64_t from_end = last_batch - batch_no;  // 0: stays in registers; 1..kLdsHeld: stays in LDS
+      const bool on_chip = WHITEN && from_end <= kLdsHeld;
       // issue every load of up to kSegBatch segments before touching any of them
       float r[kSegBatch][4], v[kSegBatch][4], w[kSegBatch][4];
       int valid[kSegBatch];
@@ -212,10 +221,10 @@ __global__ __launch_bounds__(kRcThreads) void gae_kernel(GaeArgs a) {
         if (valid[b] > 0) {
           const int64_t i = row * cols + (int64_t)seg * kSeg + slot * 4;
           st4<VEC>(a.ret, i, valid[b], r_out, streaming);
-          if (!held) {
-            st4<VEC>(a.adv, i, valid[b], a_out, streaming && !WHITEN);  // with WHITEN: read back after the rendezvous
-          }
+          if (!on_chip) st4<VEC>(a.adv, i, valid[b], a_out, streaming && !WHITEN);  // WHITEN: read back after the rendezvous
         }
+        if (WHITEN && from_end >= 1 && from_end <= kLdsHeld)
+          lds_keep[(from_end - 1) * kSegBatch + b][tid] = make_float4(a_out[0], a_out[1], a_out[2], a_out[3]);
 #pragma unroll
         for (int e = 0; e < 4; ++e) keep[b][e] = a_out[e];
       }
@@ -250,52 +259,41 @@ __global__ __launch_bounds__(kRcThreads) void gae_kernel(GaeArgs a) {
     return;
   }
   const bool open = last || gate_wait(a.wk.ticket, a.spin_limit);
-  if (open) {
-    const float mean = peer_load_f32(a.stats), rstd = peer_load_f32(a.stats + 1);
-    if (held) {
+  // A wait that ran out leaves the advantages raw (the host is told through moments[4]): what is in memory stays as it
+  // is, what was kept on chip is stored unchanged.
+  const float mean = open ? peer_load_f32(a.stats) : 0.f, rstd = open ? peer_load_f32(a.stats + 1) : 1.f;
+  batch_no = 0;
+  for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x)
+    for (int top = nseg - 1; top >= 0; top -= kSegBatch, ++batch_no) {  // the same walk: every thread meets its own columns
+      const int64_t from_end = last_batch - batch_no;
+      if (!open && from_end > kLdsHeld) continue;
+      float x[kSegBatch][4];
+      int n_ok[kSegBatch];
 #pragma unroll
       for (int b = 0; b < kSegBatch; ++b) {
-        const int seg = nseg - 1 - b;
+        const int seg = top - b;
         const int64_t c = (int64_t)seg * kSeg + slot * 4;
         const int64_t left = cols - c;
-        const int n_ok = seg < 0 ? 0 : (left >= 4 ? 4 : (left > 0 ? (int)left : 0));
-        if (n_ok <= 0) continue;
-        float o[4];
+        n_ok[b] = seg < 0 ? 0 : (left >= 4 ? 4 : (left > 0 ? (int)left : 0));
+        if (n_ok[b] <= 0) continue;
+        if (from_end == 0) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = (keep[b][e] - mean) * rstd;
-        st4<VEC>(a.adv, (int64_t)blockIdx.x * cols + c, n_ok, o, streaming);
-      }
-    } else {  // every thread revisits the 4-column groups it wrote itself
-      for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x)
-        for (int64_t c = (int64_t)slot * 4; c < cols; c += (int64_t)kRcThreads * 4 * 4) {
-          float x[4][4];
-          int n_ok[4];
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const int64_t cu = c + (int64_t)u * kRcThreads * 4;
-            const int64_t left = cols - cu;
-            n_ok[u] = left >= 4 ? 4 : (left > 0 ? (int)left : 0);
-            if (n_ok[u] > 0) ld4<VEC>(a.adv, row * cols + cu, n_ok[u], x[u], false);
-          }
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            if (n_ok[u] <= 0) continue;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) x[u][e] = (x[u][e] - mean) * rstd;
-            st4<VEC>(a.adv, row * cols + c + (int64_t)u * kRcThreads * 4, n_ok[u], x[u], streaming);
-          }
+          for (int e = 0; e < 4; ++e) x[b][e] = keep[b][e];
+        } else if (from_end <= kLdsHeld) {
+          const float4 k4 = lds_keep[(from_end - 1) * kSegBatch + b][tid];
+          x[b][0] = k4.x, x[b][1] = k4.y, x[b][2] = k4.z, x[b][3] = k4.w;
+        } else {
+          ld4<VEC>(a.adv, row * cols + c, n_ok[b], x[b], false);
         }
-    }
-  } else if (held) {  // timed out: leave the raw advantages, the host is told through moments[4]
+      }
 #pragma unroll
-    for (int b = 0; b < kSegBatch; ++b) {
-      const int seg = nseg - 1 - b;
-      const int64_t c = (int64_t)seg * kSeg + slot * 4;
-      const int64_t left = cols - c;
-      const int n_ok = seg < 0 ? 0 : (left >= 4 ? 4 : (left > 0 ? (int)left : 0));
-      if (n_ok > 0) st4<VEC>(a.adv, (int64_t)blockIdx.x * cols + c, n_ok, keep[b], streaming);
+      for (int b = 0; b < kSegBatch; ++b) {
+        if (n_ok[b] <= 0) continue;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[b][e] = (x[b][e] - mean) * rstd;
+        st4<VEC>(a.adv, row * cols + (int64_t)(top - b) * kSeg + slot * 4, n_ok[b], x[b], streaming);
+      }
     }
-  }
   const unsigned verdict = gate_depart(a.wk.ticket);
   if (verdict != 0 && tid == 0) a.moments[4] = verdict > 1 ? 1.0 : 0.0;
 }

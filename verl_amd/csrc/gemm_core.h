@@ -42,15 +42,26 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kTile = 256;                    // output tile edge
 constexpr int kBK = 64;                       // k extent of one slab
-constexpr int kWavesR = 4;                    // wavefronts along r
+// Wavefronts along r: 4 (eight wavefronts of 64 x 128, two per SIMD) is what ships.  2 (four wavefronts of
+// 128 x 128, one per SIMD, accumulators in the 256 AGPRs) reads a third fewer fragments per MFMA and lets the board
+// clock 10 % higher on random data, but loses more than that at the per-slab barrier: forward 13.7 against 13.2 ms,
+// gradient GEMMs 33.0 against 27.3 ms per step at 16384 x 152064 x 3584.
+#ifndef VAMD_WAVES_R
+#define VAMD_WAVES_R 4
+#endif
+constexpr int kWavesR = VAMD_WAVES_R;         // wavefronts along r
 constexpr int kWavesC = 2;                    // wavefronts along c
-constexpr int kThreads = 64 * kWavesR * kWavesC;
-constexpr int kNB = kTile / 32 / kWavesR;     // 32-row blocks per wavefront    (2)
+constexpr int kWaves = kWavesR * kWavesC;
+constexpr int kThreads = 64 * kWaves;
+constexpr int kNB = kTile / 32 / kWavesR;     // 32-row blocks per wavefront
 constexpr int kMB = kTile / 32 / kWavesC;     // 32-column blocks per wavefront (4)
-constexpr int kLoads = kTile * 8 / kThreads;  // 16-byte memory -> LDS transfers per lane per operand slab (4)
+constexpr int kLoads = kTile * 8 / kThreads;  // 16-byte memory -> LDS transfers per lane per operand slab
+constexpr int kStepMfmas = kMB * kNB;         // MFMAs of one 16-k step of a wavefront
 constexpr int kSlabBytes = kTile * kBK * 2;   // 32 KB
 constexpr int kLdsBytes = 4 * kSlabBytes;     // R,C x 2 stages = 128 KB
-static_assert(kNB == 2 && kMB == 4 && kLoads == 4, "slab_iter's slot schedule is written for this layout");
+static_assert(kMB == 4 && (kNB == 2 || kNB == 4), "FragAddr holds four block offsets");
+static_assert(kMB + kNB <= kStepMfmas && 2 * kLoads <= kStepMfmas, "a step has one slot per MFMA");
+static_assert((8 * kWaves) % 16 == 0 && (2 * kWaves) % 4 == 0, "the swizzles must not change between loads");
 
 // One GEMM operand as the tile engine sees it.
 struct Operand {
@@ -153,8 +164,8 @@ __device__ __forceinline__ void load_to_lds_16(const u32x4& rsrc, unsigned voff,
                : "memory", "m0");
 }
 
-// Memory -> LDS transfer of one operand slab: 4 loads of 16 bytes per lane.  Load i of wavefront
-// w fills the 1 KB LDS block (w + 8 i) of the slab:
+// Memory -> LDS transfer of one operand slab: kLoads loads of 16 bytes per lane.  Load i of wavefront
+// w fills the 1 KB LDS block (w + kWaves i) of the slab:
 //   direct : block b = rows 8 b .. 8 b + 7; lane L sits at row 8 b + L / 8, chunk position L % 8,
 //            and fetches logical chunk (L % 8) ^ swizzle of that row -- 8 lanes cover one whole
 //            128 B line of the memory row;
@@ -176,18 +187,18 @@ struct SlabDma {
     if constexpr (!KMAJOR) {
       const unsigned row = 8u * w + (lane >> 3);
       voff = row * ld_bytes + (((lane & 7u) ^ (unsigned)swizzle_direct((int)row)) << 4);
-      step = 64u * ld_bytes;
+      step = (8u * kWaves) * ld_bytes;
     } else {
       const unsigned k = 2u * w + (lane >> 5);
       voff = k * ld_bytes + (((lane & 31u) ^ (4u * (k & 3u))) << 4);
-      step = 16u * ld_bytes;
+      step = (2u * kWaves) * ld_bytes;
     }
     lds_wave = __builtin_amdgcn_readfirstlane(w * 1024u);
   }
 
   // slab_lds: LDS byte address of the operand's slab in the stage being filled
   __device__ __forceinline__ void issue_one(int i, const SlabSrc& src, unsigned slab_lds) const {
-    load_to_lds_16(src.rsrc, voff, src.soff + (unsigned)i * step, slab_lds + lds_wave + (unsigned)i * 8192u);
+    load_to_lds_16(src.rsrc, voff, src.soff + (unsigned)i * step, slab_lds + lds_wave + (unsigned)i * (kWaves * 1024u));
   }
 };
 
@@ -258,9 +269,9 @@ __device__ __forceinline__ void slab_iter(const SlabDma<RK>& dr, const SlabDma<C
                                           const SlabSrc& c2, char* cur, const char* nxt, const FragAddr<RK>& fr,
                                           const FragAddr<CK>& fc, Frags& f0, Accum& acc) {
   Frags f1;
-#define VAMD_MFMA(F, i)                                                                                            \
-  acc.a[(i) >> 1][(i) & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F.c[(i) >> 1], F.r[(i) & 1],                    \
-                                                                     acc.a[(i) >> 1][(i) & 1], 0, 0, 0)
+#define VAMD_MFMA(F, i)                                                                                              \
+  acc.a[(i) / kNB][(i) % kNB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F.c[(i) / kNB], F.r[(i) % kNB],                 \
+                                                                        acc.a[(i) / kNB][(i) % kNB], 0, 0, 0)
 #define VAMD_FRAG(G, base, i, s)                                            \
   do {                                                                      \
     if ((i) < kMB) G.c[(i)] = fc.read((base) + kSlabBytes, (s), (i));        \
@@ -268,19 +279,19 @@ __device__ __forceinline__ void slab_iter(const SlabDma<RK>& dr, const SlabDma<C
   } while (0)
 #define VAMD_SLOT_END __builtin_amdgcn_sched_barrier(0)
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < kStepMfmas; ++i) {
     VAMD_MFMA(f0, i);
     VAMD_FRAG(f1, cur, i, 1);
     VAMD_SLOT_END;
   }
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < kStepMfmas; ++i) {
     VAMD_MFMA(f1, i);
     VAMD_FRAG(f0, cur, i, 2);
     VAMD_SLOT_END;
   }
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < kStepMfmas; ++i) {
     VAMD_MFMA(f0, i);
     VAMD_FRAG(f1, cur, i, 3);
     VAMD_SLOT_END;
@@ -288,11 +299,11 @@ __device__ __forceinline__ void slab_iter(const SlabDma<RK>& dr, const SlabDma<C
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
   VAMD_SLOT_END;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < kStepMfmas; ++i) {
     VAMD_MFMA(f1, i);
     VAMD_FRAG(f0, nxt, i, 0);
-    if (i < 4) dr.issue_one(i, r2, lds_address(cur));
-    else dc.issue_one(i - 4, c2, lds_address(cur) + kSlabBytes);
+    if (i < kLoads) dr.issue_one(i, r2, lds_address(cur));
+    else if (i < 2 * kLoads) dc.issue_one(i - kLoads, c2, lds_address(cur) + kSlabBytes);
     VAMD_SLOT_END;
   }
 #undef VAMD_MFMA
