@@ -50,7 +50,7 @@ struct Carver {
 int device_cu_count();
 // Workgroups of `threads` threads of `kernel` (no dynamic LDS) that the current device holds at the same time:
 // the grid limit of kernels whose workgroups wait for each other.  Cached per (device, kernel).
-int resident_workgroups(const void* kernel, int threads);
+int resident_workgroups(const void* kernel, int threads, size_t dynamic_lds_bytes = 0);
 // Grid for `items` units of work on a kernel whose workgroups wait for each other: at most `resident`, and chosen so
 // that every workgroup walks the same number of items (2048 items on 1536 resident workgroups: 1024 x 2, not
 // 1536 of which a third walk two).

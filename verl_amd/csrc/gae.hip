@@ -27,6 +27,8 @@ constexpr int kSegBatch = 4;     // segments whose loads are issued together (48
 constexpr int kPieces = kSegBatch * (kRcThreads / 64);  // (segment, wavefront) pieces of a batch, in walk order
 static_assert(kPieces == 16, "wavefront 0 scans the piece totals inside one row of 16 lanes");
 
+constexpr int kGaeLdsHeld = 2;   // batches of a workgroup that wait in LDS across the rendezvous (32 KiB)
+
 struct GaeWork {
   unsigned* ticket;   // workspace head: zero on entry, zero on exit
   double* partials;   // per workgroup the 4 masked moments of the raw advantages; slot-major
@@ -73,6 +75,7 @@ struct GaeArgs {
   double* moments;  // [5]: sum m, sum g m, sum g^2 m, count, 1.0 if the rendezvous timed out
   float* stats;     // [4]: mean, rstd, shift
   unsigned spin_limit;
+  int lds_held;     // batches per workgroup that wait in LDS (the launch's dynamic LDS holds them)
 };
 
 template <bool VEC, class M, bool WHITEN>
@@ -89,10 +92,11 @@ __global__ __launch_bounds__(kRcThreads) void gae_kernel(GaeArgs a) {
   const int64_t cols = a.cols;
   const int nseg = (int)((cols + kSeg - 1) / kSeg);
   // With whitening, the advantages of the last batches a workgroup walks stay on chip across the rendezvous (the very
-  // last in registers, the kLdsHeld before it in LDS, each thread its own columns): they are neither stored raw nor
+  // last in registers, up to two before it in LDS when the launch brought the room, each thread its own columns): they are neither stored raw nor
   // read back.  At 512 x 4096 that is everything; at 2048 x 16384 on 1024 workgroups three batches of eight.
-  constexpr int kLdsHeld = 2;
-  __shared__ float4 lds_keep[WHITEN ? kLdsHeld * kSegBatch : 1][kRcThreads];
+  extern __shared__ float4 lds_keep_raw[];  // [a.lds_held * kSegBatch][kRcThreads], sized by the launch
+  float4(*lds_keep)[kRcThreads] = reinterpret_cast<float4(*)[kRcThreads]>(lds_keep_raw);
+  const int kLdsHeld = WHITEN ? a.lds_held : 0;
   const int batches_per_row = (nseg + kSegBatch - 1) / kSegBatch;
   const int64_t own_rows = (a.rows - blockIdx.x + gridDim.x - 1) / gridDim.x;
   const int64_t last_batch = own_rows * batches_per_row - 1;
@@ -262,6 +266,20 @@ __global__ __launch_bounds__(kRcThreads) void gae_kernel(GaeArgs a) {
   // A wait that ran out leaves the advantages raw (the host is told through moments[4]): what is in memory stays as it
   // is, what was kept on chip is stored unchanged.
   const float mean = open ? peer_load_f32(a.stats) : 0.f, rstd = open ? peer_load_f32(a.stats + 1) : 1.f;
+  if (last_batch == 0) {  // one row of one batch (512 x 4096 is such a launch): straight from the registers
+#pragma unroll
+    for (int b = 0; b < kSegBatch; ++b) {
+      const int seg = nseg - 1 - b;
+      const int64_t c = (int64_t)seg * kSeg + slot * 4;
+      const int64_t left = cols - c;
+      const int n_ok = seg < 0 ? 0 : (left >= 4 ? 4 : (left > 0 ? (int)left : 0));
+      if (n_ok <= 0) continue;
+      float o[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) o[e] = (keep[b][e] - mean) * rstd;
+      st4<VEC>(a.adv, (int64_t)blockIdx.x * cols + c, n_ok, o, streaming);
+    }
+  } else {
   batch_no = 0;
   for (int64_t row = blockIdx.x; row < a.rows; row += gridDim.x)
     for (int top = nseg - 1; top >= 0; top -= kSegBatch, ++batch_no) {  // the same walk: every thread meets its own columns
@@ -294,6 +312,7 @@ __global__ __launch_bounds__(kRcThreads) void gae_kernel(GaeArgs a) {
         st4<VEC>(a.adv, row * cols + (int64_t)(top - b) * kSeg + slot * 4, n_ok[b], x[b], streaming);
       }
     }
+  }
   const unsigned verdict = gate_depart(a.wk.ticket);
   if (verdict != 0 && tid == 0) a.moments[4] = verdict > 1 ? 1.0 : 0.0;
 }
@@ -339,8 +358,20 @@ extern "C" int vamd_gae(const float* rewards, const float* values, const void* m
   // beyond that a workgroup walks several rows.
   auto launch = [&](auto kernel) -> int {
     int64_t grid = batch;
-    if (whiten) grid = balanced_waiting_grid(batch, resident_workgroups(reinterpret_cast<const void*>(kernel), kRcThreads));
-    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kRcThreads), 0, s, a);
+    size_t lds = 0;
+    a.lds_held = 0;
+    if (whiten) {
+      // LDS for the batches that wait on chip beside the one in registers: none when a workgroup walks a single batch
+      const int64_t batches_per_row = (length + (int64_t)kSeg * kSegBatch - 1) / ((int64_t)kSeg * kSegBatch);
+      const void* k = reinterpret_cast<const void*>(kernel);
+      grid = balanced_waiting_grid(batch, resident_workgroups(k, kRcThreads, 0));
+      if ((batch + grid - 1) / grid * batches_per_row > 1) {
+        a.lds_held = kGaeLdsHeld;
+        lds = (size_t)kGaeLdsHeld * kSegBatch * kRcThreads * sizeof(float4);
+        grid = balanced_waiting_grid(batch, resident_workgroups(k, kRcThreads, lds));
+      }
+    }
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kRcThreads), lds, s, a);
     return VAMD_OK;
   };
   VAMD_MASK_DISPATCH(mask_dtype, M, {

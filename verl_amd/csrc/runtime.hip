@@ -3,6 +3,7 @@
 #include <stdlib.h>
 
 #include <map>
+#include <tuple>
 #include <mutex>
 #include <utility>
 
@@ -34,16 +35,17 @@ int device_cu_count() {
   return cached[dev];
 }
 
-int resident_workgroups(const void* kernel, int threads) {
+int resident_workgroups(const void* kernel, int threads, size_t dynamic_lds_bytes) {
   static std::mutex mu;
-  static std::map<std::pair<int, const void*>, int> cache;
+  static std::map<std::tuple<int, const void*, size_t>, int> cache;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) dev = 0;
   std::lock_guard<std::mutex> lock(mu);
-  auto it = cache.find({dev, kernel});
+  auto it = cache.find({dev, kernel, dynamic_lds_bytes});
   if (it != cache.end()) return it->second;
   int per_cu = 0;
-  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess || per_cu < 1) per_cu = 1;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, dynamic_lds_bytes) != hipSuccess || per_cu < 1)
+    per_cu = 1;
   // The runtime's figure follows vector registers and LDS; a kernel with close to a hundred scalar registers was
   // seen to fit one wavefront per SIMD fewer than it says (2048 workgroups of 256 threads did not all become
   // resident, 1792 would have).  Waiting kernels must never overestimate, so two waves per SIMD are held back.
@@ -53,7 +55,7 @@ int resident_workgroups(const void* kernel, int threads) {
   int cus = 0;
   if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 1;
   const int n = per_cu * cus;
-  cache[{dev, kernel}] = n;
+  cache[{dev, kernel, dynamic_lds_bytes}] = n;
   return n;
 }
 
