@@ -90,24 +90,27 @@ __global__ __launch_bounds__(kRcThreads) void otb_scan_kernel(const float* __res
                                                               float* returns, float* __restrict__ w_cum,
                                                               OtbPacked pk) {
   const int64_t base = (int64_t)blockIdx.x * cols;
+  // one workgroup per row: the launch is past the caches when rows x cols is (the inputs are read once; returns and
+  // W are read again by the baseline launch, but two tensors of that size do not survive in the caches either)
+  const bool streaming = streams_past_caches((int64_t)gridDim.x * cols);
   __shared__ double wave_tot[2][4];
   row_running_sum<true>(
       cols, wave_tot,
       [&](int64_t c, int valid, float (&v)[4]) {
         float m[4];
-        ld4<VEC>(rewards, base + c, valid, v);
-        ldmask4<VEC>(mask, base + c, valid, m);
+        ld4<VEC>(rewards, base + c, valid, v, streaming);
+        ldmask4<VEC>(mask, base + c, valid, m, false);  // read again by the forward walk
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = e < valid ? v[e] * m[e] : 0.f;
       },
-      [&](int64_t c, int valid, const float (&o)[4]) { st4<VEC>(returns, base + c, valid, o); });
+      [&](int64_t c, int valid, const float (&o)[4]) { st4<VEC>(returns, base + c, valid, o, streaming && !PACK); });
   __syncthreads();  // the forward walks below own other columns than the walk above did
   if constexpr (PACK) {
     const double n = row_running_sum<false>(
         cols, wave_tot,
         [&](int64_t c, int valid, float (&v)[4]) {
           float m[4];
-          ldmask4<VEC>(mask, base + c, valid, m);
+          ldmask4<VEC>(mask, base + c, valid, m, false);
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = (e < valid && m[e] != 0.f) ? 1.f : 0.f;
         },
@@ -125,12 +128,12 @@ __global__ __launch_bounds__(kRcThreads) void otb_scan_kernel(const float* __res
       cols, wave_tot,
       [&](int64_t c, int valid, float (&v)[4]) {
         float lp[4], q[4], iw[4];
-        ld4<VEC>(old_lp, base + c, valid, lp);
-        ld4<VEC>(pi2, base + c, valid, q);
-        ldmask4<VEC>(mask, base + c, valid, keep_m);
-        if (ISW) ld4<VEC>(isw, base + c, valid, iw);
+        ld4<VEC>(old_lp, base + c, valid, lp, streaming);
+        ld4<VEC>(pi2, base + c, valid, q, streaming);
+        ldmask4<VEC>(mask, base + c, valid, keep_m, false);
+        if (ISW) ld4<VEC>(isw, base + c, valid, iw, streaming);
         if constexpr (PACK) {
-          ld4<VEC>(returns, base + c, valid, keep_g);
+          ld4<VEC>(returns, base + c, valid, keep_g, false);
 #pragma unroll
           for (int e = 0; e < 4; ++e) keep_rank[e] = e < valid ? pk.rank[base + c + e] : 0;
         }
@@ -150,7 +153,7 @@ __global__ __launch_bounds__(kRcThreads) void otb_scan_kernel(const float* __res
               pk.g[base + keep_rank[e]] = keep_g[e];
             }
         } else {
-          st4<VEC>(w_cum, base + c, valid, o);
+          st4<VEC>(w_cum, base + c, valid, o, streaming);
         }
       });
 }
@@ -171,7 +174,7 @@ __device__ __forceinline__ void otb_mask4(const M* __restrict__ mask, const OtbG
 #pragma unroll
     for (int e = 0; e < 4; ++e) m[e] = (e < valid && col + e < n) ? 1.f : 0.f;
   } else {
-    ldmask4<VEC>(mask, row * cols + col, valid, m);
+    ldmask4<VEC>(mask, row * cols + col, valid, m, false);
   }
 }
 
@@ -185,7 +188,9 @@ template <bool VEC, class M>
 __global__ __launch_bounds__(kRcThreads) void otb_baseline_kernel(const float* returns,
                                                                   const float* __restrict__ w_cum,
                                                                   const M* __restrict__ mask, OtbGroups gr,
-                                                                  int64_t cols, int segs, float eps, float* adv) {
+                                                                  int64_t cols, int segs, float eps, float* adv,
+                                                                  int streaming_launch) {
+  const bool streaming = streaming_launch != 0;
   const int64_t g = blockIdx.x / segs;
   const int64_t col = (int64_t)(blockIdx.x % segs) * kOtbSeg + threadIdx.x * 4;
   const int64_t left = cols - col;
@@ -202,8 +207,8 @@ __global__ __launch_bounds__(kRcThreads) void otb_baseline_kernel(const float* r
         for (int e = 0; e < 4; ++e) R[k][e] = W[k][e] = m[k][e] = 0.f;
         if (i0 + k < last) {
           const int64_t row = gr.rows_by_group[i0 + k];
-          ld4<VEC>(returns, row * cols + col, valid, R[k]);
-          ld4<VEC>(w_cum, row * cols + col, valid, W[k]);
+          ld4<VEC>(returns, row * cols + col, valid, R[k], false);  // read again below
+          ld4<VEC>(w_cum, row * cols + col, valid, W[k], streaming);
           otb_mask4<VEC>(mask, gr, row, cols, col, valid, m[k]);
         }
       }
@@ -231,7 +236,7 @@ __global__ __launch_bounds__(kRcThreads) void otb_baseline_kernel(const float* r
       if (i0 + k < last) {
         row[k] = gr.rows_by_group[i0 + k];
         cut[k] = gr.tail_start ? gr.tail_start[row[k]] : cols;
-        ld4<VEC>(returns, row[k] * cols + col, valid, R[k]);
+        ld4<VEC>(returns, row[k] * cols + col, valid, R[k], false);
         otb_mask4<VEC>(mask, gr, row[k], cols, col, valid, m[k]);
       }
     }
@@ -243,7 +248,7 @@ __global__ __launch_bounds__(kRcThreads) void otb_baseline_kernel(const float* r
         const float b = col + e < cut[k] ? num[e] : 0.f;
         R[k][e] = m[k][e] != 0.f ? (R[k][e] - b) * m[k][e] : 0.f;
       }
-      st4<VEC>(adv, row[k] * cols + col, valid, R[k]);
+      st4<VEC>(adv, row[k] * cols + col, valid, R[k], streaming);
     }
   }
 }
@@ -312,6 +317,7 @@ extern "C" int vamd_otb_advantage(const float* rewards, const void* mask, int ma
   const int segs = (int)((length + kOtbSeg - 1) / kOtbSeg);  // 1024-column segments of the baseline pass
   const dim3 threads(kRcThreads), per_row((unsigned)batch), per_group((unsigned)(n_groups * segs)),
       per_chunk((unsigned)(batch * chunks));
+  const int past_caches = batch * length >= (int64_t)kStreamingGrid * 4096 ? 1 : 0;
 #define VAMD_OTB(V, W)                                                                                              \
   do {                                                                                                              \
     if (packed) {                                                                                                   \
@@ -319,14 +325,14 @@ extern "C" int vamd_otb_advantage(const float* rewards, const void* mask, int ma
                          sum_pi_squared, is_weights, length, returns, w_cum, pk);                                   \
       if (n_groups > 0)                                                                                             \
         hipLaunchKernelGGL((otb_baseline_kernel<V, M>), per_group, threads, 0, s, pk.g, pk.w, mk, gr, length,        \
-                           segs, epsilon, pk.g);                                                                    \
+                           segs, epsilon, pk.g, 0);                                                                 \
       hipLaunchKernelGGL((otb_unpack_kernel<V, M>), per_chunk, threads, 0, s, pk.g, pk.rank, mk, length, chunks,     \
                          advantages);                                                                               \
     } else {                                                                                                        \
       hipLaunchKernelGGL((otb_scan_kernel<V, M, W, false>), per_row, threads, 0, s, rewards, mk, old_log_probs,      \
                          sum_pi_squared, is_weights, length, returns, w_cum, pk);                                   \
       hipLaunchKernelGGL((otb_baseline_kernel<V, M>), per_group, threads, 0, s, returns, w_cum, mk, gr, length,      \
-                         segs, epsilon, advantages);                                                                \
+                         segs, epsilon, advantages, past_caches);                                                   \
     }                                                                                                               \
   } while (0)
   VAMD_MASK_DISPATCH(mask_dtype, M, {
