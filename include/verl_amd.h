@@ -246,9 +246,12 @@ int vamd_affine_by_stats(const float* values, const float* stats, int64_t n, flo
  * rewards, values [B, L] fp32, mask [B, L]; advantages (whitened) and returns [B, L] fp32 out.
  * The recurrence is evaluated as a chunked associative scan (a most-recent-valid-value scan for the
  * bootstrap value, then a one-variable affine scan for the advantage); masked steps carry the state.
- * whiten == 0 leaves the raw advantages (the value before :261).  With whiten != 0 the whole estimator is one
+ * whiten == 0 leaves the raw advantages (the value before :261).  With whiten == 1 the whole estimator is one
  * launch whose workgroups meet once (the grid is capped at what the device holds at a time): the masked
- * moments are folded, and every workgroup whitens what it produced.
+ * moments are folded, and every workgroup whitens what it produced.  whiten == 2 does the same in two launches
+ * whose workgroups never wait for each other; VAMD_WAITING_KERNELS=0 in the environment makes 1 behave as 2 (and
+ * keeps vamd_grpo_advantage / vamd_group_outcome_advantage to their several-launch paths), for a GPU that other
+ * long-running kernels share.
  * moments_out (5 doubles, may be NULL) receives the masked moments of the raw advantages (sum m, sum g m,
  * sum g^2 m, count) so the host can raise masked_var's M in {0,1} error; moments_out[4] is 0, or 1 if the
  * workgroups' bounded wait for each other ran out (the advantages are then left raw; VAMD_GATE_SPIN_LIMIT in the

@@ -62,6 +62,10 @@ inline int64_t balanced_waiting_grid(int64_t items, int64_t resident) {
 // Poll limit of the launch-wide rendezvous: VAMD_GATE_SPIN_LIMIT in the environment (tests set 0 to force the
 // timed-out path), else `standard`.
 unsigned gate_spin_limit(unsigned standard);
+// False when VAMD_WAITING_KERNELS=0 in the environment: the entry points then keep to launches whose workgroups
+// never wait for each other (one or two launches more), for a GPU shared with long-running kernels of other streams
+// or processes, where a launch's workgroups may not all be resident together.
+bool waiting_kernels_allowed();
 
 // mask element -> (weight, member) following masked_sum: weight = (float)m, member = m != 0
 template <class M>

@@ -374,6 +374,9 @@ extern "C" int vamd_gae(const float* rewards, const float* values, const void* m
     hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kRcThreads), lds, s, a);
     return VAMD_OK;
   };
+  // whiten == 2, or waiting kernels switched off: the scan launch leaves the statistics, a second launch applies them
+  const bool apart = whiten != 0 && (whiten == 2 || !waiting_kernels_allowed());
+  if (apart) whiten = 0;
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(length, {rewards, values, advantages, returns}, mask, sizeof(M));
     if (whiten) {
@@ -385,5 +388,6 @@ extern "C" int vamd_gae(const float* rewards, const float* values, const void* m
     }
   });
   VAMD_LAUNCH_CHECK();
+  if (apart) return vamd_affine_by_stats(advantages, a.stats, batch * length, advantages, stream);
   return VAMD_OK;
 }

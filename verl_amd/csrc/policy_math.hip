@@ -1829,7 +1829,8 @@ extern "C" int vamd_group_outcome_advantage(const float* rewards, const void* ma
                              reduce_workspace_bytes(batch, length, 4), stream);
     if (st != VAMD_OK) return st;
   }
-  if (estimator == VAMD_ADV_GRPO && batch <= kGrpoRowsLimit) {
+  const bool may_wait = waiting_kernels_allowed();
+  if (may_wait && estimator == VAMD_ADV_GRPO && batch <= kGrpoRowsLimit) {
     GrpoRowsArgs ra;
     ra.rewards = rewards;
     ra.mask = mask;
@@ -1857,7 +1858,7 @@ extern "C" int vamd_group_outcome_advantage(const float* rewards, const void* ma
     VAMD_LAUNCH_CHECK();
     return VAMD_OK;
   }
-  if (n_groups <= kGrpoInlineGroups && batch * chunks <= kInlineFoldRecords) {
+  if (may_wait && n_groups <= kGrpoInlineGroups && batch * chunks <= kInlineFoldRecords) {
     // one launch, if the device holds every workgroup of it at the same time
     bool launched = false;
     VAMD_MASK_DISPATCH(mask_dtype, M, {

@@ -59,6 +59,11 @@ int resident_workgroups(const void* kernel, int threads, size_t dynamic_lds_byte
   return n;
 }
 
+bool waiting_kernels_allowed() {
+  const char* e = getenv("VAMD_WAITING_KERNELS");
+  return !(e && e[0] == '0' && e[1] == 0);
+}
+
 unsigned gate_spin_limit(unsigned standard) {
   if (const char* e = getenv("VAMD_GATE_SPIN_LIMIT")) {
     char* end = nullptr;

@@ -10,6 +10,7 @@ they are staged to the current GPU and results come back on the input's device.
 from __future__ import annotations
 
 from enum import Enum
+import warnings
 from typing import Any, Callable, Optional
 
 import numpy as np
@@ -142,6 +143,15 @@ def _mask_matrix(mask: torch.Tensor, dev: torch.device, shape) -> tuple[torch.Te
     return m, code
 
 
+_WARNED = set()
+
+
+def _warn_once(text: str) -> None:
+    if text not in _WARNED:
+        _WARNED.add(text)
+        warnings.warn(text, RuntimeWarning, stacklevel=3)
+
+
 @register_adv_est(AdvantageEstimator.GAE)
 def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torch.Tensor,
                                  response_mask: torch.Tensor, gamma, lam):
@@ -164,11 +174,18 @@ def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torc
         mom = torch.empty(5, dtype=torch.float64, device=dev)
         Lb = _cabi.lib()
         ws = _cabi.ticket_workspace(Lb.vamd_gae_workspace_bytes(B, Lc), dev)
-        with _cabi.device_guard(dev):
-            _cabi.check(Lb.vamd_gae(r.data_ptr(), v.data_ptr(), m.data_ptr(), code, B, Lc, float(gamma), float(lam),
-                                    1, adv.data_ptr(), ret.data_ptr(), mom.data_ptr(), ws.data_ptr(), ws.numel(),
-                                    _cabi.stream_ptr(dev)))
-        mom_host = mom.tolist()
+        for whiten in (1, 2):   # 1: one launch whose workgroups meet once; 2: two launches, nobody waits
+            with _cabi.device_guard(dev):
+                _cabi.check(Lb.vamd_gae(r.data_ptr(), v.data_ptr(), m.data_ptr(), code, B, Lc, float(gamma),
+                                        float(lam), whiten, adv.data_ptr(), ret.data_ptr(), mom.data_ptr(),
+                                        ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
+            mom_host = mom.tolist()
+            if mom_host[4] == 0.0:
+                break
+            # the workgroups' bounded wait for each other ran out (a GPU shared with long-running kernels): the
+            # advantages were left unwhitened; do it again without waiting
+            _warn_once("vamd_gae: the one-launch estimator timed out waiting for its workgroups; using two launches "
+                       "(set VAMD_WAITING_KERNELS=0 to make that the rule)")
         verl_F._raise_on_tiny_mask(mom_host[0])
         if mom_host[4] != 0.0:
             raise RuntimeError("vamd_gae: the workgroups' bounded wait for the whitening statistics ran out; "
