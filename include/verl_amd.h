@@ -8,9 +8,10 @@
  *     (workspace, workspace_bytes); the matching *_workspace_bytes() gives the size needed;
  *   - the reductions (masked moments, agg_loss, policy / value / KL loss, the advantage
  *     estimators) finish inside one launch through arrival counters in the FIRST
- *     VAMD_TICKET_BYTES of their workspace: those bytes must be zero on entry and are zero again
- *     when the call has completed, so a caller may zero a buffer once and reuse it for calls that
- *     are ordered on one stream;
+ *     VAMD_TICKET_BYTES of their workspace: those bytes must be zero on entry, or as an earlier
+ *     call of this library left them, and are zero again when the call has completed -- except the
+ *     32-bit word at byte 132, an epoch that vamd_grpo_advantage advances and nothing else reads --
+ *     so a caller may zero a buffer once and reuse it for calls that are ordered on one stream;
  *   - return value: 0 on success, a negative VAMD_E* code otherwise; vamd_last_error() returns a
  *     thread-local description of the last failure on the calling thread;
  *   - "mask" arguments come with a VAMD_MASK_* code naming their element type; the value used is

@@ -1053,6 +1053,9 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rows_kernel(GrpoRowsArgs a) {
   // 2048 x 16384); with one row each everybody finishes together and one launch-wide meeting is quicker (14.4
   // against 16.6 us at 512 x 4096).
   const bool by_group = gridDim.x < a.rows;
+  // read before anything else: whoever arrives last does so after this workgroup has arrived, hence after this load
+  const unsigned epoch_on_entry =
+      by_group ? 0u : __hip_atomic_load(a.ticket + kEpochWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   // One bit per mask element this workgroup owns, kept in LDS across the meeting when they fit, so that pass 2 only
   // stores.  A thread that met a mask value other than 0 and 1 reads its mask again instead.
   static_assert(kGroups * 4 <= 16, "one 16-bit word per thread and chunk");
@@ -1105,10 +1108,31 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rows_kernel(GrpoRowsArgs a) {
 #pragma unroll
   for (int r = 0; r < 2; ++r) member[r] = grpo_member_bits(a.gid, a.rows, (int64_t)blockIdx.x + (int64_t)r * gridDim.x);
   bool all_open = true;
-  if (!by_group) {  // one meeting of the whole launch; the last arrival opens the gate at once, there is nothing to fold
+  if (!by_group) {
+    // One meeting of the whole launch, with nothing to fold and nobody to report to (a row whose wait ran out is NaN),
+    // so it needs no departure count: the gate is an epoch word that the last arrival advances after it has put the
+    // arrival counters back to zero; the others wait for the word to differ from what they read on entry.
     const bool last = last_block_arrives(a.ticket);  // waits for this workgroup's stores first
-    if (last && threadIdx.x == 0) gate_release(a.ticket);
-    all_open = last || gate_wait(a.ticket, a.spin_limit);
+    if (last) {
+      ticket_reset(a.ticket);
+      if (threadIdx.x == 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __hip_atomic_store(a.ticket + kEpochWord, epoch_on_entry + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    } else {
+      __shared__ unsigned moved;
+      if (threadIdx.x == 0) {
+        unsigned seen = epoch_on_entry;
+        for (unsigned spins = 0;; ++spins) {
+          seen = __hip_atomic_load(a.ticket + kEpochWord, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (seen != epoch_on_entry || spins >= a.spin_limit) break;
+          __builtin_amdgcn_s_sleep(4);
+        }
+        moved = seen != epoch_on_entry ? 1u : 0u;
+      }
+      __syncthreads();
+      all_open = moved != 0u;
+    }
   }
   slot = 0;
   unsigned polls = 0;
@@ -1201,8 +1225,8 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rows_kernel(GrpoRowsArgs a) {
       }
     }
   }
-  // the last workgroup to leave clears the ready bytes with the counters: the area is zero again for the next call
-  if (gate_depart(a.ticket) != 0 && by_group)
+  // by group: the last workgroup to leave clears the ready bytes with the counters, zero again for the next call
+  if (by_group && gate_depart(a.ticket) != 0)
     for (int64_t w = threadIdx.x; w < (a.rows + 3) / 4; w += kRcThreads)  // four rows' bytes per word
       __hip_atomic_store(reinterpret_cast<unsigned*>(grpo_ready_byte(a.ticket, w * 4)), 0u, __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);

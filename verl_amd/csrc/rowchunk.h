@@ -262,6 +262,9 @@ __device__ __forceinline__ void ticket_reset(unsigned* counters) {
 // The words live inside the counter area: departures at word 16 of each counter's 256-byte slot, the release flag
 // at word 32 and the timed-out flag at word 48 of slot 0.
 constexpr int kDepartWord = 16, kReleaseWord = 32, kTimedOutWord = 48;
+// Word 33 of slot 0 is an epoch that only ever advances (a meeting without a departure count releases its waiters by
+// changing it): the one word of the area that is NOT zero between calls; nothing else reads it.
+constexpr int kEpochWord = 33;
 constexpr unsigned kGateSpinLimit = 1u << 22;  // polls of about half a microsecond: seconds, not forever
 
 __device__ __forceinline__ void gate_release(unsigned* counters) {  // thread 0, after its peer stores
