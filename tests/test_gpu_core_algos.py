@@ -386,6 +386,32 @@ def test_grpo_mask_kinds_over_chunked_and_shared_rows(dev, B, L, mask_kind):
     assert torch.equal(got.cpu() == 0, want == 0)
 
 
+@pytest.mark.parametrize("B,L,G,no_waiting", [(9000, 40, 3000, False), (9000, 40, 700, False), (5200, 37, 2400, True),
+                                             (3000, 5000, 300, True)])
+def test_grpo_on_the_several_launch_paths(dev, monkeypatch, B, L, G, no_waiting):
+    """Batches beyond what the one-launch kernel takes (8192 responses), and any batch with waiting kernels switched
+    off, go through row sums, group statistics (in LDS, or one thread per group beyond 2048 groups) and a broadcast."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    torch.manual_seed(B + G); random.seed(B + G); np.random.seed(B + G)
+    if no_waiting:
+        monkeypatch.setenv("VAMD_WAITING_KERNELS", "0")
+    index = _make_group_index(B, G)
+    mask = _rand_mask(B, L)
+    rewards = torch.randn(B, L) * mask
+    scores = rewards.double().sum(-1).numpy()
+    spread = np.zeros(G)
+    for gidx in range(G):
+        sel = scores[index == gidx]
+        spread[gidx] = np.ptp(sel) if len(sel) > 1 else 1.0
+    rows = torch.from_numpy(spread[index] > 1e-2)      # nearly tied groups are decided by fp32 rounding of a score
+    got, _ = CA.compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    w32, _ = O.grpo_outcome_advantage(rewards.clone(), mask, index)
+    w64, _ = O.grpo_outcome_advantage(rewards.double(), mask.double(), index)
+    err = (got.cpu().double() - w64)[rows].abs().max().item()
+    assert err <= max(2 * (w32.double() - w64)[rows].abs().max().item(), 2e-5), err
+    assert torch.equal(got.cpu() == 0, w32 == 0)
+
+
 def test_grpo_nearly_equal_scores_are_held_to_fp64(dev):
     """Two-member groups whose scores nearly coincide: (s - mean) / (std + eps) divides rounding noise by a tiny
     std, and the reference's own fp32 mean / std is then 1e-4 away from the exact value.  The kernel carries the
