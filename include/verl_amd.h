@@ -270,9 +270,11 @@ int vamd_gae(const float* rewards, const float* values, const void* mask, int ma
  * groupwise.as_torch_index does).  std_mode 0: unbiased torch.std (loop form); 1:
  * sqrt(clamp(var, min=eps)) (vectorised form).  scores_out [B] (may be NULL) receives the
  * normalised scalar per response.
- * Up to 2048 (row, 4096-column) pieces and 512 groups the estimator is one launch whose workgroups meet once
- * (bounded wait, as in vamd_gae); a workgroup whose wait runs out stores NaN advantages.  Larger inputs take a
- * row-sum launch, a statistics launch and a broadcast launch.
+ * Up to 8192 responses the estimator is one launch: every workgroup leaves its rows' scores in memory, waits
+ * (a bounded number of polls) for the scores of its groups' other members, and derives the group statistics
+ * itself; a workgroup whose wait runs out sums the members' rows itself, to the same bits, so the result does
+ * not depend on the launch's workgroups all running at once.  Larger batches, and VAMD_WAITING_KERNELS=0, take
+ * a row-sum launch, a statistics launch and a broadcast launch.
  */
 size_t vamd_grpo_workspace_bytes(int64_t batch, int64_t length, int64_t n_groups);
 int vamd_grpo_advantage(const float* rewards, const void* mask, int mask_dtype, const int64_t* group_ids,

@@ -1007,8 +1007,9 @@ __global__ __launch_bounds__(kRcThreads) void grpo_single_launch_kernel(const fl
 // scalar * mask.  Every workgroup repeats a little arithmetic, none waits for a single workgroup to do all of it.
 // Between the passes a workgroup waits either at one meeting of the whole launch or, when it walks several rows,
 // for the ready bytes of its groups' members only.  A workgroup that owns at most kGrpoHeldSlots chunks keeps its
-// mask as bits in LDS between the passes and only stores afterwards.  REQUIREMENT: the workgroups of the launch are
-// resident together; the waits are bounded, and a row whose wait ran out is stored as NaN.
+// mask as bits in LDS between the passes and only stores afterwards.  The waits are bounded; a
+// workgroup whose wait ran out (the launch's workgroups were not all running at once) sums the rows of its groups'
+// members itself, so the launch finishes with the right result whatever the device lets run together.
 constexpr int kGrpoHeldSlots = 32;  // chunks of one workgroup whose mask bits stay in LDS (16 KB)
 struct GrpoRowsArgs {
   const float* rewards;
@@ -1042,6 +1043,26 @@ __device__ __forceinline__ unsigned grpo_member_bits(const int64_t* __restrict__
       bits |= (gid[(int64_t)k * kRcThreads + threadIdx.x] == g ? 1u : 0u) << k;
   }
   return bits;
+}
+
+// The unmasked sum of one row of rewards, valid in thread 0: the same chunk order and workgroup reduction whoever
+// computes it, so that a workgroup that has to work out another row's score itself arrives at the same bits.
+template <bool VEC>
+__device__ __forceinline__ double grpo_row_sum(const float* __restrict__ rewards, int64_t row, int64_t cols, int chunks,
+                                               bool streaming, double* smem) {
+  double total = 0.0;
+  for (int c = 0; c < chunks; ++c) {
+    const ChunkPos pos(row, c, cols);
+    float v[kGroups][4];
+    load_groups<VEC>(rewards, pos, v, streaming);
+    float s = 0;
+#pragma unroll
+    for (int g = 0; g < kGroups; ++g) s += (v[g][0] + v[g][1]) + (v[g][2] + v[g][3]);
+    total += (double)s;
+  }
+  double acc[1] = {total};
+  block_sum<1, kRcThreads>(acc, smem);
+  return acc[0];
 }
 
 template <bool VEC, class M>
@@ -1109,7 +1130,7 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rows_kernel(GrpoRowsArgs a) {
   for (int r = 0; r < 2; ++r) member[r] = grpo_member_bits(a.gid, a.rows, (int64_t)blockIdx.x + (int64_t)r * gridDim.x);
   bool all_open = true;
   if (!by_group) {
-    // One meeting of the whole launch, with nothing to fold and nobody to report to (a row whose wait ran out is NaN),
+    // One meeting of the whole launch, with nothing to fold and nobody to report to (a workgroup whose wait ran out helps itself),
     // so it needs no departure count: the gate is an epoch word that the last arrival advances after it has put the
     // arrival counters back to zero; the others wait for the word to differ from what they read on entry.
     const bool last = last_block_arrives(a.ticket);  // waits for this workgroup's stores first
@@ -1138,7 +1159,7 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rows_kernel(GrpoRowsArgs a) {
   unsigned polls = 0;
   // two rows at a time: their group statistics share one pass over the scores and one workgroup reduction
   for (int64_t base = blockIdx.x; base < a.rows; base += 2 * (int64_t)gridDim.x) {
-    float scalar[2] = {__int_as_float(0x7fc00000), __int_as_float(0x7fc00000)};  // a wait that ran out stores NaN
+    float scalar[2] = {0.f, 0.f};
     if (base != blockIdx.x)
 #pragma unroll
       for (int r = 0; r < 2; ++r) member[r] = grpo_member_bits(a.gid, a.rows, base + (int64_t)r * gridDim.x);
@@ -1159,12 +1180,10 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rows_kernel(GrpoRowsArgs a) {
         }
       }
     const bool open = by_group ? __syncthreads_and(ready) != 0 : all_open;
-    if (by_group && !open && threadIdx.x == 0)
-      __hip_atomic_store(a.ticket + kTimedOutWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // count, sum and sum of squares of (score - own score) over the group: differences of fp32 scores are exact
+    // in double, and shifted by the row's own score the one-pass variance loses nothing to cancellation
+    double own[2], cs[6];
     if (open) {
-      // count, sum and sum of squares of (score - own score) over the group: differences of fp32 scores are exact
-      // in double, and shifted by the row's own score the one-pass variance loses nothing to cancellation
-      double own[2], cs[6];
 #pragma unroll
       for (int r = 0; r < 2; ++r) {
         const int64_t row = base + (int64_t)r * gridDim.x;
@@ -1179,6 +1198,28 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rows_kernel(GrpoRowsArgs a) {
         }
       }
       block_sum<6, kRcThreads>(cs, smem);
+    } else {
+      // The wait ran out (the launch's workgroups are not all running, say on a GPU that other work shares): this
+      // workgroup sums the rows of its groups' members itself, to the same bits their owners arrive at, and depends
+      // on nobody.  Every thread walks all responses; the sums of the members end up in thread 0.
+#pragma unroll
+      for (int r = 0; r < 2; ++r) {
+        const int64_t row = base + (int64_t)r * gridDim.x;
+        cs[3 * r] = cs[3 * r + 1] = cs[3 * r + 2] = 0.0;
+        own[r] = 0.0;
+        if (row >= a.rows) continue;
+        const int64_t g = a.gid[row];
+        own[r] = (double)(float)grpo_row_sum<VEC>(a.rewards, row, a.cols, a.chunks, streaming, smem);
+        for (int64_t i = 0; i < a.rows; ++i) {
+          if (a.gid[i] != g) continue;
+          const double d = (double)(float)grpo_row_sum<VEC>(a.rewards, i, a.cols, a.chunks, streaming, smem) - own[r];
+          cs[3 * r] += 1.0;
+          cs[3 * r + 1] += d;
+          cs[3 * r + 2] += d * d;
+        }
+      }
+    }
+    {
       if (threadIdx.x == 0) {
 #pragma unroll
         for (int r = 0; r < 2; ++r) {
@@ -1220,7 +1261,7 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rows_kernel(GrpoRowsArgs a) {
 #pragma unroll
         for (int g = 0; g < kGroups; ++g)
 #pragma unroll
-          for (int e = 0; e < 4; ++e) w[g][e] = open ? w[g][e] * scalar[r] : scalar[r];
+          for (int e = 0; e < 4; ++e) w[g][e] *= scalar[r];
         store_groups<VEC>(a.out, pos, w, streaming);
       }
     }
