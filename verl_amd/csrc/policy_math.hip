@@ -958,48 +958,6 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rowsum_kernel(const float* __
   }
 }
 
-// The whole estimator in ONE launch, for launches small enough that every workgroup is resident (the host checks):
-// a workgroup loads its 4096 columns of rewards AND of the mask, contributes its row-sum record, and the workgroup
-// that arrives last turns the records into the per-response scalars and opens the gate; the others wait there
-// (bounded), then every workgroup multiplies the mask it already holds by its row's scalar and stores.  A
-// workgroup whose wait runs out stores NaN: nothing downstream can mistake that for an advantage.
-template <bool VEC, class M>
-__global__ __launch_bounds__(kRcThreads) void grpo_single_launch_kernel(const float* __restrict__ x,
-                                                                        const M* __restrict__ mask, int64_t cols,
-                                                                        int chunks, Work wk, GrpoArgs ga,
-                                                                        float* __restrict__ out, unsigned spin_limit) {
-  const int64_t row = blockIdx.x / chunks;
-  const int chunk = blockIdx.x % chunks;
-  const ChunkPos pos(row, chunk, cols);
-  float v[kGroups][4], w[kGroups][4];
-  load_groups<VEC>(x, pos, v);
-  load_mask_groups<VEC>(mask, pos, w);
-  float s = 0;
-#pragma unroll
-  for (int g = 0; g < kGroups; ++g) s += (v[g][0] + v[g][1]) + (v[g][2] + v[g][3]);
-  __shared__ double smem[4];
-  double acc[1] = {s};
-  block_sum<1, kRcThreads>(acc, smem);
-  if (threadIdx.x == 0) store_record<1>(wk.partials, row, chunk, ga.rows, chunks, acc);
-  const bool last = last_block_arrives(wk.ticket);
-  if (last) {
-    __shared__ int g_cnt[kGrpoInlineGroups];
-    __shared__ double g_sum[kGrpoInlineGroups], g_sq[kGrpoInlineGroups];
-    grpo_scalars_from_records<true, 4, kRcThreads>(wk.partials, chunks, ga, g_cnt, g_sum, g_sq);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // every thread's scalars are on their way to memory ...
-    __syncthreads();                                     // ... before thread 0 opens the gate
-    if (threadIdx.x == 0) gate_release(wk.ticket);
-  }
-  const bool open = last || gate_wait(wk.ticket, spin_limit);
-  const float a = open ? peer_load_f32(ga.scalars + row) : __int_as_float(0x7fc00000);
-#pragma unroll
-  for (int g = 0; g < kGroups; ++g)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) w[g][e] = open ? w[g][e] * a : a;
-  store_groups<VEC>(out, pos, w);
-  gate_depart(wk.ticket);
-}
-
 // GRPO proper, up to a few thousand responses, in one launch without a serial statistics step: workgroup b owns rows
 // b, b + grid, ...  Pass 1 leaves every row's score (the unmasked row sum, fp32 like the reference's) in memory; in
 // pass 2 each workgroup finds the other members of its rows' groups by comparing the group ids (a few KB,
@@ -1922,26 +1880,6 @@ extern "C" int vamd_group_outcome_advantage(const float* rewards, const void* ma
     });
     VAMD_LAUNCH_CHECK();
     return VAMD_OK;
-  }
-  if (may_wait && n_groups <= kGrpoInlineGroups && batch * chunks <= kInlineFoldRecords) {
-    // one launch, if the device holds every workgroup of it at the same time
-    bool launched = false;
-    VAMD_MASK_DISPATCH(mask_dtype, M, {
-      const bool vec = can_vectorize(length, {rewards, advantages}, mask, sizeof(M));
-      auto go = [&](auto kernel) {
-        if (batch * chunks > resident_workgroups(reinterpret_cast<const void*>(kernel), kRcThreads)) return;
-        hipLaunchKernelGGL(kernel, dim3((unsigned)(batch * chunks)), dim3(kRcThreads), 0, s, rewards,
-                           static_cast<const M*>(mask), length, chunks, wk, ga, advantages,
-                           gate_spin_limit(kGateSpinLimit));
-        launched = true;
-      };
-      if (vec) go(grpo_single_launch_kernel<true, M>);
-      else go(grpo_single_launch_kernel<false, M>);
-    });
-    if (launched) {
-      VAMD_LAUNCH_CHECK();
-      return VAMD_OK;
-    }
   }
   // records per row of the row-sum pass: one per chunk, or one per row once there are enough rows to fill the device
   const int span = (batch >= 1024 && chunks > 1) ? chunks : 1;
