@@ -374,6 +374,25 @@ def _read_sclk_mhz():
     return None
 
 
+def _read_power_w():
+    """Board power in watts as the driver reports it (hwmon power1_input, microwatts), and the cap; (None, None) if
+    unreadable."""
+    import glob
+
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")):
+        try:
+            watts = int(open(path).read().strip()) / 1e6
+            cap = None
+            try:
+                cap = int(open(path.replace("power1_input", "power1_cap")).read().strip()) / 1e6
+            except (OSError, ValueError):
+                pass
+            return watts, cap
+        except (OSError, ValueError):
+            continue
+    return None, None
+
+
 def _sclk_sampler():
     """Background reader of the shader clock, for the ceiling probe: returns (stop, samples).  Reads sysfs, starts no
     other program."""
@@ -385,7 +404,7 @@ def _sclk_sampler():
         while not stop.is_set():
             mhz = _read_sclk_mhz()
             if mhz:
-                samples.append((time.time(), mhz))
+                samples.append((time.time(), mhz, _read_power_w()[0]))
             stop.wait(0.05)
 
     th = threading.Thread(target=run, daemon=True)
@@ -429,8 +448,11 @@ def mfma_ceiling_probe(dev, n: int, h: int, v: int, seconds: float = 1.5) -> dic
         torch.cuda.synchronize()
         t_end = time.time()
         ms = e0.elapsed_time(e1) / reps
-        clk = [m for (t, m) in samples if t_begin + 0.4 * (t_end - t_begin) <= t <= t_end]
-        return {"ms": ms, "PFLOPs": flops / ms / 1e12, "sclk_MHz": (sum(clk) / len(clk)) if clk else None}
+        late = [(m, p) for (t, m, p) in samples if t_begin + 0.4 * (t_end - t_begin) <= t <= t_end]
+        clk = [m for m, _ in late]
+        pw = [p for _, p in late if p is not None]
+        return {"ms": ms, "PFLOPs": flops / ms / 1e12, "sclk_MHz": (sum(clk) / len(clk)) if clk else None,
+                "board_W": (sum(pw) / len(pw)) if pw else None}
 
     for kind in ("zeros", "random"):
         if kind == "zeros":
@@ -458,8 +480,9 @@ def mfma_ceiling_probe(dev, n: int, h: int, v: int, seconds: float = 1.5) -> dic
         res[kind]["vendor_gemm_TN_d_weight"] = run_for(lambda: torch.matmul(z.t(), hid, out=dw), 2.0 * n * vc * h)
         del hid, w, wc, z, dh, dw
     stop.set()
-    res["note"] = ("ms per call; PFLOP/s on 2*M*N*K; sclk from the driver's sysfs table over the second half of each "
-                   "run (None when it cannot be read); vendor GEMMs on one 16384-column vocabulary chunk")
+    res["board_power_cap_W"] = _read_power_w()[1]
+    res["note"] = ("ms per call; PFLOP/s on 2*M*N*K; sclk and board power from the driver's sysfs files over the second "
+                   "half of each run (None when they cannot be read); vendor GEMMs on one 16384-column vocabulary chunk")
     return res
 
 

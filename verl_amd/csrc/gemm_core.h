@@ -3,16 +3,20 @@
 //
 // One workgroup = 512 threads = 8 wavefronts (two per SIMD, so that one wavefront's LDS traffic
 // and epilogue arithmetic issue in the shadow of the other's MFMAs) laid out 4 x 2 over a
-// 256 x 256 output tile; each wavefront owns a 64 (rows) x 128 (columns) sub-tile as 2 x 4
-// blocks of v_mfma_f32_32x32x16_bf16 (128 fp32 accumulators per lane).  The engine computes
+// 256 x 256 output tile; each wavefront owns a 64 (rows) x 128 (columns) sub-tile as 4 x 8
+// blocks of v_mfma_f32_16x16x32_bf16 (128 fp32 accumulators per lane).  The 16 x 16 x 32 shape is
+// chosen for energy: it touches half the accumulator registers per flop of the 32 x 32 x 16 shape,
+// and on operands that toggle the board sustains 2.12 against 1.87 PFLOP/s with it in a pure MFMA
+// loop (the clock this part holds is set by power, so flops per joule are flops per second).
+// The engine computes
 //
 //     Out[r][c] = sum_k  R[r][k] * C[c][k]
 //
 // where the R operand ("rows of the output") feeds the MFMA B input and the C operand
 // ("columns of the output") feeds the MFMA A input.  With that choice a lane of the accumulator
-// block holds ONE output row (r = lane % 32) and runs of 4 consecutive output columns, so
-// row-wise reductions over c (the softmax over the vocabulary) stay inside a lane and row-major
-// stores are 8/16-byte vectors.
+// block holds ONE output row (r = lane % 16) and 4 consecutive output columns (4 (lane / 16) ..),
+// so row-wise reductions over c (the softmax over the vocabulary) stay inside a lane and
+// row-major stores are 8/16-byte vectors.
 //
 // Operand slabs (256 x 64 k, 32 KB) travel from memory straight into LDS with
 // buffer_load_dwordx4 ... lds: no staging registers, no LDS store instructions, and a wavefront
@@ -42,26 +46,22 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kTile = 256;                    // output tile edge
 constexpr int kBK = 64;                       // k extent of one slab
-// Wavefronts along r: 4 (eight wavefronts of 64 x 128, two per SIMD) is what ships.  2 (four wavefronts of
-// 128 x 128, one per SIMD, accumulators in the 256 AGPRs) reads a third fewer fragments per MFMA and lets the board
-// clock 10 % higher on random data, but loses more than that at the per-slab barrier: forward 13.7 against 13.2 ms,
-// gradient GEMMs 33.0 against 27.3 ms per step at 16384 x 152064 x 3584.
-#ifndef VAMD_WAVES_R
-#define VAMD_WAVES_R 4
-#endif
-constexpr int kWavesR = VAMD_WAVES_R;         // wavefronts along r
+constexpr int kWavesR = 4;                    // wavefronts along r
 constexpr int kWavesC = 2;                    // wavefronts along c
 constexpr int kWaves = kWavesR * kWavesC;
 constexpr int kThreads = 64 * kWaves;
-constexpr int kNB = kTile / 32 / kWavesR;     // 32-row blocks per wavefront
-constexpr int kMB = kTile / 32 / kWavesC;     // 32-column blocks per wavefront (4)
-constexpr int kLoads = kTile * 8 / kThreads;  // 16-byte memory -> LDS transfers per lane per operand slab
-constexpr int kStepMfmas = kMB * kNB;         // MFMAs of one 16-k step of a wavefront
+constexpr int kBlk = 16;                      // edge of an MFMA output block
+constexpr int kNB = kTile / kBlk / kWavesR;   // 16-row blocks per wavefront    (4)
+constexpr int kMB = kTile / kBlk / kWavesC;   // 16-column blocks per wavefront (8)
+constexpr int kLoads = kTile * 8 / kThreads;  // 16-byte memory -> LDS transfers per lane per operand slab (4)
+constexpr int kSteps = kBK / 32;              // 32-k MFMA steps per slab (2)
 constexpr int kSlabBytes = kTile * kBK * 2;   // 32 KB
 constexpr int kLdsBytes = 4 * kSlabBytes;     // R,C x 2 stages = 128 KB
-static_assert(kMB == 4 && (kNB == 2 || kNB == 4), "FragAddr holds four block offsets");
-static_assert(kMB + kNB <= kStepMfmas && 2 * kLoads <= kStepMfmas, "a step has one slot per MFMA");
-static_assert((8 * kWaves) % 16 == 0 && (2 * kWaves) % 4 == 0, "the swizzles must not change between loads");
+static_assert(kNB == 4 && kMB == 8 && kLoads == 4 && kSteps == 2, "slab_iter's slot schedule is written for this layout");
+// A four-wavefront layout (128 x 128 per wavefront, one per SIMD) issues a third fewer LDS reads and lets the board
+// clock 10 % higher, but was measured slower: with one wavefront per SIMD nothing fills the cycles it spends at the
+// per-slab barrier and in the epilogue (forward 13.7 against 13.2 ms, gradient GEMMs 33.0 against 27.3 ms per step at
+// 16384 x 152064 x 3584 with the 32 x 32 x 16 instruction).
 
 // One GEMM operand as the tile engine sees it.
 struct Operand {
@@ -72,7 +72,7 @@ struct Operand {
 };
 
 struct Accum {
-  f32x16 a[kMB][kNB];  // [mb: 32-wide block along c][nb: 32-wide block along r]
+  f32x4 a[kMB][kNB];  // [mb: 16-wide block along c][nb: 16-wide block along r]
 };
 
 __device__ __forceinline__ void accum_zero(Accum& acc) {
@@ -81,15 +81,15 @@ __device__ __forceinline__ void accum_zero(Accum& acc) {
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc.a[mb][nb][v] = 0.f;
+      for (int v = 0; v < 4; ++v) acc.a[mb][nb][v] = 0.f;
 }
 
 // Position of the calling lane inside the workgroup tile.
 struct LanePos {
   int wr;  // wavefront's quarter along r (0..3)
   int wc;  // wavefront's half along c (0/1)
-  int lr;  // lane % 32 : r offset inside a 32-block
-  int lh;  // lane / 32 : which 4-column group of every 8 the lane holds
+  int lx;  // lane % 16 : r offset inside a 16-block
+  int lq;  // lane / 16 : which 4-column group of a block's 16 the lane holds
 };
 
 __device__ __forceinline__ LanePos lane_pos() {
@@ -98,17 +98,17 @@ __device__ __forceinline__ LanePos lane_pos() {
   const int w = t >> 6;
   p.wr = w % kWavesR;
   p.wc = w / kWavesR;
-  p.lr = t & 31;
-  p.lh = (t >> 5) & 1;
+  p.lx = t & 15;
+  p.lq = (t >> 4) & 3;
   return p;
 }
 
 // Column offset inside the 256-wide tile of accumulator element (mb, v) for this lane.
 __device__ __forceinline__ int acc_col(const LanePos& p, int mb, int v) {
-  return p.wc * (kMB * 32) + mb * 32 + 8 * (v >> 2) + 4 * p.lh + (v & 3);
+  return p.wc * (kMB * kBlk) + mb * kBlk + 4 * p.lq + v;
 }
 // Row offset inside the 256-tall tile of accumulator block nb for this lane.
-__device__ __forceinline__ int acc_row(const LanePos& p, int nb) { return p.wr * (kNB * 32) + nb * 32 + p.lr; }
+__device__ __forceinline__ int acc_row(const LanePos& p, int nb) { return p.wr * (kNB * kBlk) + nb * kBlk + p.lx; }
 
 // ---------------------------------------------------------------------------------------------
 // LDS layouts and their swizzles.
@@ -203,112 +203,106 @@ struct SlabDma {
 };
 
 // ---------------------------------------------------------------------------------------------
-// Per-lane LDS addressing of MFMA fragments.  A fragment is the 8 consecutive k (k = 16 s + 8 lh
-// + 0..7 of k-step s) of slab row x = 32 * block + lr.
-//   direct : one ds_read_b128 at  x * 128 + (((2 s + lh) ^ swizzle(x)) << 4);
-//   kmajor : two transposing 8-byte reads.  Within 16 lanes, lane i addresses the 8 bytes at
-//            (k row k0 + i / 4, x0 + 4 (i % 4)) and receives the 4 k of x0 + i; lanes 0-15 /
-//            16-31 take x0 = 0 / 16 of the block, lanes 32-63 the k-half lh = 1.
+// Per-lane LDS addressing of MFMA fragments.  A fragment of the 16 x 16 x 32 instruction is, for lane
+// (lx = lane % 16, lq = lane / 16), the 8 consecutive k (k = 32 s + 8 lq + 0..7 of k-step s) of slab row
+// x = 16 * block + lx.
+//   direct : one ds_read_b128 at  x * 128 + (((4 s + lq) ^ swizzle(x)) << 4);
+//   kmajor : two transposing 8-byte reads.  Within the 16 lanes of one lq, lane i addresses the 8 bytes at
+//            (k row k0 + i / 4, x0 + 4 (i % 4)) and receives the 4 k (k0 .. k0 + 3) of x0 + i; the second read
+//            takes k0 + 4.
 template <bool KMAJOR>
 struct FragAddr {
-  // direct: off[s] = lane part for k-step s, block adds 4096 b.  kmajor: off[b] = lane part for
-  // block b of the wavefront, k-step adds 8192 s (+ 2048 for the second read).
-  int off[4];
+  // direct: off[s] = lane part for k-step s, block adds 2048 b.  kmajor: off[b] = lane part for
+  // block b of the wavefront, k-step adds 16384 s (+ 2048 for the second read).
+  int off[KMAJOR ? kMB : kSteps];
 
-  // first_block: index of the wavefront's first 32-row block inside the slab
+  // first_block: index of the wavefront's first 16-row block inside the slab
   __device__ __forceinline__ void init(int first_block, int nblocks) {
     const int l = threadIdx.x & 63;
+    const int lx = l & 15, lq = l >> 4;
     if constexpr (!KMAJOR) {
-      const int lr = l & 31, lh = l >> 5;
 #pragma unroll
-      for (int s = 0; s < 4; ++s) off[s] = (first_block * 32 + lr) * 128 + (((2 * s + lh) ^ swizzle_direct(lr)) << 4);
+      for (int s = 0; s < kSteps; ++s)
+        off[s] = (first_block * kBlk + lx) * 128 + (((4 * s + lq) ^ swizzle_direct(lx)) << 4);
     } else {
-      const int g = l >> 4, i = l & 15;
-      const int q = i >> 2;                       // (k & 3) of the addressed row: every k offset is a multiple of 4
-      const int k0 = 8 * (g >> 1) + q;
-      const int x_in_blk = 16 * (g & 1) + 4 * (i & 3);
+      const int q = lx >> 2;  // (k & 3) of the addressed row: every k offset added later is a multiple of 4
+      const int k0 = 8 * lq + q;
 #pragma unroll
-      for (int b = 0; b < 4; ++b)
-        off[b] = b < nblocks ? k0 * 512 + 64 * ((first_block + b) ^ q) + 2 * x_in_blk : 0;
+      for (int b = 0; b < kMB; ++b) {
+        const int blk = first_block + b;
+        off[b] = b < nblocks ? k0 * 512 + 64 * ((blk >> 1) ^ q) + 32 * (blk & 1) + 8 * (lx & 3) : 0;
+      }
     }
   }
 
   __device__ __forceinline__ bf16x8 read(const char* slab, int s, int b) const {
     if constexpr (!KMAJOR) {
-      return *reinterpret_cast<const bf16x8*>(slab + off[s] + b * 4096);
+      return *reinterpret_cast<const bf16x8*>(slab + off[s] + b * (kBlk * 128));
     } else {
       typedef bf16x4 __attribute__((address_space(3))) * tr_ptr_t;
-      const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((tr_ptr_t)(slab + off[b] + s * 8192));
-      const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((tr_ptr_t)(slab + off[b] + s * 8192 + 2048));
+      const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((tr_ptr_t)(slab + off[b] + s * 16384));
+      const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((tr_ptr_t)(slab + off[b] + s * 16384 + 2048));
       return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     }
   }
 };
 
-// MFMA fragments of one 16-k step: kMB blocks of C and kNB blocks of R.
+// MFMA fragments in flight.  The kNB blocks of R of both k-steps of a slab are held whole; the blocks of C stream
+// through a ring of four: group G of a slab (G = 8 * k-step + mb, four MFMAs each) reads ring slot G % 4.
 struct Frags {
-  bf16x8 c[kMB], r[kNB];
+  bf16x8 r[kSteps][kNB];
+  bf16x8 c[4];
 };
 
 // ---------------------------------------------------------------------------------------------
-// One slab (64 k = four 16-k steps of 8 MFMAs per wavefront) of the software pipeline.
+// One slab (64 k = two 32-k steps of 32 MFMAs per wavefront) of the software pipeline.
 //
-// The body is written as 32 slots "one MFMA + at most one memory instruction group", each closed
-// by a scheduling barrier so the compiler keeps the order:
+// The body is 64 slots "one MFMA + at most two memory instruction groups", each closed by a scheduling barrier so
+// the compiler keeps the order.  Slot j = 4 G + nb multiplies block (mb = G % 8, nb) of k-step G / 8.
 //
-//   step 0..2 : MFMAs of step s | fragment reads of step s + 1 from `cur`
-//   -- wait for this wavefront's transfers of slab it+1, workgroup barrier --
-//   step 3    : MFMAs of step 3 | step-0 fragment reads of slab it+1 from `nxt`
-//                               | transfers of slab it+2 into `cur` (every wavefront has its last
-//                                 fragments of `cur` in registers once the barrier is passed)
+//   slots  0..51 : the C fragment of group G + 3 is read from `cur` in the first slot of group G (its ring slot was
+//                  last used by group G - 1); the R fragments of k-step 1 are read in groups 1..4
+//   after slot 55: wait for this wavefront's LDS reads and for its transfers of slab it+1, workgroup barrier:
+//                  nobody reads `cur` any more, and `nxt` is complete
+//   slots 56..63 : the fragments the next slab starts with (R of k-step 0, C of groups 0..2) are read from `nxt`,
+//                  and the transfers of slab it+2 into `cur` are issued
 //
-// so a transfer has three steps of MFMA work to land before anyone waits for it, and nothing
-// inside the steps depends on memory.
+// so a transfer has 56 slots of MFMA work to land before anyone waits for it, and nothing inside the slots depends on
+// memory.  On entry f holds R of k-step 0 and C of groups 0..2 of this slab.
 template <bool RK, bool CK>
 __device__ __forceinline__ void slab_iter(const SlabDma<RK>& dr, const SlabDma<CK>& dc, const SlabSrc& r2,
                                           const SlabSrc& c2, char* cur, const char* nxt, const FragAddr<RK>& fr,
-                                          const FragAddr<CK>& fc, Frags& f0, Accum& acc) {
-  Frags f1;
-#define VAMD_MFMA(F, i)                                                                                              \
-  acc.a[(i) / kNB][(i) % kNB] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(F.c[(i) / kNB], F.r[(i) % kNB],                 \
-                                                                        acc.a[(i) / kNB][(i) % kNB], 0, 0, 0)
-#define VAMD_FRAG(G, base, i, s)                                            \
-  do {                                                                      \
-    if ((i) < kMB) G.c[(i)] = fc.read((base) + kSlabBytes, (s), (i));        \
-    else if ((i) < kMB + kNB) G.r[(i) - kMB] = fr.read((base), (s), (i) - kMB); \
-  } while (0)
-#define VAMD_SLOT_END __builtin_amdgcn_sched_barrier(0)
+                                          const FragAddr<CK>& fc, Frags& f, Accum& acc) {
 #pragma unroll
-  for (int i = 0; i < kStepMfmas; ++i) {
-    VAMD_MFMA(f0, i);
-    VAMD_FRAG(f1, cur, i, 1);
-    VAMD_SLOT_END;
+  for (int j = 0; j < 64; ++j) {
+    const int G = j >> 2, nb = j & 3, ks = G >> 3, mb = G & 7;
+    acc.a[mb][nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.c[G & 3], f.r[ks][nb], acc.a[mb][nb], 0, 0, 0);
+    if (j < 52) {
+      if (nb == 0) {
+        const int g3 = G + 3;  // <= 15: still this slab
+        f.c[g3 & 3] = fc.read(cur + kSlabBytes, g3 >> 3, g3 & 7);
+      }
+      if (nb == 1 && G >= 1 && G <= kNB) f.r[1][G - 1] = fr.read(cur, 1, G - 1);
+    } else if (j >= 56) {
+      const int k = j - 56;
+      if (k == 0) f.c[0] = fc.read(nxt + kSlabBytes, 0, 0);
+      if (k < kNB) f.r[0][k] = fr.read(nxt, 0, k);
+      if (k == 4) f.c[1] = fc.read(nxt + kSlabBytes, 0, 1);
+      if (k == 5) f.c[2] = fc.read(nxt + kSlabBytes, 0, 2);
+      // eight transfers over slots 57..63: one each in 57..60, two each in 62 and 63, none beside the reads of 56 and 61
+      if (k >= 1 && k <= 4) dr.issue_one(k - 1, r2, lds_address(cur));
+      if (k == 6) {
+        dc.issue_one(0, c2, lds_address(cur) + kSlabBytes);
+        dc.issue_one(1, c2, lds_address(cur) + kSlabBytes);
+      }
+      if (k == 7) {
+        dc.issue_one(2, c2, lds_address(cur) + kSlabBytes);
+        dc.issue_one(3, c2, lds_address(cur) + kSlabBytes);
+      }
+    }
+    if (j == 55) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
   }
-#pragma unroll
-  for (int i = 0; i < kStepMfmas; ++i) {
-    VAMD_MFMA(f1, i);
-    VAMD_FRAG(f0, cur, i, 2);
-    VAMD_SLOT_END;
-  }
-#pragma unroll
-  for (int i = 0; i < kStepMfmas; ++i) {
-    VAMD_MFMA(f0, i);
-    VAMD_FRAG(f1, cur, i, 3);
-    VAMD_SLOT_END;
-  }
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  VAMD_SLOT_END;
-#pragma unroll
-  for (int i = 0; i < kStepMfmas; ++i) {
-    VAMD_MFMA(f1, i);
-    VAMD_FRAG(f0, nxt, i, 0);
-    if (i < kLoads) dr.issue_one(i, r2, lds_address(cur));
-    else if (i < 2 * kLoads) dc.issue_one(i - kLoads, c2, lds_address(cur) + kSlabBytes);
-    VAMD_SLOT_END;
-  }
-#undef VAMD_MFMA
-#undef VAMD_FRAG
-#undef VAMD_SLOT_END
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -373,11 +367,11 @@ __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, in
   }
   advance();  // cursor now on slab 2
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-  Frags f0;
+  Frags f;
 #pragma unroll
-  for (int i = 0; i < kMB; ++i) f0.c[i] = fc.read(lds + kSlabBytes, 0, i);
+  for (int i = 0; i < kNB; ++i) f.r[0][i] = fr.read(lds, 0, i);
 #pragma unroll
-  for (int i = 0; i < kNB; ++i) f0.r[i] = fr.read(lds, 0, i);
+  for (int i = 0; i < 3; ++i) f.c[i] = fc.read(lds + kSlabBytes, 0, i);
 
   int stage = 0;
   for (int tile = 0; tile < ntiles; ++tile) {
@@ -387,7 +381,7 @@ __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, in
     for (int kt = 0; kt < k_slabs; ++kt) {
       char* cur = lds + stage * 2 * kSlabBytes;
       const char* nxt = lds + (stage ^ 1) * 2 * kSlabBytes;
-      slab_iter<R_KMAJOR, C_KMAJOR>(dr, dc, src_r, src_c, cur, nxt, fr, fc, f0, acc);
+      slab_iter<R_KMAJOR, C_KMAJOR>(dr, dc, src_r, src_c, cur, nxt, fr, fc, f, acc);
       advance();
       stage ^= 1;
     }

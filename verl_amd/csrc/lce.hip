@@ -87,7 +87,49 @@ struct SplitSched {
   }
 };
 
-constexpr int kCacheStageBytes = (kThreads / 64) * 4096;  // one 32 x 32 fp32 block per wavefront
+// The epilogues that write matrices hand the accumulators through a 4 KB LDS patch private to the
+// wavefront (the 32 KB the pipeline leaves free), 32 x 32 values at a time (2 x 2 MFMA blocks), so that
+// global accesses are whole 128-byte rows of fp32 (64-byte rows of bf16) touched by 8 consecutive
+// lanes instead of 16-byte pieces of 16 different rows.  After the exchange lane L holds columns
+// 4 (L % 8) .. + 3 of rows 8 i + L / 8 (i = 0..3) of the 32 x 32 patch.  LDS operations of one wavefront
+// execute in issue order, so the patch needs no barrier, only the waits that order its writes and reads.
+constexpr int kNB2 = kNB / 2, kMB2 = kMB / 2;  // 32 x 32 patches per wavefront along r and c
+struct BlockExchange {
+  char* stage;  // this wavefront's patch
+  int lx, lq, rd_row, rd_chunk;
+  __device__ __forceinline__ void init(char* lds_after_pipeline, const LanePos& p) {
+    stage = lds_after_pipeline + (threadIdx.x >> 6) * 4096;
+    lx = p.lx;
+    lq = p.lq;
+    rd_row = (threadIdx.x & 63) >> 3;
+    rd_chunk = threadIdx.x & 7;
+  }
+  // blk[cb][rb]: the four 16 x 16 blocks of the patch, cb along c, rb along r
+  __device__ __forceinline__ void run(const f32x4 (&blk)[2][2], f32x4 (&out)[4]) const {
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+        const int row = 16 * rb + lx;
+        *reinterpret_cast<f32x4*>(stage + row * 128 + (((4 * cb + lq) ^ ((row >> 1) & 7)) << 4)) = blk[cb][rb];
+      }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 8 * i + rd_row;
+      out[i] = *reinterpret_cast<const f32x4*>(stage + row * 128 + ((rd_chunk ^ ((row >> 1) & 7)) << 4));
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+  // the patch (mb2, nb2) of an accumulator
+  __device__ __forceinline__ void run(const Accum& acc, int mb2, int nb2, f32x4 (&out)[4]) const {
+    const f32x4 blk[2][2] = {{acc.a[2 * mb2][2 * nb2], acc.a[2 * mb2][2 * nb2 + 1]},
+                             {acc.a[2 * mb2 + 1][2 * nb2], acc.a[2 * mb2 + 1][2 * nb2 + 1]}};
+    run(blk, out);
+  }
+};
+
+constexpr int kCacheStageBytes = (kThreads / 64) * 4096;  // one 32 x 32 fp32 patch per wavefront
 
 // Per-lane online-softmax state for the kNB token slots (nb) the lane owns.  With CACHE the
 // scaled logits of every valid (token, vocabulary column) are also written out in fp32, so the
@@ -103,54 +145,43 @@ struct FwdEpi {
   int lab[kNB];
   float rcp_t;
   float* z_cache;  // CACHE: [n_tokens][vocab]
-  char* stage;     // CACHE: this wavefront's 4 KB LDS patch
+  BlockExchange ex;  // CACHE
   int tok0;        // CACHE: first token row of the wavefront
   int n_tokens;
 
   __device__ __forceinline__ void operator()(Accum& acc, int /*r0*/, int c0) {
     const bool ragged = c0 + kTile > vocab;
+    if constexpr (CACHE) {
 #pragma unroll
-    for (int nb = 0; nb < kNB; ++nb) {
-      if constexpr (CACHE) {
-        // Each 32 x 32 block goes through a 4 KB LDS patch private to the wavefront so that the
-        // global stores are whole 128-byte rows (8 lanes x 16 bytes) instead of 16-byte pieces of
-        // 32 different rows.  LDS operations of one wavefront execute in issue order, so the
-        // patch needs no barrier, only the waits that order its writes and reads.
-        const int lane = threadIdx.x & 63;
-        const int rd_row = lane >> 3, rd_chunk = lane & 7;
+      for (int nb2 = 0; nb2 < kNB2; ++nb2)
 #pragma unroll
-        for (int mb = 0; mb < kMB; ++mb) {
+        for (int mb2 = 0; mb2 < kMB2; ++mb2) {
+          f32x4 blk[2][2];
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            const f32x4 z = {acc.a[mb][nb][4 * g] * rcp_t, acc.a[mb][nb][4 * g + 1] * rcp_t,
-                             acc.a[mb][nb][4 * g + 2] * rcp_t, acc.a[mb][nb][4 * g + 3] * rcp_t};
-            *reinterpret_cast<f32x4*>(stage + p.lr * 128 + (((2 * g + p.lh) ^ ((p.lr >> 1) & 7)) << 4)) = z;
-          }
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) blk[cb][rb] = acc.a[2 * mb2 + cb][2 * nb2 + rb] * rcp_t;
           f32x4 out[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const int row = 8 * i + rd_row;
-            out[i] = *reinterpret_cast<const f32x4*>(stage + row * 128 + ((rd_chunk ^ ((row >> 1) & 7)) << 4));
-          }
-          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-          const int col = c0 + p.wc * 128 + mb * 32 + 4 * rd_chunk;
+          ex.run(blk, out);
+          const int col = c0 + p.wc * 128 + mb2 * 32 + 4 * ex.rd_chunk;
           if (col < vocab) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-              const int tok = tok0 + nb * 32 + 8 * i + rd_row;
+              const int tok = tok0 + nb2 * 32 + 8 * i + ex.rd_row;
               if (tok < n_tokens)
                 __builtin_nontemporal_store(out[i], reinterpret_cast<f32x4*>(z_cache + (int64_t)tok * vocab + col));
             }
           }
         }
-      }
+    }
+#pragma unroll
+    for (int nb = 0; nb < kNB; ++nb) {
       float ymax = kNegBig;
       // pass 1: scale into the log2 domain in place, mask the vocabulary tail, tile max
 #pragma unroll
       for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
+        for (int v = 0; v < 4; ++v) {
           float y = acc.a[mb][nb][v] * scale2;
           if (ragged) y = (c0 + acc_col(p, mb, v) < vocab) ? y : kNegBig;
           acc.a[mb][nb][v] = y;
@@ -162,8 +193,8 @@ struct FwdEpi {
 #pragma unroll
         for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int col = mb * 32 + 8 * (v >> 2) + 4 * p.lh + (v & 3);
+          for (int v = 0; v < 4; ++v) {
+            const int col = mb * kBlk + 4 * p.lq + v;
             zl[nb] += (col == rel) ? acc.a[mb][nb][v] * kLn2 : 0.f;
           }
       }
@@ -173,7 +204,7 @@ struct FwdEpi {
 #pragma unroll
       for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
+        for (int v = 0; v < 4; ++v) {
           const float y = acc.a[mb][nb][v];
           const float e = fast_exp2(y - m_new);
           s_ += e;
@@ -241,33 +272,35 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
     epi.lab[nb] = tok < a.n_tokens ? (int)a.labels[tok] : -1;
   }
   epi.z_cache = a.z_cache;
-  epi.stage = lds + kLdsBytes + (threadIdx.x >> 6) * 4096;
-  epi.tok0 = sched.r0_ + epi.p.wr * (kNB * 32);
+  epi.ex.init(lds + kLdsBytes, epi.p);
+  epi.tok0 = sched.r0_ + epi.p.wr * (kNB * kBlk);
   epi.n_tokens = a.n_tokens;
 
   run_tiles<false, false>(a.hidden, a.weight, a.k_slabs, sched, epi, lds);
 
-  // merge the two lane halves (they hold disjoint vocabulary columns of the same token) ...
+  // merge the four lane quarters (they hold disjoint vocabulary columns of the same token) ...
 #pragma unroll
-  for (int nb = 0; nb < kNB; ++nb) {
-    const float m2 = __shfl_xor(epi.m[nb], 32, 64);
-    const float s2 = __shfl_xor(epi.s[nb], 32, 64);
-    const float sy2 = __shfl_xor(epi.sy[nb], 32, 64);
-    const float z2 = __shfl_xor(epi.zl[nb], 32, 64);
-    if (PI2) {
-      const float q2 = __shfl_xor(epi.s2[nb], 32, 64);
-      merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], epi.s2[nb], m2, s2, sy2, q2);
-    } else {
-      merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], m2, s2, sy2);
+  for (int step = 16; step <= 32; step *= 2)
+#pragma unroll
+    for (int nb = 0; nb < kNB; ++nb) {
+      const float m2 = __shfl_xor(epi.m[nb], step, 64);
+      const float s2 = __shfl_xor(epi.s[nb], step, 64);
+      const float sy2 = __shfl_xor(epi.sy[nb], step, 64);
+      const float z2 = __shfl_xor(epi.zl[nb], step, 64);
+      if (PI2) {
+        const float q2 = __shfl_xor(epi.s2[nb], step, 64);
+        merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], epi.s2[nb], m2, s2, sy2, q2);
+      } else {
+        merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], m2, s2, sy2);
+      }
+      epi.zl[nb] += z2;
     }
-    epi.zl[nb] += z2;
-  }
   // ... then the two wavefronts that share a token quarter (wc = 0/1), through LDS (once every
   // wavefront's last slab transfers have landed).
   __syncthreads();
   float4* red = reinterpret_cast<float4*>(lds);                     // [2][256]
   float* redq = reinterpret_cast<float*>(lds + 2 * kTile * 16);    // [2][256] squared sums
-  if (epi.p.lh == 0) {
+  if (epi.p.lq == 0) {
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
       red[epi.p.wc * kTile + acc_row(epi.p, nb)] = make_float4(epi.m[nb], epi.s[nb], epi.sy[nb], epi.zl[nb]);
@@ -335,36 +368,6 @@ __device__ __forceinline__ u32x2 pack_bf16x4(float a, float b, float c, float d)
 
 __device__ __forceinline__ float bf16_bits_to_float(unsigned h) { return __uint_as_float(h << 16); }
 
-// The backward epilogues hand each 32 x 32 accumulator block through a 4 KB LDS patch private to the
-// wavefront (the 32 KB the pipeline leaves free), so that global accesses are whole 128-byte rows
-// of fp32 (64-byte rows of bf16) touched by 8 consecutive lanes instead of 16-byte pieces of 32
-// different rows.  After the exchange lane L holds columns 4 (L % 8) .. + 3 of rows 8 i + L / 8.
-struct BlockExchange {
-  char* stage;  // this wavefront's patch
-  int lr, lh, rd_row, rd_chunk;
-  __device__ __forceinline__ void init(char* lds_after_pipeline, const LanePos& p) {
-    stage = lds_after_pipeline + (threadIdx.x >> 6) * 4096;
-    lr = p.lr;
-    lh = p.lh;
-    rd_row = (threadIdx.x & 63) >> 3;
-    rd_chunk = threadIdx.x & 7;
-  }
-  __device__ __forceinline__ void run(const f32x16& blk, f32x4 (&out)[4]) const {
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 v = {blk[4 * g], blk[4 * g + 1], blk[4 * g + 2], blk[4 * g + 3]};
-      *reinterpret_cast<f32x4*>(stage + lr * 128 + (((2 * g + lh) ^ ((lr >> 1) & 7)) << 4)) = v;
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row = 8 * i + rd_row;
-      out[i] = *reinterpret_cast<const f32x4*>(stage + row * 128 + ((rd_chunk ^ ((row >> 1) & 7)) << 4));
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  }
-};
-
 struct RecomputeArgs {
   Operand hidden;  // R: [n_tokens][H]
   Operand weight;  // C: rows of this vocabulary chunk, x_extent = vocab - chunk_c0
@@ -389,38 +392,50 @@ struct RecomputeEpi {
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const RecomputeArgs& A = *a;
 #pragma unroll
-    for (int nb = 0; nb < kNB; ++nb) {
-      const int tok = r0 + acc_row(p, nb);
-      const bool live = tok < A.n_tokens;
-      float lse2 = 0.f, mz = 0.f, glp = 0.f, gent = 0.f;
-      int rel = -1;
-      if (live) {
-        lse2 = A.lse[tok] * kLog2e;
-        mz = A.mean_z[tok];
-        glp = (A.g_lp ? A.g_lp[tok] : 0.f) * A.rcp_t;
-        gent = (A.g_ent ? A.g_ent[tok] : A.g_ent_scalar) * A.rcp_t;
-        rel = (int)A.labels[tok] - A.chunk_c0 - c0 - p.wc * 128;
-      }
-      const bool hit = __any(rel >= 0 && rel < 128);
+    for (int nb2 = 0; nb2 < kNB2; ++nb2) {
+      // the lane's two token rows of this 32-row patch
+      float lse2[2], mz[2], glp[2], gent[2];
+      int rel[2];
+      bool live[2];
 #pragma unroll
-      for (int mb = 0; mb < kMB; ++mb) {
-        f32x16 d;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const float x = acc.a[mb][nb][v];
-          const float prob = fast_exp2(fmaf(x, A.scale2, -lse2));
-          const float u = fmaf(gent, fmaf(x, A.rcp_t, -mz), glp);  // g_lp/T + g_ent/T * (z - mean_z)
-          float dzv = -prob * u;
-          const int col = mb * 32 + 8 * (v >> 2) + 4 * p.lh + (v & 3);
-          if (hit) dzv += (col == rel) ? glp : 0.f;
-          const bool ok = live && (c0 + p.wc * 128 + col) < A.vocab_left;
-          d[v] = ok ? dzv : 0.f;
+      for (int rb = 0; rb < 2; ++rb) {
+        const int tok = r0 + acc_row(p, 2 * nb2 + rb);
+        live[rb] = tok < A.n_tokens;
+        lse2[rb] = mz[rb] = glp[rb] = gent[rb] = 0.f;
+        rel[rb] = -1;
+        if (live[rb]) {
+          lse2[rb] = A.lse[tok] * kLog2e;
+          mz[rb] = A.mean_z[tok];
+          glp[rb] = (A.g_lp ? A.g_lp[tok] : 0.f) * A.rcp_t;
+          gent[rb] = (A.g_ent ? A.g_ent[tok] : A.g_ent_scalar) * A.rcp_t;
+          rel[rb] = (int)A.labels[tok] - A.chunk_c0 - c0 - p.wc * 128;
         }
+      }
+      const bool hit = __any((rel[0] >= 0 && rel[0] < 128) || (rel[1] >= 0 && rel[1] < 128));
+#pragma unroll
+      for (int mb2 = 0; mb2 < kMB2; ++mb2) {
+        f32x4 d[2][2];
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+          for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+              const int mb = 2 * mb2 + cb;
+              const float x = acc.a[mb][2 * nb2 + rb][v];
+              const float prob = fast_exp2(fmaf(x, A.scale2, -lse2[rb]));
+              const float u = fmaf(gent[rb], fmaf(x, A.rcp_t, -mz[rb]), glp[rb]);  // g_lp/T + g_ent/T * (z - mean_z)
+              float dzv = -prob * u;
+              const int col = mb * kBlk + 4 * p.lq + v;
+              if (hit) dzv += (col == rel[rb]) ? glp[rb] : 0.f;
+              const bool ok = live[rb] && (c0 + p.wc * 128 + col) < A.vocab_left;
+              d[cb][rb][v] = ok ? dzv : 0.f;
+            }
         // every row of the panel is written, padding rows and columns as zeros
         f32x4 o[4];
         ex.run(d, o);
-        const int col0 = c0 + p.wc * 128 + mb * 32 + 4 * ex.rd_chunk;
-        const int64_t row0 = r0 + p.wr * (kNB * 32) + nb * 32 + ex.rd_row;
+        const int col0 = c0 + p.wc * 128 + mb2 * 32 + 4 * ex.rd_chunk;
+        const int64_t row0 = r0 + p.wr * (kNB * kBlk) + nb2 * 32 + ex.rd_row;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
           *reinterpret_cast<u32x2*>(A.dz + (row0 + 8 * i) * A.dz_ld + col0) =
@@ -511,14 +526,14 @@ struct DHiddenEpi {
     const bool read_prev = A.mode == kAddF32 || A.mode == kFinalBf16AddPrev;
     const bool to_f32 = A.mode == kStoreF32 || A.mode == kAddF32;
 #pragma unroll
-    for (int nb = 0; nb < kNB; ++nb)
+    for (int nb = 0; nb < kNB2; ++nb)
 #pragma unroll
-      for (int mb = 0; mb < kMB; ++mb) {
+      for (int mb = 0; mb < kMB2; ++mb) {
         f32x4 v[4];
-        ex.run(acc.a[mb][nb], v);
+        ex.run(acc, mb, nb, v);
         const int col = c0 + p.wc * 128 + mb * 32 + 4 * ex.rd_chunk;
         if (col >= A.c_valid) continue;
-        const int row0 = r0 + p.wr * (kNB * 32) + nb * 32 + ex.rd_row;
+        const int row0 = r0 + p.wr * (kNB * kBlk) + nb * 32 + ex.rd_row;
         f32x4 prev[4];
         if (read_prev) {
 #pragma unroll
@@ -548,14 +563,14 @@ struct DWeightEpi {
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const GemmOutArgs& A = *a;
 #pragma unroll
-    for (int nb = 0; nb < kNB; ++nb)
+    for (int nb = 0; nb < kNB2; ++nb)
 #pragma unroll
-      for (int mb = 0; mb < kMB; ++mb) {
+      for (int mb = 0; mb < kMB2; ++mb) {
         f32x4 v[4];
-        ex.run(acc.a[mb][nb], v);
+        ex.run(acc, mb, nb, v);
         const int col = c0 + p.wc * 128 + mb * 32 + 4 * ex.rd_chunk;
         if (col >= A.c_valid) continue;
-        const int row0 = r0 + p.wr * (kNB * 32) + nb * 32 + ex.rd_row;
+        const int row0 = r0 + p.wr * (kNB * kBlk) + nb * 32 + ex.rd_row;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int row = row0 + 8 * i;
