@@ -479,10 +479,25 @@ def mfma_ceiling_probe(dev, n: int, h: int, v: int, seconds: float = 1.5) -> dic
         res[kind]["vendor_gemm_NN_d_hidden"] = run_for(lambda: torch.matmul(z, wc, out=dh), 2.0 * n * vc * h)
         res[kind]["vendor_gemm_TN_d_weight"] = run_for(lambda: torch.matmul(z.t(), hid, out=dw), 2.0 * n * vc * h)
         del hid, w, wc, z, dh, dw
+        # the matrix instruction alone, operands in registers: what is left of the peak when nothing moves data
+        wgs, iters = 256, 4000
+        if kind == "zeros":
+            seed = torch.zeros(wgs * 512 * 32, dtype=torch.int32, device=dev)
+        else:   # bf16 pairs with exponents near 1 and random signs / mantissas
+            lo = torch.randint(0, 1 << 16, (wgs * 512 * 32,), device=dev, generator=g, dtype=torch.int32)
+            hi = torch.randint(0, 1 << 16, (wgs * 512 * 32,), device=dev, generator=g, dtype=torch.int32)
+            seed = ((lo & 0x80FF) | 0x3F00) | (((hi & 0x80FF) | 0x3F00) << 16)
+        sink = torch.empty(wgs * 512, device=dev)
+        for shape, name in ((0, "mfma_only_32x32x16"), (1, "mfma_only_16x16x32")):
+            flops = float(L.vamd_mfma_yardstick_flops(shape, wgs, iters))
+            res[kind][name] = run_for(
+                lambda: _cabi.check(L.vamd_mfma_yardstick(shape, seed.data_ptr(), sink.data_ptr(), wgs, iters, st)), flops)
+        del seed, sink
     stop.set()
     res["board_power_cap_W"] = _read_power_w()[1]
     res["note"] = ("ms per call; PFLOP/s on 2*M*N*K; sclk and board power from the driver's sysfs files over the second "
-                   "half of each run (None when they cannot be read); vendor GEMMs on one 16384-column vocabulary chunk")
+                   "half of each run (None when they cannot be read); vendor GEMMs on one 16384-column vocabulary chunk; "
+                   "mfma_only_*: the bf16 matrix instruction of that shape in a register-only loop, 8 wavefronts per CU")
     return res
 
 

@@ -92,6 +92,15 @@ int vamd_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream);
 /* out[i] = a[i] + b[i] + c[i] + d[i] over n floats (n % 4 == 0, 16-byte aligned pointers): a second yardstick,
  * the memory traffic of a fused loss kernel with its gradient and nothing else.  No counterpart in the reference. */
 int vamd_sum4(const float* a, const float* b, const float* c, const float* d, float* out, int64_t n, void* stream);
+/* Benchmark aid (no counterpart in the reference): a loop of independent bf16 matrix instructions on register
+ * operands, no memory traffic, `workgroups` workgroups of 8 wavefronts, `iters` rounds of 8 (32x32x16) or 32
+ * (16x16x32) instructions per wavefront.  seed: workgroups * 512 * 32 device words the operand fragments are taken
+ * from (zeros: nothing toggles; random bf16: the data the board's power management sees in a real GEMM);
+ * out: workgroups * 512 floats.  vamd_mfma_yardstick_flops gives the flops of one launch. */
+#define VAMD_MFMA_32X32X16 0
+#define VAMD_MFMA_16X16X32 1
+int64_t vamd_mfma_yardstick_flops(int shape, int workgroups, int iters);
+int vamd_mfma_yardstick(int shape, const void* seed, float* out, int workgroups, int iters, void* stream);
 
 /* ------------------------------------------------------------------------------------------
  * Fused vocab-projection log-prob / entropy head.

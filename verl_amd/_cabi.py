@@ -33,6 +33,8 @@ SIGNATURES = {
     "vamd_last_error": (c_char_p, []),
     "vamd_copy_bytes": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "vamd_sum4": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
+    "vamd_mfma_yardstick_flops": (c_int64, [c_int, c_int, c_int]),
+    "vamd_mfma_yardstick": (c_int, [c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "vamd_lce_forward_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "vamd_lce_forward": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p,
                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),

@@ -149,5 +149,79 @@ extern "C" int vamd_sum4(const float* a, const float* b, const float* c, const f
   return VAMD_OK;
 }
 
+// Pure matrix-instruction loop, no memory traffic: what the matrix pipes deliver under the board's power management
+// when nothing else draws power.  Every wavefront keeps 4 + 4 operand fragments (from `seed`, so the caller chooses
+// how much they toggle) and 128 accumulator registers, and issues independent MFMAs round robin.
+typedef __bf16 ys_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float ys_f32x16 __attribute__((ext_vector_type(16)));
+template <int SHAPE>
+__global__ __launch_bounds__(512) void mfma_yardstick_kernel(const uint32_t* __restrict__ seed, float* __restrict__ out,
+                                                             int iters) {
+  ys_bf16x8 a[4], b[4];
+  const uint32_t* s = seed + ((size_t)blockIdx.x * 512 + threadIdx.x) * 32;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    union {
+      uint32_t u[4];
+      ys_bf16x8 v;
+    } ua, ub;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      ua.u[j] = s[i * 8 + j];
+      ub.u[j] = s[i * 8 + 4 + j];
+    }
+    a[i] = ua.v;
+    b[i] = ub.v;
+  }
+  float sum = 0.f;
+  if constexpr (SHAPE == VAMD_MFMA_32X32X16) {
+    ys_f32x16 acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i & 3], b[i >> 1], acc[i], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 16; ++j) sum += acc[i][j];
+  } else {
+    vamd::ys_f32x4 acc[32];
+#pragma unroll
+    for (int i = 0; i < 32; ++i) acc[i] = vamd::ys_f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 32; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i & 3], b[(i >> 2) & 3], acc[i], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 32; ++i) sum += (acc[i][0] + acc[i][1]) + (acc[i][2] + acc[i][3]);
+  }
+  out[(size_t)blockIdx.x * 512 + threadIdx.x] = sum;
+}
+
+extern "C" int64_t vamd_mfma_yardstick_flops(int shape, int workgroups, int iters) {
+  if (workgroups <= 0 || iters <= 0) return 0;
+  // per iteration and wavefront: 8 x 32768 flops, or 32 x 16384 flops
+  const int64_t per_iter = shape == VAMD_MFMA_32X32X16 ? 8ll * 32768 : 32ll * 16384;
+  return (int64_t)workgroups * 8 * iters * per_iter;
+}
+
+extern "C" int vamd_mfma_yardstick(int shape, const void* seed, float* out, int workgroups, int iters, void* stream) {
+  using namespace vamd;
+  VAMD_REQUIRE(seed && out && workgroups > 0 && iters > 0, "mfma_yardstick: need seed, out, workgroups > 0, iters > 0");
+  VAMD_REQUIRE(shape == VAMD_MFMA_32X32X16 || shape == VAMD_MFMA_16X16X32, "mfma_yardstick: unknown shape %d", shape);
+  if (shape == VAMD_MFMA_32X32X16)
+    hipLaunchKernelGGL(mfma_yardstick_kernel<VAMD_MFMA_32X32X16>, dim3((unsigned)workgroups), dim3(512), 0,
+                       (hipStream_t)stream, static_cast<const uint32_t*>(seed), out, iters);
+  else
+    hipLaunchKernelGGL(mfma_yardstick_kernel<VAMD_MFMA_16X16X32>, dim3((unsigned)workgroups), dim3(512), 0,
+                       (hipStream_t)stream, static_cast<const uint32_t*>(seed), out, iters);
+  VAMD_LAUNCH_CHECK();
+  return VAMD_OK;
+}
+
 extern "C" int vamd_abi_version(void) { return VAMD_ABI_VERSION; }
 extern "C" const char* vamd_last_error(void) { return vamd::g_error; }
