@@ -5,6 +5,7 @@ equivalence tests an absolute floor of 1e-6 accompanies it (values that cancel t
 index handling is checked bit-exactly (zeros stay exact zeros, group membership by label).
 """
 import math
+import os
 import random
 import types
 import uuid
@@ -161,6 +162,8 @@ def test_gae_bounded_wait_runs_out_without_hanging(dev, monkeypatch):
     back at zero and the result is right."""
     from verl_amd import _cabi
     from verl_amd.trainer.ppo import core_algos as CA
+    if os.environ.get("VAMD_WAITING_KERNELS") == "0":
+        pytest.skip("waiting kernels are switched off in this environment: nothing can time out")
     B, L = 512, 4096
     g = torch.Generator().manual_seed(3)
     r, v = torch.randn(B, L, generator=g).to(dev), torch.randn(B, L, generator=g).to(dev)
