@@ -12,6 +12,7 @@ moves each product by up to half a bf16 ulp.  Those tests add the resulting wors
 2**-8 * E, E = |d_logits| @ |W| resp. |d_logits|^T @ |hidden| from the oracle.
 """
 import math
+import random
 
 import pytest
 import torch
@@ -117,6 +118,32 @@ def test_backward_small_shapes(dev, backward_mode, n, h, v, T):
     _, _, want_dh, want_dw = _oracle(hidden, weight, labels, T, g_lp.float(), g_ent.float())
     _close_bf16(dh, want_dh, "d_hidden")
     _close_bf16(dw, want_dw, "d_weight")
+
+
+def _random_head_shapes(count, seed):
+    rng = random.Random(seed)
+    return [(rng.randint(1, 700), rng.choice([128, 256, 384, 640]), rng.randint(1, 3000), rng.choice([0.5, 1.0, 1.7]))
+            for _ in range(count)]
+
+
+@pytest.mark.parametrize("n,h,v,T", _random_head_shapes(14, seed=2024))
+def test_random_small_shapes_fwd_bwd(dev, n, h, v, T):
+    """Seeded random shapes: token counts, vocabulary sizes and hidden sizes that leave every kind of ragged tile
+    (a last tile of one row or one column, vocabularies below one MFMA block, k extents of two to ten slabs)."""
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    hidden, weight, labels = _make(n, h, v, seed=n * 31 + v)
+    g = torch.Generator().manual_seed(v)
+    g_ent = (torch.rand(n, generator=g) - 0.5).bfloat16()
+    g_lp = ((torch.rand(n, generator=g) - 0.5) * 2).bfloat16()
+    hd = hidden.to(dev).requires_grad_(); wd = weight.to(dev).requires_grad_()
+    lp, ent = linear_cross_entropy(hd, wd, labels.to(dev), T)
+    want_lp, want_ent, want_dh, want_dw, e_dh, e_dw = _oracle_with_scale(hidden, weight, labels, T, g_lp.float(),
+                                                                         g_ent.float(), "cpu")
+    assert (lp.cpu() - want_lp).abs().max().item() <= ATOL
+    assert (ent.cpu() - want_ent).abs().max().item() <= ATOL
+    dh, dw = torch.autograd.grad((ent, lp), (hd, wd), (g_ent.to(dev).float(), g_lp.to(dev).float()))
+    _close_bf16(dh, want_dh, "d_hidden", e_dh)     # temperatures below 1 scale d_logits up, and with it its bf16 rounding
+    _close_bf16(dw, want_dw, "d_weight", e_dw)
 
 
 def test_backward_multi_chunk_and_accumulate(dev):
