@@ -538,7 +538,7 @@ def head_kernel_times(L, step, prof_steps: int) -> dict:
     return kernels
 
 
-def other_head_configs(dev, steps: int) -> dict:
+def other_head_configs(dev, steps: int, with_cpu: bool = True) -> dict:
     """BASELINE configs[0] (Qwen2.5-0.5B head shape, forward only) and configs[4] (Llama-3-8B head shape, 65536
     tokens as eight 8192-token chunks, T = 0.7, entropy coefficient folded into the backward, weight gradient summed
     over the chunks in fp32), timed end to end through the host mirror."""
@@ -566,6 +566,19 @@ def other_head_configs(dev, steps: int) -> dict:
         ms = timed(lambda: K.linear_cross_entropy(hid, w, lab, 1.0), 20)
     res["qwen0.5b_forward_only"] = {"n_tokens": n, "hidden_size": h, "vocab": v, "ms": ms, "tokens_per_s": n / ms * 1e3,
                                     "PFLOPs_algorithmic": 2.0 * n * v * h / ms / 1e12}
+    if with_cpu:   # this configuration is small enough to run in full on the host: the oracle's chunked torch backend
+        import oracle as O
+
+        torch.set_num_threads(os.cpu_count() or 1)
+        hc, wc, lc = hid.cpu(), w.cpu(), lab.cpu()
+        t0 = time.perf_counter()
+        with torch.no_grad():
+            O.fused_linear_for_ppo_chunked(hc, wc, lc, 1.0, 512)
+        dt = time.perf_counter() - t0
+        res["qwen0.5b_forward_only"]["cpu_baseline"] = {
+            "value": n / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"all {n} tokens, chunked torch backend, bf16 GEMMs, forward once, {dt:.2f} s"}
+        del hc, wc, lc
     del hid, w, lab
     n, h, v, T, chunk = 65536, 4096, 128256, 0.7, 8192
     hid = torch.randn(n, h, device=dev, generator=g).bfloat16()
@@ -773,7 +786,7 @@ def main() -> None:
     torch.cuda.empty_cache()
     line["mfma_ceiling_probe"] = mfma_ceiling_probe(dev, n, h, v, seconds=args.ceiling_seconds)
     torch.cuda.empty_cache()
-    line["head_other_configs"] = other_head_configs(dev, args.steps)
+    line["head_other_configs"] = other_head_configs(dev, args.steps, with_cpu=args.cpu_tokens > 0)
     torch.cuda.empty_cache()
     line["unfused_logits_rows"] = unfused_logits_rates(dev)
     torch.cuda.empty_cache()
