@@ -406,6 +406,66 @@ def test_vocabulary_not_a_multiple_of_eight(dev, n, h, v):
     _close_bf16(dw, want_dw, "d_weight", e_dw)
 
 
+def test_head_forward_backward_replays_from_a_hip_graph(dev):
+    """The head's entry points allocate nothing and clear nothing with memset, so a forward + backward (recompute
+    mode, three vocabulary chunks) can be captured once and replayed: three replays on fresh operands, eager work
+    in between, each bit-equal to the eager calls."""
+    from verl_amd import _cabi
+    Lb = _cabi.lib()
+    n, h, v, T = 600, 256, 3000, 0.7
+    gen = torch.Generator(device=dev).manual_seed(9)
+    hidden = torch.empty(n, h, device=dev, dtype=torch.bfloat16)
+    weight = torch.empty(v, h, device=dev, dtype=torch.bfloat16)
+    labels = torch.empty(n, device=dev, dtype=torch.int64)
+    g_lp = torch.empty(n, device=dev)
+    chunk = 1024
+    ws_f = torch.empty(Lb.vamd_lce_forward_workspace_bytes(n, h, v), dtype=torch.uint8, device=dev)
+    ws_b = torch.empty(Lb.vamd_lce_backward_workspace_bytes(n, h, v, chunk), dtype=torch.uint8, device=dev)
+
+    def outputs():
+        f = lambda: torch.empty(n, device=dev)
+        return dict(lp=f(), ent=f(), lse=f(), mz=f(), dh=torch.empty_like(hidden), dw=torch.empty_like(weight))
+
+    def step(o):
+        st = _cabi.stream_ptr(dev)
+        P = lambda t: t.data_ptr()
+        _cabi.check(Lb.vamd_lce_forward(P(hidden), P(weight), P(labels), n, h, v, 1.0 / T, P(o["lp"]), P(o["ent"]),
+                                        P(o["lse"]), P(o["mz"]), None, None, P(ws_f), ws_f.numel(), st))
+        _cabi.check(Lb.vamd_lce_backward(P(hidden), P(weight), P(labels), n, h, v, 1.0 / T, P(o["lse"]), P(o["mz"]),
+                                         P(g_lp), None, 0.001, None, P(o["dh"]), P(o["dw"]), _cabi.DW_STORE, None,
+                                         chunk, P(ws_b), ws_b.numel(), st))
+
+    def refill():
+        hidden.copy_(torch.randn(n, h, device=dev, generator=gen).bfloat16())
+        weight.copy_((torch.randn(v, h, device=dev, generator=gen) * 0.05).bfloat16())
+        labels.copy_(torch.randint(0, v, (n,), device=dev, generator=gen))
+        g_lp.copy_(torch.randn(n, device=dev, generator=gen))
+
+    refill()
+    captured = outputs()
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        step(captured)                                           # warm-up outside the capture
+    torch.cuda.current_stream(dev).wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(captured)
+    for _ in range(3):
+        refill()
+        eager = outputs()
+        step(eager)
+        torch.cuda.synchronize()
+        for t in captured.values():
+            t.fill_(float("nan")) if t.is_floating_point() else None
+        graph.replay()
+        torch.cuda.synchronize()
+        for name in eager:
+            assert torch.equal(captured[name], eager[name]), name
+    want = OH.head_fp32_ground_truth(hidden.cpu(), weight.cpu(), labels.cpu(), T)
+    assert (captured["lp"].cpu() - want[0]).abs().max().item() <= ATOL
+
+
 def test_forward_without_grad_keeps_no_logits(dev, monkeypatch):
     """Under torch.no_grad() (the actor's compute_log_prob) no [tokens, vocab] tensor is allocated even when the
     weight requires grad and the logits cache is switched on."""
