@@ -466,6 +466,24 @@ def test_head_forward_backward_replays_from_a_hip_graph(dev):
     assert (captured["lp"].cpu() - want[0]).abs().max().item() <= ATOL
 
 
+@pytest.mark.parametrize("shape", [0, 1])
+def test_mfma_yardstick_runs_and_counts_its_flops(dev, shape):
+    """The register-only matrix-instruction loop of the benchmark: with every operand 1.0 each accumulator grows by
+    the instruction's k extent per round, so the sum a thread reports is known exactly."""
+    from verl_amd import _cabi
+    Lb = _cabi.lib()
+    wgs, iters = 4, 3
+    ones = torch.full((wgs * 512 * 32,), 0x3F803F80, dtype=torch.int32, device=dev)      # two bf16 1.0 per word
+    out = torch.empty(wgs * 512, device=dev)
+    _cabi.check(Lb.vamd_mfma_yardstick(shape, ones.data_ptr(), out.data_ptr(), wgs, iters, _cabi.stream_ptr(dev)))
+    torch.cuda.synchronize()
+    k, accs = (16, 8 * 16) if shape == 0 else (32, 32 * 4)      # k per instruction; accumulator values per thread
+    assert torch.equal(out, torch.full_like(out, float(iters * k * accs)))
+    per_wave = (8 * 32768) if shape == 0 else (32 * 16384)
+    assert Lb.vamd_mfma_yardstick_flops(shape, wgs, iters) == wgs * 8 * iters * per_wave
+    assert Lb.vamd_mfma_yardstick(7, ones.data_ptr(), out.data_ptr(), wgs, iters, _cabi.stream_ptr(dev)) != 0
+
+
 def test_forward_without_grad_keeps_no_logits(dev, monkeypatch):
     """Under torch.no_grad() (the actor's compute_log_prob) no [tokens, vocab] tensor is allocated even when the
     weight requires grad and the logits cache is switched on."""
