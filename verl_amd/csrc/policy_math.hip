@@ -82,36 +82,46 @@ template <bool VEC, class M>
 __global__ __launch_bounds__(kRcThreads) void moments_kernel(const float* __restrict__ values,
                                                              const float* __restrict__ minus,
                                                              const M* __restrict__ mask, int64_t rows,
-                                                             int64_t cols, int chunks, int per_row, Work wk,
+                                                             int64_t cols, int chunks, int span, int per_row, Work wk,
                                                              MomentOuts out) {
+  // A workgroup walks `span` consecutive 4096-column chunks of its row and leaves one record (`chunks` counts those
+  // spans): at 128 MB per tensor a quarter of the workgroup reductions and records, and few enough records for the
+  // last workgroup to fold them itself.
   const int64_t row = blockIdx.x / chunks;
   const int chunk = blockIdx.x % chunks;
-  const ChunkPos pos(row, chunk, cols);
-  float x[kGroups][4], w[kGroups][4];
-  load_groups<VEC>(values, pos, x);
-  if (minus) {  // moments of values - minus
-    float y[kGroups][4];
-    load_groups<VEC>(minus, pos, y);
+  const bool streaming = streams_past_caches(rows * cols);  // the grid counts spans, not chunks
+  double acc[4] = {0.0, 0.0, 0.0, 0.0};
+  for (int u = 0; u < span; ++u) {
+    const ChunkPos pos(row, chunk * span + u, cols);
+    float x[kGroups][4], w[kGroups][4];
+    load_groups<VEC>(values, pos, x, streaming);
+    if (minus) {  // moments of values - minus
+      float y[kGroups][4];
+      load_groups<VEC>(minus, pos, y, streaming);
+#pragma unroll
+      for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[g][e] -= y[g][e];
+    }
+    load_mask_groups<VEC>(mask, pos, w, streaming);
+    float s0 = 0, s1 = 0, s2 = 0, cnt = 0;
 #pragma unroll
     for (int g = 0; g < kGroups; ++g)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) x[g][e] -= y[g][e];
+      for (int e = 0; e < 4; ++e) {
+        const bool in = w[g][e] != 0.f;
+        const float v = in ? x[g][e] : 0.f;  // where(mask.bool(), values, 0)
+        s0 += w[g][e];
+        s1 += v * w[g][e];
+        s2 += v * v * w[g][e];
+        cnt += in ? 1.f : 0.f;
+      }
+    acc[0] += (double)s0;
+    acc[1] += (double)s1;
+    acc[2] += (double)s2;
+    acc[3] += (double)cnt;
   }
-  load_mask_groups<VEC>(mask, pos, w);
-  float s0 = 0, s1 = 0, s2 = 0, cnt = 0;
-#pragma unroll
-  for (int g = 0; g < kGroups; ++g)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const bool in = w[g][e] != 0.f;
-      const float v = in ? x[g][e] : 0.f;  // where(mask.bool(), values, 0)
-      s0 += w[g][e];
-      s1 += v * w[g][e];
-      s2 += v * v * w[g][e];
-      cnt += in ? 1.f : 0.f;
-    }
   __shared__ double smem[16];
-  double acc[4] = {s0, s1, s2, cnt};
   block_sum<4, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
     store_record<4>(wk.partials, row, chunk, rows, chunks, acc);
@@ -1383,13 +1393,15 @@ static int masked_moments_of_difference(const float* values, const float* minus,
     return VAMD_EWORKSPACE;
   }
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const int chunks = (int)chunks_of(cols);
+  const int all_chunks = (int)chunks_of(cols);
+  const int span = record_span(rows, all_chunks);
+  const int chunks = (all_chunks + span - 1) / span;  // records per row
   const Work wk = carve_work(workspace);
   VAMD_MASK_DISPATCH(mask_dtype, M, {
     const bool vec = can_vectorize(cols, {values, minus}, mask, sizeof(M));
     VAMD_VEC_DISPATCH(vec, V, hipLaunchKernelGGL((moments_kernel<V, M>), dim3((unsigned)(rows * chunks)),
                                                  dim3(kRcThreads), 0, s, values, minus, static_cast<const M*>(mask),
-                                                 rows, cols, chunks, per_row, wk, out));
+                                                 rows, cols, chunks, span, per_row, wk, out));
   });
   VAMD_LAUNCH_CHECK();
   return VAMD_OK;
