@@ -160,6 +160,11 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
                                                0, 1.0, *none3, out.data_ptr(), *P(s, "o1"), coef.data_ptr(), wsp, wsn,
                                                st))
 
+    def gspo(s):   # variant 4, aggregated as seq-mean-token-mean (mode 2) as the reference always does
+        chk(L.vamd_policy_loss_variant_forward(4, *P(s, "a", "b", "c", "mask"), 0, None, B, Lc, 0.2, 0.2, 3.0, 1.0, 1.0,
+                                               2, 1.0, *none3, out.data_ptr(), *P(s, "o1"), coef.data_ptr(), wsp, wsn,
+                                               st))
+
     def kl_cov(s):
         chk(L.vamd_policy_loss_cov_forward(0, *P(s, "a", "b", "c", "mask"), 0, None, B, Lc, 0.2, 0.2, 0.0, 0.0, 0.0002,
                                            1.0, 0, 0, 1.0, *none3, out.data_ptr(), *P(s, "o1"), coef.data_ptr(), None,
@@ -185,7 +190,8 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
         "apply_kl_penalty": (20 * BL, kl_reward),
         "data_metrics": (24 * BL + 8 * BL, data_metrics),     # six fp32 tensors and the int64 attention mask
         "rollout_correction_token": (16 * BL, rollout_corr),
-        "policy_loss_geo_mean_fwd_grad": (20 * BL, geo_mean),  # two passes over the inputs; one is the minimum
+        "policy_loss_geo_mean_fwd_grad": (20 * BL, geo_mean),  # GMPO and GSPO: a per-sequence sum, then the per-token
+        "policy_loss_gspo_fwd_grad": (20 * BL, gspo),          # pass, in one launch over the inputs where the rows allow
         "policy_loss_kl_cov_fwd_grad": (20 * BL, kl_cov),      # statistics, keys, 3 histogram passes, loss: 12 launches
         "copy_yardstick": (8 * BL, copy),
         "sum4_yardstick": (20 * BL, sum4),                    # four tensors in, one out: the traffic of a loss with gradient

@@ -474,11 +474,15 @@ int vamd_policy_loss_forward(const float* old_log_prob, const float* log_prob, c
 /* The same pass for the other registered policy losses.  out[0..3] as above with the counters a variant
  * does not define left at 0 (GPG: all three; SAPO: both clip fractions; CISPO / GSPO:
  * pg_clipfrac_lower); ppo_kl of GSPO averages the unclamped log-ratio, as the reference does.  tau_pos /
- * tau_neg are SAPO's; clip_c is only read by VAMD_PL_VANILLA.  GSPO runs a per-row pass over
+ * tau_neg are SAPO's; clip_c is only read by VAMD_PL_VANILLA.  GSPO needs the per-row mean of
  * log_prob - old_log_prob first (its sequence-level ratio).  REINFORCE (core_algos.py:1984-2061) reports
- * only ppo_kl.  GEO_MEAN (:1635-1718) clips the log-ratio to [-clip_low, clip_high], runs a per-row pass
- * for the geometric means (is_weights enter there, as exp(mean log(w + 1e-10))), ignores mode and the four
- * agg_loss scalars (the loss is the mean over all rows) and reports all three metrics. */
+ * only ppo_kl.  GEO_MEAN (:1635-1718) clips the log-ratio to [-clip_low, clip_high], needs per-row
+ * geometric means first (is_weights enter there, as exp(mean log(w + 1e-10))), ignores mode and the four
+ * agg_loss scalars (the loss is the mean over all rows) and reports all three metrics.  The per-row
+ * quantities of GSPO and GEO_MEAN come from a pre-pass launch, or -- while the whole launch fits the
+ * device at once and VAMD_WAITING_KERNELS is not 0 -- from the loss launch itself, whose workgroups then
+ * wait for the other chunks of their row a bounded number of polls (VAMD_GATE_SPIN_LIMIT) and compute
+ * what did not arrive themselves. */
 size_t vamd_policy_loss_variant_workspace_bytes(int64_t rows, int64_t cols);
 int vamd_policy_loss_variant_forward(int variant, const float* old_log_prob, const float* log_prob,
                                      const float* advantages, const void* mask, int mask_dtype,

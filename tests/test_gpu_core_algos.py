@@ -879,6 +879,57 @@ def test_policy_loss_geo_mean(dev, with_isw, shape):
            what="d geo_mean loss / d log_prob")
 
 
+@pytest.mark.parametrize("variant", ["gspo", "geo_mean"])
+@pytest.mark.parametrize("shape", [(6, 3000), (40, 9000), (100, 17000), (700, 12500), (2, 70000), (3, 200000)])
+def test_sequence_level_losses_on_every_way_to_the_row_sums(dev, monkeypatch, variant, shape):
+    """GSPO and GMPO need a per-sequence sum before their per-token pass.  While the whole launch fits the device at
+    once (and a row has at most 32 chunks) the loss kernel exchanges the chunks' partial sums inside its one launch;
+    a workgroup whose wait for its row's other chunks is cut short (poll limit forced to zero) computes them itself,
+    to the same bits; with the waiting kernels switched off, or beyond those limits, a pre-pass launch leaves the
+    sums.  All against the oracle, loss, metrics and gradient, with the counter area back at zero."""
+    from verl_amd import _cabi
+    from verl_amd.trainer.ppo import core_algos as CA
+    B, Lc = shape
+    g = torch.Generator().manual_seed(B * 31 + Lc)
+    mask, _ = _prefix_mask(B, Lc, g, lo=3)
+    mask[1] = 0
+    old = torch.randn(B, Lc, generator=g) * 0.5 - 1
+    new = old + torch.randn(B, Lc, generator=g) * 0.2
+    adv = torch.randn(B, 1, generator=g).expand(B, Lc).contiguous()
+    isw = torch.rand(B, Lc, generator=g) + 0.5
+    cfg = _cfg(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28)
+    no = new.clone().requires_grad_()
+    if variant == "gspo":
+        fn, mode = CA.compute_policy_loss_gspo, "seq-mean-token-mean"
+        want = O.policy_loss_gspo(old, no, adv, mask, 0.2, 0.28, isw)
+    else:
+        fn, mode = CA.compute_policy_loss_geo_mean, "token-mean"
+        want = O.policy_loss_geo_mean(old, no, adv, mask, 0.2, 0.28, isw)
+    want_grad = torch.autograd.grad(want[0], no)[0]
+
+    def run():
+        nd = new.to(dev).requires_grad_()
+        loss, met = fn(old.to(dev), nd, adv.to(dev), mask.to(dev), mode, cfg, isw.to(dev))
+        grad = torch.autograd.grad(loss, nd)[0]
+        torch.cuda.synchronize()
+        assert _counter_area_is_clear(_cabi.ticket_workspace(4096, dev))
+        return loss.detach().cpu(), met, grad.cpu()
+
+    calm = run()
+    monkeypatch.setenv("VAMD_GATE_SPIN_LIMIT", "0")
+    hurried = run()
+    monkeypatch.delenv("VAMD_GATE_SPIN_LIMIT")
+    monkeypatch.setenv("VAMD_WAITING_KERNELS", "0")
+    two_launches = run()
+    monkeypatch.delenv("VAMD_WAITING_KERNELS")
+    assert torch.equal(calm[0], hurried[0]) and torch.equal(calm[2], hurried[2]) and calm[1] == hurried[1]
+    for loss, met, grad in (calm, two_launches):
+        _close(loss, want[0], what=f"{variant} loss")
+        assert abs(met["actor/pg_clipfrac"] - want[1].item()) < 1e-6
+        assert abs(met["actor/ppo_kl"] - want[2].item()) < 2e-6 * max(1.0, abs(want[2].item()))
+        _close(grad, want_grad, atol=1e-9, what=f"d {variant} loss / d log_prob")
+
+
 @pytest.mark.parametrize("loss_type", ["ppo_clip", "reinforce"])
 @pytest.mark.parametrize("rollout_is", [None, "token", "sequence"])
 @pytest.mark.parametrize("mode", ["token-mean", "seq-mean-token-sum"])

@@ -272,6 +272,8 @@ __global__ __launch_bounds__(kRcThreads) void scale_rows_kernel(const float* __r
 // =============================================================================================
 // policy loss (compute_policy_loss_vanilla, core_algos.py:1159-1250)
 // =============================================================================================
+constexpr int kRowSyncChunks = 32;            // chunks of one row whose workgroups wait for each other (131072 columns)
+constexpr unsigned kRowWaitSpins = 1u << 16;  // polls of about a microsecond; the neighbours normally arrive within a few
 struct PolicyParams {
   float ratio_lo, ratio_hi, clip_c;  // 1 - clip_low, 1 + clip_high, dual-clip constant
   int variant;                       // VAMD_PL_*
@@ -279,6 +281,8 @@ struct PolicyParams {
   const double* row_moments;         // GSPO: [rows][4], slot 0 = sum(m), slot 1 = sum((lp - old) m)
                                      // GEO_MEAN: [rows][chunks][4] partial sums of geo_rows_kernel
   float nkl_lo, nkl_hi;              // GEO_MEAN: clip range of the log-ratio, (-clip_low, +clip_high)
+  double* row_partials;              // ROWS kernels: [rows][chunks][4] partial row sums, exchanged inside the launch
+  unsigned spin_limit;               // ROWS kernels: polls a workgroup spends on its row's other chunks
 };
 
 // Per-token loss, its derivative with respect to log_prob and the metric contributions of the
@@ -381,8 +385,46 @@ __device__ __forceinline__ TokenLoss token_loss(const PolicyParams& pp, float ol
   return t;
 }
 
-// GMPO row sums (core_algos.py:1683-1704): per (row, chunk) the partial sums of the mask, of the sign-aware clipped
-// log-ratio, of the advantages and of log(is_weight + 1e-10), each times the mask.
+// The per-sequence quantity of the two losses that need one before their per-token pass, as four partial sums over
+// one chunk of the row (fp32 over a thread's 16 tokens; the caller widens and reduces them):
+//   GSPO (core_algos.py:1286-1294)      sum(m), sum((lp - old) m), 0, 0
+//   GEO_MEAN (core_algos.py:1683-1704)  sum(m), sum(k m), sum(A m), sum(log(is_weight + 1e-10) m)
+//                                       with k the log-ratio clipped on the side its advantage's sign names
+// One function for whoever computes them -- the row pre-pass kernel, the loss kernel for its own chunk, a loss
+// workgroup that has to stand in for a neighbour -- so that all arrive at the same bits.
+template <bool ISW>
+__device__ __forceinline__ void row_presums(int variant, const ChunkPos& pos, const float (&o)[kGroups][4],
+                                            const float (&n)[kGroups][4], const float (&a)[kGroups][4],
+                                            const float (&w)[kGroups][4], const float (&iw)[kGroups][4], float lo,
+                                            float hi, double (&acc)[4]) {
+  float s_m = 0, s_k = 0, s_a = 0, s_w = 0;
+#pragma unroll
+  for (int g = 0; g < kGroups; ++g)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (e >= pos.valid[g]) continue;
+      const float d = n[g][e] - o[g][e];
+      const float we = w[g][e];
+      s_m += we;
+      if (variant == VAMD_PL_GSPO) {
+        s_k += (we != 0.f ? d : 0.f) * we;  // where(mask, lp - old, 0) * mask
+      } else {
+        const float c = fminf(fmaxf(d, lo), hi);
+        const float A = a[g][e];
+        const float k = A > 0.f ? fminf(d, c) : (A < 0.f ? fmaxf(d, c) : 0.f);
+        s_k += k * we;
+        s_a += A * we;
+        if (ISW) s_w += logf(iw[g][e] + 1e-10f) * we;
+      }
+    }
+  acc[0] = s_m;
+  acc[1] = s_k;
+  acc[2] = s_a;
+  acc[3] = s_w;
+}
+
+// Row pre-pass as a launch of its own (GMPO where the loss kernel cannot exchange the sums itself): per (row, chunk)
+// the four partial sums.
 template <bool VEC, class M, bool ISW>
 __global__ __launch_bounds__(kRcThreads) void geo_rows_kernel(const float* __restrict__ old_lp,
                                                               const float* __restrict__ lp,
@@ -398,24 +440,9 @@ __global__ __launch_bounds__(kRcThreads) void geo_rows_kernel(const float* __res
   load_groups<VEC>(adv, pos, a);
   load_mask_groups<VEC>(mask, pos, w);
   if (ISW) load_groups<VEC>(isw, pos, iw);
-  float s_m = 0, s_k = 0, s_a = 0, s_w = 0;
-#pragma unroll
-  for (int g = 0; g < kGroups; ++g)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      if (e >= pos.valid[g]) continue;
-      const float d = n[g][e] - o[g][e];
-      const float c = fminf(fmaxf(d, lo), hi);
-      const float A = a[g][e];
-      const float k = A > 0.f ? fminf(d, c) : (A < 0.f ? fmaxf(d, c) : 0.f);
-      const float we = w[g][e];
-      s_m += we;
-      s_k += k * we;
-      s_a += A * we;
-      if (ISW) s_w += logf(iw[g][e] + 1e-10f) * we;
-    }
   __shared__ double smem[4 * 4];
-  double acc[4] = {s_m, s_k, s_a, s_w};
+  double acc[4];
+  row_presums<ISW>(VAMD_PL_GEO_MEAN, pos, o, n, a, w, iw, lo, hi, acc);
   block_sum<4, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
     double* p = partials + (int64_t)blockIdx.x * 4;
@@ -424,7 +451,14 @@ __global__ __launch_bounds__(kRcThreads) void geo_rows_kernel(const float* __res
   }
 }
 
-template <bool VEC, class M, bool GRAD, bool ISW, bool FOLD, int VARIANT>
+// ROWS: the kernel works out the per-sequence quantity of GSPO / GMPO itself instead of taking it from a pre-pass.
+// Every workgroup reduces the four partial sums of its own chunk from the values it holds in registers anyway; with
+// one chunk per row that is all.  With several, it leaves them in pp.row_partials, sets the ready byte of its
+// (row, chunk) and waits -- a bounded number of polls -- for the bytes of the row's other chunks, whose workgroups
+// have the neighbouring ids and start together with it.  A workgroup whose wait ran out computes the missing chunks'
+// sums itself, to the same bits, so the result does not depend on what the device lets run at the same time.  The
+// launch's last workgroup clears the ready bytes (ROWS launches always fold their own records).
+template <bool VEC, class M, bool GRAD, bool ISW, bool FOLD, int VARIANT, bool ROWS = false>
 __global__ __launch_bounds__(kRcThreads) void policy_kernel(
     const float* __restrict__ old_lp, const float* __restrict__ lp, const float* __restrict__ adv,
     const M* __restrict__ mask, const float* __restrict__ isw, int64_t rows, int64_t cols, int chunks,
@@ -442,19 +476,79 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
   const bool token_mean = ap.mode == VAMD_AGG_TOKEN_MEAN;
   float seq_lr = 0.f;
   const int variant = VARIANT >= 0 ? VARIANT : pp.variant;
-  if (variant == VAMD_PL_GSPO)  // sum((lp - old) m) / clamp(sum(m), min = 1)
-    seq_lr = (float)pp.row_moments[row * 4 + 1] / fmaxf((float)pp.row_moments[row * 4], 1.f);
-  if (variant == VAMD_PL_GEO_MEAN) {
-    double r[4] = {0, 0, 0, 0};
-    for (int c = 0; c < chunks; ++c)
+  __shared__ double smem[(5 + 3) * 4];
+  double r[4] = {0, 0, 0, 0};  // the row's four sums (GSPO, GEO_MEAN)
+  if constexpr (ROWS) {
+    __shared__ double row_sums[4];
+    double own[4];
+    row_presums<ISW>(variant, pos, o, n, a, w, iw, pp.nkl_lo, pp.nkl_hi, own);
+    block_sum<4, kRcThreads>(own, smem);  // valid in thread 0
+    bool open = true;
+    if (chunks > 1) {
+      if (threadIdx.x == 0) {
+        double* mine = pp.row_partials + (row * chunks + chunk) * 4;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) r[i] += pp.row_moments[(row * chunks + c) * 4 + i];
+        for (int i = 0; i < 4; ++i) peer_store(mine + i, own[i]);
+        ready_byte_set(wk.ticket, row * chunks + chunk);
+      }
+      bool ready = true;
+      unsigned polls = 0;
+      if ((int)threadIdx.x < chunks && (int)threadIdx.x != chunk)
+        ready = ready_byte_wait(wk.ticket, row * chunks + threadIdx.x, polls, pp.spin_limit);
+      open = __syncthreads_and(ready) != 0;
+    }
+    if (open) {
+      if (threadIdx.x == 0) {
+        for (int c = 0; c < chunks; ++c)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            r[i] += c == chunk ? own[i] : peer_load(pp.row_partials + (row * chunks + c) * 4 + i);
+      }
+    } else {
+      for (int c = 0; c < chunks; ++c) {  // uniform over the workgroup
+        double part[4];
+        if (c != chunk) {
+          const ChunkPos p2(row, c, cols);
+          float o2[kGroups][4], n2[kGroups][4], a2[kGroups][4], w2[kGroups][4], iw2[kGroups][4];
+          load_groups<VEC>(old_lp, p2, o2);
+          load_groups<VEC>(lp, p2, n2);
+          load_groups<VEC>(adv, p2, a2);
+          load_mask_groups<VEC>(mask, p2, w2);
+          if (ISW) load_groups<VEC>(isw, p2, iw2);
+          row_presums<ISW>(variant, p2, o2, n2, a2, w2, iw2, pp.nkl_lo, pp.nkl_hi, part);
+          block_sum<4, kRcThreads>(part, smem);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] += c == chunk ? own[i] : part[i];  // thread 0's are the sums
+      }
+    }
+    if (threadIdx.x == 0)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) row_sums[i] = r[i];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = row_sums[i];
+  } else {
+    if (variant == VAMD_PL_GSPO) {
+      r[0] = pp.row_moments[row * 4];
+      r[1] = pp.row_moments[row * 4 + 1];
+    }
+    if (variant == VAMD_PL_GEO_MEAN)
+      for (int c = 0; c < chunks; ++c)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) r[i] += pp.row_moments[(row * chunks + c) * 4 + i];
+  }
+  if (variant == VAMD_PL_GSPO)  // sum((lp - old) m) / clamp(sum(m), min = 1)
+    seq_lr = (float)r[1] / fmaxf((float)r[0], 1.f);
+  if (variant == VAMD_PL_GEO_MEAN) {
     const float den = (float)r[0] + 1e-8f;
     const float ratio = expf((float)r[1] / den);
     const float a_seq = (float)r[2] / den;
     const float w_seq = expf((float)r[3] / den);  // 1 when no importance weights were given (sum of logs = 0)
     seq_lr = -a_seq * ratio * w_seq / den;
   }
+  // GMPO's importance weights enter through the sequence weight above, not token by token
+  const bool isw_per_token = ISW && variant != VAMD_PL_GEO_MEAN;
   float s_loss = 0, s_m = 0, s_kl = 0, s_cf = 0, s_cfl = 0;
 #pragma unroll
   for (int g = 0; g < kGroups; ++g)
@@ -462,7 +556,7 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
     for (int e = 0; e < 4; ++e) {
       const TokenLoss t = token_loss<VARIANT>(pp, o[g][e], n[g][e], a[g][e], seq_lr);
       float loss = t.loss;
-      if (ISW) loss *= iw[g][e];
+      if (isw_per_token) loss *= iw[g][e];
       const float we = w[g][e];
       const bool in = we != 0.f;
       if (e < pos.valid[g]) {
@@ -472,10 +566,10 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
         s_cf += in ? t.cf * we : 0.f;
         s_cfl += in ? t.cfl * we : 0.f;
       }
-      if (GRAD) gr[g][e] = (ISW ? t.dloss * iw[g][e] : t.dloss) * we;
+      if (GRAD) gr[g][e] = (isw_per_token ? t.dloss * iw[g][e] : t.dloss) * we;
     }
   if (GRAD) store_groups<VEC>(grad, pos, gr);
-  __shared__ double smem[(5 + 3) * 4];
+  static_assert(!ROWS || FOLD, "a launch that sets ready bytes has a last workgroup that clears them");
   double acc[5] = {s_loss, s_m, s_kl, s_cf, s_cfl};
   block_sum<5, kRcThreads>(acc, smem);
   if (threadIdx.x == 0) {
@@ -487,6 +581,7 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
     finalize_agg<5>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
     if (threadIdx.x == 0) loss_epilogue<kEpiPolicy>(loss, msum, extra, out);
     ticket_reset(wk.ticket);
+    if (ROWS && chunks > 1) ready_bytes_clear<kRcThreads>(wk.ticket, rows * chunks);
   } else {
     if (wk.totals) totals_epilogue<5, kEpiPolicy>(wk, rows, chunks, cols, ap, coef, out, smem);
   }
@@ -995,13 +1090,9 @@ struct GrpoRowsArgs {
 };
 
 constexpr int64_t kGrpoRowsLimit = 32 * kRcThreads;  // one membership bit per thread for every 256 responses
-// One "score is in memory" byte per response, inside the counter area (zero on entry, zero on exit): the second
-// 128-byte line of the 256-byte slots 1..64, which no counter uses.  A byte per row rather than a bit: setting it
-// is a plain device-scope store, not a read-modify-write that queues up behind its neighbours'.
-static_assert(kGrpoRowsLimit <= 128 * kTicketGroups, "128 ready bytes in each first-level slot");
-__device__ __forceinline__ unsigned char* grpo_ready_byte(unsigned* ticket, int64_t row) {
-  return reinterpret_cast<unsigned char*>(ticket) + (1 + (row >> 7)) * kTicketStride + 128 + (row & 127);
-}
+// One "score is in memory" byte per response (ready_byte).
+static_assert(kGrpoRowsLimit <= kReadyBytes, "one ready byte per response");
+__device__ __forceinline__ unsigned char* grpo_ready_byte(unsigned* ticket, int64_t row) { return ready_byte(ticket, row); }
 // Bit k set: response k * 256 + threadIdx.x belongs to the group of `row` (no bits for a row past the end).
 __device__ __forceinline__ unsigned grpo_member_bits(const int64_t* __restrict__ gid, int64_t rows, int64_t row) {
   unsigned bits = 0;
@@ -1583,28 +1674,49 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
   pp.tau_pos = tau_pos;
   pp.tau_neg = tau_neg;
   pp.row_moments = nullptr;
+  pp.row_partials = nullptr;
+  pp.spin_limit = 0;
   pp.nkl_lo = pp.nkl_hi = 0.f;
-  if (variant == VAMD_PL_GSPO) {  // sequence-level log-ratio: per-row masked moments of log_prob - old_log_prob
-    double* row_moments = reinterpret_cast<double*>(static_cast<char*>(workspace) + reduce_workspace_bytes(rows, cols, 5));
-    st = masked_moments_of_difference(log_prob, old_log_prob, mask, mask_dtype, rows, cols, 1,
-                                      MomentOuts{row_moments, nullptr, nullptr, nullptr, nullptr, 1}, workspace,
-                                      reduce_workspace_bytes(rows, cols, 5), stream);
-    if (st != VAMD_OK) return st;
-    pp.row_moments = row_moments;
-  }
+  const bool per_row = variant == VAMD_PL_GSPO || variant == VAMD_PL_GEO_MEAN;  // losses built on a per-sequence quantity
+  double* const row_area =
+      reinterpret_cast<double*>(static_cast<char*>(workspace) + reduce_workspace_bytes(rows, cols, 5));
   AggParams ap = make_agg(mode, dp_size, batch_num_tokens, global_batch_size, loss_scale_factor);
   const dim3 grid((unsigned)(rows * chunks)), block(kRcThreads);
+  const float* token_weights = is_weights;  // what the per-token pass multiplies by
   if (variant == VAMD_PL_GEO_MEAN) {
     // the loss is the plain mean of the per-sequence losses over all rows (:1706): every valid token carries its
     // row's loss / M, summed per row and divided by the number of rows
     ap = make_agg(VAMD_AGG_SEQ_MEAN_TOKEN_SUM, 1.0, -1.0, (double)rows, -1.0);
     pp.nkl_lo = -clip_low;
     pp.nkl_hi = clip_high;
-    double* partials = reinterpret_cast<double*>(static_cast<char*>(workspace) + reduce_workspace_bytes(rows, cols, 5));
-    pp.row_moments = partials;
+  }
+  // The loss kernel works the per-sequence quantity out itself (one pass over the inputs, 20 against 24.5 us at
+  // 512 x 4096) when the whole launch is resident at once, so that a workgroup waiting for its row's other chunks
+  // keeps nobody from starting, and the tensors qualify for 16-byte accesses; otherwise a pre-pass leaves it in the
+  // workspace.  (With several rounds of workgroups the waits add up: 305 against 190 us at 2048 x 16384.)
+  bool rows_inline = false;
+  const int64_t resident =
+      resident_workgroups((const void*)policy_kernel<true, float, true, true, true, -1, true>, kRcThreads);
+  if (per_row && waiting_kernels_allowed() && rows * chunks <= resident && rows * chunks <= kInlineFoldRecords &&
+      rows * chunks <= kReadyBytes && chunks <= kRowSyncChunks) {
+    VAMD_MASK_DISPATCH(mask_dtype, M, {
+      rows_inline = can_vectorize(cols, {old_log_prob, log_prob, advantages, is_weights, grad_unscaled}, mask, sizeof(M));
+    });
+  }
+  if (rows_inline) {
+    pp.row_partials = row_area;
+    pp.spin_limit = gate_spin_limit(kRowWaitSpins);
+  } else if (variant == VAMD_PL_GSPO) {  // sequence-level log-ratio: per-row masked moments of log_prob - old_log_prob
+    st = masked_moments_of_difference(log_prob, old_log_prob, mask, mask_dtype, rows, cols, 1,
+                                      MomentOuts{row_area, nullptr, nullptr, nullptr, nullptr, 1}, workspace,
+                                      reduce_workspace_bytes(rows, cols, 5), stream);
+    if (st != VAMD_OK) return st;
+    pp.row_moments = row_area;
+  } else if (variant == VAMD_PL_GEO_MEAN) {
+    pp.row_moments = row_area;
 #define VAMD_GEO(V, W)                                                                                            \
   hipLaunchKernelGGL((geo_rows_kernel<V, M, W>), grid, block, 0, s, old_log_prob, log_prob, advantages, mk,       \
-                     is_weights, cols, chunks, pp.nkl_lo, pp.nkl_hi, partials)
+                     is_weights, cols, chunks, pp.nkl_lo, pp.nkl_hi, row_area)
     VAMD_MASK_DISPATCH(mask_dtype, M, {
       const bool vec = can_vectorize(cols, {old_log_prob, log_prob, advantages, is_weights}, mask, sizeof(M));
       const M* mk = static_cast<const M*>(mask);
@@ -1612,22 +1724,23 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
       else { if (is_weights) VAMD_GEO(false, true); else VAMD_GEO(false, false); }
     });
 #undef VAMD_GEO
-    is_weights = nullptr;  // already folded into the sequence loss
+    token_weights = nullptr;  // already folded into the sequence loss
   }
   bool sep = rows * chunks > kInlineFoldRecords;  // fold the records in a launch of their own
   wk.totals = sep && totals_suffice(ap.mode);     // ... unless the launch totals are all the mode needs
   // the clipped PPO loss gets kernels of its own, the other variants share one with a per-token switch
-#define VAMD_PL_LAUNCH(V, G, W, F, K)                                                                              \
-  hipLaunchKernelGGL((policy_kernel<V, M, G, W, F, K>), grid, block, 0, s, old_log_prob, log_prob, advantages, mk, \
-                     is_weights, rows, cols, chunks, pp, ap, wk, out, grad_unscaled, coef_out)
-#define VAMD_PL(V, G, W, F)                                                          \
-  if (variant == VAMD_PL_VANILLA) VAMD_PL_LAUNCH(V, G, W, F, VAMD_PL_VANILLA); \
-  else VAMD_PL_LAUNCH(V, G, W, F, -1)
+#define VAMD_PL_LAUNCH(V, G, W, F, K, R)                                                                              \
+  hipLaunchKernelGGL((policy_kernel<V, M, G, W, F, K, (R) && (V) && (F)>), grid, block, 0, s, old_log_prob, log_prob, advantages, mk, \
+                     token_weights, rows, cols, chunks, pp, ap, wk, out, grad_unscaled, coef_out)
+#define VAMD_PL(V, G, W, F)                                                           \
+  if (variant == VAMD_PL_VANILLA) VAMD_PL_LAUNCH(V, G, W, F, VAMD_PL_VANILLA, false); \
+  else if (rows_inline) VAMD_PL_LAUNCH(V, G, W, F, -1, true); /* rows_inline implies 16-byte accesses */ \
+  else VAMD_PL_LAUNCH(V, G, W, F, -1, false)
 #define VAMD_PL_GW(V, F)                                                                             \
-  if (grad_unscaled) { if (is_weights) { VAMD_PL(V, true, true, F); } else { VAMD_PL(V, true, false, F); } } \
-  else { if (is_weights) { VAMD_PL(V, false, true, F); } else { VAMD_PL(V, false, false, F); } }
+  if (grad_unscaled) { if (token_weights) { VAMD_PL(V, true, true, F); } else { VAMD_PL(V, true, false, F); } } \
+  else { if (token_weights) { VAMD_PL(V, false, true, F); } else { VAMD_PL(V, false, false, F); } }
   VAMD_MASK_DISPATCH(mask_dtype, M, {
-    const bool vec = can_vectorize(cols, {old_log_prob, log_prob, advantages, is_weights, grad_unscaled}, mask,
+    const bool vec = can_vectorize(cols, {old_log_prob, log_prob, advantages, token_weights, grad_unscaled}, mask,
                                    sizeof(M));
     const M* mk = static_cast<const M*>(mask);
     sep = sep && vec;

@@ -325,6 +325,36 @@ __device__ __forceinline__ float peer_load_f32(const float* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// "My partial result is in memory" bytes, one per producer (a response, a (row, chunk) record), inside the counter
+// area and therefore zero on entry and to be left zero on exit: the second 128-byte line of the 256-byte slots
+// 1..64, which no counter uses.  A byte per producer rather than a bit: setting it is a plain device-scope store, not
+// a read-modify-write that queues up behind its neighbours'.
+constexpr int64_t kReadyBytes = 128 * kTicketGroups;
+__device__ __forceinline__ unsigned char* ready_byte(unsigned* ticket, int64_t i) {
+  return reinterpret_cast<unsigned char*>(ticket) + (1 + (i >> 7)) * kTicketStride + 128 + (i & 127);
+}
+// thread 0, after the device-coherent stores of the result
+__device__ __forceinline__ void ready_byte_set(unsigned* ticket, int64_t i) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __hip_atomic_store(ready_byte(ticket, i), (unsigned char)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Polls byte i at most `limit` more times in total (`polls` counts across calls); false = gave up.
+__device__ __forceinline__ bool ready_byte_wait(unsigned* ticket, int64_t i, unsigned& polls, unsigned limit) {
+  const unsigned char* flag = ready_byte(ticket, i);
+  while (__hip_atomic_load(flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0) {
+    if (polls++ >= limit) return false;
+    __builtin_amdgcn_s_sleep(4);
+  }
+  return true;
+}
+// The whole workgroup: bytes 0 .. count-1 back to zero (four bytes per word), by whoever leaves the launch last.
+template <int NT>
+__device__ __forceinline__ void ready_bytes_clear(unsigned* ticket, int64_t count) {
+  for (int64_t w = threadIdx.x; w < (count + 3) / 4; w += NT)
+    __hip_atomic_store(reinterpret_cast<unsigned*>(ready_byte(ticket, w * 4)), 0u, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Lane exchange inside the vector ALU (data-parallel primitives): a lane without a source in the pattern, or in a
 // row the mask leaves out, receives `none`.  The wavefront scans use the shifts by 1, 2, 4, 8 inside a row of 16
 // lanes (0x111 .. 0x118), the last lane of rows 0 / 2 into rows 1 / 3 (0x142, row mask 0xA), lane 31 into rows 2
