@@ -58,10 +58,10 @@ constexpr int kSteps = kBK / 32;              // 32-k MFMA steps per slab (2)
 constexpr int kSlabBytes = kTile * kBK * 2;   // 32 KB
 constexpr int kLdsBytes = 4 * kSlabBytes;     // R,C x 2 stages = 128 KB
 static_assert(kNB == 4 && kMB == 8 && kLoads == 4 && kSteps == 2, "slab_iter's slot schedule is written for this layout");
-// A four-wavefront layout (128 x 128 per wavefront, one per SIMD) issues a third fewer LDS reads and lets the board
-// clock 10 % higher, but was measured slower: with one wavefront per SIMD nothing fills the cycles it spends at the
-// per-slab barrier and in the epilogue (forward 13.7 against 13.2 ms, gradient GEMMs 33.0 against 27.3 ms per step at
-// 16384 x 152064 x 3584 with the 32 x 32 x 16 instruction).
+// A four-wavefront layout (128 x 128 per wavefront, one per SIMD, accumulators in the AGPRs) issues a third fewer LDS
+// reads but was measured slower, and hungrier per flop: with one wavefront per SIMD nothing fills the cycles it spends
+// at the barriers and in the epilogue (forward 14.0 against 12.9 ms, gradient GEMMs 35.4 against 25.9 ms per step at
+// 16384 x 152064 x 3584 with this instruction and schedule; 869 against 795 W per PFLOP/s above the idle board).
 
 // One GEMM operand as the tile engine sees it.
 struct Operand {
