@@ -263,9 +263,11 @@ struct Frags {
 //   slots  0..51 : the C fragment of group G + 3 is read from `cur` in the first slot of group G (its ring slot was
 //                  last used by group G - 1); the R fragments of k-step 1 are read in groups 1..4
 //   after slot 21: every R fragment of the slab is in registers; a first workgroup barrier frees the R half of `cur`,
-//                  and the R transfers of slab it+2 go into it one at a time in slots 26, 34, 42 and 50
-//   after slot 55: wait for this wavefront's LDS reads and for its transfers of slab it+1 (all but its four newest
-//                  transfers, which belong to slab it+2), second workgroup barrier: nobody reads `cur` any more, and
+//                  and the R transfers of slab it+2 go into it one at a time in slots 26, 34, 42 and 50 (with them,
+//                  in slots 30 and 38, the two transfers of a K-major C slab that cover k-step 0, which nobody reads
+//                  after slot 16: 25.2 against 25.6 ms per step in the gradient GEMMs)
+//   after slot 55: wait for this wavefront's LDS reads and for its transfers of slab it+1 (all but its four or six
+//                  newest transfers, which belong to slab it+2), second workgroup barrier: nobody reads `cur` any more, and
 //                  `nxt` is complete
 //   slots 56..63 : the fragments the next slab starts with (R of k-step 0, C of groups 0..2) are read from `nxt`,
 //                  and the C transfers of slab it+2 into `cur` are issued
@@ -293,22 +295,33 @@ __device__ __forceinline__ void slab_iter(const SlabDma<RK>& dr, const SlabDma<C
       // last R fragment, read in slot 17, has arrived
       if (j == 21) asm volatile("s_waitcnt lgkmcnt(1)\n\ts_barrier" ::: "memory");
       if (j >= 26 && (j - 26) % 8 == 0) dr.issue_one((j - 26) / 8, r2, lds_address(cur));
+      // a K-major C slab lies in LDS k row by k row: the rows of k-step 0 (its transfers 0 and 1) were last read in
+      // slot 16, so they are as free as R by now
+      if (CK && (j == 30 || j == 38)) dc.issue_one((j - 30) / 8, c2, lds_address(cur) + kSlabBytes);
     } else if (j >= 56) {
       const int k = j - 56;
       if (k == 0) f.c[0] = fc.read(nxt + kSlabBytes, 0, 0);
       if (k < kNB) f.r[0][k] = fr.read(nxt, 0, k);
       if (k == 4) f.c[1] = fc.read(nxt + kSlabBytes, 0, 1);
       if (k == 5) f.c[2] = fc.read(nxt + kSlabBytes, 0, 2);
-      // four C transfers in the slots that carry at most one read
-      if (k == 1 || k == 3 || k == 6 || k == 7)
-        dc.issue_one(k == 1 ? 0 : k == 3 ? 1 : k - 4, c2, lds_address(cur) + kSlabBytes);
+      // the C transfers that are left, in slots that carry at most one read
+      if (CK) {
+        if (k == 3 || k == 6) dc.issue_one(k == 3 ? 2 : 3, c2, lds_address(cur) + kSlabBytes);
+      } else {
+        if (k == 1 || k == 3 || k == 6 || k == 7)
+          dc.issue_one(k == 1 ? 0 : k == 3 ? 1 : k - 4, c2, lds_address(cur) + kSlabBytes);
+      }
     }
-    // transfers complete in issue order, so "at most kLoads outstanding" leaves only the R transfers of slab it+2
-    if (j == 55) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    // transfers complete in issue order, so "at most n outstanding" leaves only the n transfers of slab it+2 issued
+    // so far: four for R, and two more when C is K-major
+    if (j == 55) {
+      if (CK) asm volatile("s_waitcnt vmcnt(6) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
     __builtin_amdgcn_sched_barrier(0);
   }
 }
-static_assert(kLoads == 4, "the s_waitcnt vmcnt(4) of slab_iter counts the R transfers of one slab");
+static_assert(kLoads == 4, "the s_waitcnt vmcnt(4 / 6) of slab_iter counts the transfers of slab it+2 issued before it");
 
 // ---------------------------------------------------------------------------------------------
 // Persistent, software-pipelined walk over a list of output tiles.
