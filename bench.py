@@ -30,10 +30,10 @@ COPY_YARDSTICK_BYTES = 1 << 30
 # rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by the readings of the 1 GiB copy in the same run
 # (2048 and 1024 bytes per unit); see profiles/head_fwd_bwd_qwen7b_hbm_traffic.md.  Counters cannot be read
 # from inside this process, so the figure is recorded here and only reported for the shape it was measured on.
-MEASURED_TRAFFIC_BYTES = {"lce_dgrad_kernel": 6.56e9 + 0.353e9,       # per full chunk, either backward mode
-                          "lce_forward_kernel": 36.2e9 + 0.007e9,    # without the logits cache (the default)
-                          "lce_forward_kernel_with_cache": 43.1e9 + 9.98e9,
-                          "lce_recompute_kernel": 2.85e9 + 0.611e9, "lce_dlogits_kernel": 1.125e9 + 0.537e9}
+MEASURED_TRAFFIC_BYTES = {"lce_dgrad_kernel": 6.68e9 + 0.353e9,       # per full chunk, either backward mode
+                          "lce_forward_kernel": 39.2e9 + 0.007e9,    # without the logits cache (the default)
+                          "lce_forward_kernel_with_cache": 46.3e9 + 9.98e9,
+                          "lce_recompute_kernel": 2.83e9 + 0.612e9, "lce_dlogits_kernel": 1.125e9 + 0.537e9}
 GEMMS_PER_STEP = {"lce_forward_kernel": 1, "lce_recompute_kernel": 1, "lce_dgrad_kernel": 2}
 
 
