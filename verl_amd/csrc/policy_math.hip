@@ -1695,10 +1695,9 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
   // keeps nobody from starting, and the tensors qualify for 16-byte accesses; otherwise a pre-pass leaves it in the
   // workspace.  (With several rounds of workgroups the waits add up: 305 against 190 us at 2048 x 16384.)
   bool rows_inline = false;
-  const int64_t resident =
-      resident_workgroups((const void*)policy_kernel<true, float, true, true, true, -1, true>, kRcThreads);
-  if (per_row && waiting_kernels_allowed() && rows * chunks <= resident && rows * chunks <= kInlineFoldRecords &&
-      rows * chunks <= kReadyBytes && chunks <= kRowSyncChunks) {
+  if (per_row && waiting_kernels_allowed() && rows * chunks <= kInlineFoldRecords && rows * chunks <= kReadyBytes &&
+      chunks <= kRowSyncChunks &&
+      rows * chunks <= resident_workgroups((const void*)policy_kernel<true, float, true, true, true, -1, true>, kRcThreads)) {
     VAMD_MASK_DISPATCH(mask_dtype, M, {
       rows_inline = can_vectorize(cols, {old_log_prob, log_prob, advantages, is_weights, grad_unscaled}, mask, sizeof(M));
     });
