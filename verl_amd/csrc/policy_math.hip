@@ -1693,7 +1693,7 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
   // The loss kernel works the per-sequence quantity out itself (one pass over the inputs, 20 against 24.5 us at
   // 512 x 4096) when the whole launch is resident at once, so that a workgroup waiting for its row's other chunks
   // keeps nobody from starting, and the tensors qualify for 16-byte accesses; otherwise a pre-pass leaves it in the
-  // workspace.  (With several rounds of workgroups the waits add up: 305 against 190 us at 2048 x 16384.)
+  // workspace.  (With more workgroups than fit the device at once the waits add up: 305 against 190 us at 2048 x 16384.)
   bool rows_inline = false;
   if (per_row && waiting_kernels_allowed() && rows * chunks <= kInlineFoldRecords && rows * chunks <= kReadyBytes &&
       chunks <= kRowSyncChunks &&
