@@ -670,6 +670,9 @@ def main() -> None:
                     help="only the matrix-pipe ceiling probe (zeros against random operands, vendor GEMMs beside "
                          "the forward kernel): what a counter pass for the shader clock runs")
     ap.add_argument("--ceiling-seconds", type=float, default=1.5, help="how long the probe keeps each kernel running")
+    ap.add_argument("--policy-math-only", action="store_true",
+                    help="only the [B, L] kernels at B = 2048, L = 16384 after the 1 GiB copy: what a counter pass for "
+                         "their memory traffic runs")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: --gpus {args.gpus} is not supported (every box here has one GPU; "
@@ -687,6 +690,17 @@ def main() -> None:
     n, h, v, T = 16384, 3584, 152064, 1.0
     if args.ceiling_only:
         print(json.dumps({"mfma_ceiling_probe": mfma_ceiling_probe(dev, n, h, v, seconds=args.ceiling_seconds)}))
+        return
+    if args.policy_math_only:
+        a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)   # the copy the counters are scaled by
+        b = torch.empty_like(a)
+        _cabi.check(_cabi.lib().vamd_copy_bytes(a.data_ptr(), b.data_ptr(), a.numel(), _cabi.stream_ptr(dev)))
+        torch.cuda.synchronize()
+        del a, b
+        only = {"grpo_advantage", "policy_loss_fwd", "policy_loss_fwd_grad", "gae_scan_whiten", "value_loss_fwd_grad",
+                "kl_loss_fwd_grad", "masked_moments", "apply_kl_penalty", "data_metrics"}
+        print(json.dumps({"policy_math_b2048_l16384": policy_math_rates(dev, with_cpu=False, B=2048, Lc=16384,
+                                                                         n_groups=256, only=only)}))
         return
     g = torch.Generator(device=dev).manual_seed(0)
     hidden = torch.randn(n, h, device=dev, generator=g).bfloat16().requires_grad_()
