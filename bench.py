@@ -63,11 +63,14 @@ def cpu_baseline(n_cpu: int, h: int, v: int, temperature: float) -> dict:
     }
 
 
-def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_groups: int = 64, only=None) -> dict:
+def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_groups: int = 64, only=None,
+                      buffer_sets: int | None = None) -> dict:
     """The [B, L] kernels (B = 512, L = 4096 is the size of the GRPO / policy-loss and GAE benchmark configurations): microseconds per call from HIP events
     over 48 calls (best of three such loops) that rotate through 8 buffer sets, 16 at the smaller size (so that even the two-tensor ops
     touch more than the 256 MB Infinity Cache before they come back to a set), the algorithmic bytes of
-    the op, and the fraction of 8 TB/s that gives.  ``cpu_ms`` is the CPU oracle on one buffer set."""
+    the op, and the fraction of 8 TB/s that gives.  ``cpu_ms`` is the CPU oracle on one buffer set.
+    ``buffer_sets=1`` times the same calls on one set that stays in the caches (what a kernel sees whose inputs the
+    kernel before it has just written): how much of a call at this size is waiting for memory at all."""
     import torch
 
     import oracle as O
@@ -76,6 +79,8 @@ def policy_math_rates(dev, with_cpu: bool, B: int = 512, Lc: int = 4096, n_group
     L = _cabi.lib()
     BL = B * Lc
     nset = 16 if BL * 4 * 2 * 8 < (300 << 20) else 8   # two fp32 tensors per set must add up to more than the cache
+    if buffer_sets is not None:
+        nset = buffer_sets
     g = torch.Generator(device=dev).manual_seed(0)
 
     def mk():
@@ -811,6 +816,11 @@ def main() -> None:
     line["unfused_logits_rows"] = unfused_logits_rates(dev)
     torch.cuda.empty_cache()
     line["policy_math_b512_l4096"] = policy_math_rates(dev, with_cpu=args.cpu_tokens > 0)
+    resident = policy_math_rates(dev, with_cpu=False, buffer_sets=1,
+                                 only={"grpo_advantage", "policy_loss_fwd", "policy_loss_fwd_grad", "gae_scan_whiten",
+                                       "value_loss_fwd_grad", "kl_loss_fwd_grad", "masked_moments", "copy_yardstick",
+                                       "sum4_yardstick"})
+    line["policy_math_b512_l4096_cache_resident_us"] = {k: v["us"] for k, v in resident.items()}
     line["policy_math_python_path_b512_l4096"] = policy_math_python_path(dev)
     # the same kernels on 16 x larger tensors, where the fixed ~8 us of the single-launch reduction no longer dominates
     line["policy_math_b2048_l16384"] = policy_math_rates(dev, with_cpu=False, B=2048, Lc=16384, n_groups=256)
