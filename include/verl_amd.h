@@ -81,7 +81,7 @@ extern "C" {
 
 /* Bumped whenever an entry point changes its signature or a workspace its layout; a binding compares it with
  * the header it was written against. */
-#define VAMD_ABI_VERSION 4
+#define VAMD_ABI_VERSION 5
 int vamd_abi_version(void);
 const char* vamd_last_error(void);
 
@@ -163,7 +163,11 @@ int vamd_lce_forward_static(const void* hidden, const void* weight, const int64_
  *     VAMD_DW_F32_ADD          d_weight_acc32 += g                               (d_weight may be NULL)
  *     VAMD_DW_F32_ADD_FINISH   d_weight_acc32 += g; d_weight = bf16(d_weight_acc32): the sum over all token
  *                              chunks is rounded once
+ *     VAMD_DW_NONE             no weight gradient: the d_weight GEMM is not run (a frozen lm_head)
  *   d_weight_acc32: [vocab, hidden_size] fp32, 16-byte aligned, for the three F32 modes.
+ *   d_hidden may be NULL when the hidden states need no gradient: the d_hidden GEMM is then not run.  Like the
+ *   reference's torch backend, which allocates and accumulates only the gradients whose inputs require them
+ *   (verl/utils/experimental/torch_functional.py:150-156, :184-187); one of the two must be asked for.
  * vocab_chunk = 0 lets the library choose how many vocabulary columns of d_logits are staged
  * at a time (the workspace holds one [n_pad, vocab_chunk] bf16 panel plus an fp32 d_hidden
  * accumulator); pass the same value to the workspace query.
@@ -173,6 +177,7 @@ int vamd_lce_forward_static(const void* hidden, const void* weight, const int64_
 #define VAMD_DW_F32_STORE 2
 #define VAMD_DW_F32_ADD 3
 #define VAMD_DW_F32_ADD_FINISH 4
+#define VAMD_DW_NONE 5
 size_t vamd_lce_backward_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab, int64_t vocab_chunk);
 int vamd_lce_backward(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
                       int64_t hidden_size, int64_t vocab, float rcp_temperature, const float* lse,
@@ -195,7 +200,10 @@ int vamd_lce_timing_collect(double* ms_by_kernel_host, int64_t* launches_by_kern
  * fused head is off.  logprobs_from_logits / _v2 / _naive (verl/utils/torch_functional.py:72-100, :148-200),
  * entropy_from_logits / entropy_from_logits_with_chunking (:224-263).
  *   logits [n_rows, vocab] with row pitch ld (elements), element type VAMD_DT_*; arithmetic in fp32;
- *   labels [n_rows] int64 in [0, vocab) (may be NULL when logprobs is NULL).
+ *   labels [n_rows] int64 (may be NULL when logprobs is NULL).  A label outside [0, vocab) -- an ignore index such
+ *   as -100, a padding id -- reads no logit: its logprobs entry is 0 and it receives no one-hot term in the
+ *   backward pass (the reference's gather would fault on it; 0 is what flash-attn's cross_entropy_loss returns
+ *   for its ignore index).
  *   logprobs = z[label] - lse(z); entropy = lse(z) - sum softmax(z) z; lse and mean_z (= sum softmax(z) z) are
  *   what the backward pass needs.  Every output is fp32 [n_rows] and may be NULL if not wanted.
  * One pass over the logits (online softmax), no workspace. */
@@ -215,7 +223,9 @@ int vamd_row_softmax_backward(const void* logits, int dtype, int64_t n_rows, int
                               const float* d_entropy, void* d_logits, int64_t ld_out, void* stream);
 /* clip_by_value (verl/utils/torch_functional.py:203-221): out = max(min(x, hi), lo) over n fp32 elements, and its
  * gradients with torch's rule for binary min / max (the selected operand takes the gradient, equal operands half
- * each); d_x / d_lo / d_hi may be NULL. */
+ * each); d_x / d_lo / d_hi may be NULL.  A NaN in x, lo or hi gives a NaN output, as torch.min / torch.max of two
+ * tensors do, and (every comparison with it being false) the whole upstream gradient to both operands of that
+ * min / max, which is what torch's backward formulas produce. */
 int vamd_clip_by_value(const float* x, const float* lo, const float* hi, int64_t n, float* out, void* stream);
 int vamd_clip_by_value_backward(const float* x, const float* lo, const float* hi, const float* grad_out, int64_t n,
                                 float* d_x, float* d_lo, float* d_hi, void* stream);

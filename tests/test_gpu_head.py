@@ -120,6 +120,53 @@ def test_backward_small_shapes(dev, backward_mode, n, h, v, T):
     _close_bf16(dw, want_dw, "d_weight")
 
 
+@pytest.mark.parametrize("frozen", ["weight", "hidden"])
+@pytest.mark.parametrize("n,h,v", [(129, 256, 1152), (700, 256, 8192), (1388, 512, 20000)])
+def test_backward_runs_only_the_gradients_that_are_needed(dev, backward_mode, frozen, n, h, v):
+    """An input that requires no gradient gets none and its GEMM is skipped (reference torch backend,
+    verl/utils/experimental/torch_functional.py:150-156, :184-187); the gradient that is computed equals, bit for
+    bit, the one the two-sided backward pass gives."""
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+    from verl_amd.utils.experimental.torch_functional import FusedLinearForPPO
+    hidden, weight, labels = _make(n, h, v, seed=11 * n + v)
+    g = torch.Generator().manual_seed(n + 1)
+    g_ent = (torch.rand(n, generator=g) - 0.5).bfloat16().float()
+    g_lp = ((torch.rand(n, generator=g) - 0.5) * 2).bfloat16().float()
+    _, _, want_dh, want_dw = _oracle(hidden, weight, labels, 1.5, g_lp, g_ent)
+    for op in (lambda a, b, c: linear_cross_entropy(a, b, c, 1.5), lambda a, b, c: FusedLinearForPPO()(a, b, c, 1.5)):
+        hd = hidden.to(dev).requires_grad_(); wd = weight.to(dev).requires_grad_()
+        lp, ent = op(hd, wd, labels.to(dev))
+        both_dh, both_dw = torch.autograd.grad((ent, lp), (hd, wd), (g_ent.to(dev).to(ent.dtype), g_lp.to(dev).to(lp.dtype)))
+        h1 = hidden.to(dev).requires_grad_(frozen != "hidden")
+        w1 = weight.to(dev).requires_grad_(frozen != "weight")
+        lp, ent = op(h1, w1, labels.to(dev))
+        (ent.float() * g_ent.to(dev) + lp.float() * g_lp.to(dev)).sum().backward()
+        if frozen == "weight":
+            assert w1.grad is None
+            _close_bf16(h1.grad, want_dh, "d_hidden with a frozen weight")
+            assert torch.equal(h1.grad, both_dh)
+        else:
+            assert h1.grad is None
+            _close_bf16(w1.grad, want_dw, "d_weight with detached hidden states")
+            assert torch.equal(w1.grad, both_dw)
+
+
+def test_backward_c_abi_refuses_a_call_that_asks_for_nothing(dev):
+    from verl_amd import _cabi
+    from verl_amd.utils.kernel.linear_cross_entropy import efficient_entropy_backward, efficient_entropy_forward
+    hidden, weight, labels = _make(64, 128, 256, seed=1)
+    hd, wd, ld = hidden.to(dev), weight.to(dev), labels.to(dev)
+    _, _, lse, mean_z = efficient_entropy_forward(hd, wd, ld)
+    assert efficient_entropy_backward(None, None, hd, wd, ld, lse, mean_z, need_d_hidden=False,
+                                      need_d_weight=False) == (None, None)
+    L = _cabi.lib()
+    ws = _cabi.workspace(L.vamd_lce_backward_workspace_bytes(64, 128, 256, 0), dev)
+    rc = L.vamd_lce_backward(hd.data_ptr(), wd.data_ptr(), ld.data_ptr(), 64, 128, 256, 1.0, lse.data_ptr(),
+                             mean_z.data_ptr(), None, None, 0.0, None, None, None, _cabi.DW_NONE, None, 0,
+                             ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev))
+    assert rc == -1 and b"neither" in L.vamd_last_error()
+
+
 def _random_head_shapes(count, seed):
     rng = random.Random(seed)
     return [(rng.randint(1, 700), rng.choice([128, 256, 384, 640]), rng.randint(1, 3000), rng.choice([0.5, 1.0, 1.7]))

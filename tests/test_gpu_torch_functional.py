@@ -163,6 +163,90 @@ def test_clip_by_value_and_its_gradients(dev):
         assert a.shape == b.shape and torch.allclose(a.cpu(), b, rtol=1e-5, atol=1e-5)
 
 
+def test_labels_outside_the_vocabulary_read_nothing(dev):
+    """An ignore index (-100) or a padding id >= vocab gives a log-prob of 0 and no one-hot term in the gradient;
+    the rows beside it are untouched."""
+    import verl_amd.utils.torch_functional as F
+    n, v = 12, 515
+    z, labels = _logits(n, v, torch.float32, seed=21)
+    bad = labels.clone()
+    bad[3], bad[7], bad[11] = -100, v, -1
+    ok = torch.ones(n, dtype=torch.bool)
+    ok[[3, 7, 11]] = False
+    for dtype in (torch.float32, torch.bfloat16):
+        zd = z.to(dtype).to(dev).requires_grad_()
+        lp = F.logprobs_from_logits(zd, bad.to(dev), inplace_backward=False)
+        want = OM.logprobs_from_logits(z.to(dtype).double(), labels)
+        _assert_close(lp[ok.to(dev)], want[ok], dtype, "in-range rows")
+        assert (lp[~ok.to(dev)] == 0).all()
+        d, = torch.autograd.grad(lp.float().sum(), zd)
+        # rows without a valid label: -softmax(z), whose entries sum to -1
+        row_sums = d.float().sum(-1).cpu()
+        assert torch.allclose(row_sums[~ok], torch.full((3,), -1.0), atol=2e-2 if dtype != torch.float32 else 1e-5)
+        assert torch.allclose(row_sums[ok], torch.zeros(int(ok.sum())), atol=2e-2 if dtype != torch.float32 else 1e-5)
+
+
+def test_second_backward_through_inplace_logprobs_raises(dev):
+    import verl_amd.utils.torch_functional as F
+    z, labels = _logits(6, 256, torch.float32, seed=8)
+    logits = z.to(dev).requires_grad_() * 1.0
+    lp = F.logprobs_from_logits(logits, labels.to(dev), inplace_backward=True)
+    lp.sum().backward(retain_graph=True)
+    with pytest.raises(RuntimeError, match="inplace_backward"):
+        lp.sum().backward()
+
+
+def test_clip_by_value_hands_nan_on_like_torch(dev):
+    import verl_amd.utils.torch_functional as F
+    nan = float("nan")
+    x = torch.tensor([nan, 0.5, 0.5, nan, 2.0, -3.0])
+    lo = torch.tensor([0.0, nan, 0.0, nan, 0.0, 0.0])
+    hi = torch.tensor([1.0, 1.0, nan, 1.0, 1.0, 1.0])
+    up = torch.tensor([1.0, 2.0, 3.0, 4.0, 5.0, 6.0])
+    cpu = [t.clone().requires_grad_() for t in (x, lo, hi)]
+    want = OM.clip_by_value(*cpu)
+    want_grads = torch.autograd.grad(want, cpu, up)
+    gpu = [t.to(dev).requires_grad_() for t in (x, lo, hi)]
+    got = F.clip_by_value(*gpu)
+    assert torch.equal(torch.isnan(got.cpu()), torch.isnan(want.detach()))
+    assert torch.equal(torch.nan_to_num(got.cpu(), nan=7.0), torch.nan_to_num(want.detach(), nan=7.0))
+    for name, a, b in zip(("x", "tensor_min", "tensor_max"), torch.autograd.grad(got, gpu, up.to(dev)), want_grads):
+        assert torch.equal(a.cpu(), b), f"gradient with respect to {name}: {a.cpu().tolist()} != {b.tolist()}"
+
+
+@pytest.mark.parametrize("shift_mean", [True, False])
+@pytest.mark.parametrize("mask_kind", ["bool", "weights"])
+def test_masked_var_and_whiten_gradients(dev, shift_mean, mask_kind):
+    """``masked_var`` / ``masked_whiten`` are plain differentiable torch in the reference
+    (verl/utils/torch_functional.py:304-339); the gradients here are closed forms, compared with autograd through
+    the oracle's restatement in fp64."""
+    import verl_amd.utils.torch_functional as F
+    g = torch.Generator().manual_seed(17)
+    values = torch.randn(6, 700, generator=g) * 2.0 + 0.7
+    mask = torch.rand(6, 700, generator=g) < 0.55
+    mask = mask if mask_kind == "bool" else mask.float() * (0.5 + torch.rand(6, 700, generator=g))
+    up = torch.randn(6, 700, generator=g)
+    v64 = values.double().requires_grad_()
+    m64 = mask.double() if mask_kind == "weights" else mask
+    want_var = OM.masked_var(v64, m64)
+    want_dvar, = torch.autograd.grad(want_var, v64)
+    want_w = OM.masked_whiten(v64, m64, shift_mean)
+    want_dw, = torch.autograd.grad(want_w, v64, up.double())
+    vd = values.to(dev).requires_grad_()
+    var = F.masked_var(vd, mask.to(dev))
+    assert var.requires_grad
+    assert torch.allclose(var.detach().cpu().double(), want_var.detach(), rtol=1e-5)
+    dvar, = torch.autograd.grad(var, vd)
+    assert torch.allclose(dvar.cpu().double(), want_dvar, rtol=1e-4, atol=1e-9), (dvar.cpu().double() - want_dvar).abs().max()
+    w = F.masked_whiten(vd, mask.to(dev), shift_mean)
+    assert torch.allclose(w.detach().cpu().double(), want_w.detach(), rtol=1e-5, atol=1e-5)
+    dw, = torch.autograd.grad(w, vd, up.to(dev))
+    err = (dw.cpu().double() - want_dw).abs().max().item()
+    assert err <= 1e-5 * want_dw.abs().max().item() + 1e-7, err
+    # without requires_grad nothing is recorded
+    assert not F.masked_whiten(values.to(dev), mask.to(dev), shift_mean).requires_grad
+
+
 @pytest.mark.parametrize("axis", [None, -1, 0, 1, 2, (0, 2), (1, 2), (0, 1, 2)])
 @pytest.mark.parametrize("mask_dtype", [torch.float32, torch.bool, torch.int64])
 def test_masked_sum_and_mean_any_axis_with_gradients(dev, axis, mask_dtype):

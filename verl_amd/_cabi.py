@@ -18,7 +18,7 @@ _lib = None
 
 MASK_F32, MASK_I64, MASK_U8, MASK_I32 = 0, 1, 2, 3
 # d_weight_mode of vamd_lce_backward (VAMD_DW_*)
-DW_STORE, DW_ADD_BF16, DW_F32_STORE, DW_F32_ADD, DW_F32_ADD_FINISH = 0, 1, 2, 3, 4
+DW_STORE, DW_ADD_BF16, DW_F32_STORE, DW_F32_ADD, DW_F32_ADD_FINISH, DW_NONE = 0, 1, 2, 3, 4, 5
 LCE_TIMING_KERNELS = 5
 AGG_MODES = {
     "token-mean": 0,
@@ -133,7 +133,7 @@ def lib_path() -> str:
     return _LIB_PATH
 
 
-ABI_VERSION = 4  # VAMD_ABI_VERSION of include/verl_amd.h
+ABI_VERSION = 5  # VAMD_ABI_VERSION of include/verl_amd.h
 
 
 def load_library(path: str | None = None) -> ctypes.CDLL:

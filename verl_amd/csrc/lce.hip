@@ -910,13 +910,15 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
                                  size_t workspace_bytes, void* stream) {
   int st = check_head_shapes(n_tokens, hidden_size, vocab, logits_cache);
   if (st != VAMD_OK) return st;
-  VAMD_REQUIRE(hidden && weight && labels && lse && mean_z && d_hidden, "lce_backward: null pointer");
+  VAMD_REQUIRE(hidden && weight && labels && lse && mean_z, "lce_backward: null pointer");
   VAMD_REQUIRE(rcp_temperature > 0.f, "lce_backward: temperature must be positive");
-  VAMD_REQUIRE(d_weight_mode >= VAMD_DW_STORE && d_weight_mode <= VAMD_DW_F32_ADD_FINISH,
+  VAMD_REQUIRE(d_weight_mode >= VAMD_DW_STORE && d_weight_mode <= VAMD_DW_NONE,
                "lce_backward: unknown d_weight_mode %d", d_weight_mode);
+  const bool want_dw = d_weight_mode != VAMD_DW_NONE;
+  VAMD_REQUIRE(d_hidden || want_dw, "lce_backward: neither d_hidden nor a weight gradient is asked for");
   {
     const bool writes_bf16 = d_weight_mode <= VAMD_DW_ADD_BF16 || d_weight_mode == VAMD_DW_F32_ADD_FINISH;
-    const bool uses_f32 = d_weight_mode >= VAMD_DW_F32_STORE;
+    const bool uses_f32 = want_dw && d_weight_mode >= VAMD_DW_F32_STORE;
     VAMD_REQUIRE(!writes_bf16 || d_weight, "lce_backward: d_weight_mode %d writes d_weight, which is null", d_weight_mode);
     VAMD_REQUIRE(!uses_f32 || (d_weight_acc32 && reinterpret_cast<uintptr_t>(d_weight_acc32) % 16 == 0),
                  "lce_backward: d_weight_mode %d needs a 16-byte aligned d_weight_acc32", d_weight_mode);
@@ -944,7 +946,7 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
   Carver carve(workspace);
   const int64_t pitch = dz_pitch(cv);
   uint16_t* dz = carve.take<uint16_t>((size_t)n_pad * pitch);
-  float* acc32 = n_chunks > 1 ? carve.take<float>((size_t)n_tokens * hidden_size) : nullptr;
+  float* acc32 = (n_chunks > 1 && d_hidden) ? carve.take<float>((size_t)n_tokens * hidden_size) : nullptr;
   const uint16_t* hid = static_cast<const uint16_t*>(hidden);
   const uint16_t* wgt = static_cast<const uint16_t*>(weight);
   const int h_tiles = (int)ceil_div(hidden_size, kTile);
@@ -1013,7 +1015,7 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
     gh.R = Operand{dz, pitch, (int)n_pad, (int)cv};
     gh.C = Operand{wgt + c0 * hidden_size, hidden_size, (int)hidden_size, (int)left};
     gh.k_slabs = (int)ceil_div(cols, kBK);
-    gh.r_tiles = tok_tiles;
+    gh.r_tiles = d_hidden ? tok_tiles : 0;  // an input that needs no gradient leaves its GEMM an empty tile list
     gh.c_tiles = h_tiles;
     gh.r_valid = (int)n_tokens;
     gh.c_valid = (int)hidden_size;
@@ -1029,7 +1031,7 @@ extern "C" int vamd_lce_backward(const void* hidden, const void* weight, const i
     gw.R = Operand{dz, pitch, (int)(ceil_div(cols, 8) * 8), (int)n_pad};
     gw.C = Operand{hid, hidden_size, (int)hidden_size, (int)n_tokens};
     gw.k_slabs = (int)ceil_div(n_tokens, kBK);
-    gw.r_tiles = chunk_tiles;
+    gw.r_tiles = want_dw ? chunk_tiles : 0;
     gw.c_tiles = h_tiles;
     gw.r_valid = (int)cols;
     gw.c_valid = (int)hidden_size;

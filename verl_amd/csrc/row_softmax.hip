@@ -165,7 +165,11 @@ __global__ __launch_bounds__(kRowThreads) void row_softmax_stats_kernel(StatsArg
     if (a.lse) a.lse[r] = lse;
     if (a.mean_z) a.mean_z[r] = mz;
     if (a.entropy) a.entropy[r] = lse - mz;
-    if (a.logprobs) a.logprobs[r] = to_float(row[a.labels[r]], D()) - lse;
+    if (a.logprobs) {
+      // a label outside [0, cols) (an ignore index such as -100, a padding id) reads nothing and yields 0
+      const int64_t lab = a.labels[r];
+      a.logprobs[r] = (lab >= 0 && lab < a.cols) ? to_float(row[lab], D()) - lse : 0.f;
+    }
   }
 }
 
@@ -234,16 +238,21 @@ __global__ __launch_bounds__(kRowThreads) void row_softmax_backward_kernel(Backw
   }
 }
 
+// min / max that hand a NaN operand on, like torch.min / torch.max of two tensors (fminf / fmaxf drop it)
+__device__ __forceinline__ float min_nan(float a, float b) { return (a != a || b != b) ? a + b : fminf(a, b); }
+__device__ __forceinline__ float max_nan(float a, float b) { return (a != a || b != b) ? a + b : fmaxf(a, b); }
+
 // out = max(min(x, hi), lo)
 __global__ __launch_bounds__(256) void clip_kernel(const float* __restrict__ x, const float* __restrict__ lo,
                                                    const float* __restrict__ hi, int64_t n, float* __restrict__ out) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
-    out[i] = fmaxf(fminf(x[i], hi[i]), lo[i]);
+    out[i] = max_nan(min_nan(x[i], hi[i]), lo[i]);
 }
 
 // Gradients of max(min(x, hi), lo) the way torch's binary min / max hand them out: the smaller (larger) operand
-// takes the gradient, equal operands take half each.
+// takes the gradient, equal operands take half each; an operand loses its share only where the comparison says it
+// lost, so where a NaN makes every comparison false both operands receive the whole gradient, as in torch.
 __global__ __launch_bounds__(256) void clip_backward_kernel(const float* __restrict__ x, const float* __restrict__ lo,
                                                             const float* __restrict__ hi, const float* __restrict__ g,
                                                             int64_t n, float* __restrict__ dx, float* __restrict__ dlo,
@@ -251,12 +260,15 @@ __global__ __launch_bounds__(256) void clip_backward_kernel(const float* __restr
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
     const float xv = x[i], l = lo[i], h = hi[i], gv = g[i];
-    const float a = fminf(xv, h);
-    const float a_x = xv < h ? 1.f : (xv == h ? 0.5f : 0.f);  // d min(x, hi) / dx; the rest goes to hi
-    const float o_a = a > l ? 1.f : (a == l ? 0.5f : 0.f);    // d max(a, lo) / da; the rest goes to lo
+    const float a = min_nan(xv, h);
+    const float tie1 = xv == h ? 0.5f : 1.f, tie2 = a == l ? 0.5f : 1.f;
+    const float a_x = xv > h ? 0.f : tie1;  // d min(x, hi) / dx
+    const float a_h = xv < h ? 0.f : tie1;  // d min(x, hi) / dhi
+    const float o_a = a < l ? 0.f : tie2;   // d max(a, lo) / da
+    const float o_l = a > l ? 0.f : tie2;   // d max(a, lo) / dlo
     if (dx) dx[i] = gv * o_a * a_x;
-    if (dhi) dhi[i] = gv * o_a * (1.f - a_x);
-    if (dlo) dlo[i] = gv * (1.f - o_a);
+    if (dhi) dhi[i] = gv * o_a * a_h;
+    if (dlo) dlo[i] = gv * o_l;
   }
 }
 

@@ -56,14 +56,12 @@ class FusedLinearForPPOFunction(torch.autograd.Function):
             dlog_probs = dlog_probs.reshape(-1)
         if dentropy is not None:
             dentropy = dentropy.reshape(-1)
+        # only the gradient GEMMs whose inputs require a gradient are run (reference :150-156, :184-187)
         dhidden_states, dvocab_weights = efficient_entropy_backward(
-            dlog_probs, dentropy, hidden_states, vocab_weights, input_ids, lse, mean_z, 0, ctx.temperature)
-        if not ctx.needs_input_grad[0]:
-            dhidden_states = None
-        elif ctx.orig_ndim == 3:
+            dlog_probs, dentropy, hidden_states, vocab_weights, input_ids, lse, mean_z, 0, ctx.temperature,
+            need_d_hidden=ctx.needs_input_grad[0], need_d_weight=ctx.needs_input_grad[1])
+        if dhidden_states is not None and ctx.orig_ndim == 3:
             dhidden_states = dhidden_states.view(ctx.orig_batch_size, -1, hidden_states.shape[-1])
-        if not ctx.needs_input_grad[1]:
-            dvocab_weights = None
         return dhidden_states, dvocab_weights, None, None, None
 
 

@@ -104,7 +104,8 @@ def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse,
                                temperature: float = 1.0, dist_process_group=None, d_entropy_scalar: float = 0.0,
                                d_weight_out: torch.Tensor | None = None, vocab_chunk: int = 0,
                                logits_cache: torch.Tensor | None = None,
-                               d_weight_acc32: torch.Tensor | None = None, acc32_step: str | None = None):
+                               d_weight_acc32: torch.Tensor | None = None, acc32_step: str | None = None,
+                               need_d_hidden: bool = True, need_d_weight: bool = True):
     """Host side of the backward kernels (reference kernels.py:1512-1723).
 
     ``dlogprobs`` / ``dentropy`` may be ``None`` (no contribution).  ``d_entropy_scalar`` adds a
@@ -115,6 +116,10 @@ def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse,
     ``weight.grad +=`` in bf16 training; with ``d_weight_acc32`` (fp32 ``[vocab, hidden]``) the sum is kept
     in fp32 and ``acc32_step`` says which call this is: ``"first"`` (store), ``"middle"`` (add) or ``"last"``
     (add, then write the sum, rounded once, to ``d_weight_out`` or a fresh tensor).
+    ``need_d_hidden`` / ``need_d_weight``: ``False`` for an input that requires no gradient (a frozen ``lm_head``,
+    detached hidden states): its gradient GEMM is not run and ``None`` is returned in its place, as the reference's
+    torch backend allocates and accumulates only the gradients its inputs require
+    (verl/utils/experimental/torch_functional.py:150-156, :184-187).
     Returns ``(d_hidden, d_weight)`` in ``hidden.dtype``; ``d_weight`` is ``None`` for the "first" and
     "middle" steps of an fp32 accumulation.
     """
@@ -145,8 +150,13 @@ def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse,
     if labels.dtype != torch.int64:
         labels = labels.to(torch.int64)
     L = _cabi.lib()
-    d_hidden = torch.empty_like(hidden)
-    if d_weight_acc32 is not None:
+    if not (need_d_hidden or need_d_weight):
+        return None, None
+    d_hidden = torch.empty_like(hidden) if need_d_hidden else None
+    if not need_d_weight:
+        assert d_weight_out is None and d_weight_acc32 is None, "no weight gradient was asked for"
+        mode, d_weight = _cabi.DW_NONE, None
+    elif d_weight_acc32 is not None:
         assert acc32_step in ("first", "middle", "last"), "acc32_step must be 'first', 'middle' or 'last'"
         assert d_weight_acc32.shape == weight.shape and d_weight_acc32.dtype == torch.float32
         assert d_weight_acc32.is_contiguous() and d_weight_acc32.device == dev
@@ -163,7 +173,7 @@ def efficient_entropy_backward(dlogprobs, dentropy, hidden, weight, labels, lse,
         _cabi.check(L.vamd_lce_backward(hidden.data_ptr(), weight.data_ptr(), labels.data_ptr(), n, h, v,
                                         1.0 / temperature, lse.data_ptr(), mean_z.data_ptr(), _cabi.ptr(dlogprobs),
                                         _cabi.ptr(dentropy), float(d_entropy_scalar), _cabi.ptr(logits_cache),
-                                        d_hidden.data_ptr(), _cabi.ptr(d_weight), mode, _cabi.ptr(d_weight_acc32),
+                                        _cabi.ptr(d_hidden), _cabi.ptr(d_weight), mode, _cabi.ptr(d_weight_acc32),
                                         int(vocab_chunk), ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
     return d_hidden, d_weight
 
@@ -242,8 +252,10 @@ class LinearCrossEntropy(torch.autograd.Function):
             dlogprobs = dlogprobs.reshape(-1)
         d_hidden, d_weight = efficient_entropy_backward(
             dlogprobs, dentropy, hidden, weight, labels, lse, mean_z, ctx.REDUCTION, ctx.temperature,
-            ctx.dist_process_group, logits_cache=cache)
-        d_hidden = d_hidden.view(ctx.original_hidden_shape)
+            ctx.dist_process_group, logits_cache=cache,
+            need_d_hidden=ctx.needs_input_grad[0], need_d_weight=ctx.needs_input_grad[1])
+        if d_hidden is not None:
+            d_hidden = d_hidden.view(ctx.original_hidden_shape)
         return (d_hidden, d_weight, None, None, None, None, None)
 
 

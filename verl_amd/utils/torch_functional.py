@@ -75,8 +75,17 @@ class _LogProbsFromLogits(torch.autograd.Function):
         return logprobs.to(logits.dtype).view(logits.shape[:-1])
 
     @staticmethod
+    @torch.autograd.function.once_differentiable
     def backward(ctx, g):
         rows, lab, lse = ctx.saved_tensors
+        if ctx.in_place:
+            # the logits are about to become their own gradient: a second pass over this node would read gradients
+            # where it expects logits
+            if getattr(ctx, "logits_overwritten", False):
+                raise RuntimeError("logprobs_from_logits(inplace_backward=True) wrote the gradient over the logits in "
+                                   "its first backward pass and cannot run a second one; pass inplace_backward=False "
+                                   "to keep the logits")
+            ctx.logits_overwritten = True
         d = _row_backward(rows, ctx.ld, lab, lse, None, g, None, ctx.in_place)
         return d.view(ctx.shape), None, None
 
@@ -101,8 +110,11 @@ class _EntropyFromLogits(torch.autograd.Function):
 
 def logprobs_from_logits(logits: torch.Tensor, labels: torch.Tensor, inplace_backward: bool = True) -> torch.Tensor:
     """Log-probability of ``labels`` under ``softmax(logits)``, shape ``logits.shape[:-1]``, dtype of ``logits``
-    (reference torch_functional.py:72-100).  With ``inplace_backward`` the backward pass writes the gradient over
-    the logits, as the reference's flash-attn path does: pass ``False`` when the logits are used again."""
+    (reference torch_functional.py:72-100).  With ``inplace_backward`` (the default, as in the reference) the
+    backward pass WRITES THE GRADIENT OVER THE LOGITS' STORAGE, as the reference's flash-attn path does
+    (``cross_entropy_loss(..., inplace_backward=True)``); the reference does so only where flash-attn is
+    installed, this function always.  Pass ``False`` when the logits are read again after the backward pass or
+    the graph is backpropagated twice (a second pass raises instead of differentiating gradients)."""
     return _LogProbsFromLogits.apply(logits, labels, inplace_backward)
 
 
@@ -334,14 +346,7 @@ def _raise_on_tiny_mask(mask_sum: float) -> None:
         raise ValueError("The sum of the mask is one, which can cause a division by zero.")
 
 
-def masked_var(values: torch.Tensor, mask: torch.Tensor, unbiased: bool = True) -> torch.Tensor:
-    """Masked variance with Bessel's factor (reference torch_functional.py:304-319).  The reference centres by
-    the mean in a second fp32 pass; here one pass accumulates count, sum and sum of squares in fp64 and the
-    variance is ``(S2 - 2 mean S1 + mean^2 S0) / S0`` evaluated in fp64.  With fp32 inputs the cancellation
-    costs a relative error of about ``(mean / std)^2 * 1e-16``: below fp32 resolution while ``|mean| / std``
-    stays under about 1e4."""
-    _, mom, _ = _global_moments(values, mask)
-    s0, s1, s2, _ = (x for x in mom.to("cpu").tolist())
+def _var_from_moments(s0: float, s1: float, s2: float, unbiased: bool) -> torch.Tensor:
     mean = torch.tensor(s1, dtype=torch.float32) / (torch.tensor(s0, dtype=torch.float32) + 1e-8)
     md = float(mean)
     var = torch.tensor(s2 - 2.0 * md * s1 + md * md * s0, dtype=torch.float32) / (
@@ -349,12 +354,65 @@ def masked_var(values: torch.Tensor, mask: torch.Tensor, unbiased: bool = True) 
     if unbiased:
         _raise_on_tiny_mask(s0)
         var = var * torch.tensor(s0 / (s0 - 1.0), dtype=torch.float32)
-    return var.to(values.device)
+    return var
 
 
-def masked_whiten(values: torch.Tensor, mask: torch.Tensor, shift_mean: bool = True) -> torch.Tensor:
-    """(values - mean) * rsqrt(var + 1e-8) on every element (reference torch_functional.py:322-339): one launch for
-    the masked moments and the statistics, one for the elementwise pass."""
+def _affine_masked(v, stats, m, code):
+    """``((v - stats[0]) * stats[1] + stats[2]) * mask`` through ``vamd_affine_by_stats_masked``."""
+    out = torch.empty_like(v)
+    dev = v.device
+    with _cabi.device_guard(dev):
+        _cabi.check(_cabi.lib().vamd_affine_by_stats_masked(v.data_ptr(), stats.data_ptr(), m.data_ptr(), code,
+                                                            v.numel(), out.data_ptr(), _cabi.stream_ptr(dev)))
+    return out
+
+
+def _variance_gradient_terms(s0: float, s1: float, unbiased: bool):
+    """With D = sum(mask) + 1e-8 and mean = S1 / D:  d var / d v_k = scale * w_k * (v_k - centre), where
+    centre = mean + (S1 - mean S0) / D carries the dependence of the mean on v_k (the second term is what the
+    epsilon in D leaves of sum_i w_i (v_i - mean)) and scale = 2 / D times Bessel's factor."""
+    d = s0 + 1e-8
+    mean = s1 / d
+    centre = mean + (s1 - mean * s0) / d
+    scale = 2.0 / d * (s0 / (s0 - 1.0) if unbiased else 1.0)
+    return mean, centre, scale, d
+
+
+class _MaskedVar(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, values, mask, unbiased: bool):
+        v, mom, dev = _global_moments(values, mask)
+        s0, s1, s2, _ = mom.to("cpu").tolist()
+        var = _var_from_moments(s0, s1, s2, unbiased)
+        m, code = _cabi.mask_code(_cabi.on_device(mask, dev).reshape(v.shape))
+        ctx.save_for_backward(v, m)
+        ctx.meta = (code, s0, s1, unbiased, tuple(values.shape), values.dtype, values.device)
+        return var.to(values.device)
+
+    @staticmethod
+    def backward(ctx, g):
+        v, m = ctx.saved_tensors
+        code, s0, s1, unbiased, shape, dtype, device = ctx.meta
+        _, centre, scale, _ = _variance_gradient_terms(s0, s1, unbiased)
+        gs = g.detach().to(device=v.device, dtype=torch.float32).reshape(1)
+        stats = torch.cat([gs.new_tensor([centre]), gs * scale, gs.new_zeros(2)])
+        return _affine_masked(v, stats, m, code).view(shape).to(device=device, dtype=dtype), None, None
+
+
+def masked_var(values: torch.Tensor, mask: torch.Tensor, unbiased: bool = True) -> torch.Tensor:
+    """Masked variance with Bessel's factor (reference torch_functional.py:304-319), differentiable in
+    ``values``.  The reference centres by the mean in a second fp32 pass; here one pass accumulates count, sum and
+    sum of squares in fp64 and the variance is ``(S2 - 2 mean S1 + mean^2 S0) / S0`` evaluated in fp64.  With
+    fp32 inputs the cancellation costs a relative error of about ``(mean / std)^2 * 1e-16``: below fp32
+    resolution while ``|mean| / std`` stays under about 1e4."""
+    if values.requires_grad and torch.is_grad_enabled():
+        return _MaskedVar.apply(values, mask, unbiased)
+    _, mom, _ = _global_moments(values, mask)
+    s0, s1, s2, _ = mom.to("cpu").tolist()
+    return _var_from_moments(s0, s1, s2, unbiased).to(values.device)
+
+
+def _masked_whiten_forward(values, mask, shift_mean: bool):
     dev = _cabi.compute_device(values, mask)
     v, m, code = _as_matrix(values, mask, dev)
     rows, cols = v.shape
@@ -368,5 +426,47 @@ def masked_whiten(values: torch.Tensor, mask: torch.Tensor, shift_mean: bool = T
         _cabi.check(L.vamd_masked_reduce(v.data_ptr(), m.data_ptr(), code, rows, cols, 0, mom.data_ptr(), None, None,
                                          None, stats.data_ptr(), int(shift_mean), ws.data_ptr(), ws.numel(), s))
         _cabi.check(L.vamd_affine_by_stats(v.data_ptr(), stats.data_ptr(), v.numel(), out.data_ptr(), s))
+    return out, v, m, code, mom, stats
+
+
+class _MaskedWhiten(torch.autograd.Function):
+    """Gradient of ``out_j = (v_j - mean) r [+ mean]`` with ``r = rsqrt(var + 1e-8)``, mean and var taken over the
+    mask: ``d_k = g_k r + w_k [(1[not shift] - r) G0 / D - r^3 G1 (d var / d v_k) / 2]`` with ``G0 = sum g`` and
+    ``G1 = sum g (v - mean)`` over every element.  G0 and ``sum g v`` come from one masked-moments launch that
+    takes ``g`` as the weights; the bracket is one ``vamd_affine_by_stats_masked`` pass."""
+
+    @staticmethod
+    def forward(ctx, values, mask, shift_mean: bool):
+        out, v, m, code, mom, stats = _masked_whiten_forward(values, mask, shift_mean)
+        s0, s1 = mom[:2].tolist()
+        _raise_on_tiny_mask(s0)
+        ctx.save_for_backward(v, m, stats)
+        ctx.meta = (code, s0, s1, shift_mean, tuple(values.shape), values.dtype, values.device)
+        return out.view(values.shape).to(values.device)
+
+    @staticmethod
+    def backward(ctx, g):
+        v, m, stats = ctx.saved_tensors
+        code, s0, s1, shift_mean, shape, dtype, device = ctx.meta
+        dev = v.device
+        mean, centre, scale, d = _variance_gradient_terms(s0, s1, True)
+        gs = g.detach().to(device=dev, dtype=torch.float32).reshape(v.shape).contiguous()
+        gm = _moments(v, gs, per_row=False)            # sum g, sum g v (g as weights), in fp64 on the device
+        r = stats[1].to(torch.float64)
+        g0, g1 = gm[0], gm[1] - mean * gm[0]
+        slope = -0.5 * r * r * r * g1 * scale            # multiplies w_k (v_k - centre)
+        const = ((0.0 if shift_mean else 1.0) - r) * g0 / d
+        st = torch.stack([torch.full_like(slope, centre), slope, const, torch.zeros_like(slope)]).to(torch.float32)
+        res = _affine_masked(v, st, m, code)
+        res.add_(gs * stats[1])
+        return res.view(shape).to(device=device, dtype=dtype), None, None
+
+
+def masked_whiten(values: torch.Tensor, mask: torch.Tensor, shift_mean: bool = True) -> torch.Tensor:
+    """(values - mean) * rsqrt(var + 1e-8) on every element (reference torch_functional.py:322-339): one launch for
+    the masked moments and the statistics, one for the elementwise pass.  Differentiable in ``values``."""
+    if values.requires_grad and torch.is_grad_enabled():
+        return _MaskedWhiten.apply(values, mask, shift_mean)
+    out, _, _, _, mom, _ = _masked_whiten_forward(values, mask, shift_mean)
     _raise_on_tiny_mask(mom[0].item())   # the reference raises here too; the pass above is already queued
     return out.view(values.shape).to(values.device)
