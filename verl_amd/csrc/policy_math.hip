@@ -51,7 +51,7 @@ __device__ __forceinline__ void totals_epilogue(const Work& wk, int64_t rows, in
     for (int64_t r = threadIdx.x; r < rows; r += kRcThreads) coef[r] = c_all;
   ticket_reset(wk.ticket);
 }
-inline bool totals_suffice(int mode) {
+__host__ __device__ inline bool totals_suffice(int mode) {
   return mode == VAMD_AGG_TOKEN_MEAN || mode == VAMD_AGG_SEQ_MEAN_TOKEN_SUM_NORM;
 }
 
@@ -221,6 +221,10 @@ __global__ __launch_bounds__(kRcThreads) void agg_kernel(const float* __restrict
     store_record<2>(wk.partials, row, chunk, rows, chunks, acc);
   }
   if constexpr (FOLD) {
+    if (totals_suffice(ap.mode)) {  // no per-row pass: the launch totals are all these modes need
+      totals_epilogue<2, kEpiAgg>(wk, rows, chunks, cols, ap, coef, out_loss, smem);
+      return;
+    }
     if (!last_block_arrives(wk.ticket)) return;
     double loss, msum, extra[1];
     finalize_agg<2>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
@@ -576,6 +580,10 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
     store_record<5>(wk.partials, row, chunk, rows, chunks, acc);
   }
   if constexpr (FOLD) {
+    if (!ROWS && totals_suffice(ap.mode)) {  // no per-row pass: the launch totals are all these modes need
+      totals_epilogue<5, kEpiPolicy>(wk, rows, chunks, cols, ap, coef, out, smem);
+      return;
+    }
     if (!last_block_arrives(wk.ticket)) return;
     double loss, msum, extra[3];
     finalize_agg<5>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
@@ -638,6 +646,10 @@ __global__ __launch_bounds__(kRcThreads) void value_kernel(
     store_record<3>(wk.partials, row, chunk, rows, chunks, acc);
   }
   if constexpr (FOLD) {
+    if (totals_suffice(ap.mode)) {  // no per-row pass: the launch totals are all these modes need
+      totals_epilogue<3, kEpiValue>(wk, rows, chunks, cols, ap, coef, out, smem);
+      return;
+    }
     if (!last_block_arrives(wk.ticket)) return;
     double loss, msum, extra[1];
     finalize_agg<3>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
@@ -729,6 +741,10 @@ __global__ __launch_bounds__(kRcThreads) void kl_loss_kernel(
     store_record<2>(wk.partials, row, chunk, rows, chunks, acc);
   }
   if constexpr (FOLD) {
+    if (totals_suffice(ap.mode)) {  // no per-row pass: the launch totals are all these modes need
+      totals_epilogue<2, kEpiKl>(wk, rows, chunks, cols, ap, coef, out, smem);
+      return;
+    }
     if (!last_block_arrives(wk.ticket)) return;
     double loss, msum, extra[1];
     finalize_agg<2>(wk.partials, rows, chunks, cols, ap, coef, loss, msum, extra, smem);
