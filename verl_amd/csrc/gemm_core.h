@@ -164,6 +164,21 @@ __device__ __forceinline__ void load_to_lds_16(const u32x4& rsrc, unsigned voff,
                : "memory", "m0");
 }
 
+// The same for 4 bytes per lane: lane L's dword lands at lds_base + 4 L (256 consecutive bytes per instruction).
+__device__ __forceinline__ void load_to_lds_4(const u32x4& rsrc, unsigned voff, unsigned lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tbuffer_load_dword %0, %1, 0 offen lds"
+               :
+               : "v"(voff), "s"(rsrc), "s"(lds_base)
+               : "memory", "m0");
+}
+// Buffer resource over `bytes` bytes at p (raw 32-bit format, reads past the end return zero).
+__device__ __forceinline__ u32x4 span_rsrc(const void* p, int64_t bytes) {
+  if (bytes < 0) bytes = 0;
+  if (bytes > 0xffffffffll) bytes = 0xffffffffll;
+  const uint64_t base = reinterpret_cast<uint64_t>(p);
+  return u32x4{(unsigned)base, (unsigned)(base >> 32) & 0xffffu, (unsigned)bytes, 0x00020000u};
+}
+
 // Memory -> LDS transfer of one operand slab: kLoads loads of 16 bytes per lane.  Load i of wavefront
 // w fills the 1 KB LDS block (w + kWaves i) of the slab:
 //   direct : block b = rows 8 b .. 8 b + 7; lane L sits at row 8 b + L / 8, chunk position L % 8,
@@ -329,6 +344,12 @@ static_assert(kLoads == 4, "the s_waitcnt vmcnt(4 / 6) of slab_iter counts the t
 //   Sched : int count();  void tile(int i, int& r0, int& c0);
 //   Epi   : void operator()(Accum& acc, int r0, int c0);   (registers + global memory only, or LDS
 //           beyond the first kLdsBytes)
+//           void prefetch(int tile, int r0, int c0);  called by every wavefront before the first slab of tile
+//           `tile` is multiplied: memory -> LDS transfers issued here have landed, and are visible to the
+//           whole workgroup, when that tile's epilogue runs (they are older than every slab transfer the tile
+//           issues, and the slab pipeline's waits and barriers cover them); an epilogue that needs per-row
+//           values stages them this way instead of loading them itself, which would have it wait out its own
+//           loads AND every slab transfer in flight (one counter counts both)
 //
 // All (tile, slab) pairs of the workgroup form one stream of slabs; slab it+1 is landing in LDS
 // and slab it+2 is requested while slab it is multiplied, across tile boundaries too, so only the
@@ -384,6 +405,7 @@ __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, in
     dc.issue_one(i, src_c, lds_address(lds) + 3 * kSlabBytes);
   }
   advance();  // cursor now on slab 2
+  epi.prefetch(0, r0, c0);
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
   Frags f;
 #pragma unroll
@@ -396,6 +418,7 @@ __device__ __forceinline__ void run_tiles(const Operand& R, const Operand& C, in
     Accum acc;
     accum_zero(acc);
     sched.tile(tile, r0, c0);
+    if (tile > 0) epi.prefetch(tile, r0, c0);
     for (int kt = 0; kt < k_slabs; ++kt) {
       char* cur = lds + stage * 2 * kSlabBytes;
       const char* nxt = lds + (stage ^ 1) * 2 * kSlabBytes;

@@ -149,6 +149,7 @@ struct FwdEpi {
   int tok0;        // CACHE: first token row of the wavefront
   int n_tokens;
 
+  __device__ __forceinline__ void prefetch(int, int, int) {}
   __device__ __forceinline__ void operator()(Accum& acc, int /*r0*/, int c0) {
     const bool ragged = c0 + kTile > vocab;
     if constexpr (CACHE) {
@@ -177,16 +178,26 @@ struct FwdEpi {
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
       float ymax = kNegBig;
-      // pass 1: scale into the log2 domain in place, mask the vocabulary tail, tile max
+      // pass 1: scale into the log2 domain in place, mask the vocabulary tail (last tile only), tile max
+      if (ragged) {
 #pragma unroll
-      for (int mb = 0; mb < kMB; ++mb)
+        for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-          float y = acc.a[mb][nb][v] * scale2;
-          if (ragged) y = (c0 + acc_col(p, mb, v) < vocab) ? y : kNegBig;
-          acc.a[mb][nb][v] = y;
-          ymax = fmaxf(ymax, y);
-        }
+          for (int v = 0; v < 4; ++v) {
+            const float y = (c0 + acc_col(p, mb, v) < vocab) ? acc.a[mb][nb][v] * scale2 : kNegBig;
+            acc.a[mb][nb][v] = y;
+            ymax = fmaxf(ymax, y);
+          }
+      } else {
+#pragma unroll
+        for (int mb = 0; mb < kMB; ++mb)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const float y = acc.a[mb][nb][v] * scale2;
+            acc.a[mb][nb][v] = y;
+            ymax = fmaxf(ymax, y);
+          }
+      }
       // label logit: only when some lane's label falls in this wavefront's 128 columns
       const int rel = lab[nb] - c0 - p.wc * 128;
       if (__any(rel >= 0 && rel < 128)) {
@@ -385,62 +396,163 @@ struct RecomputeArgs {
   int dz_ld;
 };
 
+// The same hand-over for a bf16 result: the wavefront's patch holds 32 rows x 32 columns of bf16 (2 KB), rounded
+// before the exchange, so the LDS traffic is half that of the fp32 patch and the global stores are 16 bytes per
+// lane: a store instruction covers 16 rows x 64 bytes.  16-byte chunk c of row r lives at position c ^ ((r >> 2) & 3)
+// so that the 8-byte writes of 16 rows at one column spread over the banks.  After the exchange lane L holds columns
+// 8 (L % 4) .. + 7 of rows 16 i + L / 4 (i = 0, 1).
+struct BlockExchangeBf16 {
+  char* stage;
+  int lx, lq, rd_row, rd_chunk;
+  __device__ __forceinline__ void init(char* area, const LanePos& p) {
+    stage = area + (threadIdx.x >> 6) * 2048;
+    lx = p.lx;
+    lq = p.lq;
+    rd_row = (threadIdx.x & 63) >> 2;
+    rd_chunk = threadIdx.x & 3;
+  }
+  __device__ __forceinline__ void run(const f32x4 (&blk)[2][2], u32x4 (&out)[2]) const {
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+        const int row = 16 * rb + lx;
+        const int chunk = (2 * cb + (lq >> 1)) ^ ((row >> 2) & 3);
+        *reinterpret_cast<u32x2*>(stage + row * 64 + chunk * 16 + (lq & 1) * 8) =
+            pack_bf16x4(blk[cb][rb][0], blk[cb][rb][1], blk[cb][rb][2], blk[cb][rb][3]);
+      }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int row = 16 * i + rd_row;
+      out[i] = *reinterpret_cast<const u32x4*>(stage + row * 64 + ((rd_chunk ^ ((row >> 2) & 3)) << 4));
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+};
+constexpr int kBf16StageBytes = (kThreads / 64) * 2048;  // one 32 x 32 bf16 patch per wavefront
+
+// Per-token inputs of the d_logits epilogue (lse, mean_z, g_lp, label, g_ent) for the 256 tokens of a tile, staged
+// in LDS by memory -> LDS transfers issued when the tile's first slab starts (prefetch): five arrays of 256 dwords,
+// two sets used in turn so that a tile's transfers never land in what the previous tile's epilogue still reads.
+constexpr int kTokArrays = 5, kTokSetBytes = kTokArrays * kTile * 4;
+constexpr int kRecomputeExtraLds = kBf16StageBytes + 2 * kTokSetBytes;
+static_assert(kRecomputeExtraLds <= kCacheStageBytes, "the recompute kernel is launched with the cache stage's LDS");
+
 struct RecomputeEpi {
   LanePos p;
   const RecomputeArgs* a;
-  BlockExchange ex;
+  BlockExchangeBf16 ex;
+  char* tok_stage;  // [2][kTokArrays][256] dwords
+  int parity;       // set of the tile whose epilogue runs next
+
+  __device__ __forceinline__ void init(char* lds_after_pipeline, const LanePos& pos, const RecomputeArgs* args) {
+    p = pos;
+    a = args;
+    ex.init(lds_after_pipeline, pos);
+    tok_stage = lds_after_pipeline + kBf16StageBytes;
+    parity = 0;
+  }
+
+  // wavefront w brings in half (w & 1) of array (w >> 1): 0 lse, 1 mean_z, 2 g_lp, 3 labels (low dwords); the
+  // wavefronts 0 and 1 also bring in g_ent when it is a tensor
+  __device__ __forceinline__ void prefetch(int tile, int r0, int /*c0*/) {
+    const RecomputeArgs& A = *a;
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const unsigned lane = threadIdx.x & 63u;
+    const int arr = w >> 1, half = w & 1;
+    const unsigned set_lds = lds_address(tok_stage) + (unsigned)(tile & 1) * kTokSetBytes;
+    const void* src = arr == 0 ? (const void*)A.lse : arr == 1 ? (const void*)A.mean_z
+                      : arr == 2 ? (const void*)A.g_lp : (const void*)A.labels;
+    const unsigned elt = arr == 3 ? 8u : 4u;
+    if (src) {  // uniform over the wavefront
+      const u32x4 rs = span_rsrc(src, (int64_t)A.n_tokens * elt);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const unsigned tok = (unsigned)r0 + half * 128u + i * 64u + lane;
+        load_to_lds_4(rs, tok * elt, set_lds + arr * (kTile * 4) + (half * 128u + i * 64u) * 4u);
+      }
+    }
+    if (A.g_ent && w < 2) {
+      const u32x4 rs = span_rsrc(A.g_ent, (int64_t)A.n_tokens * 4);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const unsigned tok = (unsigned)r0 + half * 128u + i * 64u + lane;
+        load_to_lds_4(rs, tok * 4u, set_lds + 4 * (kTile * 4) + (half * 128u + i * 64u) * 4u);
+      }
+    }
+  }
+
+  // d_logits of the two token rows (rb) x 128 columns the lane holds of 32-row patch nb2, rounded, handed over and
+  // stored.  PLAIN: a tile inside the matrix with no label in the wavefront's 128 columns -- nothing but the
+  // arithmetic, four multiply-adds and an exponential per element; otherwise the one-hot term and the zeros for
+  // padding rows and columns come in through two comparisons per element (no branches).
+  //   code[rb]: 4 mb + v of the element of row rb that holds the label's column, or -1
+  //   lim[rb] : columns of the wavefront's 128 that exist for row rb (0 for a padding row), minus 4 lq
+  template <bool PLAIN>
+  __device__ __forceinline__ void patch_rows(Accum& acc, int nb2, int r0, int c0, const float (&lse2)[2],
+                                             const float (&mz)[2], const float (&glp)[2], const float (&gent)[2],
+                                             const int (&code)[2], const int (&lim)[2]) {
+    const RecomputeArgs& A = *a;
+#pragma unroll
+    for (int mb2 = 0; mb2 < kMB2; ++mb2) {
+      f32x4 d[2][2];
+#pragma unroll
+      for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int mb = 2 * mb2 + cb;
+            const float x = acc.a[mb][2 * nb2 + rb][v];
+            const float prob = fast_exp2(fmaf(x, A.scale2, -lse2[rb]));
+            const float u = fmaf(gent[rb], fmaf(x, A.rcp_t, -mz[rb]), glp[rb]);  // g_lp/T + g_ent/T * (z - mean_z)
+            if constexpr (PLAIN) {
+              d[cb][rb][v] = -prob * u;
+            } else {
+              const float onehot = code[rb] == 4 * mb + v ? glp[rb] : 0.f;
+              const float dzv = fmaf(-prob, u, onehot);
+              d[cb][rb][v] = (mb * kBlk + v) < lim[rb] ? dzv : 0.f;  // every row of the panel is written, padding as zeros
+            }
+          }
+      u32x4 o[2];
+      ex.run(d, o);
+      const int col0 = c0 + p.wc * 128 + mb2 * 32 + 8 * ex.rd_chunk;
+      const int64_t row0 = r0 + p.wr * (kNB * kBlk) + nb2 * 32 + ex.rd_row;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) *reinterpret_cast<u32x4*>(A.dz + (row0 + 16 * i) * A.dz_ld + col0) = o[i];
+    }
+  }
+
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const RecomputeArgs& A = *a;
+    const float* tokf = reinterpret_cast<const float*>(tok_stage + parity * kTokSetBytes);
+    const int* toki = reinterpret_cast<const int*>(tokf);
+    parity ^= 1;
+    const bool inside = r0 + kTile <= A.n_tokens && c0 + kTile <= A.vocab_left;  // uniform over the workgroup
+    const int cols_left = A.vocab_left - c0 - p.wc * 128 - 4 * p.lq;
 #pragma unroll
     for (int nb2 = 0; nb2 < kNB2; ++nb2) {
       // the lane's two token rows of this 32-row patch
       float lse2[2], mz[2], glp[2], gent[2];
-      int rel[2];
-      bool live[2];
+      int code[2], lim[2];
+      bool hit = false;
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb) {
-        const int tok = r0 + acc_row(p, 2 * nb2 + rb);
-        live[rb] = tok < A.n_tokens;
-        lse2[rb] = mz[rb] = glp[rb] = gent[rb] = 0.f;
-        rel[rb] = -1;
-        if (live[rb]) {
-          lse2[rb] = A.lse[tok] * kLog2e;
-          mz[rb] = A.mean_z[tok];
-          glp[rb] = (A.g_lp ? A.g_lp[tok] : 0.f) * A.rcp_t;
-          gent[rb] = (A.g_ent ? A.g_ent[tok] : A.g_ent_scalar) * A.rcp_t;
-          rel[rb] = (int)A.labels[tok] - A.chunk_c0 - c0 - p.wc * 128;
-        }
+        const int t = acc_row(p, 2 * nb2 + rb);  // row inside the tile
+        lse2[rb] = tokf[t] * kLog2e;
+        mz[rb] = tokf[kTile + t];
+        glp[rb] = (A.g_lp ? tokf[2 * kTile + t] : 0.f) * A.rcp_t;
+        gent[rb] = (A.g_ent ? tokf[4 * kTile + t] : A.g_ent_scalar) * A.rcp_t;
+        const int rel = toki[3 * kTile + t] - A.chunk_c0 - c0 - p.wc * 128;  // label's column among the wavefront's 128
+        const bool here = rel >= 0 && rel < 128;
+        hit = hit || here;
+        // the lane holds columns 16 mb + 4 lq + v: the label's is one of them when its 4-column group is lq
+        code[rb] = (here && ((rel >> 2) & 3) == p.lq) ? 4 * (rel >> 4) + (rel & 3) : -1;
+        lim[rb] = r0 + t < A.n_tokens ? cols_left : 0;
       }
-      const bool hit = __any((rel[0] >= 0 && rel[0] < 128) || (rel[1] >= 0 && rel[1] < 128));
-#pragma unroll
-      for (int mb2 = 0; mb2 < kMB2; ++mb2) {
-        f32x4 d[2][2];
-#pragma unroll
-        for (int cb = 0; cb < 2; ++cb)
-#pragma unroll
-          for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-              const int mb = 2 * mb2 + cb;
-              const float x = acc.a[mb][2 * nb2 + rb][v];
-              const float prob = fast_exp2(fmaf(x, A.scale2, -lse2[rb]));
-              const float u = fmaf(gent[rb], fmaf(x, A.rcp_t, -mz[rb]), glp[rb]);  // g_lp/T + g_ent/T * (z - mean_z)
-              float dzv = -prob * u;
-              const int col = mb * kBlk + 4 * p.lq + v;
-              if (hit) dzv += (col == rel[rb]) ? glp[rb] : 0.f;
-              const bool ok = live[rb] && (c0 + p.wc * 128 + col) < A.vocab_left;
-              d[cb][rb][v] = ok ? dzv : 0.f;
-            }
-        // every row of the panel is written, padding rows and columns as zeros
-        f32x4 o[4];
-        ex.run(d, o);
-        const int col0 = c0 + p.wc * 128 + mb2 * 32 + 4 * ex.rd_chunk;
-        const int64_t row0 = r0 + p.wr * (kNB * kBlk) + nb2 * 32 + ex.rd_row;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          *reinterpret_cast<u32x2*>(A.dz + (row0 + 8 * i) * A.dz_ld + col0) =
-              pack_bf16x4(o[i][0], o[i][1], o[i][2], o[i][3]);
-      }
+      if (inside && !__any(hit)) patch_rows<true>(acc, nb2, r0, c0, lse2, mz, glp, gent, code, lim);
+      else patch_rows<false>(acc, nb2, r0, c0, lse2, mz, glp, gent, code, lim);
     }
   }
 };
@@ -453,9 +565,7 @@ __global__ __launch_bounds__(kThreads) void lce_recompute_kernel(RecomputeArgs a
   sched.nwg = gridDim.x;
   sched.wg = xcd_regroup(blockIdx.x, gridDim.x);
   RecomputeEpi epi;
-  epi.p = lane_pos();
-  epi.a = &a;
-  epi.ex.init(lds + kLdsBytes, epi.p);
+  epi.init(lds + kLdsBytes, lane_pos(), &a);
   run_tiles<false, false>(a.hidden, a.weight, a.k_slabs, sched, epi, lds);
 }
 
@@ -521,6 +631,7 @@ struct DHiddenEpi {
   LanePos p;
   const GemmOutArgs* a;
   BlockExchange ex;
+  __device__ __forceinline__ void prefetch(int, int, int) {}
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const GemmOutArgs& A = *a;
     const bool read_prev = A.mode == kAddF32 || A.mode == kFinalBf16AddPrev;
@@ -560,6 +671,7 @@ struct DWeightEpi {
   LanePos p;
   const GemmOutArgs* a;
   BlockExchange ex;
+  __device__ __forceinline__ void prefetch(int, int, int) {}
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const GemmOutArgs& A = *a;
 #pragma unroll
