@@ -130,6 +130,7 @@ struct BlockExchange {
 };
 
 constexpr int kCacheStageBytes = (kThreads / 64) * 4096;  // one 32 x 32 fp32 patch per wavefront
+constexpr int kFwdTokenLds = kTile * 4 + kThreads * kNB * 4;  // forward without a cache: labels + label-logit sums
 
 // Per-lane online-softmax state for the kNB token slots (nb) the lane owns.  With CACHE the
 // scaled logits of every valid (token, vocabulary column) are also written out in fp32, so the
@@ -141,8 +142,13 @@ struct FwdEpi {
   LanePos p;
   float scale2;
   int vocab;
-  float m[kNB], s[kNB], sy[kNB], zl[kNB], s2[kNB];
-  int lab[kNB];
+  float m[kNB], s[kNB], sy[kNB], s2[kNB];
+  // The labels of the lane's token rows and the label-logit sums live in LDS behind the pipeline's stages when the
+  // kernel has LDS to spare (no logits cache), in registers otherwise: with them in registers the kernel spilled,
+  // and every reload of a spilled value waits out the slab transfers in flight (one counter counts both).
+  float zl[CACHE ? kNB : 1];
+  int lab[CACHE ? kNB : 1];
+  unsigned lab_lds, zl_lds;  // LDS byte addresses: labels [256] by tile row; sums [kThreads][kNB]
   float rcp_t;
   float* z_cache;  // CACHE: [n_tokens][vocab]
   BlockExchange ex;  // CACHE
@@ -199,15 +205,27 @@ struct FwdEpi {
           }
       }
       // label logit: only when some lane's label falls in this wavefront's 128 columns
-      const int rel = lab[nb] - c0 - p.wc * 128;
+      typedef int __attribute__((address_space(3))) * lds_i32_t;
+      typedef float __attribute__((address_space(3))) * lds_f32_t;
+      int label;
+      if constexpr (CACHE) label = lab[nb];
+      else label = *(lds_i32_t)(uintptr_t)(lab_lds + 4u * (unsigned)acc_row(p, nb));
+      const int rel = label - c0 - p.wc * 128;
       if (__any(rel >= 0 && rel < 128)) {
+        float add = 0.f;
 #pragma unroll
         for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
             const int col = mb * kBlk + 4 * p.lq + v;
-            zl[nb] += (col == rel) ? acc.a[mb][nb][v] * kLn2 : 0.f;
+            add += (col == rel) ? acc.a[mb][nb][v] * kLn2 : 0.f;
           }
+        if constexpr (CACHE) {
+          zl[nb] += add;
+        } else {
+          const lds_f32_t slot = (lds_f32_t)(uintptr_t)(zl_lds + 4u * (threadIdx.x * kNB + nb));
+          *slot += add;
+        }
       }
       const float m_new = fmaxf(m[nb], ymax);
       const float resc = fast_exp2(m[nb] - m_new);
@@ -277,10 +295,27 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
     epi.m[nb] = kNegBig;
     epi.s[nb] = 0.f;
     epi.sy[nb] = 0.f;
-    epi.zl[nb] = 0.f;
     epi.s2[nb] = 0.f;
-    const int tok = sched.r0_ + acc_row(epi.p, nb);
-    epi.lab[nb] = tok < a.n_tokens ? (int)a.labels[tok] : -1;
+    if constexpr (CACHE) {
+      epi.zl[nb] = 0.f;
+      const int tok = sched.r0_ + acc_row(epi.p, nb);
+      epi.lab[nb] = tok < a.n_tokens ? (int)a.labels[tok] : -1;
+    }
+  }
+  if constexpr (!CACHE) {
+    typedef float __attribute__((address_space(3))) * lds_f32_t;
+    epi.lab_lds = lds_address(lds + kLdsBytes);
+    epi.zl_lds = epi.lab_lds + kTile * 4;
+#pragma unroll
+    for (int nb = 0; nb < kNB; ++nb) *(lds_f32_t)(uintptr_t)(epi.zl_lds + 4u * (threadIdx.x * kNB + nb)) = 0.f;
+    // the low dwords of the tile's 256 labels, 64 per wavefront of the first four, straight into LDS; a token past
+    // the end reads as label 0, whose sums nobody looks at.  The transfers are older than every slab transfer, so
+    // the pipeline's first wait and barrier cover them.
+    const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (w < 4) {
+      const u32x4 rs = span_rsrc(a.labels, (int64_t)a.n_tokens * 8);
+      load_to_lds_4(rs, ((unsigned)sched.r0_ + 64u * w + (threadIdx.x & 63u)) * 8u, epi.lab_lds + 64u * w * 4u);
+    }
   }
   epi.z_cache = a.z_cache;
   epi.ex.init(lds + kLdsBytes, epi.p);
@@ -289,6 +324,13 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
 
   run_tiles<false, false>(a.hidden, a.weight, a.k_slabs, sched, epi, lds);
 
+  float zl[kNB];
+#pragma unroll
+  for (int nb = 0; nb < kNB; ++nb) {
+    typedef float __attribute__((address_space(3))) * lds_f32_t;
+    if constexpr (CACHE) zl[nb] = epi.zl[nb];
+    else zl[nb] = *(lds_f32_t)(uintptr_t)(epi.zl_lds + 4u * (threadIdx.x * kNB + nb));
+  }
   // merge the four lane quarters (they hold disjoint vocabulary columns of the same token) ...
 #pragma unroll
   for (int step = 16; step <= 32; step *= 2)
@@ -297,14 +339,14 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
       const float m2 = __shfl_xor(epi.m[nb], step, 64);
       const float s2 = __shfl_xor(epi.s[nb], step, 64);
       const float sy2 = __shfl_xor(epi.sy[nb], step, 64);
-      const float z2 = __shfl_xor(epi.zl[nb], step, 64);
+      const float z2 = __shfl_xor(zl[nb], step, 64);
       if (PI2) {
         const float q2 = __shfl_xor(epi.s2[nb], step, 64);
         merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], epi.s2[nb], m2, s2, sy2, q2);
       } else {
         merge_state(epi.m[nb], epi.s[nb], epi.sy[nb], m2, s2, sy2);
       }
-      epi.zl[nb] += z2;
+      zl[nb] += z2;
     }
   // ... then the two wavefronts that share a token quarter (wc = 0/1), through LDS (once every
   // wavefront's last slab transfers have landed).
@@ -314,7 +356,7 @@ __global__ __launch_bounds__(kThreads) void lce_forward_kernel(FwdArgs a) {
   if (epi.p.lq == 0) {
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
-      red[epi.p.wc * kTile + acc_row(epi.p, nb)] = make_float4(epi.m[nb], epi.s[nb], epi.sy[nb], epi.zl[nb]);
+      red[epi.p.wc * kTile + acc_row(epi.p, nb)] = make_float4(epi.m[nb], epi.s[nb], epi.sy[nb], zl[nb]);
       if (PI2) redq[epi.p.wc * kTile + acc_row(epi.p, nb)] = epi.s2[nb];
     }
   }
@@ -526,8 +568,12 @@ struct RecomputeEpi {
 
   __device__ __forceinline__ void operator()(Accum& acc, int r0, int c0) {
     const RecomputeArgs& A = *a;
-    const float* tokf = reinterpret_cast<const float*>(tok_stage + parity * kTokSetBytes);
-    const int* toki = reinterpret_cast<const int*>(tokf);
+    // read through LDS-typed pointers: as generic pointers some of these became flat loads, whose wait also
+    // waits out every slab transfer in flight
+    typedef const float __attribute__((address_space(3))) * lds_f32_t;
+    typedef const int __attribute__((address_space(3))) * lds_i32_t;
+    const lds_f32_t tokf = (lds_f32_t)(uintptr_t)(lds_address(tok_stage) + (unsigned)parity * kTokSetBytes);
+    const lds_i32_t toki = (lds_i32_t)tokf;
     parity ^= 1;
     const bool inside = r0 + kTile <= A.n_tokens && c0 + kTile <= A.vocab_left;  // uniform over the workgroup
     const int cols_left = A.vocab_left - c0 - p.wc * 128 - 4 * p.lq;
@@ -767,8 +813,8 @@ static int ensure_lds_attributes() {
   std::lock_guard<std::mutex> lock(mu);
   if (done[dev]) return VAMD_OK;
   int s;
-  if ((s = allow_big_lds(lce_forward_kernel<false, false>)) != VAMD_OK) return s;
-  if ((s = allow_big_lds(lce_forward_kernel<false, true>)) != VAMD_OK) return s;
+  if ((s = allow_big_lds(lce_forward_kernel<false, false>, kLdsBytes + kFwdTokenLds)) != VAMD_OK) return s;
+  if ((s = allow_big_lds(lce_forward_kernel<false, true>, kLdsBytes + kFwdTokenLds)) != VAMD_OK) return s;
   if ((s = allow_big_lds(lce_forward_kernel<true, false>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) return s;
   if ((s = allow_big_lds(lce_forward_kernel<true, true>, kLdsBytes + kCacheStageBytes)) != VAMD_OK) return s;
   if ((s = allow_big_lds(lce_recompute_kernel, kLdsBytes + kCacheStageBytes)) != VAMD_OK) return s;
@@ -903,8 +949,10 @@ static int lce_forward_launch(const void* hidden, const void* weight, const int6
       else
         hipLaunchKernelGGL((lce_forward_kernel<true, false>), grid, block, kLdsBytes + kCacheStageBytes, s, a);
     } else {
-      if (sum_pi_squared) hipLaunchKernelGGL((lce_forward_kernel<false, true>), grid, block, kLdsBytes, s, a);
-      else hipLaunchKernelGGL((lce_forward_kernel<false, false>), grid, block, kLdsBytes, s, a);
+      if (sum_pi_squared)
+        hipLaunchKernelGGL((lce_forward_kernel<false, true>), grid, block, kLdsBytes + kFwdTokenLds, s, a);
+      else
+        hipLaunchKernelGGL((lce_forward_kernel<false, false>), grid, block, kLdsBytes + kFwdTokenLds, s, a);
     }
   }
   VAMD_LAUNCH_CHECK();
