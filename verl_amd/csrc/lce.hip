@@ -26,6 +26,11 @@ namespace vamd {
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 constexpr float kNegBig = -1.0e30f;  // stands in for -inf so that (x - x) and 0 * x stay finite
+// What a column past the end of the vocabulary holds in place of its product.  Times any sensible
+// log2(e) / temperature it stays below kNegBig, the running maximum's start value (or overflows to -inf, which the
+// maximum ignores as well): the maximum is never taken from it, so its exponent is hugely negative against every
+// maximum there can be and it contributes exactly 0 to the sums (0 times a finite number).
+constexpr float kNoColumn = -3.0e38f;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -73,7 +78,7 @@ struct FwdArgs {
   int tok_tiles, voc_tiles, splits;
   float scale2;      // log2(e) / temperature
   float rcp_t;       // 1 / temperature
-  float4* partials;  // [splits][tok_tiles * 256] : (max2, sum, sum_y, label logit)
+  float4* partials;  // [splits][tok_tiles * 256] : (max in the log2 domain, sum e, sum e x with x = hidden . weight, label logit)
   float* z_cache;    // optional [n_tokens][vocab] fp32 logits / temperature, kept for the backward
   float* pi2_partials;  // optional [splits][tok_tiles * 256] : sum of e^2 relative to the same max
 };
@@ -183,26 +188,22 @@ struct FwdEpi {
     }
 #pragma unroll
     for (int nb = 0; nb < kNB; ++nb) {
-      float ymax = kNegBig;
-      // pass 1: scale into the log2 domain in place, mask the vocabulary tail (last tile only), tile max
+      // pass 1: tile maximum of the raw products (the vocabulary tail of the last tile replaced in place)
+      float xmax = kNegBig;
       if (ragged) {
 #pragma unroll
         for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
-            const float y = (c0 + acc_col(p, mb, v) < vocab) ? acc.a[mb][nb][v] * scale2 : kNegBig;
-            acc.a[mb][nb][v] = y;
-            ymax = fmaxf(ymax, y);
+            const float x = (c0 + acc_col(p, mb, v) < vocab) ? acc.a[mb][nb][v] : kNoColumn;
+            acc.a[mb][nb][v] = x;
+            xmax = fmaxf(xmax, x);
           }
       } else {
 #pragma unroll
         for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
-          for (int v = 0; v < 4; ++v) {
-            const float y = acc.a[mb][nb][v] * scale2;
-            acc.a[mb][nb][v] = y;
-            ymax = fmaxf(ymax, y);
-          }
+          for (int v = 0; v < 4; ++v) xmax = fmaxf(xmax, acc.a[mb][nb][v]);
       }
       // label logit: only when some lane's label falls in this wavefront's 128 columns
       typedef int __attribute__((address_space(3))) * lds_i32_t;
@@ -218,7 +219,7 @@ struct FwdEpi {
 #pragma unroll
           for (int v = 0; v < 4; ++v) {
             const int col = mb * kBlk + 4 * p.lq + v;
-            add += (col == rel) ? acc.a[mb][nb][v] * kLn2 : 0.f;
+            add += (col == rel) ? acc.a[mb][nb][v] * rcp_t : 0.f;
           }
         if constexpr (CACHE) {
           zl[nb] += add;
@@ -227,17 +228,19 @@ struct FwdEpi {
           *slot += add;
         }
       }
-      const float m_new = fmaxf(m[nb], ymax);
+      // pass 2: the running state in the log2 domain, three operations and an exponential per element:
+      // e = 2^(x scale2 - m), s += e, sy += e x (the raw product: the 1 / temperature goes on at the very end)
+      const float m_new = fmaxf(m[nb], xmax * scale2);
       const float resc = fast_exp2(m[nb] - m_new);
       float s_ = s[nb] * resc, sy_ = sy[nb] * resc, s2_ = PI2 ? s2[nb] * resc * resc : 0.f;
 #pragma unroll
       for (int mb = 0; mb < kMB; ++mb)
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
-          const float y = acc.a[mb][nb][v];
-          const float e = fast_exp2(y - m_new);
+          const float x = acc.a[mb][nb][v];
+          const float e = fast_exp2(fmaf(x, scale2, -m_new));
           s_ += e;
-          sy_ = fmaf(e, y, sy_);
+          sy_ = fmaf(e, x, sy_);
           if (PI2) s2_ = fmaf(e, e, s2_);
         }
       m[nb] = m_new;
@@ -381,6 +384,7 @@ struct MergeArgs {
   const float4* partials;
   const float* pi2_partials;  // null unless sum_pi_squared is wanted
   int splits, stride, n_tokens;
+  float rcp_t;  // the partial sums of e * (hidden . weight) carry no 1 / temperature yet
   float* logprobs;
   float* entropy;
   float* lse;
@@ -400,7 +404,7 @@ __global__ __launch_bounds__(256) void lce_merge_kernel(MergeArgs a) {
   }
   if (a.pi2_partials) a.sum_pi_squared[tok] = q / (s * s);
   const float lse = (m + log2f(s)) * kLn2;
-  const float mz = (sy / s) * kLn2;
+  const float mz = (sy / s) * a.rcp_t;
   a.lse[tok] = lse;
   a.mean_z[tok] = mz;
   a.entropy[tok] = lse - mz;
@@ -533,7 +537,7 @@ struct RecomputeEpi {
   //   lim[rb] : columns of the wavefront's 128 that exist for row rb (0 for a padding row), minus 4 lq
   template <bool PLAIN>
   __device__ __forceinline__ void patch_rows(Accum& acc, int nb2, int r0, int c0, const float (&lse2)[2],
-                                             const float (&mz)[2], const float (&glp)[2], const float (&gent)[2],
+                                             const float (&u1)[2], const float (&u0)[2], const float (&glp)[2],
                                              const int (&code)[2], const int (&lim)[2]) {
     const RecomputeArgs& A = *a;
 #pragma unroll
@@ -548,7 +552,7 @@ struct RecomputeEpi {
             const int mb = 2 * mb2 + cb;
             const float x = acc.a[mb][2 * nb2 + rb][v];
             const float prob = fast_exp2(fmaf(x, A.scale2, -lse2[rb]));
-            const float u = fmaf(gent[rb], fmaf(x, A.rcp_t, -mz[rb]), glp[rb]);  // g_lp/T + g_ent/T * (z - mean_z)
+            const float u = fmaf(u1[rb], x, u0[rb]);  // g_lp/T + g_ent/T * (z - mean_z), z = x / T
             if constexpr (PLAIN) {
               d[cb][rb][v] = -prob * u;
             } else {
@@ -580,16 +584,18 @@ struct RecomputeEpi {
 #pragma unroll
     for (int nb2 = 0; nb2 < kNB2; ++nb2) {
       // the lane's two token rows of this 32-row patch
-      float lse2[2], mz[2], glp[2], gent[2];
+      // u = u1 x + u0 with u1 = g_ent / T^2 and u0 = g_lp / T - g_ent / T * mean_z: one multiply-add per element
+      float lse2[2], u1[2], u0[2], glp[2];
       int code[2], lim[2];
       bool hit = false;
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb) {
         const int t = acc_row(p, 2 * nb2 + rb);  // row inside the tile
         lse2[rb] = tokf[t] * kLog2e;
-        mz[rb] = tokf[kTile + t];
         glp[rb] = (A.g_lp ? tokf[2 * kTile + t] : 0.f) * A.rcp_t;
-        gent[rb] = (A.g_ent ? tokf[4 * kTile + t] : A.g_ent_scalar) * A.rcp_t;
+        const float gent = (A.g_ent ? tokf[4 * kTile + t] : A.g_ent_scalar) * A.rcp_t;
+        u1[rb] = gent * A.rcp_t;
+        u0[rb] = fmaf(-gent, tokf[kTile + t], glp[rb]);
         const int rel = toki[3 * kTile + t] - A.chunk_c0 - c0 - p.wc * 128;  // label's column among the wavefront's 128
         const bool here = rel >= 0 && rel < 128;
         hit = hit || here;
@@ -597,8 +603,8 @@ struct RecomputeEpi {
         code[rb] = (here && ((rel >> 2) & 3) == p.lq) ? 4 * (rel >> 4) + (rel & 3) : -1;
         lim[rb] = r0 + t < A.n_tokens ? cols_left : 0;
       }
-      if (inside && !__any(hit)) patch_rows<true>(acc, nb2, r0, c0, lse2, mz, glp, gent, code, lim);
-      else patch_rows<false>(acc, nb2, r0, c0, lse2, mz, glp, gent, code, lim);
+      if (inside && !__any(hit)) patch_rows<true>(acc, nb2, r0, c0, lse2, u1, u0, glp, code, lim);
+      else patch_rows<false>(acc, nb2, r0, c0, lse2, u1, u0, glp, code, lim);
     }
   }
 };
@@ -638,9 +644,9 @@ __global__ __launch_bounds__(256) void lce_dlogits_kernel(DLogitsArgs a) {
   const int col = a.chunk_c0 + j;
   if (tok < a.n_tokens && col < a.vocab) {  // vocab % 8 == 0: the 8 columns are all in or all out
     const float lse2 = a.lse[tok] * kLog2e;
-    const float mz = a.mean_z[tok];
     const float glp = (a.g_lp ? a.g_lp[tok] : 0.f) * a.rcp_t;
     const float gent = (a.g_ent ? a.g_ent[tok] : a.g_ent_scalar) * a.rcp_t;
+    const float u0 = fmaf(-gent, a.mean_z[tok], glp);  // as in the recompute epilogue, with z in place of x / T
     const int rel = (int)a.labels[tok] - col;
     const f32x4* src = reinterpret_cast<const f32x4*>(a.z_cache + (int64_t)tok * a.vocab + col);
     const f32x4 z0 = __builtin_nontemporal_load(src), z1 = __builtin_nontemporal_load(src + 1);
@@ -649,8 +655,8 @@ __global__ __launch_bounds__(256) void lce_dlogits_kernel(DLogitsArgs a) {
     for (int e = 0; e < 8; ++e) {
       const float z = e < 4 ? z0[e] : z1[e - 4];
       const float prob = fast_exp2(fmaf(z, kLog2e, -lse2));
-      const float u = fmaf(gent, z - mz, glp);
-      d[e] = -prob * u + ((e == rel) ? glp : 0.f);
+      const float u = fmaf(gent, z, u0);
+      d[e] = fmaf(-prob, u, (e == rel) ? glp : 0.f);
     }
     const u32x2 lo = pack_bf16x4(d[0], d[1], d[2], d[3]), hi = pack_bf16x4(d[4], d[5], d[6], d[7]);
     out = u32x4{lo[0], lo[1], hi[0], hi[1]};
@@ -964,6 +970,7 @@ static int lce_forward_launch(const void* hidden, const void* weight, const int6
   m.splits = a.splits;
   m.stride = a.tok_tiles * kTile;
   m.n_tokens = (int)n_tokens;
+  m.rcp_t = rcp_temperature;
   m.logprobs = logprobs;
   m.entropy = entropy;
   m.lse = lse;
