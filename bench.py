@@ -26,14 +26,23 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 KERNEL_NAMES = ["lce_forward_kernel", "lce_merge_kernel", "lce_recompute_kernel", "lce_dgrad_kernel", "lce_dlogits_kernel"]
 # MFMA GEMMs of 2*N*V*H flops each that a kernel performs per step
 COPY_YARDSTICK_BYTES = 1 << 30
-# L2 <-> fabric bytes of one full-chunk launch (16384 vocabulary columns) of each kernel at this workload:
-# rocprofv3 FETCH_SIZE + WRITE_SIZE, scaled by the readings of the 1 GiB copy in the same run
-# (2048 and 1024 bytes per unit); see profiles/head_fwd_bwd_qwen7b_hbm_traffic.md.  Counters cannot be read
-# from inside this process, so the figure is recorded here and only reported for the shape it was measured on.
-MEASURED_TRAFFIC_BYTES = {"lce_dgrad_kernel": 6.68e9 + 0.353e9,       # per full chunk, either backward mode
-                          "lce_forward_kernel": 39.2e9 + 0.007e9,    # without the logits cache (the default)
-                          "lce_forward_kernel_with_cache": 46.3e9 + 9.98e9,
-                          "lce_recompute_kernel": 2.83e9 + 0.612e9, "lce_dlogits_kernel": 1.125e9 + 0.537e9}
+# L2 <-> fabric bytes of one full-chunk launch (16384 vocabulary columns) of each kernel at this workload come from
+# counter passes (rocprofv3 FETCH_SIZE and WRITE_SIZE, scaled by the readings of the 1 GiB copy in the same run).
+# Counters cannot be read from inside this process, so the pass that writes profiles/head_fwd_bwd_qwen7b_hbm_traffic.md
+# also writes the figures, with the commit they were taken at, to this file; the bench line quotes both.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "head_traffic.json")
+
+
+def measured_traffic(kernel: str):
+    """(bytes per full-chunk launch, commit of the measurement) of `kernel`, or (None, None) without a counter pass."""
+    try:
+        rec = json.load(open(TRAFFIC_FILE))
+        fetch, write = rec["bytes_per_launch"][kernel]
+        return float(fetch) + float(write), rec.get("commit")
+    except (OSError, KeyError, ValueError, TypeError):
+        return None, None
+
+
 GEMMS_PER_STEP = {"lce_forward_kernel": 1, "lce_recompute_kernel": 1, "lce_dgrad_kernel": 2}
 
 
@@ -504,6 +513,34 @@ def mfma_ceiling_probe(dev, n: int, h: int, v: int, seconds: float = 1.5) -> dic
             res[kind][name] = run_for(
                 lambda: _cabi.check(L.vamd_mfma_yardstick(shape, seed.data_ptr(), sink.data_ptr(), wgs, iters, st)), flops)
         del seed, sink
+    # The other two head shapes of the configuration list, forward kernel and vendor NT GEMM over the whole
+    # vocabulary, zeros against random operands: whether the clock (power) or the pipeline (stalls) holds them back.
+    for name, (n2, h2, v2) in (("qwen0.5b_head_2048x896x151936", (2048, 896, 151936)),
+                               ("llama8b_chunk_8192x4096x128256", (8192, 4096, 128256))):
+        lab2 = torch.randint(0, v2, (n2,), device=dev, generator=g)
+        outs2 = [torch.empty(n2, device=dev) for _ in range(4)]
+        ws2 = torch.empty(L.vamd_lce_forward_workspace_bytes(n2, h2, v2), dtype=torch.uint8, device=dev)
+        z2 = torch.empty(n2, v2, device=dev, dtype=torch.bfloat16)
+        res[name] = {}
+        for kind in ("zeros", "random"):
+            if kind == "zeros":
+                hid = torch.zeros(n2, h2, device=dev, dtype=torch.bfloat16)
+                w = torch.zeros(v2, h2, device=dev, dtype=torch.bfloat16)
+            else:
+                hid = torch.randn(n2, h2, device=dev, generator=g).bfloat16()
+                w = (torch.randn(v2, h2, device=dev, generator=g) * 0.02).bfloat16()
+
+            def fwd2():
+                _cabi.check(L.vamd_lce_forward(hid.data_ptr(), w.data_ptr(), lab2.data_ptr(), n2, h2, v2, 1.0,
+                                               *(o.data_ptr() for o in outs2), None, None, ws2.data_ptr(), ws2.numel(),
+                                               st))
+
+            res[name][kind] = {
+                "lce_forward_kernel": run_for(fwd2, 2.0 * n2 * v2 * h2),
+                "vendor_gemm_NT_logits": run_for(lambda: torch.matmul(hid, w.t(), out=z2), 2.0 * n2 * v2 * h2),
+            }
+            del hid, w
+        del lab2, outs2, ws2, z2
     stop.set()
     res["board_power_cap_W"] = _read_power_w()[1]
     res["note"] = ("ms per call; PFLOP/s on 2*M*N*K; sclk and board power from the driver's sysfs files over the second "
@@ -753,7 +790,8 @@ def main() -> None:
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_BF16_TFLOPS,
-        "traffic": MEASURED_TRAFFIC_BYTES.get(dom),
+        "traffic": measured_traffic(dom)[0],
+        "traffic_measured_at_commit": measured_traffic(dom)[1],
         "flops_per_launch": flops_per_launch,
         "avg_launch_ms": d["avg_ms"],
         **fractions(ms_per_step, default_cached),
