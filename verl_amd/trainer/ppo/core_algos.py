@@ -9,6 +9,8 @@ they are staged to the current GPU and results come back on the input's device.
 """
 from __future__ import annotations
 
+import collections
+
 from enum import Enum
 import warnings
 from typing import Any, Callable, Optional
@@ -194,16 +196,41 @@ def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torc
         return adv.view(token_level_rewards.shape).to(out_dev), ret.view(token_level_rewards.shape).to(out_dev)
 
 
+_GROUP_ID_CACHE: "collections.OrderedDict" = collections.OrderedDict()
+_GROUP_ID_CACHE_SIZE = 8
+
+
+def _group_ids_on_device(index, vectorized: bool, dev: torch.device):
+    """``contiguous_group_ids(index)`` as a device tensor, and the number of groups.  The trainer hands the same
+    ``uid`` array to every estimator call of a step, and factorising the labels plus copying 4 KB to the device
+    costs more than the advantage kernel itself, so the last few results are kept, keyed by the labels' content
+    (numpy arrays: dtype, shape and raw bytes -- for object arrays the bytes are the addresses of the label
+    objects, which the kept array keeps alive).  Anything else is factorised afresh."""
+    key = None
+    if isinstance(index, np.ndarray):
+        key = (index.dtype.str, index.shape, hash(index.tobytes()), bool(vectorized), dev)
+        hit = _GROUP_ID_CACHE.get(key)
+        if hit is not None:
+            _GROUP_ID_CACHE.move_to_end(key)
+            return hit[0], hit[1]
+    ids, G = contiguous_group_ids(index, vectorized=vectorized)
+    ids = ids.to(dev)
+    if key is not None:
+        _GROUP_ID_CACHE[key] = (ids, G, index)
+        while len(_GROUP_ID_CACHE) > _GROUP_ID_CACHE_SIZE:
+            _GROUP_ID_CACHE.popitem(last=False)
+    return ids, G
+
+
 def _grpo(token_level_rewards, response_mask, index, epsilon, norm_adv_by_std_in_grpo, std_mode):
     with torch.no_grad():
         dev = _cabi.compute_device(token_level_rewards, response_mask)
         r = _matrix(token_level_rewards, dev)
         m, code = _mask_matrix(response_mask, dev, r.shape)
         B, Lc = r.shape
-        ids, G = contiguous_group_ids(index, vectorized=std_mode == 1)
+        ids, G = _group_ids_on_device(index, std_mode == 1, dev)
         if ids.numel() != B:
             raise ValueError(f"index has {ids.numel()} entries for a batch of {B}")
-        ids = ids.to(dev)
         adv = torch.empty_like(r)
         Lb = _cabi.lib()
         ws = _cabi.ticket_workspace(Lb.vamd_grpo_workspace_bytes(B, Lc, G), dev)
@@ -546,8 +573,9 @@ class _PolicyLoss(torch.autograd.Function):
         rows, cols = lp.shape
         need_grad = ctx.needs_input_grad[0]
         Lb = _cabi.lib()
-        out = torch.empty(4, dtype=torch.float32, device=dev)
-        coef = torch.empty(rows, dtype=torch.float32, device=dev)
+        # one allocation for the four result floats and the per-row coefficients (16-byte aligned both)
+        buf = torch.empty(4 + rows, dtype=torch.float32, device=dev)
+        out, coef = buf[:4], buf[4:]
         g = torch.empty_like(lp) if need_grad else None
         ws = _cabi.ticket_workspace(Lb.vamd_policy_loss_variant_workspace_bytes(rows, cols), dev)
         with _cabi.device_guard(dev):
@@ -563,7 +591,7 @@ class _PolicyLoss(torch.autograd.Function):
         ctx.in_dtype = log_prob.dtype
         out = out.to(log_prob.device)
         ctx.mark_non_differentiable(out)
-        return out[0].clone(), out
+        return out[0], out   # a view: the loss and the metrics share the floats the kernel wrote
 
     @staticmethod
     def backward(ctx, d_loss, _d_out):
@@ -916,8 +944,8 @@ class _ValueLoss(torch.autograd.Function):
         rows, cols = vp.shape
         need_grad = ctx.needs_input_grad[0]
         Lb = _cabi.lib()
-        out = torch.empty(2, dtype=torch.float32, device=dev)
-        coef = torch.empty(rows, dtype=torch.float32, device=dev)
+        buf = torch.empty(4 + rows, dtype=torch.float32, device=dev)   # results and per-row coefficients, one allocation
+        out, coef = buf[:2], buf[4:]
         g = torch.empty_like(vp) if need_grad else None
         ws = _cabi.ticket_workspace(Lb.vamd_value_loss_workspace_bytes(rows, cols), dev)
         with _cabi.device_guard(dev):
@@ -932,7 +960,7 @@ class _ValueLoss(torch.autograd.Function):
         ctx.in_dtype = vpreds.dtype
         out = out.to(vpreds.device)
         ctx.mark_non_differentiable(out)
-        return out[0].clone(), out
+        return out[0], out   # a view: the loss and the metrics share the floats the kernel wrote
 
     @staticmethod
     def backward(ctx, d_loss, _d_out):
