@@ -233,6 +233,29 @@ def test_gae_bounded_wait_leaves_every_advantage_raw_or_whitened(dev, monkeypatc
         assert mom[4].item() != 0.0
 
 
+def test_grpo_group_ids_follow_the_labels_when_the_array_is_reused(dev):
+    """The host mirror keeps the last few factorised label arrays on the device; the key is the labels' content, so
+    an array that the caller rewrites in place, or another array with the same labels, gives the right groups."""
+    from verl_amd.trainer.ppo.core_algos import compute_grpo_outcome_advantage
+    g = torch.Generator().manual_seed(12)
+    B, L = 64, 300
+    rewards = torch.randn(B, L, generator=g)
+    mask = (torch.rand(B, L, generator=g) < 0.8).float()
+    index = np.repeat(np.arange(B // 8), 8)
+    first, _ = compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    again, _ = compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index.copy())
+    assert torch.equal(first, again)
+    assert torch.allclose(first.cpu(), O.grpo_outcome_advantage(rewards.clone(), mask, index)[0], rtol=1e-5, atol=1e-6)
+    index[:] = np.repeat(np.arange(B // 4), 4)          # same object, new grouping
+    other, _ = compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    assert torch.allclose(other.cpu(), O.grpo_outcome_advantage(rewards.clone(), mask, index)[0], rtol=1e-5, atol=1e-6)
+    assert not torch.equal(other, first)
+    uid = np.array([f"prompt-{i // 8}" for i in range(B)], dtype=object)   # object labels: keyed by the objects
+    a, _ = compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), uid)
+    b, _ = compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), uid)
+    assert torch.equal(a, b) and torch.equal(a, first)
+
+
 @pytest.mark.parametrize("B,L", [(512, 4096), (3000, 300), (2400, 4500), (64, 40000)])
 def test_grpo_single_launch_bounded_wait_runs_out_without_hanging(dev, monkeypatch, B, L):
     """The one-launch GRPO estimator with its poll limit forced to zero, on both ways of waiting (one meeting of the
