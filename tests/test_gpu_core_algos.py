@@ -171,12 +171,23 @@ def test_gae_bounded_wait_runs_out_without_hanging(dev, monkeypatch):
     want_adv, want_ret = O.gae_advantage_return(r.cpu().double(), v.cpu().double(), m.cpu().double(), 1.0, 0.95)
     monkeypatch.setenv("VAMD_GATE_SPIN_LIMIT", "0")
     CA._WARNED.clear()
-    with pytest.warns(RuntimeWarning, match="timed out"):
-        adv, ret = CA.compute_gae_advantage_return(r, v, m, 1.0, 0.95)
-    torch.cuda.synchronize()
-    assert (adv.cpu().double() - want_adv).abs().max().item() <= 2e-5 * want_adv.abs().max().item()
-    ws = _cabi.ticket_workspace(4096, dev)
-    assert _counter_area_is_clear(ws)
+    CA._GAE_WAIT_TIMED_OUT.clear()
+    try:
+        with pytest.warns(RuntimeWarning, match="timed out"):
+            adv, ret = CA.compute_gae_advantage_return(r, v, m, 1.0, 0.95)
+        torch.cuda.synchronize()
+        assert (adv.cpu().double() - want_adv).abs().max().item() <= 2e-5 * want_adv.abs().max().item()
+        ws = _cabi.ticket_workspace(4096, dev)
+        assert _counter_area_is_clear(ws)
+        # the time-out is remembered: the next call takes the two-launch form at once (no second warning, no polling)
+        assert CA._GAE_WAIT_TIMED_OUT
+        import warnings
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")
+            adv, ret = CA.compute_gae_advantage_return(r, v, m, 1.0, 0.95)
+        assert (adv.cpu().double() - want_adv).abs().max().item() <= 2e-5 * want_adv.abs().max().item()
+    finally:
+        CA._GAE_WAIT_TIMED_OUT.clear()
     monkeypatch.delenv("VAMD_GATE_SPIN_LIMIT")
     adv, ret = CA.compute_gae_advantage_return(r, v, m, 1.0, 0.95)
     assert (adv.cpu().double() - want_adv).abs().max().item() <= 2e-5 * want_adv.abs().max().item()
@@ -1221,7 +1232,12 @@ def test_benchmark_config_gae_value_policy_loss(dev):
     values = torch.randn(B, L, generator=g)
     adv, ret = CA.compute_gae_advantage_return(rewards.to(dev), values.to(dev), mask.to(dev), 1.0, 0.95)
     want_adv, want_ret = O.gae_advantage_return(rewards, values, mask, 1.0, 0.95)
-    _close(ret, want_ret, atol=1e-5, what="returns"); _close(adv, want_adv, atol=1e-5, what="advantages")
+    # rtol 1e-5, and for entries near zero a floor stated in units of the data: the scan adds the same fp32 terms in
+    # another order than the sequential recurrence, so two results differ by a few units in the last place of the
+    # LARGEST partial sum they went through, not of their own (possibly cancelled) value: 8 ulp of max |value|
+    ulp8 = lambda t: 8 * torch.finfo(torch.float32).eps * t.abs().max().item()
+    _close(ret, want_ret, atol=ulp8(want_ret), what="returns")
+    _close(adv, want_adv, atol=ulp8(want_adv), what="advantages")
     vpreds = values + torch.randn(B, L, generator=g) * 0.5
     vd = vpreds.to(dev).requires_grad_(); vo = vpreds.clone().requires_grad_()
     vloss, vfrac = CA.compute_value_loss(vd, ret, values.to(dev), mask.to(dev), 0.5)

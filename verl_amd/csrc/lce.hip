@@ -836,9 +836,12 @@ static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // channels instead of landing on a power-of-two stride.
 static inline int64_t dz_pitch(int64_t cv) { return cv + 128; }
 
-static int fwd_splits(int64_t tok_tiles, int64_t voc_tiles) {
+// max_rows: most partial-state rows (splits x padded tokens) the caller's buffer holds; the built-in buffer of the
+// entry point that allocates nothing is sized for 256 CUs and must serve a part with more of them too.
+static int fwd_splits(int64_t tok_tiles, int64_t voc_tiles, int64_t max_rows = INT64_MAX) {
   const int cus = device_cu_count();
   int64_t sp = cus / tok_tiles;  // as many workgroups as fit in one round over the CUs
+  if (sp > max_rows / (tok_tiles * kTile)) sp = max_rows / (tok_tiles * kTile);
   if (sp < 1) sp = 1;
   if (sp > voc_tiles) sp = voc_tiles;
   return (int)sp;
@@ -925,7 +928,7 @@ extern "C" size_t vamd_lce_forward_workspace_bytes(int64_t n_tokens, int64_t hid
 static int lce_forward_launch(const void* hidden, const void* weight, const int64_t* labels, int64_t n_tokens,
                               int64_t hidden_size, int64_t vocab, float rcp_temperature, float* logprobs,
                               float* entropy, float* lse, float* mean_z, float* logits_cache, float* sum_pi_squared,
-                              void* workspace, void* stream) {
+                              void* workspace, void* stream, int64_t max_rows = INT64_MAX) {
 
   FwdArgs a;
   a.hidden = Operand{static_cast<const uint16_t*>(hidden), hidden_size, (int)n_tokens, (int)hidden_size};
@@ -936,7 +939,7 @@ static int lce_forward_launch(const void* hidden, const void* weight, const int6
   a.k_slabs = (int)(hidden_size / kBK);
   a.tok_tiles = (int)ceil_div(n_tokens, kTile);
   a.voc_tiles = (int)ceil_div(vocab, kTile);
-  a.splits = fwd_splits(a.tok_tiles, a.voc_tiles);
+  a.splits = fwd_splits(a.tok_tiles, a.voc_tiles, max_rows);
   a.scale2 = rcp_temperature * kLog2e;
   a.rcp_t = rcp_temperature;
   a.partials = static_cast<float4*>(workspace);
@@ -1045,18 +1048,18 @@ extern "C" int vamd_lce_forward_static(const void* hidden, const void* weight, c
   int st = check_forward_args(hidden, weight, labels, n_tokens, hidden_size, vocab, rcp_temperature, logprobs, entropy,
                               lse, mean_z, nullptr);
   if (st != VAMD_OK) return st;
-  const size_t need = vamd_lce_forward_workspace_bytes(n_tokens, hidden_size, vocab);
-  VAMD_REQUIRE(n_tokens <= VAMD_LCE_STATIC_MAX_TOKENS && need <= kStaticScratchBytes,
-               "lce_forward_static: %lld tokens need %zu bytes of scratch; the built-in buffer serves at most %d "
-               "tokens (%zu bytes): use vamd_lce_forward with a caller workspace",
-               (long long)n_tokens, need, (int)VAMD_LCE_STATIC_MAX_TOKENS, kStaticScratchBytes);
+  VAMD_REQUIRE(n_tokens <= VAMD_LCE_STATIC_MAX_TOKENS,
+               "lce_forward_static: %lld tokens; the built-in buffer serves at most %d tokens per call: use "
+               "vamd_lce_forward with a caller workspace",
+               (long long)n_tokens, (int)VAMD_LCE_STATIC_MAX_TOKENS);
   if ((st = ensure_lds_attributes()) != VAMD_OK) return st;
   void* ws = nullptr;
   if ((st = static_scratch_pointer(&ws)) != VAMD_OK) return st;
   // Every partial the merge kernel reads is written by the forward kernel of the same call, so
   // nothing in the buffer has to start at zero and a previous call's contents do not matter.
+  // the vocabulary splits are capped so that splits x padded tokens fits the buffer whatever the CU count
   return lce_forward_launch(hidden, weight, labels, n_tokens, hidden_size, vocab, rcp_temperature, logprobs, entropy,
-                            lse, mean_z, nullptr, sum_pi_squared, ws, stream);
+                            lse, mean_z, nullptr, sum_pi_squared, ws, stream, VAMD_LCE_STATIC_MAX_TOKENS);
 }
 
 extern "C" size_t vamd_lce_backward_workspace_bytes(int64_t n_tokens, int64_t hidden_size, int64_t vocab,
