@@ -85,23 +85,6 @@ extern "C" {
 int vamd_abi_version(void);
 const char* vamd_last_error(void);
 
-/* Measurement aid (no counterpart in the reference): a plain 16-byte-per-lane copy of `bytes`
- * (a multiple of 16, both pointers 16-byte aligned) from src to dst.  Profilers read its memory
- * counters next to those of the other kernels to turn counter units into bytes. */
-int vamd_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream);
-/* out[i] = a[i] + b[i] + c[i] + d[i] over n floats (n % 4 == 0, 16-byte aligned pointers): a second yardstick,
- * the memory traffic of a fused loss kernel with its gradient and nothing else.  No counterpart in the reference. */
-int vamd_sum4(const float* a, const float* b, const float* c, const float* d, float* out, int64_t n, void* stream);
-/* Benchmark aid (no counterpart in the reference): a loop of independent bf16 matrix instructions on register
- * operands, no memory traffic, `workgroups` workgroups of 8 wavefronts, `iters` rounds of 8 (32x32x16) or 32
- * (16x16x32) instructions per wavefront.  seed: workgroups * 512 * 32 device words the operand fragments are taken
- * from (zeros: nothing toggles; random bf16: the data the board's power management sees in a real GEMM);
- * out: workgroups * 512 floats.  vamd_mfma_yardstick_flops gives the flops of one launch. */
-#define VAMD_MFMA_32X32X16 0
-#define VAMD_MFMA_16X16X32 1
-int64_t vamd_mfma_yardstick_flops(int shape, int workgroups, int iters);
-int vamd_mfma_yardstick(int shape, const void* seed, float* out, int workgroups, int iters, void* stream);
-
 /* ------------------------------------------------------------------------------------------
  * Fused vocab-projection log-prob / entropy head.
  * Replaces kernels.efficient_entropy_forward / efficient_entropy_backward behind
@@ -185,15 +168,6 @@ int vamd_lce_backward(const void* hidden, const void* weight, const int64_t* lab
                       const float* logits_cache, void* d_hidden, void* d_weight, int d_weight_mode,
                       float* d_weight_acc32, int64_t vocab_chunk, void* workspace, size_t workspace_bytes,
                       void* stream);
-
-/* Benchmark aid (no counterpart in the reference): with timing enabled, every head kernel
- * launch of the process is bracketed by HIP events on its stream.  vamd_lce_timing_collect
- * waits for them and adds up milliseconds and launch counts per kernel, indexed
- * 0 forward, 1 merge, 2 d_logits panel from recomputed logits (the recompute GEMM), 3 gradient GEMMs
- * (d_hidden + d_weight), 4 d_logits panel from cached logits (arrays of VAMD_LCE_TIMING_KERNELS). */
-#define VAMD_LCE_TIMING_KERNELS 5
-int vamd_lce_timing_enable(int on);
-int vamd_lce_timing_collect(double* ms_by_kernel_host, int64_t* launches_by_kernel_host);
 
 /* ------------------------------------------------------------------------------------------
  * Per-token log-prob / entropy from materialised logits: the unfused definitions the actor uses when the
@@ -558,6 +532,38 @@ int vamd_kl_loss_forward(const float* logprob, const float* ref_logprob, const v
                          double batch_num_tokens, double global_batch_size, double loss_scale_factor, float* out,
                          float* grad_unscaled, float* coef_out, void* workspace, size_t workspace_bytes,
                          void* stream);
+
+/* ==========================================================================================
+ * MEASUREMENT AIDS.  Nothing below is part of the drop-in: none of these entry points has a counterpart in the
+ * reference and no caller of the policy math needs them.  They exist so that bench.py and the profiler passes
+ * can time kernels on their launch stream, turn counter units into bytes and read the board's matrix-pipe
+ * ceiling with the library's own code.
+ * ========================================================================================== */
+/* Measurement aid (no counterpart in the reference): a plain 16-byte-per-lane copy of `bytes`
+ * (a multiple of 16, both pointers 16-byte aligned) from src to dst.  Profilers read its memory
+ * counters next to those of the other kernels to turn counter units into bytes. */
+int vamd_copy_bytes(const void* src, void* dst, int64_t bytes, void* stream);
+/* out[i] = a[i] + b[i] + c[i] + d[i] over n floats (n % 4 == 0, 16-byte aligned pointers): a second yardstick,
+ * the memory traffic of a fused loss kernel with its gradient and nothing else.  No counterpart in the reference. */
+int vamd_sum4(const float* a, const float* b, const float* c, const float* d, float* out, int64_t n, void* stream);
+/* Benchmark aid (no counterpart in the reference): a loop of independent bf16 matrix instructions on register
+ * operands, no memory traffic, `workgroups` workgroups of 8 wavefronts, `iters` rounds of 8 (32x32x16) or 32
+ * (16x16x32) instructions per wavefront.  seed: workgroups * 512 * 32 device words the operand fragments are taken
+ * from (zeros: nothing toggles; random bf16: the data the board's power management sees in a real GEMM);
+ * out: workgroups * 512 floats.  vamd_mfma_yardstick_flops gives the flops of one launch. */
+#define VAMD_MFMA_32X32X16 0
+#define VAMD_MFMA_16X16X32 1
+int64_t vamd_mfma_yardstick_flops(int shape, int workgroups, int iters);
+int vamd_mfma_yardstick(int shape, const void* seed, float* out, int workgroups, int iters, void* stream);
+
+/* Benchmark aid (no counterpart in the reference): with timing enabled, every head kernel
+ * launch of the process is bracketed by HIP events on its stream.  vamd_lce_timing_collect
+ * waits for them and adds up milliseconds and launch counts per kernel, indexed
+ * 0 forward, 1 merge, 2 d_logits panel from recomputed logits (the recompute GEMM), 3 gradient GEMMs
+ * (d_hidden + d_weight), 4 d_logits panel from cached logits (arrays of VAMD_LCE_TIMING_KERNELS). */
+#define VAMD_LCE_TIMING_KERNELS 5
+int vamd_lce_timing_enable(int on);
+int vamd_lce_timing_collect(double* ms_by_kernel_host, int64_t* launches_by_kernel_host);
 
 #ifdef __cplusplus
 }
