@@ -815,6 +815,22 @@ def main() -> None:
     else:
         os.environ["VAMD_LCE_LOGITS_CACHE_GB"] = saved_env
 
+    # One-sided steps in the default mode: the backward runs only the gradient GEMM of the input that requires a
+    # gradient (a frozen head / LoRA on the trunk; or a head fine-tuned on detached hidden states).
+    def one_sided(wrt):
+        def run():
+            lp, ent = linear_cross_entropy(hidden, weight, labels, T)
+            return torch.autograd.grad((lp, ent), (wrt,), (g_lp, g_ent))
+        return run
+
+    for key, wrt, what in (("frozen_weight", hidden, "d_hidden only"), ("frozen_hidden", weight, "d_weight only")):
+        r = time_head_mode(one_sided(wrt), args.steps, args.warmup, n, dev)
+        hw_gemms = 2.0 if default_cached else 3.0     # forward + (recompute) + one gradient GEMM
+        modes[key] = {**r, "default": False, "gradients": what,
+                      "step_algorithmic_frac": 2.0 * gemm_flops / (r["ms_per_step"] * 1e-3) / peak,
+                      "step_hardware_frac": hw_gemms * gemm_flops / (r["ms_per_step"] * 1e-3) / peak,
+                      "kernels": head_kernel_times(L, one_sided(wrt), prof_steps)}
+
     line = {
         "metric": "tokens/s fwd+bwd logprob+entropy head @Qwen2.5-7B shape; MFMA util %",
         "value": tokens_per_s,

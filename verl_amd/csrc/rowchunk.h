@@ -128,12 +128,14 @@ __device__ __forceinline__ void for_each_group(int64_t row, int chunk, int64_t c
 struct ChunkPos {
   int64_t idx[kGroups];  // flat index of the group's first element
   int valid[kGroups];    // 0..4 elements of the group exist
-  __device__ __forceinline__ ChunkPos(int64_t row, int chunk, int64_t cols) {
+  // `thread`: position among the 256 threads that walk the chunk (a workgroup that holds several chunks of a row
+  // passes threadIdx.x % 256 and gives every 256 threads a chunk; a chunk past the end of the row has no valid group)
+  __device__ __forceinline__ ChunkPos(int64_t row, int chunk, int64_t cols, int thread = threadIdx.x) {
     const int64_t c_begin = (int64_t)chunk * kChunk;
     const int64_t c_end = (c_begin + kChunk) < cols ? (c_begin + kChunk) : cols;
 #pragma unroll
     for (int g = 0; g < kGroups; ++g) {
-      const int64_t c = c_begin + ((int64_t)g * kRcThreads + threadIdx.x) * 4;
+      const int64_t c = c_begin + ((int64_t)g * kRcThreads + thread) * 4;
       const int64_t left = c_end - c;
       valid[g] = left >= 4 ? 4 : (left > 0 ? (int)left : 0);
       idx[g] = row * cols + c;
@@ -603,8 +605,9 @@ inline AggParams make_agg_params(int mode, double dp, double bnt, double gbs, do
 
 // Called by ONE workgroup of NT threads (the last one of the launch to arrive, or a launch of its own).  partials: slot-major records (record_at) with slot 0 =
 // sum(loss * w) and slot 1 = sum(w); slots >= 2 are summed over everything into extra[].
-// Writes loss (double, thread 0) and coef[rows].
-template <int NV, int NT = kRcThreads, bool COHERENT = true>
+// Writes loss (double, thread 0) and coef[rows].  FLIGHT: chunk records of a row loaded together in the first pass
+// (registers for FLIGHT x 2 x NV doubles; 1 where a row has a single record).
+template <int NV, int NT = kRcThreads, bool COHERENT = true, int FLIGHT = 4>
 __device__ void finalize_agg(const double* __restrict__ partials, int64_t rows, int chunks, int64_t cols,
                              const AggParams& ap, float* __restrict__ coef, double& loss_out, double& msum_out,
                              double (&extra)[NV > 2 ? NV - 2 : 1], double* smem) {
@@ -619,7 +622,7 @@ __device__ void finalize_agg(const double* __restrict__ partials, int64_t rows, 
     const int64_t rr[2] = {r0, r0 + NT};
     const bool have[2] = {true, rr[1] < rows};
     double row[2][NV];
-    fold_row_records<NV, NV, 2, COHERENT>(partials, rr, have, rows, chunks, row);
+    fold_row_records<NV, NV, 2, COHERENT, FLIGHT>(partials, rr, have, rows, chunks, row);
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
       if (!have[k]) break;
