@@ -312,7 +312,38 @@ def policy_math_chain(dev, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> 
     return {"launches_per_chain": 4, "eager_us": timed(chain), "hip_graph_us": timed(graph.replay)}
 
 
-def policy_math_python_path(dev, B: int = 512, Lc: int = 4096, n_groups: int = 64) -> dict:
+def _host_profiles(ops: dict, calls: int = 1000, top: int = 14) -> dict:
+    """cProfile over `calls` calls of each op: where the host time of a call goes, microseconds per call, the `top`
+    entries by own time (a profiled call runs about 1.5 times slower than an unprofiled one)."""
+    import cProfile
+    import pstats
+
+    import torch
+
+    out = {}
+    for name, fn in ops.items():
+        for _ in range(500):   # long enough for the device to leave its idle clocks
+            fn()
+        torch.cuda.synchronize()
+        pr = cProfile.Profile()
+        t0 = time.perf_counter()
+        pr.enable()
+        for _ in range(calls):
+            fn()
+        torch.cuda.synchronize()
+        pr.disable()
+        wall = (time.perf_counter() - t0) / calls * 1e6
+        st = pstats.Stats(pr)
+        rows = []
+        for (fname, line, func), (cc, nc, tt, ct, _) in st.stats.items():
+            rows.append({"function": f"{os.path.basename(fname)}:{line}({func})", "calls_per_call": nc / calls,
+                         "own_us": tt / calls * 1e6, "cumulative_us": ct / calls * 1e6})
+        rows.sort(key=lambda r: -r["own_us"])
+        out[name] = {"wall_us_per_call_profiled": wall, "top": rows[:top]}
+    return out
+
+
+def policy_math_python_path(dev, B: int = 512, Lc: int = 4096, n_groups: int = 64, profile: bool = False) -> dict:
     """The same operations called the way the trainer calls them -- through the functions of
     ``verl_amd.trainer.ppo.core_algos`` / ``verl_amd.utils.torch_functional`` with torch tensors on the GPU --
     so that argument checks, output allocation, ctypes marshalling and the host synchronisations the interfaces
@@ -352,16 +383,26 @@ def policy_math_python_path(dev, B: int = 512, Lc: int = 4096, n_groups: int = 6
         loss, _ = CA.compute_value_loss(vpreds, returns, values, mask, 0.5, "token-mean")
         torch.autograd.grad(loss, vpreds)
 
+    def both_losses_one_backward():
+        # the way an update step meets them: both losses in one graph, one backward call for the sum
+        pl, _ = CA.compute_policy_loss_vanilla(old, new, adv, mask, "token-mean", Cfg)
+        vl, _ = CA.compute_value_loss(vpreds, returns, values, mask, 0.5, "token-mean")
+        torch.autograd.grad(pl + 0.5 * vl, (new, vpreds))
+
     ops = {
         "grpo_advantage": lambda: CA.compute_grpo_outcome_advantage(rewards, mask, index),
         "policy_loss_fwd": policy_fwd,
         "policy_loss_fwd_grad": policy_fwd_bwd,
         "gae_scan_whiten": lambda: CA.compute_gae_advantage_return(rewards, values, mask, 1.0, 0.95),
         "value_loss_fwd_grad": value_fwd_bwd,
+        "policy_and_value_loss_one_backward": both_losses_one_backward,
         "masked_mean": lambda: VF.masked_mean(values, mask),
         "masked_whiten": lambda: VF.masked_whiten(values, mask),
         "agg_loss_token_mean": lambda: CA.agg_loss(values, mask, "token-mean"),
     }
+    if profile:
+        return _host_profiles({k: ops[k] for k in ("policy_loss_fwd", "policy_loss_fwd_grad", "value_loss_fwd_grad",
+                                                   "policy_and_value_loss_one_backward")})
     res = {}
     for name, fn in ops.items():
         for _ in range(5):
@@ -712,6 +753,8 @@ def main() -> None:
                     help="only the matrix-pipe ceiling probe (zeros against random operands, vendor GEMMs beside "
                          "the forward kernel): what a counter pass for the shader clock runs")
     ap.add_argument("--ceiling-seconds", type=float, default=1.5, help="how long the probe keeps each kernel running")
+    ap.add_argument("--python-path-profile", action="store_true",
+                    help="only a cProfile table of the Python mirror's loss calls (host time per call)")
     ap.add_argument("--policy-math-only", action="store_true",
                     help="only the [B, L] kernels at B = 2048, L = 16384 after the 1 GiB copy: what a counter pass for "
                          "their memory traffic runs")
@@ -732,6 +775,9 @@ def main() -> None:
     n, h, v, T = 16384, 3584, 152064, 1.0
     if args.ceiling_only:
         print(json.dumps({"mfma_ceiling_probe": mfma_ceiling_probe(dev, n, h, v, seconds=args.ceiling_seconds)}))
+        return
+    if args.python_path_profile:
+        print(json.dumps({"python_path_host_profile_b512_l4096": policy_math_python_path(dev, profile=True)}))
         return
     if args.policy_math_only:
         a = torch.empty(1 << 30, dtype=torch.uint8, device=dev)   # the copy the counters are scaled by
