@@ -864,8 +864,11 @@ def main() -> None:
     # One-sided steps in the default mode: the backward runs only the gradient GEMM of the input that requires a
     # gradient (a frozen head / LoRA on the trunk; or a head fine-tuned on detached hidden states).
     def one_sided(wrt):
+        h = hidden if wrt is hidden else hidden.detach()   # the frozen input does not require a gradient
+        w = weight if wrt is weight else weight.detach()
+
         def run():
-            lp, ent = linear_cross_entropy(hidden, weight, labels, T)
+            lp, ent = linear_cross_entropy(h, w, labels, T)
             return torch.autograd.grad((lp, ent), (wrt,), (g_lp, g_ent))
         return run
 
