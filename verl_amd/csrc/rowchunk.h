@@ -28,14 +28,17 @@ inline int64_t chunks_of(int64_t cols) { return cols <= 0 ? 1 : (cols + kChunk -
 
 inline bool aligned_to(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
 
-// Streaming hint.  A launch of this many workgroups (4096 columns each: 128 MB per fp32 tensor) touches more than the
-// caches hold, so nothing it reads or writes will be found there again: its loads and stores are issued non-temporal,
-// which on this part is worth 7 - 9 % of HBM bandwidth (two-tensor read 6.3 -> 6.9 TB/s, four-in one-out
-// 5.5 -> 6.2 TB/s at 128 MB per tensor).  Smaller launches keep the default policy: their tensors (8 MB at the
-// benchmark size) are usually still cached from the kernel that produced them, and are read again by the next one.
+// Streaming hint.  A launch of this many workgroups (4096 columns each: 64 MB per fp32 tensor, and these kernels
+// touch three to six tensors) moves more than the 256 MB Infinity Cache holds, so nothing it reads or writes will be
+// found there again: its loads and stores are issued non-temporal, which on this part is worth 7 - 9 % of HBM
+// bandwidth at 128 MB per tensor (two-tensor read 6.3 -> 6.9 TB/s, four-in one-out 5.5 -> 6.2 TB/s) and 10 - 20 % at
+// 64 MB (2048 x 8192: policy loss with gradient 71.5 -> 64.6 us, GRPO 47.0 -> 38.9 us).  It measured faster still at
+// 32 MB per tensor on cold buffers, but there the working set fits the cache and a consumer may find it there, so
+// smaller launches keep the default policy: their tensors (8 MB at the benchmark size) are usually still cached from
+// the kernel that produced them, and are read again by the next one.
 // The test is uniform over the launch, so it costs one scalar branch per access.
 // Kernels whose grid is not one workgroup per 4096 columns pass the flag themselves (streams_past_caches(elements)).
-constexpr unsigned kStreamingGrid = 8192;
+constexpr unsigned kStreamingGrid = 4096;
 __device__ __forceinline__ bool launch_streams_past_caches() { return gridDim.x >= kStreamingGrid; }
 __device__ __forceinline__ bool streams_past_caches(int64_t elements) {
   return elements >= (int64_t)kStreamingGrid * 4096;

@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void sum4_kernel(const ys_f32x4* __restrict__ 
   }
 }
 
-constexpr int64_t kStreamingBytes = 128ll << 20;  // per tensor: the size from which the [B, L] kernels stream
+constexpr int64_t kStreamingBytes = 64ll << 20;  // per tensor: the size from which the [B, L] kernels stream
 
 }  // namespace vamd
 
