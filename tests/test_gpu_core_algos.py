@@ -964,6 +964,47 @@ def test_sequence_level_losses_on_every_way_to_the_row_sums(dev, monkeypatch, va
         _close(grad, want_grad, atol=1e-9, what=f"d {variant} loss / d log_prob")
 
 
+@pytest.mark.parametrize("variant", ["gspo", "geo_mean"])
+@pytest.mark.parametrize("mask_dtype", [torch.bool, torch.int64, torch.int32, torch.float32])
+@pytest.mark.parametrize("with_isw", [False, True])
+@pytest.mark.parametrize("with_grad", [False, True])
+def test_sequence_level_losses_with_one_workgroup_per_row(dev, monkeypatch, variant, mask_dtype, with_isw, with_grad):
+    """Rows of two to four 4096-column chunks whose workgroups may not wait for each other (here: waiting kernels
+    switched off) are held whole by one 1024-thread workgroup.  Every mask type, with and without importance weights,
+    with and without the gradient, a ragged last chunk and an empty row, against the oracle."""
+    from verl_amd import _cabi
+    from verl_amd.trainer.ppo import core_algos as CA
+    monkeypatch.setenv("VAMD_WAITING_KERNELS", "0")
+    B, Lc = 33, 8200
+    g = torch.Generator().manual_seed(B * 7 + Lc + int(with_isw))
+    mask, _ = _prefix_mask(B, Lc, g, lo=3)
+    mask[1] = 0
+    mask[5] = 1                                                 # a row that uses all three chunks
+    old = torch.randn(B, Lc, generator=g) * 0.5 - 1
+    new = old + torch.randn(B, Lc, generator=g) * 0.2
+    adv = torch.randn(B, 1, generator=g).expand(B, Lc).contiguous()
+    isw = (torch.rand(B, Lc, generator=g) + 0.5) if with_isw else None
+    cfg = _cfg(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28)
+    no = new.clone().requires_grad_()
+    if variant == "gspo":
+        fn, mode = CA.compute_policy_loss_gspo, "seq-mean-token-mean"
+        want = O.policy_loss_gspo(old, no, adv, mask, 0.2, 0.28, isw)
+    else:
+        fn, mode = CA.compute_policy_loss_geo_mean, "token-mean"
+        want = O.policy_loss_geo_mean(old, no, adv, mask, 0.2, 0.28, isw)
+    nd = new.to(dev).requires_grad_(with_grad)
+    loss, met = fn(old.to(dev), nd, adv.to(dev), mask.to(mask_dtype).to(dev), mode, cfg,
+                   None if isw is None else isw.to(dev))
+    _close(loss, want[0], what=f"{variant} loss")
+    assert abs(met["actor/pg_clipfrac"] - want[1].item()) < 1e-6
+    assert abs(met["actor/ppo_kl"] - want[2].item()) < 2e-6 * max(1.0, abs(want[2].item()))
+    if with_grad:
+        _close(torch.autograd.grad(loss, nd)[0], torch.autograd.grad(want[0], no)[0], atol=1e-9,
+               what=f"d {variant} loss / d log_prob")
+    torch.cuda.synchronize()
+    assert _counter_area_is_clear(_cabi.ticket_workspace(4096, dev))
+
+
 @pytest.mark.parametrize("loss_type", ["ppo_clip", "reinforce"])
 @pytest.mark.parametrize("rollout_is", [None, "token", "sequence"])
 @pytest.mark.parametrize("mode", ["token-mean", "seq-mean-token-sum"])

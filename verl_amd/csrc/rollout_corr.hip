@@ -72,25 +72,28 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
     float s[kRcSums];  // per-thread partials over 16 elements in fp32, widened after every chunk
 #pragma unroll
     for (int i = 0; i < kRcSums; ++i) s[i] = 0.f;
-    float o[kGroups][4], r[kGroups][4], m[kGroups][4], wt[kGroups][4];
+    float o[kGroups][4], r[kGroups][4], m[kGroups][4];
     const bool streaming = streams_past_caches(a.rows * a.cols);  // the grid counts spans of chunks, not chunks
     load_groups<VEC>(a.old_lp, pos, o, streaming);
     if (a.roll_lp) load_groups<VEC>(a.roll_lp, pos, r, streaming);
     load_mask_groups<VEC>(mask, pos, m, streaming);
 #pragma unroll
-    for (int k = 0; k < kGroups; ++k)
+    for (int k = 0; k < kGroups; ++k) {
+      float wt[4];  // the group's weights leave as soon as they exist: 16 registers fewer than holding the chunk's
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        wt[k][e] = 0.f;
+        wt[e] = 0.f;
         if (e >= pos.valid[k] || m[k][e] == 0.f) continue;
         s[kRcM] += 1.f;
         s[kRcOld] += o[k][e];
         if (!a.roll_lp) continue;
         const float d = o[k][e] - r[k][e];
-        const float w = expf(fminf(fmaxf(d, -kSafetyBound), kSafetyBound));
+        const float dc = fminf(fmaxf(d, -kSafetyBound), kSafetyBound);
+        const float w = expf(dc);
+        const float ed = d == dc ? w : expf(d);  // one exponential per token unless the clamp acted
         s[kRcRoll] += r[k][e];
         s[kRcD] += d;
-        s[kRcK3] += expf(d) - d - 1.f;
+        s[kRcK3] += ed - d - 1.f;
         s[kRcRho2] += w * w;
         if (a.level == VAMD_IS_TOKEN) {
           const float c = fminf(fmaxf(w, a.lower), a.thr);
@@ -103,10 +106,12 @@ __global__ __launch_bounds__(kRcThreads) void rollout_stats_kernel(RcArgs a, con
           s[kRcLow] += w < a.lower ? 1.f : 0.f;
           wmax = fmaxf(wmax, w);
           wmin = fminf(wmin, w);
-          wt[k][e] = t;
+          wt[e] = t;
         }
       }
-    if (a.level == VAMD_IS_TOKEN && a.weights) store_groups<VEC>(a.weights, pos, wt, streaming);
+      if (a.level == VAMD_IS_TOKEN && a.weights && pos.valid[k] > 0)
+        st4<VEC>(a.weights, pos.idx[k], pos.valid[k], wt, streaming);
+    }
 #pragma unroll
     for (int i = 0; i < kRcSums; ++i) acc[i] += (double)s[i];
   }
