@@ -77,6 +77,7 @@ from .trainer import (  # noqa: F401
     compute_data_metrics,
     pad_to_response_window,
     variance_proxy_metrics,
+    pf_ppo_weights,
 )
 from .rollout_corr import (  # noqa: F401
     offpolicy_metrics,

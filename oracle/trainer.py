@@ -114,3 +114,25 @@ def variance_proxy_metrics(batch, gradient_norm=None):
     out["variance_proxy/expected_a_squared"] = (adv**2).mean().item()
     out["variance_proxy/expected_w"] = w_sum.mean().item()
     return out
+
+
+@torch.no_grad()
+def pf_ppo_weights(token_level_scores, reweight_method="pow", weight_pow=2.0):
+    """The resampling probabilities of compute_pf_ppo_reweight_data, verl/trainer/ppo/core_algos.py:1921-1954,
+    written sequence by sequence: weight from the sequence's total score, plus 1e-8, floored at 1e-8, normalised the
+    way ``torch.multinomial`` normalises.  (The draw itself is a call of ``torch.multinomial`` and has no restatement.)"""
+    scores = [float(row.sum()) for row in token_level_scores]
+    best, worst = max(scores), min(scores)
+    weights = []
+    for sc in scores:
+        if reweight_method == "pow":
+            w = abs(sc) ** weight_pow
+        elif reweight_method == "max_min":
+            w = 1.0 if sc in (best, worst) else 0.0
+        elif reweight_method == "max_random":
+            w = 0.4 if sc == best else 0.1
+        else:
+            raise ValueError(f"Unsupported reweight_method: {reweight_method}")
+        weights.append(max(w + 1e-8, 1e-8))
+    total = sum(weights)
+    return torch.tensor([w / total for w in weights], dtype=torch.float64)

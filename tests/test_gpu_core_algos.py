@@ -1470,9 +1470,60 @@ def test_compute_advantage_dispatch(dev):
     with pytest.raises(AssertionError, match="sum_pi_squared"):
         data = _data({k: v for k, v in batch.items() if k not in ("sum_pi_squared", "reward_baselines")}, {"uid": uid})
         RT.compute_advantage(data, CA.AdvantageEstimator.OPTIMAL_TOKEN_BASELINE, config=cfg)
+    # PF-PPO: after GAE the batch is resampled row by row; every field moves with its row
     cfg.use_pf_ppo = True
-    with pytest.raises(NotImplementedError):
-        RT.compute_advantage(_data(dict(batch), {"uid": uid}), CA.AdvantageEstimator.GAE, config=cfg)
+    cfg.pf_ppo = {"reweight_method": "pow", "weight_pow": 2.0}
+    data = _data({k: v for k, v in batch.items() if k != "reward_baselines"}, {"uid": uid})
+    data.batch["token_level_scores"] = data.batch["token_level_rewards"].clone()
+    torch.manual_seed(5)
+    out = RT.compute_advantage(data, CA.AdvantageEstimator.GAE, gamma=0.99, lam=0.95, config=cfg)
+    assert out is not data and set(out.batch.keys()) == set(data.batch.keys())
+    want = O.gae_advantage_return(rewards, values, m, 0.99, 0.95)
+    full = {k: v.cpu() for k, v in data.batch.items()}            # data itself now holds the GAE outputs, unresampled
+    _close(full["advantages"], want[0], atol=2e-5, what="gae adv before resampling")
+    # recover the drawn indices from a field whose rows are all different
+    picks = [int((full["token_level_rewards"] == row).all(dim=1).nonzero()[0]) for row in out.batch["token_level_rewards"].cpu()]
+    assert len(picks) == B
+    for key, tensor in out.batch.items():
+        assert torch.equal(tensor.cpu(), full[key][picks]), key
+    assert list(out.non_tensor_batch["uid"]) == [uid[i] for i in picks]
+
+
+@pytest.mark.parametrize("method", ["pow", "max_min", "max_random"])
+def test_pf_ppo_reweight_data(dev, method):
+    """Resampling weights against the oracle's restatement (through the empirical frequencies of many draws and,
+    exactly, through the weight function), reproducibility under the seed, every field moved with its row, the
+    source object untouched, and the reference's error for an unknown method."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    g = torch.Generator().manual_seed(11)
+    B, Lc = 12, 9
+    scores = torch.randn(B, Lc, generator=g)
+    scores[3] = scores[7]                                        # a tie for some rank
+    want_p = O.pf_ppo_weights(scores, method, 1.5)
+    got_w = CA._pf_ppo_weights(scores.to(dev).sum(-1), method, 1.5).double().cpu() + 1e-8
+    assert torch.allclose(got_w / got_w.sum(), want_p, rtol=1e-5, atol=1e-12)
+    tags = np.array([f"row{i}" for i in range(B)], dtype=object)
+    data = _data({"token_level_scores": scores.to(dev), "ids": torch.arange(B, device=dev)}, {"uid": tags, "l": list(range(B))})
+    data.meta_info = {"per_row": [10 * i for i in range(B)], "other": [1, 2, 3], "name": "x"}
+    torch.manual_seed(3)
+    a = CA.compute_pf_ppo_reweight_data(data, method, 1.5)
+    torch.manual_seed(3)
+    b = CA.compute_pf_ppo_reweight_data(data, method, 1.5)
+    picks = a.batch["ids"].cpu().tolist()
+    assert picks == b.batch["ids"].cpu().tolist() and len(picks) == B
+    assert torch.equal(a.batch["token_level_scores"].cpu(), scores[picks])
+    assert list(a.non_tensor_batch["uid"]) == [f"row{i}" for i in picks] and a.non_tensor_batch["l"] == picks
+    assert a.meta_info == {"per_row": [10 * i for i in picks], "other": [1, 2, 3], "name": "x"}
+    assert torch.equal(data.batch["ids"].cpu(), torch.arange(B)) and data.meta_info["per_row"][1] == 10
+    # empirical frequencies over 400 resamplings of 12 draws: within 5 sigma of the oracle's probabilities
+    counts = torch.zeros(B, dtype=torch.float64)
+    for _ in range(400):
+        counts += torch.bincount(CA.compute_pf_ppo_reweight_data(data, method, 1.5).batch["ids"].cpu(), minlength=B)
+    n = counts.sum().item()
+    sigma = torch.sqrt(n * want_p * (1 - want_p)) + 1.0
+    assert ((counts - n * want_p).abs() <= 5 * sigma).all(), (counts / n, want_p)
+    with pytest.raises(ValueError, match="Unsupported reweight_method"):
+        CA.compute_pf_ppo_reweight_data(data, "softmax", 2.0)
 
 
 def test_data_metrics_reference_mock_batch(dev):

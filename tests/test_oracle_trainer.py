@@ -142,3 +142,19 @@ def test_variance_proxy_by_hand():
     assert m["variance_proxy/expected_w"] == pytest.approx((1 + 6) / 2)
     assert m["variance_proxy/proxy1_signal_strength"] == 0.0 and m["variance_proxy/proxy3_pure_noise"] == 0.0
     assert O.variance_proxy_metrics({"advantages": batch["advantages"]}) == {}
+
+
+def test_pf_ppo_weights_by_hand():
+    # sequence scores 2, -1, 0, 2 (no reference test holds a vector for this function: values worked by hand)
+    scores = torch.tensor([[1.0, 1.0], [-1.0, 0.0], [0.0, 0.0], [0.5, 1.5]])
+    p = O.pf_ppo_weights(scores, "pow", 2.0)            # 4, 1, 0, 4 (+1e-8 each) over 9
+    assert p.tolist() == pytest.approx([4 / 9, 1 / 9, 1e-8 / 9, 4 / 9], rel=1e-6, abs=1e-12)
+    p = O.pf_ppo_weights(scores, "pow", 1.0)            # |score|
+    assert p.tolist() == pytest.approx([2 / 5, 1 / 5, 1e-8 / 5, 2 / 5], rel=1e-6, abs=1e-12)
+    p = O.pf_ppo_weights(scores, "max_min", 2.0)        # both best sequences and the worst one
+    assert p.tolist() == pytest.approx([1 / 3, 1 / 3, 1e-8 / 3, 1 / 3], rel=1e-6, abs=1e-12)
+    p = O.pf_ppo_weights(scores, "max_random", 2.0)     # 0.4 for the best, 0.1 for the rest
+    assert p.tolist() == pytest.approx([0.4, 0.1, 0.1, 0.4], rel=1e-6)
+    assert p.sum().item() == pytest.approx(1.0)
+    with pytest.raises(ValueError, match="Unsupported reweight_method"):
+        O.pf_ppo_weights(scores, "softmax", 2.0)

@@ -1782,10 +1782,16 @@ extern "C" int vamd_policy_loss_variant_forward(int variant, const float* old_lo
   // workspace.  (With more workgroups than fit the device at once the waits add up: 305 against 190 us at 2048 x 16384.)
   bool rows_inline = false;
   if (per_row && waiting_kernels_allowed() && rows * chunks <= kInlineFoldRecords && rows * chunks <= kReadyBytes &&
-      chunks <= kRowSyncChunks &&
-      rows * chunks <= resident_workgroups((const void*)policy_kernel<true, float, true, true, true, -1, true>, kRcThreads)) {
+      chunks <= kRowSyncChunks) {
     VAMD_MASK_DISPATCH(mask_dtype, M, {
-      rows_inline = can_vectorize(cols, {old_log_prob, log_prob, advantages, is_weights, grad_unscaled}, mask, sizeof(M));
+      // occupancy of the instantiation that would be launched (mask type, gradient and weights change its registers)
+      const void* k = grad_unscaled
+          ? (is_weights ? (const void*)policy_kernel<true, M, true, true, true, -1, true>
+                        : (const void*)policy_kernel<true, M, true, false, true, -1, true>)
+          : (is_weights ? (const void*)policy_kernel<true, M, false, true, true, -1, true>
+                        : (const void*)policy_kernel<true, M, false, false, true, -1, true>);
+      rows_inline = rows * chunks <= resident_workgroups(k, kRcThreads) &&
+                    can_vectorize(cols, {old_log_prob, log_prob, advantages, is_weights, grad_unscaled}, mask, sizeof(M));
     });
   }
   if (per_row && !rows_inline && chunks > 1 && chunks <= kWholeRowChunks) {

@@ -1013,6 +1013,53 @@ def compute_value_loss(vpreds: torch.Tensor, returns: torch.Tensor, values: torc
     return vf_loss, out[1]
 
 
+# ---- PF-PPO data reweighting -----------------------------------------------------------------------
+@torch.no_grad()
+def _pf_ppo_weights(scores: torch.Tensor, reweight_method: str, weight_pow: float) -> torch.Tensor:
+    """Resampling weight of every sequence from its total score (reference core_algos.py:1921-1947)."""
+    if reweight_method == "pow":
+        return torch.pow(torch.abs(scores), weight_pow)
+    if reweight_method == "max_min":
+        return torch.where((scores == torch.max(scores)) | (scores == torch.min(scores)), 1.0, 0.0)
+    if reweight_method == "max_random":
+        return torch.where(scores == torch.max(scores), 0.4, 0.1)
+    raise ValueError(f"Unsupported reweight_method: {reweight_method}")
+
+
+def compute_pf_ppo_reweight_data(data, reweight_method: str = "pow", weight_pow: float = 2.0):
+    """Resample the batch with replacement, each sequence drawn with a probability proportional to a weight of its
+    total ``token_level_scores`` (reference core_algos.py:1905-1980): ``"pow"`` = ``|score| ** weight_pow``,
+    ``"max_min"`` = the best and the worst sequences only, ``"max_random"`` = 0.4 for the best against 0.1 for the
+    rest; ``1e-8`` is added to every weight.  Every tensor of ``data.batch``, every array or list of
+    ``data.non_tensor_batch`` and every ``meta_info`` list as long as the batch is taken at the same drawn indices.
+    Returns a new object of the type of ``data``; ``data`` itself is left as it was.  Host-side bookkeeping on whatever
+    device the batch lives on (one ``torch.multinomial`` and one gather per tensor); no kernel of the library runs."""
+    import copy
+
+    scores = data.batch["token_level_scores"].sum(dim=-1)
+    weights = torch.clamp(_pf_ppo_weights(scores, reweight_method, weight_pow) + 1e-8, min=1e-8)
+    batch_size = scores.shape[0]
+    sample_indices = torch.multinomial(weights, batch_size, replacement=True)
+    resampled_batch = {key: tensor[sample_indices] for key, tensor in data.batch.items()}
+    picks = sample_indices.cpu().numpy()
+    resampled_non_tensor = {}
+    for key, array in getattr(data, "non_tensor_batch", {}).items():
+        resampled_non_tensor[key] = array[picks] if isinstance(array, np.ndarray) else [array[i] for i in picks]
+    resampled_meta = {}
+    for key, value in (getattr(data, "meta_info", None) or {}).items():
+        resampled_meta[key] = [value[i] for i in picks] if isinstance(value, list) and len(value) == batch_size else value
+    out = copy.copy(data)   # the reference deep-copies and then replaces the same three fields
+    out.batch = type(data.batch)(resampled_batch)
+    try:
+        out.batch.batch_size = data.batch.batch_size
+    except AttributeError:   # a batch type that derives its size from its tensors
+        pass
+    out.non_tensor_batch = resampled_non_tensor
+    if hasattr(data, "meta_info"):
+        out.meta_info = resampled_meta
+    return out
+
+
 # ---- KL penalty -----------------------------------------------------------------------------------
 _KL_KINDS = {"kl": 0, "k1": 0, "abs": 1, "mse": 2, "k2": 2, "low_var_kl": 3, "k3": 3}
 

@@ -52,9 +52,10 @@ def compute_advantage(data, adv_estimator, gamma: float = 1.0, lam: float = 1.0,
     other estimator through the registry with ``token_level_rewards``, ``response_mask``, ``config``
     and whichever of ``uid`` / ``reward_baselines`` the batch holds.
 
-    Two differences from the reference: the optimal-token-baseline estimators also receive
-    ``old_log_probs`` here (they require it; the reference's dispatcher does not pass it), and the
-    PF-PPO reweighting after GAE (``config.use_pf_ppo``) raises ``NotImplementedError``.
+    One difference from the reference: the optimal-token-baseline estimators also receive
+    ``old_log_probs`` here (they require it; the reference's dispatcher does not pass it).  With
+    ``config.use_pf_ppo`` the batch is resampled after GAE as there (:172-177) and the resampled
+    object is what is returned.
     """
     if "response_mask" not in data.batch.keys():
         data.batch["response_mask"] = compute_response_mask(data)
@@ -63,7 +64,10 @@ def compute_advantage(data, adv_estimator, gamma: float = 1.0, lam: float = 1.0,
             token_level_rewards=data.batch["token_level_rewards"], values=data.batch["values"],
             response_mask=data.batch["response_mask"], gamma=gamma, lam=lam)
         if config is not None and config.get("use_pf_ppo", False):
-            raise NotImplementedError("PF-PPO data reweighting is not part of verl_amd")
+            data.batch["advantages"] = advantages
+            data.batch["returns"] = returns
+            return core_algos.compute_pf_ppo_reweight_data(data, config.pf_ppo.get("reweight_method"),
+                                                           config.pf_ppo.get("weight_pow"))
     elif adv_estimator == AdvantageEstimator.GRPO:
         advantages, returns = core_algos.compute_grpo_outcome_advantage(
             token_level_rewards=data.batch["token_level_rewards"], response_mask=data.batch["response_mask"],
