@@ -203,6 +203,7 @@ __global__ __launch_bounds__(kRowThreads) void row_softmax_backward_kernel(Backw
   const float glp = a.d_logprobs ? a.d_logprobs[r] : 0.f;
   const float gent = a.d_entropy ? a.d_entropy[r] : 0.f;
   const float mz = a.d_entropy ? a.mean_z[r] : 0.f;
+  const float t0 = fmaf(-gent, mz, glp);  // g_lp + g_ent (z - mean_z) = g_ent z + t0
   const int64_t label = a.d_logprobs ? a.labels[r] : -1;
   const int64_t stride = (int64_t)kRowThreads * G;
   const int64_t c0 = (int64_t)chunk * stride * F + (int64_t)threadIdx.x * G;
@@ -226,13 +227,21 @@ __global__ __launch_bounds__(kRowThreads) void row_softmax_backward_kernel(Backw
     } else {
       load_group<D, false>(row, c, a.cols, 0.f, x[u]);
     }
-    const int64_t hit = label - c;  // where the label sits in this group, if 0 <= hit < G: one wide compare per group
+    // four or five operations and an exponential per element; with 16-bit logits the arithmetic is as long as the memory time,
+    // so the one-hot term is added afterwards, by the one thread of the row whose group holds the label
 #pragma unroll
     for (int e = 0; e < G; ++e) {
       const float z = x[u][e];
       const float p = __builtin_amdgcn_exp2f(fmaf(z, kLog2e, -lse2));
-      const float t = fmaf(gent, z - mz, glp);  // g_lp + g_ent (z - mean_z)
-      x[u][e] = -p * t + ((hit == e) ? glp : 0.f);
+      // fp32 logits keep the difference z - mean_z (exact where the two are close); for 16-bit logits, whose
+      // output rounding is a thousand times coarser, the subtraction is folded into t0
+      const float t = sizeof(T) == 4 ? fmaf(gent, z - mz, glp) : fmaf(gent, z, t0);
+      x[u][e] = -p * t;
+    }
+    const int64_t hit = label - c;  // where the label sits in this group, if 0 <= hit < G
+    if (hit >= 0 && hit < G) {
+#pragma unroll
+      for (int e = 0; e < G; ++e) x[u][e] += (hit == e) ? glp : 0.f;
     }
     store_group<D, VEC>(out, c, a.cols, x[u]);
   }
