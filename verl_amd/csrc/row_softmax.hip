@@ -19,8 +19,8 @@ constexpr float kNegBig = -1.0e30f;
 
 // kVec: elements per 16-byte load; kBackwardLoads: such loads per thread in the backward kernel
 struct F32 { using type = float; static constexpr int kVec = 4; static constexpr int kBackwardLoads = 2; };
-struct BF16 { using type = uint16_t; static constexpr int kVec = 8; static constexpr int kBackwardLoads = 4; };
-struct F16 { using type = _Float16; static constexpr int kVec = 8; static constexpr int kBackwardLoads = 4; };
+struct BF16 { using type = uint16_t; static constexpr int kVec = 8; static constexpr int kBackwardLoads = 1; };
+struct F16 { using type = _Float16; static constexpr int kVec = 8; static constexpr int kBackwardLoads = 1; };
 
 __device__ __forceinline__ float to_float(float x, F32) { return x; }
 __device__ __forceinline__ float to_float(uint16_t x, BF16) { return __uint_as_float((unsigned)x << 16); }
@@ -190,7 +190,9 @@ struct BackwardArgs {
 // One workgroup per (row, chunk of kRowThreads * G * F columns).  F = D::kBackwardLoads 16-byte loads per thread:
 // small workgroups in large numbers keep more of the read and the write stream in flight than few workgroups that
 // loop (4096 x 152064 fp32 logits: 798 us with 8 KiB per workgroup, 841 with 16 KiB, 913 with a resident grid that
-// walks the items and requests the next one before it stores).
+// walks the items and requests the next one before it stores).  What counts is the elements per workgroup, about
+// 2048: one load per thread for 16-bit logits (bf16, steady state: 461 us with four loads, 404 with two, 378 with
+// one), two for fp32 (828 us; 863 with one).  Trimming the arithmetic per element changed nothing measurable.
 template <class D, bool VEC>
 __global__ __launch_bounds__(kRowThreads) void row_softmax_backward_kernel(BackwardArgs a) {
   using T = typename D::type;
@@ -227,8 +229,9 @@ __global__ __launch_bounds__(kRowThreads) void row_softmax_backward_kernel(Backw
     } else {
       load_group<D, false>(row, c, a.cols, 0.f, x[u]);
     }
-    // four or five operations and an exponential per element; with 16-bit logits the arithmetic is as long as the memory time,
-    // so the one-hot term is added afterwards, by the one thread of the row whose group holds the label
+    // the label's place in this group as a 32-bit index (-1: not here): one 32-bit compare per element below
+    const int64_t hit64 = label - c;
+    const int hit = (hit64 >= 0 && hit64 < G) ? (int)hit64 : -1;
 #pragma unroll
     for (int e = 0; e < G; ++e) {
       const float z = x[u][e];
@@ -236,12 +239,7 @@ __global__ __launch_bounds__(kRowThreads) void row_softmax_backward_kernel(Backw
       // fp32 logits keep the difference z - mean_z (exact where the two are close); for 16-bit logits, whose
       // output rounding is a thousand times coarser, the subtraction is folded into t0
       const float t = sizeof(T) == 4 ? fmaf(gent, z - mz, glp) : fmaf(gent, z, t0);
-      x[u][e] = -p * t;
-    }
-    const int64_t hit = label - c;  // where the label sits in this group, if 0 <= hit < G
-    if (hit >= 0 && hit < G) {
-#pragma unroll
-      for (int e = 0; e < G; ++e) x[u][e] += (hit == e) ? glp : 0.f;
+      x[u][e] = fmaf(-p, t, (hit == e) ? glp : 0.f);
     }
     store_group<D, VEC>(out, c, a.cols, x[u]);
   }
