@@ -215,7 +215,9 @@ def _group_ids_on_device(index, vectorized: bool, dev: torch.device):
     objects, which the kept array keeps alive).  Anything else is factorised afresh."""
     key = None
     if isinstance(index, np.ndarray):
-        key = (index.dtype.str, index.shape, hash(index.tobytes()), bool(vectorized), dev)
+        # the bytes themselves, not their hash: a dictionary compares keys in full, so two label arrays can never
+        # be taken for each other
+        key = (index.dtype.str, index.shape, index.tobytes(), bool(vectorized), dev)
         hit = _GROUP_ID_CACHE.get(key)
         if hit is not None:
             _GROUP_ID_CACHE.move_to_end(key)
