@@ -1005,6 +1005,35 @@ def test_sequence_level_losses_with_one_workgroup_per_row(dev, monkeypatch, vari
     assert _counter_area_is_clear(_cabi.ticket_workspace(4096, dev))
 
 
+@pytest.mark.parametrize("variant", ["gspo", "geo_mean"])
+def test_sequence_level_losses_whole_rows_streaming_size(dev, variant):
+    """1100 rows of four chunks: more workgroups than the in-kernel exchange allows and more than 2^24 elements per
+    tensor, i.e. the one-workgroup-per-row kernel on its non-temporal loads and stores, against the oracle."""
+    from verl_amd.trainer.ppo import core_algos as CA
+    B, Lc = 1100, 16384
+    g = torch.Generator().manual_seed(77)
+    mask, _ = _prefix_mask(B, Lc, g, lo=3)
+    mask[1] = 0
+    old = torch.randn(B, Lc, generator=g) * 0.5 - 1
+    new = old + torch.randn(B, Lc, generator=g) * 0.2
+    adv = torch.randn(B, 1, generator=g).expand(B, Lc).contiguous()
+    cfg = _cfg(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28)
+    no = new.clone().requires_grad_()
+    if variant == "gspo":
+        fn, mode = CA.compute_policy_loss_gspo, "seq-mean-token-mean"
+        want = O.policy_loss_gspo(old, no, adv, mask, 0.2, 0.28, None)
+    else:
+        fn, mode = CA.compute_policy_loss_geo_mean, "token-mean"
+        want = O.policy_loss_geo_mean(old, no, adv, mask, 0.2, 0.28, None)
+    nd = new.to(dev).requires_grad_()
+    loss, met = fn(old.to(dev), nd, adv.to(dev), mask.to(dev), mode, cfg, None)
+    _close(loss, want[0], what=f"{variant} loss")
+    assert abs(met["actor/pg_clipfrac"] - want[1].item()) < 1e-6
+    assert abs(met["actor/ppo_kl"] - want[2].item()) < 2e-6 * max(1.0, abs(want[2].item()))
+    _close(torch.autograd.grad(loss, nd)[0], torch.autograd.grad(want[0], no)[0], atol=1e-9,
+           what=f"d {variant} loss / d log_prob")
+
+
 @pytest.mark.parametrize("loss_type", ["ppo_clip", "reinforce"])
 @pytest.mark.parametrize("rollout_is", [None, "token", "sequence"])
 @pytest.mark.parametrize("mode", ["token-mean", "seq-mean-token-sum"])
