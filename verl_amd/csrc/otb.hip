@@ -178,7 +178,8 @@ __device__ __forceinline__ void otb_mask4(const M* __restrict__ mask, const OtbG
   }
 }
 
-constexpr int kOtbRows = 4;  // rows of a group whose loads are in flight together
+constexpr int kOtbRows = 4;  // rows of a larger group whose loads are in flight together
+constexpr int kOtbHeld = 8;  // a group of up to this many rows is held in registers between its loads and its stores
 
 // One workgroup per (group, 1024-column segment), a thread per 4 columns: the group's rows are added up in index
 // order, kOtbRows of them in flight at a time (a group is a handful of rows, so the launch needs narrow segments to
@@ -198,6 +199,46 @@ __global__ __launch_bounds__(kRcThreads) void otb_baseline_kernel(const float* r
   if (valid == 0) return;
   const int64_t first = gr.group_offsets[g], last = gr.group_offsets[g + 1];
   float num[4] = {0.f, 0.f, 0.f, 0.f}, den[4] = {0.f, 0.f, 0.f, 0.f};
+  if (last - first > 1 && last - first <= kOtbHeld) {
+    // A group of up to kOtbHeld rows stays in registers from its one round of loads to its stores: nothing is read a
+    // second time and the workgroup makes one trip to memory instead of four.  Same additions in the same order as
+    // the general path below.
+    float R[kOtbHeld][4], W[kOtbHeld][4], m[kOtbHeld][4];
+    int64_t row[kOtbHeld];
+#pragma unroll
+    for (int k = 0; k < kOtbHeld; ++k) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) R[k][e] = W[k][e] = m[k][e] = 0.f;
+      row[k] = first + k < last ? gr.rows_by_group[first + k] : -1;
+      if (row[k] >= 0) {
+        ld4<VEC>(returns, row[k] * cols + col, valid, R[k], streaming);
+        ld4<VEC>(w_cum, row[k] * cols + col, valid, W[k], streaming);
+        otb_mask4<VEC>(mask, gr, row[k], cols, col, valid, m[k]);
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kOtbHeld; ++k)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (m[k][e] != 0.f) {
+          num[e] += R[k][e] * W[k][e] * m[k][e];
+          den[e] += W[k][e] * m[k][e];
+        }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) num[e] = num[e] / (den[e] + eps);
+#pragma unroll
+    for (int k = 0; k < kOtbHeld; ++k) {
+      if (row[k] < 0) continue;
+      const int64_t cut = gr.tail_start ? gr.tail_start[row[k]] : cols;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float b = col + e < cut ? num[e] : 0.f;
+        R[k][e] = m[k][e] != 0.f ? (R[k][e] - b) * m[k][e] : 0.f;
+      }
+      st4<VEC>(adv, row[k] * cols + col, valid, R[k], streaming);
+    }
+    return;
+  }
   if (last - first > 1) {
     for (int64_t i0 = first; i0 < last; i0 += kOtbRows) {
       float R[kOtbRows][4], W[kOtbRows][4], m[kOtbRows][4];
