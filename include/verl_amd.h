@@ -85,6 +85,16 @@ extern "C" {
 int vamd_abi_version(void);
 const char* vamd_last_error(void);
 
+/* Process-wide switch for the kernels whose workgroups wait for each other inside one launch (vamd_gae with
+ * whiten = 1, vamd_grpo_advantage, GSPO / GMPO in vamd_policy_loss_variant_forward): 0 keeps every entry point to
+ * launches that never wait, 1 allows the waiting forms, a negative value hands the decision back to the environment
+ * variable VAMD_WAITING_KERNELS (unset or anything but "0" = allowed).  Meant for a host that has seen one bounded
+ * wait run out (vamd_gae reports it in moments_out[4]) on a GPU it shares with other long-running kernels: a
+ * time-out costs about a second of polling, and the conditions behind it rarely go away between two calls.
+ * No counterpart in the reference, whose estimators are sequences of torch launches. */
+void vamd_set_waiting_kernels(int allowed);
+int vamd_waiting_kernels_enabled(void);
+
 /* ------------------------------------------------------------------------------------------
  * Fused vocab-projection log-prob / entropy head.
  * Replaces kernels.efficient_entropy_forward / efficient_entropy_backward behind

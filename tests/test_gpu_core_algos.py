@@ -171,7 +171,8 @@ def test_gae_bounded_wait_runs_out_without_hanging(dev, monkeypatch):
     want_adv, want_ret = O.gae_advantage_return(r.cpu().double(), v.cpu().double(), m.cpu().double(), 1.0, 0.95)
     monkeypatch.setenv("VAMD_GATE_SPIN_LIMIT", "0")
     CA._WARNED.clear()
-    CA._GAE_WAIT_TIMED_OUT.clear()
+    L_ = _cabi.lib()
+    assert L_.vamd_waiting_kernels_enabled() == 1
     try:
         with pytest.warns(RuntimeWarning, match="timed out"):
             adv, ret = CA.compute_gae_advantage_return(r, v, m, 1.0, 0.95)
@@ -179,15 +180,17 @@ def test_gae_bounded_wait_runs_out_without_hanging(dev, monkeypatch):
         assert (adv.cpu().double() - want_adv).abs().max().item() <= 2e-5 * want_adv.abs().max().item()
         ws = _cabi.ticket_workspace(4096, dev)
         assert _counter_area_is_clear(ws)
-        # the time-out is remembered: the next call takes the two-launch form at once (no second warning, no polling)
-        assert CA._GAE_WAIT_TIMED_OUT
+        # the time-out is remembered by the library: every kernel that waits inside a launch is switched off, so the
+        # next call takes the two-launch form at once (no second warning, no polling), and so would GRPO
+        assert L_.vamd_waiting_kernels_enabled() == 0
         import warnings
         with warnings.catch_warnings():
             warnings.simplefilter("error")
             adv, ret = CA.compute_gae_advantage_return(r, v, m, 1.0, 0.95)
         assert (adv.cpu().double() - want_adv).abs().max().item() <= 2e-5 * want_adv.abs().max().item()
     finally:
-        CA._GAE_WAIT_TIMED_OUT.clear()
+        L_.vamd_set_waiting_kernels(-1)   # back to what the environment says
+    assert L_.vamd_waiting_kernels_enabled() == 1
     monkeypatch.delenv("VAMD_GATE_SPIN_LIMIT")
     adv, ret = CA.compute_gae_advantage_return(r, v, m, 1.0, 0.95)
     assert (adv.cpu().double() - want_adv).abs().max().item() <= 2e-5 * want_adv.abs().max().item()

@@ -31,6 +31,8 @@ AGG_MODES = {
 SIGNATURES = {
     "vamd_abi_version": (c_int, []),
     "vamd_last_error": (c_char_p, []),
+    "vamd_set_waiting_kernels": (None, [c_int]),
+    "vamd_waiting_kernels_enabled": (c_int, []),
     "vamd_copy_bytes": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "vamd_sum4": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "vamd_mfma_yardstick_flops": (c_int64, [c_int, c_int, c_int]),

@@ -9,6 +9,8 @@
 
 #include "common.h"
 
+#include <atomic>
+
 namespace vamd {
 
 static thread_local char g_error[512] = "";
@@ -59,7 +61,13 @@ int resident_workgroups(const void* kernel, int threads, size_t dynamic_lds_byte
   return n;
 }
 
+// Process-wide switch over the environment variable: -1 = not set (the variable decides), 0 / 1 = set by
+// vamd_set_waiting_kernels().  A host that has seen one waiting kernel time out switches all of them off at once.
+static std::atomic<int> g_waiting_override{-1};
+
 bool waiting_kernels_allowed() {
+  const int o = g_waiting_override.load(std::memory_order_relaxed);
+  if (o >= 0) return o != 0;
   const char* e = getenv("VAMD_WAITING_KERNELS");
   return !(e && e[0] == '0' && e[1] == 0);
 }
@@ -225,3 +233,9 @@ extern "C" int vamd_mfma_yardstick(int shape, const void* seed, float* out, int 
 
 extern "C" int vamd_abi_version(void) { return VAMD_ABI_VERSION; }
 extern "C" const char* vamd_last_error(void) { return vamd::g_error; }
+
+extern "C" void vamd_set_waiting_kernels(int allowed) {
+  vamd::g_waiting_override.store(allowed < 0 ? -1 : (allowed != 0 ? 1 : 0), std::memory_order_relaxed);
+}
+
+extern "C" int vamd_waiting_kernels_enabled(void) { return vamd::waiting_kernels_allowed() ? 1 : 0; }

@@ -148,7 +148,6 @@ def _mask_matrix(mask: torch.Tensor, dev: torch.device, shape) -> tuple[torch.Te
 _WARNED = set()
 
 
-_GAE_WAIT_TIMED_OUT: list = []   # non-empty once vamd_gae's one-launch form has timed out in this process
 
 
 def _warn_once(text: str) -> None:
@@ -179,10 +178,12 @@ def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torc
         mom = torch.empty(5, dtype=torch.float64, device=dev)
         Lb = _cabi.lib()
         ws = _cabi.ticket_workspace(Lb.vamd_gae_workspace_bytes(B, Lc), dev)
-        # 1: one launch whose workgroups meet once; 2: two launches, nobody waits.  Once the meeting has timed out in
-        # this process (a GPU shared with long-running kernels) later calls go straight to 2: a time-out costs about a
-        # second of polling, and the conditions that caused it rarely go away between two calls.
-        for whiten in ((2,) if _GAE_WAIT_TIMED_OUT else (1, 2)):
+        # 1: one launch whose workgroups meet once (the library itself takes the two-launch form when waiting kernels
+        # are switched off); 2: two launches, nobody waits.  Once the meeting has timed out in this process (a GPU
+        # shared with long-running kernels) the waiting kernels are switched off for the whole library -- GRPO and the
+        # sequence-level losses included: a time-out costs about a second of polling, and the conditions that caused it
+        # rarely go away between two calls.
+        for whiten in (1, 2):
             with _cabi.device_guard(dev):
                 _cabi.check(Lb.vamd_gae(r.data_ptr(), v.data_ptr(), m.data_ptr(), code, B, Lc, float(gamma),
                                         float(lam), whiten, adv.data_ptr(), ret.data_ptr(), mom.data_ptr(),
@@ -192,9 +193,10 @@ def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torc
                 break
             # the workgroups' bounded wait for each other ran out (a GPU shared with long-running kernels): the
             # advantages were left unwhitened; do it again without waiting
-            _GAE_WAIT_TIMED_OUT.append(True)
-            _warn_once("vamd_gae: the one-launch estimator timed out waiting for its workgroups; using two launches "
-                       "from now on (set VAMD_WAITING_KERNELS=0 to make that the rule from the start)")
+            Lb.vamd_set_waiting_kernels(0)
+            _warn_once("vamd_gae: the one-launch estimator timed out waiting for its workgroups; kernels that wait "
+                       "inside a launch are switched off from now on (set VAMD_WAITING_KERNELS=0 to make that the "
+                       "rule from the start)")
         verl_F._raise_on_tiny_mask(mom_host[0])
         if mom_host[4] != 0.0:
             raise RuntimeError("vamd_gae: the workgroups' bounded wait for the whitening statistics ran out; "
