@@ -880,6 +880,31 @@ def main() -> None:
                       "step_hardware_frac": hw_gemms * gemm_flops / (r["ms_per_step"] * 1e-3) / peak,
                       "kernels": head_kernel_times(L, one_sided(wrt), prof_steps)}
 
+    # The same step with the upstream gradients of 40 % of the tokens zero, in runs (prompt tokens between responses,
+    # which the loss masks out): the backward kernels run over the other tokens only.  Beside it the same gradients
+    # with that switched off.
+    keep = (torch.arange(n, device=dev) % 2048) >= 820          # 820 prompt tokens in every 2048
+    g_lp_masked, g_ent_masked = g_lp * keep, g_ent * keep
+
+    def masked_step():
+        lp, ent = linear_cross_entropy(hidden, weight, labels, T)
+        return torch.autograd.grad((lp, ent), (hidden, weight), (g_lp_masked, g_ent_masked))
+
+    saved_skip = os.environ.get("VAMD_LCE_SKIP_ZERO_GRAD_TOKENS")
+    masked = {}
+    import verl_amd.utils.kernel.linear_cross_entropy as head_module
+    for key, flag in (("active_tokens_only", "1"), ("all_tokens", "0")):
+        os.environ["VAMD_LCE_SKIP_ZERO_GRAD_TOKENS"] = flag
+        head_module._ACTIVE_PROBE["rest"] = 0   # the steps before found every token active: look again now
+        r = time_head_mode(masked_step, args.steps, args.warmup, n, dev)
+        masked[key] = {"ms_per_step": r["ms_per_step"], "tokens_per_s": r["tokens_per_s"]}
+    if saved_skip is None:
+        del os.environ["VAMD_LCE_SKIP_ZERO_GRAD_TOKENS"]
+    else:
+        os.environ["VAMD_LCE_SKIP_ZERO_GRAD_TOKENS"] = saved_skip
+    modes["prompt_tokens_masked_40pct"] = {**masked, "default": False,
+                                           "zero_gradient_tokens": int(n - int(keep.sum())), "of_tokens": n}
+
     line = {
         "metric": "tokens/s fwd+bwd logprob+entropy head @Qwen2.5-7B shape; MFMA util %",
         "value": tokens_per_s,

@@ -151,6 +151,57 @@ def test_backward_runs_only_the_gradients_that_are_needed(dev, backward_mode, fr
             assert torch.equal(w1.grad, both_dw)
 
 
+@pytest.mark.parametrize("n,h,v,zero_share", [(700, 256, 8192, 0.45), (1388, 512, 20000, 0.8), (300, 256, 1152, 1.0),
+                                              (513, 256, 4096, 0.05)])
+def test_backward_leaves_out_tokens_without_upstream_gradient(dev, monkeypatch, n, h, v, zero_share):
+    """Tokens whose upstream gradients are both zero (prompt tokens under a response mask) are left out of the
+    backward kernels: d_hidden is the same bits as over all tokens (zero rows where nothing came in), d_weight the
+    same sum in another grouping; both against the oracle.  A share of zeros below one in ten changes nothing; a
+    batch of nothing but zeros gives zero gradients without a launch."""
+    from verl_amd.utils.kernel import linear_cross_entropy as K
+    from verl_amd.utils.experimental.torch_functional import FusedLinearForPPO
+    hidden, weight, labels = _make(n, h, v, seed=3 * n + v)
+    g = torch.Generator().manual_seed(n + 7)
+    g_ent = (torch.rand(n, generator=g) - 0.5).bfloat16().float()
+    g_lp = ((torch.rand(n, generator=g) - 0.5) * 2).bfloat16().float()
+    masked = torch.zeros(n, dtype=torch.bool)
+    run = 0                                                       # runs of masked tokens, like prompts between responses
+    while run < n:
+        length = int(torch.randint(20, 120, (1,), generator=g))
+        if torch.rand(1, generator=g).item() < zero_share:
+            masked[run:run + length] = True
+        run += length
+    if zero_share == 1.0:
+        masked[:] = True
+    g_ent[masked] = 0.0
+    g_lp[masked] = 0.0
+    _, _, want_dh, want_dw = _oracle(hidden, weight, labels, 1.5, g_lp, g_ent)
+    seen = []
+    real = K.backward_over_active_tokens
+    monkeypatch.setattr(K, "backward_over_active_tokens", lambda idx, *a, **k: (seen.append(int(idx.numel())), real(idx, *a, **k))[1])
+    import verl_amd.utils.experimental.torch_functional as E
+    monkeypatch.setattr(E, "backward_over_active_tokens", K.backward_over_active_tokens)
+    for op in (lambda a, b, c: K.linear_cross_entropy(a, b, c, 1.5), lambda a, b, c: FusedLinearForPPO()(a, b, c, 1.5)):
+        grads = {}
+        for skip in ("1", "0"):
+            monkeypatch.setenv("VAMD_LCE_SKIP_ZERO_GRAD_TOKENS", skip)
+            K._ACTIVE_PROBE["rest"] = 0                           # look at the gradients in this call
+            seen.clear()
+            hd = hidden.to(dev).requires_grad_(); wd = weight.to(dev).requires_grad_()
+            lp, ent = op(hd, wd, labels.to(dev))
+            grads[skip] = torch.autograd.grad((ent, lp), (hd, wd), (g_ent.to(dev).to(ent.dtype), g_lp.to(dev).to(lp.dtype)))
+            expect_compaction = skip == "1" and int(masked.sum()) * 10 >= n
+            assert (seen == [n - int(masked.sum())]) if expect_compaction else (seen == []), (skip, seen)
+            # a call that found (nearly) everything active is followed by calls that do not look
+            assert K._ACTIVE_PROBE["rest"] == (K._ACTIVE_PROBE_REST if skip == "1" and not expect_compaction else 0)
+        dh, dw = grads["1"]
+        assert torch.equal(dh, grads["0"][0])
+        assert (dh[masked.to(dev)] == 0).all()
+        _close_bf16(dh, want_dh, "d_hidden over the active tokens")
+        _close_bf16(dw, want_dw, "d_weight over the active tokens")
+        _close_bf16(dw, grads["0"][1].float().cpu(), "d_weight: active tokens against all tokens")
+
+
 def test_backward_c_abi_refuses_a_call_that_asks_for_nothing(dev):
     from verl_amd import _cabi
     from verl_amd.utils.kernel.linear_cross_entropy import efficient_entropy_backward, efficient_entropy_forward

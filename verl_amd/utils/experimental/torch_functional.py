@@ -14,7 +14,8 @@ from typing import Optional
 
 import torch
 
-from ..kernel.linear_cross_entropy import efficient_entropy_backward, efficient_entropy_forward
+from ..kernel.linear_cross_entropy import (active_token_index, backward_over_active_tokens,
+                                           efficient_entropy_backward, efficient_entropy_forward)
 
 
 class FusedLinearForPPOFunction(torch.autograd.Function):
@@ -56,10 +57,18 @@ class FusedLinearForPPOFunction(torch.autograd.Function):
             dlog_probs = dlog_probs.reshape(-1)
         if dentropy is not None:
             dentropy = dentropy.reshape(-1)
-        # only the gradient GEMMs whose inputs require a gradient are run (reference :150-156, :184-187)
-        dhidden_states, dvocab_weights = efficient_entropy_backward(
-            dlog_probs, dentropy, hidden_states, vocab_weights, input_ids, lse, mean_z, 0, ctx.temperature,
-            need_d_hidden=ctx.needs_input_grad[0], need_d_weight=ctx.needs_input_grad[1])
+        # only the gradient GEMMs whose inputs require a gradient are run (reference :150-156, :184-187), and only over
+        # the tokens whose upstream gradients are not both zero (prompt tokens, which the loss masks out)
+        need_dh, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        idx = active_token_index(dlog_probs, dentropy, hidden_states.shape[0]) if (need_dh or need_dw) else None
+        if idx is not None:
+            dhidden_states, dvocab_weights = backward_over_active_tokens(
+                idx, dlog_probs, dentropy, hidden_states, vocab_weights, input_ids, lse, mean_z, ctx.temperature,
+                need_dh, need_dw)
+        else:
+            dhidden_states, dvocab_weights = efficient_entropy_backward(
+                dlog_probs, dentropy, hidden_states, vocab_weights, input_ids, lse, mean_z, 0, ctx.temperature,
+                need_d_hidden=need_dh, need_d_weight=need_dw)
         if dhidden_states is not None and ctx.orig_ndim == 3:
             dhidden_states = dhidden_states.view(ctx.orig_batch_size, -1, hidden_states.shape[-1])
         return dhidden_states, dvocab_weights, None, None, None
