@@ -117,9 +117,12 @@ __device__ __forceinline__ int acc_row(const LanePos& p, int nb) { return p.wr *
 //   ds_read_b128 is served 16 lanes (256 B, all 64 banks) per cycle; a fragment read touches 16
 //   consecutive rows at one logical chunk, i.e. 8 even and 8 odd rows (two rows span the banks),
 //   so rows of equal parity must land on 8 different chunk positions.
-// kmajor slab : row k (512 B = 32 chunks of 16 B); chunk c lives at position c ^ (4 (k & 3)).
-//   A transposing read touches, per 32 lanes, 4 consecutive k rows x 64 B at one x block; rows
-//   are 512 B apart (the same banks), so the XOR moves the 4 rows to 4 different 64 B groups.
+// kmajor slab : row k (512 B = 32 chunks of 16 B); chunk c lives at position c ^ (4 (k & 3)) ^ (2 ((k >> 3) & 1)).
+//   A transposing 8-byte read is served 32 lanes at a time, and those address 8 k rows (k = 8 lq + 0..3 for two
+//   values of lq) x 32 B at one x block; rows are 512 B apart (the same banks), so the first XOR moves the 4 rows of
+//   a quad to 4 different 64 B groups and the second puts the rows of the odd lq in the other 32 B half: the 8 rows
+//   cover the 64 banks once (with the first XOR alone the two lq groups collided: 45 % of the LDS cycles of the
+//   gradient GEMMs were bank-conflict cycles).
 __device__ __forceinline__ int swizzle_direct(int row) { return (row >> 1) & 7; }
 
 // Where one slab of an operand comes from: a buffer resource whose base is the operand's tile
@@ -185,7 +188,7 @@ __device__ __forceinline__ u32x4 span_rsrc(const void* p, int64_t bytes) {
 //            and fetches logical chunk (L % 8) ^ swizzle of that row -- 8 lanes cover one whole
 //            128 B line of the memory row;
 //   kmajor : block b = k rows 2 b, 2 b + 1; lane L sits at k row 2 b + L / 32, chunk position
-//            L % 32, and fetches logical chunk (L % 32) ^ 4 (k & 3) -- 32 lanes cover 512
+//            L % 32, and fetches logical chunk (L % 32) ^ 4 (k & 3) ^ 2 ((k >> 3) & 1) -- 32 lanes cover 512
 //            contiguous bytes of the memory row.
 // Both swizzles are unchanged by the + 64 rows (direct) / + 16 k rows (kmajor) between loads, so
 // the per-lane address is ONE 32-bit offset; everything that changes between loads, slabs and
@@ -205,7 +208,7 @@ struct SlabDma {
       step = (8u * kWaves) * ld_bytes;
     } else {
       const unsigned k = 2u * w + (lane >> 5);
-      voff = k * ld_bytes + (((lane & 31u) ^ (4u * (k & 3u))) << 4);
+      voff = k * ld_bytes + (((lane & 31u) ^ (4u * (k & 3u)) ^ (2u * ((k >> 3) & 1u))) << 4);
       step = (2u * kWaves) * ld_bytes;
     }
     lds_wave = __builtin_amdgcn_readfirstlane(w * 1024u);
@@ -245,7 +248,7 @@ struct FragAddr {
 #pragma unroll
       for (int b = 0; b < kMB; ++b) {
         const int blk = first_block + b;
-        off[b] = b < nblocks ? k0 * 512 + 64 * ((blk >> 1) ^ q) + 32 * (blk & 1) + 8 * (lx & 3) : 0;
+        off[b] = b < nblocks ? k0 * 512 + 64 * ((blk >> 1) ^ q) + 32 * ((blk & 1) ^ (lq & 1)) + 8 * (lx & 3) : 0;
       }
     }
   }
