@@ -413,9 +413,9 @@ __device__ __forceinline__ void row_presums(int variant, const ChunkPos& pos, co
       if (variant == VAMD_PL_GSPO) {
         s_k += (we != 0.f ? d : 0.f) * we;  // where(mask, lp - old, 0) * mask
       } else {
-        const float c = fminf(fmaxf(d, lo), hi);
+        // min(d, clamp(d, lo, hi)) is min(d, hi) and max(d, clamp(d, lo, hi)) is max(d, lo) (lo <= hi)
         const float A = a[g][e];
-        const float k = A > 0.f ? fminf(d, c) : (A < 0.f ? fmaxf(d, c) : 0.f);
+        const float k = A > 0.f ? fminf(d, hi) : (A < 0.f ? fmaxf(d, lo) : 0.f);
         s_k += k * we;
         s_a += A * we;
         if (ISW) s_w += logf(iw[g][e] + 1e-10f) * we;
