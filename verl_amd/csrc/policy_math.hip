@@ -330,13 +330,15 @@ __device__ __forceinline__ TokenLoss token_loss(const PolicyParams& pp, float ol
       // seq_lr carries q = -(A_seq ratio_seq w_seq) / (M + 1e-8): every valid token of the row holds the loss q
       // (their sum is the sequence loss), and d loss / d log_prob is q where the token's log-ratio enters the
       // geometric mean unclipped
-      const float c = fminf(fmaxf(d, pp.nkl_lo), pp.nkl_hi);
-      const float ind = A > 0.f ? (d <= pp.nkl_hi ? 1.f : 0.f) : (A < 0.f ? (d >= pp.nkl_lo ? 1.f : 0.f) : 0.f);
+      // written with & and | on purpose: short-circuit forms became a branch per token
+      const bool up = A > 0.f, down = A < 0.f;
+      const bool above = d > pp.nkl_hi, below = d < pp.nkl_lo;  // outside the clip range (d != clamp(d))
+      const bool passes = (up & !above) | (down & !below);
       t.loss = seq_lr;
-      t.dloss = seq_lr * ind;
+      t.dloss = passes ? seq_lr : 0.f;
       t.kl = -d;
-      t.cf = (d != c && A > 0.f) ? 1.f : 0.f;
-      t.cfl = (d != c && A < 0.f) ? 1.f : 0.f;
+      t.cf = (up & (above | below)) ? 1.f : 0.f;
+      t.cfl = (down & (above | below)) ? 1.f : 0.f;
     } break;
     case VAMD_PL_CISPO: {
       const float r = expf(k);
@@ -406,7 +408,8 @@ __device__ __forceinline__ void row_presums(int variant, const ChunkPos& pos, co
   for (int g = 0; g < kGroups; ++g)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      if (e >= pos.valid[g]) continue;
+      // elements past the end of the row were loaded as zeros with weight zero: they add nothing, and leaving the
+      // test out keeps the sixteen tokens of a thread free of branches
       const float d = n[g][e] - o[g][e];
       const float we = w[g][e];
       s_m += we;
