@@ -393,6 +393,25 @@ __device__ __forceinline__ TokenLoss token_loss(const PolicyParams& pp, float ol
   return t;
 }
 
+// f(std::integral_constant<int, variant>): for a kernel built with the variant fixed, that variant; otherwise the
+// runtime one, so that the caller's token loop exists once per variant instead of switching per token.
+template <int VARIANT, class F>
+__device__ __forceinline__ void with_policy_variant(int variant, F&& f) {
+  if constexpr (VARIANT >= 0) {
+    f(std::integral_constant<int, VARIANT>());
+  } else {
+    switch (variant) {
+      case VAMD_PL_GPG: f(std::integral_constant<int, VAMD_PL_GPG>()); break;
+      case VAMD_PL_CISPO: f(std::integral_constant<int, VAMD_PL_CISPO>()); break;
+      case VAMD_PL_SAPO: f(std::integral_constant<int, VAMD_PL_SAPO>()); break;
+      case VAMD_PL_GSPO: f(std::integral_constant<int, VAMD_PL_GSPO>()); break;
+      case VAMD_PL_REINFORCE: f(std::integral_constant<int, VAMD_PL_REINFORCE>()); break;
+      case VAMD_PL_GEO_MEAN: f(std::integral_constant<int, VAMD_PL_GEO_MEAN>()); break;
+      default: f(std::integral_constant<int, VAMD_PL_VANILLA>()); break;
+    }
+  }
+}
+
 // The per-sequence quantity of the two losses that need one before their per-token pass, as four partial sums over
 // one chunk of the row (fp32 over a thread's 16 tokens; the caller widens and reduces them):
 //   GSPO (core_algos.py:1286-1294)      sum(m), sum((lp - old) m), 0, 0
@@ -559,28 +578,33 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
   // GMPO's importance weights enter through the sequence weight above, not token by token
   const bool isw_per_token = ISW && variant != VAMD_PL_GEO_MEAN;
   float s_loss = 0, s_m = 0, s_kl = 0, s_cf = 0, s_cfl = 0;
+  // a kernel built for every variant (VARIANT = -1) picks the variant once, here, and runs that variant's copy of
+  // the token loop: chosen per token, the sixteen tokens of a thread were sixteen seven-way switches
+  with_policy_variant<VARIANT>(variant, [&](auto which) {
+    constexpr int V = decltype(which)::value;
 #pragma unroll
-  for (int g = 0; g < kGroups; ++g)
+    for (int g = 0; g < kGroups; ++g)
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const TokenLoss t = token_loss<VARIANT>(pp, o[g][e], n[g][e], a[g][e], seq_lr);
-      float loss = t.loss;
-      if (isw_per_token) loss *= iw[g][e];
-      const float we = w[g][e];
-      const bool in = we != 0.f;
-      // Elements past the end of the row were loaded as zeros with weight zero and add nothing, so the test is
-      // redundant.  The small launches (FOLD) are faster without its sixteen branches (512 x 4096: 16.1 -> 15.8 us
-      // with the gradient); the large ones are faster with it (2048 x 16384: 115 against 117 us), where the
-      // compiler then holds all of a thread's loads in registers at once.
-      if (FOLD || e < pos.valid[g]) {
-        s_loss += ((token_mean && !in) ? 0.f : loss) * we;
-        s_m += we;
-        s_kl += in ? t.kl * we : 0.f;
-        s_cf += in ? t.cf * we : 0.f;
-        s_cfl += in ? t.cfl * we : 0.f;
+      for (int e = 0; e < 4; ++e) {
+        const TokenLoss t = token_loss<V>(pp, o[g][e], n[g][e], a[g][e], seq_lr);
+        float loss = t.loss;
+        if (isw_per_token) loss *= iw[g][e];
+        const float we = w[g][e];
+        const bool in = we != 0.f;
+        // Elements past the end of the row were loaded as zeros with weight zero and add nothing, so the test is
+        // redundant.  The small launches (FOLD) are faster without its sixteen branches (512 x 4096: 16.1 -> 15.8
+        // us with the gradient); the large ones are faster with it (2048 x 16384: 115 against 117 us), where the
+        // compiler then holds all of a thread's loads in registers at once.
+        if (FOLD || e < pos.valid[g]) {
+          s_loss += ((token_mean && !in) ? 0.f : loss) * we;
+          s_m += we;
+          s_kl += in ? t.kl * we : 0.f;
+          s_cf += in ? t.cf * we : 0.f;
+          s_cfl += in ? t.cfl * we : 0.f;
+        }
+        if (GRAD) gr[g][e] = (isw_per_token ? t.dloss * iw[g][e] : t.dloss) * we;
       }
-      if (GRAD) gr[g][e] = (isw_per_token ? t.dloss * iw[g][e] : t.dloss) * we;
-    }
+  });
   if (GRAD) store_groups<VEC>(grad, pos, gr);
   static_assert(!ROWS || FOLD, "a launch that sets ready bytes has a last workgroup that clears them");
   double acc[5] = {s_loss, s_m, s_kl, s_cf, s_cfl};
