@@ -627,6 +627,61 @@ def head_kernel_times(L, step, prof_steps: int) -> dict:
     return kernels
 
 
+def composed_actor_step(dev, steps: int) -> dict:
+    """One actor update step the way the trainer composes it, at the benchmark's head shape as 4 sequences of 4096
+    tokens: head -> per-token log-prob and entropy -> clipped policy loss + entropy bonus + KL loss -> one backward
+    through everything.  Beside it the same step with the three losses replaced by plain sums of the head's outputs:
+    the difference is what the losses cost inside a step (kernels, their Python mirror and their share of autograd),
+    where called alone a loss with its backward pays a whole autograd launch of its own."""
+    import types
+
+    import torch
+
+    from verl_amd.trainer.ppo import core_algos as CA
+    from verl_amd.utils.kernel.linear_cross_entropy import linear_cross_entropy
+
+    B, Lc, h, v = 4, 4096, 3584, 152064
+    n = B * Lc
+    g = torch.Generator(device=dev).manual_seed(9)
+    hidden = torch.randn(n, h, device=dev, generator=g).bfloat16().requires_grad_()
+    weight = (torch.randn(v, h, device=dev, generator=g) * 0.02).bfloat16().requires_grad_()
+    labels = torch.randint(0, v, (n,), device=dev, generator=g)
+    lens = torch.randint(Lc // 2, Lc + 1, (B,), device=dev, generator=g)
+    mask = (torch.arange(Lc, device=dev)[None, :] < lens[:, None]).float()
+    adv = torch.randn(B, Lc, device=dev, generator=g)
+    cfg = types.SimpleNamespace(clip_ratio=0.2, clip_ratio_low=None, clip_ratio_high=None, global_batch_info={})
+    cfg.get = lambda k, d=None: getattr(cfg, k, d)
+    with torch.no_grad():
+        old_lp, _ = linear_cross_entropy(hidden, weight, labels, 1.0)
+        old_lp = old_lp.view(B, Lc) + 0.05 * torch.randn(B, Lc, device=dev, generator=g)
+        ref_lp = old_lp + 0.05 * torch.randn(B, Lc, device=dev, generator=g)
+
+    def with_losses():
+        lp, ent = linear_cross_entropy(hidden, weight, labels, 1.0)
+        lp, ent = lp.view(B, Lc), ent.view(B, Lc)
+        pg, _ = CA.compute_policy_loss_vanilla(old_lp, lp, adv, mask, "token-mean", cfg)
+        loss = pg - 0.001 * CA.agg_loss(ent, mask, "token-mean") + 0.01 * CA.compute_kl_loss(lp, ref_lp, mask)
+        torch.autograd.grad(loss, (hidden, weight))
+
+    def plain_sums():
+        lp, ent = linear_cross_entropy(hidden, weight, labels, 1.0)
+        torch.autograd.grad((lp * mask.view(-1)).sum() - 0.001 * (ent * mask.view(-1)).sum(), (hidden, weight))
+
+    def timed(fn):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / steps * 1e3
+
+    a, b = timed(with_losses), timed(plain_sums)
+    return {"batch": B, "response_length": Lc, "hidden_size": h, "vocab": v, "ms_with_policy_entropy_kl_losses": a,
+            "ms_with_plain_sums_instead": b, "losses_share_ms": a - b}
+
+
 def other_head_configs(dev, steps: int, with_cpu: bool = True) -> dict:
     """BASELINE configs[0] (Qwen2.5-0.5B head shape, forward only) and configs[4] (Llama-3-8B head shape, 65536
     tokens as eight 8192-token chunks, T = 0.7, entropy coefficient folded into the backward, weight gradient summed
@@ -940,6 +995,8 @@ def main() -> None:
     line["mfma_ceiling_probe"] = mfma_ceiling_probe(dev, n, h, v, seconds=args.ceiling_seconds)
     torch.cuda.empty_cache()
     line["head_other_configs"] = other_head_configs(dev, args.steps, with_cpu=args.cpu_tokens > 0)
+    torch.cuda.empty_cache()
+    line["actor_step_composed_b4_l4096"] = composed_actor_step(dev, args.steps)
     torch.cuda.empty_cache()
     line["unfused_logits_rows"] = unfused_logits_rates(dev)
     torch.cuda.empty_cache()
