@@ -9,8 +9,10 @@
  *   - the reductions (masked moments, agg_loss, policy / value / KL loss, the advantage
  *     estimators) finish inside one launch through arrival counters in the FIRST
  *     VAMD_TICKET_BYTES of their workspace: those bytes must be zero on entry, or as an earlier
- *     call of this library left them, and are zero again when the call has completed -- except the
- *     32-bit word at byte 132, an epoch that vamd_grpo_advantage advances and nothing else reads --
+ *     call of this library left them, and are zero again when the call has completed -- except two
+ *     32-bit words that no kernel depends on: byte 132, an epoch that vamd_grpo_advantage advances, and
+ *     byte 136 (VAMD_TICKET_GAVE_UP_OFFSET), a count of the workgroups that gave up a bounded wait on this
+ *     buffer and carried on by other means, which a host may read now and then --
  *     so a caller may zero a buffer once and reuse it for calls that are ordered on one stream;
  *   - return value: 0 on success, a negative VAMD_E* code otherwise; vamd_last_error() returns a
  *     thread-local description of the last failure on the calling thread;
@@ -37,6 +39,7 @@ extern "C" {
 #define VAMD_EHIP (-3)      /* a HIP runtime call failed; see vamd_last_error() */
 
 #define VAMD_TICKET_BYTES 16640 /* 65 arrival counters, 256 bytes apart */
+#define VAMD_TICKET_GAVE_UP_OFFSET 136 /* u32: workgroups that ever gave up a bounded wait on this buffer */
 
 #define VAMD_MASK_F32 0
 #define VAMD_MASK_I64 1

@@ -39,3 +39,17 @@ def dev():
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
     return torch.device("cuda:0")
+
+
+@pytest.fixture(autouse=True)
+def _waiting_kernels_as_the_environment_says(request):
+    """Tests force time-outs of the kernels that wait inside a launch; the host mirror reacts to those by switching
+    such kernels off for the process.  Every GPU test starts from what the environment says."""
+    yield
+    if "dev" in request.fixturenames:
+        from verl_amd import _cabi
+        from verl_amd.trainer.ppo import core_algos as CA
+
+        _cabi.lib().vamd_set_waiting_kernels(-1)
+        CA._WAITING_WATCH["calls"] = 0
+        CA._WAITING_WATCH["seen"].clear()

@@ -284,6 +284,7 @@ def test_grpo_single_launch_bounded_wait_runs_out_without_hanging(dev, monkeypat
     index = np.repeat(np.arange(B // 8), 8)
     want, _ = O.grpo_outcome_advantage(rewards.clone(), mask, index)
     calm, _ = compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
+    gave_up_before = _cabi.waiting_gave_up(_cabi.ticket_workspace(4096, dev))
     monkeypatch.setenv("VAMD_GATE_SPIN_LIMIT", "0")
     adv, _ = compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
     torch.cuda.synchronize()
@@ -293,8 +294,46 @@ def test_grpo_single_launch_bounded_wait_runs_out_without_hanging(dev, monkeypat
     assert torch.allclose(adv.cpu(), want, rtol=1e-5, atol=1e-6)
     ws = _cabi.ticket_workspace(4096, dev)
     assert _counter_area_is_clear(ws)
+    if os.environ.get("VAMD_WAITING_KERNELS") != "0":
+        # the workgroups that gave up were counted (with one meeting of the whole launch every workgroup but the last
+        # gives up; workgroups that wait for their groups' members may find them all there already)
+        gave_up = _cabi.waiting_gave_up(ws) - gave_up_before
+        assert gave_up > 0 if (B, L) == (512, 4096) else gave_up >= 0
     again, _ = compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), index)
     assert torch.equal(again, calm)
+
+
+def test_waiting_kernels_are_switched_off_once_workgroups_are_seen_giving_up(dev, monkeypatch):
+    """GRPO and the sequence-level losses recover from a wait that ran out inside the kernel; the host mirror looks at
+    the count of such workgroups every so many calls and, once it has grown, switches the waiting kernels off for the
+    process (results unchanged)."""
+    from verl_amd import _cabi
+    from verl_amd.trainer.ppo import core_algos as CA
+    if os.environ.get("VAMD_WAITING_KERNELS") == "0":
+        pytest.skip("waiting kernels are switched off in this environment")
+    L_ = _cabi.lib()
+    B, Lc = 512, 4096
+    g = torch.Generator().manual_seed(8)
+    rewards = torch.randn(B, Lc, generator=g).to(dev)
+    mask = (torch.rand(B, Lc, generator=g) < 0.8).float().to(dev)
+    index = np.repeat(np.arange(B // 8), 8)
+    calm, _ = CA.compute_grpo_outcome_advantage(rewards, mask, index)
+    monkeypatch.setattr(CA, "_WAITING_CHECK_EVERY", 1)
+    CA._WARNED.clear()
+    try:
+        CA.compute_grpo_outcome_advantage(rewards, mask, index)      # the first look notes where the count stands
+        assert L_.vamd_waiting_kernels_enabled() == 1
+        monkeypatch.setenv("VAMD_GATE_SPIN_LIMIT", "0")
+        with pytest.warns(RuntimeWarning, match="gave up waiting"):
+            hurried, _ = CA.compute_grpo_outcome_advantage(rewards, mask, index)
+        monkeypatch.delenv("VAMD_GATE_SPIN_LIMIT")
+        assert torch.equal(hurried, calm)
+        assert L_.vamd_waiting_kernels_enabled() == 0
+        apart, _ = CA.compute_grpo_outcome_advantage(rewards, mask, index)   # row sums, statistics, broadcast
+        assert torch.allclose(apart, calm, rtol=1e-5, atol=1e-6)
+    finally:
+        L_.vamd_set_waiting_kernels(-1)
+    assert L_.vamd_waiting_kernels_enabled() == 1
 
 
 def test_gae_multi_turn_fixture_and_errors(dev):
@@ -327,10 +366,11 @@ def test_gae_multi_turn_fixture_and_errors(dev):
 
 # ---- GRPO ---------------------------------------------------------------------------------------
 def _counter_area_is_clear(ws):
-    """The first VAMD_TICKET_BYTES of a reduction workspace are zero between calls, except the epoch word (word 33),
-    which only ever advances."""
+    """The first VAMD_TICKET_BYTES of a reduction workspace are zero between calls, except the epoch word (word 33)
+    and the give-up count (word 34), which only ever advance."""
     words = ws[:16640].view(torch.int32).clone()
     words[33] = 0
+    words[34] = 0   # the count of workgroups that ever gave up a wait: not zero between calls either
     return int(words.abs().sum()) == 0
 
 

@@ -234,6 +234,15 @@ def ticket_workspace(nbytes: int, device: torch.device) -> torch.Tensor:
     return buf
 
 
+GAVE_UP_OFFSET = 136  # VAMD_TICKET_GAVE_UP_OFFSET
+
+
+def waiting_gave_up(ticket_ws: torch.Tensor) -> int:
+    """How many workgroups have given up a bounded wait on this counter buffer since it was zeroed (waits for the
+    stream: it reads four bytes back)."""
+    return int(ticket_ws[GAVE_UP_OFFSET:GAVE_UP_OFFSET + 4].view(torch.int32).item())
+
+
 def mask_code(mask: torch.Tensor) -> tuple[torch.Tensor, int]:
     """Contiguous mask in one of the element types the kernels read, with its VAMD_MASK_* code."""
     dt = mask.dtype

@@ -524,6 +524,7 @@ __global__ __launch_bounds__(kRcThreads) void policy_kernel(
       if ((int)threadIdx.x < chunks && (int)threadIdx.x != chunk)
         ready = ready_byte_wait(wk.ticket, row * chunks + threadIdx.x, polls, pp.spin_limit);
       open = __syncthreads_and(ready) != 0;
+      if (!open && threadIdx.x == 0) note_gave_up(wk.ticket);
     }
     if (open) {
       if (threadIdx.x == 0) {
@@ -1345,6 +1346,7 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rows_kernel(GrpoRowsArgs a) {
           __builtin_amdgcn_s_sleep(4);
         }
         moved = seen != epoch_on_entry ? 1u : 0u;
+        if (!moved) note_gave_up(a.ticket);
       }
       __syncthreads();
       all_open = moved != 0u;
@@ -1375,6 +1377,7 @@ __global__ __launch_bounds__(kRcThreads) void grpo_rows_kernel(GrpoRowsArgs a) {
         }
       }
     const bool open = by_group ? __syncthreads_and(ready) != 0 : all_open;
+    if (by_group && !open && threadIdx.x == 0) note_gave_up(a.ticket);
     // count, sum and sum of squares of (score - own score) over the group: differences of fp32 scores are exact
     // in double, and shifted by the row's own score the one-pass variance loses nothing to cancellation
     double own[2], cs[6];

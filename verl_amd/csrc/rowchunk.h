@@ -270,6 +270,14 @@ constexpr int kDepartWord = 16, kReleaseWord = 32, kTimedOutWord = 48;
 // Word 33 of slot 0 is an epoch that only ever advances (a meeting without a departure count releases its waiters by
 // changing it): the one word of the area that is NOT zero between calls; nothing else reads it.
 constexpr int kEpochWord = 33;
+// Word 34 of slot 0 counts the workgroups that ever gave up a bounded wait on this buffer (and carried on by other
+// means): like the epoch it is not zero between calls and no kernel reads it.  A host reads it now and then to learn
+// that the waiting kernels time out on this device (they recover by themselves, at the price of their spin limit).
+constexpr int kGaveUpWord = 34;
+static_assert(kGaveUpWord * 4 == VAMD_TICKET_GAVE_UP_OFFSET, "the header documents where the count lives");
+__device__ __forceinline__ void note_gave_up(unsigned* counters) {  // one thread of the workgroup that gave up
+  __hip_atomic_fetch_add(counters + kGaveUpWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 constexpr unsigned kGateSpinLimit = 1u << 22;  // polls of about half a microsecond: seconds, not forever
 
 __device__ __forceinline__ void gate_release(unsigned* counters) {  // thread 0, after its peer stores
@@ -285,7 +293,10 @@ __device__ __forceinline__ bool gate_wait(unsigned* counters, unsigned spin_limi
       if (seen != 0 || spins >= spin_limit) break;
       __builtin_amdgcn_s_sleep(4);
     }
-    if (seen == 0) __hip_atomic_store(counters + kTimedOutWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (seen == 0) {
+      __hip_atomic_store(counters + kTimedOutWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      note_gave_up(counters);
+    }
     released = seen;
   }
   __syncthreads();

@@ -205,6 +205,30 @@ def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torc
         return adv.view(token_level_rewards.shape).to(out_dev), ret.view(token_level_rewards.shape).to(out_dev)
 
 
+# GRPO and the sequence-level losses recover from a wait that ran out inside their kernels and tell nobody; the
+# kernels count such workgroups in their counter buffer, and every _WAITING_CHECK_EVERY-th call looks at the count
+# (four bytes read back: a synchronisation, hence not on every call).  A count that has grown switches the waiting
+# kernels off for the process, like a time-out of GAE does.
+_WAITING_CHECK_EVERY = 64
+_WAITING_WATCH = {"calls": 0, "seen": {}}
+
+
+def _watch_waiting_kernels(ticket_ws: torch.Tensor) -> None:
+    _WAITING_WATCH["calls"] += 1
+    if _WAITING_WATCH["calls"] % _WAITING_CHECK_EVERY:
+        return
+    if torch.cuda.is_current_stream_capturing() or not _cabi.lib().vamd_waiting_kernels_enabled():
+        return
+    count = _cabi.waiting_gave_up(ticket_ws)
+    # the first look at a buffer only notes where its count stands; growth after that is what counts
+    if count > _WAITING_WATCH["seen"].get(ticket_ws.data_ptr(), count):
+        _cabi.lib().vamd_set_waiting_kernels(0)
+        _warn_once("workgroups of a kernel that waits inside its launch gave up waiting (a GPU shared with "
+                   "long-running kernels); such kernels are switched off from now on (set VAMD_WAITING_KERNELS=0 to "
+                   "make that the rule from the start)")
+    _WAITING_WATCH["seen"][ticket_ws.data_ptr()] = count
+
+
 _GROUP_ID_CACHE: "collections.OrderedDict" = collections.OrderedDict()
 _GROUP_ID_CACHE_SIZE = 8
 
@@ -250,6 +274,7 @@ def _grpo(token_level_rewards, response_mask, index, epsilon, norm_adv_by_std_in
                                                float(epsilon), int(bool(norm_adv_by_std_in_grpo)), std_mode,
                                                adv.data_ptr(), None, ws.data_ptr(), ws.numel(),
                                                _cabi.stream_ptr(dev)))
+        _watch_waiting_kernels(ws)
         out = adv.view(token_level_rewards.shape).to(token_level_rewards.device)
         return out, out
 
@@ -615,6 +640,8 @@ class _PolicyLoss(torch.autograd.Function):
                                                             clip_high, clip_c, tau_pos, tau_neg, mode, dp_size, bnt,
                                                             gbs, lsf, out.data_ptr(), _cabi.ptr(g), coef.data_ptr(),
                                                             ws.data_ptr(), ws.numel(), _cabi.stream_ptr(dev)))
+        if variant in (_PL["gspo"], _PL["geo_mean"]):
+            _watch_waiting_kernels(ws)
         if need_grad:
             ctx.save_for_backward(g, coef)
         ctx.in_shape = log_prob.shape
